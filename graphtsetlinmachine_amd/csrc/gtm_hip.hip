@@ -1,0 +1,830 @@
+// Graph Tsetlin Machine hot path for gfx950 (MI355X): HIP kernels and the
+// C ABI declared in include/gtm_abi.h.
+//
+// All arithmetic is 32-bit bitwise/integer work on wave64; nothing here is
+// GEMM-shaped, so no MFMA.  Layouts are the reference's (see gtm_abi.h).
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "../../include/gtm_abi.h"
+#include "philox.h"
+
+namespace {
+
+// ------------------------------------------------------------------ errors
+
+thread_local std::string g_error;
+
+int fail(int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_error = buf;
+    return code;
+}
+
+int check_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(GTM_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+    return GTM_OK;
+}
+
+// --------------------------------------------------------- derived constants
+
+struct Dims {
+    int K, C, LA, MC, NC, B, MB, M;
+    uint32_t filter, mfilter;
+};
+
+uint32_t tail_filter(int bits) {
+    int r = bits % 32;
+    return r == 0 ? 0xFFFFFFFFu : ~(0xFFFFFFFFu << r);
+}
+
+int validate(const gtm_config *cfg, Dims *d) {
+    if (!cfg) return fail(GTM_ERR_INVALID, "cfg is NULL");
+    if (cfg->classes < 1 || cfg->classes > 65535) return fail(GTM_ERR_INVALID, "classes=%d out of range", cfg->classes);
+    if (cfg->clauses < 1) return fail(GTM_ERR_INVALID, "clauses=%d", cfg->clauses);
+    if (cfg->literals < 1) return fail(GTM_ERR_INVALID, "literals=%d", cfg->literals);
+    if (cfg->state_bits < 1 || cfg->state_bits > 32) return fail(GTM_ERR_INVALID, "state_bits=%d out of 1..32", cfg->state_bits);
+    if (cfg->threshold < 1) return fail(GTM_ERR_INVALID, "threshold=%d", cfg->threshold);
+    if (cfg->max_nodes < 1) return fail(GTM_ERR_INVALID, "max_nodes=%d", cfg->max_nodes);
+    if (cfg->depth < 1 || cfg->depth > GTM_MAX_DEPTH) return fail(GTM_ERR_INVALID, "depth=%d out of 1..%d", cfg->depth, GTM_MAX_DEPTH);
+    if (cfg->message_size < 1 || cfg->message_bits < 1) return fail(GTM_ERR_INVALID, "message_size/message_bits must be >= 1");
+    if (cfg->message_bits > 64) return fail(GTM_ERR_INVALID, "message_bits=%d > 64", cfg->message_bits);
+    d->K = cfg->classes;
+    d->C = cfg->clauses;
+    d->LA = (cfg->literals - 1) / 32 + 1;
+    d->MC = (2 * cfg->message_size - 1) / 32 + 1;
+    d->NC = (cfg->max_nodes - 1) / 32 + 1;
+    d->B = cfg->state_bits;
+    d->MB = cfg->message_bits;
+    d->M = cfg->message_size;
+    d->filter = tail_filter(cfg->literals);
+    d->mfilter = tail_filter(2 * cfg->message_size);
+    return GTM_OK;
+}
+
+int validate_graphs(const gtm_config *cfg, const gtm_graphs *g, int first, int n) {
+    if (!g) return fail(GTM_ERR_INVALID, "graphs is NULL");
+    if (!g->X || !g->node_type || !g->node_index || !g->number_of_graph_nodes)
+        return fail(GTM_ERR_INVALID, "graphs has NULL arrays");
+    if (g->number_of_node_types < 1) return fail(GTM_ERR_INVALID, "number_of_node_types=%d", g->number_of_node_types);
+    if (g->max_number_of_graph_nodes > cfg->max_nodes)
+        return fail(GTM_ERR_INVALID, "graphs hold up to %d nodes but the model was sized for max_nodes=%d",
+                    g->max_number_of_graph_nodes, cfg->max_nodes);
+    if (first < 0 || n < 0 || (int64_t)first + n > g->number_of_graphs)
+        return fail(GTM_ERR_INVALID, "graph range [%d, %d) outside 0..%d", first, first + n, g->number_of_graphs);
+    return GTM_OK;
+}
+
+uint32_t feedback_threshold(double s) {
+    double t = 65536.0 / s;
+    if (!(t < 65536.0)) return 65536u;
+    if (t < 0.0) return 0u;
+    return (uint32_t)t;
+}
+
+uint64_t q_threshold(double q, int classes) {
+    double p = q / (double)(classes - 1 > 1 ? classes - 1 : 1);
+    if (p > 1.0) p = 1.0;
+    if (p < 0.0) p = 0.0;
+    return (uint64_t)(p * 4294967296.0);
+}
+
+inline unsigned blocks_for(int64_t items, int per_block) { return (unsigned)((items + per_block - 1) / per_block); }
+
+constexpr int TPB = 256;
+
+__device__ __forceinline__ int chunks_of(int n) { return n == 0 ? 1 : (n - 1) / 32 + 1; }  // C division of kernels.py:289
+__device__ __forceinline__ uint32_t node_filter_of(int n) {
+    int r = n % 32;
+    return r == 0 ? 0xFFFFFFFFu : ~(0xFFFFFFFFu << r);
+}
+
+// ------------------------------------------------------------------ kernels
+
+// K11/K12: every automaton to state 2^(B-1)-1; optional weights.
+__global__ void k_prepare_bank(uint32_t *bank, int64_t words, int B) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < words) bank[i] = ((int)(i % B) == B - 1) ? 0u : 0xFFFFFFFFu;
+}
+
+__global__ void k_prepare_weights(int32_t *w, int K, int C, int negative, uint32_t k0, uint32_t k1, uint32_t step) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= K * C) return;
+    int class_id = i / C, clause = i % C;
+    int v = 1;
+    if (negative == 1) {
+        philox_out r = philox4x32_10((uint32_t)clause, (uint32_t)class_id, step, GTM_TAG_PREPARE, k0, k1);
+        v = 1 - 2 * (int)(r.v[0] & 1u);
+    }
+    w[i] = v;
+}
+
+// Include plane of a bank, word-major ([chunk][clause]) so that lanes that
+// hold consecutive clauses read consecutive addresses; also the include count
+// of kernels.py:251-277.
+__global__ void k_include_plane(const uint32_t *__restrict__ bank, int C, int chunks, int B, uint32_t filter,
+                                uint32_t *__restrict__ inc_t, int32_t *n_incl, int accumulate) {
+    int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    int count = 0;
+    for (int w = 0; w < chunks; ++w) {
+        uint32_t v = bank[((int64_t)c * chunks + w) * B + (B - 1)];
+        if (w == chunks - 1) v &= filter;
+        inc_t[(int64_t)w * C + c] = v;
+        count += __popc(v);
+    }
+    if (n_incl) n_incl[c] = accumulate ? n_incl[c] + count : count;
+}
+
+// K1 / K2: truth of clause c at the <=32 nodes of chunk nc of graph b.
+// rows_mode 0: literal rows are X rows of the graph (base node_index[g]);
+// rows_mode 1: literal rows are the graph's packed messages (base b*max_nodes).
+template <int REG_CHUNKS>
+__global__ void k_clause_node_bits(const uint32_t *__restrict__ inc_t, int C, int chunks, const uint32_t *__restrict__ rows,
+                                   int rows_mode, int max_nodes, const uint32_t *__restrict__ node_type, int n_types,
+                                   const uint32_t *__restrict__ node_index, const uint32_t *__restrict__ n_nodes_arr,
+                                   int first_graph, int NC, const uint32_t *__restrict__ cond, uint32_t *__restrict__ out,
+                                   int clause_blocks) {
+    int64_t blk = blockIdx.x;
+    int cb = (int)(blk % clause_blocks);
+    int64_t rest = blk / clause_blocks;
+    int nc = (int)(rest % NC);
+    int b = (int)(rest / NC);
+    int c = cb * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    int g = first_graph + b;
+    int n = (int)n_nodes_arr[g];
+    int64_t base = (int64_t)node_index[g];
+    const uint32_t *rbase = rows_mode == 0 ? rows + base * chunks : rows + (int64_t)b * max_nodes * chunks;
+    uint32_t word;
+    if (nc >= chunks_of(n) || n == 0) {
+        word = 0xFFFFFFFFu;  // kernels.py:443-466: chunks past the graph are left all ones
+    } else {
+        uint32_t inc[REG_CHUNKS > 0 ? REG_CHUNKS : 1];
+        if (REG_CHUNKS > 0) {
+#pragma unroll
+            for (int w = 0; w < REG_CHUNKS; ++w) inc[w] = w < chunks ? inc_t[(int64_t)w * C + c] : 0u;
+        }
+        int my_type = c % n_types;
+        word = 0;
+        int node0 = nc * 32;
+        int lim = n - node0 < 32 ? n - node0 : 32;
+        for (int p = 0; p < lim; ++p) {
+            int node = node0 + p;
+            const uint32_t *row = rbase + (int64_t)node * chunks;  // uniform across the wave
+            uint32_t violated = 0;
+            if (REG_CHUNKS > 0) {
+#pragma unroll
+                for (int w = 0; w < REG_CHUNKS; ++w)
+                    if (w < chunks) violated |= inc[w] & ~row[w];
+            } else {
+                for (int w = 0; w < chunks; ++w) violated |= inc_t[(int64_t)w * C + c] & ~row[w];
+            }
+            bool ok = violated == 0 && (int)node_type[base + node] == my_type;
+            word |= (uint32_t)ok << p;
+        }
+    }
+    int64_t o = ((int64_t)b * C + c) * NC + nc;
+    if (cond) word &= cond[o];
+    out[o] = word;
+}
+
+// K3: packed messages start as "no message": positive half 0, negated half 1.
+__global__ void k_messages_blank(uint32_t *clause_X, int64_t words, int MC, int M) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= words) return;
+    int m = (int)(i % MC);
+    int lo = m * 32, hi = lo + 32;
+    int a = lo > M ? lo : M, z = hi < 2 * M ? hi : 2 * M;
+    uint32_t v = 0;
+    if (a < z) {
+        int len = z - a;
+        uint32_t ones = len == 32 ? 0xFFFFFFFFu : ((1u << len) - 1u);
+        v = ones << (a - lo);
+    }
+    clause_X[i] = v;
+}
+
+// K4 (+K5): each true (clause, source node) sets, at every out-neighbour, the
+// clause's hypervector bits rotated by the edge type and clears their
+// negations (kernels.py:571-588), straight into the packed words.
+__global__ void k_messages_scatter(const uint32_t *__restrict__ bitmap, int C, int NC, const uint32_t *__restrict__ hv,
+                                   int MB, int M, int MC, int max_nodes, const uint32_t *__restrict__ node_index,
+                                   const uint32_t *__restrict__ n_nodes_arr, const uint32_t *__restrict__ n_edges,
+                                   const uint32_t *__restrict__ edge_index, const uint32_t *__restrict__ edge,
+                                   int first_graph, int64_t total, uint32_t *clause_X) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    int nc = (int)(i % NC);
+    int64_t rest = i / NC;
+    int c = (int)(rest % C);
+    int b = (int)(rest / C);
+    int g = first_graph + b;
+    int n = (int)n_nodes_arr[g];
+    if (n == 0 || nc >= chunks_of(n)) return;
+    uint32_t word = bitmap[i];
+    if (nc == chunks_of(n) - 1) word &= node_filter_of(n);
+    if (word == 0) return;
+    int64_t base = (int64_t)node_index[g];
+    uint32_t *cx = clause_X + (int64_t)b * max_nodes * MC;
+    while (word) {
+        int p = __ffs(word) - 1;
+        word &= word - 1;
+        int64_t row = base + nc * 32 + p;
+        uint32_t ne = n_edges[row];
+        int64_t e0 = edge_index[row];
+        for (uint32_t e = 0; e < ne; ++e) {
+            uint32_t dst = edge[(e0 + e) * 2];
+            uint32_t type = edge[(e0 + e) * 2 + 1];
+            for (int j = 0; j < MB; ++j) {
+                uint32_t pos = (hv[(int64_t)c * MB + j] + type) % (uint32_t)M;
+                uint32_t neg = pos + (uint32_t)M;
+                atomicOr(&cx[(int64_t)dst * MC + (pos >> 5)], 1u << (pos & 31));
+                atomicAnd(&cx[(int64_t)dst * MC + (neg >> 5)], ~(1u << (neg & 31)));
+            }
+        }
+    }
+}
+
+__global__ void k_fill_i32(int32_t *p, int64_t n, int32_t v) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// K6: a block covers TPB clauses of one graph; per class one wave reduction
+// and one atomicAdd per wave.
+__global__ void k_class_sums(const uint32_t *__restrict__ bitmap, int C, int NC, int K,
+                             const int32_t *__restrict__ weights, const uint32_t *__restrict__ n_nodes_arr,
+                             int first_graph, int clause_blocks, int32_t *class_sum) {
+    int b = blockIdx.x / clause_blocks;
+    int c = (blockIdx.x % clause_blocks) * blockDim.x + threadIdx.x;
+    int n = (int)n_nodes_arr[first_graph + b];
+    bool fired = false;
+    if (c < C) {
+        int nch = chunks_of(n);
+        const uint32_t *row = bitmap + ((int64_t)b * C + c) * NC;
+        uint32_t any = 0;
+        for (int k = 0; k < nch - 1; ++k) any |= row[k];
+        any |= row[nch - 1] & node_filter_of(n);
+        fired = any != 0;
+    }
+    if (__ballot(fired) == 0) return;
+    for (int k = 0; k < K; ++k) {
+        int v = fired ? weights[(int64_t)k * C + c] : 0;
+        for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+        if ((threadIdx.x & 63) == 0 && v != 0) atomicAdd(&class_sum[(int64_t)b * K + k], v);
+    }
+}
+
+// K7: uniform choice among the true nodes of each clause.
+__global__ void k_select_clause_node(const uint32_t *__restrict__ bitmap, int C, int NC, int n, uint32_t k0, uint32_t k1,
+                                     uint32_t step, int32_t *clause_node) {
+    int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const uint32_t *row = bitmap + (int64_t)c * NC;
+    int nch = n == 0 ? 0 : (n - 1) / 32 + 1;  // an empty graph has no node to pick (kernels.py:336)
+    uint32_t last = node_filter_of(n);
+    int count = 0;
+    for (int k = 0; k < nch; ++k) count += __popc(k == nch - 1 ? row[k] & last : row[k]);
+    int node = -1;
+    if (count > 0) {
+        philox_out r = philox4x32_10((uint32_t)c, 0u, step, GTM_TAG_CLAUSE_NODE, k0, k1);
+        int pick = (int)(((uint64_t)r.v[0] * (uint64_t)count) >> 32);
+        for (int k = 0; k < nch; ++k) {
+            uint32_t w = k == nch - 1 ? row[k] & last : row[k];
+            int pc = __popc(w);
+            if (pick < pc) {
+                for (int j = 0; j < pick; ++j) w &= w - 1;
+                node = k * 32 + __ffs(w) - 1;
+                break;
+            }
+            pick -= pc;
+        }
+    }
+    clause_node[c] = node;
+}
+
+// K8: feedback decision per (class, clause) and weight update.
+__global__ void k_select_clause_updates(int32_t *weights, const int32_t *__restrict__ class_sum,
+                                        const int32_t *__restrict__ y, int K, int C, int T, int negative,
+                                        uint64_t q_thr, uint32_t k0, uint32_t k1, uint32_t step,
+                                        const int32_t *__restrict__ clause_node, int32_t *update) {
+    int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    bool fired = clause_node[c] != -1;
+    for (int k = 0; k < K; ++k) {
+        int cs = class_sum[k];
+        cs = cs > T ? T : (cs < -T ? -T : cs);
+        int yk = y[k];
+        int target = 1 - 2 * (cs > yk);
+        int w = weights[(int64_t)k * C + c];
+        int sign = (w >= 0) - (w < 0);
+        int err = yk - cs;
+        err = err < 0 ? -err : err;
+        philox_out r = philox4x32_10((uint32_t)c, (uint32_t)k, step, GTM_TAG_CLAUSE_UPDATES, k0, k1);
+        bool skip = (target == -1 && (uint64_t)r.v[0] >= q_thr) ||
+                    ((uint64_t)r.v[1] * (uint64_t)(2 * (int64_t)T) >= ((uint64_t)err << 32));
+        int u = skip ? 0 : target * sign;
+        update[(int64_t)k * C + c] = u;
+        if (u > 0 && fired && (w < 0 ? -(int64_t)w : (int64_t)w) < 2147483647) {
+            weights[(int64_t)k * C + c] = w + sign;
+        } else if (u < 0 && fired) {
+            w -= sign;
+            if (negative == 0 && w < 1) w = 1;
+            weights[(int64_t)k * C + c] = w;
+        }
+    }
+}
+
+// kernels.py:55-96 on one word of 32 automata held as B bit planes.
+__device__ __forceinline__ void ta_inc(uint32_t *ta, int B, uint32_t active) {
+    uint32_t carry = active;
+    for (int b = 0; b < B && carry; ++b) {
+        uint32_t v = ta[b];
+        ta[b] = v ^ carry;
+        carry &= v;
+    }
+    if (carry)
+        for (int b = 0; b < B; ++b) ta[b] |= carry;
+}
+
+__device__ __forceinline__ void ta_dec(uint32_t *ta, int B, uint32_t active) {
+    uint32_t carry = active;
+    for (int b = 0; b < B && carry; ++b) {
+        uint32_t v = ta[b];
+        ta[b] = v ^ carry;
+        carry &= ~v;
+    }
+    if (carry)
+        for (int b = 0; b < B; ++b) ta[b] &= ~carry;
+}
+
+// K9 / K10: one thread per (clause, automaton word); the classes are applied
+// in ascending order to that word, as kernels.py:205-207,236-238 do per clause
+// (words of a clause do not interact, so splitting by word keeps the result).
+__global__ void k_update(uint32_t *bank, int C, int chunks, int B, int K, int boost, int max_included, uint32_t thr16,
+                         uint32_t k0, uint32_t k1, uint32_t step, uint32_t bank_id,
+                         const int32_t *__restrict__ clause_node, const int32_t *__restrict__ n_incl,
+                         const uint32_t *__restrict__ rows, const int32_t *__restrict__ update) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)C * chunks) return;
+    int c = (int)(i / chunks), w = (int)(i % chunks);
+    int node = clause_node[c];
+    bool fired = node != -1;
+    bool within = n_incl[c] <= max_included;
+    uint32_t x = fired ? rows[(int64_t)node * chunks + w] : 0u;
+    uint32_t *ta = bank + i * B;
+    for (int k = 0; k < K; ++k) {
+        int u = update[(int64_t)k * C + c];
+        if (u > 0) {
+            uint32_t fb = gtm_feedback_bits(k0, k1, (uint32_t)c, (uint32_t)w, step, bank_id, (uint32_t)k, thr16);
+            if (fired && within) {
+                ta_inc(ta, B, boost == 1 ? x : (x & ~fb));
+                ta_dec(ta, B, ~x & fb);
+            } else {
+                ta_dec(ta, B, fb);
+            }
+        } else if (u < 0 && fired) {
+            ta_inc(ta, B, ~x & ~ta[B - 1]);
+        }
+    }
+}
+
+// ------------------------------------------------------------ launch helpers
+
+int launch_clause_node_bits(const Dims &d, const gtm_graphs *g, int first, int n_graphs, const uint32_t *inc_t,
+                            int chunks, const uint32_t *rows, int rows_mode, int max_nodes, const uint32_t *cond,
+                            uint32_t *out, hipStream_t st) {
+    int clause_blocks = (d.C + TPB - 1) / TPB;
+    int64_t blocks = (int64_t)clause_blocks * d.NC * n_graphs;
+    if (blocks == 0) return GTM_OK;
+    if (blocks > 0x7FFFFFFF) return fail(GTM_ERR_INVALID, "batch too large for one launch (%lld blocks)", (long long)blocks);
+#define GTM_LAUNCH_CNB(R)                                                                                        \
+    hipLaunchKernelGGL((k_clause_node_bits<R>), dim3((unsigned)blocks), dim3(TPB), 0, st, inc_t, d.C, chunks, rows, \
+                       rows_mode, max_nodes, g->node_type, g->number_of_node_types, g->node_index,                \
+                       g->number_of_graph_nodes, first, d.NC, cond, out, clause_blocks)
+    if (chunks <= 2) GTM_LAUNCH_CNB(2);
+    else if (chunks <= 4) GTM_LAUNCH_CNB(4);
+    else if (chunks <= 8) GTM_LAUNCH_CNB(8);
+    else if (chunks <= 16) GTM_LAUNCH_CNB(16);
+    else GTM_LAUNCH_CNB(0);
+#undef GTM_LAUNCH_CNB
+    return check_launch("clause_node_bits");
+}
+
+struct Key {
+    uint32_t k0, k1;
+};
+Key key_of(const gtm_config *cfg) { return Key{(uint32_t)(cfg->seed & 0xFFFFFFFFu), (uint32_t)(cfg->seed >> 32)}; }
+
+// Workspace carving -----------------------------------------------------------
+
+size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct ScoreWs {
+    uint32_t *inc_t;     // [max(LA,MC)][C]
+    uint32_t *bitmap_a;  // [batch][C][NC]
+    uint32_t *bitmap_b;  // [batch][C][NC] (depth > 1)
+    uint32_t *clause_X;  // [batch][max_nodes][MC] (depth > 1)
+    size_t bytes;
+};
+
+ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base) {
+    ScoreWs w;
+    size_t off = 0;
+    int chunks = cfg->depth > 1 && d.MC > d.LA ? d.MC : d.LA;
+    auto take = [&](size_t bytes) {
+        char *p = base ? base + off : nullptr;
+        off += align_up(bytes);
+        return p;
+    };
+    w.inc_t = (uint32_t *)take((size_t)chunks * d.C * 4);
+    w.bitmap_a = (uint32_t *)take((size_t)batch * d.C * d.NC * 4);
+    if (cfg->depth > 1) {
+        w.bitmap_b = (uint32_t *)take((size_t)batch * d.C * d.NC * 4);
+        w.clause_X = (uint32_t *)take((size_t)batch * cfg->max_nodes * d.MC * 4);
+    } else {
+        w.bitmap_b = nullptr;
+        w.clause_X = nullptr;
+    }
+    w.bytes = off;
+    return w;
+}
+
+struct FitWs {
+    uint32_t *inc_t;
+    uint32_t *bitmap_a, *bitmap_b;
+    uint32_t *clause_X[GTM_MAX_DEPTH - 1];  // per message layer, kept for K10
+    int32_t *class_sum;                     // [K]
+    int32_t *clause_node;                   // [C]
+    int32_t *n_incl;                        // [C]
+    int32_t *update;                        // [K][C]
+    size_t bytes;
+};
+
+FitWs carve_fit(const Dims &d, const gtm_config *cfg, char *base) {
+    FitWs w;
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        char *p = base ? base + off : nullptr;
+        off += align_up(bytes);
+        return p;
+    };
+    int chunks = cfg->depth > 1 && d.MC > d.LA ? d.MC : d.LA;
+    w.inc_t = (uint32_t *)take((size_t)chunks * d.C * 4);
+    w.bitmap_a = (uint32_t *)take((size_t)d.C * d.NC * 4);
+    w.bitmap_b = (uint32_t *)take((size_t)d.C * d.NC * 4);
+    for (int l = 0; l < GTM_MAX_DEPTH - 1; ++l)
+        w.clause_X[l] = l < cfg->depth - 1 ? (uint32_t *)take((size_t)cfg->max_nodes * d.MC * 4) : nullptr;
+    w.class_sum = (int32_t *)take((size_t)d.K * 4);
+    w.clause_node = (int32_t *)take((size_t)d.C * 4);
+    w.n_incl = (int32_t *)take((size_t)d.C * 4);
+    w.update = (int32_t *)take((size_t)d.K * d.C * 4);
+    w.bytes = off;
+    return w;
+}
+
+// Operator bodies shared by the per-kernel entry points and the driver loops ----
+
+int op_include_plane(const Dims &d, const uint32_t *bank, int chunks, uint32_t filter, uint32_t *inc_t, int32_t *n_incl,
+                     int accumulate, hipStream_t st) {
+    hipLaunchKernelGGL(k_include_plane, dim3(blocks_for(d.C, TPB)), dim3(TPB), 0, st, bank, d.C, chunks, d.B, filter,
+                       inc_t, n_incl, accumulate);
+    return check_launch("include_plane");
+}
+
+int op_exchange(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, int first, int n_graphs,
+                const uint32_t *hv, const uint32_t *bitmap, uint32_t *clause_X, hipStream_t st) {
+    if (n_graphs == 0) return GTM_OK;
+    int64_t words = (int64_t)n_graphs * cfg->max_nodes * d.MC;
+    hipLaunchKernelGGL(k_messages_blank, dim3(blocks_for(words, TPB)), dim3(TPB), 0, st, clause_X, words, d.MC, d.M);
+    if (int rc = check_launch("messages_blank")) return rc;
+    if (g->total_edges > 0) {
+        if (!g->number_of_graph_node_edges || !g->edge || !g->edge_index)
+            return fail(GTM_ERR_INVALID, "graphs with edges need number_of_graph_node_edges, edge and edge_index");
+        int64_t total = (int64_t)n_graphs * d.C * d.NC;
+        hipLaunchKernelGGL(k_messages_scatter, dim3(blocks_for(total, TPB)), dim3(TPB), 0, st, bitmap, d.C, d.NC, hv,
+                           d.MB, d.M, d.MC, cfg->max_nodes, g->node_index, g->number_of_graph_nodes,
+                           g->number_of_graph_node_edges, g->edge_index, g->edge, first, total, clause_X);
+        if (int rc = check_launch("messages_scatter")) return rc;
+    }
+    return GTM_OK;
+}
+
+int op_class_sums(const Dims &d, const gtm_graphs *g, int first, int n_graphs, const uint32_t *bitmap,
+                  const int32_t *weights, int32_t *class_sum, hipStream_t st) {
+    if (n_graphs == 0) return GTM_OK;
+    int64_t n = (int64_t)n_graphs * d.K;
+    hipLaunchKernelGGL(k_fill_i32, dim3(blocks_for(n, TPB)), dim3(TPB), 0, st, class_sum, n, 0);
+    if (int rc = check_launch("fill")) return rc;
+    int clause_blocks = (d.C + TPB - 1) / TPB;
+    hipLaunchKernelGGL(k_class_sums, dim3((unsigned)(clause_blocks * (int64_t)n_graphs)), dim3(TPB), 0, st, bitmap, d.C,
+                       d.NC, d.K, weights, g->number_of_graph_nodes, first, clause_blocks, class_sum);
+    return check_launch("class_sums");
+}
+
+// The graph-independent part of `_evaluate` for a batch (tm.py:563-662).
+// Leaves the final bitmap in *final_bitmap.
+int run_evaluate(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, int first, int n_graphs,
+                 uint32_t *inc_t, uint32_t *bm_a, uint32_t *bm_b, uint32_t *const *clause_X, bool keep_layers,
+                 int32_t *n_incl, int32_t *class_sum, uint32_t **final_bitmap, hipStream_t st) {
+    if (int rc = op_include_plane(d, s->ta_state, d.LA, d.filter, inc_t, n_incl, 0, st)) return rc;
+    if (int rc = launch_clause_node_bits(d, g, first, n_graphs, inc_t, d.LA, g->X, 0, cfg->max_nodes, nullptr, bm_a, st))
+        return rc;
+    uint32_t *cur = bm_a, *nxt = bm_b;
+    for (int layer = 0; layer < cfg->depth - 1; ++layer) {
+        uint32_t *cx = keep_layers ? clause_X[layer] : clause_X[0];
+        if (int rc = op_exchange(d, cfg, g, first, n_graphs, s->hypervectors, cur, cx, st)) return rc;
+        if (int rc = op_include_plane(d, s->message_ta_state[layer], d.MC, d.mfilter, inc_t, n_incl, 1, st)) return rc;
+        if (int rc = launch_clause_node_bits(d, g, first, n_graphs, inc_t, d.MC, cx, 1, cfg->max_nodes, cur, nxt, st))
+            return rc;
+        uint32_t *t = cur;
+        cur = nxt;
+        nxt = t;
+    }
+    if (int rc = op_class_sums(d, g, first, n_graphs, cur, s->clause_weights, class_sum, st)) return rc;
+    *final_bitmap = cur;
+    return GTM_OK;
+}
+
+int validate_state(const gtm_config *cfg, const gtm_state *s) {
+    if (!s) return fail(GTM_ERR_INVALID, "state is NULL");
+    if (!s->ta_state || !s->clause_weights) return fail(GTM_ERR_INVALID, "state has NULL ta_state or clause_weights");
+    for (int l = 0; l < cfg->depth - 1; ++l)
+        if (!s->message_ta_state[l]) return fail(GTM_ERR_INVALID, "state lacks message_ta_state[%d]", l);
+    if (cfg->depth > 1 && !s->hypervectors) return fail(GTM_ERR_INVALID, "state lacks hypervectors");
+    return GTM_OK;
+}
+
+}  // namespace
+
+// =============================================================== C ABI
+
+extern "C" {
+
+int gtm_abi_version(void) { return GTM_ABI_VERSION; }
+
+const char *gtm_last_error(void) { return g_error.c_str(); }
+
+int gtm_prepare(const gtm_config *cfg, uint64_t step, uint32_t *ta_state, int32_t *clause_weights, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (!ta_state || !clause_weights) return fail(GTM_ERR_INVALID, "NULL buffer");
+    hipStream_t st = (hipStream_t)stream;
+    int64_t words = (int64_t)d.C * d.LA * d.B;
+    hipLaunchKernelGGL(k_prepare_bank, dim3(blocks_for(words, TPB)), dim3(TPB), 0, st, ta_state, words, d.B);
+    if (int rc = check_launch("prepare_bank")) return rc;
+    Key k = key_of(cfg);
+    hipLaunchKernelGGL(k_prepare_weights, dim3(blocks_for((int64_t)d.K * d.C, TPB)), dim3(TPB), 0, st, clause_weights,
+                       d.K, d.C, cfg->negative_clauses, k.k0, k.k1, (uint32_t)step);
+    return check_launch("prepare_weights");
+}
+
+int gtm_prepare_message_ta_state(const gtm_config *cfg, uint32_t *message_ta_state, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (!message_ta_state) return fail(GTM_ERR_INVALID, "NULL buffer");
+    int64_t words = (int64_t)d.C * d.MC * d.B;
+    hipLaunchKernelGGL(k_prepare_bank, dim3(blocks_for(words, TPB)), dim3(TPB), 0, (hipStream_t)stream,
+                       message_ta_state, words, d.B);
+    return check_launch("prepare_bank");
+}
+
+int gtm_calculate_messages(const gtm_config *cfg, const gtm_graphs *graphs, int32_t first_graph, int32_t n_graphs,
+                           const uint32_t *ta_state, uint32_t *include_plane, uint32_t *clause_node_output,
+                           int32_t *number_of_include_actions, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (int rc = validate_graphs(cfg, graphs, first_graph, n_graphs)) return rc;
+    if (!ta_state || !clause_node_output || !include_plane) return fail(GTM_ERR_INVALID, "NULL buffer");
+    hipStream_t st = (hipStream_t)stream;
+    if (int rc = op_include_plane(d, ta_state, d.LA, d.filter, include_plane, number_of_include_actions, 0, st)) return rc;
+    return launch_clause_node_bits(d, graphs, first_graph, n_graphs, include_plane, d.LA, graphs->X, 0, cfg->max_nodes,
+                                   nullptr, clause_node_output, st);
+}
+
+int gtm_exchange_messages(const gtm_config *cfg, const gtm_graphs *graphs, int32_t first_graph, int32_t n_graphs,
+                          const uint32_t *hypervectors, const uint32_t *clause_node_output, uint32_t *clause_X,
+                          void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (int rc = validate_graphs(cfg, graphs, first_graph, n_graphs)) return rc;
+    if (!hypervectors || !clause_node_output || !clause_X) return fail(GTM_ERR_INVALID, "NULL buffer");
+    return op_exchange(d, cfg, graphs, first_graph, n_graphs, hypervectors, clause_node_output, clause_X,
+                       (hipStream_t)stream);
+}
+
+int gtm_calculate_messages_conditional(const gtm_config *cfg, const gtm_graphs *graphs, int32_t first_graph,
+                                       int32_t n_graphs, const uint32_t *message_ta_state, uint32_t *include_plane,
+                                       const uint32_t *clause_node_output_condition, uint32_t *clause_node_output,
+                                       int32_t *number_of_include_actions, const uint32_t *clause_X, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (int rc = validate_graphs(cfg, graphs, first_graph, n_graphs)) return rc;
+    if (!message_ta_state || !clause_node_output_condition || !clause_node_output || !clause_X || !include_plane)
+        return fail(GTM_ERR_INVALID, "NULL buffer");
+    hipStream_t st = (hipStream_t)stream;
+    if (int rc = op_include_plane(d, message_ta_state, d.MC, d.mfilter, include_plane, number_of_include_actions, 1, st))
+        return rc;
+    return launch_clause_node_bits(d, graphs, first_graph, n_graphs, include_plane, d.MC, clause_X, 1, cfg->max_nodes,
+                                   clause_node_output_condition, clause_node_output, st);
+}
+
+int gtm_evaluate(const gtm_config *cfg, const gtm_graphs *graphs, int32_t first_graph, int32_t n_graphs,
+                 const uint32_t *clause_node_output, const int32_t *clause_weights, int32_t *class_sum,
+                 void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (int rc = validate_graphs(cfg, graphs, first_graph, n_graphs)) return rc;
+    if (!clause_node_output || !clause_weights || !class_sum) return fail(GTM_ERR_INVALID, "NULL buffer");
+    return op_class_sums(d, graphs, first_graph, n_graphs, clause_node_output, clause_weights, class_sum,
+                         (hipStream_t)stream);
+}
+
+}  // extern "C"
+
+namespace {
+
+// Training operators take the example's node count from the host copy that
+// the caller passes (the driver loop reads it once per dataset).
+int op_select_clause_node(const Dims &d, const gtm_config *cfg, int n_nodes, uint64_t step, const uint32_t *bitmap,
+                          int32_t *clause_node, hipStream_t st) {
+    Key k = key_of(cfg);
+    hipLaunchKernelGGL(k_select_clause_node, dim3(blocks_for(d.C, TPB)), dim3(TPB), 0, st, bitmap, d.C, d.NC, n_nodes,
+                       k.k0, k.k1, (uint32_t)step, clause_node);
+    return check_launch("select_clause_node");
+}
+
+int op_select_clause_updates(const Dims &d, const gtm_config *cfg, uint64_t step, int32_t *weights,
+                             const int32_t *class_sum, const int32_t *y_row, const int32_t *clause_node,
+                             int32_t *update, hipStream_t st) {
+    Key k = key_of(cfg);
+    hipLaunchKernelGGL(k_select_clause_updates, dim3(blocks_for(d.C, TPB)), dim3(TPB), 0, st, weights, class_sum, y_row,
+                       d.K, d.C, cfg->threshold, cfg->negative_clauses, q_threshold(cfg->q, cfg->classes), k.k0, k.k1,
+                       (uint32_t)step, clause_node, update);
+    return check_launch("select_clause_updates");
+}
+
+int op_update(const Dims &d, const gtm_config *cfg, uint64_t step, int bank_id, uint32_t *bank, int chunks,
+              const int32_t *clause_node, const int32_t *n_incl, const uint32_t *rows, const int32_t *update,
+              hipStream_t st) {
+    Key k = key_of(cfg);
+    int64_t items = (int64_t)d.C * chunks;
+    hipLaunchKernelGGL(k_update, dim3(blocks_for(items, TPB)), dim3(TPB), 0, st, bank, d.C, chunks, d.B, d.K,
+                       cfg->boost_true_positive_feedback, cfg->max_included_literals,
+                       feedback_threshold(cfg->s[bank_id]), k.k0, k.k1, (uint32_t)step, (uint32_t)bank_id, clause_node,
+                       n_incl, rows, update);
+    return check_launch("update");
+}
+
+}  // namespace
+
+extern "C" {
+
+int gtm_select_clause_node(const gtm_config *cfg, const gtm_graphs *graphs, int32_t example, uint64_t step,
+                           const uint32_t *clause_node_output, int32_t *clause_node, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (int rc = validate_graphs(cfg, graphs, example, 1)) return rc;
+    if (!clause_node_output || !clause_node) return fail(GTM_ERR_INVALID, "NULL buffer");
+    uint32_t n = 0;
+    hipError_t e = hipMemcpyAsync(&n, graphs->number_of_graph_nodes + example, 4, hipMemcpyDeviceToHost,
+                                  (hipStream_t)stream);
+    if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+    if (e != hipSuccess) return fail(GTM_ERR_HIP, "reading node count: %s", hipGetErrorString(e));
+    return op_select_clause_node(d, cfg, (int)n, step, clause_node_output, clause_node, (hipStream_t)stream);
+}
+
+int gtm_select_clause_updates(const gtm_config *cfg, uint64_t step, int32_t *clause_weights,
+                              const int32_t *class_sum, const int32_t *encoded_Y, int32_t example,
+                              const int32_t *clause_node, int32_t *class_clause_update, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (!clause_weights || !class_sum || !encoded_Y || !clause_node || !class_clause_update || example < 0)
+        return fail(GTM_ERR_INVALID, "NULL buffer or negative example");
+    return op_select_clause_updates(d, cfg, step, clause_weights, class_sum, encoded_Y + (int64_t)example * d.K,
+                                    clause_node, class_clause_update, (hipStream_t)stream);
+}
+
+int gtm_update(const gtm_config *cfg, const gtm_graphs *graphs, int32_t example, uint64_t step,
+               uint32_t *ta_state, const int32_t *clause_node, const int32_t *number_of_include_actions,
+               const int32_t *class_clause_update, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (int rc = validate_graphs(cfg, graphs, example, 1)) return rc;
+    if (!ta_state || !clause_node || !number_of_include_actions || !class_clause_update)
+        return fail(GTM_ERR_INVALID, "NULL buffer");
+    uint32_t base = 0;
+    hipError_t e = hipMemcpyAsync(&base, graphs->node_index + example, 4, hipMemcpyDeviceToHost, (hipStream_t)stream);
+    if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+    if (e != hipSuccess) return fail(GTM_ERR_HIP, "reading node index: %s", hipGetErrorString(e));
+    return op_update(d, cfg, step, 0, ta_state, d.LA, clause_node, number_of_include_actions,
+                     graphs->X + (int64_t)base * d.LA, class_clause_update, (hipStream_t)stream);
+}
+
+int gtm_update_message(const gtm_config *cfg, uint64_t step, int32_t bank, uint32_t *message_ta_state,
+                       const int32_t *clause_node, const int32_t *number_of_include_actions,
+                       const uint32_t *clause_X, const int32_t *class_clause_update, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (bank < 1 || bank >= cfg->depth) return fail(GTM_ERR_INVALID, "bank=%d outside 1..%d", bank, cfg->depth - 1);
+    if (!message_ta_state || !clause_node || !number_of_include_actions || !clause_X || !class_clause_update)
+        return fail(GTM_ERR_INVALID, "NULL buffer");
+    return op_update(d, cfg, step, bank, message_ta_state, d.MC, clause_node, number_of_include_actions, clause_X,
+                     class_clause_update, (hipStream_t)stream);
+}
+
+size_t gtm_score_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs, int32_t batch) {
+    Dims d;
+    if (validate(cfg, &d) || batch < 1) return 0;
+    (void)graphs;
+    return carve_score(d, cfg, batch, nullptr).bytes;
+}
+
+int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, int32_t first_graph,
+              int32_t n_graphs, int32_t batch, void *workspace, size_t workspace_bytes, int32_t *class_sum,
+              void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (int rc = validate_graphs(cfg, graphs, first_graph, n_graphs)) return rc;
+    if (int rc = validate_state(cfg, state)) return rc;
+    if (batch < 1) return fail(GTM_ERR_INVALID, "batch=%d", batch);
+    if (!class_sum) return fail(GTM_ERR_INVALID, "class_sum is NULL");
+    ScoreWs w = carve_score(d, cfg, batch, (char *)workspace);
+    if (!workspace || workspace_bytes < w.bytes)
+        return fail(GTM_ERR_INVALID, "workspace of %zu bytes needed, %zu given", w.bytes, workspace_bytes);
+    hipStream_t st = (hipStream_t)stream;
+    for (int done = 0; done < n_graphs; done += batch) {
+        int nb = n_graphs - done < batch ? n_graphs - done : batch;
+        uint32_t *final_bitmap = nullptr;
+        uint32_t *layers[1] = {w.clause_X};
+        if (int rc = run_evaluate(d, cfg, graphs, state, first_graph + done, nb, w.inc_t, w.bitmap_a, w.bitmap_b, layers,
+                                  false, nullptr, class_sum + (int64_t)done * d.K, &final_bitmap, st))
+            return rc;
+    }
+    return GTM_OK;
+}
+
+size_t gtm_fit_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs) {
+    Dims d;
+    if (validate(cfg, &d)) return 0;
+    (void)graphs;
+    return carve_fit(d, cfg, nullptr).bytes;
+}
+
+int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, const int32_t *encoded_Y,
+            int32_t first_example, int32_t n_examples, uint64_t first_step, void *workspace,
+            size_t workspace_bytes, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (int rc = validate_graphs(cfg, graphs, first_example, n_examples)) return rc;
+    if (int rc = validate_state(cfg, state)) return rc;
+    if (!encoded_Y) return fail(GTM_ERR_INVALID, "encoded_Y is NULL");
+    FitWs w = carve_fit(d, cfg, (char *)workspace);
+    if (!workspace || workspace_bytes < w.bytes)
+        return fail(GTM_ERR_INVALID, "workspace of %zu bytes needed, %zu given", w.bytes, workspace_bytes);
+    if (n_examples == 0) return GTM_OK;
+    hipStream_t st = (hipStream_t)stream;
+    // node counts and offsets of the examples, read once
+    std::string host((size_t)n_examples * 8, '\0');
+    uint32_t *h_n = (uint32_t *)host.data();
+    uint32_t *h_base = h_n + n_examples;
+    hipError_t e = hipMemcpyAsync(h_n, graphs->number_of_graph_nodes + first_example, (size_t)n_examples * 4,
+                                  hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess)
+        e = hipMemcpyAsync(h_base, graphs->node_index + first_example, (size_t)n_examples * 4, hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return fail(GTM_ERR_HIP, "reading graph sizes: %s", hipGetErrorString(e));
+
+    for (int i = 0; i < n_examples; ++i) {
+        int ex = first_example + i;
+        uint64_t step = first_step + (uint64_t)i;
+        uint32_t *final_bitmap = nullptr;
+        if (int rc = run_evaluate(d, cfg, graphs, state, ex, 1, w.inc_t, w.bitmap_a, w.bitmap_b, w.clause_X, true,
+                                  w.n_incl, w.class_sum, &final_bitmap, st))
+            return rc;
+        if (int rc = op_select_clause_node(d, cfg, (int)h_n[i], step, final_bitmap, w.clause_node, st)) return rc;
+        if (int rc = op_select_clause_updates(d, cfg, step, state->clause_weights, w.class_sum,
+                                              encoded_Y + (int64_t)ex * d.K, w.clause_node, w.update, st))
+            return rc;
+        if (int rc = op_update(d, cfg, step, 0, state->ta_state, d.LA, w.clause_node, w.n_incl,
+                               graphs->X + (int64_t)h_base[i] * d.LA, w.update, st))
+            return rc;
+        for (int layer = 0; layer < cfg->depth - 1; ++layer)
+            if (int rc = op_update(d, cfg, step, layer + 1, state->message_ta_state[layer], d.MC, w.clause_node,
+                                   w.n_incl, w.clause_X[layer], w.update, st))
+                return rc;
+    }
+    return GTM_OK;
+}
+
+}  // extern "C"

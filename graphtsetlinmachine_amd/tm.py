@@ -1,0 +1,476 @@
+"""Graph Tsetlin Machine models on the HIP hot path.
+
+Host-side mirror of the reference's ``CommonTsetlinMachine`` and its public
+subclasses (GraphTsetlinMachine/tm.py:38-1072): same constructor arguments,
+same ``fit / score / predict / get_state / save / load / ta_action /
+get_weights`` and the same state layouts, so pickles made by ``save`` carry
+the reference's 24 keys with the reference's array shapes and dtypes.
+
+What differs underneath: the per-graph Python loop with a device
+synchronisation after every launch (tm.py:563-747, 786-812) is replaced by
+one C-ABI call per ``fit`` epoch / per ``score`` (``gtm_fit`` / ``gtm_score``),
+torch tensors only own the device memory, and random decisions come from a
+counter-based generator keyed by ``seed`` (argument added at the end of the
+constructor; drawn from NumPy's global generator when omitted, so
+``np.random.seed`` still makes runs repeatable).  ``grid`` and ``block`` are
+accepted and ignored: launch shapes are chosen by the library.
+"""
+
+import ctypes
+import pickle
+import sys
+
+import numpy as np
+import torch
+
+from . import _abi
+
+
+def _device():
+    if not torch.cuda.is_available():
+        raise _abi.GtmError("no GPU visible: the Graph Tsetlin Machine hot path runs on the HIP device only")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _to_device(array):
+    """uint32/int32 NumPy array -> int32 torch tensor on the GPU (same bits)."""
+    a = np.ascontiguousarray(array)
+    if a.dtype == np.uint32:
+        a = a.view(np.int32)
+    return torch.from_numpy(a.reshape(-1)).to(_device())
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() > 0 else ctypes.c_void_p(0)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class _DeviceGraphs:
+    """Device copy of a Graphs object's arrays (tm.py:528-555, 759-784)."""
+
+    def __init__(self, graphs):
+        self.signature = graphs.signature
+        self.number_of_graphs = int(graphs.number_of_graphs)
+        self.max_nodes = int(graphs.max_number_of_graph_nodes)
+        self.tensors = {
+            "X": _to_device(graphs.X),
+            "node_type": _to_device(graphs.node_type),
+            "number_of_graph_node_edges": _to_device(graphs.number_of_graph_node_edges),
+            "edge": _to_device(graphs.edge),
+            "node_index": _to_device(graphs.node_index),
+            "edge_index": _to_device(graphs.edge_index),
+            "number_of_graph_nodes": _to_device(graphs.number_of_graph_nodes),
+        }
+        d = _abi.GraphsDesc()
+        for name, t in self.tensors.items():
+            setattr(d, name, _ptr(t))
+        d.number_of_graphs = self.number_of_graphs
+        d.number_of_node_types = graphs.number_of_node_types()
+        d.max_number_of_graph_nodes = self.max_nodes
+        d.total_nodes = int(graphs.number_of_nodes)
+        d.total_edges = int(graphs.edge.shape[0])
+        self.desc = d
+
+
+class CommonTsetlinMachine:
+    def __init__(
+        self,
+        number_of_clauses,
+        T,
+        s,
+        q=1.0,
+        max_included_literals=None,
+        boost_true_positive_feedback=1,
+        number_of_state_bits=8,
+        depth=1,
+        message_size=256,
+        message_bits=2,
+        double_hashing=False,
+        one_hot_encoding=False,
+        grid=(16 * 13 * 4, 1, 1),
+        block=(128, 1, 1),
+        seed=None,
+    ):
+        self.number_of_clauses = number_of_clauses
+        self.number_of_clause_chunks = (number_of_clauses - 1) // 32 + 1
+        self.T = int(T)
+        self.depth = depth
+        self.s = s if type(s) == tuple else (s,) * self.depth  # tm.py:63-66
+        self.q = q
+        self.max_included_literals = max_included_literals
+        self.boost_true_positive_feedback = boost_true_positive_feedback
+        self.number_of_state_bits = number_of_state_bits
+        self.message_size = message_size
+        self.message_bits = message_bits
+        self.double_hashing = double_hashing
+        self.one_hot_encoding = one_hot_encoding
+        self.grid = grid
+        self.block = block
+
+        self.graphs_signature_train = np.array([])
+        self.graphs_signature_test = np.array([])
+        self.encoded_Y = np.array([])
+        self.ta_state = np.array([])
+        self.message_ta_state = [np.array([])] * (self.depth - 1)
+        self.clause_weights = np.array([])
+
+        # Clause message hypervectors (tm.py:90-106): which message bits a
+        # true clause sets at its neighbours.
+        if self.one_hot_encoding:
+            self.message_bits = 1
+            self.hypervectors = np.zeros((number_of_clauses, 1), dtype=np.uint32)  # filled in _init
+        elif self.double_hashing:
+            from sympy import prevprime
+
+            self.message_bits = 2
+            prime = int(prevprime(self.message_size))
+            ids = np.arange(number_of_clauses, dtype=np.int64)
+            self.hypervectors = np.stack([ids % self.message_size, prime - (ids % prime)], axis=1).astype(np.uint32)
+        else:
+            indexes = np.arange(self.message_size, dtype=np.uint32)
+            self.hypervectors = np.zeros((number_of_clauses, self.message_bits), dtype=np.uint32)
+            for i in range(number_of_clauses):
+                self.hypervectors[i, :] = np.random.choice(indexes, size=(self.message_bits), replace=False)
+
+        if seed is None:
+            seed = int(np.random.randint(0, 2**32, dtype=np.uint64)) | (int(np.random.randint(0, 2**32, dtype=np.uint64)) << 32)
+        self.seed = int(seed)
+        self.step = 0  # training examples seen so far; addresses the random draws
+
+        self.initialized = False
+        self._train_graphs = None
+        self._test_graphs = None
+        self._workspace = None
+        self._encoded_Y_gpu = None
+
+    # ------------------------------------------------------------ sizing
+
+    def _init(self, graphs):
+        """tm.py:414-435."""
+        if self.one_hot_encoding:
+            n_edge_types = len(graphs.edge_type_id)
+            self.message_size = self.number_of_clauses * max(1, n_edge_types)
+            self.hypervectors[:, 0] = np.arange(self.number_of_clauses) * n_edge_types
+        self.number_of_features = graphs.hypervector_size
+        self.number_of_literals = self.number_of_features * 2
+        self.number_of_ta_chunks = int((self.number_of_literals - 1) // 32 + 1)
+        self.number_of_message_features = self.message_size
+        self.number_of_message_literals = self.number_of_message_features * 2
+        self.number_of_message_chunks = int((self.number_of_message_literals - 1) // 32 + 1)
+        if self.max_included_literals is None:
+            self.max_included_literals = self.number_of_literals
+        self.max_number_of_graph_nodes = graphs.max_number_of_graph_nodes
+        self._allocate()
+        self.initialized = True
+
+    def _allocate(self):
+        """tm.py:110-124."""
+        dev = _device()
+        C, B = self.number_of_clauses, self.number_of_state_bits
+        self.ta_state_gpu = torch.empty(C * self.number_of_ta_chunks * B, dtype=torch.int32, device=dev)
+        self.message_ta_state_gpu = [
+            torch.empty(C * self.number_of_message_chunks * B, dtype=torch.int32, device=dev)
+            for _ in range(self.depth - 1)
+        ]
+        self.clause_weights_gpu = torch.empty(self.number_of_outputs * C, dtype=torch.int32, device=dev)
+        self.hypervectors_gpu = _to_device(self.hypervectors)
+        st = _abi.State()
+        st.ta_state = _ptr(self.ta_state_gpu)
+        for i, t in enumerate(self.message_ta_state_gpu):
+            st.message_ta_state[i] = t.data_ptr()
+        st.clause_weights = _ptr(self.clause_weights_gpu)
+        st.hypervectors = _ptr(self.hypervectors_gpu)
+        self._state = st
+
+    def _config(self, max_nodes):
+        return _abi.make_config(
+            classes=self.number_of_outputs,
+            clauses=self.number_of_clauses,
+            literals=self.number_of_literals,
+            state_bits=self.number_of_state_bits,
+            boost_true_positive_feedback=self.boost_true_positive_feedback,
+            threshold=self.T,
+            q=self.q,
+            max_included_literals=self.max_included_literals,
+            negative_clauses=self.negative_clauses,
+            max_nodes=int(max_nodes),
+            message_size=self.message_size,
+            message_bits=self.message_bits,
+            depth=self.depth,
+            s=self.s,
+            seed=self.seed,
+        )
+
+    def _workspace_of(self, nbytes):
+        if self._workspace is None or self._workspace.numel() < nbytes:
+            self._workspace = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=_device())
+        return self._workspace
+
+    # ------------------------------------------------------------- training
+
+    def _prepare(self, cfg, with_message_banks):
+        _abi.call("gtm_prepare", ctypes.byref(cfg), self.step, _ptr(self.ta_state_gpu), _ptr(self.clause_weights_gpu), _stream())
+        if with_message_banks:
+            for t in self.message_ta_state_gpu:
+                _abi.call("gtm_prepare_message_ta_state", ctypes.byref(cfg), _ptr(t), _stream())
+
+    def _init_fit(self, graphs, encoded_Y, incremental):
+        """tm.py:515-561."""
+        if not self.initialized:
+            self._init(graphs)
+            self._prepare(self._config(graphs.max_number_of_graph_nodes), True)
+        elif incremental == False:  # noqa: E712  (the reference re-initialises layer 0 only, tm.py:524-526)
+            self._prepare(self._config(graphs.max_number_of_graph_nodes), False)
+        if self._train_graphs is None or not np.array_equal(self.graphs_signature_train, graphs.signature):
+            self.graphs_signature_train = graphs.signature
+            self._train_graphs = _DeviceGraphs(graphs)
+        if self._encoded_Y_gpu is None or not np.array_equal(self.encoded_Y, encoded_Y):
+            self.encoded_Y = encoded_Y
+            self._encoded_Y_gpu = _to_device(np.ascontiguousarray(encoded_Y, dtype=np.int32))
+
+    def _fit(self, graphs, encoded_Y, epochs=100, incremental=False):
+        """tm.py:664-752; each epoch is one gtm_fit call."""
+        self._init_fit(graphs, encoded_Y, incremental)
+        dg = self._train_graphs
+        cfg = self._config(max(dg.max_nodes, 1))
+        need = _abi.lib.gtm_fit_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc))
+        ws = self._workspace_of(need)
+        for _ in range(epochs):
+            _abi.call(
+                "gtm_fit", ctypes.byref(cfg), ctypes.byref(dg.desc), ctypes.byref(self._state),
+                _ptr(self._encoded_Y_gpu), 0, dg.number_of_graphs, self.step, _ptr(ws), ws.numel(), _stream(),
+            )
+            self.step += dg.number_of_graphs
+        torch.cuda.current_stream().synchronize()
+        self.ta_state = np.array([])
+        self.clause_weights = np.array([])
+
+    # ------------------------------------------------------------ inference
+
+    def _score_init(self, graphs):
+        """tm.py:754-784."""
+        if not self.initialized:
+            print("Error: Model not trained.")
+            sys.exit(-1)
+        if self._train_graphs is not None and np.array_equal(self.graphs_signature_train, graphs.signature):
+            return self._train_graphs  # same data already resident
+        if self._test_graphs is None or not np.array_equal(self.graphs_signature_test, graphs.signature):
+            self.graphs_signature_test = graphs.signature
+            self._test_graphs = _DeviceGraphs(graphs)
+        return self._test_graphs
+
+    def _score(self, graphs, batch=None):
+        """tm.py:786-812 as one gtm_score call."""
+        dg = self._score_init(graphs)
+        cfg = self._config(max(dg.max_nodes, 1))
+        n = dg.number_of_graphs
+        if batch is None:
+            per_graph = max(1, _abi.lib.gtm_score_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc), 1))
+            batch = int(max(1, min(n, (1 << 30) // per_graph, 1 << 16)))
+        need = _abi.lib.gtm_score_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc), batch)
+        ws = self._workspace_of(need)
+        out = torch.empty(n * self.number_of_outputs, dtype=torch.int32, device=_device())
+        _abi.call(
+            "gtm_score", ctypes.byref(cfg), ctypes.byref(dg.desc), ctypes.byref(self._state), 0, n, batch,
+            _ptr(ws), ws.numel(), _ptr(out), _stream(),
+        )
+        return out.cpu().numpy().reshape(n, self.number_of_outputs)
+
+    # ------------------------------------------------------------- state I/O
+
+    def _download(self):
+        C, B = self.number_of_clauses, self.number_of_state_bits
+        self.ta_state = self.ta_state_gpu.cpu().numpy().view(np.uint32).reshape(C * self.number_of_ta_chunks * B)
+        self.message_ta_state = [t.cpu().numpy().view(np.uint32) for t in self.message_ta_state_gpu]
+        self.clause_weights = self.clause_weights_gpu.cpu().numpy()
+
+    def ta_action(self, depth, clause, ta):
+        """tm.py:126-142: is literal `ta` of `clause` included at layer `depth`?"""
+        self._download()
+        B = self.number_of_state_bits
+        if depth == 0:
+            bank = self.ta_state.reshape(self.number_of_clauses, self.number_of_ta_chunks, B)
+        else:
+            bank = self.message_ta_state[depth - 1].reshape(self.number_of_clauses, self.number_of_message_chunks, B)
+        return (bank[clause, ta // 32, B - 1] & (1 << (ta % 32))) > 0
+
+    def get_weights(self):
+        """tm.py:207-211."""
+        if np.array_equal(self.clause_weights, np.array([])):
+            self.clause_weights = self.clause_weights_gpu.cpu().numpy()
+        return self.clause_weights.reshape((self.number_of_outputs, self.number_of_clauses))
+
+    def get_state(self):
+        """tm.py:281-287: the 10-tuple, always read fresh from the device."""
+        self._download()
+        return (
+            self.ta_state, self.clause_weights, self.number_of_outputs, self.number_of_clauses,
+            self.number_of_literals, self.depth, self.number_of_state_bits, self.number_of_ta_chunks,
+            self.min_y, self.max_y,
+        )
+
+    def set_state(self, state):
+        """tm.py:289-310.  Restores the layer-0 bank and the weights into an
+        initialised model of the same shape (the reference's version leaves
+        message banks and kernels unset)."""
+        (ta_state, weights, self.number_of_outputs, self.number_of_clauses, self.number_of_literals,
+         self.depth, self.number_of_state_bits, self.number_of_ta_chunks, self.min_y, self.max_y) = state
+        if not self.initialized:
+            raise _abi.GtmError("set_state needs an initialised model; use load() to build one from a saved state")
+        self.ta_state_gpu.copy_(_to_device(np.asarray(ta_state, dtype=np.uint32)))
+        self.clause_weights_gpu.copy_(_to_device(np.asarray(weights, dtype=np.int32)))
+        self.graphs_signature_train = np.array([])
+        self.graphs_signature_test = np.array([])
+        self._train_graphs = self._test_graphs = None
+        self.encoded_Y = np.array([])
+        self._encoded_Y_gpu = None
+        self.ta_state = np.array([])
+        self.clause_weights = np.array([])
+
+    def save(self, fname=""):
+        """tm.py:312-362: the reference's 24 keys plus the generator position."""
+        self._download()
+        state_dict = {
+            "ta_state": self.ta_state,
+            "message_ta_state": self.message_ta_state,
+            "clause_weights": self.clause_weights,
+            "hypervectors": self.hypervectors,
+            "number_of_outputs": self.number_of_outputs,
+            "number_of_literals": self.number_of_literals,
+            "number_of_message_literals": self.number_of_message_literals,
+            "min_y": self.min_y,
+            "max_y": self.max_y,
+            "negative_clauses": self.negative_clauses,
+            "max_number_of_graph_nodes": self.max_number_of_graph_nodes,
+            "number_of_clauses": self.number_of_clauses,
+            "T": self.T,
+            "s": self.s,
+            "q": self.q,
+            "max_included_literals": self.max_included_literals,
+            "boost_true_positive_feedback": self.boost_true_positive_feedback,
+            "number_of_state_bits": self.number_of_state_bits,
+            "depth": self.depth,
+            "message_size": self.message_size,
+            "message_bits": self.message_bits,
+            "double_hashing": self.double_hashing,
+            "one_hot_encoding": self.one_hot_encoding,
+            # not in the reference: where the counter-based generator stands
+            "rng_seed": self.seed,
+            "rng_step": self.step,
+        }
+        if len(fname) > 0:
+            print(f"Saving model to {fname}.")
+            with open(fname, "wb") as f:
+                pickle.dump(state_dict, f)
+        return state_dict
+
+    def load(self, state_dict={}, fname=""):
+        """tm.py:364-412."""
+        if len(fname) == 0 and len(state_dict) == 0:
+            print("Error: No file or state_dict provided. Pass either a file name or a state_dict.")
+            return
+        if len(fname) > 0:
+            print(f"Loading model from {fname}.")
+            with open(fname, "rb") as f:
+                state_dict = pickle.load(f)
+        self.ta_state = state_dict["ta_state"]
+        self.message_ta_state = state_dict["message_ta_state"]
+        self.clause_weights = state_dict["clause_weights"]
+        self.hypervectors = state_dict["hypervectors"]
+        self.number_of_outputs = state_dict["number_of_outputs"]
+        self.number_of_literals = state_dict["number_of_literals"]
+        self.number_of_message_literals = state_dict["number_of_message_literals"]
+        self.min_y = state_dict["min_y"]
+        self.max_y = state_dict["max_y"]
+        self.negative_clauses = state_dict["negative_clauses"]
+        self.max_number_of_graph_nodes = state_dict["max_number_of_graph_nodes"]
+        self.message_size = state_dict["message_size"]
+        self.seed = int(state_dict.get("rng_seed", self.seed))
+        self.step = int(state_dict.get("rng_step", 0))
+
+        self.number_of_features = self.number_of_literals // 2
+        self.number_of_ta_chunks = int((self.number_of_literals - 1) // 32 + 1)
+        self.number_of_message_features = self.number_of_message_literals // 2
+        self.number_of_message_chunks = int((self.number_of_message_literals - 1) // 32 + 1)
+        if self.max_included_literals is None:
+            self.max_included_literals = self.number_of_literals
+
+        self._allocate()
+        self.ta_state_gpu.copy_(_to_device(np.asarray(self.ta_state, dtype=np.uint32)))
+        for t, host in zip(self.message_ta_state_gpu, self.message_ta_state):
+            t.copy_(_to_device(np.asarray(host, dtype=np.uint32)))
+        self.clause_weights_gpu.copy_(_to_device(np.asarray(self.clause_weights, dtype=np.int32)))
+        self._train_graphs = self._test_graphs = None
+        self.graphs_signature_train = np.array([])
+        self.graphs_signature_test = np.array([])
+        self.initialized = True
+
+
+class MultiClassGraphTsetlinMachine(CommonTsetlinMachine):
+    """tm.py:903-959."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.negative_clauses = 1
+
+    def fit(self, graphs, Y, epochs=100, incremental=False):
+        Y = np.asarray(Y)
+        self.number_of_outputs = int(np.max(Y) + 1)
+        self.max_y = None
+        self.min_y = None
+        encoded_Y = np.empty((Y.shape[0], self.number_of_outputs), dtype=np.int32)
+        for i in range(self.number_of_outputs):
+            encoded_Y[:, i] = np.where(Y == i, self.T, -self.T)
+        self._fit(graphs, encoded_Y, epochs=epochs, incremental=incremental)
+
+    def score(self, graphs):
+        return self._score(graphs)
+
+    def predict(self, graphs):
+        return np.argmax(self.score(graphs), axis=1)
+
+
+class MultiOutputGraphTsetlinMachine(CommonTsetlinMachine):
+    """tm.py:961-1017."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.negative_clauses = 1
+
+    def fit(self, graphs, Y, epochs=100, incremental=False):
+        Y = np.asarray(Y)
+        self.number_of_outputs = Y.shape[1]
+        self.max_y = None
+        self.min_y = None
+        encoded_Y = np.where(Y == 1, self.T, -self.T).astype(np.int32)
+        self._fit(graphs, encoded_Y, epochs=epochs, incremental=incremental)
+
+    def score(self, graphs):
+        return self._score(graphs)
+
+    def predict(self, graphs):
+        return (self.score(graphs) >= 0).astype(np.uint32)
+
+
+class GraphTsetlinMachine(CommonTsetlinMachine):
+    """tm.py:1019-1072."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.negative_clauses = 1
+
+    def fit(self, graphs, Y, epochs=100, incremental=False):
+        self.number_of_outputs = 1
+        self.max_y = None
+        self.min_y = None
+        encoded_Y = np.where(np.asarray(Y) == 1, self.T, -self.T).astype(np.int32).reshape(-1, 1)
+        self._fit(graphs, encoded_Y, epochs=epochs, incremental=incremental)
+
+    def score(self, graphs):
+        return self._score(graphs)[:, 0]
+
+    def predict(self, graphs):
+        return self.score(graphs) >= 0

@@ -1,0 +1,182 @@
+/*
+ * C ABI of the MI355X Graph Tsetlin Machine hot path (libgtm_hip.so).
+ *
+ * The reference has no C interface: its operator boundary is PyCUDA's
+ * `fn.prepared_call(grid, block, *args)` on kernels JIT-compiled from
+ * GraphTsetlinMachine/kernels.py with the model's hyper-parameters baked in as
+ * #defines (tm.py:437-513).  Each entry point below replaces one of those
+ * prepared kernels (or one of the driver loops that chain them) and cites it.
+ * The #defines travel in `gtm_config`; grid/block shapes are chosen inside.
+ *
+ * Conventions
+ *  - every pointer inside the structs and in the argument lists is a DEVICE
+ *    pointer owned by the caller (the Python side takes them from torch
+ *    tensors); the library never allocates or frees device memory;
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *    all work is enqueued on it and no entry point synchronises;
+ *  - the return value is GTM_OK or an error code; gtm_last_error() gives the
+ *    text for the calling thread.  No C++ exception crosses the boundary;
+ *  - memory layouts are the reference's: X uint32 [nodes][LA_CHUNKS];
+ *    ta_state uint32 [CLAUSES][chunks][STATE_BITS] (bit-sliced, top plane =
+ *    include mask); clause_weights int32 [CLASSES][CLAUSES]; clause/node
+ *    bitmaps uint32 [CLAUSES][NODE_CHUNKS] per graph; packed messages uint32
+ *    [max_nodes][MESSAGE_CHUNKS] per graph;
+ *  - random decisions come from Philox4x32-10 keyed by `seed` and addressed by
+ *    (clause, class or word, training step, purpose); they do not depend on
+ *    the launch shape.
+ */
+#ifndef GTM_ABI_H
+#define GTM_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GTM_ABI_VERSION 1
+#define GTM_MAX_DEPTH 8
+
+#define GTM_OK 0
+#define GTM_ERR_INVALID 1 /* bad argument or configuration */
+#define GTM_ERR_HIP 2     /* a HIP call or kernel launch failed */
+
+/* The macros injected at tm.py:438-464, plus depth, s and the RNG seed. */
+typedef struct gtm_config {
+    int32_t classes;                      /* CLASSES */
+    int32_t clauses;                      /* CLAUSES */
+    int32_t literals;                     /* LITERALS = 2 * hypervector_size */
+    int32_t state_bits;                   /* STATE_BITS (1..32) */
+    int32_t boost_true_positive_feedback; /* BOOST_TRUE_POSITIVE_FEEDBACK */
+    int32_t threshold;                    /* THRESHOLD (T) */
+    int32_t max_included_literals;        /* MAX_INCLUDED_LITERALS */
+    int32_t negative_clauses;             /* NEGATIVE_CLAUSES */
+    int32_t max_nodes;                    /* MAX_NODES: bitmap row stride = ceil(max_nodes/32) words */
+    int32_t message_size;                 /* MESSAGE_SIZE */
+    int32_t message_bits;                 /* MESSAGE_BITS */
+    int32_t depth;                        /* number of layers (tm.py:62) */
+    double q;                             /* Q */
+    double s[GTM_MAX_DEPTH];              /* s per layer (tm.py:63-66) */
+    uint64_t seed;                        /* Philox key */
+} gtm_config;
+
+/* Device copies of the arrays of a Graphs object (graphs.py:38,101-112,128-129). */
+typedef struct gtm_graphs {
+    const uint32_t *X;                          /* [total_nodes][LA_CHUNKS] */
+    const uint32_t *node_type;                  /* [total_nodes] */
+    const uint32_t *number_of_graph_node_edges; /* [total_nodes] */
+    const uint32_t *edge;                       /* [total_edges][2] = (destination, type) */
+    const uint32_t *node_index;                 /* [number_of_graphs] */
+    const uint32_t *edge_index;                 /* [total_nodes] */
+    const uint32_t *number_of_graph_nodes;      /* [number_of_graphs] */
+    int32_t number_of_graphs;
+    int32_t number_of_node_types;      /* Graphs.number_of_node_types() */
+    int32_t max_number_of_graph_nodes; /* must be <= gtm_config.max_nodes */
+    int32_t reserved;
+    int64_t total_nodes;
+    int64_t total_edges;
+} gtm_graphs;
+
+/* The model's device buffers (tm.py:110-124). */
+typedef struct gtm_state {
+    uint32_t *ta_state;                            /* [CLAUSES][LA_CHUNKS][STATE_BITS] */
+    uint32_t *message_ta_state[GTM_MAX_DEPTH - 1]; /* [CLAUSES][MESSAGE_CHUNKS][STATE_BITS] each */
+    int32_t *clause_weights;                       /* [CLASSES][CLAUSES] */
+    const uint32_t *hypervectors;                  /* [CLAUSES][MESSAGE_BITS] */
+} gtm_state;
+
+int gtm_abi_version(void);
+const char *gtm_last_error(void);
+
+/* ---- one entry point per reference kernel ------------------------------ */
+
+/* `prepare` (kernels.py:638-664; called at tm.py:518,525): TA bank to state
+ * 2^(B-1)-1, weights to random +-1 (NEGATIVE_CLAUSES == 1) or 1. */
+int gtm_prepare(const gtm_config *cfg, uint64_t step, uint32_t *ta_state, int32_t *clause_weights, void *stream);
+
+/* `prepare_message_ta_state` (kernels.py:622-636; tm.py:521). */
+int gtm_prepare_message_ta_state(const gtm_config *cfg, uint32_t *message_ta_state, void *stream);
+
+/* `calculate_messages` (kernels.py:407-468; tm.py:582-593) for graphs
+ * [first_graph, first_graph + n_graphs): clause_node_output is
+ * [n_graphs][CLAUSES][NODE_CHUNKS]; number_of_include_actions [CLAUSES] may
+ * be NULL.  include_plane is caller-provided scratch of LA_CHUNKS * CLAUSES
+ * words; it receives the bank's include masks word-major ([chunk][clause]),
+ * the form the evaluation kernel reads coalesced. */
+int gtm_calculate_messages(const gtm_config *cfg, const gtm_graphs *graphs, int32_t first_graph, int32_t n_graphs,
+                           const uint32_t *ta_state, uint32_t *include_plane, uint32_t *clause_node_output,
+                           int32_t *number_of_include_actions, void *stream);
+
+/* `prepare_messages` + `exchange_messages` + `encode_messages`
+ * (kernels.py:532-615; tm.py:599-630) fused: writes the packed message
+ * literals clause_X [n_graphs][max_nodes][MESSAGE_CHUNKS] directly, without
+ * the one-int-per-literal scratch. */
+int gtm_exchange_messages(const gtm_config *cfg, const gtm_graphs *graphs, int32_t first_graph, int32_t n_graphs,
+                          const uint32_t *hypervectors, const uint32_t *clause_node_output, uint32_t *clause_X,
+                          void *stream);
+
+/* `calculate_messages_conditional` (kernels.py:470-530; tm.py:633-645).
+ * number_of_include_actions (may be NULL) is incremented; include_plane is
+ * scratch of MESSAGE_CHUNKS * CLAUSES words as above. */
+int gtm_calculate_messages_conditional(const gtm_config *cfg, const gtm_graphs *graphs, int32_t first_graph,
+                                       int32_t n_graphs, const uint32_t *message_ta_state, uint32_t *include_plane,
+                                       const uint32_t *clause_node_output_condition, uint32_t *clause_node_output,
+                                       int32_t *number_of_include_actions, const uint32_t *clause_X, void *stream);
+
+/* `evaluate` (kernels.py:279-317; tm.py:652-659) including the zeroing of
+ * class_sum that the driver does from the host (tm.py:578-579): class_sum is
+ * [n_graphs][CLASSES], overwritten. */
+int gtm_evaluate(const gtm_config *cfg, const gtm_graphs *graphs, int32_t first_graph, int32_t n_graphs,
+                 const uint32_t *clause_node_output, const int32_t *clause_weights, int32_t *class_sum,
+                 void *stream);
+
+/* `select_clause_node` (kernels.py:319-354; tm.py:693-700) for graph `example`. */
+int gtm_select_clause_node(const gtm_config *cfg, const gtm_graphs *graphs, int32_t example, uint64_t step,
+                           const uint32_t *clause_node_output, int32_t *clause_node, void *stream);
+
+/* `select_clause_updates` (kernels.py:356-405; tm.py:704-714). encoded_Y is
+ * [number_of_graphs][CLASSES]; class_clause_update [CLASSES][CLAUSES]. */
+int gtm_select_clause_updates(const gtm_config *cfg, uint64_t step, int32_t *clause_weights,
+                              const int32_t *class_sum, const int32_t *encoded_Y, int32_t example,
+                              const int32_t *clause_node, int32_t *class_clause_update, void *stream);
+
+/* `update` (kernels.py:213-242; tm.py:718-730): Type I/II feedback on the
+ * layer-0 bank with s = cfg->s[0]. */
+int gtm_update(const gtm_config *cfg, const gtm_graphs *graphs, int32_t example, uint64_t step,
+               uint32_t *ta_state, const int32_t *clause_node, const int32_t *number_of_include_actions,
+               const int32_t *class_clause_update, void *stream);
+
+/* `update_message` (kernels.py:185-211; tm.py:735-746) on message bank
+ * `bank` (1 .. depth-1) with s = cfg->s[bank]; clause_X is that layer's
+ * [max_nodes][MESSAGE_CHUNKS] block for the example. */
+int gtm_update_message(const gtm_config *cfg, uint64_t step, int32_t bank, uint32_t *message_ta_state,
+                       const int32_t *clause_node, const int32_t *number_of_include_actions,
+                       const uint32_t *clause_X, const int32_t *class_clause_update, void *stream);
+
+/* ---- the driver loops --------------------------------------------------- */
+
+/* Scratch needed by gtm_score for sub-batches of `batch` graphs. */
+size_t gtm_score_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs, int32_t batch);
+
+/* `_score` (tm.py:786-812): class sums [n_graphs][CLASSES] of graphs
+ * [first_graph, first_graph + n_graphs), evaluated `batch` graphs at a time. */
+int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, int32_t first_graph,
+              int32_t n_graphs, int32_t batch, void *workspace, size_t workspace_bytes, int32_t *class_sum,
+              void *stream);
+
+/* Scratch needed by gtm_fit. */
+size_t gtm_fit_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs);
+
+/* The inner loop of `_fit` (tm.py:669-747) over examples
+ * [first_example, first_example + n_examples), strictly in order (online
+ * learning: example e+1 sees the state left by e).  Example i uses training
+ * step first_step + i for its random draws. */
+int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, const int32_t *encoded_Y,
+            int32_t first_example, int32_t n_examples, uint64_t first_step, void *workspace,
+            size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GTM_ABI_H */

@@ -321,7 +321,8 @@ def build_messages(cfg, number_of_nodes, hypervectors, bitmap, n_edges, edge):
 
 def clause_outputs(cfg, bitmap, number_of_nodes):
     """1 where the clause is true at some node (kernels.py:297-308)."""
-    n_chunks = (number_of_nodes - 1) // 32 + 1
+    # C division: an empty graph still reads one (unmasked) chunk, kernels.py:289-295
+    n_chunks = 1 if number_of_nodes == 0 else (number_of_nodes - 1) // 32 + 1
     words = bitmap[:, :n_chunks].copy()
     words[:, -1] &= U32(_node_filter(number_of_nodes))
     return (words != 0).any(axis=1)
@@ -345,6 +346,8 @@ def select_clause_node(cfg, seed, step, bitmap, number_of_nodes):
     The reference takes ``list[curand % len]``; here the index is
     ``(r * len) >> 32`` with ``r`` the first Philox word at counter
     ``(clause, 0, step, TAG_CLAUSE_NODE)``."""
+    if number_of_nodes == 0:
+        return np.full(cfg.clauses, -1, dtype=np.int32)
     truth = _unpack_bitmap(bitmap, number_of_nodes)
     count = truth.sum(axis=1).astype(np.int64)
     k0, k1 = _key(seed)

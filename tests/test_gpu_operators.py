@@ -1,0 +1,211 @@
+"""HIP path vs the CPU oracle, one operator at a time, through the C ABI.
+
+Bar: bit-exact (everything here is integer / bitwise work)."""
+
+import copy
+
+import numpy as np
+import pytest
+
+from oracle import gtm_oracle as o
+from tests import helpers
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    # seed, graphs kwargs, model kwargs
+    dict(seed=1, g=dict(n_graphs=5, max_nodes=40, hv_size=20), m=dict(classes=3, clauses=70, depth=1)),
+    dict(seed=2, g=dict(n_graphs=4, max_nodes=70, hv_size=16, node_types=("a", "b"), edge_types=("x", "y", "z")),
+         m=dict(classes=2, clauses=33, depth=2, message_size=37)),
+    dict(seed=3, g=dict(n_graphs=3, max_nodes=32, hv_size=64, min_nodes=32), m=dict(classes=4, clauses=300, depth=3,
+                                                                                  message_size=64, message_bits=3)),
+    dict(seed=4, g=dict(n_graphs=6, max_nodes=3, hv_size=300, hv_bits=3, n_symbols=9),
+         m=dict(classes=5, clauses=20, depth=2, message_size=16, message_bits=1, state_bits=4)),
+]
+
+
+def build(shape, include_density=0.03):
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    m = dict(shape["m"])
+    depth = m.pop("depth")
+    cfg = helpers.oracle_config(graphs, **m, depth=depth)
+    model = helpers.random_model(shape["seed"], cfg, depth, s=(1.0, 3.0, 2.0)[:depth], include_density=include_density)
+    return graphs, cfg, model
+
+
+def graph_slices(graphs, e):
+    n = int(graphs.number_of_graph_nodes[e])
+    base = int(graphs.node_index[e])
+    n_edges = graphs.number_of_graph_node_edges[base:base + n]
+    e0 = int(graphs.edge_index[base]) if n else 0
+    edge = graphs.edge[e0:e0 + int(n_edges.astype(np.int64).sum())]
+    return n, base, n_edges, edge
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "shape%d" % s["seed"])
+@pytest.mark.parametrize("density", [0.0, 0.03, 0.5])
+def test_inference_operators(shape, density):
+    from tests.gpu_harness import Device, host
+
+    graphs, cfg, model = build(shape, density)
+    dev = Device(model, graphs)
+    G = graphs.number_of_graphs
+    bitmap, n_incl = dev.calculate_messages(0, G)
+    h_bitmap = host(bitmap, np.uint32, (G, cfg.clauses, cfg.node_chunks))
+    h_incl = host(n_incl, np.int32, (cfg.clauses,))
+    expect = []
+    for e in range(G):
+        n, base, n_edges, edge = graph_slices(graphs, e)
+        bm, incl = o.calculate_messages(cfg, model.ta_state, graphs.node_type[base:base + n],
+                                        graphs.number_of_node_types(), n, graphs.X[base:base + n])
+        expect.append(bm)
+        assert np.array_equal(h_bitmap[e], bm), "calculate_messages graph %d" % e
+    assert np.array_equal(h_incl, incl)
+
+    cur, cur_host = bitmap, np.stack(expect)
+    for layer in range(model.depth - 1):
+        cx = dev.exchange_messages(0, G, cur)
+        h_cx = host(cx, np.uint32, (G, cfg.max_nodes, cfg.message_chunks))
+        nxt = dev.calculate_messages_conditional(0, G, layer, cur, n_incl, cx)
+        h_nxt = host(nxt, np.uint32, (G, cfg.clauses, cfg.node_chunks))
+        new_host = []
+        for e in range(G):
+            n, base, n_edges, edge = graph_slices(graphs, e)
+            want_cx = o.build_messages(cfg, n, model.hypervectors, cur_host[e], n_edges, edge)
+            assert np.array_equal(h_cx[e, :n], want_cx), "messages layer %d graph %d" % (layer, e)
+            bm, incl = o.calculate_messages_conditional(
+                cfg, model.message_ta_state[layer], graphs.node_type[base:base + n], graphs.number_of_node_types(),
+                n, cur_host[e], np.zeros(cfg.clauses, dtype=np.int32), want_cx)
+            assert np.array_equal(h_nxt[e], bm), "conditional layer %d graph %d" % (layer, e)
+            new_host.append(bm)
+        cur, cur_host = nxt, np.stack(new_host)
+
+    sums = host(dev.evaluate(0, G, cur), np.int32, (G, cfg.classes))
+    for e in range(G):
+        n = int(graphs.number_of_graph_nodes[e])
+        assert np.array_equal(sums[e], o.evaluate(cfg, cur_host[e], model.clause_weights, n))
+    # the whole driver loop, at two batch sizes
+    want = o.score(model, graphs)
+    assert np.array_equal(dev.score(0, G, G), want)
+    assert np.array_equal(dev.score(1, G - 1, 2), want[1:])
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "shape%d" % s["seed"])
+def test_include_counts_accumulate(shape):
+    from tests.gpu_harness import Device, host
+
+    graphs, cfg, model = build(shape, 0.1)
+    if model.depth < 2:
+        pytest.skip("needs a message layer")
+    dev = Device(model, graphs)
+    bitmap, n_incl = dev.calculate_messages(0, 1)
+    cx = dev.exchange_messages(0, 1, bitmap)
+    dev.calculate_messages_conditional(0, 1, 0, bitmap, n_incl, cx)
+    inc0 = o._popcount32(o._include_plane(model.ta_state, cfg.state_bits, cfg.filter)).sum(axis=1)
+    inc1 = o._popcount32(o._include_plane(model.message_ta_state[0], cfg.state_bits, cfg.message_filter)).sum(axis=1)
+    assert np.array_equal(host(n_incl, np.int32, (cfg.clauses,)), inc0 + inc1)
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "shape%d" % s["seed"])
+@pytest.mark.parametrize("boost,max_included", [(1, None), (0, None), (1, 3)])
+def test_training_operators(shape, boost, max_included):
+    from tests.gpu_harness import Device, host
+    from graphtsetlinmachine_amd.tm import _to_device
+
+    graphs, cfg, model = build(shape, 0.03)
+    cfg.boost_true_positive_feedback = boost
+    if max_included is not None:
+        cfg.max_included_literals = max_included
+    dev = Device(model, graphs)
+    rng = np.random.default_rng(shape["seed"])
+    Y = o.encode_labels(rng.integers(0, cfg.classes, size=graphs.number_of_graphs), cfg.classes, cfg.threshold)
+    for e in range(graphs.number_of_graphs):
+        step = 1000 + e
+        n, base, n_edges, edge = graph_slices(graphs, e)
+        ref = copy.deepcopy(model)
+        bitmap, class_sum, n_incl, layers = o.evaluate_graph(ref, graphs, e)
+        d_bitmap = _to_device(bitmap)
+
+        want_node = o.select_clause_node(cfg, model.seed, step, bitmap, n)
+        got_node = dev.select_clause_node(e, step, d_bitmap)
+        assert np.array_equal(host(got_node, np.int32, (cfg.clauses,)), want_node)
+
+        weights = model.clause_weights.copy()
+        want_upd = o.select_clause_updates(cfg, model.seed, step, weights, class_sum, Y[e], want_node)
+        got_upd = dev.select_clause_updates(step, _to_device(class_sum), Y, e, got_node)
+        assert np.array_equal(host(got_upd, np.int32, (cfg.classes, cfg.clauses)), want_upd)
+        assert np.array_equal(host(dev.weights, np.int32, weights.shape), weights)
+
+        d_incl = _to_device(n_incl)
+        ta = model.ta_state.copy()
+        o.update(cfg, model.seed, step, model.s[0], ta, want_node, n_incl, graphs.X[base:base + n], want_upd)
+        dev.update(e, step, got_node, d_incl, got_upd)
+        got_ta, got_banks, _ = dev.download()
+        assert np.array_equal(got_ta, ta), "update graph %d" % e
+        for layer in range(model.depth - 1):
+            bank = model.message_ta_state[layer].copy()
+            o.update_message(cfg, model.seed, step, layer + 1, model.s[layer + 1], bank, want_node, n_incl,
+                             layers[layer], want_upd)
+            cx = np.zeros((cfg.max_nodes, cfg.message_chunks), dtype=np.uint32)
+            cx[:n] = layers[layer]
+            dev.update_message(step, layer + 1, got_node, d_incl, _to_device(cx), got_upd)
+            assert np.array_equal(dev.download()[1][layer], bank), "update_message graph %d layer %d" % (e, layer)
+            model.message_ta_state[layer] = bank
+        model.ta_state = ta
+        model.clause_weights = weights
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "shape%d" % s["seed"])
+def test_fit_trajectory_bit_exact(shape):
+    """gtm_fit over a few epochs leaves exactly the oracle's automata and weights."""
+    from tests.gpu_harness import Device
+
+    graphs, cfg, model = build(shape, 0.02)
+    dev = Device(model, graphs)
+    rng = np.random.default_rng(shape["seed"] + 100)
+    Y = o.encode_labels(rng.integers(0, cfg.classes, size=graphs.number_of_graphs), cfg.classes, cfg.threshold)
+    G = graphs.number_of_graphs
+    for epoch in range(3):
+        o.fit(model, graphs, Y)
+        dev.fit(Y, 0, G, epoch * G)
+        ta, banks, w = dev.download()
+        assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
+        assert np.array_equal(ta, model.ta_state), "layer-0 automata after epoch %d" % epoch
+        for layer in range(model.depth - 1):
+            assert np.array_equal(banks[layer], model.message_ta_state[layer]), "bank %d epoch %d" % (layer, epoch)
+    assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
+
+
+def test_prepare_matches_oracle():
+    import ctypes
+    from tests.gpu_harness import abi_config, dev_u32, host
+    from graphtsetlinmachine_amd import _abi
+    from graphtsetlinmachine_amd.tm import _ptr, _stream
+
+    cfg = o.Config(classes=3, clauses=77, literals=40, state_bits=6, max_nodes=5, message_size=19)
+    acfg = abi_config(cfg, 2, 1.0, seed=0xDEADBEEFCAFE)
+    ta = dev_u32((cfg.clauses, cfg.la_chunks, cfg.state_bits))
+    w = dev_u32((cfg.classes, cfg.clauses))
+    bank = dev_u32((cfg.clauses, cfg.message_chunks, cfg.state_bits))
+    _abi.call("gtm_prepare", ctypes.byref(acfg), 5, _ptr(ta), _ptr(w), _stream())
+    _abi.call("gtm_prepare_message_ta_state", ctypes.byref(acfg), _ptr(bank), _stream())
+    want_ta, want_w = o.prepare(cfg, 0xDEADBEEFCAFE, 5)
+    assert np.array_equal(host(ta, np.uint32, want_ta.shape), want_ta)
+    assert np.array_equal(host(w, np.int32, want_w.shape), want_w)
+    assert np.array_equal(host(bank, np.uint32, (cfg.clauses, cfg.message_chunks, cfg.state_bits)),
+                          o.prepare_message_ta_state(cfg))
+    assert set(np.unique(want_w)) == {-1, 1}
+
+
+def test_bad_arguments_are_reported():
+    import ctypes
+    from tests.gpu_harness import abi_config
+    from graphtsetlinmachine_amd import _abi
+
+    cfg = o.Config(classes=2, clauses=4, literals=8, max_nodes=2)
+    acfg = abi_config(cfg, 1, 1.0, 1)
+    with pytest.raises(_abi.GtmError, match="NULL"):
+        _abi.call("gtm_prepare", ctypes.byref(acfg), 0, None, None, None)
+    acfg.state_bits = 40
+    with pytest.raises(_abi.GtmError, match="state_bits"):
+        _abi.call("gtm_prepare_message_ta_state", ctypes.byref(acfg), None, None)
