@@ -1,0 +1,194 @@
+#!/usr/bin/env python3
+"""Benchmark of the Graph Tsetlin Machine hot path on one MI355X.
+
+A "step" is one pass of batched inference (clause evaluation per node ->
+class sums) over the workload's test graphs, with the encoded graphs and the
+model state already resident in HBM.  The model state comes from training on
+the GPU for one epoch over a sample of the training graphs, so include masks
+have a trained density rather than being empty.
+
+Prints ONE JSON line (rank 0 / the only process).
+"""
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=20)
+    p.add_argument("--warmup", type=int, default=3)
+    p.add_argument("--workload", default="convolutional_images")
+    p.add_argument("--graphs", type=int, default=10000, help="test graphs scored per step")
+    p.add_argument("--train-graphs", type=int, default=5000, help="training graphs used to produce the model state")
+    p.add_argument("--train-epochs", type=int, default=1)
+    p.add_argument("--cpu-sample", type=int, default=None, help="graphs timed on the CPU oracle")
+    p.add_argument("--no-cpu", action="store_true")
+    return p.parse_args()
+
+
+def eval_bytes_per_graph(n_nodes, la_chunks, clauses, node_chunks):
+    """Algorithmic bytes of one layer-0 clause evaluation of one graph: its X
+    rows, node types and the include plane in; the clause x node bitmap and the
+    include counts out."""
+    return n_nodes * la_chunks * 4 + n_nodes * 4 + clauses * la_chunks * 4 + clauses * node_chunks * 4 + clauses * 4
+
+
+def time_clause_eval(tm, graphs, repeats):
+    """Average duration of the clause-evaluation launch over the whole batch,
+    from HIP events recorded on the stream the kernels are enqueued on."""
+    import torch
+
+    from graphtsetlinmachine_amd import _abi
+    from graphtsetlinmachine_amd.tm import _ptr, _stream
+
+    dg = tm._score_init(graphs)
+    cfg = tm._config(max(dg.max_nodes, 1))
+    n = dg.number_of_graphs
+    nc = (max(dg.max_nodes, 1) - 1) // 32 + 1
+    bitmap = torch.empty(n * tm.number_of_clauses * nc, dtype=torch.int32, device="cuda")
+    plane = torch.empty(tm.number_of_ta_chunks * tm.number_of_clauses, dtype=torch.int32, device="cuda")
+
+    def launch():
+        _abi.call("gtm_calculate_messages", ctypes.byref(cfg), ctypes.byref(dg.desc), 0, n, _ptr(tm.ta_state_gpu),
+                  _ptr(plane), _ptr(bitmap), None, _stream())
+
+    launch()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(repeats):
+        launch()
+    stop.record()
+    torch.cuda.synchronize()
+    return "k_clause_node_bits", start.elapsed_time(stop) / repeats
+
+
+def mean_included_literals(tm):
+    import numpy as np
+
+    bank = tm.get_state()[0].reshape(tm.number_of_clauses, tm.number_of_ta_chunks, tm.number_of_state_bits)
+    plane = bank[:, :, tm.number_of_state_bits - 1]
+    return float(np.unpackbits(plane.view(np.uint8)).sum()) / tm.number_of_clauses
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; inference shards by graph range and training by clause, "
+              "but no multi-GPU path is part of it. Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from graphtsetlinmachine_amd import _abi, workloads
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    torch.cuda.set_device(0)
+    t0 = time.time()
+    wl = workloads.BUILDERS[args.workload](n_train=args.train_graphs, n_test=args.graphs)
+    t_data = time.time() - t0
+
+    np.random.seed(42)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
+    # training throughput (also produces the state that inference is timed on)
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=0, incremental=True)  # allocate + upload only
+    torch.cuda.synchronize()
+    t0 = time.time()
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=args.train_epochs, incremental=True)
+    torch.cuda.synchronize()
+    t_train = time.time() - t0
+    train_gps = args.train_graphs * args.train_epochs / t_train
+
+    test = wl.graphs_test
+    tm.score_device(test)  # uploads the test graphs
+    for _ in range(args.warmup):
+        tm.score_device(test)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        sums = tm.score_device(test)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1000.0 / args.steps
+    event_ms = start.elapsed_time(stop) / args.steps
+    value = args.graphs * args.steps / wall
+
+    sums_host = sums.cpu().numpy().reshape(args.graphs, -1)
+    accuracy = float((sums_host.argmax(axis=1) == wl.Y_test).mean())
+
+    # roofline of the clause-evaluation kernel: algorithmic bytes / kernel time
+    n_nodes = int(test.max_number_of_graph_nodes)
+    la = tm.number_of_ta_chunks
+    b_eval = eval_bytes_per_graph(n_nodes, la, tm.number_of_clauses, (n_nodes - 1) // 32 + 1)
+    kernel_name, kernel_ms = time_clause_eval(tm, test, repeats=max(3, args.steps))
+    achieved = b_eval * args.graphs / (kernel_ms * 1e-3) / 1e9
+    compulsory = (n_nodes * la * 4 + n_nodes * 4 + tm.number_of_outputs * 4) * args.graphs
+    roofline = {
+        "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+        "kernel": kernel_name, "kernel_ms": round(kernel_ms, 4),
+        "algorithmic_bytes_per_graph": b_eval,
+        "compulsory_GBs": round(compulsory / (kernel_ms * 1e-3) / 1e9, 1),
+    }
+
+    cpu = None
+    if not args.no_cpu:
+        from oracle import gtm_oracle as o
+
+        sample = args.cpu_sample or max(8, min(args.graphs, int(4e9 // (tm.number_of_clauses * n_nodes * la * 60))))
+        sample = min(sample, args.graphs)
+        state = tm.get_state()
+        cfg = o.Config(classes=tm.number_of_outputs, clauses=tm.number_of_clauses, literals=tm.number_of_literals,
+                       state_bits=tm.number_of_state_bits, threshold=tm.T, q=tm.q,
+                       max_included_literals=tm.max_included_literals, max_nodes=n_nodes,
+                       message_size=tm.message_size, message_bits=tm.message_bits)
+        model = o.new_model(cfg, tm.depth, tm.s, tm.hypervectors, seed=tm.seed)
+        model.ta_state = state[0].reshape(cfg.clauses, cfg.la_chunks, cfg.state_bits).copy()
+        model.message_ta_state = [b.reshape(cfg.clauses, cfg.message_chunks, cfg.state_bits).copy()
+                                  for b in tm.message_ta_state]
+        model.clause_weights = state[1].reshape(cfg.classes, cfg.clauses).copy()
+        t0 = time.perf_counter()
+        want = o.score(model, test, range(sample))
+        t_cpu = time.perf_counter() - t0
+        if not np.array_equal(want, sums_host[:sample]):
+            print("bench.py: GPU class sums differ from the CPU oracle on the sample", file=sys.stderr)
+            sys.exit(1)
+        cpu = {"value": round(sample / t_cpu, 2), "unit": "graphs/s", "cores": 1, "kind": "port",
+               "sample": "NumPy oracle, inference on the first %d test graphs (%.1f s), checked equal to the GPU sums"
+                         % (sample, t_cpu)}
+
+    line = {
+        "metric": "inference graphs/sec on 1 MI355X (%s)" % args.workload,
+        "value": round(value, 1), "unit": "graphs/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u32", "data": "synthetic",
+        "config": {"workload": args.workload, "graphs_per_step": args.graphs, "nodes_per_graph": n_nodes,
+                   "clauses": tm.number_of_clauses, "literals": tm.number_of_literals, "depth": tm.depth,
+                   "classes": tm.number_of_outputs, "state": "trained %d epoch(s) on %d graphs on the GPU"
+                   % (args.train_epochs, args.train_graphs),
+                   "mean_included_literals": round(mean_included_literals(tm), 2)},
+        "roofline": roofline, "cpu_baseline": cpu,
+        "train_graphs_per_s": round(train_gps, 1), "test_accuracy": round(accuracy, 4),
+        "event_ms_per_step": round(event_ms, 4), "data_build_s": round(t_data, 1),
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

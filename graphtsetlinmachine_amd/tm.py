@@ -264,6 +264,12 @@ class CommonTsetlinMachine:
 
     def _score(self, graphs, batch=None):
         """tm.py:786-812 as one gtm_score call."""
+        n = int(graphs.number_of_graphs)
+        return self.score_device(graphs, batch).cpu().numpy().reshape(n, self.number_of_outputs)
+
+    def score_device(self, graphs, batch=None):
+        """Class sums as a flat int32 device tensor [graphs * outputs]; work is
+        only enqueued on the current stream."""
         dg = self._score_init(graphs)
         cfg = self._config(max(dg.max_nodes, 1))
         n = dg.number_of_graphs
@@ -277,7 +283,7 @@ class CommonTsetlinMachine:
             "gtm_score", ctypes.byref(cfg), ctypes.byref(dg.desc), ctypes.byref(self._state), 0, n, batch,
             _ptr(ws), ws.numel(), _ptr(out), _stream(),
         )
-        return out.cpu().numpy().reshape(n, self.number_of_outputs)
+        return out
 
     # ------------------------------------------------------------- state I/O
 

@@ -1,0 +1,129 @@
+"""The public model API on the GPU against the oracle driven the same way."""
+
+import numpy as np
+import pytest
+
+from graphtsetlinmachine_amd import workloads
+from oracle import gtm_oracle as o
+from tests import helpers
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_twin(tm, graphs):
+    cfg = o.Config(classes=tm.number_of_outputs, clauses=tm.number_of_clauses, literals=tm.number_of_literals,
+                   state_bits=tm.number_of_state_bits, boost_true_positive_feedback=tm.boost_true_positive_feedback,
+                   threshold=tm.T, q=tm.q, max_included_literals=tm.max_included_literals,
+                   max_nodes=int(graphs.max_number_of_graph_nodes), message_size=tm.message_size,
+                   message_bits=tm.message_bits)
+    return o.new_model(cfg, tm.depth, tm.s, tm.hypervectors, seed=tm.seed)
+
+
+def assert_same_state(tm, model):
+    state = tm.save()
+    assert np.array_equal(state["ta_state"], model.ta_state.reshape(-1))
+    assert np.array_equal(state["clause_weights"].reshape(model.clause_weights.shape), model.clause_weights)
+    for got, want in zip(state["message_ta_state"], model.message_ta_state):
+        assert np.array_equal(got, want.reshape(-1))
+
+
+def test_noisy_xor_end_to_end_matches_oracle_and_learns():
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    wl = workloads.noisy_xor(1500, 500)
+    np.random.seed(3)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=99)
+    model = None
+    for epoch in range(2):
+        tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
+        if model is None:
+            model = oracle_twin(tm, wl.graphs_train)
+        o.fit(model, wl.graphs_train, o.encode_labels(wl.Y_train, 2, tm.T))
+        assert_same_state(tm, model)
+    sums = tm.score(wl.graphs_test)
+    assert np.array_equal(sums, o.score(model, wl.graphs_test))
+    assert np.array_equal(tm.predict(wl.graphs_test), sums.argmax(axis=1))
+    assert (tm.predict(wl.graphs_test) == wl.Y_test).mean() == 1.0
+    assert (tm.predict(wl.graphs_train) == wl.Y_train).mean() >= 0.975
+    # introspection used by every demo's tail
+    assert tm.get_weights().shape == (2, 10)
+    plane = model.ta_state[:, :, 7]
+    for clause in (0, 9):
+        for ta in (0, 17, 33, 63):
+            assert bool(tm.ta_action(0, clause, ta)) == bool((plane[clause, ta // 32] >> (ta % 32)) & 1)
+    assert tm.get_state()[2:8] == (2, 10, 64, 2, 8, 2)
+
+
+def test_save_load_roundtrip_and_resume(tmp_path):
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    wl = workloads.noisy_xor(300, 100)
+    np.random.seed(4)
+    a = MultiClassGraphTsetlinMachine(**wl.params, seed=5)
+    a.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
+    path = str(tmp_path / "model.pkl")
+    state = a.save(path)
+    reference_keys = {
+        "ta_state", "message_ta_state", "clause_weights", "hypervectors", "number_of_outputs", "number_of_literals",
+        "number_of_message_literals", "min_y", "max_y", "negative_clauses", "max_number_of_graph_nodes",
+        "number_of_clauses", "T", "s", "q", "max_included_literals", "boost_true_positive_feedback",
+        "number_of_state_bits", "depth", "message_size", "message_bits", "double_hashing", "one_hot_encoding",
+    }
+    assert reference_keys <= set(state)
+    assert state["ta_state"].dtype == np.uint32 and state["ta_state"].shape == (10 * 2 * 8,)
+    assert state["clause_weights"].dtype == np.int32
+    b = MultiClassGraphTsetlinMachine(**wl.params, seed=777)
+    b.load(fname=path)
+    assert np.array_equal(b.score(wl.graphs_test), a.score(wl.graphs_test))
+    # resuming from the file continues exactly where the first model would have gone
+    a.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
+    b.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
+    sa, sb = a.save(), b.save()
+    assert np.array_equal(sa["ta_state"], sb["ta_state"]) and np.array_equal(sa["clause_weights"], sb["clause_weights"])
+    assert np.array_equal(sa["message_ta_state"][0], sb["message_ta_state"][0])
+
+
+def test_ragged_multi_type_graphs_depth3_match_oracle():
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    train = helpers.random_graphs(50, n_graphs=40, max_nodes=45, hv_size=24, node_types=("a", "b"),
+                                  edge_types=("l", "r", "u"), max_degree=3)
+    test = helpers.random_graphs(51, n_graphs=25, max_nodes=60, parent=train, node_types=("a", "b"),
+                                 edge_types=("l", "r", "u"), max_degree=3)  # larger graphs than seen in training
+    rng = np.random.default_rng(1)
+    Y = rng.integers(0, 3, size=40)
+    np.random.seed(8)
+    tm = MultiClassGraphTsetlinMachine(60, 40, (2.0, 1.5, 3.0), depth=3, message_size=48, message_bits=2,
+                                       max_included_literals=12, seed=2024)
+    tm.fit(train, Y, epochs=2, incremental=True)
+    model = oracle_twin(tm, train)
+    o.fit(model, train, o.encode_labels(Y, 3, tm.T), epochs=2)
+    assert_same_state(tm, model)
+    model.cfg = oracle_twin(tm, test).cfg  # bitmap stride follows the scored data set
+    assert np.array_equal(tm.score(test), o.score(model, test))
+
+
+def test_fit_not_incremental_resets_layer_zero_only():
+    """tm.py:524-526: a second fit(incremental=False) re-runs `prepare` only."""
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    wl = workloads.noisy_xor(200, 50)
+    np.random.seed(6)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=11)
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=1)
+    before = tm.save()
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=0)
+    after = tm.save()
+    fresh = o.prepare(oracle_twin(tm, wl.graphs_train).cfg, 11, tm.step)
+    assert np.array_equal(after["ta_state"], fresh[0].reshape(-1))
+    assert np.array_equal(after["clause_weights"].reshape(2, -1), fresh[1])
+    assert np.array_equal(after["message_ta_state"][0], before["message_ta_state"][0])
+
+
+def test_score_before_fit_exits_like_the_reference():
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    wl = workloads.noisy_xor(10, 10)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=1)
+    with pytest.raises(SystemExit):
+        tm.score(wl.graphs_test)
