@@ -79,7 +79,7 @@ def mean_included_literals(tm):
     import numpy as np
 
     bank = tm.get_state()[0].reshape(tm.number_of_clauses, tm.number_of_ta_chunks, tm.number_of_state_bits)
-    plane = bank[:, :, tm.number_of_state_bits - 1]
+    plane = np.ascontiguousarray(bank[:, :, tm.number_of_state_bits - 1])
     return float(np.unpackbits(plane.view(np.uint8)).sum()) / tm.number_of_clauses
 
 

@@ -53,6 +53,7 @@ class GraphsDesc(C.Structure):
         ("reserved", C.c_int32),
         ("total_nodes", C.c_int64),
         ("total_edges", C.c_int64),
+        ("tiles", C.c_void_p),
     ]
 
 
@@ -87,6 +88,8 @@ PROTOTYPES = {
     "gtm_select_clause_updates": (C.c_int, [_CFG, _U64, _P, _P, _P, _I, _P, _P, _P]),
     "gtm_update": (C.c_int, [_CFG, _GR, _I, _U64, _P, _P, _P, _P, _P]),
     "gtm_update_message": (C.c_int, [_CFG, _U64, _I, _P, _P, _P, _P, _P, _P]),
+    "gtm_tiles_bytes": (_SZ, [_CFG, _GR]),
+    "gtm_build_tiles": (C.c_int, [_CFG, _GR, _P, _P]),
     "gtm_score_workspace_bytes": (_SZ, [_CFG, _GR, _I]),
     "gtm_score": (C.c_int, [_CFG, _GR, _ST, _I, _I, _I, _P, _SZ, _P, _P]),
     "gtm_fit_workspace_bytes": (_SZ, [_CFG, _GR]),

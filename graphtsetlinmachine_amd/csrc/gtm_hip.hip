@@ -12,6 +12,7 @@
 
 #include "../../include/gtm_abi.h"
 #include "philox.h"
+#include "score_tiles.h"
 
 namespace {
 
@@ -431,6 +432,10 @@ Key key_of(const gtm_config *cfg) { return Key{(uint32_t)(cfg->seed & 0xFFFFFFFF
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct ScoreWs {
+    uint16_t *lists;     // [C][list_stride]  (literal-major tile path)
+    int32_t *count8;     // [C]
+    int32_t *wt;         // [C][K]
+    int list_stride;
     uint32_t *inc_t;     // [max(LA,MC)][C]
     uint32_t *bitmap_a;  // [batch][C][NC]
     uint32_t *bitmap_b;  // [batch][C][NC] (depth > 1)
@@ -447,6 +452,10 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base)
         off += align_up(bytes);
         return p;
     };
+    w.list_stride = (cfg->literals + 8 + 7) & ~7;
+    w.lists = (uint16_t *)take((size_t)d.C * w.list_stride * 2);
+    w.count8 = (int32_t *)take((size_t)d.C * 4);
+    w.wt = (int32_t *)take((size_t)d.C * d.K * 4);
     w.inc_t = (uint32_t *)take((size_t)chunks * d.C * 4);
     w.bitmap_a = (uint32_t *)take((size_t)batch * d.C * d.NC * 4);
     if (cfg->depth > 1) {
@@ -563,6 +572,28 @@ int validate_state(const gtm_config *cfg, const gtm_state *s) {
         if (!s->message_ta_state[l]) return fail(GTM_ERR_INVALID, "state lacks message_ta_state[%d]", l);
     if (cfg->depth > 1 && !s->hypervectors) return fail(GTM_ERR_INVALID, "state lacks hypervectors");
     return GTM_OK;
+}
+
+// Depth-1 inference on literal-major tiles (see score_tiles.h).
+int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
+                   const ScoreWs &w, int first, int n_graphs, int32_t *class_sum, hipStream_t st) {
+    hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB)), dim3(TPB), 0, st, s->ta_state, d.C, d.LA, d.B,
+                       d.filter, d.K, s->clause_weights, tg.rows - 1, w.list_stride, w.lists, w.count8, w.wt);
+    if (int rc = check_launch("compile_clauses")) return rc;
+    constexpr int NW = 8;
+    size_t lds = (size_t)tg.rows * tg.tw * 4 + (size_t)tg.gpt * d.K * 4;
+    static thread_local size_t lds_set = 0;
+    if (lds > lds_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)k_score_tiles<NW>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)lds);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
+        lds_set = lds;
+    }
+    int tile0 = first / tg.gpt, tile1 = (first + n_graphs - 1) / tg.gpt;
+    hipLaunchKernelGGL((k_score_tiles<NW>), dim3(tile1 - tile0 + 1), dim3(NW * 64), lds, st, g->tiles, tg, cfg->literals,
+                       g->number_of_node_types, d.C, d.K, w.lists, w.list_stride, w.count8, w.wt, tile0, first,
+                       n_graphs, class_sum);
+    return check_launch("score_tiles");
 }
 
 }  // namespace
@@ -743,6 +774,30 @@ int gtm_update_message(const gtm_config *cfg, uint64_t step, int32_t bank, uint3
                      class_clause_update, (hipStream_t)stream);
 }
 
+size_t gtm_tiles_bytes(const gtm_config *cfg, const gtm_graphs *graphs) {
+    Dims d;
+    if (validate(cfg, &d) || !graphs || graphs->number_of_graphs < 1 || graphs->number_of_node_types < 1) return 0;
+    TileGeom tg = tile_geometry(cfg->literals, graphs->number_of_node_types, graphs->max_number_of_graph_nodes,
+                                graphs->number_of_graphs, d.K);
+    if (!tg.ok) return 0;
+    return (size_t)tg.n_tiles * tg.rows * tg.tw * 4;
+}
+
+int gtm_build_tiles(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *tiles, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (int rc = validate_graphs(cfg, graphs, 0, 0)) return rc;
+    if (!tiles) return fail(GTM_ERR_INVALID, "tiles is NULL");
+    TileGeom tg = tile_geometry(cfg->literals, graphs->number_of_node_types, graphs->max_number_of_graph_nodes,
+                                graphs->number_of_graphs, d.K);
+    if (!tg.ok) return fail(GTM_ERR_INVALID, "this data set's shape has no tile layout (gtm_tiles_bytes() == 0)");
+    int64_t total = (int64_t)tg.n_tiles * tg.rows * tg.tw;
+    hipLaunchKernelGGL(k_build_tiles, dim3(blocks_for(total, TPB)), dim3(TPB), 0, (hipStream_t)stream, graphs->X,
+                       graphs->node_type, graphs->node_index, graphs->number_of_graph_nodes, graphs->number_of_graphs,
+                       d.LA, cfg->literals, graphs->number_of_node_types, tg, total, tiles);
+    return check_launch("build_tiles");
+}
+
 size_t gtm_score_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs, int32_t batch) {
     Dims d;
     if (validate(cfg, &d) || batch < 1) return 0;
@@ -763,6 +818,11 @@ int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *
     if (!workspace || workspace_bytes < w.bytes)
         return fail(GTM_ERR_INVALID, "workspace of %zu bytes needed, %zu given", w.bytes, workspace_bytes);
     hipStream_t st = (hipStream_t)stream;
+    if (cfg->depth == 1 && graphs->tiles && n_graphs > 0) {
+        TileGeom tg = tile_geometry(cfg->literals, graphs->number_of_node_types, graphs->max_number_of_graph_nodes,
+                                    graphs->number_of_graphs, d.K);
+        if (tg.ok) return score_on_tiles(d, cfg, graphs, state, tg, w, first_graph, n_graphs, class_sum, st);
+    }
     for (int done = 0; done < n_graphs; done += batch) {
         int nb = n_graphs - done < batch ? n_graphs - done : batch;
         uint32_t *final_bitmap = nullptr;

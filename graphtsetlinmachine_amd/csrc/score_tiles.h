@@ -1,0 +1,194 @@
+// Batched depth-1 inference on literal-major tiles.
+//
+// The dense form of clause evaluation tests every clause against every word
+// of every node (CLAUSES x nodes x LA_CHUNKS word operations per graph) and is
+// bound by integer VALU throughput, not by HBM.  A clause is an AND of few
+// literals, so this path turns the data instead: for a tile of graphs it keeps
+// one bit-row per LITERAL (bit n of the row = that literal at node slot n of
+// the tile), staged in LDS, and a clause's truth over all node slots of the
+// tile is the AND of the rows of its included literals only.  The result is
+// the same bits as kernels.py:443-466 computes; no clause/node bitmap is
+// written because `evaluate` (kernels.py:297-315) only needs "true at some
+// node of the graph".
+//
+// Tile layout in HBM (built once per data set by k_build_tiles):
+//   tiles[tile][row][tw] uint32, rows = LITERALS + node_types + 1
+//     row l < LITERALS          bit-row of literal l
+//     row LITERALS + t          valid nodes of node type t
+//     last row                  all ones (pads literal lists)
+//   node slots: graph j of the tile owns `slot_bits` consecutive bits starting
+//   at j * slot_bits; slot_bits is a power of two < 32 for tiny graphs, else a
+//   whole number of 32-bit words.
+#pragma once
+
+struct TileGeom {
+    int slot_bits;   // bits per graph slot
+    int slot_words;  // words per graph slot (0 when slot_bits < 32)
+    int gpt;         // graphs per tile
+    int tw;          // words per tile row (<= 64)
+    int rows;        // LITERALS + node types + 1
+    int n_tiles;
+    int ok;          // geometry supported by the fused kernel
+};
+
+constexpr int TILE_MAX_WORDS = 64;
+constexpr size_t TILE_LDS_BUDGET = 156 * 1024;  // of the 160 KB per CU
+
+inline TileGeom tile_geometry(int literals, int n_types, int max_nodes, int n_graphs, int classes) {
+    TileGeom g{};
+    if (max_nodes < 1) max_nodes = 1;
+    if (max_nodes <= 16) {
+        int s = 1;
+        while (s < max_nodes) s <<= 1;
+        g.slot_bits = s;
+        g.slot_words = 0;
+        g.tw = TILE_MAX_WORDS;
+        g.gpt = TILE_MAX_WORDS * 32 / s;
+    } else {
+        g.slot_words = (max_nodes - 1) / 32 + 1;
+        g.slot_bits = g.slot_words * 32;
+        g.gpt = g.slot_words <= TILE_MAX_WORDS ? TILE_MAX_WORDS / g.slot_words : 0;
+        g.tw = g.gpt * g.slot_words;
+    }
+    g.rows = literals + n_types + 1;
+    g.n_tiles = g.gpt > 0 ? (n_graphs + g.gpt - 1) / g.gpt : 0;
+    size_t lds = (size_t)g.rows * g.tw * 4 + (size_t)g.gpt * classes * 4;
+    g.ok = g.gpt > 0 && lds <= TILE_LDS_BUDGET && literals < 65535 - 8;
+    return g;
+}
+
+// One thread per tile word: gathers its 32 node slots.
+__global__ void k_build_tiles(const uint32_t *__restrict__ X, const uint32_t *__restrict__ node_type,
+                              const uint32_t *__restrict__ node_index, const uint32_t *__restrict__ n_nodes_arr,
+                              int G, int LA, int literals, int n_types, TileGeom tg, int64_t total,
+                              uint32_t *__restrict__ tiles) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    int w = (int)(i % tg.tw);
+    int64_t rest = i / tg.tw;
+    int row = (int)(rest % tg.rows);
+    int tile = (int)(rest / tg.rows);
+    uint32_t out = 0;
+    if (row == tg.rows - 1) {
+        out = 0xFFFFFFFFu;
+    } else {
+        for (int b = 0; b < 32; ++b) {
+            int pos = w * 32 + b;
+            int j = pos / tg.slot_bits, n = pos % tg.slot_bits;
+            int64_t g = (int64_t)tile * tg.gpt + j;
+            if (j >= tg.gpt || g >= G) continue;
+            int count = (int)n_nodes_arr[g];
+            if (count == 0 && n == 0) {
+                // kernels.py:289-295,443-466: for a graph without nodes the reference's
+                // chunk arithmetic leaves every clause true; slot bit 0 carries that.
+                out |= 1u << b;
+                continue;
+            }
+            if (n >= count) continue;
+            int64_t node = (int64_t)node_index[g] + n;
+            uint32_t bit;
+            if (row < literals)
+                bit = (X[node * LA + (row >> 5)] >> (row & 31)) & 1u;
+            else
+                bit = (int)node_type[node] == row - literals;
+            out |= bit << b;
+        }
+    }
+    tiles[i] = out;
+}
+
+// Per call: each clause's included literals as a list of row ids padded to a
+// multiple of 8 with the all-ones row, and the weights clause-major.
+__global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int LA, int B, uint32_t filter, int K,
+                                  const int32_t *__restrict__ weights, int ones_row, int stride,
+                                  uint16_t *__restrict__ lists, int32_t *__restrict__ count8, int32_t *__restrict__ wt) {
+    int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    uint16_t *list = lists + (int64_t)c * stride;
+    int n = 0;
+    for (int w = 0; w < LA; ++w) {
+        uint32_t m = bank[((int64_t)c * LA + w) * B + (B - 1)];
+        if (w == LA - 1) m &= filter;
+        while (m) {
+            int b = __ffs(m) - 1;
+            m &= m - 1;
+            list[n++] = (uint16_t)(w * 32 + b);
+        }
+    }
+    int padded = (n + 7) & ~7;
+    for (int i = n; i < padded; ++i) list[i] = (uint16_t)ones_row;
+    count8[c] = padded;
+    for (int k = 0; k < K; ++k) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
+}
+
+// One workgroup per tile.  The tile's bit-rows are copied to LDS once; each
+// wave then walks its share of the clauses.  The clause id and its literal
+// list are wave-uniform (scalar loads); lane L holds word L of the running AND.
+template <int NWAVES>
+__global__ __launch_bounds__(NWAVES * 64) void k_score_tiles(
+    const uint32_t *__restrict__ tiles, TileGeom tg, int literals, int n_types, int C, int K,
+    const uint16_t *__restrict__ lists, int stride, const int32_t *__restrict__ count8,
+    const int32_t *__restrict__ wt, int tile0, int first_graph, int n_graphs, int32_t *__restrict__ class_sum) {
+    extern __shared__ uint32_t lds[];
+    const int tw = tg.tw;
+    uint32_t *bt = lds;
+    int32_t *sums = (int32_t *)(lds + (size_t)tg.rows * tw);
+    const int tile = tile0 + blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    const uint32_t *src = tiles + (int64_t)tile * tg.rows * tw;
+    for (int i = tid; i < tg.rows * tw; i += NWAVES * 64) bt[i] = src[i];
+    for (int i = tid; i < tg.gpt * K; i += NWAVES * 64) sums[i] = 0;
+    __syncthreads();
+
+    const bool active = lane < tw;
+    const uint32_t *col = bt + (active ? lane : 0);
+    for (int c = wave; c < C; c += NWAVES) {
+        uint32_t acc = active ? col[(literals + c % n_types) * tw] : 0u;
+        const int cnt = count8[c];
+        const uint4 *lp = reinterpret_cast<const uint4 *>(lists + (int64_t)c * stride);
+        for (int j = 0; j < cnt; j += 8) {
+            uint4 ids = lp[j >> 3];
+            acc &= col[(ids.x & 0xFFFFu) * tw];
+            acc &= col[(ids.x >> 16) * tw];
+            acc &= col[(ids.y & 0xFFFFu) * tw];
+            acc &= col[(ids.y >> 16) * tw];
+            acc &= col[(ids.z & 0xFFFFu) * tw];
+            acc &= col[(ids.z >> 16) * tw];
+            acc &= col[(ids.w & 0xFFFFu) * tw];
+            acc &= col[(ids.w >> 16) * tw];
+            if (__ballot(acc != 0) == 0) break;  // false at every node slot of the tile
+        }
+        const unsigned long long nz = __ballot(acc != 0);
+        if (nz == 0) continue;
+        if (tg.slot_words > 0) {
+            // graph j owns lanes [j*slot_words, (j+1)*slot_words)
+            unsigned long long mine = nz >> ((lane < tg.gpt ? lane : 0) * tg.slot_words);
+            if (tg.slot_words < 64) mine &= (1ull << tg.slot_words) - 1ull;
+            const unsigned long long gm = __ballot(lane < tg.gpt && mine != 0);
+            for (int p = lane; p < tg.gpt * K; p += 64) {
+                int j = p / K, k = p - j * K;
+                if ((gm >> j) & 1ull) atomicAdd(&sums[p], wt[(int64_t)c * K + k]);
+            }
+        } else {
+            // several graphs per word: walk the non-empty slots of this lane's word
+            const int per_word = 32 / tg.slot_bits;
+            const uint32_t slot_mask = (1u << tg.slot_bits) - 1u;  // slot_bits <= 16
+            while (acc) {
+                int sub = (__ffs(acc) - 1) / tg.slot_bits;
+                acc &= ~(slot_mask << (sub * tg.slot_bits));
+                int j = lane * per_word + sub;
+                for (int k = 0; k < K; ++k) atomicAdd(&sums[j * K + k], wt[(int64_t)c * K + k]);
+            }
+        }
+    }
+    __syncthreads();
+    const int64_t g0 = (int64_t)tile * tg.gpt;
+    for (int i = tid; i < tg.gpt * K; i += NWAVES * 64) {
+        int64_t g = g0 + i / K;
+        if (g >= first_graph && g < (int64_t)first_graph + n_graphs)
+            class_sum[(g - first_graph) * K + (i % K)] = sums[i];
+    }
+}

@@ -72,7 +72,23 @@ class _DeviceGraphs:
         d.max_number_of_graph_nodes = self.max_nodes
         d.total_nodes = int(graphs.number_of_nodes)
         d.total_edges = int(graphs.edge.shape[0])
+        d.tiles = None
         self.desc = d
+        self.tiles = None
+        self._tiles_tried = False
+
+    def ensure_tiles(self, cfg):
+        """Build the literal-major tile layout once per data set (used by
+        depth-1 inference); shapes without such a layout keep tiles = NULL."""
+        if self._tiles_tried:
+            return
+        self._tiles_tried = True
+        nbytes = _abi.lib.gtm_tiles_bytes(ctypes.byref(cfg), ctypes.byref(self.desc))
+        if nbytes == 0:
+            return
+        self.tiles = torch.empty(nbytes // 4, dtype=torch.int32, device=_device())
+        _abi.call("gtm_build_tiles", ctypes.byref(cfg), ctypes.byref(self.desc), _ptr(self.tiles), _stream())
+        self.desc.tiles = self.tiles.data_ptr()
 
 
 class CommonTsetlinMachine:
@@ -273,6 +289,8 @@ class CommonTsetlinMachine:
         dg = self._score_init(graphs)
         cfg = self._config(max(dg.max_nodes, 1))
         n = dg.number_of_graphs
+        if self.depth == 1:
+            dg.ensure_tiles(cfg)
         if batch is None:
             per_graph = max(1, _abi.lib.gtm_score_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc), 1))
             batch = int(max(1, min(n, (1 << 30) // per_graph, 1 << 16)))

@@ -76,6 +76,7 @@ typedef struct gtm_graphs {
     int32_t reserved;
     int64_t total_nodes;
     int64_t total_edges;
+    const uint32_t *tiles; /* optional: literal-major tiles from gtm_build_tiles, or NULL */
 } gtm_graphs;
 
 /* The model's device buffers (tm.py:110-124). */
@@ -156,11 +157,23 @@ int gtm_update_message(const gtm_config *cfg, uint64_t step, int32_t bank, uint3
 
 /* ---- the driver loops --------------------------------------------------- */
 
+/* A second, derived layout of a data set for batched depth-1 inference: per
+ * tile of graphs one bit-row per literal over the tile's node slots (plus one
+ * row per node type), so that a clause is evaluated as the AND of the rows of
+ * its included literals only.  Stands where the reference uploads X once per
+ * data set (tm.py:759-763).  gtm_tiles_bytes() is 0 when the data set's shape
+ * has no such layout (then leave gtm_graphs.tiles NULL); gtm_build_tiles()
+ * fills a caller-owned buffer of that size from X / node_type. */
+size_t gtm_tiles_bytes(const gtm_config *cfg, const gtm_graphs *graphs);
+int gtm_build_tiles(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *tiles, void *stream);
+
 /* Scratch needed by gtm_score for sub-batches of `batch` graphs. */
 size_t gtm_score_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs, int32_t batch);
 
 /* `_score` (tm.py:786-812): class sums [n_graphs][CLASSES] of graphs
- * [first_graph, first_graph + n_graphs), evaluated `batch` graphs at a time. */
+ * [first_graph, first_graph + n_graphs), evaluated `batch` graphs at a time.
+ * With depth == 1 and graphs->tiles set, one fused kernel evaluates all
+ * clauses and accumulates the class sums without writing a bitmap. */
 int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, int32_t first_graph,
               int32_t n_graphs, int32_t batch, void *workspace, size_t workspace_bytes, int32_t *class_sum,
               void *stream);

@@ -110,6 +110,15 @@ class Device:
                   _ptr(clause_node), _ptr(n_incl), _ptr(cx), _ptr(updates), _stream())
 
     # --- driver loops ----------------------------------------------------
+    def build_tiles(self):
+        nbytes = _abi.lib.gtm_tiles_bytes(ctypes.byref(self.acfg), ctypes.byref(self.dg.desc))
+        if nbytes == 0:
+            return False
+        self.tiles = torch.empty(nbytes // 4, dtype=torch.int32, device="cuda")
+        _abi.call("gtm_build_tiles", ctypes.byref(self.acfg), ctypes.byref(self.dg.desc), _ptr(self.tiles), _stream())
+        self.dg.desc.tiles = self.tiles.data_ptr()
+        return True
+
     def score(self, first, n, batch):
         need = _abi.lib.gtm_score_workspace_bytes(ctypes.byref(self.acfg), ctypes.byref(self.dg.desc), batch)
         ws = torch.empty(need, dtype=torch.uint8, device="cuda")

@@ -7,7 +7,7 @@ from oracle import gtm_oracle as o
 
 
 def random_graphs(seed, n_graphs=6, max_nodes=40, hv_size=20, hv_bits=2, n_symbols=7, node_types=("Plain",),
-                  edge_types=("Plain",), max_degree=3, min_nodes=1, parent=None):
+                  edge_types=("Plain",), max_degree=3, min_nodes=1, parent=None, sizes=None):
     """Ragged graphs built through the per-call API: several node and edge
     types, self-loops, parallel edges, nodes without out-edges."""
     rng = np.random.default_rng(seed)
@@ -19,7 +19,7 @@ def random_graphs(seed, n_graphs=6, max_nodes=40, hv_size=20, hv_bits=2, n_symbo
         np.random.set_state(saved)
     else:
         g = Graphs(n_graphs, init_with=parent)
-    sizes = rng.integers(min_nodes, max_nodes + 1, size=n_graphs)
+    sizes = rng.integers(min_nodes, max_nodes + 1, size=n_graphs) if sizes is None else np.asarray(sizes)
     for i, n in enumerate(sizes):
         g.set_number_of_graph_nodes(i, int(n))
     g.prepare_node_configuration()

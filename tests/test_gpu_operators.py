@@ -209,3 +209,55 @@ def test_bad_arguments_are_reported():
     acfg.state_bits = 40
     with pytest.raises(_abi.GtmError, match="state_bits"):
         _abi.call("gtm_prepare_message_ta_state", ctypes.byref(acfg), None, None)
+
+
+TILE_SHAPES = [
+    # tiny graphs (several per word), one word, several words, exactly 64 words, more than one node type
+    dict(seed=11, g=dict(n_graphs=300, max_nodes=1, hv_size=40), classes=3, clauses=50),
+    dict(seed=12, g=dict(n_graphs=200, max_nodes=3, hv_size=16, node_types=("a", "b")), classes=2, clauses=64),
+    dict(seed=13, g=dict(n_graphs=70, max_nodes=16, min_nodes=9, hv_size=20), classes=4, clauses=33),
+    dict(seed=14, g=dict(n_graphs=40, max_nodes=31, min_nodes=17, hv_size=64), classes=10, clauses=200),
+    dict(seed=15, g=dict(n_graphs=23, max_nodes=361, min_nodes=300, hv_size=128, max_degree=0), classes=10, clauses=120),
+    dict(seed=16, g=dict(n_graphs=5, max_nodes=2048, min_nodes=1990, hv_size=16, max_degree=0, node_types=("a", "b", "c")),
+         classes=2, clauses=40),
+]
+
+
+@pytest.mark.parametrize("shape", TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
+@pytest.mark.parametrize("density", [0.0, 0.02, 0.2])
+def test_tile_scoring_equals_oracle(shape, density):
+    """Depth-1 gtm_score on literal-major tiles == oracle == the bitmap path."""
+    from tests.gpu_harness import Device
+
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    cfg = helpers.oracle_config(graphs, classes=shape["classes"], clauses=shape["clauses"])
+    model = helpers.random_model(shape["seed"], cfg, 1, include_density=density)
+    model.ta_state[3, :, cfg.state_bits - 1] = 0  # an empty clause among the random ones
+    dev = Device(model, graphs)
+    G = graphs.number_of_graphs
+    plain = dev.score(0, G, G)
+    assert dev.build_tiles(), "this shape should have a tile layout"
+    tiled = dev.score(0, G, G)
+    assert np.array_equal(tiled, plain)
+    sample = sorted(set([0, 1, G // 2, G - 1]))
+    want = o.score(model, graphs, sample)
+    assert np.array_equal(tiled[sample], want)
+    # a range that starts and ends inside tiles
+    if G > 7:
+        assert np.array_equal(dev.score(3, G - 5, G), plain[3:G - 2])
+
+
+def test_empty_graphs_score_like_the_reference_arithmetic():
+    """A graph without nodes: the reference's chunk arithmetic (C division,
+    kernels.py:289-295) leaves every clause true, so it scores sum_c W[k][c]."""
+    from tests.gpu_harness import Device
+
+    g = helpers.random_graphs(17, n_graphs=6, hv_size=16, sizes=[5, 0, 33, 1, 0, 40])
+    cfg = helpers.oracle_config(g, classes=3, clauses=20)
+    model = helpers.random_model(5, cfg, 1, include_density=0.05)
+    want = o.score(model, g)
+    assert np.array_equal(want[1], model.clause_weights.sum(axis=1)) and np.array_equal(want[4], want[1])
+    dev = Device(model, g)
+    assert np.array_equal(dev.score(0, 6, 6), want)
+    assert dev.build_tiles()
+    assert np.array_equal(dev.score(0, 6, 6), want)
