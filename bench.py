@@ -45,34 +45,15 @@ def eval_bytes_per_graph(n_nodes, la_chunks, clauses, node_chunks):
     return n_nodes * la_chunks * 4 + n_nodes * 4 + clauses * la_chunks * 4 + clauses * node_chunks * 4 + clauses * 4
 
 
-def time_clause_eval(tm, graphs, repeats):
-    """Average duration of the clause-evaluation launch over the whole batch,
-    from HIP events recorded on the stream the kernels are enqueued on."""
-    import torch
-
+def read_kernel_profile():
+    """(kernel name, launches, total ms) of the clause-evaluation kernel since
+    profiling was enabled: HIP events recorded inside the library around each
+    launch, on the stream the kernel runs on."""
     from graphtsetlinmachine_amd import _abi
-    from graphtsetlinmachine_amd.tm import _ptr, _stream
 
-    dg = tm._score_init(graphs)
-    cfg = tm._config(max(dg.max_nodes, 1))
-    n = dg.number_of_graphs
-    nc = (max(dg.max_nodes, 1) - 1) // 32 + 1
-    bitmap = torch.empty(n * tm.number_of_clauses * nc, dtype=torch.int32, device="cuda")
-    plane = torch.empty(tm.number_of_ta_chunks * tm.number_of_clauses, dtype=torch.int32, device="cuda")
-
-    def launch():
-        _abi.call("gtm_calculate_messages", ctypes.byref(cfg), ctypes.byref(dg.desc), 0, n, _ptr(tm.ta_state_gpu),
-                  _ptr(plane), _ptr(bitmap), None, _stream())
-
-    launch()
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(repeats):
-        launch()
-    stop.record()
-    torch.cuda.synchronize()
-    return "k_clause_node_bits", start.elapsed_time(stop) / repeats
+    name, launches, total = ctypes.c_char_p(), ctypes.c_int32(), ctypes.c_double()
+    _abi.call("gtm_profile_read", ctypes.byref(name), ctypes.byref(launches), ctypes.byref(total))
+    return name.value.decode(), launches.value, total.value
 
 
 def mean_included_literals(tm):
@@ -118,6 +99,7 @@ def main():
         tm.score_device(test)
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    _abi.call("gtm_profile_enable", 1)
     t0 = time.perf_counter()
     start.record()
     for _ in range(args.steps):
@@ -125,6 +107,8 @@ def main():
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    kernel_name, launches, kernel_total_ms = read_kernel_profile()
+    _abi.call("gtm_profile_enable", 0)
     ms_per_step = wall * 1000.0 / args.steps
     event_ms = start.elapsed_time(stop) / args.steps
     value = args.graphs * args.steps / wall
@@ -136,13 +120,16 @@ def main():
     n_nodes = int(test.max_number_of_graph_nodes)
     la = tm.number_of_ta_chunks
     b_eval = eval_bytes_per_graph(n_nodes, la, tm.number_of_clauses, (n_nodes - 1) // 32 + 1)
-    kernel_name, kernel_ms = time_clause_eval(tm, test, repeats=max(3, args.steps))
-    achieved = b_eval * args.graphs / (kernel_ms * 1e-3) / 1e9
-    compulsory = (n_nodes * la * 4 + n_nodes * 4 + tm.number_of_outputs * 4) * args.graphs
+    # every launch of the kernel inside the timed region; a step may split its graphs over several launches
+    kernel_ms = kernel_total_ms / max(launches, 1)
+    graphs_per_launch = args.graphs * args.steps / max(launches, 1)
+    achieved = b_eval * graphs_per_launch / (kernel_ms * 1e-3) / 1e9
+    compulsory = (n_nodes * la * 4 + n_nodes * 4 + tm.number_of_outputs * 4) * graphs_per_launch
     roofline = {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-        "kernel": kernel_name, "kernel_ms": round(kernel_ms, 4),
+        "kernel": kernel_name, "kernel_ms": round(kernel_ms, 4), "launches": launches,
+        "graphs_per_launch": graphs_per_launch,
         "algorithmic_bytes_per_graph": b_eval,
         "compulsory_GBs": round(compulsory / (kernel_ms * 1e-3) / 1e9, 1),
     }
@@ -151,7 +138,8 @@ def main():
     if not args.no_cpu:
         from oracle import gtm_oracle as o
 
-        sample = args.cpu_sample or max(8, min(args.graphs, int(4e9 // (tm.number_of_clauses * n_nodes * la * 60))))
+        # the NumPy oracle costs ~3.5 ns per clause x node x word; aim at ~15 s
+        sample = args.cpu_sample or max(8, int(15.0 / (tm.number_of_clauses * n_nodes * la * tm.depth * 3.5e-9)))
         sample = min(sample, args.graphs)
         state = tm.get_state()
         cfg = o.Config(classes=tm.number_of_outputs, clauses=tm.number_of_clauses, literals=tm.number_of_literals,

@@ -36,6 +36,36 @@ int check_launch(const char *what) {
     return GTM_OK;
 }
 
+// --------------------------------------------------------------- profiling
+// When enabled (gtm_profile_enable), the launch of the dominant kernel of a
+// driver loop is bracketed by HIP events on the caller's stream.
+
+struct Profile {
+    bool on = false;
+    const char *name = "";
+    static constexpr int MAX = 512;
+    hipEvent_t start[MAX], stop[MAX];
+    int created = 0, used = 0;
+};
+Profile g_prof;
+
+void profile_start(const char *name, hipStream_t st) {
+    if (!g_prof.on || g_prof.used >= Profile::MAX) return;
+    if (g_prof.used >= g_prof.created) {
+        if (hipEventCreate(&g_prof.start[g_prof.created]) != hipSuccess) return;
+        if (hipEventCreate(&g_prof.stop[g_prof.created]) != hipSuccess) return;
+        ++g_prof.created;
+    }
+    g_prof.name = name;
+    (void)hipEventRecord(g_prof.start[g_prof.used], st);
+}
+
+void profile_stop(hipStream_t st) {
+    if (!g_prof.on || g_prof.used >= g_prof.created) return;
+    (void)hipEventRecord(g_prof.stop[g_prof.used], st);
+    ++g_prof.used;
+}
+
 // --------------------------------------------------------- derived constants
 
 struct Dims {
@@ -433,7 +463,6 @@ size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct ScoreWs {
     uint16_t *lists;     // [C][list_stride]  (literal-major tile path)
-    int32_t *count8;     // [C]
     int32_t *wt;         // [C][K]
     int list_stride;
     uint32_t *inc_t;     // [max(LA,MC)][C]
@@ -452,9 +481,8 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base)
         off += align_up(bytes);
         return p;
     };
-    w.list_stride = (cfg->literals + 8 + 7) & ~7;
-    w.lists = (uint16_t *)take((size_t)d.C * w.list_stride * 2);
-    w.count8 = (int32_t *)take((size_t)d.C * 4);
+    w.list_stride = ((cfg->literals + 1 + 7) & ~7) + 8;  // header + literals, padded to blocks of 8, + 1 block
+    w.lists = (uint16_t *)take((size_t)d.C * w.list_stride * 2 + 16);
     w.wt = (int32_t *)take((size_t)d.C * d.K * 4);
     w.inc_t = (uint32_t *)take((size_t)chunks * d.C * 4);
     w.bitmap_a = (uint32_t *)take((size_t)batch * d.C * d.NC * 4);
@@ -547,8 +575,10 @@ int run_evaluate(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, cons
                  uint32_t *inc_t, uint32_t *bm_a, uint32_t *bm_b, uint32_t *const *clause_X, bool keep_layers,
                  int32_t *n_incl, int32_t *class_sum, uint32_t **final_bitmap, hipStream_t st) {
     if (int rc = op_include_plane(d, s->ta_state, d.LA, d.filter, inc_t, n_incl, 0, st)) return rc;
+    profile_start("k_clause_node_bits", st);
     if (int rc = launch_clause_node_bits(d, g, first, n_graphs, inc_t, d.LA, g->X, 0, cfg->max_nodes, nullptr, bm_a, st))
         return rc;
+    profile_stop(st);
     uint32_t *cur = bm_a, *nxt = bm_b;
     for (int layer = 0; layer < cfg->depth - 1; ++layer) {
         uint32_t *cx = keep_layers ? clause_X[layer] : clause_X[0];
@@ -578,9 +608,9 @@ int validate_state(const gtm_config *cfg, const gtm_state *s) {
 int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
                    const ScoreWs &w, int first, int n_graphs, int32_t *class_sum, hipStream_t st) {
     hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB)), dim3(TPB), 0, st, s->ta_state, d.C, d.LA, d.B,
-                       d.filter, d.K, s->clause_weights, tg.rows - 1, w.list_stride, w.lists, w.count8, w.wt);
+                       d.filter, d.K, s->clause_weights, tg.rows - 1, tg.tw, w.list_stride, w.lists, w.wt);
     if (int rc = check_launch("compile_clauses")) return rc;
-    constexpr int NW = 8;
+    constexpr int NW = 16;
     size_t lds = (size_t)tg.rows * tg.tw * 4 + (size_t)tg.gpt * d.K * 4;
     static thread_local size_t lds_set = 0;
     if (lds > lds_set) {
@@ -590,10 +620,13 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         lds_set = lds;
     }
     int tile0 = first / tg.gpt, tile1 = (first + n_graphs - 1) / tg.gpt;
+    profile_start("k_score_tiles", st);
     hipLaunchKernelGGL((k_score_tiles<NW>), dim3(tile1 - tile0 + 1), dim3(NW * 64), lds, st, g->tiles, tg, cfg->literals,
-                       g->number_of_node_types, d.C, d.K, w.lists, w.list_stride, w.count8, w.wt, tile0, first,
-                       n_graphs, class_sum);
-    return check_launch("score_tiles");
+                       g->number_of_node_types, d.C, d.K, w.lists, w.list_stride, w.wt, tile0, first, n_graphs,
+                       class_sum);
+    if (int rc = check_launch("score_tiles")) return rc;
+    profile_stop(st);
+    return GTM_OK;
 }
 
 }  // namespace
@@ -772,6 +805,29 @@ int gtm_update_message(const gtm_config *cfg, uint64_t step, int32_t bank, uint3
         return fail(GTM_ERR_INVALID, "NULL buffer");
     return op_update(d, cfg, step, bank, message_ta_state, d.MC, clause_node, number_of_include_actions, clause_X,
                      class_clause_update, (hipStream_t)stream);
+}
+
+int gtm_profile_enable(int on) {
+    g_prof.on = on != 0;
+    g_prof.used = 0;
+    return GTM_OK;
+}
+
+int gtm_profile_read(const char **kernel_name, int32_t *launches, double *total_ms) {
+    if (!kernel_name || !launches || !total_ms) return fail(GTM_ERR_INVALID, "NULL output");
+    double total = 0.0;
+    for (int i = 0; i < g_prof.used; ++i) {
+        hipError_t e = hipEventSynchronize(g_prof.stop[i]);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, g_prof.start[i], g_prof.stop[i]);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "reading profile events: %s", hipGetErrorString(e));
+        total += ms;
+    }
+    *kernel_name = g_prof.name;
+    *launches = g_prof.used;
+    *total_ms = total;
+    g_prof.used = 0;
+    return GTM_OK;
 }
 
 size_t gtm_tiles_bytes(const gtm_config *cfg, const gtm_graphs *graphs) {

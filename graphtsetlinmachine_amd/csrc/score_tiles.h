@@ -97,38 +97,53 @@ __global__ void k_build_tiles(const uint32_t *__restrict__ X, const uint32_t *__
     tiles[i] = out;
 }
 
-// Per call: each clause's included literals as a list of row ids padded to a
-// multiple of 8 with the all-ones row, and the weights clause-major.
+// Per call: each clause's included literals as a list of 16-bit LDS word
+// offsets (row * tw), in blocks of 8 entries (one 16-byte scalar load each).
+// Entry 0 of the first block is the number of blocks; unused entries point at
+// the all-ones row.  Also the weights clause-major.
 __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int LA, int B, uint32_t filter, int K,
-                                  const int32_t *__restrict__ weights, int ones_row, int stride,
-                                  uint16_t *__restrict__ lists, int32_t *__restrict__ count8, int32_t *__restrict__ wt) {
+                                  const int32_t *__restrict__ weights, int ones_row, int tw, int stride,
+                                  uint16_t *__restrict__ lists, int32_t *__restrict__ wt) {
     int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= C) return;
     uint16_t *list = lists + (int64_t)c * stride;
-    int n = 0;
+    int n = 1;
     for (int w = 0; w < LA; ++w) {
         uint32_t m = bank[((int64_t)c * LA + w) * B + (B - 1)];
         if (w == LA - 1) m &= filter;
         while (m) {
             int b = __ffs(m) - 1;
             m &= m - 1;
-            list[n++] = (uint16_t)(w * 32 + b);
+            list[n++] = (uint16_t)((w * 32 + b) * tw);
         }
     }
     int padded = (n + 7) & ~7;
-    for (int i = n; i < padded; ++i) list[i] = (uint16_t)ones_row;
-    count8[c] = padded;
+    for (int i = n; i < padded + 8; ++i) list[i] = (uint16_t)(ones_row * tw);  // one block of slack for prefetch
+    list[0] = (uint16_t)(padded >> 3);
     for (int k = 0; k < K; ++k) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
+}
+
+__device__ __forceinline__ uint32_t and8(uint32_t acc, const uint32_t *col, uint4 ids, bool skip_first) {
+    if (!skip_first) acc &= col[ids.x & 0xFFFFu];
+    acc &= col[ids.x >> 16];
+    acc &= col[ids.y & 0xFFFFu];
+    acc &= col[ids.y >> 16];
+    acc &= col[ids.z & 0xFFFFu];
+    acc &= col[ids.z >> 16];
+    acc &= col[ids.w & 0xFFFFu];
+    acc &= col[ids.w >> 16];
+    return acc;
 }
 
 // One workgroup per tile.  The tile's bit-rows are copied to LDS once; each
 // wave then walks its share of the clauses.  The clause id and its literal
-// list are wave-uniform (scalar loads); lane L holds word L of the running AND.
+// list are wave-uniform (scalar loads, issued one block ahead); lane L holds
+// word L of the running AND.
 template <int NWAVES>
 __global__ __launch_bounds__(NWAVES * 64) void k_score_tiles(
     const uint32_t *__restrict__ tiles, TileGeom tg, int literals, int n_types, int C, int K,
-    const uint16_t *__restrict__ lists, int stride, const int32_t *__restrict__ count8,
-    const int32_t *__restrict__ wt, int tile0, int first_graph, int n_graphs, int32_t *__restrict__ class_sum) {
+    const uint16_t *__restrict__ lists, int stride, const int32_t *__restrict__ wt, int tile0, int first_graph,
+    int n_graphs, int32_t *__restrict__ class_sum) {
     extern __shared__ uint32_t lds[];
     const int tw = tg.tw;
     uint32_t *bt = lds;
@@ -145,44 +160,50 @@ __global__ __launch_bounds__(NWAVES * 64) void k_score_tiles(
 
     const bool active = lane < tw;
     const uint32_t *col = bt + (active ? lane : 0);
-    for (int c = wave; c < C; c += NWAVES) {
+    const int stride4 = stride >> 3;  // list stride in 16-byte blocks
+    const uint4 *all = reinterpret_cast<const uint4 *>(lists);
+
+    int c = wave;
+    uint4 head = all[(int64_t)(c < C ? c : 0) * stride4];
+    while (c < C) {
+        const int cn = c + NWAVES;
+        const uint4 *lp = all + (int64_t)c * stride4;
+        const uint4 head_next = all[(int64_t)(cn < C ? cn : c) * stride4];  // next clause, fetched early
+        uint4 block = lp[1];
+        const int nb = head.x & 0xFFFFu;
         uint32_t acc = active ? col[(literals + c % n_types) * tw] : 0u;
-        const int cnt = count8[c];
-        const uint4 *lp = reinterpret_cast<const uint4 *>(lists + (int64_t)c * stride);
-        for (int j = 0; j < cnt; j += 8) {
-            uint4 ids = lp[j >> 3];
-            acc &= col[(ids.x & 0xFFFFu) * tw];
-            acc &= col[(ids.x >> 16) * tw];
-            acc &= col[(ids.y & 0xFFFFu) * tw];
-            acc &= col[(ids.y >> 16) * tw];
-            acc &= col[(ids.z & 0xFFFFu) * tw];
-            acc &= col[(ids.z >> 16) * tw];
-            acc &= col[(ids.w & 0xFFFFu) * tw];
-            acc &= col[(ids.w >> 16) * tw];
+        acc = and8(acc, col, head, true);
+        for (int j = 1; j < nb; ++j) {
+            const uint4 ahead = lp[j + 1];
             if (__ballot(acc != 0) == 0) break;  // false at every node slot of the tile
+            acc = and8(acc, col, block, false);
+            block = ahead;
         }
         const unsigned long long nz = __ballot(acc != 0);
-        if (nz == 0) continue;
-        if (tg.slot_words > 0) {
-            // graph j owns lanes [j*slot_words, (j+1)*slot_words)
-            unsigned long long mine = nz >> ((lane < tg.gpt ? lane : 0) * tg.slot_words);
-            if (tg.slot_words < 64) mine &= (1ull << tg.slot_words) - 1ull;
-            const unsigned long long gm = __ballot(lane < tg.gpt && mine != 0);
-            for (int p = lane; p < tg.gpt * K; p += 64) {
-                int j = p / K, k = p - j * K;
-                if ((gm >> j) & 1ull) atomicAdd(&sums[p], wt[(int64_t)c * K + k]);
-            }
-        } else {
-            // several graphs per word: walk the non-empty slots of this lane's word
-            const int per_word = 32 / tg.slot_bits;
-            const uint32_t slot_mask = (1u << tg.slot_bits) - 1u;  // slot_bits <= 16
-            while (acc) {
-                int sub = (__ffs(acc) - 1) / tg.slot_bits;
-                acc &= ~(slot_mask << (sub * tg.slot_bits));
-                int j = lane * per_word + sub;
-                for (int k = 0; k < K; ++k) atomicAdd(&sums[j * K + k], wt[(int64_t)c * K + k]);
+        if (nz != 0) {
+            if (tg.slot_words > 0) {
+                // graph j owns lanes [j*slot_words, (j+1)*slot_words)
+                unsigned long long mine = nz >> ((lane < tg.gpt ? lane : 0) * tg.slot_words);
+                if (tg.slot_words < 64) mine &= (1ull << tg.slot_words) - 1ull;
+                const unsigned long long gm = __ballot(lane < tg.gpt && mine != 0);
+                for (int p = lane; p < tg.gpt * K; p += 64) {
+                    int j = p / K, k = p - j * K;
+                    if ((gm >> j) & 1ull) atomicAdd(&sums[p], wt[(int64_t)c * K + k]);
+                }
+            } else {
+                // several graphs per word: walk the non-empty slots of this lane's word
+                const int per_word = 32 / tg.slot_bits;
+                const uint32_t slot_mask = (1u << tg.slot_bits) - 1u;  // slot_bits <= 16
+                while (acc) {
+                    int sub = (__ffs(acc) - 1) / tg.slot_bits;
+                    acc &= ~(slot_mask << (sub * tg.slot_bits));
+                    int j = lane * per_word + sub;
+                    for (int k = 0; k < K; ++k) atomicAdd(&sums[j * K + k], wt[(int64_t)c * K + k]);
+                }
             }
         }
+        head = head_next;
+        c = cn;
     }
     __syncthreads();
     const int64_t g0 = (int64_t)tile * tg.gpt;

@@ -189,6 +189,17 @@ int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *st
             int32_t first_example, int32_t n_examples, uint64_t first_step, void *workspace,
             size_t workspace_bytes, void *stream);
 
+/* ---- measurement -------------------------------------------------------- */
+
+/* No counterpart in the reference.  While enabled, gtm_score / gtm_fit bracket
+ * each launch of their clause-evaluation kernel (the dominant kernel) with HIP
+ * events on the caller's stream (at most 512 launches are kept).
+ * gtm_profile_read() waits for those events, returns the kernel's name, the
+ * number of launches seen and their summed duration, and clears the record.
+ * Not thread-safe; meant for the benchmark. */
+int gtm_profile_enable(int on);
+int gtm_profile_read(const char **kernel_name, int32_t *launches, double *total_ms);
+
 #ifdef __cplusplus
 }
 #endif
