@@ -604,11 +604,16 @@ int validate_state(const gtm_config *cfg, const gtm_state *s) {
     return GTM_OK;
 }
 
+// Words of bit rows in a tile buffer, padded so that the row counts after them are 8-byte aligned.
+size_t tiles_words(const TileGeom &tg) { return ((size_t)tg.n_tiles * tg.rows * tg.tw + 1) & ~(size_t)1; }
+
 // Depth-1 inference on literal-major tiles (see score_tiles.h).
 int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
                    const ScoreWs &w, int first, int n_graphs, int32_t *class_sum, hipStream_t st) {
-    hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB)), dim3(TPB), 0, st, s->ta_state, d.C, d.LA, d.B,
-                       d.filter, d.K, s->clause_weights, tg.rows - 1, tg.tw, w.list_stride, w.lists, w.wt);
+    const uint32_t *order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
+    hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C, d.LA,
+                       d.B, d.filter, d.K, s->clause_weights, cfg->literals, tg.rows - 1, tg.tw, w.list_stride, order,
+                       w.lists, w.wt);
     if (int rc = check_launch("compile_clauses")) return rc;
     constexpr int NW = 16;
     size_t lds = (size_t)tg.rows * tg.tw * 4 + (size_t)tg.gpt * d.K * 4;
@@ -836,7 +841,8 @@ size_t gtm_tiles_bytes(const gtm_config *cfg, const gtm_graphs *graphs) {
     TileGeom tg = tile_geometry(cfg->literals, graphs->number_of_node_types, graphs->max_number_of_graph_nodes,
                                 graphs->number_of_graphs, d.K);
     if (!tg.ok) return 0;
-    return (size_t)tg.n_tiles * tg.rows * tg.tw * 4;
+    // bit rows, one 64-bit population count per row, the literal order
+    return tiles_words(tg) * 4 + (size_t)tg.rows * 8 + (size_t)cfg->literals * 4;
 }
 
 int gtm_build_tiles(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *tiles, void *stream) {
@@ -847,11 +853,22 @@ int gtm_build_tiles(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *t
     TileGeom tg = tile_geometry(cfg->literals, graphs->number_of_node_types, graphs->max_number_of_graph_nodes,
                                 graphs->number_of_graphs, d.K);
     if (!tg.ok) return fail(GTM_ERR_INVALID, "this data set's shape has no tile layout (gtm_tiles_bytes() == 0)");
+    hipStream_t st = (hipStream_t)stream;
     int64_t total = (int64_t)tg.n_tiles * tg.rows * tg.tw;
-    hipLaunchKernelGGL(k_build_tiles, dim3(blocks_for(total, TPB)), dim3(TPB), 0, (hipStream_t)stream, graphs->X,
-                       graphs->node_type, graphs->node_index, graphs->number_of_graph_nodes, graphs->number_of_graphs,
-                       d.LA, cfg->literals, graphs->number_of_node_types, tg, total, tiles);
-    return check_launch("build_tiles");
+    hipLaunchKernelGGL(k_build_tiles, dim3(blocks_for(total, TPB)), dim3(TPB), 0, st, graphs->X, graphs->node_type,
+                       graphs->node_index, graphs->number_of_graph_nodes, graphs->number_of_graphs, d.LA,
+                       cfg->literals, graphs->number_of_node_types, tg, total, tiles);
+    if (int rc = check_launch("build_tiles")) return rc;
+    int32_t *counts = (int32_t *)(tiles + tiles_words(tg));
+    hipLaunchKernelGGL(k_fill_i32, dim3(blocks_for(tg.rows * 2, TPB)), dim3(TPB), 0, st, counts, (int64_t)tg.rows * 2, 0);
+    if (int rc = check_launch("fill")) return rc;
+    int64_t total_rows = (int64_t)tg.n_tiles * tg.rows;
+    hipLaunchKernelGGL(k_row_counts, dim3(blocks_for(total_rows, TPB)), dim3(TPB), 0, st, tiles, tg, total_rows,
+                       (unsigned long long *)counts);
+    if (int rc = check_launch("row_counts")) return rc;
+    hipLaunchKernelGGL(k_row_order, dim3(blocks_for(cfg->literals, TPB)), dim3(TPB), 0, st,
+                       (const unsigned long long *)counts, cfg->literals, (uint32_t *)(counts + (size_t)tg.rows * 2));
+    return check_launch("row_order");
 }
 
 size_t gtm_score_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs, int32_t batch) {

@@ -97,30 +97,67 @@ __global__ void k_build_tiles(const uint32_t *__restrict__ X, const uint32_t *__
     tiles[i] = out;
 }
 
-// Per call: each clause's included literals as a list of 16-bit LDS word
-// offsets (row * tw), in blocks of 8 entries (one 16-byte scalar load each).
-// Entry 0 of the first block is the number of blocks; unused entries point at
-// the all-ones row.  Also the weights clause-major.
+// Number of set bits of every row over all tiles (how often a literal holds in
+// this data set); row_count[rows], zeroed by the caller.
+__global__ void k_row_counts(const uint32_t *__restrict__ tiles, TileGeom tg, int64_t total_rows,
+                             unsigned long long *__restrict__ row_count) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total_rows) return;
+    int row = (int)(i % tg.rows);
+    const uint32_t *p = tiles + i * tg.tw;
+    unsigned long long n = 0;
+    for (int w = 0; w < tg.tw; ++w) n += __popc(p[w]);
+    if (n) atomicAdd(&row_count[row], n);
+}
+
+// Literal rows ordered by how often they hold in the data set, rarest first:
+// order[r] = literal with rank r under the key (row_count, literal).  One
+// thread per literal counts the keys below its own.
+__global__ void k_row_order(const unsigned long long *__restrict__ row_count, int literals,
+                            uint32_t *__restrict__ order) {
+    int l = blockIdx.x * blockDim.x + threadIdx.x;
+    if (l >= literals) return;
+    unsigned long long mine = row_count[l];
+    int rank = 0;
+    for (int m = 0; m < literals; ++m) {
+        unsigned long long other = row_count[m];
+        rank += (other < mine) || (other == mine && m < l);
+    }
+    order[rank] = (uint32_t)l;
+}
+
+// Per call, one wave per clause: the clause's included literals as a list of
+// 16-bit LDS word offsets (row * tw) in blocks of 8 entries (one 16-byte scalar
+// load each).  Entry 0 of the first block is the number of blocks; unused
+// entries point at the all-ones row.  The literals are emitted in `order`, so
+// the ones that hold least often come first and the running AND dies (and the
+// walk stops) as early as it can; the order does not change the result.  Also
+// the weights clause-major.
 __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int LA, int B, uint32_t filter, int K,
-                                  const int32_t *__restrict__ weights, int ones_row, int tw, int stride,
-                                  uint16_t *__restrict__ lists, int32_t *__restrict__ wt) {
-    int c = blockIdx.x * blockDim.x + threadIdx.x;
+                                  const int32_t *__restrict__ weights, int literals, int ones_row, int tw,
+                                  int stride, const uint32_t *__restrict__ order, uint16_t *__restrict__ lists,
+                                  int32_t *__restrict__ wt) {
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (c >= C) return;
     uint16_t *list = lists + (int64_t)c * stride;
-    int n = 1;
-    for (int w = 0; w < LA; ++w) {
-        uint32_t m = bank[((int64_t)c * LA + w) * B + (B - 1)];
-        if (w == LA - 1) m &= filter;
-        while (m) {
-            int b = __ffs(m) - 1;
-            m &= m - 1;
-            list[n++] = (uint16_t)((w * 32 + b) * tw);
-        }
+    const uint32_t *inc = bank + (int64_t)c * LA * B + (B - 1);
+    int n = 1;  // entry 0 is the header
+    for (int r0 = 0; r0 < literals; r0 += 64) {
+        int r = r0 + lane;
+        uint32_t lit = r < literals ? order[r] : 0u;
+        uint32_t w = lit >> 5;
+        uint32_t word = inc[(int64_t)w * B];
+        if ((int)w == LA - 1) word &= filter;
+        bool included = r < literals && ((word >> (lit & 31)) & 1u);
+        unsigned long long mask = __ballot(included);
+        if (included) list[n + __popcll(mask & ((1ull << lane) - 1ull))] = (uint16_t)(lit * tw);
+        n += __popcll(mask);
     }
-    int padded = (n + 7) & ~7;
-    for (int i = n; i < padded + 8; ++i) list[i] = (uint16_t)(ones_row * tw);  // one block of slack for prefetch
-    list[0] = (uint16_t)(padded >> 3);
-    for (int k = 0; k < K; ++k) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
+    const int padded = (n + 7) & ~7;
+    for (int i = n + lane; i < padded + 8; i += 64) list[i] = (uint16_t)(ones_row * tw);  // + one block of slack
+    if (lane == 0) list[0] = (uint16_t)(padded >> 3);
+    for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
 }
 
 __device__ __forceinline__ uint32_t and8(uint32_t acc, const uint32_t *col, uint4 ids, bool skip_first) {
@@ -163,15 +200,27 @@ __global__ __launch_bounds__(NWAVES * 64) void k_score_tiles(
     const int stride4 = stride >> 3;  // list stride in 16-byte blocks
     const uint4 *all = reinterpret_cast<const uint4 *>(lists);
 
+    // lane p < gpt*K adds weight k = p % K to graph j = p / K of the tile
+    const int pairs = tg.gpt * K;
+    const int my_j = lane / K, my_k = lane - my_j * K;
+    const bool pair_lane = tg.slot_words > 0 && lane < pairs;
+    const int my_shift = (lane < tg.gpt ? lane : 0) * tg.slot_words;
+    const unsigned long long slot_lanes = tg.slot_words >= 64 ? ~0ull : (1ull << tg.slot_words) - 1ull;
+
     int c = wave;
+    int type_row = literals + c % n_types;
+    const int type_step = NWAVES % n_types;
     uint4 head = all[(int64_t)(c < C ? c : 0) * stride4];
     while (c < C) {
         const int cn = c + NWAVES;
         const uint4 *lp = all + (int64_t)c * stride4;
         const uint4 head_next = all[(int64_t)(cn < C ? cn : c) * stride4];  // next clause, fetched early
         uint4 block = lp[1];
+        const int my_weight = pair_lane ? wt[(int64_t)c * K + my_k] : 0;  // needed only if the clause fires
         const int nb = head.x & 0xFFFFu;
-        uint32_t acc = active ? col[(literals + c % n_types) * tw] : 0u;
+        uint32_t acc = active ? col[type_row * tw] : 0u;
+        type_row += type_step;
+        if (type_row >= literals + n_types) type_row -= n_types;
         acc = and8(acc, col, head, true);
         for (int j = 1; j < nb; ++j) {
             const uint4 ahead = lp[j + 1];
@@ -183,10 +232,9 @@ __global__ __launch_bounds__(NWAVES * 64) void k_score_tiles(
         if (nz != 0) {
             if (tg.slot_words > 0) {
                 // graph j owns lanes [j*slot_words, (j+1)*slot_words)
-                unsigned long long mine = nz >> ((lane < tg.gpt ? lane : 0) * tg.slot_words);
-                if (tg.slot_words < 64) mine &= (1ull << tg.slot_words) - 1ull;
-                const unsigned long long gm = __ballot(lane < tg.gpt && mine != 0);
-                for (int p = lane; p < tg.gpt * K; p += 64) {
+                const unsigned long long gm = __ballot(lane < tg.gpt && ((nz >> my_shift) & slot_lanes) != 0);
+                if (pair_lane && ((gm >> my_j) & 1ull)) atomicAdd(&sums[lane], my_weight);
+                for (int p = lane + 64; p < pairs; p += 64) {
                     int j = p / K, k = p - j * K;
                     if ((gm >> j) & 1ull) atomicAdd(&sums[p], wt[(int64_t)c * K + k]);
                 }
