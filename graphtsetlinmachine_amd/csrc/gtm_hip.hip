@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <cstdlib>
 #include <string>
 
 #include "../../include/gtm_abi.h"
@@ -462,7 +463,7 @@ Key key_of(const gtm_config *cfg) { return Key{(uint32_t)(cfg->seed & 0xFFFFFFFF
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct ScoreWs {
-    uint16_t *lists;     // [C][list_stride]  (literal-major tile path)
+    uint32_t *lists;     // [C][list_stride]  (literal-major tile path)
     int32_t *wt;         // [C][K]
     int list_stride;
     uint32_t *inc_t;     // [max(LA,MC)][C]
@@ -481,8 +482,8 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base)
         off += align_up(bytes);
         return p;
     };
-    w.list_stride = ((cfg->literals + 1 + 7) & ~7) + 8;  // header + literals, padded to blocks of 8, + 1 block
-    w.lists = (uint16_t *)take((size_t)d.C * w.list_stride * 2 + 16);
+    w.list_stride = ((cfg->literals + 2 + 31) & ~31);  // header + type row + literals, padded to 32 entries
+    w.lists = (uint32_t *)take((size_t)d.C * w.list_stride * 4);
     w.wt = (int32_t *)take((size_t)d.C * d.K * 4);
     w.inc_t = (uint32_t *)take((size_t)chunks * d.C * 4);
     w.bitmap_a = (uint32_t *)take((size_t)batch * d.C * d.NC * 4);
@@ -608,30 +609,50 @@ int validate_state(const gtm_config *cfg, const gtm_state *s) {
 size_t tiles_words(const TileGeom &tg) { return ((size_t)tg.n_tiles * tg.rows * tg.tw + 1) & ~(size_t)1; }
 
 // Depth-1 inference on literal-major tiles (see score_tiles.h).
-int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
-                   const ScoreWs &w, int first, int n_graphs, int32_t *class_sum, hipStream_t st) {
-    const uint32_t *order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
-    hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C, d.LA,
-                       d.B, d.filter, d.K, s->clause_weights, cfg->literals, tg.rows - 1, tg.tw, w.list_stride, order,
-                       w.lists, w.wt);
-    if (int rc = check_launch("compile_clauses")) return rc;
-    constexpr int NW = 16;
-    size_t lds = (size_t)tg.rows * tg.tw * 4 + (size_t)tg.gpt * d.K * 4;
+int max_lane_words() {
+    const char *e = getenv("GTM_TILE_LANE_WORDS");  // 1, 2 or 4: upper bound on words per lane (tuning aid)
+    int v = e ? atoi(e) : 4;
+    return v == 1 || v == 2 ? v : 4;
+}
+
+TileGeom geometry_for(const gtm_config *cfg, const gtm_graphs *g, int classes) {
+    return tile_geometry(cfg->literals, g->number_of_node_types, g->max_number_of_graph_nodes, g->number_of_graphs,
+                         classes, max_lane_words());
+}
+
+template <int NW, int LW>
+int launch_score_tiles(const Dims &d, const gtm_graphs *g, const TileGeom &tg, const ScoreWs &w, int first,
+                       int n_graphs, int32_t *class_sum, hipStream_t st) {
+    size_t lds = tile_lds_bytes(tg, d.K);
     static thread_local size_t lds_set = 0;
     if (lds > lds_set) {
-        hipError_t e = hipFuncSetAttribute((const void *)k_score_tiles<NW>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)lds);
+        hipError_t e = hipFuncSetAttribute((const void *)k_score_tiles<NW, LW>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
         lds_set = lds;
     }
     int tile0 = first / tg.gpt, tile1 = (first + n_graphs - 1) / tg.gpt;
     profile_start("k_score_tiles", st);
-    hipLaunchKernelGGL((k_score_tiles<NW>), dim3(tile1 - tile0 + 1), dim3(NW * 64), lds, st, g->tiles, tg, cfg->literals,
-                       g->number_of_node_types, d.C, d.K, w.lists, w.list_stride, w.wt, tile0, first, n_graphs,
-                       class_sum);
+    hipLaunchKernelGGL((k_score_tiles<NW, LW>), dim3(tile1 - tile0 + 1), dim3(NW * 64), lds, st, g->tiles, tg, d.C, d.K,
+                       w.lists, w.list_stride, w.wt, tile0, first, n_graphs, class_sum);
     if (int rc = check_launch("score_tiles")) return rc;
     profile_stop(st);
     return GTM_OK;
+}
+
+int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
+                   const ScoreWs &w, int first, int n_graphs, int32_t *class_sum, hipStream_t st) {
+    const uint32_t *order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
+    hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C, d.LA,
+                       d.B, d.filter, d.K, s->clause_weights, cfg->literals, g->number_of_node_types, tg.tw,
+                       w.list_stride, order, w.lists, w.wt);
+    if (int rc = check_launch("compile_clauses")) return rc;
+    constexpr int NW = 16;
+    switch (tg.lw) {
+        case 1: return launch_score_tiles<NW, 1>(d, g, tg, w, first, n_graphs, class_sum, st);
+        case 2: return launch_score_tiles<NW, 2>(d, g, tg, w, first, n_graphs, class_sum, st);
+        default: return launch_score_tiles<NW, 4>(d, g, tg, w, first, n_graphs, class_sum, st);
+    }
 }
 
 }  // namespace
@@ -838,8 +859,7 @@ int gtm_profile_read(const char **kernel_name, int32_t *launches, double *total_
 size_t gtm_tiles_bytes(const gtm_config *cfg, const gtm_graphs *graphs) {
     Dims d;
     if (validate(cfg, &d) || !graphs || graphs->number_of_graphs < 1 || graphs->number_of_node_types < 1) return 0;
-    TileGeom tg = tile_geometry(cfg->literals, graphs->number_of_node_types, graphs->max_number_of_graph_nodes,
-                                graphs->number_of_graphs, d.K);
+    TileGeom tg = geometry_for(cfg, graphs, d.K);
     if (!tg.ok) return 0;
     // bit rows, one 64-bit population count per row, the literal order
     return tiles_words(tg) * 4 + (size_t)tg.rows * 8 + (size_t)cfg->literals * 4;
@@ -850,8 +870,7 @@ int gtm_build_tiles(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *t
     if (int rc = validate(cfg, &d)) return rc;
     if (int rc = validate_graphs(cfg, graphs, 0, 0)) return rc;
     if (!tiles) return fail(GTM_ERR_INVALID, "tiles is NULL");
-    TileGeom tg = tile_geometry(cfg->literals, graphs->number_of_node_types, graphs->max_number_of_graph_nodes,
-                                graphs->number_of_graphs, d.K);
+    TileGeom tg = geometry_for(cfg, graphs, d.K);
     if (!tg.ok) return fail(GTM_ERR_INVALID, "this data set's shape has no tile layout (gtm_tiles_bytes() == 0)");
     hipStream_t st = (hipStream_t)stream;
     int64_t total = (int64_t)tg.n_tiles * tg.rows * tg.tw;
@@ -892,8 +911,7 @@ int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *
         return fail(GTM_ERR_INVALID, "workspace of %zu bytes needed, %zu given", w.bytes, workspace_bytes);
     hipStream_t st = (hipStream_t)stream;
     if (cfg->depth == 1 && graphs->tiles && n_graphs > 0) {
-        TileGeom tg = tile_geometry(cfg->literals, graphs->number_of_node_types, graphs->max_number_of_graph_nodes,
-                                    graphs->number_of_graphs, d.K);
+        TileGeom tg = geometry_for(cfg, graphs, d.K);
         if (tg.ok) return score_on_tiles(d, cfg, graphs, state, tg, w, first_graph, n_graphs, class_sum, st);
     }
     for (int done = 0; done < n_graphs; done += batch) {

@@ -18,43 +18,58 @@
 //     last row                  all ones (pads literal lists)
 //   node slots: graph j of the tile owns `slot_bits` consecutive bits starting
 //   at j * slot_bits; slot_bits is a power of two < 32 for tiny graphs, else a
-//   whole number of 32-bit words.
+//   whole number of 32-bit words (a multiple of the words one lane holds).
 #pragma once
 
 struct TileGeom {
-    int slot_bits;   // bits per graph slot
-    int slot_words;  // words per graph slot (0 when slot_bits < 32)
-    int gpt;         // graphs per tile
-    int tw;          // words per tile row (<= 64)
-    int rows;        // LITERALS + node types + 1
+    int slot_bits;        // bits per graph slot
+    int slot_words;       // words per graph slot (0 when slot_bits < 32)
+    int gpt;              // graphs per tile
+    int tw;               // words per tile row
+    int rows;             // LITERALS + node types + 1
     int n_tiles;
-    int ok;          // geometry supported by the fused kernel
+    int lw;               // words of a row held by one lane (1, 2 or 4)
+    int lanes_per_graph;  // slot_words / lw (0 when slot_bits < 32)
+    int ok;               // geometry supported by the fused kernel
 };
 
-constexpr int TILE_MAX_WORDS = 64;
 constexpr size_t TILE_LDS_BUDGET = 156 * 1024;  // of the 160 KB per CU
+constexpr int TILE_LDS_PAD_WORDS = 256;         // readable words after the last row
 
-inline TileGeom tile_geometry(int literals, int n_types, int max_nodes, int n_graphs, int classes) {
-    TileGeom g{};
+inline size_t tile_lds_bytes(const TileGeom &g, int classes) {
+    return ((size_t)g.rows * g.tw + TILE_LDS_PAD_WORDS + (size_t)g.gpt * classes) * 4;
+}
+
+// The widest lanes (most graphs per wave instruction) whose tile fits in LDS.
+inline TileGeom tile_geometry(int literals, int n_types, int max_nodes, int n_graphs, int classes, int max_lw = 4) {
+    TileGeom last{};
     if (max_nodes < 1) max_nodes = 1;
-    if (max_nodes <= 16) {
-        int s = 1;
-        while (s < max_nodes) s <<= 1;
-        g.slot_bits = s;
-        g.slot_words = 0;
-        g.tw = TILE_MAX_WORDS;
-        g.gpt = TILE_MAX_WORDS * 32 / s;
-    } else {
-        g.slot_words = (max_nodes - 1) / 32 + 1;
-        g.slot_bits = g.slot_words * 32;
-        g.gpt = g.slot_words <= TILE_MAX_WORDS ? TILE_MAX_WORDS / g.slot_words : 0;
-        g.tw = g.gpt * g.slot_words;
+    for (int lw = max_lw; lw >= 1; lw >>= 1) {
+        TileGeom g{};
+        g.lw = lw;
+        const int max_words = 64 * lw;
+        if (max_nodes <= 16) {
+            int s = 1;
+            while (s < max_nodes) s <<= 1;
+            g.slot_bits = s;
+            g.tw = max_words;
+            g.gpt = max_words * 32 / s;
+        } else {
+            g.slot_words = ((max_nodes - 1) / 32 + 1 + lw - 1) / lw * lw;
+            g.slot_bits = g.slot_words * 32;
+            g.lanes_per_graph = g.slot_words / lw;
+            g.gpt = g.slot_words <= max_words ? max_words / g.slot_words : 0;
+            g.tw = g.gpt * g.slot_words;
+            if (g.tw & 3) g.tw = (g.tw + 3) & ~3;  // rows stay 16-byte aligned
+        }
+        g.rows = literals + n_types + 1;
+        g.n_tiles = g.gpt > 0 ? (n_graphs + g.gpt - 1) / g.gpt : 0;
+        g.ok = g.gpt > 0 && tile_lds_bytes(g, classes) <= TILE_LDS_BUDGET;
+        if (g.ok) return g;
+        last = g;
     }
-    g.rows = literals + n_types + 1;
-    g.n_tiles = g.gpt > 0 ? (n_graphs + g.gpt - 1) / g.gpt : 0;
-    size_t lds = (size_t)g.rows * g.tw * 4 + (size_t)g.gpt * classes * 4;
-    g.ok = g.gpt > 0 && lds <= TILE_LDS_BUDGET && literals < 65535 - 8;
-    return g;
+    last.ok = 0;
+    return last;
 }
 
 // One thread per tile word: gathers its 32 node slots.
@@ -70,7 +85,9 @@ __global__ void k_build_tiles(const uint32_t *__restrict__ X, const uint32_t *__
     int tile = (int)(rest / tg.rows);
     uint32_t out = 0;
     if (row == tg.rows - 1) {
-        out = 0xFFFFFFFFu;
+        // all ones over the graph slots; words that only pad the row stay 0 so
+        // that they never keep a clause alive
+        out = (tg.slot_words == 0 || w < tg.gpt * tg.slot_words) ? 0xFFFFFFFFu : 0u;
     } else {
         for (int b = 0; b < 32; ++b) {
             int pos = w * 32 + b;
@@ -126,23 +143,27 @@ __global__ void k_row_order(const unsigned long long *__restrict__ row_count, in
     order[rank] = (uint32_t)l;
 }
 
-// Per call, one wave per clause: the clause's included literals as a list of
-// 16-bit LDS word offsets (row * tw) in blocks of 8 entries (one 16-byte scalar
-// load each).  Entry 0 of the first block is the number of blocks; unused
-// entries point at the all-ones row.  The literals are emitted in `order`, so
-// the ones that hold least often come first and the running AND dies (and the
-// walk stops) as early as it can; the order does not change the result.  Also
-// the weights clause-major.
+// Per call, one wave per clause: the rows the clause ANDs together, as 32-bit
+// LDS byte offsets (row * tw * 4).  Entry 0 = number of 8-entry blocks in use,
+// entry 1 = the row of the clause's node type (kernels.py:447), then its
+// included literals in `order`: the ones that hold least often come first, so
+// the running AND dies (and the walk stops) as early as it can; the order does
+// not change the result.  The list starts with a chunk of 32 entries that the
+// scoring kernel fetches one clause ahead; unused entries point at the
+// all-ones row.  Also the weights clause-major.
 __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int LA, int B, uint32_t filter, int K,
-                                  const int32_t *__restrict__ weights, int literals, int ones_row, int tw,
-                                  int stride, const uint32_t *__restrict__ order, uint16_t *__restrict__ lists,
+                                  const int32_t *__restrict__ weights, int literals, int n_types, int tw,
+                                  int stride, const uint32_t *__restrict__ order, uint32_t *__restrict__ lists,
                                   int32_t *__restrict__ wt) {
     const int lane = threadIdx.x & 63;
     const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (c >= C) return;
-    uint16_t *list = lists + (int64_t)c * stride;
+    const uint32_t row_bytes = (uint32_t)tw * 4u;
+    const uint32_t ones = (uint32_t)(literals + n_types) * row_bytes;
+    uint32_t *list = lists + (int64_t)c * stride;
     const uint32_t *inc = bank + (int64_t)c * LA * B + (B - 1);
-    int n = 1;  // entry 0 is the header
+    if (lane == 0) list[1] = (uint32_t)(literals + c % n_types) * row_bytes;
+    int n = 2;
     for (int r0 = 0; r0 < literals; r0 += 64) {
         int r = r0 + lane;
         uint32_t lit = r < literals ? order[r] : 0u;
@@ -151,107 +172,191 @@ __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int 
         if ((int)w == LA - 1) word &= filter;
         bool included = r < literals && ((word >> (lit & 31)) & 1u);
         unsigned long long mask = __ballot(included);
-        if (included) list[n + __popcll(mask & ((1ull << lane) - 1ull))] = (uint16_t)(lit * tw);
+        if (included) list[n + __popcll(mask & ((1ull << lane) - 1ull))] = lit * row_bytes;
         n += __popcll(mask);
     }
     const int padded = (n + 7) & ~7;
-    for (int i = n + lane; i < padded + 8; i += 64) list[i] = (uint16_t)(ones_row * tw);  // + one block of slack
-    if (lane == 0) list[0] = (uint16_t)(padded >> 3);
+    const int fill_to = padded < 32 ? 32 : padded;
+    for (int i = n + lane; i < fill_to; i += 64) list[i] = ones;
+    if (lane == 0) list[0] = (uint32_t)(padded >> 3);
     for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
 }
 
-__device__ __forceinline__ uint32_t and8(uint32_t acc, const uint32_t *col, uint4 ids, bool skip_first) {
-    if (!skip_first) acc &= col[ids.x & 0xFFFFu];
-    acc &= col[ids.x >> 16];
-    acc &= col[ids.y & 0xFFFFu];
-    acc &= col[ids.y >> 16];
-    acc &= col[ids.z & 0xFFFFu];
-    acc &= col[ids.z >> 16];
-    acc &= col[ids.w & 0xFFFFu];
-    acc &= col[ids.w >> 16];
-    return acc;
-}
+struct alignas(32) Block8 {
+    uint32_t v[8];
+};
+struct alignas(128) Chunk32 {
+    uint32_t v[32];
+};
+
+// LW words of a tile row per lane, with the load width that goes with it.
+template <int LW>
+struct LaneWords;
+template <>
+struct LaneWords<1> {
+    uint32_t w[1];
+    __device__ __forceinline__ void load(const char *p) { w[0] = *reinterpret_cast<const uint32_t *>(p); }
+};
+template <>
+struct LaneWords<2> {
+    uint32_t w[2];
+    __device__ __forceinline__ void load(const char *p) {
+        uint2 v = *reinterpret_cast<const uint2 *>(p);
+        w[0] = v.x;
+        w[1] = v.y;
+    }
+};
+template <>
+struct LaneWords<4> {
+    uint32_t w[4];
+    __device__ __forceinline__ void load(const char *p) {
+        uint4 v = *reinterpret_cast<const uint4 *>(p);
+        w[0] = v.x;
+        w[1] = v.y;
+        w[2] = v.z;
+        w[3] = v.w;
+    }
+};
 
 // One workgroup per tile.  The tile's bit-rows are copied to LDS once; each
-// wave then walks its share of the clauses.  The clause id and its literal
-// list are wave-uniform (scalar loads, issued one block ahead); lane L holds
-// word L of the running AND.
-template <int NWAVES>
+// wave then walks its share of the clauses.  The clause id and its row list
+// are wave-uniform: the first 32 entries of a clause arrive by scalar loads
+// issued while the previous clause is being evaluated.  Lane L holds words
+// [L*LW, (L+1)*LW) of the running AND.
+template <int NWAVES, int LW>
 __global__ __launch_bounds__(NWAVES * 64) void k_score_tiles(
-    const uint32_t *__restrict__ tiles, TileGeom tg, int literals, int n_types, int C, int K,
-    const uint16_t *__restrict__ lists, int stride, const int32_t *__restrict__ wt, int tile0, int first_graph,
-    int n_graphs, int32_t *__restrict__ class_sum) {
+    const uint32_t *__restrict__ tiles, TileGeom tg, int C, int K, const uint32_t *__restrict__ lists, int stride,
+    const int32_t *__restrict__ wt, int tile0, int first_graph, int n_graphs, int32_t *__restrict__ class_sum) {
     extern __shared__ uint32_t lds[];
     const int tw = tg.tw;
     uint32_t *bt = lds;
-    int32_t *sums = (int32_t *)(lds + (size_t)tg.rows * tw);
+    int32_t *sums = (int32_t *)(lds + (size_t)tg.rows * tw + TILE_LDS_PAD_WORDS);
     const int tile = tile0 + blockIdx.x;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    const uint32_t *src = tiles + (int64_t)tile * tg.rows * tw;
-    for (int i = tid; i < tg.rows * tw; i += NWAVES * 64) bt[i] = src[i];
-    for (int i = tid; i < tg.gpt * K; i += NWAVES * 64) sums[i] = 0;
+    {  // tile -> LDS, 16 bytes per thread and trip, several loads in flight
+        const uint4 *src = reinterpret_cast<const uint4 *>(tiles + (int64_t)tile * tg.rows * tw);
+        uint4 *dst = reinterpret_cast<uint4 *>(bt);
+        const int n4 = (tg.rows * tw) >> 2;  // tw is a multiple of 4
+        for (int i = tid; i < n4; i += NWAVES * 64 * 4) {
+            uint4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int at = i + u * NWAVES * 64;
+                v[u] = at < n4 ? src[at] : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int at = i + u * NWAVES * 64;
+                if (at < n4) dst[at] = v[u];
+            }
+        }
+        for (int i = tid; i < TILE_LDS_PAD_WORDS + tg.gpt * K; i += NWAVES * 64) bt[tg.rows * tw + i] = 0;
+    }
     __syncthreads();
 
-    const bool active = lane < tw;
-    const uint32_t *col = bt + (active ? lane : 0);
-    const int stride4 = stride >> 3;  // list stride in 16-byte blocks
-    const uint4 *all = reinterpret_cast<const uint4 *>(lists);
+    // Lanes past the row width read the words after the row (inside the
+    // allocation) so that they fall on banks no other lane of the access uses;
+    // their running AND starts at 0 and stays 0.
+    const bool active = lane * LW < tw;
+    const char *col = reinterpret_cast<const char *>(bt + lane * LW);
 
     // lane p < gpt*K adds weight k = p % K to graph j = p / K of the tile
     const int pairs = tg.gpt * K;
     const int my_j = lane / K, my_k = lane - my_j * K;
     const bool pair_lane = tg.slot_words > 0 && lane < pairs;
-    const int my_shift = (lane < tg.gpt ? lane : 0) * tg.slot_words;
-    const unsigned long long slot_lanes = tg.slot_words >= 64 ? ~0ull : (1ull << tg.slot_words) - 1ull;
+    const int my_shift = (lane < tg.gpt ? lane : 0) * tg.lanes_per_graph;
+    const unsigned long long slot_lanes = tg.lanes_per_graph >= 64 ? ~0ull : (1ull << tg.lanes_per_graph) - 1ull;
 
-    int c = wave;
-    int type_row = literals + c % n_types;
-    const int type_step = NWAVES % n_types;
-    uint4 head = all[(int64_t)(c < C ? c : 0) * stride4];
-    while (c < C) {
-        const int cn = c + NWAVES;
-        const uint4 *lp = all + (int64_t)c * stride4;
-        const uint4 head_next = all[(int64_t)(cn < C ? cn : c) * stride4];  // next clause, fetched early
-        uint4 block = lp[1];
-        const int my_weight = pair_lane ? wt[(int64_t)c * K + my_k] : 0;  // needed only if the clause fires
-        const int nb = head.x & 0xFFFFu;
-        uint32_t acc = active ? col[type_row * tw] : 0u;
-        type_row += type_step;
-        if (type_row >= literals + n_types) type_row -= n_types;
-        acc = and8(acc, col, head, true);
-        for (int j = 1; j < nb; ++j) {
-            const uint4 ahead = lp[j + 1];
-            if (__ballot(acc != 0) == 0) break;  // false at every node slot of the tile
-            acc = and8(acc, col, block, false);
-            block = ahead;
-        }
-        const unsigned long long nz = __ballot(acc != 0);
-        if (nz != 0) {
-            if (tg.slot_words > 0) {
-                // graph j owns lanes [j*slot_words, (j+1)*slot_words)
-                const unsigned long long gm = __ballot(lane < tg.gpt && ((nz >> my_shift) & slot_lanes) != 0);
-                if (pair_lane && ((gm >> my_j) & 1ull)) atomicAdd(&sums[lane], my_weight);
-                for (int p = lane + 64; p < pairs; p += 64) {
-                    int j = p / K, k = p - j * K;
-                    if ((gm >> j) & 1ull) atomicAdd(&sums[p], wt[(int64_t)c * K + k]);
-                }
-            } else {
-                // several graphs per word: walk the non-empty slots of this lane's word
-                const int per_word = 32 / tg.slot_bits;
-                const uint32_t slot_mask = (1u << tg.slot_bits) - 1u;  // slot_bits <= 16
-                while (acc) {
-                    int sub = (__ffs(acc) - 1) / tg.slot_bits;
-                    acc &= ~(slot_mask << (sub * tg.slot_bits));
-                    int j = lane * per_word + sub;
-                    for (int k = 0; k < K; ++k) atomicAdd(&sums[j * K + k], wt[(int64_t)c * K + k]);
+    auto any_bit = [](const LaneWords<LW> &a) {
+        uint32_t m = a.w[0];
+#pragma unroll
+        for (int u = 1; u < LW; ++u) m |= a.w[u];
+        return m != 0;
+    };
+    auto and_row = [&](LaneWords<LW> &acc, uint32_t byte_offset) {
+        LaneWords<LW> r;
+        r.load(col + byte_offset);
+#pragma unroll
+        for (int u = 0; u < LW; ++u) acc.w[u] &= r.w[u];
+    };
+
+    auto evaluate = [&](const Chunk32 &head, const uint32_t *list, const int32_t *weights_of_clause) {
+        const int my_weight = pair_lane ? weights_of_clause[my_k] : 0;  // needed only if the clause fires
+        const int nb = (int)head.v[0];
+        LaneWords<LW> acc;
+#pragma unroll
+        for (int u = 0; u < LW; ++u) acc.w[u] = active ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+        for (int i = 1; i < 8; ++i) and_row(acc, head.v[i]);
+        // stop as soon as the clause is false at every node slot of the tile
+        if (nb > 1 && __ballot(any_bit(acc)) != 0) {
+#pragma unroll
+            for (int i = 8; i < 16; ++i) and_row(acc, head.v[i]);
+            if (nb > 2 && __ballot(any_bit(acc)) != 0) {
+#pragma unroll
+                for (int i = 16; i < 24; ++i) and_row(acc, head.v[i]);
+                if (nb > 3 && __ballot(any_bit(acc)) != 0) {
+#pragma unroll
+                    for (int i = 24; i < 32; ++i) and_row(acc, head.v[i]);
+                    const Block8 *bp = reinterpret_cast<const Block8 *>(list) + 4;
+                    for (int j = 4; j < nb && __ballot(any_bit(acc)) != 0; ++j) {
+                        const Block8 block = *bp++;
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) and_row(acc, block.v[i]);
+                    }
                 }
             }
         }
-        head = head_next;
-        c = cn;
+        const unsigned long long nz = __ballot(any_bit(acc));
+        if (nz == 0) return;
+        if (tg.slot_words > 0) {
+            // graph j owns lanes [j*lanes_per_graph, (j+1)*lanes_per_graph)
+            const unsigned long long gm = __ballot(lane < tg.gpt && ((nz >> my_shift) & slot_lanes) != 0);
+            if (pair_lane && ((gm >> my_j) & 1ull)) atomicAdd(&sums[lane], my_weight);
+            for (int p = lane + 64; p < pairs; p += 64) {
+                int j = p / K, k = p - j * K;
+                if ((gm >> j) & 1ull) atomicAdd(&sums[p], weights_of_clause[k]);
+            }
+        } else {
+            // several graphs per word: walk the non-empty slots of this lane's words
+            const int per_word = 32 / tg.slot_bits;
+            const uint32_t slot_mask = (1u << tg.slot_bits) - 1u;  // slot_bits <= 16
+#pragma unroll
+            for (int u = 0; u < LW; ++u) {
+                uint32_t m = acc.w[u];
+                while (m) {
+                    int sub = (__ffs(m) - 1) / tg.slot_bits;
+                    m &= ~(slot_mask << (sub * tg.slot_bits));
+                    int j = (lane * LW + u) * per_word + sub;
+                    for (int k = 0; k < K; ++k) atomicAdd(&sums[j * K + k], weights_of_clause[k]);
+                }
+            }
+        }
+    };
+
+    // Two clauses per trip so that the chunk fetched ahead never has to be
+    // copied.  Pointers step by NWAVES clauses; past the end they stay on the
+    // wave's last clause (a valid address whose data is not used).
+    const int64_t list_step = (int64_t)NWAVES * stride;
+    const int wt_step = NWAVES * K;
+    const int first = wave < C ? wave : 0;
+    const uint32_t *list_a = lists + (int64_t)first * stride;
+    const int32_t *wt_a = wt + (int64_t)first * K;
+    Chunk32 a = *reinterpret_cast<const Chunk32 *>(list_a);
+    for (int c = wave; c < C; c += 2 * NWAVES) {
+        const bool has_b = c + NWAVES < C;
+        const uint32_t *list_b = has_b ? list_a + list_step : list_a;
+        const int32_t *wt_b = has_b ? wt_a + wt_step : wt_a;
+        const Chunk32 b = *reinterpret_cast<const Chunk32 *>(list_b);
+        evaluate(a, list_a, wt_a);
+        const bool has_a = c + 2 * NWAVES < C;
+        list_a = has_a ? list_b + list_step : list_b;
+        wt_a = has_a ? wt_b + wt_step : wt_b;
+        a = *reinterpret_cast<const Chunk32 *>(list_a);
+        if (has_b) evaluate(b, list_b, wt_b);
     }
     __syncthreads();
     const int64_t g0 = (int64_t)tile * tg.gpt;
