@@ -23,6 +23,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
+# HBM bytes per graph that k_score_tiles moves on the convolutional workload, from rocprofv3 --pmc runs
+# (FETCH_SIZE x 2 KiB, the factor a 256 MiB copy kernel calibrates, + WRITE_SIZE x 1 KiB, over 10,000 graphs).
+MEASURED_TRAFFIC_BYTES_PER_GRAPH = {"convolutional_images": (72096.1 * 2 + 406.2) * 1024 / 10000}
+
 
 def parse():
     p = argparse.ArgumentParser()
@@ -31,7 +35,7 @@ def parse():
     p.add_argument("--warmup", type=int, default=3)
     p.add_argument("--workload", default="convolutional_images")
     p.add_argument("--graphs", type=int, default=10000, help="test graphs scored per step")
-    p.add_argument("--train-graphs", type=int, default=5000, help="training graphs used to produce the model state")
+    p.add_argument("--train-graphs", type=int, default=60000, help="training graphs used to produce the model state")
     p.add_argument("--train-epochs", type=int, default=1)
     p.add_argument("--cpu-sample", type=int, default=None, help="graphs timed on the CPU oracle")
     p.add_argument("--no-cpu", action="store_true")
@@ -127,7 +131,9 @@ def main():
     compulsory = (n_nodes * la * 4 + n_nodes * 4 + tm.number_of_outputs * 4) * graphs_per_launch
     roofline = {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": (round(MEASURED_TRAFFIC_BYTES_PER_GRAPH[args.workload] * graphs_per_launch)
+                    if args.workload in MEASURED_TRAFFIC_BYTES_PER_GRAPH and kernel_name == "k_score_tiles" else None),
         "kernel": kernel_name, "kernel_ms": round(kernel_ms, 4), "launches": launches,
         "graphs_per_launch": graphs_per_launch,
         "algorithmic_bytes_per_graph": b_eval,

@@ -482,7 +482,8 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base)
         off += align_up(bytes);
         return p;
     };
-    w.list_stride = ((cfg->literals + 2 + 31) & ~31);  // header + type row + literals, padded to 32 entries
+    // header + type row + literals, padded to 32 entries, + 32 entries that the kernel may fetch ahead unused
+    w.list_stride = ((cfg->literals + 2 + 31) & ~31) + 32;
     w.lists = (uint32_t *)take((size_t)d.C * w.list_stride * 4);
     w.wt = (int32_t *)take((size_t)d.C * d.K * 4);
     w.inc_t = (uint32_t *)take((size_t)chunks * d.C * 4);

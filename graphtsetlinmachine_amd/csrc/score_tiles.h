@@ -176,7 +176,7 @@ __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int 
         n += __popcll(mask);
     }
     const int padded = (n + 7) & ~7;
-    const int fill_to = padded < 32 ? 32 : padded;
+    const int fill_to = padded < 32 ? 32 : (padded + 15) & ~15;
     for (int i = n + lane; i < fill_to; i += 64) list[i] = ones;
     if (lane == 0) list[0] = (uint32_t)(padded >> 3);
     for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
@@ -184,6 +184,9 @@ __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int 
 
 struct alignas(32) Block8 {
     uint32_t v[8];
+};
+struct alignas(64) Chunk16 {
+    uint32_t v[16];
 };
 struct alignas(128) Chunk32 {
     uint32_t v[32];
@@ -293,6 +296,9 @@ __global__ __launch_bounds__(NWAVES * 64) void k_score_tiles(
         for (int i = 1; i < 8; ++i) and_row(acc, head.v[i]);
         // stop as soon as the clause is false at every node slot of the tile
         if (nb > 1 && __ballot(any_bit(acc)) != 0) {
+            // entries past the first chunk, 16 at a time, requested one step before they are needed
+            const Chunk16 *tp = reinterpret_cast<const Chunk16 *>(list) + 2;
+            Chunk16 tail = *tp;
 #pragma unroll
             for (int i = 8; i < 16; ++i) and_row(acc, head.v[i]);
             if (nb > 2 && __ballot(any_bit(acc)) != 0) {
@@ -301,11 +307,15 @@ __global__ __launch_bounds__(NWAVES * 64) void k_score_tiles(
                 if (nb > 3 && __ballot(any_bit(acc)) != 0) {
 #pragma unroll
                     for (int i = 24; i < 32; ++i) and_row(acc, head.v[i]);
-                    const Block8 *bp = reinterpret_cast<const Block8 *>(list) + 4;
-                    for (int j = 4; j < nb && __ballot(any_bit(acc)) != 0; ++j) {
-                        const Block8 block = *bp++;
+                    for (int j = 4; j < nb && __ballot(any_bit(acc)) != 0; j += 2) {
+                        const Chunk16 ahead = *++tp;
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) and_row(acc, block.v[i]);
+                        for (int i = 0; i < 8; ++i) and_row(acc, tail.v[i]);
+                        if (j + 1 < nb && __ballot(any_bit(acc)) != 0) {
+#pragma unroll
+                            for (int i = 8; i < 16; ++i) and_row(acc, tail.v[i]);
+                        }
+                        tail = ahead;
                     }
                 }
             }
