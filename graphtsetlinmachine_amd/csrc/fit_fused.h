@@ -1,0 +1,300 @@
+// One training step (tm.py:669-747) of a depth-1 model in two kernels.
+//
+//   k_fit_eval      K1 + K6 + K7: each wave takes clauses in turn.  The graph's
+//                   literal-major rows (see score_tiles.h) are staged in LDS;
+//                   the clause's truth over the graph's nodes is the AND of
+//                   the rows of its included literals, read off the include
+//                   plane of the automaton bank.  Writes the clause/node
+//                   bitmap, the include count and the picked node, and adds
+//                   the clause's weights to the class sums.
+//   k_fit_feedback  K8 + K9: a block owns a few clauses; first one thread per
+//                   (clause, class) decides the feedback and moves the weight,
+//                   then one thread per (clause, automaton word) applies Type
+//                   I / II feedback for the classes in order.
+//
+// Nothing but the class sums crosses clause boundaries, which is why the pair
+// needs a single device-wide dependency per graph.
+#pragma once
+
+constexpr int FIT_EVAL_BLOCK = 256;
+
+struct FitGraph {
+    int tile;        // tile holding the graph
+    int word0;       // first word of the graph's slot inside a tile row
+    int words;       // words of the slot that hold nodes of this graph
+    int shift;       // bit offset inside word0 (tiny graphs), else 0
+    uint32_t mask;   // valid bits of the word (tiny graphs), else all ones
+};
+
+__host__ __device__ inline FitGraph fit_graph_slot(const TileGeom &tg, int graph, int n_nodes) {
+    FitGraph f;
+    f.tile = graph / tg.gpt;
+    int j = graph - f.tile * tg.gpt;
+    if (tg.slot_words > 0) {
+        f.word0 = j * tg.slot_words;
+        f.words = n_nodes == 0 ? 1 : (n_nodes - 1) / 32 + 1;
+        f.shift = 0;
+        f.mask = 0xFFFFFFFFu;
+    } else {
+        int bit = j * tg.slot_bits;
+        f.word0 = bit >> 5;
+        f.words = 1;
+        f.shift = bit & 31;
+        f.mask = tg.slot_bits >= 32 ? 0xFFFFFFFFu : ((1u << tg.slot_bits) - 1u);
+    }
+    return f;
+}
+
+// K1 + K6 + K7 for one graph.  A block stages the graph's literal-major rows
+// (plus an all-ones row) in LDS; each wave then takes clauses in turn.  The
+// clause is wave-uniform: its include words come in by scalar loads straight
+// from the top bit plane of the automaton bank, their set bits are walked on
+// the scalar unit, and lane L ANDs word L of every included literal's row, 8
+// LDS reads in flight at a time.  STAGE = false reads the rows from the tile
+// in global memory instead (graphs whose rows do not fit in LDS).
+template <bool STAGE>
+__global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
+    const uint32_t *__restrict__ tiles, TileGeom tg, FitGraph fg, int n_nodes, int literals, int n_types, int C, int LA,
+    int B, int K, int NC, uint32_t filter, const uint32_t *__restrict__ bank, const int32_t *__restrict__ weights,
+    uint32_t k0, uint32_t k1, uint32_t step, uint32_t *__restrict__ bitmap, int32_t *__restrict__ n_incl,
+    int32_t *__restrict__ clause_node, int32_t *class_sum) {
+    extern __shared__ uint32_t rows_lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int WAVES = FIT_EVAL_BLOCK / 64;
+    const uint32_t *tile = tiles + (int64_t)fg.tile * tg.rows * tg.tw + fg.word0;
+    const int stride = STAGE ? fg.words : tg.tw;
+    const int ones_row = literals + n_types;  // in the tile this is the all-ones row as well
+    const uint32_t *rows = tile;
+    if (STAGE) {
+        const int total = (literals + n_types + 1) * fg.words;
+        for (int base = 0; base < total; base += FIT_EVAL_BLOCK * 8) {
+            uint32_t v[8];
+            int at[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                int i = base + u * FIT_EVAL_BLOCK + tid;
+                int r = i / fg.words, w = i - r * fg.words;
+                at[u] = i < total ? i : -1;
+                v[u] = i < total ? tile[(int64_t)r * tg.tw + w] : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (at[u] >= 0) rows_lds[at[u]] = v[u];
+        }
+        __syncthreads();
+        rows = rows_lds;
+    }
+
+    const bool active = lane < fg.words;
+    const uint32_t *col = rows + (active ? lane : 0);
+    int partial = 0;  // lane k < K: this wave's contribution to class k
+    for (int c = blockIdx.x * WAVES + wave; c < C; c += gridDim.x * WAVES) {
+        const uint32_t *inc = bank + (int64_t)c * LA * B + (B - 1);
+        uint32_t acc = active ? col[(int64_t)(literals + c % n_types) * stride] : 0u;
+        int included = 0;
+        for (int w = 0; w < LA; ++w) {
+            uint32_t m = __builtin_amdgcn_readfirstlane(inc[(int64_t)w * B]);
+            if (w == LA - 1) m &= filter;
+            included += __popc(m);
+            while (m) {
+                int row[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    row[u] = m ? (w << 5) + __builtin_ctz(m) : ones_row;
+                    m &= m - 1;
+                }
+                uint32_t r[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) r[u] = col[(int64_t)row[u] * stride];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) acc &= r[u];
+            }
+        }
+        const uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
+        uint32_t *out = bitmap + (int64_t)c * NC;
+        // chunks past the graph are left all ones, as kernels.py:443-466 leaves them
+        for (int i = lane; i < NC; i += 64) out[i] = i < fg.words ? (i == lane ? v : 0u) : 0xFFFFFFFFu;
+        // true nodes before this lane's word, and in total
+        const int pc = __popc(v);
+        int before = pc;
+        for (int off = 1; off < 64; off <<= 1) {
+            int t = __shfl_up(before, off);
+            if (lane >= off) before += t;
+        }
+        const int true_nodes = __shfl(before, 63);
+        before -= pc;
+        bool fired = true_nodes > 0;
+        int node = -1;
+        if (n_nodes == 0) {
+            if (lane == 0) out[0] = 0xFFFFFFFFu;  // the reference's arithmetic for a graph without nodes (kernels.py:289-295)
+            fired = true;
+        } else if (fired) {
+            // K7: the pick-th true node, pick = (r * count) >> 32
+            philox_out r = philox4x32_10((uint32_t)c, 0u, step, GTM_TAG_CLAUSE_NODE, k0, k1);
+            const int pick = (int)(((uint64_t)r.v[0] * (uint64_t)true_nodes) >> 32);
+            const bool mine = pick >= before && pick < before + pc;
+            int candidate = 0;
+            if (mine) {
+                uint32_t t = v;
+                for (int j = before; j < pick; ++j) t &= t - 1;
+                candidate = lane * 32 + __ffs(t) - 1;
+            }
+            const unsigned long long owner = __ballot(mine);
+            node = __shfl(candidate, __ffsll((long long)owner) - 1);
+        }
+        if (lane == 0) {
+            clause_node[c] = node;
+            n_incl[c] = included;
+        }
+        // K6
+        if (fired) {
+            if (K <= 64) {
+                if (lane < K) partial += weights[(int64_t)lane * C + c];
+            } else {
+                for (int k = lane; k < K; k += 64) atomicAdd(&class_sum[k], weights[(int64_t)k * C + c]);
+            }
+        }
+    }
+    if (K <= 64 && lane < K && partial != 0) atomicAdd(&class_sum[lane], partial);
+}
+
+// kernels.py:55-96 on one word of 32 automata whose MAXB >= B bit planes sit in registers.
+template <int MAXB>
+__device__ __forceinline__ void reg_inc(uint32_t (&ta)[MAXB], int B, uint32_t active) {
+    uint32_t carry = active;
+#pragma unroll
+    for (int b = 0; b < MAXB; ++b)
+        if (b < B) {
+            uint32_t v = ta[b];
+            ta[b] = v ^ carry;
+            carry &= v;
+        }
+#pragma unroll
+    for (int b = 0; b < MAXB; ++b)
+        if (b < B) ta[b] |= carry;  // residual carry: saturate
+}
+
+template <int MAXB>
+__device__ __forceinline__ void reg_dec(uint32_t (&ta)[MAXB], int B, uint32_t active) {
+    uint32_t carry = active;
+#pragma unroll
+    for (int b = 0; b < MAXB; ++b)
+        if (b < B) {
+            uint32_t v = ta[b];
+            ta[b] = v ^ carry;
+            carry &= ~v;
+        }
+#pragma unroll
+    for (int b = 0; b < MAXB; ++b)
+        if (b < B) ta[b] &= ~carry;
+}
+
+// Type I / II feedback of kernels.py:141-183 (and :98-139 for message banks)
+// for all classes in order on one automaton word; returns the include plane.
+template <int MAXB>
+__device__ __forceinline__ uint32_t feedback_word(uint32_t *ta_global, int B, int K, const int32_t *u_of, int u_stride,
+                                                  bool fired, bool within, int boost, uint32_t x, uint32_t k0,
+                                                  uint32_t k1, uint32_t c, uint32_t w, uint32_t step, uint32_t bank_id,
+                                                  uint32_t thr16) {
+    uint32_t ta[MAXB];
+#pragma unroll
+    for (int b = 0; b < MAXB; ++b) ta[b] = b < B ? ta_global[b] : 0u;
+    for (int k = 0; k < K; ++k) {
+        const int u = u_of[(int64_t)k * u_stride];
+        if (u > 0) {
+            uint32_t fb = gtm_feedback_bits(k0, k1, c, w, step, bank_id, (uint32_t)k, thr16);
+            if (fired && within) {
+                reg_inc<MAXB>(ta, B, boost == 1 ? x : (x & ~fb));
+                reg_dec<MAXB>(ta, B, ~x & fb);
+            } else {
+                reg_dec<MAXB>(ta, B, fb);
+            }
+        } else if (u < 0 && fired) {
+            uint32_t top = 0;
+#pragma unroll
+            for (int b = 0; b < MAXB; ++b)
+                if (b == B - 1) top = ta[b];
+            reg_inc<MAXB>(ta, B, ~x & ~top);
+        }
+    }
+    uint32_t top = 0;
+#pragma unroll
+    for (int b = 0; b < MAXB; ++b)
+        if (b < B) {
+            ta_global[b] = ta[b];
+            if (b == B - 1) top = ta[b];
+        }
+    return top;
+}
+
+__device__ __forceinline__ uint32_t feedback_word_any(uint32_t *ta_global, int B, int K, const int32_t *u_of,
+                                                      int u_stride, bool fired, bool within, int boost, uint32_t x,
+                                                      uint32_t k0, uint32_t k1, uint32_t c, uint32_t w, uint32_t step,
+                                                      uint32_t bank_id, uint32_t thr16) {
+    if (B <= 8)
+        return feedback_word<8>(ta_global, B, K, u_of, u_stride, fired, within, boost, x, k0, k1, c, w, step, bank_id, thr16);
+    if (B <= 16)
+        return feedback_word<16>(ta_global, B, K, u_of, u_stride, fired, within, boost, x, k0, k1, c, w, step, bank_id, thr16);
+    return feedback_word<32>(ta_global, B, K, u_of, u_stride, fired, within, boost, x, k0, k1, c, w, step, bank_id, thr16);
+}
+
+// K8 + K9 for `cpb` clauses per block; see the header comment.
+__global__ void k_fit_feedback(uint32_t *bank, int32_t *weights, const int32_t *class_sum,
+                               int32_t *class_sum_next, const int32_t *__restrict__ y, int C, int LA, int B, int K,
+                               int T, int negative, int boost, int max_included, uint64_t q_thr,
+                               uint32_t thr16, uint32_t k0, uint32_t k1, uint32_t step,
+                               const int32_t *__restrict__ clause_node, const int32_t *__restrict__ n_incl,
+                               const uint32_t *__restrict__ X_rows, int cpb) {
+    extern __shared__ int32_t upd[];  // [cpb][K]
+    const int tid = threadIdx.x;
+    const int c_base = blockIdx.x * cpb;
+    if (blockIdx.x == 0)  // the next step accumulates into the other buffer
+        for (int k = tid; k < K; k += blockDim.x) class_sum_next[k] = 0;
+
+    for (int i = tid; i < cpb * K; i += blockDim.x) {
+        const int c = c_base + i / K, k = i % K;
+        int u = 0;
+        if (c < C) {
+            int cs = class_sum[k];
+            cs = cs > T ? T : (cs < -T ? -T : cs);
+            const int yk = y[k];
+            const int target = 1 - 2 * (cs > yk);
+            int w = weights[(int64_t)k * C + c];
+            const int sign = (w >= 0) - (w < 0);
+            int err = yk - cs;
+            err = err < 0 ? -err : err;
+            philox_out r = philox4x32_10((uint32_t)c, (uint32_t)k, step, GTM_TAG_CLAUSE_UPDATES, k0, k1);
+            const bool skip = (target == -1 && (uint64_t)r.v[0] >= q_thr) ||
+                              ((uint64_t)r.v[1] * (uint64_t)(2 * (int64_t)T) >= ((uint64_t)err << 32));
+            u = skip ? 0 : target * sign;
+            const bool fired = clause_node[c] != -1;
+            if (u > 0 && fired && (w < 0 ? -(int64_t)w : (int64_t)w) < 2147483647) {
+                weights[(int64_t)k * C + c] = w + sign;
+            } else if (u < 0 && fired) {
+                w -= sign;
+                if (negative == 0 && w < 1) w = 1;
+                weights[(int64_t)k * C + c] = w;
+            }
+        }
+        upd[i] = u;
+    }
+    __syncthreads();
+
+    for (int i = tid; i < cpb * LA; i += blockDim.x) {
+        const int local = i / LA, w = i - local * LA;
+        const int c = c_base + local;
+        if (c >= C) continue;
+        const int32_t *u_of = upd + local * K;
+        bool any = false;
+        for (int k = 0; k < K; ++k) any |= u_of[k] != 0;
+        if (!any) continue;
+        const int node = clause_node[c];
+        const bool fired = node != -1;
+        const bool within = n_incl[c] <= max_included;
+        const uint32_t x = fired ? X_rows[(int64_t)node * LA + w] : 0u;
+        uint32_t *ta = bank + ((int64_t)c * LA + w) * B;
+        feedback_word_any(ta, B, K, u_of, 1, fired, within, boost, x, k0, k1, (uint32_t)c, (uint32_t)w, step, 0u, thr16);
+    }
+}

@@ -400,6 +400,8 @@ __device__ __forceinline__ void ta_dec(uint32_t *ta, int B, uint32_t active) {
         for (int b = 0; b < B; ++b) ta[b] &= ~carry;
 }
 
+#include "fit_fused.h"
+
 // K9 / K10: one thread per (clause, automaton word); the classes are applied
 // in ascending order to that word, as kernels.py:205-207,236-238 do per clause
 // (words of a clause do not interact, so splitting by word keeps the result).
@@ -415,20 +417,8 @@ __global__ void k_update(uint32_t *bank, int C, int chunks, int B, int K, int bo
     bool within = n_incl[c] <= max_included;
     uint32_t x = fired ? rows[(int64_t)node * chunks + w] : 0u;
     uint32_t *ta = bank + i * B;
-    for (int k = 0; k < K; ++k) {
-        int u = update[(int64_t)k * C + c];
-        if (u > 0) {
-            uint32_t fb = gtm_feedback_bits(k0, k1, (uint32_t)c, (uint32_t)w, step, bank_id, (uint32_t)k, thr16);
-            if (fired && within) {
-                ta_inc(ta, B, boost == 1 ? x : (x & ~fb));
-                ta_dec(ta, B, ~x & fb);
-            } else {
-                ta_dec(ta, B, fb);
-            }
-        } else if (u < 0 && fired) {
-            ta_inc(ta, B, ~x & ~ta[B - 1]);
-        }
-    }
+    feedback_word_any(ta, B, K, update + c, C, fired, within, boost, x, k0, k1, (uint32_t)c, (uint32_t)w, step, bank_id,
+                      thr16);
 }
 
 // ------------------------------------------------------------ launch helpers
@@ -524,7 +514,7 @@ FitWs carve_fit(const Dims &d, const gtm_config *cfg, char *base) {
     w.bitmap_b = (uint32_t *)take((size_t)d.C * d.NC * 4);
     for (int l = 0; l < GTM_MAX_DEPTH - 1; ++l)
         w.clause_X[l] = l < cfg->depth - 1 ? (uint32_t *)take((size_t)cfg->max_nodes * d.MC * 4) : nullptr;
-    w.class_sum = (int32_t *)take((size_t)d.K * 4);
+    w.class_sum = (int32_t *)take((size_t)d.K * 4 * 2);  // two buffers, used alternately by the fused path
     w.clause_node = (int32_t *)take((size_t)d.C * 4);
     w.n_incl = (int32_t *)take((size_t)d.C * 4);
     w.update = (int32_t *)take((size_t)d.K * d.C * 4);
@@ -926,6 +916,65 @@ int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *
     return GTM_OK;
 }
 
+}  // extern "C"
+
+namespace {
+
+// `_fit`'s inner loop for a depth-1 model on a data set that has tiles: two
+// launches per example (fit_fused.h).
+int fit_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
+                 const FitWs &w, const int32_t *encoded_Y, int first_example, int n_examples, uint64_t first_step,
+                 const uint32_t *h_n, const uint32_t *h_base, hipStream_t st) {
+    hipLaunchKernelGGL(k_fill_i32, dim3(1), dim3(TPB), 0, st, w.class_sum, (int64_t)d.K * 2, 0);
+    if (int rc = check_launch("fill")) return rc;
+    Key key = key_of(cfg);
+    const int n_types = g->number_of_node_types;
+    const int cpb = d.LA >= TPB ? 1 : TPB / d.LA;
+    const uint64_t q_thr = q_threshold(cfg->q, cfg->classes);
+    const uint32_t thr16 = feedback_threshold(cfg->s[0]);
+    // enough waves to spread the clauses over the chip, at least ~2 clauses per wave
+    const int waves_per_block = FIT_EVAL_BLOCK / 64;
+    int eval_blocks = (d.C + 2 * waves_per_block - 1) / (2 * waves_per_block);
+    if (eval_blocks > 512) eval_blocks = 512;
+    static thread_local size_t lds_set = 0;
+    for (int i = 0; i < n_examples; ++i) {
+        const int ex = first_example + i;
+        const uint32_t step = (uint32_t)(first_step + (uint64_t)i);
+        FitGraph fg = fit_graph_slot(tg, ex, (int)h_n[i]);
+        int32_t *sum_now = w.class_sum + (size_t)(i & 1) * d.K, *sum_next = w.class_sum + (size_t)((i + 1) & 1) * d.K;
+        size_t lds = (size_t)(cfg->literals + n_types + 1) * fg.words * 4;
+        const bool stage = lds <= 96 * 1024;
+        if (stage && lds > lds_set) {
+            hipError_t e = hipFuncSetAttribute((const void *)k_fit_eval<true>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
+            lds_set = lds;
+        }
+        if (i < Profile::MAX) profile_start(stage ? "k_fit_eval<true>" : "k_fit_eval<false>", st);
+        if (stage)
+            hipLaunchKernelGGL(k_fit_eval<true>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), lds, st, g->tiles, tg, fg,
+                               (int)h_n[i], cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
+                               s->clause_weights, key.k0, key.k1, step, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
+        else
+            hipLaunchKernelGGL(k_fit_eval<false>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), 0, st, g->tiles, tg, fg,
+                               (int)h_n[i], cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
+                               s->clause_weights, key.k0, key.k1, step, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
+        if (int rc = check_launch("fit_eval")) return rc;
+        if (i < Profile::MAX) profile_stop(st);
+        hipLaunchKernelGGL(k_fit_feedback, dim3(blocks_for(d.C, cpb)), dim3(TPB), (size_t)cpb * d.K * 4, st,
+                           s->ta_state, s->clause_weights, sum_now, sum_next, encoded_Y + (int64_t)ex * d.K, d.C, d.LA,
+                           d.B, d.K, cfg->threshold, cfg->negative_clauses, cfg->boost_true_positive_feedback,
+                           cfg->max_included_literals, q_thr, thr16, key.k0, key.k1, step, w.clause_node, w.n_incl,
+                           g->X + (int64_t)h_base[i] * d.LA, cpb);
+        if (int rc = check_launch("fit_feedback")) return rc;
+    }
+    return GTM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
 size_t gtm_fit_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs) {
     Dims d;
     if (validate(cfg, &d)) return 0;
@@ -957,6 +1006,12 @@ int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *st
     if (e == hipSuccess) e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(GTM_ERR_HIP, "reading graph sizes: %s", hipGetErrorString(e));
 
+    if (cfg->depth == 1 && graphs->tiles) {
+        TileGeom tg = geometry_for(cfg, graphs, d.K);
+        if (tg.ok && tg.slot_words <= 64)  // one lane per word of the graph's slot
+            return fit_on_tiles(d, cfg, graphs, state, tg, w, encoded_Y, first_example, n_examples, first_step, h_n,
+                                h_base, st);
+    }
     for (int i = 0; i < n_examples; ++i) {
         int ex = first_example + i;
         uint64_t step = first_step + (uint64_t)i;

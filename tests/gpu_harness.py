@@ -128,7 +128,9 @@ class Device:
                   _ptr(ws), ws.numel(), _ptr(out), _stream())
         return host(out, np.int32, (n, self.cfg.classes))
 
-    def fit(self, encoded_Y, first, n, first_step):
+    def fit(self, encoded_Y, first, n, first_step, tiles=False):
+        if tiles:
+            assert self.build_tiles()
         need = _abi.lib.gtm_fit_workspace_bytes(ctypes.byref(self.acfg), ctypes.byref(self.dg.desc))
         ws = torch.empty(need, dtype=torch.uint8, device="cuda")
         y = _to_device(np.ascontiguousarray(encoded_Y, dtype=np.int32))

@@ -156,12 +156,16 @@ def test_training_operators(shape, boost, max_included):
 
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "shape%d" % s["seed"])
-def test_fit_trajectory_bit_exact(shape):
-    """gtm_fit over a few epochs leaves exactly the oracle's automata and weights."""
+@pytest.mark.parametrize("tiles", [False, True], ids=["plain", "tiles"])
+def test_fit_trajectory_bit_exact(shape, tiles):
+    """gtm_fit over a few epochs leaves exactly the oracle's automata and weights
+    (with tiles, depth-1 models take the two-kernel fused step)."""
     from tests.gpu_harness import Device
 
     graphs, cfg, model = build(shape, 0.02)
     dev = Device(model, graphs)
+    if tiles and model.depth == 1:
+        assert dev.build_tiles()
     rng = np.random.default_rng(shape["seed"] + 100)
     Y = o.encode_labels(rng.integers(0, cfg.classes, size=graphs.number_of_graphs), cfg.classes, cfg.threshold)
     G = graphs.number_of_graphs
@@ -245,6 +249,48 @@ def test_tile_scoring_equals_oracle(shape, density):
     # a range that starts and ends inside tiles
     if G > 7:
         assert np.array_equal(dev.score(3, G - 5, G), plain[3:G - 2])
+
+
+@pytest.mark.parametrize("shape", TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
+@pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 6, 5)])
+def test_fused_fit_on_every_tile_geometry(shape, boost, max_included, state_bits):
+    """The fused depth-1 training step == the oracle == the per-operator path."""
+    from tests.gpu_harness import Device
+
+    g = dict(shape["g"])
+    g["n_graphs"] = min(g["n_graphs"], 24)
+    graphs = helpers.random_graphs(shape["seed"], **g)
+    cfg = helpers.oracle_config(graphs, classes=shape["classes"], clauses=shape["clauses"], T=30, boost=boost,
+                                max_included=max_included, state_bits=state_bits)
+    model = helpers.random_model(shape["seed"], cfg, 1, s=3.0, include_density=0.02)
+    dev = Device(model, graphs)
+    assert dev.build_tiles()
+    rng = np.random.default_rng(shape["seed"])
+    G = graphs.number_of_graphs
+    Y = o.encode_labels(rng.integers(0, cfg.classes, size=G), cfg.classes, cfg.threshold)
+    for epoch in range(2):
+        o.fit(model, graphs, Y)
+        dev.fit(Y, 0, G, epoch * G)
+        ta, _, w = dev.download()
+        assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
+        assert np.array_equal(ta, model.ta_state), "automata after epoch %d" % epoch
+    assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
+
+
+def test_fused_fit_with_an_empty_graph():
+    from tests.gpu_harness import Device
+
+    g = helpers.random_graphs(19, n_graphs=6, hv_size=16, sizes=[5, 0, 33, 1, 0, 40])
+    cfg = helpers.oracle_config(g, classes=3, clauses=20, T=20)
+    model = helpers.random_model(5, cfg, 1, s=2.0, include_density=0.05)
+    dev = Device(model, g)
+    assert dev.build_tiles()
+    Y = o.encode_labels(np.array([0, 1, 2, 0, 1, 2]), 3, cfg.threshold)
+    o.fit(model, g, Y, epochs=2)
+    dev.fit(Y, 0, 6, 0)
+    dev.fit(Y, 0, 6, 6)
+    ta, _, w = dev.download()
+    assert np.array_equal(w, model.clause_weights) and np.array_equal(ta, model.ta_state)
 
 
 def test_empty_graphs_score_like_the_reference_arithmetic():
