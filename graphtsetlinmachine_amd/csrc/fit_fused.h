@@ -94,24 +94,33 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
         const uint32_t *inc = bank + (int64_t)c * LA * B + (B - 1);
         uint32_t acc = active ? col[(int64_t)(literals + c % n_types) * stride] : 0u;
         int included = 0;
-        for (int w = 0; w < LA; ++w) {
-            uint32_t m = __builtin_amdgcn_readfirstlane(inc[(int64_t)w * B]);
-            if (w == LA - 1) m &= filter;
-            included += __popc(m);
-            while (m) {
-                int row[8];
+        for (int w0 = 0; w0 < LA; w0 += 64) {
+            // lane w fetches include word w0 + w: one memory latency for up to 64 words
+            uint32_t mine = w0 + lane < LA ? inc[(int64_t)(w0 + lane) * B] : 0u;
+            if (w0 + lane == LA - 1) mine &= filter;
+            unsigned long long nonzero = __ballot(mine != 0);
+            included += __popc(mine);  // summed over the lanes below
+            while (nonzero) {
+                const int wl = __ffsll((long long)nonzero) - 1;
+                nonzero &= nonzero - 1;
+                uint32_t m = __builtin_amdgcn_readlane(mine, wl);
+                const int base = (w0 + wl) << 5;
+                while (m) {
+                    int row[8];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    row[u] = m ? (w << 5) + __builtin_ctz(m) : ones_row;
-                    m &= m - 1;
+                    for (int u = 0; u < 8; ++u) {
+                        row[u] = m ? base + __builtin_ctz(m) : ones_row;
+                        m &= m - 1;
+                    }
+                    uint32_t r[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) r[u] = col[(int64_t)row[u] * stride];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc &= r[u];
                 }
-                uint32_t r[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) r[u] = col[(int64_t)row[u] * stride];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) acc &= r[u];
             }
         }
+        for (int off = 32; off > 0; off >>= 1) included += __shfl_xor(included, off);
         const uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
         uint32_t *out = bitmap + (int64_t)c * NC;
         // chunks past the graph are left all ones, as kernels.py:443-466 leaves them

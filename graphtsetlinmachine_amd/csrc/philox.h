@@ -63,6 +63,7 @@ GTM_HD philox_out philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t 
 // Stands for the 32 `curand_uniform <= 1/s` draws of kernels.py:113-118,157-162.
 GTM_HD uint32_t gtm_feedback_bits(uint32_t k0, uint32_t k1, uint32_t clause, uint32_t word, uint32_t step,
                                   uint32_t bank, uint32_t class_id, uint32_t threshold16) {
+    if (threshold16 >= 65536u) return 0xFFFFFFFFu;  // s <= 1: every 16-bit value is below the threshold
     const uint32_t c3 = GTM_TAG_FEEDBACK | (bank << 8) | (class_id << 16);
     uint32_t bits = 0;
 #pragma unroll
