@@ -202,18 +202,20 @@ __device__ __forceinline__ void reg_dec(uint32_t (&ta)[MAXB], int B, uint32_t ac
 
 // Type I / II feedback of kernels.py:141-183 (and :98-139 for message banks)
 // for all classes in order on one automaton word; returns the include plane.
+// `fb_of`, when not NULL, holds the feedback bits of class k at fb_of[k] (computed elsewhere by the
+// same gtm_feedback_bits call).
 template <int MAXB>
 __device__ __forceinline__ uint32_t feedback_word(uint32_t *ta_global, int B, int K, const int32_t *u_of, int u_stride,
                                                   bool fired, bool within, int boost, uint32_t x, uint32_t k0,
                                                   uint32_t k1, uint32_t c, uint32_t w, uint32_t step, uint32_t bank_id,
-                                                  uint32_t thr16) {
+                                                  uint32_t thr16, const uint32_t *fb_of = nullptr) {
     uint32_t ta[MAXB];
 #pragma unroll
     for (int b = 0; b < MAXB; ++b) ta[b] = b < B ? ta_global[b] : 0u;
     for (int k = 0; k < K; ++k) {
         const int u = u_of[(int64_t)k * u_stride];
         if (u > 0) {
-            uint32_t fb = gtm_feedback_bits(k0, k1, c, w, step, bank_id, (uint32_t)k, thr16);
+            uint32_t fb = fb_of ? fb_of[k] : gtm_feedback_bits(k0, k1, c, w, step, bank_id, (uint32_t)k, thr16);
             if (fired && within) {
                 reg_inc<MAXB>(ta, B, boost == 1 ? x : (x & ~fb));
                 reg_dec<MAXB>(ta, B, ~x & fb);
@@ -241,12 +243,27 @@ __device__ __forceinline__ uint32_t feedback_word(uint32_t *ta_global, int B, in
 __device__ __forceinline__ uint32_t feedback_word_any(uint32_t *ta_global, int B, int K, const int32_t *u_of,
                                                       int u_stride, bool fired, bool within, int boost, uint32_t x,
                                                       uint32_t k0, uint32_t k1, uint32_t c, uint32_t w, uint32_t step,
-                                                      uint32_t bank_id, uint32_t thr16) {
+                                                      uint32_t bank_id, uint32_t thr16, const uint32_t *fb_of = nullptr) {
     if (B <= 8)
-        return feedback_word<8>(ta_global, B, K, u_of, u_stride, fired, within, boost, x, k0, k1, c, w, step, bank_id, thr16);
+        return feedback_word<8>(ta_global, B, K, u_of, u_stride, fired, within, boost, x, k0, k1, c, w, step, bank_id, thr16, fb_of);
     if (B <= 16)
-        return feedback_word<16>(ta_global, B, K, u_of, u_stride, fired, within, boost, x, k0, k1, c, w, step, bank_id, thr16);
-    return feedback_word<32>(ta_global, B, K, u_of, u_stride, fired, within, boost, x, k0, k1, c, w, step, bank_id, thr16);
+        return feedback_word<16>(ta_global, B, K, u_of, u_stride, fired, within, boost, x, k0, k1, c, w, step, bank_id, thr16, fb_of);
+    return feedback_word<32>(ta_global, B, K, u_of, u_stride, fired, within, boost, x, k0, k1, c, w, step, bank_id, thr16, fb_of);
+}
+
+// Sum over the wave of a small per-lane count (< 64), and the sum over the lanes below this one,
+// from ballots of the count's bits: no cross-lane data movement.
+__device__ __forceinline__ void wave_count_scan(int count, int lane, int *total, int *before) {
+    const unsigned long long below = (1ull << lane) - 1ull;
+    int t = 0, b = 0;
+#pragma unroll
+    for (int bit = 0; bit < 6; ++bit) {
+        const unsigned long long has = __ballot((count >> bit) & 1);
+        t += __popcll(has) << bit;
+        b += __popcll(has & below) << bit;
+    }
+    *total = t;
+    *before = b;
 }
 
 // K8 + K9 for `cpb` clauses per block; see the header comment.

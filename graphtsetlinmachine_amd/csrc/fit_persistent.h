@@ -1,0 +1,351 @@
+// A whole run of training examples (the loop at tm.py:669-747) of a depth-1
+// model in ONE cooperative launch.
+//
+// Each workgroup owns a contiguous range of clauses for the whole run and keeps
+// their automata (all bit planes) and weights in LDS; they go back to global
+// memory once, at the end.  Per example a workgroup
+//   1. evaluates its clauses on the graph's literal-major rows (staged in LDS,
+//      the next graph's rows are fetched while waiting at the barrier),
+//      picks the nodes, and adds its clauses' votes to the class sums in
+//      global memory;
+//   2. meets the other workgroups at a device-wide barrier (the class sums are
+//      the only thing that crosses clause boundaries, kernels.py:310-315);
+//   3. decides the feedback and updates its automata and weights in LDS.
+// Class sums and barrier are one thing: the sum of class k is a 64-bit word whose
+// low 48 bits hold the (biased) sum and whose high 16 bits count the workgroups
+// that have added their share.  A workgroup adds (1 << 48) + share with one
+// device-scope atomic per class and then polls the words until the count equals
+// the number of workgroups: when it does, the low bits are the final sum.  One
+// atomic per class carries both, so nothing has to be ordered against a separate
+// barrier word and no cache is flushed or invalidated.  The words live in a ring
+// of three slots so that no slot is reset while someone may still read it.
+//
+// The wait is bounded: after `spin_limit` polls a workgroup raises the abort
+// flag and every workgroup leaves the loop at its next check, so the grid always
+// drains.  The host reports the flag as an error.
+#pragma once
+
+constexpr int FITP_BLOCK = 1024;  // 16 waves: one clause per wave in flight, four waves per SIMD hide each other's latencies
+
+struct FitPersistParams {
+    // data set
+    const uint32_t *tiles;
+    const uint32_t *X;
+    const uint32_t *node_index;
+    const uint32_t *n_nodes;
+    const int32_t *encoded_Y;
+    TileGeom tg;
+    int first_example, n_examples;
+    uint32_t first_step;
+    // model
+    uint32_t *bank;
+    int32_t *weights;
+    int literals, n_types, C, LA, B, K, T, negative, boost, max_included;
+    uint32_t filter, thr16, k0, k1;
+    uint64_t q_thr;
+    // coordination
+    unsigned long long *class_sum;  // [3][K], every word FITP_BIAS on entry
+    uint32_t *abort_flag;           // [1], zero on entry
+    uint32_t spin_limit;
+    int clauses_per_group;
+    int rows_words;       // LDS words of one staged graph: (literals + n_types + 1) * max slot words
+    int max_words;        // words per graph slot that can hold nodes
+};
+
+__device__ __forceinline__ void fitp_stage_rows(const FitPersistParams &p, const FitGraph &fg, uint32_t *dst, int tid) {
+    const uint32_t *tile = p.tiles + (int64_t)fg.tile * p.tg.rows * p.tg.tw + fg.word0;
+    const int words = fg.words;
+    const int total = (p.literals + p.n_types + 1) * words;
+    // element i = r * words + w; a thread visits i = tid, tid + 256, ...: (r, w) advance without dividing
+    const int dr = FITP_BLOCK / words, dw = FITP_BLOCK - dr * words;
+    int r = tid / words, w = tid - r * words;
+    for (int base = tid; base < total; base += FITP_BLOCK * 8) {
+        uint32_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            v[u] = base + u * FITP_BLOCK < total ? tile[(int64_t)r * p.tg.tw + w] : 0u;
+            r += dr;
+            w += dw;
+            if (w >= words) {
+                w -= words;
+                ++r;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (base + u * FITP_BLOCK < total) dst[base + u * FITP_BLOCK] = v[u];
+    }
+}
+
+constexpr unsigned long long FITP_BIAS = 1ull << 47;      // a class sum s is stored as s + FITP_BIAS in bits 0..47
+constexpr unsigned long long FITP_ARRIVED = 1ull << 48;   // one arrival in bits 48..63
+constexpr int FITP_PREFETCH = 8;  // words of the next graph's rows a thread holds in registers while evaluating
+
+// Address of element `i` of the staged rows (i = row * words + w) inside the graph's tile.
+__device__ __forceinline__ const uint32_t *fitp_row_word(const FitPersistParams &p, const FitGraph &fg, int i) {
+    const int r = i / fg.words, w = i - r * fg.words;
+    return p.tiles + ((int64_t)fg.tile * p.tg.rows + r) * p.tg.tw + fg.word0 + w;
+}
+
+__global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams p) {
+    extern __shared__ uint32_t lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int WAVES = FITP_BLOCK / 64;
+    const int c0 = blockIdx.x * p.clauses_per_group;
+    const int n_own = min(p.clauses_per_group, p.C - c0);
+    const int LA = p.LA, B = p.B, K = p.K;
+    const int own_max = p.clauses_per_group;
+
+    // LDS carve-up
+    uint32_t *rows_buf[2] = {lds, lds + p.rows_words};
+    uint32_t *ta = lds + 2 * p.rows_words;                     // [own][LA][B]
+    int32_t *wts = (int32_t *)(ta + (size_t)own_max * LA * B);  // [own][K]
+    int32_t *upd = wts + (size_t)own_max * K;                  // [own][K]
+    int32_t *node_of = upd + (size_t)own_max * K;              // [own]
+    int32_t *incl_of = node_of + own_max;                      // [own]
+    int32_t *sums = incl_of + own_max;                         // [K] class sums of the example
+    int32_t *votes = sums + K;                                 // [K] this group's share of the class sums
+    uint32_t *gate = (uint32_t *)(votes + K);                  // [own][K][2] random words of the feedback gates
+    uint32_t *fbits = gate + 2 * (size_t)own_max * K;          // [own][LA][K] Type I feedback bits
+    __shared__ int go_on;
+
+    // own state -> LDS
+    for (int k = tid; k < K; k += FITP_BLOCK) votes[k] = 0;
+    for (int i = tid; i < n_own * LA * B; i += FITP_BLOCK) ta[i] = p.bank[(int64_t)c0 * LA * B + i];
+    for (int i = tid; i < n_own * K; i += FITP_BLOCK) {
+        int cl = i / K, k = i - cl * K;
+        wts[i] = p.weights[(int64_t)k * p.C + c0 + cl];
+    }
+    const int last = p.first_example + p.n_examples - 1;
+    int n_now = 0, n_next = 0;          // node counts of example i and i + 1
+    uint32_t base_now = 0, base_next = 0;  // node_index of example i and i + 1
+    if (p.n_examples > 0) {
+        n_now = (int)p.n_nodes[p.first_example];
+        base_now = p.node_index[p.first_example];
+        const int e1 = min(p.first_example + 1, last);
+        n_next = (int)p.n_nodes[e1];
+        base_next = p.node_index[e1];
+        FitGraph fg0 = fit_graph_slot(p.tg, p.first_example, n_now);
+        fitp_stage_rows(p, fg0, rows_buf[0], tid);
+    }
+    __syncthreads();
+
+    const int ones_row = p.literals + p.n_types;
+    for (int i = 0; i < p.n_examples; ++i) {
+        const int ex = p.first_example + i;
+        const uint32_t step = p.first_step + (uint32_t)i;
+        const FitGraph fg = fit_graph_slot(p.tg, ex, n_now);
+        const uint32_t *rows = rows_buf[i & 1];
+        unsigned long long *slot_now = p.class_sum + (size_t)(i % 3) * K;
+
+        // ---- 0. requests that can be in flight while this example is evaluated: the next graph's
+        // rows (into registers) and the sizes of the graph after it
+        const bool has_next = i + 1 < p.n_examples;
+        const FitGraph fn = fit_graph_slot(p.tg, has_next ? ex + 1 : ex, has_next ? n_next : n_now);
+        const int next_total = has_next ? (p.literals + p.n_types + 1) * fn.words : 0;
+        uint32_t pre[FITP_PREFETCH];
+        {
+            // element at = row * words + w; a thread's elements are FITP_BLOCK apart: step (row, w) without dividing
+            const uint32_t *tile = p.tiles + (int64_t)fn.tile * p.tg.rows * p.tg.tw + fn.word0;
+            const int dr = FITP_BLOCK / fn.words, dw = FITP_BLOCK - dr * fn.words;
+            int r = tid / fn.words, w = tid - r * fn.words;
+#pragma unroll
+            for (int u = 0; u < FITP_PREFETCH; ++u) {
+                pre[u] = tid + u * FITP_BLOCK < next_total ? tile[(int64_t)r * p.tg.tw + w] : 0u;
+                r += dr;
+                w += dw;
+                if (w >= fn.words) {
+                    w -= fn.words;
+                    ++r;
+                }
+            }
+        }
+        const int e2 = min(ex + 2, last);
+        const int n_after = (int)p.n_nodes[e2];
+        const uint32_t base_after = p.node_index[e2];
+
+        // ---- 1. evaluate own clauses (K1 + K7), votes (K6)
+        const bool active = lane < fg.words;
+        const uint32_t *col = rows + (active ? lane : 0);
+        const int stride = fg.words;
+        for (int cl = wave; cl < n_own; cl += WAVES) {
+            const int c = c0 + cl;
+            const uint32_t *inc = ta + (size_t)cl * LA * B + (B - 1);
+            uint32_t acc = active ? col[(p.literals + c % p.n_types) * stride] : 0u;
+            int included = 0;
+            for (int w0 = 0; w0 < LA; w0 += 64) {
+                uint32_t mine = w0 + lane < LA ? inc[(w0 + lane) * B] : 0u;
+                if (w0 + lane == LA - 1) mine &= p.filter;
+                unsigned long long nonzero = __ballot(mine != 0);
+                while (nonzero) {
+                    const int wl = __ffsll((long long)nonzero) - 1;
+                    nonzero &= nonzero - 1;
+                    uint32_t m = __builtin_amdgcn_readlane(mine, wl);
+                    included += __popc(m);
+                    const int base = (w0 + wl) << 5;
+                    while (m) {
+                        int row[8];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) {
+                            row[u] = m ? base + __builtin_ctz(m) : ones_row;
+                            m &= m - 1;
+                        }
+                        uint32_t r[8];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) r[u] = col[row[u] * stride];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) acc &= r[u];
+                    }
+                }
+            }
+            const uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
+            const int pc = __popc(v);
+            int true_nodes, before;
+            wave_count_scan(pc, lane, &true_nodes, &before);
+            bool fired = true_nodes > 0;
+            int node = -1;
+            if (n_now == 0) {
+                fired = true;  // the reference's arithmetic for a graph without nodes (kernels.py:289-295)
+            } else if (fired) {
+                philox_out r = philox4x32_10((uint32_t)c, 0u, step, GTM_TAG_CLAUSE_NODE, p.k0, p.k1);
+                const int pick = (int)(((uint64_t)r.v[0] * (uint64_t)true_nodes) >> 32);
+                const bool mine_is = pick >= before && pick < before + pc;
+                int candidate = 0;
+                if (mine_is) {
+                    uint32_t t = v;
+                    for (int j = before; j < pick; ++j) t &= t - 1;
+                    candidate = lane * 32 + __ffs(t) - 1;
+                }
+                const unsigned long long owner = __ballot(mine_is);
+                node = __builtin_amdgcn_readlane(candidate, __ffsll((long long)owner) - 1);
+            }
+            if (lane == 0) {
+                node_of[cl] = node;
+                incl_of[cl] = included;
+            }
+            if (fired)
+                for (int k = lane; k < K; k += 64) atomicAdd(&votes[k], wts[cl * K + k]);  // LDS
+        }
+
+        // ---- 2. class sums across the device (see the header comment)
+        __syncthreads();  // the group's votes are complete
+        for (int k = tid; k < K; k += FITP_BLOCK) {
+            __hip_atomic_fetch_add(&slot_now[k], FITP_ARRIVED + (unsigned long long)(long long)votes[k], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            votes[k] = 0;
+        }
+        // Work that does not need the class sums is done while the other groups arrive: the next
+        // graph's rows go to LDS, the random numbers of the feedback gates, the literals of the
+        // picked nodes.
+        {
+            uint32_t *dst = rows_buf[(i + 1) & 1];
+#pragma unroll
+            for (int u = 0; u < FITP_PREFETCH; ++u) {
+                const int at = tid + u * FITP_BLOCK;
+                if (at < next_total) dst[at] = pre[u];
+            }
+            for (int at = tid + FITP_PREFETCH * FITP_BLOCK; at < next_total; at += FITP_BLOCK)
+                dst[at] = *fitp_row_word(p, fn, at);
+        }
+        for (int j = tid; j < n_own * K; j += FITP_BLOCK) {
+            const int cl = j / K, k = j - cl * K;
+            philox_out r = philox4x32_10((uint32_t)(c0 + cl), (uint32_t)k, step, GTM_TAG_CLAUSE_UPDATES, p.k0, p.k1);
+            gate[2 * j] = r.v[0];
+            gate[2 * j + 1] = r.v[1];
+        }
+        uint32_t x_mine = 0;  // literals word of this thread's (clause, word) item, first pass of the update loop
+        if (tid < n_own * LA) {
+            const int cl = tid / LA, w = tid - cl * LA;
+            const int node = node_of[cl];
+            if (node != -1) x_mine = p.X[((int64_t)base_now + node) * LA + w];
+        }
+        if (tid == 0) go_on = 1;
+        __syncthreads();
+        for (int k = tid; k < K; k += FITP_BLOCK) {
+            uint32_t polls = 0;
+            unsigned long long word;
+            bool ok = true;
+            while (((word = __hip_atomic_load(&slot_now[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 48) <
+                   (unsigned long long)gridDim.x) {
+                if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
+                    ++polls > p.spin_limit) {
+                    __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ok = false;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            if (!ok) go_on = 0;
+            sums[k] = (int32_t)(long long)((word & (FITP_ARRIVED - 1)) - FITP_BIAS);
+        }
+        __syncthreads();
+        if (!go_on) break;  // uniform over the group; every group leaves at its next check
+        // slot (i+2)%3 was last read for example i-1; everybody is past that: reset it for example i+2
+        if (blockIdx.x == 0)
+            for (int k = tid; k < K; k += FITP_BLOCK)
+                __hip_atomic_store(&p.class_sum[(size_t)((i + 2) % 3) * K + k], FITP_BIAS, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+
+        // ---- 3. feedback (K8) and automaton updates (K9) on the LDS copies
+        const int32_t *y = p.encoded_Y + (int64_t)ex * K;
+        for (int j = tid; j < n_own * K; j += FITP_BLOCK) {
+            const int cl = j / K, k = j - cl * K;
+            int cs = sums[k];
+            cs = cs > p.T ? p.T : (cs < -p.T ? -p.T : cs);
+            const int yk = y[k];
+            const int target = 1 - 2 * (cs > yk);
+            int w = wts[j];
+            const int sign = (w >= 0) - (w < 0);
+            int err = yk - cs;
+            err = err < 0 ? -err : err;
+            const bool skip = (target == -1 && (uint64_t)gate[2 * j] >= p.q_thr) ||
+                              ((uint64_t)gate[2 * j + 1] * (uint64_t)(2 * (int64_t)p.T) >= ((uint64_t)err << 32));
+            const int u = skip ? 0 : target * sign;
+            const bool fired = node_of[cl] != -1;
+            if (u > 0 && fired && (w < 0 ? -(int64_t)w : (int64_t)w) < 2147483647) {
+                wts[j] = w + sign;
+            } else if (u < 0 && fired) {
+                w -= sign;
+                if (p.negative == 0 && w < 1) w = 1;
+                wts[j] = w;
+            }
+            upd[j] = u;
+        }
+        __syncthreads();
+        // Type I feedback bits, one thread per (clause, word, class) that needs them
+        for (int j = tid; j < n_own * LA * K; j += FITP_BLOCK) {
+            const int k = j % K, cw = j / K;
+            const int cl = cw / LA, w = cw - cl * LA;
+            if (upd[cl * K + k] > 0)
+                fbits[j] = gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
+        }
+        __syncthreads();
+        const uint32_t *X_rows = p.X + (int64_t)base_now * LA;
+        for (int j = tid; j < n_own * LA; j += FITP_BLOCK) {
+            const int cl = j / LA, w = j - cl * LA;
+            const int32_t *u_of = upd + cl * K;
+            bool any = false;
+            for (int k = 0; k < K; ++k) any |= u_of[k] != 0;
+            if (!any) continue;
+            const int node = node_of[cl];
+            const bool fired = node != -1;
+            const bool within = incl_of[cl] <= p.max_included;
+            const uint32_t x = !fired ? 0u : (j == tid ? x_mine : X_rows[(int64_t)node * LA + w]);
+            feedback_word_any(ta + (size_t)j * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1,
+                              (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, p.thr16, fbits + (size_t)j * K);
+        }
+        __syncthreads();
+        n_now = n_next;
+        base_now = base_next;
+        n_next = n_after;
+        base_next = base_after;
+    }
+    // own state -> global memory (also after an abort: every clause is left as of some whole step)
+    for (int i = tid; i < n_own * LA * B; i += FITP_BLOCK) p.bank[(int64_t)c0 * LA * B + i] = ta[i];
+    for (int i = tid; i < n_own * K; i += FITP_BLOCK) {
+        int cl = i / K, k = i - cl * K;
+        p.weights[(int64_t)k * p.C + c0 + cl] = wts[i];
+    }
+}

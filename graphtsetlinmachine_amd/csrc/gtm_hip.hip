@@ -287,6 +287,12 @@ __global__ void k_messages_scatter(const uint32_t *__restrict__ bitmap, int C, i
     }
 }
 
+// p[0..n) = v, p[n..total) = 0
+__global__ void k_fill_u64(unsigned long long *p, int64_t n, unsigned long long v, int64_t total) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) p[i] = i < n ? v : 0ull;
+}
+
 __global__ void k_fill_i32(int32_t *p, int64_t n, int32_t v) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
@@ -401,6 +407,7 @@ __device__ __forceinline__ void ta_dec(uint32_t *ta, int B, uint32_t active) {
 }
 
 #include "fit_fused.h"
+#include "fit_persistent.h"
 
 // K9 / K10: one thread per (clause, automaton word); the classes are applied
 // in ascending order to that word, as kernels.py:205-207,236-238 do per clause
@@ -514,7 +521,8 @@ FitWs carve_fit(const Dims &d, const gtm_config *cfg, char *base) {
     w.bitmap_b = (uint32_t *)take((size_t)d.C * d.NC * 4);
     for (int l = 0; l < GTM_MAX_DEPTH - 1; ++l)
         w.clause_X[l] = l < cfg->depth - 1 ? (uint32_t *)take((size_t)cfg->max_nodes * d.MC * 4) : nullptr;
-    w.class_sum = (int32_t *)take((size_t)d.K * 4 * 2);  // two buffers, used alternately by the fused path
+    // the fused paths rotate class-sum buffers: 2 x int32 [K], or 3 x 64-bit [K] followed by an abort flag
+    w.class_sum = (int32_t *)take(((size_t)d.K * 6 + 2) * 4);
     w.clause_node = (int32_t *)take((size_t)d.C * 4);
     w.n_incl = (int32_t *)take((size_t)d.C * 4);
     w.update = (int32_t *)take((size_t)d.K * d.C * 4);
@@ -920,6 +928,101 @@ int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *
 
 namespace {
 
+// `_fit`'s inner loop as one cooperative launch (fit_persistent.h).  Returns
+// GTM_OK with *done = false when this device / shape cannot run it, so that the
+// caller falls back to per-example launches.
+int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
+                   const FitWs &w, const int32_t *encoded_Y, int first_example, int n_examples, uint64_t first_step,
+                   hipStream_t st, bool *done) {
+    *done = false;
+    if (getenv("GTM_NO_PERSISTENT_FIT")) return GTM_OK;
+    int dev = 0, coop = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return GTM_OK;
+    if (hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) != hipSuccess || !coop) return GTM_OK;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) return GTM_OK;
+
+    FitPersistParams p{};
+    p.max_words = tg.slot_words > 0 ? tg.slot_words : 1;
+    p.rows_words = (cfg->literals + g->number_of_node_types + 1) * p.max_words;
+    // one clause per wave and step where the chip has room for that many groups
+    const int waves = FITP_BLOCK / 64;
+    int per_group = (d.C + cus - 1) / cus;
+    if (per_group < waves) per_group = waves;
+    const int groups = (d.C + per_group - 1) / per_group;
+    p.clauses_per_group = per_group;
+    size_t lds_words = 2 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group * d.K +
+                       2 * (size_t)per_group + 2 * (size_t)d.K + 2 * (size_t)per_group * d.K +
+                       (size_t)per_group * d.LA * d.K;
+    size_t lds = lds_words * 4;
+    if (lds > 150 * 1024) return GTM_OK;
+    static thread_local size_t lds_set = 0;
+    if (lds > lds_set) {
+        if (hipFuncSetAttribute((const void *)k_fit_persistent, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+            hipSuccess) {
+            (void)hipGetLastError();
+            return GTM_OK;
+        }
+        lds_set = lds;
+    }
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_fit_persistent, FITP_BLOCK, lds) != hipSuccess ||
+        per_cu < 1 || groups > per_cu * cus) {
+        (void)hipGetLastError();
+        return GTM_OK;
+    }
+
+    Key key = key_of(cfg);
+    p.tiles = g->tiles;
+    p.X = g->X;
+    p.node_index = g->node_index;
+    p.n_nodes = g->number_of_graph_nodes;
+    p.encoded_Y = encoded_Y;
+    p.tg = tg;
+    p.first_example = first_example;
+    p.n_examples = n_examples;
+    p.first_step = (uint32_t)first_step;
+    p.bank = s->ta_state;
+    p.weights = s->clause_weights;
+    p.literals = cfg->literals;
+    p.n_types = g->number_of_node_types;
+    p.C = d.C;
+    p.LA = d.LA;
+    p.B = d.B;
+    p.K = d.K;
+    p.T = cfg->threshold;
+    p.negative = cfg->negative_clauses;
+    p.boost = cfg->boost_true_positive_feedback;
+    p.max_included = cfg->max_included_literals;
+    p.filter = d.filter;
+    p.thr16 = feedback_threshold(cfg->s[0]);
+    p.k0 = key.k0;
+    p.k1 = key.k1;
+    p.q_thr = q_threshold(cfg->q, cfg->classes);
+    p.class_sum = (unsigned long long *)w.class_sum;
+    p.abort_flag = (uint32_t *)(w.class_sum + (size_t)d.K * 6);
+    p.spin_limit = 4000000u;  // a few seconds of polling at the very most
+    if (const char *e = getenv("GTM_FIT_SPIN_LIMIT")) p.spin_limit = (uint32_t)strtoul(e, nullptr, 10);  // tests force the give-up path
+
+    hipLaunchKernelGGL(k_fill_u64, dim3(blocks_for((int64_t)d.K * 3 + 1, TPB)), dim3(TPB), 0, st,
+                       (unsigned long long *)w.class_sum, (int64_t)d.K * 3, FITP_BIAS, (int64_t)d.K * 3 + 1);
+    if (int rc = check_launch("fill")) return rc;
+    void *args[] = {&p};
+    profile_start("k_fit_persistent", st);
+    hipError_t e = hipLaunchCooperativeKernel((const void *)k_fit_persistent, dim3(groups), dim3(FITP_BLOCK), args,
+                                              (unsigned)lds, st);
+    if (e != hipSuccess) return fail(GTM_ERR_HIP, "cooperative launch of the training kernel: %s", hipGetErrorString(e));
+    profile_stop(st);
+    uint32_t flag = 0;
+    e = hipMemcpyAsync(&flag, p.abort_flag, 4, hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return fail(GTM_ERR_HIP, "training kernel: %s", hipGetErrorString(e));
+    if (flag != 0)
+        return fail(GTM_ERR_HIP, "training kernel gave up waiting at its device-wide barrier (%d workgroups); "
+                                 "the model state is inconsistent", groups);
+    *done = true;
+    return GTM_OK;
+}
+
 // `_fit`'s inner loop for a depth-1 model on a data set that has tiles: two
 // launches per example (fit_fused.h).
 int fit_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
@@ -1008,9 +1111,15 @@ int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *st
 
     if (cfg->depth == 1 && graphs->tiles) {
         TileGeom tg = geometry_for(cfg, graphs, d.K);
-        if (tg.ok && tg.slot_words <= 64)  // one lane per word of the graph's slot
+        if (tg.ok && tg.slot_words <= 64) {  // one lane per word of the graph's slot
+            bool done = false;
+            if (int rc = fit_persistent(d, cfg, graphs, state, tg, w, encoded_Y, first_example, n_examples, first_step,
+                                        st, &done))
+                return rc;
+            if (done) return GTM_OK;
             return fit_on_tiles(d, cfg, graphs, state, tg, w, encoded_Y, first_example, n_examples, first_step, h_n,
                                 h_base, st);
+        }
     }
     for (int i = 0; i < n_examples; ++i) {
         int ex = first_example + i;

@@ -13,7 +13,9 @@
  *    pointer owned by the caller (the Python side takes them from torch
  *    tensors); the library never allocates or frees device memory;
  *  - `stream` is a hipStream_t passed as void* (NULL = the default stream);
- *    all work is enqueued on it and no entry point synchronises;
+ *    all work is enqueued on it.  Only gtm_fit and the two single-graph
+ *    training operators that take an example index wait for the stream (to
+ *    read the example's size, and gtm_fit also to report a failed run);
  *  - the return value is GTM_OK or an error code; gtm_last_error() gives the
  *    text for the calling thread.  No C++ exception crosses the boundary;
  *  - memory layouts are the reference's: X uint32 [nodes][LA_CHUNKS];
@@ -184,7 +186,11 @@ size_t gtm_fit_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs);
 /* The inner loop of `_fit` (tm.py:669-747) over examples
  * [first_example, first_example + n_examples), strictly in order (online
  * learning: example e+1 sees the state left by e).  Example i uses training
- * step first_step + i for its random draws. */
+ * step first_step + i for its random draws.  With depth == 1 and
+ * graphs->tiles set the whole run is one cooperative launch in which each
+ * workgroup keeps its clauses' automata in LDS and the class sums are the
+ * only exchange between workgroups; if that launch gives up waiting for a
+ * workgroup (bounded wait) the call returns GTM_ERR_HIP. */
 int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, const int32_t *encoded_Y,
             int32_t first_example, int32_t n_examples, uint64_t first_step, void *workspace,
             size_t workspace_bytes, void *stream);

@@ -253,9 +253,14 @@ def test_tile_scoring_equals_oracle(shape, density):
 
 @pytest.mark.parametrize("shape", TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
 @pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 6, 5)])
-def test_fused_fit_on_every_tile_geometry(shape, boost, max_included, state_bits):
-    """The fused depth-1 training step == the oracle == the per-operator path."""
+@pytest.mark.parametrize("persistent", [True, False], ids=["one-launch", "two-per-graph"])
+def test_fused_fit_on_every_tile_geometry(shape, boost, max_included, state_bits, persistent, monkeypatch):
+    """Both fused depth-1 training paths (one cooperative launch per run of
+    examples; two launches per example) == the oracle."""
     from tests.gpu_harness import Device
+
+    if not persistent:
+        monkeypatch.setenv("GTM_NO_PERSISTENT_FIT", "1")
 
     g = dict(shape["g"])
     g["n_graphs"] = min(g["n_graphs"], 24)
@@ -307,3 +312,31 @@ def test_empty_graphs_score_like_the_reference_arithmetic():
     assert np.array_equal(dev.score(0, 6, 6), want)
     assert dev.build_tiles()
     assert np.array_equal(dev.score(0, 6, 6), want)
+
+
+def test_training_kernel_gives_up_instead_of_hanging(monkeypatch):
+    """The one-launch training kernel waits for the other workgroups with a
+    bounded number of polls.  A limit of 0 makes every wait give up at once: the
+    kernel must still drain and the call must report it."""
+    from tests.gpu_harness import Device
+    from graphtsetlinmachine_amd import _abi
+
+    shape = TILE_SHAPES[3]
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    cfg = helpers.oracle_config(graphs, classes=shape["classes"], clauses=shape["clauses"], T=30)
+    model = helpers.random_model(shape["seed"], cfg, 1, s=3.0, include_density=0.02)
+    dev = Device(model, graphs)
+    assert dev.build_tiles()
+    Y = o.encode_labels(np.zeros(graphs.number_of_graphs, dtype=np.int64), cfg.classes, cfg.threshold)
+    monkeypatch.setenv("GTM_FIT_SPIN_LIMIT", "0")
+    with pytest.raises(_abi.GtmError, match="gave up waiting"):
+        dev.fit(Y, 0, graphs.number_of_graphs, 0)
+    monkeypatch.delenv("GTM_FIT_SPIN_LIMIT")
+    # the device and the library are still usable afterwards
+    model2 = helpers.random_model(shape["seed"] + 1, cfg, 1, s=3.0, include_density=0.02)
+    dev2 = Device(model2, graphs)
+    assert dev2.build_tiles()
+    o.fit(model2, graphs, Y)
+    dev2.fit(Y, 0, graphs.number_of_graphs, 0)
+    ta, _, w = dev2.download()
+    assert np.array_equal(w, model2.clause_weights) and np.array_equal(ta, model2.ta_state)
