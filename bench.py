@@ -39,7 +39,71 @@ def parse():
     p.add_argument("--train-epochs", type=int, default=1)
     p.add_argument("--cpu-sample", type=int, default=None, help="graphs timed on the CPU oracle")
     p.add_argument("--no-cpu", action="store_true")
+    p.add_argument("--only-main", action="store_true", help="skip the short runs of the other four configurations")
     return p.parse_args()
+
+
+# (train graphs, test graphs) for the short runs of the configurations that are not the main one
+OTHER_WORKLOADS = {
+    "noisy_xor": (10000, 10000),
+    "single_node_images": (20000, 10000),
+    "convolutional_images": (5000, 2000),
+    "sequence_chains": (1000, 500),
+    "colour_convolution": (48, 32),
+}
+
+
+def oracle_twin(tm, n_nodes):
+    """The CPU oracle's model object holding the GPU model's current state."""
+    from oracle import gtm_oracle as o
+
+    state = tm.get_state()
+    cfg = o.Config(classes=tm.number_of_outputs, clauses=tm.number_of_clauses, literals=tm.number_of_literals,
+                   state_bits=tm.number_of_state_bits, threshold=tm.T, q=tm.q,
+                   max_included_literals=tm.max_included_literals, max_nodes=n_nodes,
+                   message_size=tm.message_size, message_bits=tm.message_bits)
+    model = o.new_model(cfg, tm.depth, tm.s, tm.hypervectors, seed=tm.seed)
+    model.ta_state = state[0].reshape(cfg.clauses, cfg.la_chunks, cfg.state_bits).copy()
+    model.message_ta_state = [b.reshape(cfg.clauses, cfg.message_chunks, cfg.state_bits).copy()
+                              for b in tm.message_ta_state]
+    model.clause_weights = state[1].reshape(cfg.classes, cfg.clauses).copy()
+    return model
+
+
+def short_run(name, n_train, n_test, check_graphs):
+    """Train one epoch and score once on a reduced copy of a configuration; check a few class sums
+    against the CPU oracle."""
+    import numpy as np
+    import torch
+
+    from graphtsetlinmachine_amd import workloads
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+    from oracle import gtm_oracle as o
+
+    wl = workloads.BUILDERS[name](n_train=n_train, n_test=n_test)
+    np.random.seed(42)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=0, incremental=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
+    torch.cuda.synchronize()
+    t_train = time.perf_counter() - t0
+    tm.score_device(wl.graphs_test)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    sums = tm.score_device(wl.graphs_test)
+    torch.cuda.synchronize()
+    t_test = time.perf_counter() - t0
+    sums = sums.cpu().numpy().reshape(n_test, -1)
+    model = oracle_twin(tm, int(wl.graphs_test.max_number_of_graph_nodes))
+    want = o.score(model, wl.graphs_test, range(check_graphs))
+    return {
+        "train_graphs": n_train, "test_graphs": n_test, "train_graphs_per_s": round(n_train / t_train, 1),
+        "inference_graphs_per_s": round(n_test / t_test, 1),
+        "test_accuracy": round(float((sums.argmax(axis=1) == wl.Y_test).mean()), 4),
+        "class_sums_equal_oracle_on": check_graphs if np.array_equal(want, sums[:check_graphs]) else "MISMATCH",
+    }
 
 
 def eval_bytes_per_graph(n_nodes, la_chunks, clauses, node_chunks):
@@ -147,16 +211,7 @@ def main():
         # the NumPy oracle costs ~3.5 ns per clause x node x word; aim at ~15 s
         sample = args.cpu_sample or max(8, int(15.0 / (tm.number_of_clauses * n_nodes * la * tm.depth * 3.5e-9)))
         sample = min(sample, args.graphs)
-        state = tm.get_state()
-        cfg = o.Config(classes=tm.number_of_outputs, clauses=tm.number_of_clauses, literals=tm.number_of_literals,
-                       state_bits=tm.number_of_state_bits, threshold=tm.T, q=tm.q,
-                       max_included_literals=tm.max_included_literals, max_nodes=n_nodes,
-                       message_size=tm.message_size, message_bits=tm.message_bits)
-        model = o.new_model(cfg, tm.depth, tm.s, tm.hypervectors, seed=tm.seed)
-        model.ta_state = state[0].reshape(cfg.clauses, cfg.la_chunks, cfg.state_bits).copy()
-        model.message_ta_state = [b.reshape(cfg.clauses, cfg.message_chunks, cfg.state_bits).copy()
-                                  for b in tm.message_ta_state]
-        model.clause_weights = state[1].reshape(cfg.classes, cfg.clauses).copy()
+        model = oracle_twin(tm, n_nodes)
         t0 = time.perf_counter()
         want = o.score(model, test, range(sample))
         t_cpu = time.perf_counter() - t0
@@ -166,6 +221,16 @@ def main():
         cpu = {"value": round(sample / t_cpu, 2), "unit": "graphs/s", "cores": 1, "kind": "port",
                "sample": "NumPy oracle, inference on the first %d test graphs (%.1f s), checked equal to the GPU sums"
                          % (sample, t_cpu)}
+
+    others = {}
+    if not args.only_main:
+        for name, (n_train, n_test) in OTHER_WORKLOADS.items():
+            if name == args.workload:
+                continue
+            others[name] = short_run(name, n_train, n_test, check_graphs=2 if name == "colour_convolution" else 16)
+            if others[name]["class_sums_equal_oracle_on"] == "MISMATCH":
+                print("bench.py: GPU class sums differ from the CPU oracle on %s" % name, file=sys.stderr)
+                sys.exit(1)
 
     line = {
         "metric": "inference graphs/sec on 1 MI355X (%s)" % args.workload,
@@ -180,6 +245,7 @@ def main():
         "roofline": roofline, "cpu_baseline": cpu,
         "train_graphs_per_s": round(train_gps, 1), "test_accuracy": round(accuracy, 4),
         "event_ms_per_step": round(event_ms, 4), "data_build_s": round(t_data, 1),
+        "other_workloads": others,
     }
     print(json.dumps(line))
 
