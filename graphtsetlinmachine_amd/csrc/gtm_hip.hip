@@ -944,17 +944,20 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     FitPersistParams p{};
     p.max_words = tg.slot_words > 0 ? tg.slot_words : 1;
     p.rows_words = (cfg->literals + g->number_of_node_types + 1) * p.max_words;
-    // one clause per wave and step where the chip has room for that many groups
+    // One clause per wave and step (16 per group) where that fits; fewer per group when the
+    // automata of 16 clauses do not fit in LDS and the chip has room for more groups.
     const int waves = FITP_BLOCK / 64;
+    auto lds_bytes = [&](int per_group) {
+        return (2 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group +
+                2 * (size_t)d.K + 4 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K) * 4;
+    };
+    const size_t lds_limit = 150 * 1024;
     int per_group = (d.C + cus - 1) / cus;
-    if (per_group < waves) per_group = waves;
+    if (per_group < waves && lds_bytes(waves) <= lds_limit) per_group = waves;
+    if (lds_bytes(per_group) > lds_limit) return GTM_OK;
     const int groups = (d.C + per_group - 1) / per_group;
     p.clauses_per_group = per_group;
-    size_t lds_words = 2 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group * d.K +
-                       2 * (size_t)per_group + 2 * (size_t)d.K + 2 * (size_t)per_group * d.K +
-                       (size_t)per_group * d.LA * d.K;
-    size_t lds = lds_words * 4;
-    if (lds > 150 * 1024) return GTM_OK;
+    const size_t lds = lds_bytes(per_group);
     static thread_local size_t lds_set = 0;
     if (lds > lds_set) {
         if (hipFuncSetAttribute((const void *)k_fit_persistent, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=

@@ -48,12 +48,18 @@ inline TileGeom tile_geometry(int literals, int n_types, int max_nodes, int n_gr
         TileGeom g{};
         g.lw = lw;
         const int max_words = 64 * lw;
+        g.rows = literals + n_types + 1;
         if (max_nodes <= 16) {
             int s = 1;
             while (s < max_nodes) s <<= 1;
             g.slot_bits = s;
+            // many literals: narrower rows (fewer graphs per tile) until the tile fits in LDS
             g.tw = max_words;
-            g.gpt = max_words * 32 / s;
+            g.gpt = g.tw * 32 / s;
+            while (g.tw > 4 * lw && tile_lds_bytes(g, classes) > TILE_LDS_BUDGET) {
+                g.tw >>= 1;
+                g.gpt = g.tw * 32 / s;
+            }
         } else {
             g.slot_words = ((max_nodes - 1) / 32 + 1 + lw - 1) / lw * lw;
             g.slot_bits = g.slot_words * 32;

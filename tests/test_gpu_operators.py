@@ -219,6 +219,9 @@ TILE_SHAPES = [
     # tiny graphs (several per word), one word, several words, exactly 64 words, more than one node type
     dict(seed=11, g=dict(n_graphs=300, max_nodes=1, hv_size=40), classes=3, clauses=50),
     dict(seed=12, g=dict(n_graphs=200, max_nodes=3, hv_size=16, node_types=("a", "b")), classes=2, clauses=64),
+    # many literals: the tile narrows until its rows fit in LDS
+    dict(seed=20, g=dict(n_graphs=150, max_nodes=1, hv_size=1500, n_symbols=40), classes=3, clauses=40),
+    dict(seed=21, g=dict(n_graphs=90, max_nodes=2, hv_size=700, n_symbols=30), classes=10, clauses=50),
     dict(seed=13, g=dict(n_graphs=70, max_nodes=16, min_nodes=9, hv_size=20), classes=4, clauses=33),
     dict(seed=14, g=dict(n_graphs=40, max_nodes=31, min_nodes=17, hv_size=64), classes=10, clauses=200),
     dict(seed=15, g=dict(n_graphs=23, max_nodes=361, min_nodes=300, hv_size=128, max_degree=0), classes=10, clauses=120),
