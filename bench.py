@@ -23,7 +23,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# HBM bytes per graph that k_score_tiles moves on the convolutional workload, from rocprofv3 --pmc runs
+# HBM bytes per graph that the tile scoring kernel moves on the convolutional workload, from rocprofv3 --pmc runs
 # (FETCH_SIZE x 2 KiB, the factor a 256 MiB copy kernel calibrates, + WRITE_SIZE x 1 KiB, over 10,000 graphs).
 MEASURED_TRAFFIC_BYTES_PER_GRAPH = {"convolutional_images": (72096.1 * 2 + 406.2) * 1024 / 10000}
 
@@ -197,7 +197,7 @@ def main():
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
         "traffic": (round(MEASURED_TRAFFIC_BYTES_PER_GRAPH[args.workload] * graphs_per_launch)
-                    if args.workload in MEASURED_TRAFFIC_BYTES_PER_GRAPH and kernel_name == "k_score_tiles" else None),
+                    if args.workload in MEASURED_TRAFFIC_BYTES_PER_GRAPH and kernel_name == "k_tile_layer<score>" else None),
         "kernel": kernel_name, "kernel_ms": round(kernel_ms, 4), "launches": launches,
         "graphs_per_launch": graphs_per_launch,
         "algorithmic_bytes_per_graph": b_eval,

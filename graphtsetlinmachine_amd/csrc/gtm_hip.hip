@@ -460,18 +460,29 @@ Key key_of(const gtm_config *cfg) { return Key{(uint32_t)(cfg->seed & 0xFFFFFFFF
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct ScoreWs {
-    uint32_t *lists;     // [C][list_stride]  (literal-major tile path)
-    int32_t *wt;         // [C][K]
+    uint32_t *lists;          // [C][list_stride]  (literal-major tile path)
+    int32_t *wt;              // [C][K]
     int list_stride;
-    uint32_t *inc_t;     // [max(LA,MC)][C]
-    uint32_t *bitmap_a;  // [batch][C][NC]
-    uint32_t *bitmap_b;  // [batch][C][NC] (depth > 1)
-    uint32_t *clause_X;  // [batch][max_nodes][MC] (depth > 1)
+    uint32_t *message_lists;  // [depth-1][C][message_list_stride]  (tile path, depth > 1)
+    int message_list_stride;
+    uint32_t *tile_bitmap;    // [tiles per launch][C][tw]  (tile path, depth > 1)
+    uint32_t *inc_t;          // [max(LA,MC)][C]
+    uint32_t *bitmap_a;       // [batch][C][NC]
+    uint32_t *bitmap_b;       // [batch][C][NC] (depth > 1)
+    uint32_t *clause_X;       // [batch][max_nodes][MC] (depth > 1)
     size_t bytes;
 };
 
-ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base) {
-    ScoreWs w;
+// Length of a compiled clause: header + type row + literals, padded to 32 entries, + 32 entries
+// that the kernel may fetch ahead unused.
+int clause_list_stride(int literals) { return ((literals + 2 + 31) & ~31) + 32; }
+
+// Tiles one launch group covers when the caller asks for `batch` graphs at a time.
+int tiles_per_batch(const TileGeom &tg, int batch) { return (batch + tg.gpt - 1) / tg.gpt; }
+
+// `tg`: the data set's tile geometry when the tile path will run (its buffers replace the dense ones).
+ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base, const TileGeom *tg = nullptr) {
+    ScoreWs w{};
     size_t off = 0;
     int chunks = cfg->depth > 1 && d.MC > d.LA ? d.MC : d.LA;
     auto take = [&](size_t bytes) {
@@ -479,18 +490,25 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base)
         off += align_up(bytes);
         return p;
     };
-    // header + type row + literals, padded to 32 entries, + 32 entries that the kernel may fetch ahead unused
-    w.list_stride = ((cfg->literals + 2 + 31) & ~31) + 32;
+    w.list_stride = clause_list_stride(cfg->literals);
     w.lists = (uint32_t *)take((size_t)d.C * w.list_stride * 4);
     w.wt = (int32_t *)take((size_t)d.C * d.K * 4);
+    if (tg && cfg->depth == 1) {
+        w.bytes = off;
+        return w;
+    }
+    if (tg) {
+        w.message_list_stride = clause_list_stride(2 * d.M);
+        w.message_lists = (uint32_t *)take((size_t)(cfg->depth - 1) * d.C * w.message_list_stride * 4);
+        w.tile_bitmap = (uint32_t *)take((size_t)tiles_per_batch(*tg, batch) * d.C * tg->tw * 4);
+        w.bytes = off;
+        return w;
+    }
     w.inc_t = (uint32_t *)take((size_t)chunks * d.C * 4);
     w.bitmap_a = (uint32_t *)take((size_t)batch * d.C * d.NC * 4);
     if (cfg->depth > 1) {
         w.bitmap_b = (uint32_t *)take((size_t)batch * d.C * d.NC * 4);
         w.clause_X = (uint32_t *)take((size_t)batch * cfg->max_nodes * d.MC * 4);
-    } else {
-        w.bitmap_b = nullptr;
-        w.clause_X = nullptr;
     }
     w.bytes = off;
     return w;
@@ -607,7 +625,7 @@ int validate_state(const gtm_config *cfg, const gtm_state *s) {
 // Words of bit rows in a tile buffer, padded so that the row counts after them are 8-byte aligned.
 size_t tiles_words(const TileGeom &tg) { return ((size_t)tg.n_tiles * tg.rows * tg.tw + 1) & ~(size_t)1; }
 
-// Depth-1 inference on literal-major tiles (see score_tiles.h).
+// Inference on literal-major tiles (see score_tiles.h).
 int max_lane_words() {
     const char *e = getenv("GTM_TILE_LANE_WORDS");  // 1, 2 or 4: upper bound on words per lane (tuning aid)
     int v = e ? atoi(e) : 4;
@@ -616,42 +634,112 @@ int max_lane_words() {
 
 TileGeom geometry_for(const gtm_config *cfg, const gtm_graphs *g, int classes) {
     return tile_geometry(cfg->literals, g->number_of_node_types, g->max_number_of_graph_nodes, g->number_of_graphs,
-                         classes, max_lane_words());
+                         classes, max_lane_words(), cfg->depth > 1 ? tile_message_rows(cfg->message_size) : 0);
 }
 
-template <int NW, int LW>
-int launch_score_tiles(const Dims &d, const gtm_graphs *g, const TileGeom &tg, const ScoreWs &w, int first,
-                       int n_graphs, int32_t *class_sum, hipStream_t st) {
-    size_t lds = tile_lds_bytes(tg, d.K);
+template <int NW, int LW, int SRC, bool LAST>
+int launch_tile_layer_as(const TileLayerArgs &a, int n_tiles, const char *profile_name, hipStream_t st) {
+    size_t lds = tile_layer_lds_bytes(a.tg, a.K, SRC, a.M);
     static thread_local size_t lds_set = 0;
     if (lds > lds_set) {
-        hipError_t e = hipFuncSetAttribute((const void *)k_score_tiles<NW, LW>,
+        hipError_t e = hipFuncSetAttribute((const void *)k_tile_layer<NW, LW, SRC, LAST>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
         lds_set = lds;
     }
-    int tile0 = first / tg.gpt, tile1 = (first + n_graphs - 1) / tg.gpt;
-    profile_start("k_score_tiles", st);
-    hipLaunchKernelGGL((k_score_tiles<NW, LW>), dim3(tile1 - tile0 + 1), dim3(NW * 64), lds, st, g->tiles, tg, d.C, d.K,
-                       w.lists, w.list_stride, w.wt, tile0, first, n_graphs, class_sum);
-    if (int rc = check_launch("score_tiles")) return rc;
-    profile_stop(st);
+    if (profile_name) profile_start(profile_name, st);
+    hipLaunchKernelGGL((k_tile_layer<NW, LW, SRC, LAST>), dim3(n_tiles), dim3(NW * 64), lds, st, a);
+    if (int rc = check_launch("tile_layer")) return rc;
+    if (profile_name) profile_stop(st);
     return GTM_OK;
 }
 
-int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
-                   const ScoreWs &w, int first, int n_graphs, int32_t *class_sum, hipStream_t st) {
-    const uint32_t *order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
-    hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C, d.LA,
-                       d.B, d.filter, d.K, s->clause_weights, cfg->literals, g->number_of_node_types, tg.tw,
-                       w.list_stride, order, w.lists, w.wt);
-    if (int rc = check_launch("compile_clauses")) return rc;
+template <int NW, int LW>
+int launch_tile_layer_lw(const TileLayerArgs &a, int n_tiles, int src, bool last, hipStream_t st) {
+    if (src == ROWS_MESSAGES)
+        return last ? launch_tile_layer_as<NW, LW, ROWS_MESSAGES, true>(a, n_tiles, nullptr, st)
+                    : launch_tile_layer_as<NW, LW, ROWS_MESSAGES, false>(a, n_tiles, nullptr, st);
+    if (src == ROWS_GLOBAL)
+        return last ? launch_tile_layer_as<NW, LW, ROWS_GLOBAL, true>(a, n_tiles, nullptr, st)
+                    : launch_tile_layer_as<NW, LW, ROWS_GLOBAL, false>(a, n_tiles, nullptr, st);
+    return last ? launch_tile_layer_as<NW, LW, ROWS_STAGED, true>(a, n_tiles, "k_tile_layer<score>", st)
+                : launch_tile_layer_as<NW, LW, ROWS_STAGED, false>(a, n_tiles, nullptr, st);
+}
+
+int launch_tile_layer(const TileLayerArgs &a, int n_tiles, int src, bool last, hipStream_t st) {
     constexpr int NW = 16;
-    switch (tg.lw) {
-        case 1: return launch_score_tiles<NW, 1>(d, g, tg, w, first, n_graphs, class_sum, st);
-        case 2: return launch_score_tiles<NW, 2>(d, g, tg, w, first, n_graphs, class_sum, st);
-        default: return launch_score_tiles<NW, 4>(d, g, tg, w, first, n_graphs, class_sum, st);
+    switch (a.tg.lw) {
+        case 1: return launch_tile_layer_lw<NW, 1>(a, n_tiles, src, last, st);
+        case 2: return launch_tile_layer_lw<NW, 2>(a, n_tiles, src, last, st);
+        default: return launch_tile_layer_lw<NW, 4>(a, n_tiles, src, last, st);
     }
+}
+
+// `_score`'s loop (tm.py:786-812) on tiles: per launch group of tiles, layer 0 and then one
+// launch per message layer; the clause truth rows between layers stay in w.tile_bitmap.
+int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
+                   const ScoreWs &w, int first, int n_graphs, int batch, int32_t *class_sum, hipStream_t st) {
+    const uint32_t *order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
+    const int layers = cfg->depth;
+    hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C, d.LA,
+                       d.B, d.filter, cfg->literals, 0, g->number_of_node_types, cfg->literals, tg.rows - 1, tg.tw,
+                       w.list_stride, order, w.lists, d.K, layers == 1 ? s->clause_weights : nullptr, w.wt);
+    if (int rc = check_launch("compile_clauses")) return rc;
+    for (int l = 1; l < layers; ++l) {
+        hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st,
+                           s->message_ta_state[l - 1], d.C, d.MC, d.B, d.mfilter, 2 * d.M, d.M, 0, 0, d.M, tg.tw,
+                           w.message_list_stride, (const uint32_t *)nullptr,
+                           w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride, d.K,
+                           l == layers - 1 ? s->clause_weights : nullptr, w.wt);
+        if (int rc = check_launch("compile_clauses")) return rc;
+    }
+    TileLayerArgs a{};
+    a.tiles = g->tiles;
+    a.tg = tg;
+    a.C = d.C;
+    a.K = d.K;
+    a.wt = w.wt;
+    a.bitmap = w.tile_bitmap;
+    a.M = d.M;
+    a.MB = d.MB;
+    a.G = g->number_of_graphs;
+    a.hv = s->hypervectors;
+    a.node_index = g->node_index;
+    a.n_nodes = g->number_of_graph_nodes;
+    a.n_edges = g->number_of_graph_node_edges;
+    a.edge_index = g->edge_index;
+    a.edge = g->edge;
+    if (layers == 1) {
+        // no truth rows are kept: every tile of the range in one launch
+        a.lists = w.lists;
+        a.stride = w.list_stride;
+        a.tile0 = first / tg.gpt;
+        a.first_graph = first;
+        a.n_graphs = n_graphs;
+        a.class_sum = class_sum;
+        int n_tiles = (first + n_graphs - 1) / tg.gpt - a.tile0 + 1;
+        return launch_tile_layer(a, n_tiles, tg.stage0 ? ROWS_STAGED : ROWS_GLOBAL, true, st);
+    }
+    if (g->total_edges > 0 && (!g->number_of_graph_node_edges || !g->edge || !g->edge_index))
+        return fail(GTM_ERR_INVALID, "graphs with edges need number_of_graph_node_edges, edge and edge_index");
+    const int tiles_per_launch = tiles_per_batch(tg, batch);
+    const int tile_first = first / tg.gpt, tile_last = (first + n_graphs - 1) / tg.gpt;
+    for (int t0 = tile_first; t0 <= tile_last; t0 += tiles_per_launch) {
+        const int n_tiles = tile_last - t0 + 1 < tiles_per_launch ? tile_last - t0 + 1 : tiles_per_launch;
+        a.tile0 = t0;
+        a.first_graph = first;
+        a.n_graphs = n_graphs;
+        a.class_sum = class_sum;
+        a.lists = w.lists;
+        a.stride = w.list_stride;
+        if (int rc = launch_tile_layer(a, n_tiles, tg.stage0 ? ROWS_STAGED : ROWS_GLOBAL, false, st)) return rc;
+        for (int l = 1; l < layers; ++l) {
+            a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
+            a.stride = w.message_list_stride;
+            if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1, st)) return rc;
+        }
+    }
+    return GTM_OK;
 }
 
 }  // namespace
@@ -889,11 +977,19 @@ int gtm_build_tiles(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *t
     return check_launch("row_order");
 }
 
+// The tile path runs when the data set carries tiles (gtm_build_tiles) of a supported shape.
+static bool score_uses_tiles(const gtm_config *cfg, const gtm_graphs *graphs, int classes, TileGeom *tg) {
+    if (!graphs || !graphs->tiles || graphs->number_of_graphs < 1 || graphs->number_of_node_types < 1) return false;
+    *tg = geometry_for(cfg, graphs, classes);
+    return tg->ok != 0;
+}
+
 size_t gtm_score_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs, int32_t batch) {
     Dims d;
     if (validate(cfg, &d) || batch < 1) return 0;
-    (void)graphs;
-    return carve_score(d, cfg, batch, nullptr).bytes;
+    TileGeom tg;
+    bool tiles = score_uses_tiles(cfg, graphs, d.K, &tg);
+    return carve_score(d, cfg, batch, nullptr, tiles ? &tg : nullptr).bytes;
 }
 
 int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, int32_t first_graph,
@@ -905,14 +1001,14 @@ int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *
     if (int rc = validate_state(cfg, state)) return rc;
     if (batch < 1) return fail(GTM_ERR_INVALID, "batch=%d", batch);
     if (!class_sum) return fail(GTM_ERR_INVALID, "class_sum is NULL");
-    ScoreWs w = carve_score(d, cfg, batch, (char *)workspace);
+    TileGeom tg;
+    bool tiles = score_uses_tiles(cfg, graphs, d.K, &tg);
+    ScoreWs w = carve_score(d, cfg, batch, (char *)workspace, tiles ? &tg : nullptr);
     if (!workspace || workspace_bytes < w.bytes)
         return fail(GTM_ERR_INVALID, "workspace of %zu bytes needed, %zu given", w.bytes, workspace_bytes);
     hipStream_t st = (hipStream_t)stream;
-    if (cfg->depth == 1 && graphs->tiles && n_graphs > 0) {
-        TileGeom tg = geometry_for(cfg, graphs, d.K);
-        if (tg.ok) return score_on_tiles(d, cfg, graphs, state, tg, w, first_graph, n_graphs, class_sum, st);
-    }
+    if (n_graphs == 0) return GTM_OK;
+    if (tiles) return score_on_tiles(d, cfg, graphs, state, tg, w, first_graph, n_graphs, batch, class_sum, st);
     for (int done = 0; done < n_graphs; done += batch) {
         int nb = n_graphs - done < batch ? n_graphs - done : batch;
         uint32_t *final_bitmap = nullptr;

@@ -30,52 +30,78 @@ struct TileGeom {
     int n_tiles;
     int lw;               // words of a row held by one lane (1, 2 or 4)
     int lanes_per_graph;  // slot_words / lw (0 when slot_bits < 32)
-    int ok;               // geometry supported by the fused kernel
+    int ok;               // geometry supported by the tile kernels
+    int stage0;           // the literal rows of layer 0 fit in LDS (else they are read from global memory)
 };
 
 constexpr size_t TILE_LDS_BUDGET = 156 * 1024;  // of the 160 KB per CU
 constexpr int TILE_LDS_PAD_WORDS = 256;         // readable words after the last row
 
-inline size_t tile_lds_bytes(const TileGeom &g, int classes) {
-    return ((size_t)g.rows * g.tw + TILE_LDS_PAD_WORDS + (size_t)g.gpt * classes) * 4;
+inline size_t tile_lds_bytes(int rows, const TileGeom &g, int classes) {
+    return ((size_t)rows * g.tw + TILE_LDS_PAD_WORDS + (size_t)g.gpt * classes) * 4;
 }
 
-// The widest lanes (most graphs per wave instruction) whose tile fits in LDS.
-inline TileGeom tile_geometry(int literals, int n_types, int max_nodes, int n_graphs, int classes, int max_lw = 4) {
-    TileGeom last{};
-    if (max_nodes < 1) max_nodes = 1;
-    for (int lw = max_lw; lw >= 1; lw >>= 1) {
-        TileGeom g{};
-        g.lw = lw;
-        const int max_words = 64 * lw;
-        g.rows = literals + n_types + 1;
-        if (max_nodes <= 16) {
-            int s = 1;
-            while (s < max_nodes) s <<= 1;
-            g.slot_bits = s;
-            // many literals: narrower rows (fewer graphs per tile) until the tile fits in LDS
-            g.tw = max_words;
+// Tile shape for `lw` words per lane whose `fit_rows` rows fit in LDS (ok = 0 if none does).
+inline TileGeom tile_geometry_lw(int literals, int n_types, int max_nodes, int n_graphs, int classes, int lw,
+                                 int fit_rows) {
+    TileGeom g{};
+    g.lw = lw;
+    g.rows = literals + n_types + 1;
+    const int max_words = 64 * lw;
+    if (max_nodes <= 16) {
+        int s = 1;
+        while (s < max_nodes) s <<= 1;
+        g.slot_bits = s;
+        // many rows: narrower rows (fewer graphs per tile) until the tile fits in LDS
+        g.tw = max_words;
+        g.gpt = g.tw * 32 / s;
+        while (g.tw > 4 * lw && tile_lds_bytes(fit_rows, g, classes) > TILE_LDS_BUDGET) {
+            g.tw >>= 1;
             g.gpt = g.tw * 32 / s;
-            while (g.tw > 4 * lw && tile_lds_bytes(g, classes) > TILE_LDS_BUDGET) {
-                g.tw >>= 1;
-                g.gpt = g.tw * 32 / s;
-            }
-        } else {
-            g.slot_words = ((max_nodes - 1) / 32 + 1 + lw - 1) / lw * lw;
-            g.slot_bits = g.slot_words * 32;
-            g.lanes_per_graph = g.slot_words / lw;
-            g.gpt = g.slot_words <= max_words ? max_words / g.slot_words : 0;
-            g.tw = g.gpt * g.slot_words;
-            if (g.tw & 3) g.tw = (g.tw + 3) & ~3;  // rows stay 16-byte aligned
         }
-        g.rows = literals + n_types + 1;
-        g.n_tiles = g.gpt > 0 ? (n_graphs + g.gpt - 1) / g.gpt : 0;
-        g.ok = g.gpt > 0 && tile_lds_bytes(g, classes) <= TILE_LDS_BUDGET;
-        if (g.ok) return g;
-        last = g;
+    } else {
+        g.slot_words = ((max_nodes - 1) / 32 + 1 + lw - 1) / lw * lw;
+        g.slot_bits = g.slot_words * 32;
+        g.lanes_per_graph = g.slot_words / lw;
+        g.gpt = g.slot_words <= max_words ? max_words / g.slot_words : 0;
+        // fewer graphs per tile until the rows fit
+        while (g.gpt > 1 && ((size_t)fit_rows * (((size_t)g.gpt * g.slot_words + 3) & ~(size_t)3) +
+                             TILE_LDS_PAD_WORDS + (size_t)g.gpt * classes) * 4 > TILE_LDS_BUDGET)
+            --g.gpt;
+        g.tw = (g.gpt * g.slot_words + 3) & ~3;  // rows stay 16-byte aligned
     }
-    last.ok = 0;
-    return last;
+    g.n_tiles = g.gpt > 0 ? (n_graphs + g.gpt - 1) / g.gpt : 0;
+    g.ok = g.gpt > 0 && tile_lds_bytes(fit_rows, g, classes) <= TILE_LDS_BUDGET;
+    g.stage0 = g.ok && tile_lds_bytes(g.rows, g, classes) <= TILE_LDS_BUDGET;
+    return g;
+}
+
+// The lane width with the fewest wave instructions per graph whose tile fits in LDS: one step of
+// a clause costs a wave one LDS read and `lw` ANDs whatever the number of lanes in use, and covers
+// `gpt` graphs.  `message_rows` > 0 (models with message layers) asks that that many rows fit too;
+// if the literal rows of layer 0 and the message rows cannot both fit, the message rows win and
+// layer 0 reads its rows from global memory.
+inline TileGeom tile_geometry(int literals, int n_types, int max_nodes, int n_graphs, int classes, int max_lw = 4,
+                              int message_rows = 0) {
+    if (max_nodes < 1) max_nodes = 1;
+    const int rows0 = literals + n_types + 1;
+    TileGeom best{};
+    for (int pass = 0; pass < 2; ++pass) {
+        const int fit_rows = pass == 0 ? (rows0 > message_rows ? rows0 : message_rows) : message_rows;
+        if (pass == 1 && message_rows == 0) break;
+        for (int lw = max_lw; lw >= 1; lw >>= 1) {
+            TileGeom g = tile_geometry_lw(literals, n_types, max_nodes, n_graphs, classes, lw, fit_rows);
+            if (!g.ok) {
+                if (!best.ok) best = g;
+                continue;
+            }
+            // (1 + lw) / gpt, compared without division; ties go to the wider lanes
+            if (!best.ok || (int64_t)(1 + g.lw) * best.gpt < (int64_t)(1 + best.lw) * g.gpt) best = g;
+        }
+        if (best.ok) return best;
+    }
+    best.ok = 0;
+    return best;
 }
 
 // One thread per tile word: gathers its 32 node slots.
@@ -150,42 +176,55 @@ __global__ void k_row_order(const unsigned long long *__restrict__ row_count, in
 }
 
 // Per call, one wave per clause: the rows the clause ANDs together, as 32-bit
-// LDS byte offsets (row * tw * 4).  Entry 0 = number of 8-entry blocks in use,
-// entry 1 = the row of the clause's node type (kernels.py:447), then its
-// included literals in `order`: the ones that hold least often come first, so
-// the running AND dies (and the walk stops) as early as it can; the order does
-// not change the result.  The list starts with a chunk of 32 entries that the
-// scoring kernel fetches one clause ahead; unused entries point at the
-// all-ones row.  Also the weights clause-major.
-__global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int LA, int B, uint32_t filter, int K,
-                                  const int32_t *__restrict__ weights, int literals, int n_types, int tw,
-                                  int stride, const uint32_t *__restrict__ order, uint32_t *__restrict__ lists,
-                                  int32_t *__restrict__ wt) {
+// LDS byte offsets (row * tw * 4).  Entry 0 = number of 8-entry blocks in use;
+// with n_types > 0 entry 1 = the row of the clause's node type
+// (kernels.py:447); then the clause's included literals, in `order` when
+// given: the ones that hold least often come first, so the running AND dies
+// (and the walk stops) as early as it can; the order does not change the
+// result.  With half > 0 (message banks) literal l >= half is the negation of
+// literal l - half and is stored as that row's offset with bit 31 set.  The
+// list starts with a chunk of 32 entries that the evaluating kernel fetches
+// one clause ahead; unused entries point at the all-ones row.  Also, when
+// `weights` is given, the weights clause-major.
+constexpr uint32_t TILE_NEGATED = 0x80000000u;
+
+__global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int chunks, int B, uint32_t filter,
+                                  int literals, int half, int n_types, int type_base_row, int ones_row, int tw,
+                                  int stride, const uint32_t *__restrict__ order, uint32_t *__restrict__ lists, int K,
+                                  const int32_t *__restrict__ weights, int32_t *__restrict__ wt) {
     const int lane = threadIdx.x & 63;
     const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (c >= C) return;
     const uint32_t row_bytes = (uint32_t)tw * 4u;
-    const uint32_t ones = (uint32_t)(literals + n_types) * row_bytes;
+    const uint32_t ones = (uint32_t)ones_row * row_bytes;
     uint32_t *list = lists + (int64_t)c * stride;
-    const uint32_t *inc = bank + (int64_t)c * LA * B + (B - 1);
-    if (lane == 0) list[1] = (uint32_t)(literals + c % n_types) * row_bytes;
-    int n = 2;
+    const uint32_t *inc = bank + (int64_t)c * chunks * B + (B - 1);
+    int n = 1;
+    if (n_types > 0) {
+        if (lane == 0) list[1] = (uint32_t)(type_base_row + c % n_types) * row_bytes;
+        n = 2;
+    }
     for (int r0 = 0; r0 < literals; r0 += 64) {
         int r = r0 + lane;
-        uint32_t lit = r < literals ? order[r] : 0u;
+        uint32_t lit = r < literals ? (order ? order[r] : (uint32_t)r) : 0u;
         uint32_t w = lit >> 5;
         uint32_t word = inc[(int64_t)w * B];
-        if ((int)w == LA - 1) word &= filter;
+        if ((int)w == chunks - 1) word &= filter;
         bool included = r < literals && ((word >> (lit & 31)) & 1u);
         unsigned long long mask = __ballot(included);
-        if (included) list[n + __popcll(mask & ((1ull << lane) - 1ull))] = lit * row_bytes;
+        if (included) {
+            uint32_t entry = (half > 0 && (int)lit >= half) ? ((lit - (uint32_t)half) * row_bytes) | TILE_NEGATED
+                                                            : lit * row_bytes;
+            list[n + __popcll(mask & ((1ull << lane) - 1ull))] = entry;
+        }
         n += __popcll(mask);
     }
     const int padded = (n + 7) & ~7;
     const int fill_to = padded < 32 ? 32 : (padded + 15) & ~15;
     for (int i = n + lane; i < fill_to; i += 64) list[i] = ones;
     if (lane == 0) list[0] = (uint32_t)(padded >> 3);
-    for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
+    if (weights)
+        for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
 }
 
 struct alignas(32) Block8 {
@@ -205,6 +244,7 @@ template <>
 struct LaneWords<1> {
     uint32_t w[1];
     __device__ __forceinline__ void load(const char *p) { w[0] = *reinterpret_cast<const uint32_t *>(p); }
+    __device__ __forceinline__ void store(char *p) const { *reinterpret_cast<uint32_t *>(p) = w[0]; }
 };
 template <>
 struct LaneWords<2> {
@@ -214,6 +254,7 @@ struct LaneWords<2> {
         w[0] = v.x;
         w[1] = v.y;
     }
+    __device__ __forceinline__ void store(char *p) const { *reinterpret_cast<uint2 *>(p) = make_uint2(w[0], w[1]); }
 };
 template <>
 struct LaneWords<4> {
@@ -225,108 +266,242 @@ struct LaneWords<4> {
         w[2] = v.z;
         w[3] = v.w;
     }
+    __device__ __forceinline__ void store(char *p) const {
+        *reinterpret_cast<uint4 *>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
 };
 
-// One workgroup per tile.  The tile's bit-rows are copied to LDS once; each
-// wave then walks its share of the clauses.  The clause id and its row list
-// are wave-uniform: the first 32 entries of a clause arrive by scalar loads
-// issued while the previous clause is being evaluated.  Lane L holds words
-// [L*LW, (L+1)*LW) of the running AND.
-template <int NWAVES, int LW>
-__global__ __launch_bounds__(NWAVES * 64) void k_score_tiles(
-    const uint32_t *__restrict__ tiles, TileGeom tg, int C, int K, const uint32_t *__restrict__ lists, int stride,
-    const int32_t *__restrict__ wt, int tile0, int first_graph, int n_graphs, int32_t *__restrict__ class_sum) {
+// Where a layer's bit-rows come from.
+constexpr int ROWS_STAGED = 0;   // the data set's tile (literal rows of layer 0), copied to LDS
+constexpr int ROWS_GLOBAL = 1;   // the data set's tile, read in place (rows too big for LDS)
+constexpr int ROWS_MESSAGES = 2; // message rows, built in LDS from the previous layer's bitmap
+
+struct TileLayerArgs {
+    const uint32_t *tiles;  // data set tiles (layer 0)
+    TileGeom tg;
+    int C, K;
+    const uint32_t *lists;  // compiled clauses of this layer's bank
+    int stride;
+    const int32_t *wt;      // clause-major weights (last layer)
+    int tile0, first_graph, n_graphs;
+    int32_t *class_sum;     // [n_graphs][K] (last layer)
+    uint32_t *bitmap;       // [tiles of the launch][C][tw]: clause truth per node slot, read and written in place
+    // message layers
+    int M, MB, G;
+    const uint32_t *hv;     // [C][MB]
+    const uint32_t *node_index, *n_nodes, *n_edges, *edge_index, *edge;
+};
+
+// Rows a message layer keeps in LDS: M message rows, the all-ones row, the row of graphs without nodes.
+inline int tile_message_rows(int M) { return M + 2; }
+
+inline size_t tile_layer_lds_bytes(const TileGeom &g, int classes, int src, int M) {
+    return tile_lds_bytes(src == ROWS_STAGED ? g.rows : src == ROWS_MESSAGES ? tile_message_rows(M) : 0, g, classes);
+}
+
+// One layer of clause evaluation for one tile per workgroup.
+//
+// Layer 0 (ROWS_STAGED / ROWS_GLOBAL): a clause's truth over the tile's node
+// slots is the AND of the node-type row and the rows of its included literals
+// (kernels.py:443-466).  Message layers (ROWS_MESSAGES): first the workgroup
+// builds the layer's message rows in LDS - row p has the bit of node slot n set
+// iff some clause that is true at a neighbour s with an edge s -> n of type t
+// has (h + t) mod M == p for one of its hypervector bits h (kernels.py:565-588;
+// the negated message literal p + M is the complement of row p) - then a
+// clause's truth is its previous truth AND the rows of its included message
+// literals (kernels.py:505-527).
+//
+// A wave owns a clause at a time.  The clause's row list is wave-uniform: its
+// first 32 entries arrive by scalar loads issued while the previous clause is
+// being evaluated.  Lane L holds words [L*LW, (L+1)*LW) of the running AND; after
+// every 8 rows a clause that is false at every node slot of the tile is done.
+//
+// LAST: the clause's weights are added to the class sums of the graphs where it
+// is true at some node (kernels.py:297-315) and no bitmap is written; otherwise
+// the truth row goes to `bitmap`.
+template <int NWAVES, int LW, int SRC, bool LAST>
+__global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
     extern __shared__ uint32_t lds[];
-    const int tw = tg.tw;
+    const TileGeom &tg = a.tg;
+    const int tw = tg.tw, C = a.C, K = a.K;
+    constexpr int NT = NWAVES * 64;
+    const int n_rows_lds = SRC == ROWS_STAGED ? tg.rows : SRC == ROWS_MESSAGES ? a.M + 2 : 0;
     uint32_t *bt = lds;
-    int32_t *sums = (int32_t *)(lds + (size_t)tg.rows * tw + TILE_LDS_PAD_WORDS);
-    const int tile = tile0 + blockIdx.x;
+    int32_t *sums = (int32_t *)(lds + (size_t)n_rows_lds * tw + TILE_LDS_PAD_WORDS);
+    const int tile = a.tile0 + blockIdx.x;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    uint32_t *bitmap = a.bitmap + (int64_t)blockIdx.x * C * tw;  // this tile's truth rows
 
-    {  // tile -> LDS, 16 bytes per thread and trip, several loads in flight
-        const uint4 *src = reinterpret_cast<const uint4 *>(tiles + (int64_t)tile * tg.rows * tw);
+    if (SRC == ROWS_STAGED) {  // tile -> LDS, 16 bytes per thread and trip, several loads in flight
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.tiles + (int64_t)tile * tg.rows * tw);
         uint4 *dst = reinterpret_cast<uint4 *>(bt);
         const int n4 = (tg.rows * tw) >> 2;  // tw is a multiple of 4
-        for (int i = tid; i < n4; i += NWAVES * 64 * 4) {
+        for (int i = tid; i < n4; i += NT * 4) {
             uint4 v[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                int at = i + u * NWAVES * 64;
+                int at = i + u * NT;
                 v[u] = at < n4 ? src[at] : make_uint4(0, 0, 0, 0);
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                int at = i + u * NWAVES * 64;
+                int at = i + u * NT;
                 if (at < n4) dst[at] = v[u];
             }
         }
-        for (int i = tid; i < TILE_LDS_PAD_WORDS + tg.gpt * K; i += NWAVES * 64) bt[tg.rows * tw + i] = 0;
     }
+    if (SRC == ROWS_MESSAGES) {
+        // rows 0..M-1 empty, row M all ones over the graph slots (pads the lists), row M+1 empty
+        const int used = tg.slot_words == 0 ? tw : tg.gpt * tg.slot_words;
+        for (int i = tid; i < a.M * tw; i += NT) bt[i] = 0u;
+        for (int i = tid; i < tw; i += NT) {
+            bt[a.M * tw + i] = i < used ? 0xFFFFFFFFu : 0u;
+            bt[(a.M + 1) * tw + i] = 0u;
+        }
+    }
+    for (int i = tid; i < TILE_LDS_PAD_WORDS + tg.gpt * K; i += NT) bt[(size_t)n_rows_lds * tw + i] = 0;
     __syncthreads();
 
-    // Lanes past the row width read the words after the row (inside the
-    // allocation) so that they fall on banks no other lane of the access uses;
-    // their running AND starts at 0 and stays 0.
-    const bool active = lane * LW < tw;
-    const char *col = reinterpret_cast<const char *>(bt + lane * LW);
-
-    // lane p < gpt*K adds weight k = p % K to graph j = p / K of the tile
-    const int pairs = tg.gpt * K;
-    const int my_j = lane / K, my_k = lane - my_j * K;
-    const bool pair_lane = tg.slot_words > 0 && lane < pairs;
-    const int my_shift = (lane < tg.gpt ? lane : 0) * tg.lanes_per_graph;
-    const unsigned long long slot_lanes = tg.lanes_per_graph >= 64 ? ~0ull : (1ull << tg.lanes_per_graph) - 1ull;
-
-    auto any_bit = [](const LaneWords<LW> &a) {
-        uint32_t m = a.w[0];
-#pragma unroll
-        for (int u = 1; u < LW; ++u) m |= a.w[u];
-        return m != 0;
-    };
-    auto and_row = [&](LaneWords<LW> &acc, uint32_t byte_offset) {
-        LaneWords<LW> r;
-        r.load(col + byte_offset);
-#pragma unroll
-        for (int u = 0; u < LW; ++u) acc.w[u] &= r.w[u];
-    };
-
-    auto evaluate = [&](const Chunk32 &head, const uint32_t *list, const int32_t *weights_of_clause) {
-        const int my_weight = pair_lane ? weights_of_clause[my_k] : 0;  // needed only if the clause fires
-        const int nb = (int)head.v[0];
-        LaneWords<LW> acc;
-#pragma unroll
-        for (int u = 0; u < LW; ++u) acc.w[u] = active ? 0xFFFFFFFFu : 0u;
-#pragma unroll
-        for (int i = 1; i < 8; ++i) and_row(acc, head.v[i]);
-        // stop as soon as the clause is false at every node slot of the tile
-        if (nb > 1 && __ballot(any_bit(acc)) != 0) {
-            // entries past the first chunk, 16 at a time, requested one step before they are needed
-            const Chunk16 *tp = reinterpret_cast<const Chunk16 *>(list) + 2;
-            Chunk16 tail = *tp;
-#pragma unroll
-            for (int i = 8; i < 16; ++i) and_row(acc, head.v[i]);
-            if (nb > 2 && __ballot(any_bit(acc)) != 0) {
-#pragma unroll
-                for (int i = 16; i < 24; ++i) and_row(acc, head.v[i]);
-                if (nb > 3 && __ballot(any_bit(acc)) != 0) {
-#pragma unroll
-                    for (int i = 24; i < 32; ++i) and_row(acc, head.v[i]);
-                    for (int j = 4; j < nb && __ballot(any_bit(acc)) != 0; j += 2) {
-                        const Chunk16 ahead = *++tp;
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) and_row(acc, tail.v[i]);
-                        if (j + 1 < nb && __ballot(any_bit(acc)) != 0) {
-#pragma unroll
-                            for (int i = 8; i < 16; ++i) and_row(acc, tail.v[i]);
+    if (SRC == ROWS_MESSAGES) {
+        // Row M+1: slot bit 0 of the graphs without nodes.  The reference's chunk arithmetic leaves
+        // every clause true for such a graph at every layer (kernels.py:443-466,505-527 never
+        // enter their node loop); the tile carries that in slot bit 0, which message literals
+        // therefore must not clear.
+        for (int j = tid; j < tg.gpt; j += NT) {
+            const int64_t g = (int64_t)tile * tg.gpt + j;
+            if (g < a.G && a.n_nodes[g] == 0u) {
+                const int pos = j * tg.slot_bits;
+                atomicOr(&bt[(a.M + 1) * tw + (pos >> 5)], 1u << (pos & 31));
+            }
+        }
+        // every true (clause, node slot) marks its clause's rotated hypervector bits at the node's out-neighbours
+        for (int c = wave; c < C; c += NWAVES) {
+            const uint32_t *truth = bitmap + (int64_t)c * tw;
+            for (int w = lane; w < tw; w += 64) {
+                uint32_t word = truth[w];
+                while (word) {
+                    const int pos = (w << 5) + __ffs(word) - 1;
+                    word &= word - 1;
+                    const int j = pos / tg.slot_bits, n = pos - j * tg.slot_bits;
+                    const int64_t g = (int64_t)tile * tg.gpt + j;
+                    if (g >= a.G || (uint32_t)n >= a.n_nodes[g]) continue;
+                    const int64_t row = (int64_t)a.node_index[g] + n;
+                    const uint32_t ne = a.n_edges[row];
+                    const int64_t e0 = a.edge_index[row];
+                    for (uint32_t e = 0; e < ne; ++e) {
+                        const uint32_t dst = a.edge[(e0 + e) * 2], type = a.edge[(e0 + e) * 2 + 1];
+                        const int dpos = j * tg.slot_bits + (int)dst;
+                        for (int b = 0; b < a.MB; ++b) {
+                            const uint32_t p = (a.hv[(int64_t)c * a.MB + b] + type) % (uint32_t)a.M;
+                            atomicOr(&bt[p * tw + (dpos >> 5)], 1u << (dpos & 31));
                         }
-                        tail = ahead;
                     }
                 }
             }
         }
-        const unsigned long long nz = __ballot(any_bit(acc));
+        __syncthreads();
+    }
+
+    // Lanes past the row width: their running AND starts at 0 and stays 0.  In LDS they read the
+    // words after the row (inside the allocation) so that they fall on banks no other lane of
+    // the access uses; in global memory they read the row's first words.
+    const bool active = lane * LW < tw;
+    const char *col = SRC == ROWS_GLOBAL
+                          ? reinterpret_cast<const char *>(a.tiles + (int64_t)tile * tg.rows * tw + (active ? lane * LW : 0))
+                          : reinterpret_cast<const char *>(bt + lane * LW);
+
+    // lane p < gpt*K adds weight k = p % K to graph j = p / K of the tile
+    const int pairs = tg.gpt * K;
+    const int my_j = lane / K, my_k = lane - my_j * K;
+    const bool pair_lane = LAST && tg.slot_words > 0 && lane < pairs;
+    const int my_shift = (lane < tg.gpt ? lane : 0) * tg.lanes_per_graph;
+    const unsigned long long slot_lanes = tg.lanes_per_graph >= 64 ? ~0ull : (1ull << tg.lanes_per_graph) - 1ull;
+
+    auto any_bit = [](const LaneWords<LW> &x) {
+        uint32_t m = x.w[0];
+#pragma unroll
+        for (int u = 1; u < LW; ++u) m |= x.w[u];
+        return m != 0;
+    };
+    auto and_row = [&](LaneWords<LW> &acc, uint32_t entry) {
+        LaneWords<LW> r;
+        if (SRC == ROWS_MESSAGES) {
+            r.load(col + (entry & ~TILE_NEGATED));
+            const uint32_t flip = (uint32_t)((int32_t)entry >> 31);  // all ones for a negated literal
+#pragma unroll
+            for (int u = 0; u < LW; ++u) acc.w[u] &= r.w[u] ^ flip;
+        } else {
+            r.load(col + entry);
+#pragma unroll
+            for (int u = 0; u < LW; ++u) acc.w[u] &= r.w[u];
+        }
+    };
+
+    // slot bit 0 of the graphs without nodes (message layers)
+    LaneWords<LW> empties;
+#pragma unroll
+    for (int u = 0; u < LW; ++u) empties.w[u] = 0u;
+    bool any_empty = false;
+    if (SRC == ROWS_MESSAGES) {
+        if (active) empties.load(col + (size_t)(a.M + 1) * tw * 4);
+        any_empty = __ballot(any_bit(empties)) != 0;
+    }
+
+    // `truth_in` is the clause's truth from the previous layer (message layers only)
+    auto evaluate = [&](const Chunk32 &head, const uint32_t *list, const int32_t *weights_of_clause,
+                        const LaneWords<LW> &truth_in, char *truth_out) {
+        const int my_weight = pair_lane ? weights_of_clause[my_k] : 0;  // needed only if the clause fires
+        const int nb = (int)head.v[0];
+        LaneWords<LW> acc;
+        bool alive = true;
+        if (SRC == ROWS_MESSAGES) {
+            acc = truth_in;
+            alive = __ballot(any_bit(acc)) != 0;
+        } else {
+#pragma unroll
+            for (int u = 0; u < LW; ++u) acc.w[u] = active ? 0xFFFFFFFFu : 0u;
+        }
+        if (alive) {
+#pragma unroll
+            for (int i = 1; i < 8; ++i) and_row(acc, head.v[i]);
+            // stop as soon as the clause is false at every node slot of the tile
+            if (nb > 1 && __ballot(any_bit(acc)) != 0) {
+                // entries past the first chunk, 16 at a time, requested one step before they are needed
+                const Chunk16 *tp = reinterpret_cast<const Chunk16 *>(list) + 2;
+                Chunk16 tail = *tp;
+#pragma unroll
+                for (int i = 8; i < 16; ++i) and_row(acc, head.v[i]);
+                if (nb > 2 && __ballot(any_bit(acc)) != 0) {
+#pragma unroll
+                    for (int i = 16; i < 24; ++i) and_row(acc, head.v[i]);
+                    if (nb > 3 && __ballot(any_bit(acc)) != 0) {
+#pragma unroll
+                        for (int i = 24; i < 32; ++i) and_row(acc, head.v[i]);
+                        for (int j = 4; j < nb && __ballot(any_bit(acc)) != 0; j += 2) {
+                            const Chunk16 ahead = *++tp;
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) and_row(acc, tail.v[i]);
+                            if (j + 1 < nb && __ballot(any_bit(acc)) != 0) {
+#pragma unroll
+                                for (int i = 8; i < 16; ++i) and_row(acc, tail.v[i]);
+                            }
+                            tail = ahead;
+                        }
+                    }
+                }
+            }
+        }
+        if (SRC == ROWS_MESSAGES && any_empty) {
+#pragma unroll
+            for (int u = 0; u < LW; ++u) acc.w[u] |= truth_in.w[u] & empties.w[u];
+        }
+        if (!LAST) {
+            if (active && (SRC != ROWS_MESSAGES || alive)) acc.store(truth_out);  // a dead row is already all zero in place
+            return;
+        }
+        const unsigned long long nz = alive ? __ballot(any_bit(acc)) : 0ull;
         if (nz == 0) return;
         if (tg.slot_words > 0) {
             // graph j owns lanes [j*lanes_per_graph, (j+1)*lanes_per_graph)
@@ -353,32 +528,43 @@ __global__ __launch_bounds__(NWAVES * 64) void k_score_tiles(
         }
     };
 
-    // Two clauses per trip so that the chunk fetched ahead never has to be
-    // copied.  Pointers step by NWAVES clauses; past the end they stay on the
-    // wave's last clause (a valid address whose data is not used).
-    const int64_t list_step = (int64_t)NWAVES * stride;
+    // Two clauses per trip so that the chunk fetched ahead never has to be copied.  Pointers step
+    // by NWAVES clauses; past the end they stay on the wave's last clause (a valid address whose
+    // data is not used).
+    const int64_t list_step = (int64_t)NWAVES * a.stride;
     const int wt_step = NWAVES * K;
+    const int64_t truth_step = (int64_t)NWAVES * tw * 4;
     const int first = wave < C ? wave : 0;
-    const uint32_t *list_a = lists + (int64_t)first * stride;
-    const int32_t *wt_a = wt + (int64_t)first * K;
-    Chunk32 a = *reinterpret_cast<const Chunk32 *>(list_a);
+    const uint32_t *list_a = a.lists + (int64_t)first * a.stride;
+    const int32_t *wt_a = LAST ? a.wt + (int64_t)first * K : nullptr;
+    char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
+    Chunk32 ca = *reinterpret_cast<const Chunk32 *>(list_a);
+    LaneWords<LW> ta, tb;
+#pragma unroll
+    for (int u = 0; u < LW; ++u) ta.w[u] = tb.w[u] = 0u;
+    if (SRC == ROWS_MESSAGES && active) ta.load(truth_a);
     for (int c = wave; c < C; c += 2 * NWAVES) {
         const bool has_b = c + NWAVES < C;
         const uint32_t *list_b = has_b ? list_a + list_step : list_a;
-        const int32_t *wt_b = has_b ? wt_a + wt_step : wt_a;
-        const Chunk32 b = *reinterpret_cast<const Chunk32 *>(list_b);
-        evaluate(a, list_a, wt_a);
+        const int32_t *wt_b = LAST ? (has_b ? wt_a + wt_step : wt_a) : nullptr;
+        char *truth_b = has_b ? truth_a + truth_step : truth_a;
+        const Chunk32 cb = *reinterpret_cast<const Chunk32 *>(list_b);
+        if (SRC == ROWS_MESSAGES && active) tb.load(truth_b);
+        evaluate(ca, list_a, wt_a, ta, truth_a);
         const bool has_a = c + 2 * NWAVES < C;
         list_a = has_a ? list_b + list_step : list_b;
-        wt_a = has_a ? wt_b + wt_step : wt_b;
-        a = *reinterpret_cast<const Chunk32 *>(list_a);
-        if (has_b) evaluate(b, list_b, wt_b);
+        if (LAST) wt_a = has_a ? wt_b + wt_step : wt_b;
+        truth_a = has_a ? truth_b + truth_step : truth_b;
+        ca = *reinterpret_cast<const Chunk32 *>(list_a);
+        if (SRC == ROWS_MESSAGES && active) ta.load(truth_a);
+        if (has_b) evaluate(cb, list_b, wt_b, tb, truth_b);
     }
+    if (!LAST) return;
     __syncthreads();
     const int64_t g0 = (int64_t)tile * tg.gpt;
-    for (int i = tid; i < tg.gpt * K; i += NWAVES * 64) {
+    for (int i = tid; i < tg.gpt * K; i += NT) {
         int64_t g = g0 + i / K;
-        if (g >= first_graph && g < (int64_t)first_graph + n_graphs)
-            class_sum[(g - first_graph) * K + (i % K)] = sums[i];
+        if (g >= a.first_graph && g < (int64_t)a.first_graph + a.n_graphs)
+            a.class_sum[(g - a.first_graph) * K + (i % K)] = sums[i];
     }
 }

@@ -79,7 +79,8 @@ class _DeviceGraphs:
 
     def ensure_tiles(self, cfg):
         """Build the literal-major tile layout once per data set (used by
-        depth-1 inference); shapes without such a layout keep tiles = NULL."""
+        inference and depth-1 training); shapes without such a layout keep
+        tiles = NULL."""
         if self._tiles_tried:
             return
         self._tiles_tried = True
@@ -291,11 +292,13 @@ class CommonTsetlinMachine:
         dg = self._score_init(graphs)
         cfg = self._config(max(dg.max_nodes, 1))
         n = dg.number_of_graphs
-        if self.depth == 1:
-            dg.ensure_tiles(cfg)
+        dg.ensure_tiles(cfg)
         if batch is None:
-            per_graph = max(1, _abi.lib.gtm_score_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc), 1))
-            batch = int(max(1, min(n, (1 << 30) // per_graph, 1 << 16)))
+            # as many graphs per launch group as fit in 4 GiB of workspace beyond its fixed part
+            size = lambda b: _abi.lib.gtm_score_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc), b)
+            fixed = size(1)
+            per_graph = max(1.0, (size(1025) - fixed) / 1024.0)
+            batch = int(max(1, min(n, ((4 << 30) - fixed) // per_graph, 1 << 16)))
         need = _abi.lib.gtm_score_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc), batch)
         ws = self._workspace_of(need)
         out = torch.empty(n * self.number_of_outputs, dtype=torch.int32, device=_device())

@@ -254,6 +254,52 @@ def test_tile_scoring_equals_oracle(shape, density):
         assert np.array_equal(dev.score(3, G - 5, G), plain[3:G - 2])
 
 
+DEEP_TILE_SHAPES = [
+    # several graphs per word; one word per graph; several words; 361-node graphs; literal rows too
+    # big for LDS (read in place); graphs without nodes; single-node graphs with self-loops
+    dict(seed=31, g=dict(n_graphs=120, max_nodes=3, hv_size=16, node_types=("a", "b"), edge_types=("x", "y", "z")),
+         m=dict(classes=2, clauses=33, depth=2, message_size=37)),
+    dict(seed=32, g=dict(n_graphs=60, max_nodes=16, min_nodes=9, hv_size=20),
+         m=dict(classes=4, clauses=100, depth=3, message_size=64, message_bits=3)),
+    dict(seed=33, g=dict(n_graphs=30, max_nodes=70, hv_size=16, edge_types=("x", "y")),
+         m=dict(classes=3, clauses=70, depth=2, message_size=37)),
+    dict(seed=34, g=dict(n_graphs=12, max_nodes=361, min_nodes=300, hv_size=128, edge_types=("l", "r", "u", "d")),
+         m=dict(classes=10, clauses=80, depth=2, message_size=256)),
+    dict(seed=35, g=dict(n_graphs=5, sizes=[3, 520, 40, 1, 200], hv_size=1500, n_symbols=30),
+         m=dict(classes=2, clauses=60, depth=2, message_size=32), density=0.0007),
+    dict(seed=36, g=dict(n_graphs=6, hv_size=16, sizes=[5, 0, 33, 1, 0, 40]),
+         m=dict(classes=3, clauses=20, depth=3, message_size=16, message_bits=1)),
+    dict(seed=37, g=dict(n_graphs=200, max_nodes=1, hv_size=40), m=dict(classes=3, clauses=50, depth=2, message_size=8)),
+]
+
+
+@pytest.mark.parametrize("shape", DEEP_TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
+@pytest.mark.parametrize("message_density", [0.0, 0.01, 0.1])
+def test_tile_scoring_with_message_layers(shape, message_density):
+    """gtm_score with message layers on literal-major tiles == oracle == the bitmap path."""
+    from tests.gpu_harness import Device
+
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    m = dict(shape["m"])
+    depth = m.pop("depth")
+    cfg = helpers.oracle_config(graphs, **m, depth=depth)
+    model = helpers.random_model(shape["seed"], cfg, depth, include_density=shape.get("density", 0.02),
+                                 message_density=message_density)
+    model.ta_state[3, :, cfg.state_bits - 1] = 0  # an empty clause among the random ones
+    dev = Device(model, graphs)
+    G = graphs.number_of_graphs
+    plain = dev.score(0, G, G)
+    assert dev.build_tiles(), "this shape should have a tile layout"
+    tiled = dev.score(0, G, G)
+    assert np.array_equal(tiled, plain)
+    sample = sorted(set(e for e in (0, 1, 2, 3, 4, G // 2, G - 1) if e < G))
+    assert np.array_equal(tiled[sample], o.score(model, graphs, sample))
+    # several launch groups; a range that starts and ends inside tiles
+    assert np.array_equal(dev.score(0, G, 3), plain)
+    if G > 7:
+        assert np.array_equal(dev.score(3, G - 5, 5), plain[3:G - 2])
+
+
 @pytest.mark.parametrize("shape", TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
 @pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 6, 5)])
 @pytest.mark.parametrize("persistent", [True, False], ids=["one-launch", "two-per-graph"])
