@@ -675,15 +675,70 @@ int launch_tile_layer(const TileLayerArgs &a, int n_tiles, int src, bool last, h
     }
 }
 
+template <int NW, int LW, int LA4, bool LAST>
+int launch_two_phase_as(const TileLayerArgs &a, int n_tiles, hipStream_t st) {
+    size_t lds = tile_layer_lds_bytes(a.tg, a.K, ROWS_STAGED, a.M);
+    static thread_local size_t lds_set = 0;
+    if (lds > lds_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)k_tile_two_phase<NW, LW, LA4, LAST>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
+        lds_set = lds;
+    }
+    if (LAST) profile_start("k_tile_two_phase<score>", st);
+    hipLaunchKernelGGL((k_tile_two_phase<NW, LW, LA4, LAST>), dim3(n_tiles), dim3(NW * 64), lds, st, a);
+    if (int rc = check_launch("tile_two_phase")) return rc;
+    if (LAST) profile_stop(st);
+    return GTM_OK;
+}
+
+template <int NW, int LW>
+int launch_two_phase_lw(const TileLayerArgs &a, int n_tiles, int la4, bool last, hipStream_t st) {
+#define GTM_TWO_PHASE(N)                                                         \
+    case N:                                                                      \
+        return last ? launch_two_phase_as<NW, LW, N, true>(a, n_tiles, st)       \
+                    : launch_two_phase_as<NW, LW, N, false>(a, n_tiles, st)
+    switch (la4) {
+        GTM_TWO_PHASE(1);
+        GTM_TWO_PHASE(2);
+        GTM_TWO_PHASE(3);
+        default: GTM_TWO_PHASE(4);
+    }
+#undef GTM_TWO_PHASE
+}
+
+int launch_two_phase(const TileLayerArgs &a, int n_tiles, int la4, bool last, hipStream_t st) {
+    constexpr int NW = 16;
+    switch (a.tg.lw) {
+        case 1: return launch_two_phase_lw<NW, 1>(a, n_tiles, la4, last, st);
+        case 2: return launch_two_phase_lw<NW, 2>(a, n_tiles, la4, last, st);
+        default: return launch_two_phase_lw<NW, 4>(a, n_tiles, la4, last, st);
+    }
+}
+
+// Layer 0 can run in two phases (k_tile_two_phase) on tiles of whole-word graph slots staged in
+// LDS when a node has 4, 8, 12 or 16 literal words.
+bool two_phase_layer0(const Dims &d, const TileGeom &tg) {
+    return tg.slot_words > 0 && tg.stage0 && d.LA % 4 == 0 && d.LA <= 16 && !getenv("GTM_NO_TWO_PHASE");
+}
+
 // `_score`'s loop (tm.py:786-812) on tiles: per launch group of tiles, layer 0 and then one
 // launch per message layer; the clause truth rows between layers stay in w.tile_bitmap.
 int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
                    const ScoreWs &w, int first, int n_graphs, int batch, int32_t *class_sum, hipStream_t st) {
     const uint32_t *order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
     const int layers = cfg->depth;
-    hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C, d.LA,
-                       d.B, d.filter, cfg->literals, 0, g->number_of_node_types, cfg->literals, tg.rows - 1, tg.tw,
-                       w.list_stride, order, w.lists, d.K, layers == 1 ? s->clause_weights : nullptr, w.wt);
+    const bool two_phase = two_phase_layer0(d, tg);
+    const int stride0 = two_phase ? 8 + d.LA : w.list_stride;
+    if (two_phase)
+        hipLaunchKernelGGL(k_compile_clauses_two_phase, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state,
+                           d.C, d.LA, d.B, d.filter, cfg->literals, g->number_of_node_types, cfg->literals,
+                           tg.rows - 1, tg.tw, order, w.lists, stride0, d.K,
+                           layers == 1 ? s->clause_weights : nullptr, w.wt);
+    else
+        hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C,
+                           d.LA, d.B, d.filter, cfg->literals, 0, g->number_of_node_types, cfg->literals, tg.rows - 1,
+                           tg.tw, w.list_stride, order, w.lists, d.K, layers == 1 ? s->clause_weights : nullptr, w.wt);
     if (int rc = check_launch("compile_clauses")) return rc;
     for (int l = 1; l < layers; ++l) {
         hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st,
@@ -709,16 +764,21 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     a.n_edges = g->number_of_graph_node_edges;
     a.edge_index = g->edge_index;
     a.edge = g->edge;
+    a.X = g->X;
+    auto layer0 = [&](int n_tiles, bool last) {
+        a.lists = w.lists;
+        a.stride = stride0;
+        return two_phase ? launch_two_phase(a, n_tiles, d.LA / 4, last, st)
+                         : launch_tile_layer(a, n_tiles, tg.stage0 ? ROWS_STAGED : ROWS_GLOBAL, last, st);
+    };
     if (layers == 1) {
         // no truth rows are kept: every tile of the range in one launch
-        a.lists = w.lists;
-        a.stride = w.list_stride;
         a.tile0 = first / tg.gpt;
         a.first_graph = first;
         a.n_graphs = n_graphs;
         a.class_sum = class_sum;
         int n_tiles = (first + n_graphs - 1) / tg.gpt - a.tile0 + 1;
-        return launch_tile_layer(a, n_tiles, tg.stage0 ? ROWS_STAGED : ROWS_GLOBAL, true, st);
+        return layer0(n_tiles, true);
     }
     if (g->total_edges > 0 && (!g->number_of_graph_node_edges || !g->edge || !g->edge_index))
         return fail(GTM_ERR_INVALID, "graphs with edges need number_of_graph_node_edges, edge and edge_index");
@@ -730,9 +790,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         a.first_graph = first;
         a.n_graphs = n_graphs;
         a.class_sum = class_sum;
-        a.lists = w.lists;
-        a.stride = w.list_stride;
-        if (int rc = launch_tile_layer(a, n_tiles, tg.stage0 ? ROWS_STAGED : ROWS_GLOBAL, false, st)) return rc;
+        if (int rc = layer0(n_tiles, false)) return rc;
         for (int l = 1; l < layers; ++l) {
             a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
             a.stride = w.message_list_stride;

@@ -290,6 +290,7 @@ struct TileLayerArgs {
     int M, MB, G;
     const uint32_t *hv;     // [C][MB]
     const uint32_t *node_index, *n_nodes, *n_edges, *edge_index, *edge;
+    const uint32_t *X;      // [nodes][LA] node-major literal words (two-phase layer 0)
 };
 
 // Rows a message layer keeps in LDS: M message rows, the all-ones row, the row of graphs without nodes.
@@ -558,6 +559,220 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
         ca = *reinterpret_cast<const Chunk32 *>(list_a);
         if (SRC == ROWS_MESSAGES && active) ta.load(truth_a);
         if (has_b) evaluate(cb, list_b, wt_b, tb, truth_b);
+    }
+    if (!LAST) return;
+    __syncthreads();
+    const int64_t g0 = (int64_t)tile * tg.gpt;
+    for (int i = tid; i < tg.gpt * K; i += NT) {
+        int64_t g = g0 + i / K;
+        if (g >= a.first_graph && g < (int64_t)a.first_graph + a.n_graphs)
+            a.class_sum[(g - a.first_graph) * K + (i % K)] = sums[i];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Layer 0 in two phases, for tiles of whole-word graph slots whose nodes have
+// few literal words (LA a multiple of 4, at most 16).
+//
+// Phase 1 ANDs the node-type row and the rows of the clause's 14 rarest
+// included literals, which leaves very few candidate node slots; phase 2 tests
+// each candidate against the clause's whole include mask on the node's own
+// literal words (X, node-major, as kernels.py:443-466 reads it):
+// the clause is true at the node iff (include & ~X[node]) == 0.  The result is
+// the same truth row as ANDing every included literal's row.
+//
+// Compiled clause: 16 entries of 16 bits - entry 0 = rows in use (type row +
+// literals, at most 15) | needs-phase-2 << 8; entries 1..15 = row offsets in
+// units of 16 bytes, unused ones pointing at the all-ones row - followed by the
+// LA words of the include mask.
+
+struct alignas(32) Packed8 {
+    uint32_t v[8];
+};
+template <int N>
+struct alignas(16) Words {
+    uint32_t v[N];
+};
+
+__global__ void k_compile_clauses_two_phase(const uint32_t *__restrict__ bank, int C, int chunks, int B,
+                                            uint32_t filter, int literals, int n_types, int type_base_row,
+                                            int ones_row, int tw, const uint32_t *__restrict__ order,
+                                            uint32_t *__restrict__ records, int record_words, int K,
+                                            const int32_t *__restrict__ weights, int32_t *__restrict__ wt) {
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (c >= C) return;
+    const uint32_t row16 = (uint32_t)tw >> 2;  // a row in units of 16 bytes (tw is a multiple of 4)
+    uint32_t *rec = records + (int64_t)c * record_words;
+    uint16_t *e = reinterpret_cast<uint16_t *>(rec);
+    const uint32_t *inc = bank + (int64_t)c * chunks * B + (B - 1);
+    if (lane == 0) e[1] = (uint16_t)((uint32_t)(type_base_row + c % n_types) * row16);
+    int n = 2;
+    for (int r0 = 0; r0 < literals; r0 += 64) {
+        int r = r0 + lane;
+        uint32_t lit = r < literals ? (order ? order[r] : (uint32_t)r) : 0u;
+        uint32_t w = lit >> 5;
+        uint32_t word = inc[(int64_t)w * B];
+        if ((int)w == chunks - 1) word &= filter;
+        bool included = r < literals && ((word >> (lit & 31)) & 1u);
+        unsigned long long mask = __ballot(included);
+        int at = n + __popcll(mask & ((1ull << lane) - 1ull));
+        if (included && at < 16) e[at] = (uint16_t)(lit * row16);
+        n += __popcll(mask);
+    }
+    for (int i = n + lane; i < 16; i += 64) e[i] = (uint16_t)((uint32_t)ones_row * row16);
+    if (lane == 0) e[0] = (uint16_t)((n > 16 ? 15 : n - 1) | (n > 16 ? 0x100 : 0));
+    for (int w = lane; w < chunks; w += 64) {
+        uint32_t word = inc[(int64_t)w * B];
+        if (w == chunks - 1) word &= filter;
+        rec[8 + w] = word;
+    }
+    if (weights)
+        for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
+}
+
+template <int NWAVES, int LW, int LA4, bool LAST>
+__global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a) {
+    extern __shared__ uint32_t lds[];
+    const TileGeom &tg = a.tg;
+    const int tw = tg.tw, C = a.C, K = a.K;
+    constexpr int NT = NWAVES * 64;
+    uint32_t *bt = lds;
+    int32_t *sums = (int32_t *)(lds + (size_t)tg.rows * tw + TILE_LDS_PAD_WORDS);
+    const int tile = a.tile0 + blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    uint32_t *bitmap = a.bitmap + (int64_t)blockIdx.x * C * tw;
+
+    {  // tile -> LDS
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.tiles + (int64_t)tile * tg.rows * tw);
+        uint4 *dst = reinterpret_cast<uint4 *>(bt);
+        const int n4 = (tg.rows * tw) >> 2;
+        for (int i = tid; i < n4; i += NT * 4) {
+            uint4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int at = i + u * NT;
+                v[u] = at < n4 ? src[at] : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int at = i + u * NT;
+                if (at < n4) dst[at] = v[u];
+            }
+        }
+        for (int i = tid; i < TILE_LDS_PAD_WORDS + tg.gpt * K; i += NT) bt[(size_t)tg.rows * tw + i] = 0;
+    }
+    __syncthreads();
+
+    const bool active = lane * LW < tw;
+    const char *col = reinterpret_cast<const char *>(bt + lane * LW);
+
+    // the graph whose slot this lane's words belong to, and the node of the lane's first bit
+    const int lpg = tg.lanes_per_graph;
+    const int lane_j = lane / lpg;
+    const int64_t lane_g = (int64_t)tile * tg.gpt + lane_j;
+    const bool has_graph = active && lane_j < tg.gpt && lane_g < a.G;
+    // a graph without nodes keeps its slot bit 0 (every clause is true for it) and has no node to test
+    const bool testable = has_graph && a.n_nodes[lane_g] != 0u;
+    const int64_t lane_node0 = has_graph ? (int64_t)a.node_index[lane_g] + (lane - lane_j * lpg) * (LW * 32) : 0;
+    const uint4 *x_lane = reinterpret_cast<const uint4 *>(a.X) + lane_node0 * LA4;
+
+    const int pairs = tg.gpt * K;
+    const int my_j = lane / K, my_k = lane - my_j * K;
+    const bool pair_lane = LAST && lane < pairs;
+    const int my_shift = (lane < tg.gpt ? lane : 0) * lpg;
+    const unsigned long long slot_lanes = lpg >= 64 ? ~0ull : (1ull << lpg) - 1ull;
+
+    auto any_bit = [](const LaneWords<LW> &x) {
+        uint32_t m = x.w[0];
+#pragma unroll
+        for (int u = 1; u < LW; ++u) m |= x.w[u];
+        return m != 0;
+    };
+    auto entry_of = [](const Packed8 &rec, int i) { return ((rec.v[i >> 1] >> ((i & 1) * 16)) & 0xFFFFu) << 4; };
+    auto and_row = [&](LaneWords<LW> &acc, uint32_t byte_offset) {
+        LaneWords<LW> r;
+        r.load(col + byte_offset);
+#pragma unroll
+        for (int u = 0; u < LW; ++u) acc.w[u] &= r.w[u];
+    };
+
+    auto evaluate = [&](const Packed8 &rec, const Words<4 * LA4> &include, const int32_t *weights_of_clause,
+                        char *truth_out) {
+        const int my_weight = pair_lane ? weights_of_clause[my_k] : 0;
+        const uint32_t header = rec.v[0] & 0xFFFFu;
+        LaneWords<LW> acc;
+#pragma unroll
+        for (int u = 0; u < LW; ++u) acc.w[u] = active ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+        for (int i = 1; i < 8; ++i) and_row(acc, entry_of(rec, i));
+        unsigned long long nz = __ballot(any_bit(acc));
+        if ((header & 0xFFu) > 7u && nz != 0) {
+#pragma unroll
+            for (int i = 8; i < 16; ++i) and_row(acc, entry_of(rec, i));
+            nz = __ballot(any_bit(acc));
+            if ((header & 0x100u) && nz != 0) {
+                // phase 2: every surviving node slot against the whole include mask
+#pragma unroll
+                for (int u = 0; u < LW; ++u) {
+                    uint32_t todo = testable ? acc.w[u] : 0u;
+                    while (todo) {
+                        const int b = __ffs(todo) - 1;
+                        todo &= todo - 1;
+                        const uint4 *x = x_lane + (u * 32 + b) * LA4;
+                        uint32_t violated = 0;
+#pragma unroll
+                        for (int q = 0; q < LA4; ++q) {
+                            const uint4 v = x[q];
+                            violated |= (include.v[4 * q] & ~v.x) | (include.v[4 * q + 1] & ~v.y) |
+                                        (include.v[4 * q + 2] & ~v.z) | (include.v[4 * q + 3] & ~v.w);
+                        }
+                        if (violated) acc.w[u] &= ~(1u << b);
+                    }
+                }
+                nz = __ballot(any_bit(acc));
+            }
+        }
+        if (!LAST) {
+            if (active) acc.store(truth_out);
+            return;
+        }
+        if (nz == 0) return;
+        // graph j owns lanes [j*lanes_per_graph, (j+1)*lanes_per_graph)
+        const unsigned long long gm = __ballot(lane < tg.gpt && ((nz >> my_shift) & slot_lanes) != 0);
+        if (pair_lane && ((gm >> my_j) & 1ull)) atomicAdd(&sums[lane], my_weight);
+        for (int p = lane + 64; p < pairs; p += 64) {
+            int j = p / K, k = p - j * K;
+            if ((gm >> j) & 1ull) atomicAdd(&sums[p], weights_of_clause[k]);
+        }
+    };
+
+    const int64_t rec_step = (int64_t)NWAVES * a.stride;
+    const int wt_step = NWAVES * K;
+    const int64_t truth_step = (int64_t)NWAVES * tw * 4;
+    const int first = wave < C ? wave : 0;
+    const uint32_t *rec_a = a.lists + (int64_t)first * a.stride;
+    const int32_t *wt_a = LAST ? a.wt + (int64_t)first * K : nullptr;
+    char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
+    Packed8 ra = *reinterpret_cast<const Packed8 *>(rec_a);
+    Words<4 * LA4> ma = *reinterpret_cast<const Words<4 * LA4> *>(rec_a + 8);
+    for (int c = wave; c < C; c += 2 * NWAVES) {
+        const bool has_b = c + NWAVES < C;
+        const uint32_t *rec_b = has_b ? rec_a + rec_step : rec_a;
+        const int32_t *wt_b = LAST ? (has_b ? wt_a + wt_step : wt_a) : nullptr;
+        char *truth_b = has_b ? truth_a + truth_step : truth_a;
+        const Packed8 rb = *reinterpret_cast<const Packed8 *>(rec_b);
+        const Words<4 * LA4> mb = *reinterpret_cast<const Words<4 * LA4> *>(rec_b + 8);
+        evaluate(ra, ma, wt_a, truth_a);
+        const bool has_a = c + 2 * NWAVES < C;
+        rec_a = has_a ? rec_b + rec_step : rec_b;
+        if (LAST) wt_a = has_a ? wt_b + wt_step : wt_b;
+        truth_a = has_a ? truth_b + truth_step : truth_b;
+        ra = *reinterpret_cast<const Packed8 *>(rec_a);
+        ma = *reinterpret_cast<const Words<4 * LA4> *>(rec_a + 8);
+        if (has_b) evaluate(rb, mb, wt_b, truth_b);
     }
     if (!LAST) return;
     __syncthreads();

@@ -227,6 +227,10 @@ TILE_SHAPES = [
     dict(seed=15, g=dict(n_graphs=23, max_nodes=361, min_nodes=300, hv_size=128, max_degree=0), classes=10, clauses=120),
     dict(seed=16, g=dict(n_graphs=5, max_nodes=2048, min_nodes=1990, hv_size=16, max_degree=0, node_types=("a", "b", "c")),
          classes=2, clauses=40),
+    # 12 and 16 literal words per node (layer 0 in two phases)
+    dict(seed=17, g=dict(n_graphs=30, max_nodes=100, min_nodes=20, hv_size=192, n_symbols=12), classes=3, clauses=90),
+    dict(seed=18, g=dict(n_graphs=20, max_nodes=50, hv_size=256, n_symbols=12, node_types=("a", "b")), classes=4,
+         clauses=64),
 ]
 
 
@@ -347,14 +351,15 @@ def test_fused_fit_with_an_empty_graph():
     assert np.array_equal(w, model.clause_weights) and np.array_equal(ta, model.ta_state)
 
 
-def test_empty_graphs_score_like_the_reference_arithmetic():
+@pytest.mark.parametrize("hv_size,density", [(16, 0.05), (64, 0.05), (64, 0.3)])
+def test_empty_graphs_score_like_the_reference_arithmetic(hv_size, density):
     """A graph without nodes: the reference's chunk arithmetic (C division,
     kernels.py:289-295) leaves every clause true, so it scores sum_c W[k][c]."""
     from tests.gpu_harness import Device
 
-    g = helpers.random_graphs(17, n_graphs=6, hv_size=16, sizes=[5, 0, 33, 1, 0, 40])
+    g = helpers.random_graphs(17, n_graphs=6, hv_size=hv_size, sizes=[5, 0, 33, 1, 0, 40])
     cfg = helpers.oracle_config(g, classes=3, clauses=20)
-    model = helpers.random_model(5, cfg, 1, include_density=0.05)
+    model = helpers.random_model(5, cfg, 1, include_density=density)
     want = o.score(model, g)
     assert np.array_equal(want[1], model.clause_weights.sum(axis=1)) and np.array_equal(want[4], want[1])
     dev = Device(model, g)
