@@ -631,6 +631,10 @@ __global__ void k_compile_clauses_two_phase(const uint32_t *__restrict__ bank, i
         for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
 }
 
+// The two phases of a clause are software-pipelined: a wave issues the phase-2 loads of one clause
+// (each lane the literal words of its first surviving node slot), runs phase 1 of its next clause
+// while they are in flight, and only then finishes the first.  Lanes with more than one surviving
+// slot test the others in a loop afterwards (rare once 14 literals have been applied).
 template <int NWAVES, int LW, int LA4, bool LAST>
 __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a) {
     extern __shared__ uint32_t lds[];
@@ -679,9 +683,12 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
     const int64_t lane_node0 = has_graph ? (int64_t)a.node_index[lane_g] + (lane - lane_j * lpg) * (LW * 32) : 0;
     const uint4 *x_lane = reinterpret_cast<const uint4 *>(a.X) + lane_node0 * LA4;
 
+    // lane p adds weight k = p % K to graph j = p / K of the tile, for p = lane and p = lane + 64
     const int pairs = tg.gpt * K;
-    const int my_j = lane / K, my_k = lane - my_j * K;
-    const bool pair_lane = LAST && lane < pairs;
+    const int j0 = lane / K, k0 = lane - j0 * K;
+    const int j1 = (lane + 64) / K, k1 = lane + 64 - j1 * K;
+    const bool pair0 = LAST && lane < pairs, pair1 = LAST && lane + 64 < pairs;
+    const int k0c = pair0 ? k0 : 0, k1c = pair1 ? k1 : 0;
     const int my_shift = (lane < tg.gpt ? lane : 0) * lpg;
     const unsigned long long slot_lanes = lpg >= 64 ? ~0ull : (1ull << lpg) - 1ull;
 
@@ -698,57 +705,106 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
 #pragma unroll
         for (int u = 0; u < LW; ++u) acc.w[u] &= r.w[u];
     };
+    auto violates = [](const Words<4 * LA4> &include, const uint4 *x) {
+        uint32_t violated = 0;
+#pragma unroll
+        for (int q = 0; q < LA4; ++q) {
+            const uint4 v = x[q];
+            violated |= (include.v[4 * q] & ~v.x) | (include.v[4 * q + 1] & ~v.y) | (include.v[4 * q + 2] & ~v.z) |
+                        (include.v[4 * q + 3] & ~v.w);
+        }
+        return violated != 0;
+    };
 
-    auto evaluate = [&](const Packed8 &rec, const Words<4 * LA4> &include, const int32_t *weights_of_clause,
-                        char *truth_out) {
-        const int my_weight = pair_lane ? weights_of_clause[my_k] : 0;
+    struct Pending {
+        LaneWords<LW> acc;
+        uint4 x[LA4];
+        int bit;                 // the node slot this lane has under test (index into its LW words), -1 if none
+        bool live, test;         // wave-uniform: a clause is pending / its phase 2 runs
+        unsigned long long nz;   // lanes with a surviving slot after phase 1
+        int weight0, weight1;
+        const int32_t *weights;
+        char *truth_out;
+    };
+
+    // Phase 1 and the loads of phase 2.
+    auto begin = [&](Pending &p, const Packed8 &rec, const int32_t *weights_of_clause, char *truth_out) {
+        p.live = true;
+        p.weights = weights_of_clause;
+        p.truth_out = truth_out;
+        // every load below is issued by all lanes whatever the clause does, so that the number of
+        // loads in flight is known when the pending clause is finished
+        p.weight0 = LAST ? weights_of_clause[k0c] : 0;  // needed only if the clause fires
+        p.weight1 = LAST ? weights_of_clause[k1c] : 0;
         const uint32_t header = rec.v[0] & 0xFFFFu;
         LaneWords<LW> acc;
 #pragma unroll
         for (int u = 0; u < LW; ++u) acc.w[u] = active ? 0xFFFFFFFFu : 0u;
+        if ((header & 0xFFu) > 7u) {
 #pragma unroll
-        for (int i = 1; i < 8; ++i) and_row(acc, entry_of(rec, i));
-        unsigned long long nz = __ballot(any_bit(acc));
-        if ((header & 0xFFu) > 7u && nz != 0) {
+            for (int i = 1; i < 16; ++i) and_row(acc, entry_of(rec, i));
+        } else {
 #pragma unroll
-            for (int i = 8; i < 16; ++i) and_row(acc, entry_of(rec, i));
-            nz = __ballot(any_bit(acc));
-            if ((header & 0x100u) && nz != 0) {
-                // phase 2: every surviving node slot against the whole include mask
+            for (int i = 1; i < 8; ++i) and_row(acc, entry_of(rec, i));
+        }
+        p.nz = __ballot(any_bit(acc));
+        p.test = (header & 0x100u) && p.nz != 0;
+        int bit = -1;
 #pragma unroll
-                for (int u = 0; u < LW; ++u) {
-                    uint32_t todo = testable ? acc.w[u] : 0u;
-                    while (todo) {
-                        const int b = __ffs(todo) - 1;
-                        todo &= todo - 1;
-                        const uint4 *x = x_lane + (u * 32 + b) * LA4;
-                        uint32_t violated = 0;
+        for (int u = LW - 1; u >= 0; --u) bit = acc.w[u] ? u * 32 + __ffs(acc.w[u]) - 1 : bit;
+        p.bit = testable ? bit : -1;
+        // lanes with nothing to test all read the first node's words (one cache line for the wave)
+        const uint4 *x = p.bit >= 0 ? x_lane + p.bit * LA4 : reinterpret_cast<const uint4 *>(a.X);
 #pragma unroll
-                        for (int q = 0; q < LA4; ++q) {
-                            const uint4 v = x[q];
-                            violated |= (include.v[4 * q] & ~v.x) | (include.v[4 * q + 1] & ~v.y) |
-                                        (include.v[4 * q + 2] & ~v.z) | (include.v[4 * q + 3] & ~v.w);
-                        }
-                        if (violated) acc.w[u] &= ~(1u << b);
-                    }
-                }
-                nz = __ballot(any_bit(acc));
+        for (int q = 0; q < LA4; ++q) p.x[q] = x[q];
+        p.acc = acc;
+    };
+
+    // The rest of phase 2, then the clause's votes (or its truth row).
+    auto finish = [&](Pending &p, const Words<4 * LA4> &include) {
+        if (!p.live) return;
+        p.live = false;
+        LaneWords<LW> acc = p.acc;
+        unsigned long long nz = p.nz;
+        if (p.test) {
+            if (p.bit >= 0 && violates(include, p.x)) {
+#pragma unroll
+                for (int u = 0; u < LW; ++u)
+                    if ((p.bit >> 5) == u) acc.w[u] &= ~(1u << (p.bit & 31));
             }
+#pragma unroll
+            for (int u = 0; u < LW; ++u) {
+                // surviving slots above the one already tested
+                uint32_t todo = p.bit >= 0 ? acc.w[u] : 0u;
+                if (p.bit >= u * 32 + 31) todo = 0u;
+                else if (p.bit >= u * 32) todo &= ~((2u << (p.bit - u * 32)) - 1u);
+                while (todo) {
+                    const int b = __ffs(todo) - 1;
+                    todo &= todo - 1;
+                    if (violates(include, x_lane + (u * 32 + b) * LA4)) acc.w[u] &= ~(1u << b);
+                }
+            }
+            nz = __ballot(any_bit(acc));
         }
         if (!LAST) {
-            if (active) acc.store(truth_out);
+            if (active) acc.store(p.truth_out);
             return;
         }
         if (nz == 0) return;
         // graph j owns lanes [j*lanes_per_graph, (j+1)*lanes_per_graph)
         const unsigned long long gm = __ballot(lane < tg.gpt && ((nz >> my_shift) & slot_lanes) != 0);
-        if (pair_lane && ((gm >> my_j) & 1ull)) atomicAdd(&sums[lane], my_weight);
-        for (int p = lane + 64; p < pairs; p += 64) {
-            int j = p / K, k = p - j * K;
-            if ((gm >> j) & 1ull) atomicAdd(&sums[p], weights_of_clause[k]);
+        if (pair0 && ((gm >> j0) & 1ull)) atomicAdd(&sums[lane], p.weight0);
+        if (pair1 && ((gm >> j1) & 1ull)) atomicAdd(&sums[lane + 64], p.weight1);
+        for (int q = lane + 128; q < pairs; q += 64) {
+            int j = q / K, k = q - j * K;
+            if ((gm >> j) & 1ull) atomicAdd(&sums[q], p.weights[k]);
         }
     };
 
+    // Clause records: the 8 words of row entries are fetched one clause ahead of phase 1, the
+    // include mask at the start of the clause's phase 1 (it is first needed when the clause is
+    // finished, one phase 1 later).  Pointers step by NWAVES clauses; past the end they stay on
+    // the wave's last clause (a valid address whose data is not used).
     const int64_t rec_step = (int64_t)NWAVES * a.stride;
     const int wt_step = NWAVES * K;
     const int64_t truth_step = (int64_t)NWAVES * tw * 4;
@@ -756,24 +812,32 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
     const uint32_t *rec_a = a.lists + (int64_t)first * a.stride;
     const int32_t *wt_a = LAST ? a.wt + (int64_t)first * K : nullptr;
     char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
-    Packed8 ra = *reinterpret_cast<const Packed8 *>(rec_a);
-    Words<4 * LA4> ma = *reinterpret_cast<const Words<4 * LA4> *>(rec_a + 8);
+    Packed8 ea = *reinterpret_cast<const Packed8 *>(rec_a);
+    Words<4 * LA4> ma, mb;
+    Pending pa, pb;
+    pa.live = pb.live = false;
     for (int c = wave; c < C; c += 2 * NWAVES) {
         const bool has_b = c + NWAVES < C;
         const uint32_t *rec_b = has_b ? rec_a + rec_step : rec_a;
         const int32_t *wt_b = LAST ? (has_b ? wt_a + wt_step : wt_a) : nullptr;
         char *truth_b = has_b ? truth_a + truth_step : truth_a;
-        const Packed8 rb = *reinterpret_cast<const Packed8 *>(rec_b);
-        const Words<4 * LA4> mb = *reinterpret_cast<const Words<4 * LA4> *>(rec_b + 8);
-        evaluate(ra, ma, wt_a, truth_a);
+        ma = *reinterpret_cast<const Words<4 * LA4> *>(rec_a + 8);
+        const Packed8 eb = *reinterpret_cast<const Packed8 *>(rec_b);
+        begin(pa, ea, wt_a, truth_a);
+        finish(pb, mb);
         const bool has_a = c + 2 * NWAVES < C;
         rec_a = has_a ? rec_b + rec_step : rec_b;
         if (LAST) wt_a = has_a ? wt_b + wt_step : wt_b;
         truth_a = has_a ? truth_b + truth_step : truth_b;
-        ra = *reinterpret_cast<const Packed8 *>(rec_a);
-        ma = *reinterpret_cast<const Words<4 * LA4> *>(rec_a + 8);
-        if (has_b) evaluate(rb, mb, wt_b, truth_b);
+        // without a second clause this repeats the first one and drops the result: keeping the
+        // sequence of loads the same on every trip lets the waits stay partial
+        mb = *reinterpret_cast<const Words<4 * LA4> *>(rec_b + 8);
+        ea = *reinterpret_cast<const Packed8 *>(rec_a);
+        begin(pb, eb, wt_b, truth_b);
+        pb.live = has_b;
+        finish(pa, ma);
     }
+    finish(pb, mb);
     if (!LAST) return;
     __syncthreads();
     const int64_t g0 = (int64_t)tile * tg.gpt;
