@@ -675,36 +675,41 @@ int launch_tile_layer(const TileLayerArgs &a, int n_tiles, int src, bool last, h
     }
 }
 
-template <int NW, int LW, int LA4, bool LAST>
+template <int NW, int LW, int LA4, bool LAST, bool FULL>
 int launch_two_phase_as(const TileLayerArgs &a, int n_tiles, hipStream_t st) {
     size_t lds = tile_layer_lds_bytes(a.tg, a.K, ROWS_STAGED, a.M);
     static thread_local size_t lds_set = 0;
     if (lds > lds_set) {
-        hipError_t e = hipFuncSetAttribute((const void *)k_tile_two_phase<NW, LW, LA4, LAST>,
+        hipError_t e = hipFuncSetAttribute((const void *)k_tile_two_phase<NW, LW, LA4, LAST, FULL>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
         lds_set = lds;
     }
     if (LAST) profile_start("k_tile_two_phase<score>", st);
-    hipLaunchKernelGGL((k_tile_two_phase<NW, LW, LA4, LAST>), dim3(n_tiles), dim3(NW * 64), lds, st, a);
+    hipLaunchKernelGGL((k_tile_two_phase<NW, LW, LA4, LAST, FULL>), dim3(n_tiles), dim3(NW * 64), lds, st, a);
     if (int rc = check_launch("tile_two_phase")) return rc;
     if (LAST) profile_stop(st);
     return GTM_OK;
 }
 
+template <int NW, int LW, int LA4>
+int launch_two_phase_la(const TileLayerArgs &a, int n_tiles, bool last, hipStream_t st) {
+    const bool full = a.tg.tw == 64 * LW;
+    if (last)
+        return full ? launch_two_phase_as<NW, LW, LA4, true, true>(a, n_tiles, st)
+                    : launch_two_phase_as<NW, LW, LA4, true, false>(a, n_tiles, st);
+    return full ? launch_two_phase_as<NW, LW, LA4, false, true>(a, n_tiles, st)
+                : launch_two_phase_as<NW, LW, LA4, false, false>(a, n_tiles, st);
+}
+
 template <int NW, int LW>
 int launch_two_phase_lw(const TileLayerArgs &a, int n_tiles, int la4, bool last, hipStream_t st) {
-#define GTM_TWO_PHASE(N)                                                         \
-    case N:                                                                      \
-        return last ? launch_two_phase_as<NW, LW, N, true>(a, n_tiles, st)       \
-                    : launch_two_phase_as<NW, LW, N, false>(a, n_tiles, st)
     switch (la4) {
-        GTM_TWO_PHASE(1);
-        GTM_TWO_PHASE(2);
-        GTM_TWO_PHASE(3);
-        default: GTM_TWO_PHASE(4);
+        case 1: return launch_two_phase_la<NW, LW, 1>(a, n_tiles, last, st);
+        case 2: return launch_two_phase_la<NW, LW, 2>(a, n_tiles, last, st);
+        case 3: return launch_two_phase_la<NW, LW, 3>(a, n_tiles, last, st);
+        default: return launch_two_phase_la<NW, LW, 4>(a, n_tiles, last, st);
     }
-#undef GTM_TWO_PHASE
 }
 
 int launch_two_phase(const TileLayerArgs &a, int n_tiles, int la4, bool last, hipStream_t st) {
@@ -717,9 +722,11 @@ int launch_two_phase(const TileLayerArgs &a, int n_tiles, int la4, bool last, hi
 }
 
 // Layer 0 can run in two phases (k_tile_two_phase) on tiles of whole-word graph slots staged in
-// LDS when a node has 4, 8, 12 or 16 literal words.
-bool two_phase_layer0(const Dims &d, const TileGeom &tg) {
-    return tg.slot_words > 0 && tg.stage0 && d.LA % 4 == 0 && d.LA <= 16 && !getenv("GTM_NO_TWO_PHASE");
+// LDS when a node has 4, 8, 12 or 16 literal words.  GTM_NO_TWO_PHASE (tuning aid) turns it off.
+bool two_phase_layer0(const Dims &d, const gtm_graphs *g, const TileGeom &tg) {
+    // the kernel addresses X with 32-bit byte offsets
+    const bool x_fits = (uint64_t)g->total_nodes * d.LA * 4 < (1ull << 32);
+    return tg.slot_words > 0 && tg.stage0 && d.LA % 4 == 0 && d.LA <= 16 && x_fits && !getenv("GTM_NO_TWO_PHASE");
 }
 
 // `_score`'s loop (tm.py:786-812) on tiles: per launch group of tiles, layer 0 and then one
@@ -728,7 +735,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                    const ScoreWs &w, int first, int n_graphs, int batch, int32_t *class_sum, hipStream_t st) {
     const uint32_t *order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
     const int layers = cfg->depth;
-    const bool two_phase = two_phase_layer0(d, tg);
+    const bool two_phase = two_phase_layer0(d, g, tg);
     const int stride0 = two_phase ? 8 + d.LA : w.list_stride;
     if (two_phase)
         hipLaunchKernelGGL(k_compile_clauses_two_phase, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state,

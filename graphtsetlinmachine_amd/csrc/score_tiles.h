@@ -69,6 +69,13 @@ inline TileGeom tile_geometry_lw(int literals, int n_types, int max_nodes, int n
                              TILE_LDS_PAD_WORDS + (size_t)g.gpt * classes) * 4 > TILE_LDS_BUDGET)
             --g.gpt;
         g.tw = (g.gpt * g.slot_words + 3) & ~3;  // rows stay 16-byte aligned
+        // nearly 64 lanes wide: widen the rows to all 64 lanes if that fits (the extra words are zero in
+        // the node-type rows, so kernels need not mask the last lanes off)
+        if (g.gpt > 0 && g.tw * 4 >= max_words * 3 && g.tw < max_words) {
+            TileGeom wide = g;
+            wide.tw = max_words;
+            if (tile_lds_bytes(fit_rows, wide, classes) <= TILE_LDS_BUDGET) g.tw = max_words;
+        }
     }
     g.n_tiles = g.gpt > 0 ? (n_graphs + g.gpt - 1) / g.gpt : 0;
     g.ok = g.gpt > 0 && tile_lds_bytes(fit_rows, g, classes) <= TILE_LDS_BUDGET;
@@ -635,7 +642,7 @@ __global__ void k_compile_clauses_two_phase(const uint32_t *__restrict__ bank, i
 // (each lane the literal words of its first surviving node slot), runs phase 1 of its next clause
 // while they are in flight, and only then finishes the first.  Lanes with more than one surviving
 // slot test the others in a loop afterwards (rare once 14 literals have been applied).
-template <int NWAVES, int LW, int LA4, bool LAST>
+template <int NWAVES, int LW, int LA4, bool LAST, bool FULL>
 __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a) {
     extern __shared__ uint32_t lds[];
     const TileGeom &tg = a.tg;
@@ -670,7 +677,9 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
     }
     __syncthreads();
 
-    const bool active = lane * LW < tw;
+    // FULL: rows are exactly 64 * LW words wide, padded with words that are zero in the node-type
+    // rows, so every lane holds real words and no lane needs masking off.
+    const bool active = FULL || lane * LW < tw;
     const char *col = reinterpret_cast<const char *>(bt + lane * LW);
 
     // the graph whose slot this lane's words belong to, and the node of the lane's first bit
@@ -680,15 +689,18 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
     const bool has_graph = active && lane_j < tg.gpt && lane_g < a.G;
     // a graph without nodes keeps its slot bit 0 (every clause is true for it) and has no node to test
     const bool testable = has_graph && a.n_nodes[lane_g] != 0u;
-    const int64_t lane_node0 = has_graph ? (int64_t)a.node_index[lane_g] + (lane - lane_j * lpg) * (LW * 32) : 0;
-    const uint4 *x_lane = reinterpret_cast<const uint4 *>(a.X) + lane_node0 * LA4;
+    // byte offset of that node's literal words in X (the host checks that X is smaller than 4 GiB)
+    const uint32_t lane_x0 =
+        has_graph ? (a.node_index[lane_g] + (uint32_t)(lane - lane_j * lpg) * (LW * 32)) * (LA4 * 16u) : 0u;
+    const char *x_base = reinterpret_cast<const char *>(a.X);
 
     // lane p adds weight k = p % K to graph j = p / K of the tile, for p = lane and p = lane + 64
     const int pairs = tg.gpt * K;
     const int j0 = lane / K, k0 = lane - j0 * K;
     const int j1 = (lane + 64) / K, k1 = lane + 64 - j1 * K;
     const bool pair0 = LAST && lane < pairs, pair1 = LAST && lane + 64 < pairs;
-    const int k0c = pair0 ? k0 : 0, k1c = pair1 ? k1 : 0;
+    const uint32_t k0_bytes = pair0 ? k0 * 4u : 0u, k1_bytes = pair1 ? k1 * 4u : 0u;
+    const uint32_t shift0 = pair0 ? j0 * lpg : 0, shift1 = pair1 ? j1 * lpg : 0;  // first lane of the pair's graph
     const int my_shift = (lane < tg.gpt ? lane : 0) * lpg;
     const unsigned long long slot_lanes = lpg >= 64 ? ~0ull : (1ull << lpg) - 1ull;
 
@@ -715,11 +727,26 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
         }
         return violated != 0;
     };
+    // the word set with only `bit` set (bit < 32 * LW)
+    auto one_hot = [](uint32_t bit) {
+        LaneWords<LW> m;
+        if (LW == 1) {
+            m.w[0] = 1u << (bit & 31u);
+        } else {
+#pragma unroll
+            for (int h = 0; h < LW / 2; ++h) {
+                const unsigned long long v = (LW == 2 || (int)(bit >> 6) == h) ? 1ull << (bit & 63u) : 0ull;
+                m.w[2 * h] = (uint32_t)v;
+                m.w[2 * h + 1] = (uint32_t)(v >> 32);
+            }
+        }
+        return m;
+    };
 
     struct Pending {
         LaneWords<LW> acc;
         uint4 x[LA4];
-        int bit;                 // the node slot this lane has under test (index into its LW words), -1 if none
+        uint32_t bit;            // the node slot this lane has under test (index into its LW words), ~0 if none
         bool live, test;         // wave-uniform: a clause is pending / its phase 2 runs
         unsigned long long nz;   // lanes with a surviving slot after phase 1
         int weight0, weight1;
@@ -727,15 +754,17 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
         char *truth_out;
     };
 
-    // Phase 1 and the loads of phase 2.
+    // Phase 1 and the loads of phase 2.  Every load is issued by all lanes whatever the clause
+    // does, so that the number of loads in flight is known when the pending clause is finished.
     auto begin = [&](Pending &p, const Packed8 &rec, const int32_t *weights_of_clause, char *truth_out) {
         p.live = true;
         p.weights = weights_of_clause;
         p.truth_out = truth_out;
-        // every load below is issued by all lanes whatever the clause does, so that the number of
-        // loads in flight is known when the pending clause is finished
-        p.weight0 = LAST ? weights_of_clause[k0c] : 0;  // needed only if the clause fires
-        p.weight1 = LAST ? weights_of_clause[k1c] : 0;
+        if (LAST) {  // needed only if the clause fires
+            const char *wb = reinterpret_cast<const char *>(weights_of_clause);
+            p.weight0 = *reinterpret_cast<const int32_t *>(wb + k0_bytes);
+            p.weight1 = *reinterpret_cast<const int32_t *>(wb + k1_bytes);
+        }
         const uint32_t header = rec.v[0] & 0xFFFFu;
         LaneWords<LW> acc;
 #pragma unroll
@@ -749,12 +778,17 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
         }
         p.nz = __ballot(any_bit(acc));
         p.test = (header & 0x100u) && p.nz != 0;
-        int bit = -1;
+        // lowest surviving slot of the lane; __ffs(0) - 1 is ~0, which also survives the OR and the min
+        uint32_t bit = ~0u;
 #pragma unroll
-        for (int u = LW - 1; u >= 0; --u) bit = acc.w[u] ? u * 32 + __ffs(acc.w[u]) - 1 : bit;
-        p.bit = testable ? bit : -1;
+        for (int u = LW - 1; u >= 0; --u) {
+            const uint32_t at = (uint32_t)(__ffs(acc.w[u]) - 1) | (uint32_t)(u * 32);
+            bit = at < bit ? at : bit;
+        }
+        p.bit = testable ? bit : ~0u;
         // lanes with nothing to test all read the first node's words (one cache line for the wave)
-        const uint4 *x = p.bit >= 0 ? x_lane + p.bit * LA4 : reinterpret_cast<const uint4 *>(a.X);
+        const uint32_t x_off = p.bit != ~0u ? lane_x0 + p.bit * (LA4 * 16u) : 0u;
+        const uint4 *x = reinterpret_cast<const uint4 *>(x_base + x_off);
 #pragma unroll
         for (int q = 0; q < LA4; ++q) p.x[q] = x[q];
         p.acc = acc;
@@ -767,21 +801,26 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
         LaneWords<LW> acc = p.acc;
         unsigned long long nz = p.nz;
         if (p.test) {
-            if (p.bit >= 0 && violates(include, p.x)) {
-#pragma unroll
-                for (int u = 0; u < LW; ++u)
-                    if ((p.bit >> 5) == u) acc.w[u] &= ~(1u << (p.bit & 31));
-            }
+            const bool tested = p.bit != ~0u;
+            const bool failed = violates(include, p.x) && tested;
+            // the lane's other surviving slots
+            const LaneWords<LW> hot = one_hot(p.bit);
+            LaneWords<LW> rest;
 #pragma unroll
             for (int u = 0; u < LW; ++u) {
-                // surviving slots above the one already tested
-                uint32_t todo = p.bit >= 0 ? acc.w[u] : 0u;
-                if (p.bit >= u * 32 + 31) todo = 0u;
-                else if (p.bit >= u * 32) todo &= ~((2u << (p.bit - u * 32)) - 1u);
-                while (todo) {
-                    const int b = __ffs(todo) - 1;
-                    todo &= todo - 1;
-                    if (violates(include, x_lane + (u * 32 + b) * LA4)) acc.w[u] &= ~(1u << b);
+                rest.w[u] = acc.w[u] & ~hot.w[u];
+                acc.w[u] = failed ? rest.w[u] : acc.w[u];
+            }
+            if (__ballot(tested && any_bit(rest)) != 0) {
+#pragma unroll
+                for (int u = 0; u < LW; ++u) {
+                    uint32_t todo = tested ? rest.w[u] : 0u;
+                    while (todo) {
+                        const int b = __ffs(todo) - 1;
+                        todo &= todo - 1;
+                        const uint4 *x = reinterpret_cast<const uint4 *>(x_base + (lane_x0 + (u * 32 + b) * (LA4 * 16u)));
+                        if (violates(include, x)) acc.w[u] &= ~(1u << b);
+                    }
                 }
             }
             nz = __ballot(any_bit(acc));
@@ -792,12 +831,18 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
         }
         if (nz == 0) return;
         // graph j owns lanes [j*lanes_per_graph, (j+1)*lanes_per_graph)
-        const unsigned long long gm = __ballot(lane < tg.gpt && ((nz >> my_shift) & slot_lanes) != 0);
-        if (pair0 && ((gm >> j0) & 1ull)) atomicAdd(&sums[lane], p.weight0);
-        if (pair1 && ((gm >> j1) & 1ull)) atomicAdd(&sums[lane + 64], p.weight1);
-        for (int q = lane + 128; q < pairs; q += 64) {
-            int j = q / K, k = q - j * K;
-            if ((gm >> j) & 1ull) atomicAdd(&sums[q], p.weights[k]);
+        if (lpg <= 32 && pairs <= 128) {
+            const uint32_t m = (uint32_t)slot_lanes;
+            if (pair0 && ((uint32_t)(nz >> shift0) & m) != 0) atomicAdd(&sums[lane], p.weight0);
+            if (pair1 && ((uint32_t)(nz >> shift1) & m) != 0) atomicAdd(&sums[lane + 64], p.weight1);
+        } else {
+            const unsigned long long gm = __ballot(lane < tg.gpt && ((nz >> my_shift) & slot_lanes) != 0);
+            if (pair0 && ((gm >> j0) & 1ull)) atomicAdd(&sums[lane], p.weight0);
+            if (pair1 && ((gm >> j1) & 1ull)) atomicAdd(&sums[lane + 64], p.weight1);
+            for (int q = lane + 128; q < pairs; q += 64) {
+                int j = q / K, k = q - j * K;
+                if ((gm >> j) & 1ull) atomicAdd(&sums[q], p.weights[k]);
+            }
         }
     };
 
