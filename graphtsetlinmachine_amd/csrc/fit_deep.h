@@ -1,0 +1,122 @@
+// The message layers of one training step (tm.py:595-650) for one graph.
+//
+//   k_fit_scatter_messages  K4 (+K5): one thread per (clause, node); a clause
+//                           that is true at the node sets, at every
+//                           out-neighbour, its hypervector bits rotated by the
+//                           edge type and clears their negations, straight into
+//                           the packed node-major message words (blanked first
+//                           by k_messages_blank, K3).
+//   k_fit_message_rows      the positive half of those words turned literal-
+//                           major: row p holds bit p of every node.
+//   k_fit_message_eval      K2: as k_fit_eval, but a clause starts from its
+//                           truth in the layer before and ANDs the message rows
+//                           (or their complements, for negated message
+//                           literals) that its message automata include.
+#pragma once
+
+constexpr int FIT_SCATTER_BLOCK = 256;
+
+__global__ __launch_bounds__(FIT_SCATTER_BLOCK) void k_fit_scatter_messages(
+    const uint32_t *__restrict__ bitmap, int C, int NC, int n_nodes, const uint32_t *__restrict__ hv, int MB, int M,
+    int MC, const uint32_t *__restrict__ n_edges, const uint32_t *__restrict__ edge_index,
+    const uint32_t *__restrict__ edge, uint32_t *clause_X) {
+    // n_edges / edge_index point at the graph's first node
+    const int64_t i = (int64_t)blockIdx.x * FIT_SCATTER_BLOCK + threadIdx.x;
+    const int c = (int)(i / n_nodes), n = (int)(i - (int64_t)c * n_nodes);
+    if (c >= C) return;
+    if (!((bitmap[(int64_t)c * NC + (n >> 5)] >> (n & 31)) & 1u)) return;
+    const uint32_t ne = n_edges[n];
+    const int64_t e0 = edge_index[n];
+    for (uint32_t e = 0; e < ne; ++e) {
+        const uint32_t dst = edge[(e0 + e) * 2], type = edge[(e0 + e) * 2 + 1];
+        for (int j = 0; j < MB; ++j) {
+            const uint32_t pos = (hv[(int64_t)c * MB + j] + type) % (uint32_t)M;
+            const uint32_t neg = pos + (uint32_t)M;
+            atomicOr(&clause_X[(int64_t)dst * MC + (pos >> 5)], 1u << (pos & 31));
+            atomicAnd(&clause_X[(int64_t)dst * MC + (neg >> 5)], ~(1u << (neg & 31)));
+        }
+    }
+}
+
+// One wave per (32 message literals, 64 nodes): lane n holds the node's word of
+// those literals; the ballot of bit b over the wave is row 32w + b for these 64
+// nodes.  rows[M][row_words], row_words even.
+__global__ __launch_bounds__(64) void k_fit_message_rows(const uint32_t *__restrict__ clause_X, int n_nodes, int M,
+                                                          int MC, int row_words, uint32_t *__restrict__ rows) {
+    const int lane = threadIdx.x;
+    const int w = blockIdx.x, nb = blockIdx.y;
+    const int n = nb * 64 + lane;
+    const uint32_t word = n < n_nodes ? clause_X[(int64_t)n * MC + w] : 0u;
+    unsigned long long mine = 0;
+#pragma unroll
+    for (int b = 0; b < 32; ++b) {
+        const unsigned long long column = __ballot((word >> b) & 1u);
+        if (lane == b) mine = column;
+    }
+    const int p = w * 32 + lane;
+    if (lane < 32 && p < M) {
+        rows[(int64_t)p * row_words + nb * 2] = (uint32_t)mine;
+        rows[(int64_t)p * row_words + nb * 2 + 1] = (uint32_t)(mine >> 32);
+    }
+}
+
+// K2 (+ K6 + K7 when `finish`) for one graph and one message layer.  Each wave
+// takes clauses in turn; lane L holds word L of the clause's truth over the
+// graph's nodes, starting from the layer before.  The clause's include words
+// come from the top bit plane of the layer's automaton bank; message literal
+// l < M reads row l, literal l >= M the complement of row l - M
+// (kernels.py:505-527; positions past the graph's nodes are already 0 in the
+// incoming truth).
+__global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
+    const uint32_t *__restrict__ rows, int row_words, int words, int n_nodes, int M, int C, int MC, int B, int K,
+    int NC, uint32_t filter, const uint32_t *__restrict__ bank, const int32_t *__restrict__ weights, uint32_t k0,
+    uint32_t k1, uint32_t step, int finish, const uint32_t *__restrict__ bitmap_in, uint32_t *__restrict__ bitmap_out,
+    int32_t *__restrict__ n_incl, int32_t *__restrict__ clause_node, int32_t *class_sum) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int WAVES = FIT_EVAL_BLOCK / 64;
+    const bool active = lane < words;
+    const uint32_t *col = rows + (active ? lane : 0);
+    int partial = 0;
+    for (int c = blockIdx.x * WAVES + wave; c < C; c += gridDim.x * WAVES) {
+        const uint32_t *inc = bank + (int64_t)c * MC * B + (B - 1);
+        uint32_t acc = active ? bitmap_in[(int64_t)c * NC + lane] : 0u;
+        int included = 0;
+        for (int w0 = 0; w0 < MC; w0 += 64) {
+            uint32_t mine = w0 + lane < MC ? inc[(int64_t)(w0 + lane) * B] : 0u;
+            if (w0 + lane == MC - 1) mine &= filter;
+            unsigned long long nonzero = __ballot(mine != 0);
+            included += __popc(mine);
+            // a clause that is false everywhere stays false: only its include count is needed
+            if (__ballot(acc != 0) == 0) continue;
+            while (nonzero) {
+                const int wl = __ffsll((long long)nonzero) - 1;
+                nonzero &= nonzero - 1;
+                uint32_t m = __builtin_amdgcn_readlane(mine, wl);
+                const int base = (w0 + wl) << 5;
+                while (m) {
+                    uint32_t r[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        // wave-uniform: the literal, its row, whether it is negated; unused slots read row 0 and give all ones
+                        const bool used = m != 0;
+                        const int lit = used ? base + __builtin_ctz(m) : 0;
+                        m &= m - 1;
+                        const bool negated = lit >= M;
+                        const uint32_t flip = negated ? 0xFFFFFFFFu : 0u, fill = used ? 0u : 0xFFFFFFFFu;
+                        r[u] = (col[(int64_t)(negated ? lit - M : lit) * row_words] ^ flip) | fill;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc &= r[u];
+                }
+            }
+        }
+        for (int off = 32; off > 0; off >>= 1) included += __shfl_xor(included, off);
+        const uint32_t v = active ? acc : 0u;
+        if (lane == 0) n_incl[c] += included;
+        fit_clause_tail(v, lane, words, NC, n_nodes, c, C, K, weights, k0, k1, step, finish != 0,
+                        bitmap_out + (int64_t)c * NC, clause_node, class_sum, &partial);
+    }
+    if (K <= 64 && lane < K && partial != 0) atomicAdd(&class_sum[lane], partial);
+}

@@ -45,18 +45,71 @@ __host__ __device__ inline FitGraph fit_graph_slot(const TileGeom &tg, int graph
     return f;
 }
 
+// The end of a clause's evaluation for one graph, shared by every layer: lane L holds word L of
+// the clause's truth over the graph's nodes.  Writes the clause's row of the clause/node bitmap
+// and, when `finish` is set (the last layer), picks the node the clause learns from (K7,
+// kernels.py:319-354) and adds the clause's weights to the class sums (K6, kernels.py:279-317;
+// lanes k < K keep a running sum in *partial when K <= 64).
+__device__ __forceinline__ void fit_clause_tail(uint32_t v, int lane, int words, int NC, int n_nodes, int c, int C, int K,
+                                                const int32_t *__restrict__ weights, uint32_t k0, uint32_t k1,
+                                                uint32_t step, bool finish, uint32_t *out,
+                                                int32_t *__restrict__ clause_node, int32_t *class_sum, int *partial) {
+    // chunks past the graph are left all ones, as kernels.py:443-466 leaves them
+    for (int i = lane; i < NC; i += 64) out[i] = i < words ? (i == lane ? v : 0u) : 0xFFFFFFFFu;
+    // the reference's arithmetic for a graph without nodes (kernels.py:289-295)
+    if (n_nodes == 0 && lane == 0) out[0] = 0xFFFFFFFFu;
+    if (!finish) return;
+    // true nodes before this lane's word, and in total
+    const int pc = __popc(v);
+    int before = pc;
+    for (int off = 1; off < 64; off <<= 1) {
+        int t = __shfl_up(before, off);
+        if (lane >= off) before += t;
+    }
+    const int true_nodes = __shfl(before, 63);
+    before -= pc;
+    bool fired = true_nodes > 0;
+    int node = -1;
+    if (n_nodes == 0) {
+        fired = true;
+    } else if (fired) {
+        // K7: the pick-th true node, pick = (r * count) >> 32
+        philox_out r = philox4x32_10((uint32_t)c, 0u, step, GTM_TAG_CLAUSE_NODE, k0, k1);
+        const int pick = (int)(((uint64_t)r.v[0] * (uint64_t)true_nodes) >> 32);
+        const bool mine = pick >= before && pick < before + pc;
+        int candidate = 0;
+        if (mine) {
+            uint32_t t = v;
+            for (int j = before; j < pick; ++j) t &= t - 1;
+            candidate = lane * 32 + __ffs(t) - 1;
+        }
+        const unsigned long long owner = __ballot(mine);
+        node = __shfl(candidate, __ffsll((long long)owner) - 1);
+    }
+    if (lane == 0) clause_node[c] = node;
+    // K6
+    if (fired) {
+        if (K <= 64) {
+            if (lane < K) *partial += weights[(int64_t)lane * C + c];
+        } else {
+            for (int k = lane; k < K; k += 64) atomicAdd(&class_sum[k], weights[(int64_t)k * C + c]);
+        }
+    }
+}
+
 // K1 + K6 + K7 for one graph.  A block stages the graph's literal-major rows
 // (plus an all-ones row) in LDS; each wave then takes clauses in turn.  The
 // clause is wave-uniform: its include words come in by scalar loads straight
 // from the top bit plane of the automaton bank, their set bits are walked on
 // the scalar unit, and lane L ANDs word L of every included literal's row, 8
 // LDS reads in flight at a time.  STAGE = false reads the rows from the tile
-// in global memory instead (graphs whose rows do not fit in LDS).
+// in global memory instead (graphs whose rows do not fit in LDS).  `finish` = 0
+// (models with message layers) stops after the bitmap and the include counts.
 template <bool STAGE>
 __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
     const uint32_t *__restrict__ tiles, TileGeom tg, FitGraph fg, int n_nodes, int literals, int n_types, int C, int LA,
     int B, int K, int NC, uint32_t filter, const uint32_t *__restrict__ bank, const int32_t *__restrict__ weights,
-    uint32_t k0, uint32_t k1, uint32_t step, uint32_t *__restrict__ bitmap, int32_t *__restrict__ n_incl,
+    uint32_t k0, uint32_t k1, uint32_t step, int finish, uint32_t *__restrict__ bitmap, int32_t *__restrict__ n_incl,
     int32_t *__restrict__ clause_node, int32_t *class_sum) {
     extern __shared__ uint32_t rows_lds[];
     const int tid = threadIdx.x;
@@ -122,49 +175,9 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
         }
         for (int off = 32; off > 0; off >>= 1) included += __shfl_xor(included, off);
         const uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
-        uint32_t *out = bitmap + (int64_t)c * NC;
-        // chunks past the graph are left all ones, as kernels.py:443-466 leaves them
-        for (int i = lane; i < NC; i += 64) out[i] = i < fg.words ? (i == lane ? v : 0u) : 0xFFFFFFFFu;
-        // true nodes before this lane's word, and in total
-        const int pc = __popc(v);
-        int before = pc;
-        for (int off = 1; off < 64; off <<= 1) {
-            int t = __shfl_up(before, off);
-            if (lane >= off) before += t;
-        }
-        const int true_nodes = __shfl(before, 63);
-        before -= pc;
-        bool fired = true_nodes > 0;
-        int node = -1;
-        if (n_nodes == 0) {
-            if (lane == 0) out[0] = 0xFFFFFFFFu;  // the reference's arithmetic for a graph without nodes (kernels.py:289-295)
-            fired = true;
-        } else if (fired) {
-            // K7: the pick-th true node, pick = (r * count) >> 32
-            philox_out r = philox4x32_10((uint32_t)c, 0u, step, GTM_TAG_CLAUSE_NODE, k0, k1);
-            const int pick = (int)(((uint64_t)r.v[0] * (uint64_t)true_nodes) >> 32);
-            const bool mine = pick >= before && pick < before + pc;
-            int candidate = 0;
-            if (mine) {
-                uint32_t t = v;
-                for (int j = before; j < pick; ++j) t &= t - 1;
-                candidate = lane * 32 + __ffs(t) - 1;
-            }
-            const unsigned long long owner = __ballot(mine);
-            node = __shfl(candidate, __ffsll((long long)owner) - 1);
-        }
-        if (lane == 0) {
-            clause_node[c] = node;
-            n_incl[c] = included;
-        }
-        // K6
-        if (fired) {
-            if (K <= 64) {
-                if (lane < K) partial += weights[(int64_t)lane * C + c];
-            } else {
-                for (int k = lane; k < K; k += 64) atomicAdd(&class_sum[k], weights[(int64_t)k * C + c]);
-            }
-        }
+        if (lane == 0) n_incl[c] = included;
+        fit_clause_tail(v, lane, fg.words, NC, n_nodes, c, C, K, weights, k0, k1, step, finish != 0,
+                        bitmap + (int64_t)c * NC, clause_node, class_sum, &partial);
     }
     if (K <= 64 && lane < K && partial != 0) atomicAdd(&class_sum[lane], partial);
 }
@@ -266,13 +279,24 @@ __device__ __forceinline__ void wave_count_scan(int count, int lane, int *total,
     *before = b;
 }
 
-// K8 + K9 for `cpb` clauses per block; see the header comment.
-__global__ void k_fit_feedback(uint32_t *bank, int32_t *weights, const int32_t *class_sum,
-                               int32_t *class_sum_next, const int32_t *__restrict__ y, int C, int LA, int B, int K,
+// The automaton banks one training step updates: bank 0 holds the literals of
+// the nodes (rows = the graph's X rows), bank l > 0 the message literals of
+// layer l (rows = that layer's messages, one row of `chunks` words per node).
+struct FitBanks {
+    int n;
+    int total_chunks;  // sum of chunks[]
+    uint32_t *bank[GTM_MAX_DEPTH];
+    const uint32_t *rows[GTM_MAX_DEPTH];
+    int chunks[GTM_MAX_DEPTH];
+    uint32_t thr16[GTM_MAX_DEPTH];
+};
+
+// K8 + K9 (+ K10 for the message banks) for `cpb` clauses per block; see the header comment.
+__global__ void k_fit_feedback(FitBanks banks, int32_t *weights, const int32_t *class_sum,
+                               int32_t *class_sum_next, const int32_t *__restrict__ y, int C, int B, int K,
                                int T, int negative, int boost, int max_included, uint64_t q_thr,
-                               uint32_t thr16, uint32_t k0, uint32_t k1, uint32_t step,
-                               const int32_t *__restrict__ clause_node, const int32_t *__restrict__ n_incl,
-                               const uint32_t *__restrict__ X_rows, int cpb) {
+                               uint32_t k0, uint32_t k1, uint32_t step,
+                               const int32_t *__restrict__ clause_node, const int32_t *__restrict__ n_incl, int cpb) {
     extern __shared__ int32_t upd[];  // [cpb][K]
     const int tid = threadIdx.x;
     const int c_base = blockIdx.x * cpb;
@@ -308,19 +332,41 @@ __global__ void k_fit_feedback(uint32_t *bank, int32_t *weights, const int32_t *
     }
     __syncthreads();
 
-    for (int i = tid; i < cpb * LA; i += blockDim.x) {
-        const int local = i / LA, w = i - local * LA;
+    const int per_clause = banks.total_chunks;
+    for (int i = tid; i < cpb * per_clause; i += blockDim.x) {
+        const int local = i / per_clause;
+        int w = i - local * per_clause;
         const int c = c_base + local;
         if (c >= C) continue;
         const int32_t *u_of = upd + local * K;
         bool any = false;
         for (int k = 0; k < K; ++k) any |= u_of[k] != 0;
         if (!any) continue;
+        // which bank the word belongs to (static indices: the struct stays in scalar registers)
+        int l = 0, chunks = banks.chunks[0], first = 0;
+        uint32_t *bank = banks.bank[0];
+        const uint32_t *rows = banks.rows[0];
+        uint32_t thr16 = banks.thr16[0];
+        int start = banks.chunks[0];
+#pragma unroll
+        for (int t = 1; t < GTM_MAX_DEPTH; ++t) {
+            if (t < banks.n && w >= start) {
+                l = t;
+                first = start;
+                chunks = banks.chunks[t];
+                bank = banks.bank[t];
+                rows = banks.rows[t];
+                thr16 = banks.thr16[t];
+            }
+            start += t < banks.n ? banks.chunks[t] : 0;
+        }
+        w -= first;
         const int node = clause_node[c];
         const bool fired = node != -1;
         const bool within = n_incl[c] <= max_included;
-        const uint32_t x = fired ? X_rows[(int64_t)node * LA + w] : 0u;
-        uint32_t *ta = bank + ((int64_t)c * LA + w) * B;
-        feedback_word_any(ta, B, K, u_of, 1, fired, within, boost, x, k0, k1, (uint32_t)c, (uint32_t)w, step, 0u, thr16);
+        const uint32_t x = fired ? rows[(int64_t)node * chunks + w] : 0u;
+        uint32_t *ta = bank + ((int64_t)c * chunks + w) * B;
+        feedback_word_any(ta, B, K, u_of, 1, fired, within, boost, x, k0, k1, (uint32_t)c, (uint32_t)w, step,
+                          (uint32_t)l, thr16);
     }
 }

@@ -407,6 +407,7 @@ __device__ __forceinline__ void ta_dec(uint32_t *ta, int B, uint32_t active) {
 }
 
 #include "fit_fused.h"
+#include "fit_deep.h"
 #include "fit_persistent.h"
 
 // K9 / K10: one thread per (clause, automaton word); the classes are applied
@@ -522,6 +523,8 @@ struct FitWs {
     int32_t *clause_node;                   // [C]
     int32_t *n_incl;                        // [C]
     int32_t *update;                        // [K][C]
+    uint32_t *message_rows;                 // [M][message_row_words] literal-major messages of one layer (depth > 1)
+    int message_row_words;
     size_t bytes;
 };
 
@@ -544,6 +547,8 @@ FitWs carve_fit(const Dims &d, const gtm_config *cfg, char *base) {
     w.clause_node = (int32_t *)take((size_t)d.C * 4);
     w.n_incl = (int32_t *)take((size_t)d.C * 4);
     w.update = (int32_t *)take((size_t)d.K * d.C * 4);
+    w.message_row_words = 2 * ((cfg->max_nodes + 63) / 64);
+    w.message_rows = cfg->depth > 1 ? (uint32_t *)take((size_t)d.M * w.message_row_words * 4) : nullptr;
     w.bytes = off;
     return w;
 }
@@ -1221,18 +1226,119 @@ int fit_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, cons
         if (stage)
             hipLaunchKernelGGL(k_fit_eval<true>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), lds, st, g->tiles, tg, fg,
                                (int)h_n[i], cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
-                               s->clause_weights, key.k0, key.k1, step, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
+                               s->clause_weights, key.k0, key.k1, step, 1, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
         else
             hipLaunchKernelGGL(k_fit_eval<false>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), 0, st, g->tiles, tg, fg,
                                (int)h_n[i], cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
-                               s->clause_weights, key.k0, key.k1, step, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
+                               s->clause_weights, key.k0, key.k1, step, 1, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
         if (int rc = check_launch("fit_eval")) return rc;
         if (i < Profile::MAX) profile_stop(st);
-        hipLaunchKernelGGL(k_fit_feedback, dim3(blocks_for(d.C, cpb)), dim3(TPB), (size_t)cpb * d.K * 4, st,
-                           s->ta_state, s->clause_weights, sum_now, sum_next, encoded_Y + (int64_t)ex * d.K, d.C, d.LA,
-                           d.B, d.K, cfg->threshold, cfg->negative_clauses, cfg->boost_true_positive_feedback,
-                           cfg->max_included_literals, q_thr, thr16, key.k0, key.k1, step, w.clause_node, w.n_incl,
-                           g->X + (int64_t)h_base[i] * d.LA, cpb);
+        FitBanks banks{};
+        banks.n = 1;
+        banks.total_chunks = d.LA;
+        banks.bank[0] = s->ta_state;
+        banks.rows[0] = g->X + (int64_t)h_base[i] * d.LA;
+        banks.chunks[0] = d.LA;
+        banks.thr16[0] = thr16;
+        hipLaunchKernelGGL(k_fit_feedback, dim3(blocks_for(d.C, cpb)), dim3(TPB), (size_t)cpb * d.K * 4, st, banks,
+                           s->clause_weights, sum_now, sum_next, encoded_Y + (int64_t)ex * d.K, d.C, d.B, d.K,
+                           cfg->threshold, cfg->negative_clauses, cfg->boost_true_positive_feedback,
+                           cfg->max_included_literals, q_thr, key.k0, key.k1, step, w.clause_node, w.n_incl, cpb);
+        if (int rc = check_launch("fit_feedback")) return rc;
+    }
+    return GTM_OK;
+}
+
+// One training step of a model with message layers (tm.py:669-747) in 2 + 4 launches per layer:
+// layer 0 on the graph's tile rows, then per message layer the messages (blank, scatter,
+// literal-major copy) and the conditional evaluation, then one feedback kernel over all banks.
+int fit_deep_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
+                      const FitWs &w, const int32_t *encoded_Y, int first_example, int n_examples, uint64_t first_step,
+                      const uint32_t *h_n, const uint32_t *h_base, hipStream_t st) {
+    hipLaunchKernelGGL(k_fill_i32, dim3(1), dim3(TPB), 0, st, w.class_sum, (int64_t)d.K * 2, 0);
+    if (int rc = check_launch("fill")) return rc;
+    if (g->total_edges > 0 && (!g->number_of_graph_node_edges || !g->edge || !g->edge_index))
+        return fail(GTM_ERR_INVALID, "graphs with edges need number_of_graph_node_edges, edge and edge_index");
+    Key key = key_of(cfg);
+    const int n_types = g->number_of_node_types;
+    const int layers = cfg->depth - 1;
+    const int per_clause = d.LA + layers * d.MC;
+    const int cpb = per_clause >= TPB ? 1 : TPB / per_clause;
+    const uint64_t q_thr = q_threshold(cfg->q, cfg->classes);
+    const int waves_per_block = FIT_EVAL_BLOCK / 64;
+    int eval_blocks = (d.C + 2 * waves_per_block - 1) / (2 * waves_per_block);
+    if (eval_blocks > 1024) eval_blocks = 1024;
+    static thread_local size_t lds_set = 0;
+    for (int i = 0; i < n_examples; ++i) {
+        const int ex = first_example + i;
+        const int n_nodes = (int)h_n[i];
+        const uint32_t step = (uint32_t)(first_step + (uint64_t)i);
+        FitGraph fg = fit_graph_slot(tg, ex, n_nodes);
+        int32_t *sum_now = w.class_sum + (size_t)(i & 1) * d.K, *sum_next = w.class_sum + (size_t)((i + 1) & 1) * d.K;
+        size_t lds = (size_t)(cfg->literals + n_types + 1) * fg.words * 4;
+        const bool stage = lds <= 96 * 1024;
+        if (stage && lds > lds_set) {
+            hipError_t e = hipFuncSetAttribute((const void *)k_fit_eval<true>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
+            lds_set = lds;
+        }
+        if (stage)
+            hipLaunchKernelGGL(k_fit_eval<true>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), lds, st, g->tiles, tg, fg,
+                               n_nodes, cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
+                               s->clause_weights, key.k0, key.k1, step, 0, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
+        else
+            hipLaunchKernelGGL(k_fit_eval<false>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), 0, st, g->tiles, tg, fg,
+                               n_nodes, cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
+                               s->clause_weights, key.k0, key.k1, step, 0, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
+        if (int rc = check_launch("fit_eval")) return rc;
+        uint32_t *cur = w.bitmap_a, *nxt = w.bitmap_b;
+        const int words = n_nodes == 0 ? 1 : (n_nodes - 1) / 32 + 1;
+        for (int l = 0; l < layers; ++l) {
+            uint32_t *cx = w.clause_X[l];
+            if (n_nodes > 0) {
+                const int64_t message_words = (int64_t)n_nodes * d.MC;
+                hipLaunchKernelGGL(k_messages_blank, dim3(blocks_for(message_words, TPB)), dim3(TPB), 0, st, cx,
+                                   message_words, d.MC, d.M);
+                if (int rc = check_launch("messages_blank")) return rc;
+                if (g->total_edges > 0) {
+                    const int64_t pairs = (int64_t)d.C * n_nodes;
+                    hipLaunchKernelGGL(k_fit_scatter_messages, dim3(blocks_for(pairs, FIT_SCATTER_BLOCK)),
+                                       dim3(FIT_SCATTER_BLOCK), 0, st, cur, d.C, d.NC, n_nodes, s->hypervectors, d.MB,
+                                       d.M, d.MC, g->number_of_graph_node_edges + h_base[i], g->edge_index + h_base[i],
+                                       g->edge, cx);
+                    if (int rc = check_launch("fit_scatter_messages")) return rc;
+                }
+            }
+            hipLaunchKernelGGL(k_fit_message_rows, dim3((d.M + 31) / 32, w.message_row_words / 2), dim3(64), 0, st, cx,
+                               n_nodes, d.M, d.MC, w.message_row_words, w.message_rows);
+            if (int rc = check_launch("fit_message_rows")) return rc;
+            hipLaunchKernelGGL(k_fit_message_eval, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), 0, st, w.message_rows,
+                               w.message_row_words, words, n_nodes, d.M, d.C, d.MC, d.B, d.K, d.NC, d.mfilter,
+                               s->message_ta_state[l], s->clause_weights, key.k0, key.k1, step, l == layers - 1 ? 1 : 0,
+                               cur, nxt, w.n_incl, w.clause_node, sum_now);
+            if (int rc = check_launch("fit_message_eval")) return rc;
+            uint32_t *t = cur;
+            cur = nxt;
+            nxt = t;
+        }
+        FitBanks banks{};
+        banks.n = cfg->depth;
+        banks.total_chunks = per_clause;
+        banks.bank[0] = s->ta_state;
+        banks.rows[0] = g->X + (int64_t)h_base[i] * d.LA;
+        banks.chunks[0] = d.LA;
+        banks.thr16[0] = feedback_threshold(cfg->s[0]);
+        for (int l = 0; l < layers; ++l) {
+            banks.bank[l + 1] = s->message_ta_state[l];
+            banks.rows[l + 1] = w.clause_X[l];
+            banks.chunks[l + 1] = d.MC;
+            banks.thr16[l + 1] = feedback_threshold(cfg->s[l + 1]);
+        }
+        hipLaunchKernelGGL(k_fit_feedback, dim3(blocks_for(d.C, cpb)), dim3(TPB), (size_t)cpb * d.K * 4, st, banks,
+                           s->clause_weights, sum_now, sum_next, encoded_Y + (int64_t)ex * d.K, d.C, d.B, d.K,
+                           cfg->threshold, cfg->negative_clauses, cfg->boost_true_positive_feedback,
+                           cfg->max_included_literals, q_thr, key.k0, key.k1, step, w.clause_node, w.n_incl, cpb);
         if (int rc = check_launch("fit_feedback")) return rc;
     }
     return GTM_OK;
@@ -1284,6 +1390,12 @@ int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *st
             return fit_on_tiles(d, cfg, graphs, state, tg, w, encoded_Y, first_example, n_examples, first_step, h_n,
                                 h_base, st);
         }
+    }
+    if (cfg->depth > 1 && graphs->tiles && graphs->number_of_node_types >= 1 && !getenv("GTM_NO_DEEP_FIT")) {
+        TileGeom tg = geometry_for(cfg, graphs, d.K);
+        if (tg.ok && tg.slot_words <= 64 && cfg->max_nodes <= 2048)  // one lane per word of the graph's nodes
+            return fit_deep_on_tiles(d, cfg, graphs, state, tg, w, encoded_Y, first_example, n_examples, first_step, h_n,
+                                     h_base, st);
     }
     for (int i = 0; i < n_examples; ++i) {
         int ex = first_example + i;

@@ -253,8 +253,7 @@ class CommonTsetlinMachine:
         self._init_fit(graphs, encoded_Y, incremental)
         dg = self._train_graphs
         cfg = self._config(max(dg.max_nodes, 1))
-        if self.depth == 1:
-            dg.ensure_tiles(cfg)
+        dg.ensure_tiles(cfg)
         need = _abi.lib.gtm_fit_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc))
         ws = self._workspace_of(need)
         for _ in range(epochs):

@@ -159,12 +159,12 @@ def test_training_operators(shape, boost, max_included):
 @pytest.mark.parametrize("tiles", [False, True], ids=["plain", "tiles"])
 def test_fit_trajectory_bit_exact(shape, tiles):
     """gtm_fit over a few epochs leaves exactly the oracle's automata and weights
-    (with tiles, depth-1 models take the two-kernel fused step)."""
+    (with tiles, the fused training steps run instead of one launch per operator)."""
     from tests.gpu_harness import Device
 
     graphs, cfg, model = build(shape, 0.02)
     dev = Device(model, graphs)
-    if tiles and model.depth == 1:
+    if tiles:
         assert dev.build_tiles()
     rng = np.random.default_rng(shape["seed"] + 100)
     Y = o.encode_labels(rng.integers(0, cfg.classes, size=graphs.number_of_graphs), cfg.classes, cfg.threshold)
@@ -302,6 +302,39 @@ def test_tile_scoring_with_message_layers(shape, message_density):
     assert np.array_equal(dev.score(0, G, 3), plain)
     if G > 7:
         assert np.array_equal(dev.score(3, G - 5, 5), plain[3:G - 2])
+
+
+@pytest.mark.parametrize("shape", DEEP_TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
+@pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 9, 5)])
+def test_fused_fit_with_message_layers(shape, boost, max_included, state_bits):
+    """The fused training step of models with message layers == the oracle: automata of every
+    bank and the weights after each of two epochs."""
+    from tests.gpu_harness import Device
+
+    g = dict(shape["g"])
+    if "sizes" not in g:
+        g["n_graphs"] = min(g["n_graphs"], 12)
+    graphs = helpers.random_graphs(shape["seed"], **g)
+    m = dict(shape["m"])
+    depth = m.pop("depth")
+    cfg = helpers.oracle_config(graphs, **m, depth=depth, T=30, boost=boost, max_included=max_included,
+                                state_bits=state_bits)
+    model = helpers.random_model(shape["seed"], cfg, depth, s=(3.0, 2.0, 1.5)[:depth],
+                                 include_density=shape.get("density", 0.02), message_density=0.02)
+    dev = Device(model, graphs)
+    assert dev.build_tiles()
+    rng = np.random.default_rng(shape["seed"])
+    G = graphs.number_of_graphs
+    Y = o.encode_labels(rng.integers(0, cfg.classes, size=G), cfg.classes, cfg.threshold)
+    for epoch in range(2):
+        o.fit(model, graphs, Y)
+        dev.fit(Y, 0, G, epoch * G)
+        ta, banks, w = dev.download()
+        assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
+        assert np.array_equal(ta, model.ta_state), "layer-0 automata after epoch %d" % epoch
+        for layer in range(depth - 1):
+            assert np.array_equal(banks[layer], model.message_ta_state[layer]), "bank %d epoch %d" % (layer, epoch)
+    assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
 
 
 @pytest.mark.parametrize("shape", TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
