@@ -61,17 +61,22 @@ __global__ __launch_bounds__(64) void k_fit_message_rows(const uint32_t *__restr
 }
 
 // K2 (+ K6 + K7 when `finish`) for one graph and one message layer.  Each wave
-// takes clauses in turn; lane L holds word L of the clause's truth over the
-// graph's nodes, starting from the layer before.  The clause's include words
-// come from the top bit plane of the layer's automaton bank; message literal
-// l < M reads row l, literal l >= M the complement of row l - M
-// (kernels.py:505-527; positions past the graph's nodes are already 0 in the
-// incoming truth).
+// takes clauses in turn; lane L ends up with word L of the clause's truth over
+// the graph's nodes, starting from the layer before.  The clause's include words
+// come from the top bit plane of the layer's automaton bank.  Two ways to apply
+// them, chosen per clause by the number of memory round trips each needs:
+//   by literal  every included message literal l < M ANDs row l, every l >= M the
+//               complement of row l - M (kernels.py:505-527; positions past the
+//               graph's nodes are already 0 in the incoming truth);
+//   by node     64 nodes at a time, lane = node: the node's packed message words
+//               against the clause's include words, (include & ~words) == 0, for
+//               the blocks of nodes where the clause is still true.
 __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
-    const uint32_t *__restrict__ rows, int row_words, int words, int n_nodes, int M, int C, int MC, int B, int K,
-    int NC, uint32_t filter, const uint32_t *__restrict__ bank, const int32_t *__restrict__ weights, uint32_t k0,
-    uint32_t k1, uint32_t step, int finish, const uint32_t *__restrict__ bitmap_in, uint32_t *__restrict__ bitmap_out,
-    int32_t *__restrict__ n_incl, int32_t *__restrict__ clause_node, int32_t *class_sum) {
+    const uint32_t *__restrict__ rows, int row_words, const uint32_t *__restrict__ clause_X, int words, int n_nodes,
+    int M, int C, int MC, int B, int K, int NC, uint32_t filter, const uint32_t *__restrict__ bank,
+    const int32_t *__restrict__ weights, uint32_t k0, uint32_t k1, uint32_t step, int finish,
+    const uint32_t *__restrict__ bitmap_in, uint32_t *__restrict__ bitmap_out, int32_t *__restrict__ n_incl,
+    int32_t *__restrict__ clause_node, int32_t *class_sum) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -82,33 +87,72 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
     for (int c = blockIdx.x * WAVES + wave; c < C; c += gridDim.x * WAVES) {
         const uint32_t *inc = bank + (int64_t)c * MC * B + (B - 1);
         uint32_t acc = active ? bitmap_in[(int64_t)c * NC + lane] : 0u;
+        // words of the truth row that are not zero, and the blocks of 64 nodes they cover
+        const unsigned long long live_words = __ballot(acc != 0);
+        const int live_blocks = __popcll((live_words | (live_words >> 1)) & 0x5555555555555555ull);
         int included = 0;
         for (int w0 = 0; w0 < MC; w0 += 64) {
             uint32_t mine = w0 + lane < MC ? inc[(int64_t)(w0 + lane) * B] : 0u;
             if (w0 + lane == MC - 1) mine &= filter;
             unsigned long long nonzero = __ballot(mine != 0);
-            included += __popc(mine);
+            int here = __popc(mine);
+            included += here;
             // a clause that is false everywhere stays false: only its include count is needed
-            if (__ballot(acc != 0) == 0) continue;
-            while (nonzero) {
-                const int wl = __ffsll((long long)nonzero) - 1;
-                nonzero &= nonzero - 1;
-                uint32_t m = __builtin_amdgcn_readlane(mine, wl);
-                const int base = (w0 + wl) << 5;
-                while (m) {
-                    uint32_t r[8];
+            if (live_words == 0 || nonzero == 0) continue;
+            for (int off = 32; off > 0; off >>= 1) here += __shfl_xor(here, off);
+            const int trips_by_literal = (here + 7) >> 3;
+            const int trips_by_node = live_blocks * ((__popcll(nonzero) + 7) >> 3);
+            if (trips_by_node < trips_by_literal) {
+                uint32_t result = 0;  // lane L: word L of the clause's truth after these include words
+                for (int nb = 0; nb * 2 < words; ++nb) {
+                    if (((live_words >> (nb * 2)) & 3ull) == 0) continue;
+                    const int node = nb * 64 + lane;
+                    // this node's bit of the running truth (lane = node)
+                    const uint32_t lo = __builtin_amdgcn_readlane(acc, nb * 2);
+                    const uint32_t hi = nb * 2 + 1 < 64 ? __builtin_amdgcn_readlane(acc, (nb * 2 + 1) & 63) : 0u;
+                    bool ok = ((lane < 32 ? lo >> lane : hi >> (lane - 32)) & 1u) != 0;
+                    const uint32_t *x = clause_X + (int64_t)(node < n_nodes ? node : 0) * MC + w0;
+                    unsigned long long todo = nonzero;
+                    uint32_t violated = 0;
+                    while (todo) {
+                        uint32_t xs[8], is[8];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) {
-                        // wave-uniform: the literal, its row, whether it is negated; unused slots read row 0 and give all ones
-                        const bool used = m != 0;
-                        const int lit = used ? base + __builtin_ctz(m) : 0;
-                        m &= m - 1;
-                        const bool negated = lit >= M;
-                        const uint32_t flip = negated ? 0xFFFFFFFFu : 0u, fill = used ? 0u : 0xFFFFFFFFu;
-                        r[u] = (col[(int64_t)(negated ? lit - M : lit) * row_words] ^ flip) | fill;
+                        for (int u = 0; u < 8; ++u) {
+                            const int wl = todo ? __ffsll((long long)todo) - 1 : 0;
+                            is[u] = todo ? __builtin_amdgcn_readlane(mine, wl) : 0u;
+                            todo &= todo - 1;
+                            xs[u] = x[wl];
+                        }
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) violated |= is[u] & ~xs[u];
                     }
+                    ok = ok && violated == 0;
+                    const unsigned long long truth = __ballot(ok);
+                    if (lane == nb * 2) result = (uint32_t)truth;
+                    if (lane == nb * 2 + 1) result = (uint32_t)(truth >> 32);
+                }
+                acc = result;
+            } else {
+                while (nonzero) {
+                    const int wl = __ffsll((long long)nonzero) - 1;
+                    nonzero &= nonzero - 1;
+                    uint32_t m = __builtin_amdgcn_readlane(mine, wl);
+                    const int base = (w0 + wl) << 5;
+                    while (m) {
+                        uint32_t r[8];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) acc &= r[u];
+                        for (int u = 0; u < 8; ++u) {
+                            // wave-uniform: the literal, its row, whether it is negated; unused slots read row 0 and give all ones
+                            const bool used = m != 0;
+                            const int lit = used ? base + __builtin_ctz(m) : 0;
+                            m &= m - 1;
+                            const bool negated = lit >= M;
+                            const uint32_t flip = negated ? 0xFFFFFFFFu : 0u, fill = used ? 0u : 0xFFFFFFFFu;
+                            r[u] = (col[(int64_t)(negated ? lit - M : lit) * row_words] ^ flip) | fill;
+                        }
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) acc &= r[u];
+                    }
                 }
             }
         }
