@@ -60,6 +60,102 @@ __global__ __launch_bounds__(64) void k_fit_message_rows(const uint32_t *__restr
     }
 }
 
+// ---- messages in three steps, for MESSAGE_SIZE a multiple of 32 -------------
+//
+// A message (kernels.py:565-588) factors: the bits a node sends are the OR of
+// the hypervector bits of the clauses true at it, and what a neighbour receives
+// along an edge of type t is that bit vector rotated by t.  So:
+//   k_fit_node_messages  sent[n] = OR over clauses true at n of their bits
+//   k_fit_edge_messages  got[dst] |= rotate(sent[src], type) for every edge
+//   k_fit_pack_messages  node-major packed literals (got | ~got) and the
+//                        literal-major rows of got; clears sent and got
+// which needs (true pairs x MESSAGE_BITS) LDS atomics and (edges x words)
+// global ones instead of (true pairs x edges x MESSAGE_BITS x 2) global ones.
+
+constexpr int FIT_NODE_MESSAGES_BLOCK = 256;
+constexpr int FIT_NODE_MESSAGES_CLAUSES = 1024;  // clauses per block
+
+// grid (node words in use, ceil(C / FIT_NODE_MESSAGES_CLAUSES)); dynamic LDS 32 * MW words
+__global__ __launch_bounds__(FIT_NODE_MESSAGES_BLOCK) void k_fit_node_messages(
+    const uint32_t *__restrict__ bitmap, int C, int NC, int n_nodes, const uint32_t *__restrict__ hv, int MB, int MW,
+    uint32_t *sent) {
+    extern __shared__ uint32_t vec[];  // [32 nodes][MW]
+    const int tid = threadIdx.x;
+    const int nw = blockIdx.x;
+    for (int i = tid; i < 32 * MW; i += FIT_NODE_MESSAGES_BLOCK) vec[i] = 0u;
+    __syncthreads();
+    const int c_end = min(C, (int)(blockIdx.y + 1) * FIT_NODE_MESSAGES_CLAUSES);
+    const uint32_t valid = n_nodes - nw * 32 >= 32 ? 0xFFFFFFFFu : (1u << (n_nodes - nw * 32)) - 1u;
+    for (int c = blockIdx.y * FIT_NODE_MESSAGES_CLAUSES + tid; c < c_end; c += FIT_NODE_MESSAGES_BLOCK) {
+        uint32_t word = bitmap[(int64_t)c * NC + nw] & valid;
+        while (word) {
+            const int n = __ffs(word) - 1;
+            word &= word - 1;
+            for (int j = 0; j < MB; ++j) {
+                const uint32_t h = hv[(int64_t)c * MB + j];
+                atomicOr(&vec[n * MW + (h >> 5)], 1u << (h & 31));
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < 32 * MW; i += FIT_NODE_MESSAGES_BLOCK) {
+        const int n = nw * 32 + i / MW;
+        if (vec[i] != 0u && n < n_nodes) atomicOr(&sent[(int64_t)n * MW + (i % MW)], vec[i]);
+    }
+}
+
+// One thread per (node, word of the rotated vector): for each of the node's
+// out-edges, word j of rotate(sent[node], type) ORed into got[destination].
+__global__ void k_fit_edge_messages(const uint32_t *__restrict__ sent, int n_nodes, int MW,
+                                    const uint32_t *__restrict__ n_edges, const uint32_t *__restrict__ edge_index,
+                                    const uint32_t *__restrict__ edge, uint32_t *got) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)n_nodes * MW) return;
+    const int n = (int)(i / MW), j = (int)(i % MW);
+    const uint32_t *v = sent + (int64_t)n * MW;
+    const uint32_t ne = n_edges[n];
+    const int64_t e0 = edge_index[n];
+    const uint32_t M = (uint32_t)MW * 32u;
+    for (uint32_t e = 0; e < ne; ++e) {
+        const uint32_t dst = edge[(e0 + e) * 2], shift = edge[(e0 + e) * 2 + 1] % M;
+        // bit p of the result is bit (p - shift) mod M of v
+        const int q = (int)(shift >> 5), r = (int)(shift & 31u);
+        const int a = (j - q + MW) % MW, below = (a - 1 + MW) % MW;
+        const uint32_t word = r ? (v[a] << r) | (v[below] >> (32 - r)) : v[a];
+        if (word) atomicOr(&got[(int64_t)dst * MW + j], word);
+    }
+}
+
+// One wave per (word j of the message vectors, 64 nodes), lane = node: writes
+// the node's packed literal words j (messages) and MW + j (their negations),
+// the literal-major rows 32 j .. 32 j + 31 for these 64 nodes, and clears the
+// node's words of sent and got for the next use.  clause_X is [node][2 * MW].
+__global__ __launch_bounds__(64) void k_fit_pack_messages(uint32_t *sent, uint32_t *got, int n_nodes, int MW,
+                                                           int row_words, uint32_t *__restrict__ clause_X,
+                                                           uint32_t *__restrict__ rows) {
+    const int lane = threadIdx.x;
+    const int j = blockIdx.x, nb = blockIdx.y;
+    const int n = nb * 64 + lane;
+    uint32_t word = 0u;
+    if (n < n_nodes) {
+        word = got[(int64_t)n * MW + j];
+        got[(int64_t)n * MW + j] = 0u;
+        sent[(int64_t)n * MW + j] = 0u;
+        clause_X[(int64_t)n * 2 * MW + j] = word;
+        clause_X[(int64_t)n * 2 * MW + MW + j] = ~word;
+    }
+    unsigned long long mine = 0;
+#pragma unroll
+    for (int b = 0; b < 32; ++b) {
+        const unsigned long long column = __ballot((word >> b) & 1u);
+        if (lane == b) mine = column;
+    }
+    if (lane < 32) {
+        rows[(int64_t)(j * 32 + lane) * row_words + nb * 2] = (uint32_t)mine;
+        rows[(int64_t)(j * 32 + lane) * row_words + nb * 2 + 1] = (uint32_t)(mine >> 32);
+    }
+}
+
 // K2 (+ K6 + K7 when `finish`) for one graph and one message layer.  Each wave
 // takes clauses in turn; lane L ends up with word L of the clause's truth over
 // the graph's nodes, starting from the layer before.  The clause's include words

@@ -525,6 +525,7 @@ struct FitWs {
     int32_t *update;                        // [K][C]
     uint32_t *message_rows;                 // [M][message_row_words] literal-major messages of one layer (depth > 1)
     int message_row_words;
+    uint32_t *sent, *got;                   // [max_nodes][M / 32] bit vectors sent / received per node (depth > 1)
     size_t bytes;
 };
 
@@ -549,6 +550,9 @@ FitWs carve_fit(const Dims &d, const gtm_config *cfg, char *base) {
     w.update = (int32_t *)take((size_t)d.K * d.C * 4);
     w.message_row_words = 2 * ((cfg->max_nodes + 63) / 64);
     w.message_rows = cfg->depth > 1 ? (uint32_t *)take((size_t)d.M * w.message_row_words * 4) : nullptr;
+    const size_t vector_bytes = (size_t)cfg->max_nodes * ((d.M + 31) / 32) * 4;
+    w.sent = cfg->depth > 1 ? (uint32_t *)take(vector_bytes) : nullptr;
+    w.got = cfg->depth > 1 ? (uint32_t *)take(vector_bytes) : nullptr;
     w.bytes = off;
     return w;
 }
@@ -1269,6 +1273,20 @@ int fit_deep_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g,
     int eval_blocks = (d.C + 2 * waves_per_block - 1) / (2 * waves_per_block);
     if (eval_blocks > 1024) eval_blocks = 1024;
     static thread_local size_t lds_set = 0;
+    // Messages by per-node bit vectors (fit_deep.h) when MESSAGE_SIZE is a multiple of 32 and the
+    // graph is big enough for the saved atomics to pay for the extra pass.
+    const int MW = (d.M + 31) / 32;
+    const bool factored = d.M % 32 == 0 && (size_t)32 * MW * 4 <= 48 * 1024;
+    const char *fm = getenv("GTM_FIT_FACTOR_MIN");  // clauses x nodes from which that path is taken (tuning aid)
+    const int64_t factor_min = fm ? atoll(fm) : 32768;
+    if (factored) {
+        const int64_t vector_words = (int64_t)cfg->max_nodes * MW;
+        for (uint32_t *p : {w.sent, w.got}) {
+            hipLaunchKernelGGL(k_fill_i32, dim3(blocks_for(vector_words, TPB)), dim3(TPB), 0, st, (int32_t *)p,
+                               vector_words, 0);
+            if (int rc = check_launch("fill")) return rc;
+        }
+    }
     for (int i = 0; i < n_examples; ++i) {
         const int ex = first_example + i;
         const int n_nodes = (int)h_n[i];
@@ -1296,23 +1314,42 @@ int fit_deep_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g,
         const int words = n_nodes == 0 ? 1 : (n_nodes - 1) / 32 + 1;
         for (int l = 0; l < layers; ++l) {
             uint32_t *cx = w.clause_X[l];
-            if (n_nodes > 0) {
-                const int64_t message_words = (int64_t)n_nodes * d.MC;
-                hipLaunchKernelGGL(k_messages_blank, dim3(blocks_for(message_words, TPB)), dim3(TPB), 0, st, cx,
-                                   message_words, d.MC, d.M);
-                if (int rc = check_launch("messages_blank")) return rc;
-                if (g->total_edges > 0) {
-                    const int64_t pairs = (int64_t)d.C * n_nodes;
-                    hipLaunchKernelGGL(k_fit_scatter_messages, dim3(blocks_for(pairs, FIT_SCATTER_BLOCK)),
-                                       dim3(FIT_SCATTER_BLOCK), 0, st, cur, d.C, d.NC, n_nodes, s->hypervectors, d.MB,
-                                       d.M, d.MC, g->number_of_graph_node_edges + h_base[i], g->edge_index + h_base[i],
-                                       g->edge, cx);
-                    if (int rc = check_launch("fit_scatter_messages")) return rc;
+            if (factored && (int64_t)d.C * n_nodes >= factor_min) {
+                if (n_nodes > 0) {
+                    hipLaunchKernelGGL(k_fit_node_messages,
+                                       dim3(words, (d.C + FIT_NODE_MESSAGES_CLAUSES - 1) / FIT_NODE_MESSAGES_CLAUSES),
+                                       dim3(FIT_NODE_MESSAGES_BLOCK), (size_t)32 * MW * 4, st, cur, d.C, d.NC, n_nodes,
+                                       s->hypervectors, d.MB, MW, w.sent);
+                    if (int rc = check_launch("fit_node_messages")) return rc;
+                    if (g->total_edges > 0) {
+                        hipLaunchKernelGGL(k_fit_edge_messages, dim3(blocks_for((int64_t)n_nodes * MW, TPB)), dim3(TPB), 0,
+                                           st, w.sent, n_nodes, MW, g->number_of_graph_node_edges + h_base[i],
+                                           g->edge_index + h_base[i], g->edge, w.got);
+                        if (int rc = check_launch("fit_edge_messages")) return rc;
+                    }
                 }
+                hipLaunchKernelGGL(k_fit_pack_messages, dim3(MW, w.message_row_words / 2), dim3(64), 0, st, w.sent, w.got,
+                                   n_nodes, MW, w.message_row_words, cx, w.message_rows);
+                if (int rc = check_launch("fit_pack_messages")) return rc;
+            } else {
+                if (n_nodes > 0) {
+                    const int64_t message_words = (int64_t)n_nodes * d.MC;
+                    hipLaunchKernelGGL(k_messages_blank, dim3(blocks_for(message_words, TPB)), dim3(TPB), 0, st, cx,
+                                       message_words, d.MC, d.M);
+                    if (int rc = check_launch("messages_blank")) return rc;
+                    if (g->total_edges > 0) {
+                        const int64_t pairs = (int64_t)d.C * n_nodes;
+                        hipLaunchKernelGGL(k_fit_scatter_messages, dim3(blocks_for(pairs, FIT_SCATTER_BLOCK)),
+                                           dim3(FIT_SCATTER_BLOCK), 0, st, cur, d.C, d.NC, n_nodes, s->hypervectors, d.MB,
+                                           d.M, d.MC, g->number_of_graph_node_edges + h_base[i],
+                                           g->edge_index + h_base[i], g->edge, cx);
+                        if (int rc = check_launch("fit_scatter_messages")) return rc;
+                    }
+                }
+                hipLaunchKernelGGL(k_fit_message_rows, dim3((d.M + 31) / 32, w.message_row_words / 2), dim3(64), 0, st,
+                                   cx, n_nodes, d.M, d.MC, w.message_row_words, w.message_rows);
+                if (int rc = check_launch("fit_message_rows")) return rc;
             }
-            hipLaunchKernelGGL(k_fit_message_rows, dim3((d.M + 31) / 32, w.message_row_words / 2), dim3(64), 0, st, cx,
-                               n_nodes, d.M, d.MC, w.message_row_words, w.message_rows);
-            if (int rc = check_launch("fit_message_rows")) return rc;
             hipLaunchKernelGGL(k_fit_message_eval, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), 0, st, w.message_rows,
                                w.message_row_words, cx, words, n_nodes, d.M, d.C, d.MC, d.B, d.K, d.NC, d.mfilter,
                                s->message_ta_state[l], s->clause_weights, key.k0, key.k1, step, l == layers - 1 ? 1 : 0,

@@ -306,10 +306,15 @@ def test_tile_scoring_with_message_layers(shape, message_density):
 
 @pytest.mark.parametrize("shape", DEEP_TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
 @pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 9, 5)])
-def test_fused_fit_with_message_layers(shape, boost, max_included, state_bits):
+@pytest.mark.parametrize("messages", ["by-node-vectors", "by-scatter"])
+def test_fused_fit_with_message_layers(shape, boost, max_included, state_bits, messages, monkeypatch):
     """The fused training step of models with message layers == the oracle: automata of every
-    bank and the weights after each of two epochs."""
+    bank and the weights after each of two epochs.  Both ways of building the messages (per-node
+    bit vectors rotated along the edges, taken when MESSAGE_SIZE is a multiple of 32; one scatter
+    per true clause, node and edge) are forced in turn."""
     from tests.gpu_harness import Device
+
+    monkeypatch.setenv("GTM_FIT_FACTOR_MIN", "0" if messages == "by-node-vectors" else str(1 << 60))
 
     g = dict(shape["g"])
     if "sizes" not in g:
