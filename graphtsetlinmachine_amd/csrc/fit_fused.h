@@ -17,6 +17,8 @@
 #pragma once
 
 constexpr int FIT_EVAL_BLOCK = 256;
+constexpr int FIT_WALK_ALL = 40;     // clauses with at most this many literals AND all their rows
+constexpr int FIT_FILTER_ROWS = 16;  // rows the others AND before testing nodes
 
 struct FitGraph {
     int tile;        // tile holding the graph
@@ -105,12 +107,14 @@ __device__ __forceinline__ void fit_clause_tail(uint32_t v, int lane, int words,
 // LDS reads in flight at a time.  STAGE = false reads the rows from the tile
 // in global memory instead (graphs whose rows do not fit in LDS).  `finish` = 0
 // (models with message layers) stops after the bitmap and the include counts.
+// X_rows: the graph's node-major literal words (its first node's row).
 template <bool STAGE>
 __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
     const uint32_t *__restrict__ tiles, TileGeom tg, FitGraph fg, int n_nodes, int literals, int n_types, int C, int LA,
     int B, int K, int NC, uint32_t filter, const uint32_t *__restrict__ bank, const int32_t *__restrict__ weights,
-    uint32_t k0, uint32_t k1, uint32_t step, int finish, uint32_t *__restrict__ bitmap, int32_t *__restrict__ n_incl,
-    int32_t *__restrict__ clause_node, int32_t *class_sum) {
+    uint32_t k0, uint32_t k1, uint32_t step, int finish, const uint32_t *__restrict__ X_rows,
+    uint32_t *__restrict__ bitmap, int32_t *__restrict__ n_incl, int32_t *__restrict__ clause_node,
+    int32_t *class_sum) {
     extern __shared__ uint32_t rows_lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -145,20 +149,34 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
     int partial = 0;  // lane k < K: this wave's contribution to class k
     for (int c = blockIdx.x * WAVES + wave; c < C; c += gridDim.x * WAVES) {
         const uint32_t *inc = bank + (int64_t)c * LA * B + (B - 1);
-        uint32_t acc = active ? col[(int64_t)(literals + c % n_types) * stride] : 0u;
-        int included = 0;
-        for (int w0 = 0; w0 < LA; w0 += 64) {
-            // lane w fetches include word w0 + w: one memory latency for up to 64 words
+        // lane w fetches include word w0 + w: one memory latency for up to 64 words
+        auto include_words = [&](int w0) {
             uint32_t mine = w0 + lane < LA ? inc[(int64_t)(w0 + lane) * B] : 0u;
             if (w0 + lane == LA - 1) mine &= filter;
+            return mine;
+        };
+        int included = 0;
+        uint32_t first_words = 0;
+        for (int w0 = 0; w0 < LA; w0 += 64) {
+            const uint32_t mine = include_words(w0);
+            if (w0 == 0) first_words = mine;
+            included += __popc(mine);
+        }
+        for (int off = 32; off > 0; off >>= 1) included += __shfl_xor(included, off);
+        // A clause with many literals ANDs the rows of its first FIT_FILTER_ROWS only and then tests the
+        // few nodes that are left against its whole include mask on the nodes' own literal words.
+        const bool filter_only = included > FIT_WALK_ALL && n_nodes > 0;
+        int budget = filter_only ? FIT_FILTER_ROWS : 0x7FFFFFFF;
+        uint32_t acc = active ? col[(int64_t)(literals + c % n_types) * stride] : 0u;
+        for (int w0 = 0; w0 < LA && budget > 0; w0 += 64) {
+            const uint32_t mine = w0 == 0 ? first_words : include_words(w0);
             unsigned long long nonzero = __ballot(mine != 0);
-            included += __popc(mine);  // summed over the lanes below
-            while (nonzero) {
+            while (nonzero && budget > 0) {
                 const int wl = __ffsll((long long)nonzero) - 1;
                 nonzero &= nonzero - 1;
                 uint32_t m = __builtin_amdgcn_readlane(mine, wl);
                 const int base = (w0 + wl) << 5;
-                while (m) {
+                while (m && budget > 0) {
                     int row[8];
 #pragma unroll
                     for (int u = 0; u < 8; ++u) {
@@ -170,11 +188,39 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
                     for (int u = 0; u < 8; ++u) r[u] = col[(int64_t)row[u] * stride];
 #pragma unroll
                     for (int u = 0; u < 8; ++u) acc &= r[u];
+                    budget -= 8;
                 }
             }
         }
-        for (int off = 32; off > 0; off >>= 1) included += __shfl_xor(included, off);
-        const uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
+        uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
+        if (filter_only) {
+            // lane L holds nodes 32 L .. 32 L + 31; every lane tests one of its surviving nodes per trip
+            uint32_t todo = v;
+            while (__ballot(todo != 0) != 0) {
+                const bool has = todo != 0;
+                const int b = has ? __ffs(todo) - 1 : 0;
+                todo &= todo - 1;
+                const uint32_t *x = X_rows + (int64_t)(has ? lane * 32 + b : 0) * LA;
+                uint32_t violated = 0;
+                for (int w0 = 0; w0 < LA; w0 += 64) {
+                    const uint32_t mine = w0 == 0 ? first_words : include_words(w0);
+                    unsigned long long nonzero = __ballot(mine != 0);
+                    while (nonzero) {
+                        uint32_t xs[8], is[8];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) {
+                            const int wl = nonzero ? __ffsll((long long)nonzero) - 1 : 0;
+                            is[u] = nonzero ? __builtin_amdgcn_readlane(mine, wl) : 0u;
+                            nonzero &= nonzero - 1;
+                            xs[u] = x[w0 + wl];
+                        }
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) violated |= is[u] & ~xs[u];
+                    }
+                }
+                if (has && violated) v &= ~(1u << b);
+            }
+        }
         if (lane == 0) n_incl[c] = included;
         fit_clause_tail(v, lane, fg.words, NC, n_nodes, c, C, K, weights, k0, k1, step, finish != 0,
                         bitmap + (int64_t)c * NC, clause_node, class_sum, &partial);

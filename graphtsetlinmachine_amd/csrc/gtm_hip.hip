@@ -1230,11 +1230,13 @@ int fit_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, cons
         if (stage)
             hipLaunchKernelGGL(k_fit_eval<true>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), lds, st, g->tiles, tg, fg,
                                (int)h_n[i], cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
-                               s->clause_weights, key.k0, key.k1, step, 1, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
+                               s->clause_weights, key.k0, key.k1, step, 1, g->X + (int64_t)h_base[i] * d.LA, w.bitmap_a, w.n_incl,
+                               w.clause_node, sum_now);
         else
             hipLaunchKernelGGL(k_fit_eval<false>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), 0, st, g->tiles, tg, fg,
                                (int)h_n[i], cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
-                               s->clause_weights, key.k0, key.k1, step, 1, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
+                               s->clause_weights, key.k0, key.k1, step, 1, g->X + (int64_t)h_base[i] * d.LA, w.bitmap_a, w.n_incl,
+                               w.clause_node, sum_now);
         if (int rc = check_launch("fit_eval")) return rc;
         if (i < Profile::MAX) profile_stop(st);
         FitBanks banks{};
@@ -1304,11 +1306,13 @@ int fit_deep_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g,
         if (stage)
             hipLaunchKernelGGL(k_fit_eval<true>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), lds, st, g->tiles, tg, fg,
                                n_nodes, cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
-                               s->clause_weights, key.k0, key.k1, step, 0, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
+                               s->clause_weights, key.k0, key.k1, step, 0, g->X + (int64_t)h_base[i] * d.LA, w.bitmap_a, w.n_incl,
+                               w.clause_node, sum_now);
         else
             hipLaunchKernelGGL(k_fit_eval<false>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), 0, st, g->tiles, tg, fg,
                                n_nodes, cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
-                               s->clause_weights, key.k0, key.k1, step, 0, w.bitmap_a, w.n_incl, w.clause_node, sum_now);
+                               s->clause_weights, key.k0, key.k1, step, 0, g->X + (int64_t)h_base[i] * d.LA, w.bitmap_a, w.n_incl,
+                               w.clause_node, sum_now);
         if (int rc = check_launch("fit_eval")) return rc;
         uint32_t *cur = w.bitmap_a, *nxt = w.bitmap_b;
         const int words = n_nodes == 0 ? 1 : (n_nodes - 1) / 32 + 1;

@@ -373,6 +373,48 @@ def test_fused_fit_on_every_tile_geometry(shape, boost, max_included, state_bits
     assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
 
 
+@pytest.mark.parametrize("seed,g,m", [
+    (15, dict(n_graphs=10, max_nodes=361, min_nodes=300, hv_size=128, max_degree=0), dict(classes=10, clauses=60, depth=1)),
+    (18, dict(n_graphs=12, max_nodes=50, hv_size=256, n_symbols=12, node_types=("a", "b")), dict(classes=4, clauses=64, depth=1)),
+    (13, dict(n_graphs=20, max_nodes=16, min_nodes=9, hv_size=80), dict(classes=4, clauses=33, depth=1)),
+    (34, dict(n_graphs=8, max_nodes=200, min_nodes=100, hv_size=128, edge_types=("l", "r")),
+     dict(classes=3, clauses=40, depth=2, message_size=64)),
+    (38, dict(n_graphs=6, hv_size=2200, n_symbols=30, sizes=[3, 70, 0, 1, 33, 64]), dict(classes=2, clauses=30, depth=1)),
+], ids=lambda v: str(v) if isinstance(v, int) else "")
+@pytest.mark.parametrize("density", [0.3, 0.9])
+def test_fused_fit_with_many_literals(seed, g, m, density, monkeypatch):
+    """Clauses with many included literals (the training kernel ANDs a few of their rows and
+    tests the surviving nodes against the whole include mask) == the oracle."""
+    from tests.gpu_harness import Device
+
+    monkeypatch.setenv("GTM_NO_PERSISTENT_FIT", "1")
+    graphs = helpers.random_graphs(seed, **g)
+    m = dict(m)
+    depth = m.pop("depth")
+    cfg = helpers.oracle_config(graphs, **m, depth=depth, T=30)
+    model = helpers.random_model(seed, cfg, depth, s=(4.0, 2.0)[:depth], include_density=density, message_density=0.05)
+    # dense random includes are almost never satisfied: give a third of the clauses includes that one node satisfies
+    rng = np.random.default_rng(seed)
+    for c in range(0, cfg.clauses, 3):
+        node = int(rng.integers(graphs.number_of_nodes))
+        keep = graphs.X[node].copy()
+        keep[-1] &= np.uint32(cfg.filter)
+        model.ta_state[c, :, cfg.state_bits - 1] &= keep
+    dev = Device(model, graphs)
+    assert dev.build_tiles()
+    G = graphs.number_of_graphs
+    Y = o.encode_labels(rng.integers(0, cfg.classes, size=G), cfg.classes, cfg.threshold)
+    for epoch in range(2):
+        o.fit(model, graphs, Y)
+        dev.fit(Y, 0, G, epoch * G)
+        ta, banks, w = dev.download()
+        assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
+        assert np.array_equal(ta, model.ta_state), "layer-0 automata after epoch %d" % epoch
+        for layer in range(depth - 1):
+            assert np.array_equal(banks[layer], model.message_ta_state[layer]), "bank %d epoch %d" % (layer, epoch)
+    assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
+
+
 def test_fused_fit_with_an_empty_graph():
     from tests.gpu_harness import Device
 
