@@ -17,7 +17,8 @@
 #pragma once
 
 constexpr int FIT_EVAL_BLOCK = 256;
-constexpr int FIT_WALK_ALL = 40;     // clauses with at most this many literals AND all their rows
+constexpr int FIT_WALK_ALL = 40;      // clauses with at most this many literals AND all their rows (rows in global memory)
+constexpr int FIT_WALK_ALL_LDS = 512; // the same with the rows staged in LDS
 constexpr int FIT_FILTER_ROWS = 16;  // rows the others AND before testing nodes
 
 struct FitGraph {
@@ -107,13 +108,14 @@ __device__ __forceinline__ void fit_clause_tail(uint32_t v, int lane, int words,
 // LDS reads in flight at a time.  STAGE = false reads the rows from the tile
 // in global memory instead (graphs whose rows do not fit in LDS).  `finish` = 0
 // (models with message layers) stops after the bitmap and the include counts.
-// X_rows: the graph's node-major literal words (its first node's row).
+// X_rows: the graph's node-major literal words (its first node's row); order:
+// the literals sorted by how often they hold in the data set, rarest first.
 template <bool STAGE>
 __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
     const uint32_t *__restrict__ tiles, TileGeom tg, FitGraph fg, int n_nodes, int literals, int n_types, int C, int LA,
     int B, int K, int NC, uint32_t filter, const uint32_t *__restrict__ bank, const int32_t *__restrict__ weights,
     uint32_t k0, uint32_t k1, uint32_t step, int finish, const uint32_t *__restrict__ X_rows,
-    uint32_t *__restrict__ bitmap, int32_t *__restrict__ n_incl, int32_t *__restrict__ clause_node,
+    const uint32_t *__restrict__ order, uint32_t *__restrict__ bitmap, int32_t *__restrict__ n_incl, int32_t *__restrict__ clause_node,
     int32_t *class_sum) {
     extern __shared__ uint32_t rows_lds[];
     const int tid = threadIdx.x;
@@ -165,60 +167,93 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
         for (int off = 32; off > 0; off >>= 1) included += __shfl_xor(included, off);
         // A clause with many literals ANDs the rows of its first FIT_FILTER_ROWS only and then tests the
         // few nodes that are left against its whole include mask on the nodes' own literal words.
-        const bool filter_only = included > FIT_WALK_ALL && n_nodes > 0;
-        int budget = filter_only ? FIT_FILTER_ROWS : 0x7FFFFFFF;
+        const bool filter_only = included > (STAGE ? FIT_WALK_ALL_LDS : FIT_WALK_ALL) && n_nodes > 0;
         uint32_t acc = active ? col[(int64_t)(literals + c % n_types) * stride] : 0u;
-        for (int w0 = 0; w0 < LA && budget > 0; w0 += 64) {
-            const uint32_t mine = w0 == 0 ? first_words : include_words(w0);
-            unsigned long long nonzero = __ballot(mine != 0);
-            while (nonzero && budget > 0) {
-                const int wl = __ffsll((long long)nonzero) - 1;
-                nonzero &= nonzero - 1;
-                uint32_t m = __builtin_amdgcn_readlane(mine, wl);
-                const int base = (w0 + wl) << 5;
-                while (m && budget > 0) {
+        if (filter_only && order) {
+            // the first FIT_FILTER_ROWS included literals in `order` (the ones that hold least often in the data set)
+            int budget = FIT_FILTER_ROWS;
+            for (int r0 = 0; r0 < literals && budget > 0; r0 += 64) {
+                const int r = r0 + lane;
+                const uint32_t lit = r < literals ? order[r] : 0u;
+                uint32_t word = inc[(int64_t)(lit >> 5) * B];
+                if ((int)(lit >> 5) == LA - 1) word &= filter;
+                unsigned long long picked = __ballot(r < literals && ((word >> (lit & 31u)) & 1u));
+                while (picked && budget > 0) {
                     int row[8];
 #pragma unroll
                     for (int u = 0; u < 8; ++u) {
-                        row[u] = m ? base + __builtin_ctz(m) : ones_row;
-                        m &= m - 1;
+                        row[u] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
+                        picked &= picked - 1;
                     }
-                    uint32_t r[8];
+                    uint32_t r8[8];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) r[u] = col[(int64_t)row[u] * stride];
+                    for (int u = 0; u < 8; ++u) r8[u] = col[(int64_t)row[u] * stride];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) acc &= r[u];
+                    for (int u = 0; u < 8; ++u) acc &= r8[u];
                     budget -= 8;
+                }
+            }
+        } else {
+            int budget = filter_only ? FIT_FILTER_ROWS : 0x7FFFFFFF;
+            for (int w0 = 0; w0 < LA && budget > 0; w0 += 64) {
+                const uint32_t mine = w0 == 0 ? first_words : include_words(w0);
+                unsigned long long nonzero = __ballot(mine != 0);
+                while (nonzero && budget > 0) {
+                    const int wl = __ffsll((long long)nonzero) - 1;
+                    nonzero &= nonzero - 1;
+                    uint32_t m = __builtin_amdgcn_readlane(mine, wl);
+                    const int base = (w0 + wl) << 5;
+                    while (m && budget > 0) {
+                        int row[8];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) {
+                            row[u] = m ? base + __builtin_ctz(m) : ones_row;
+                            m &= m - 1;
+                        }
+                        uint32_t r[8];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) r[u] = col[(int64_t)row[u] * stride];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) acc &= r[u];
+                        budget -= 8;
+                    }
                 }
             }
         }
         uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
         if (filter_only) {
-            // lane L holds nodes 32 L .. 32 L + 31; every lane tests one of its surviving nodes per trip
-            uint32_t todo = v;
-            while (__ballot(todo != 0) != 0) {
-                const bool has = todo != 0;
-                const int b = has ? __ffs(todo) - 1 : 0;
-                todo &= todo - 1;
-                const uint32_t *x = X_rows + (int64_t)(has ? lane * 32 + b : 0) * LA;
-                uint32_t violated = 0;
-                for (int w0 = 0; w0 < LA; w0 += 64) {
-                    const uint32_t mine = w0 == 0 ? first_words : include_words(w0);
-                    unsigned long long nonzero = __ballot(mine != 0);
-                    while (nonzero) {
-                        uint32_t xs[8], is[8];
+            // Lane L holds nodes 32 L .. 32 L + 31.  The surviving nodes are walked on the scalar unit, 8 at
+            // a time; for each, lane w compares include word w with the node's literal word w (one
+            // coalesced load per node and 64 words), and a node with any violated word is cleared.
+            unsigned long long live = __ballot(v != 0);
+            while (live) {
+                const int L = __ffsll((long long)live) - 1;
+                live &= live - 1;
+                uint32_t word = __builtin_amdgcn_readlane(v, L);
+                uint32_t cleared = 0;
+                while (word) {
+                    int bit[8];
 #pragma unroll
-                        for (int u = 0; u < 8; ++u) {
-                            const int wl = nonzero ? __ffsll((long long)nonzero) - 1 : 0;
-                            is[u] = nonzero ? __builtin_amdgcn_readlane(mine, wl) : 0u;
-                            nonzero &= nonzero - 1;
-                            xs[u] = x[w0 + wl];
-                        }
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) violated |= is[u] & ~xs[u];
+                    for (int u = 0; u < 8; ++u) {
+                        bit[u] = word ? __builtin_ctz(word) : -1;
+                        word &= word - 1;
                     }
+                    uint32_t violated[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                    for (int w0 = 0; w0 < LA; w0 += 64) {
+                        const uint32_t mine = w0 == 0 ? first_words : include_words(w0);
+                        const bool in_row = w0 + lane < LA;
+                        uint32_t xs[8];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u)
+                            xs[u] = in_row ? X_rows[(int64_t)(L * 32 + (bit[u] < 0 ? 0 : bit[u])) * LA + w0 + lane] : 0xFFFFFFFFu;
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) violated[u] |= mine & ~xs[u];
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        if (bit[u] >= 0 && __ballot(violated[u] != 0) != 0) cleared |= 1u << bit[u];
                 }
-                if (has && violated) v &= ~(1u << b);
+                if (lane == L) v &= ~cleared;
             }
         }
         if (lane == 0) n_incl[c] = included;

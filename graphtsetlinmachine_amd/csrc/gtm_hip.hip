@@ -1203,6 +1203,7 @@ int fit_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, cons
                  const uint32_t *h_n, const uint32_t *h_base, hipStream_t st) {
     hipLaunchKernelGGL(k_fill_i32, dim3(1), dim3(TPB), 0, st, w.class_sum, (int64_t)d.K * 2, 0);
     if (int rc = check_launch("fill")) return rc;
+    const uint32_t *order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;  // literals, rarest first
     Key key = key_of(cfg);
     const int n_types = g->number_of_node_types;
     const int cpb = d.LA >= TPB ? 1 : TPB / d.LA;
@@ -1230,13 +1231,13 @@ int fit_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, cons
         if (stage)
             hipLaunchKernelGGL(k_fit_eval<true>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), lds, st, g->tiles, tg, fg,
                                (int)h_n[i], cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
-                               s->clause_weights, key.k0, key.k1, step, 1, g->X + (int64_t)h_base[i] * d.LA, w.bitmap_a, w.n_incl,
-                               w.clause_node, sum_now);
+                               s->clause_weights, key.k0, key.k1, step, 1, g->X + (int64_t)h_base[i] * d.LA, order, w.bitmap_a,
+                               w.n_incl, w.clause_node, sum_now);
         else
             hipLaunchKernelGGL(k_fit_eval<false>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), 0, st, g->tiles, tg, fg,
                                (int)h_n[i], cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
-                               s->clause_weights, key.k0, key.k1, step, 1, g->X + (int64_t)h_base[i] * d.LA, w.bitmap_a, w.n_incl,
-                               w.clause_node, sum_now);
+                               s->clause_weights, key.k0, key.k1, step, 1, g->X + (int64_t)h_base[i] * d.LA, order, w.bitmap_a,
+                               w.n_incl, w.clause_node, sum_now);
         if (int rc = check_launch("fit_eval")) return rc;
         if (i < Profile::MAX) profile_stop(st);
         FitBanks banks{};
@@ -1265,6 +1266,7 @@ int fit_deep_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g,
     if (int rc = check_launch("fill")) return rc;
     if (g->total_edges > 0 && (!g->number_of_graph_node_edges || !g->edge || !g->edge_index))
         return fail(GTM_ERR_INVALID, "graphs with edges need number_of_graph_node_edges, edge and edge_index");
+    const uint32_t *order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;  // literals, rarest first
     Key key = key_of(cfg);
     const int n_types = g->number_of_node_types;
     const int layers = cfg->depth - 1;
@@ -1306,13 +1308,13 @@ int fit_deep_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g,
         if (stage)
             hipLaunchKernelGGL(k_fit_eval<true>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), lds, st, g->tiles, tg, fg,
                                n_nodes, cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
-                               s->clause_weights, key.k0, key.k1, step, 0, g->X + (int64_t)h_base[i] * d.LA, w.bitmap_a, w.n_incl,
-                               w.clause_node, sum_now);
+                               s->clause_weights, key.k0, key.k1, step, 0, g->X + (int64_t)h_base[i] * d.LA, order, w.bitmap_a,
+                               w.n_incl, w.clause_node, sum_now);
         else
             hipLaunchKernelGGL(k_fit_eval<false>, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), 0, st, g->tiles, tg, fg,
                                n_nodes, cfg->literals, n_types, d.C, d.LA, d.B, d.K, d.NC, d.filter, s->ta_state,
-                               s->clause_weights, key.k0, key.k1, step, 0, g->X + (int64_t)h_base[i] * d.LA, w.bitmap_a, w.n_incl,
-                               w.clause_node, sum_now);
+                               s->clause_weights, key.k0, key.k1, step, 0, g->X + (int64_t)h_base[i] * d.LA, order, w.bitmap_a,
+                               w.n_incl, w.clause_node, sum_now);
         if (int rc = check_launch("fit_eval")) return rc;
         uint32_t *cur = w.bitmap_a, *nxt = w.bitmap_b;
         const int words = n_nodes == 0 ? 1 : (n_nodes - 1) / 32 + 1;
