@@ -156,7 +156,7 @@ __global__ __launch_bounds__(64) void k_fit_pack_messages(uint32_t *sent, uint32
     }
 }
 
-// K2 (+ K6 + K7 when `finish`) for one graph and one message layer.  Each wave
+// K2 (+ K6 + K7 when `finish`) for one graph and one message layer.  Each block
 // takes clauses in turn; lane L ends up with word L of the clause's truth over
 // the graph's nodes, starting from the layer before.  The clause's include words
 // come from the top bit plane of the layer's automaton bank.  Two ways to apply
@@ -173,6 +173,9 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
     const int32_t *__restrict__ weights, uint32_t k0, uint32_t k1, uint32_t step, int finish,
     const uint32_t *__restrict__ bitmap_in, uint32_t *__restrict__ bitmap_out, int32_t *__restrict__ n_incl,
     int32_t *__restrict__ clause_node, int32_t *class_sum) {
+    // The waves of a block share a clause: by node they split its blocks of 64 nodes and hand
+    // their words to wave 0 through LDS; by literal wave 0 works alone.  Wave 0 ends the clause.
+    __shared__ uint32_t handed[64];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -180,12 +183,9 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
     const bool active = lane < words;
     const uint32_t *col = rows + (active ? lane : 0);
     int partial = 0;
-    for (int c = blockIdx.x * WAVES + wave; c < C; c += gridDim.x * WAVES) {
+    for (int c = blockIdx.x; c < C; c += gridDim.x) {
         const uint32_t *inc = bank + (int64_t)c * MC * B + (B - 1);
         uint32_t acc = active ? bitmap_in[(int64_t)c * NC + lane] : 0u;
-        // words of the truth row that are not zero, and the blocks of 64 nodes they cover
-        const unsigned long long live_words = __ballot(acc != 0);
-        const int live_blocks = __popcll((live_words | (live_words >> 1)) & 0x5555555555555555ull);
         int included = 0;
         for (int w0 = 0; w0 < MC; w0 += 64) {
             uint32_t mine = w0 + lane < MC ? inc[(int64_t)(w0 + lane) * B] : 0u;
@@ -193,19 +193,23 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
             unsigned long long nonzero = __ballot(mine != 0);
             int here = __popc(mine);
             included += here;
+            // words of the truth row that are not zero, and the blocks of 64 nodes they cover
+            const unsigned long long live_words = __ballot(acc != 0);
             // a clause that is false everywhere stays false: only its include count is needed
             if (live_words == 0 || nonzero == 0) continue;
+            const int live_blocks = __popcll((live_words | (live_words >> 1)) & 0x5555555555555555ull);
             for (int off = 32; off > 0; off >>= 1) here += __shfl_xor(here, off);
             const int trips_by_literal = (here + 7) >> 3;
-            const int trips_by_node = live_blocks * ((__popcll(nonzero) + 7) >> 3);
+            const int trips_by_node = ((live_blocks + WAVES - 1) / WAVES) * ((__popcll(nonzero) + 7) >> 3);
             if (trips_by_node < trips_by_literal) {
-                uint32_t result = 0;  // lane L: word L of the clause's truth after these include words
-                for (int nb = 0; nb * 2 < words; ++nb) {
+                if (tid < 64) handed[tid] = 0u;
+                __syncthreads();
+                for (int nb = wave; nb * 2 < words; nb += WAVES) {
                     if (((live_words >> (nb * 2)) & 3ull) == 0) continue;
                     const int node = nb * 64 + lane;
                     // this node's bit of the running truth (lane = node)
                     const uint32_t lo = __builtin_amdgcn_readlane(acc, nb * 2);
-                    const uint32_t hi = nb * 2 + 1 < 64 ? __builtin_amdgcn_readlane(acc, (nb * 2 + 1) & 63) : 0u;
+                    const uint32_t hi = __builtin_amdgcn_readlane(acc, (nb * 2 + 1) & 63);
                     bool ok = ((lane < 32 ? lo >> lane : hi >> (lane - 32)) & 1u) != 0;
                     const uint32_t *x = clause_X + (int64_t)(node < n_nodes ? node : 0) * MC + w0;
                     unsigned long long todo = nonzero;
@@ -224,11 +228,15 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
                     }
                     ok = ok && violated == 0;
                     const unsigned long long truth = __ballot(ok);
-                    if (lane == nb * 2) result = (uint32_t)truth;
-                    if (lane == nb * 2 + 1) result = (uint32_t)(truth >> 32);
+                    if (lane == 0) {
+                        handed[nb * 2] = (uint32_t)truth;
+                        if (nb * 2 + 1 < 64) handed[nb * 2 + 1] = (uint32_t)(truth >> 32);
+                    }
                 }
-                acc = result;
-            } else {
+                __syncthreads();
+                acc = active ? handed[lane] : 0u;  // every wave goes on with the whole row
+                __syncthreads();
+            } else if (wave == 0) {
                 while (nonzero) {
                     const int wl = __ffsll((long long)nonzero) - 1;
                     nonzero &= nonzero - 1;
@@ -251,12 +259,20 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
                     }
                 }
             }
+            if (MC > 64) {
+                // more include words follow: the other waves need wave 0's row to decide the same way
+                if (wave == 0 && active) handed[lane] = acc;
+                __syncthreads();
+                acc = active ? handed[lane] : 0u;
+                __syncthreads();
+            }
         }
+        if (wave != 0) continue;
         for (int off = 32; off > 0; off >>= 1) included += __shfl_xor(included, off);
         const uint32_t v = active ? acc : 0u;
         if (lane == 0) n_incl[c] += included;
         fit_clause_tail(v, lane, words, NC, n_nodes, c, C, K, weights, k0, k1, step, finish != 0,
                         bitmap_out + (int64_t)c * NC, clause_node, class_sum, &partial);
     }
-    if (K <= 64 && lane < K && partial != 0) atomicAdd(&class_sum[lane], partial);
+    if (wave == 0 && K <= 64 && lane < K && partial != 0) atomicAdd(&class_sum[lane], partial);
 }

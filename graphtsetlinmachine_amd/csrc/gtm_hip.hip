@@ -1356,7 +1356,7 @@ int fit_deep_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g,
                                    cx, n_nodes, d.M, d.MC, w.message_row_words, w.message_rows);
                 if (int rc = check_launch("fit_message_rows")) return rc;
             }
-            hipLaunchKernelGGL(k_fit_message_eval, dim3(eval_blocks), dim3(FIT_EVAL_BLOCK), 0, st, w.message_rows,
+            hipLaunchKernelGGL(k_fit_message_eval, dim3(d.C < 4096 ? d.C : 4096), dim3(FIT_EVAL_BLOCK), 0, st, w.message_rows,
                                w.message_row_words, cx, words, n_nodes, d.M, d.C, d.MC, d.B, d.K, d.NC, d.mfilter,
                                s->message_ta_state[l], s->clause_weights, key.k0, key.k1, step, l == layers - 1 ? 1 : 0,
                                cur, nxt, w.n_incl, w.clause_node, sum_now);
