@@ -23,9 +23,9 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# HBM bytes per graph that the tile scoring kernel moves on the convolutional workload, from rocprofv3 --pmc runs
+# HBM bytes per graph that the scoring kernel moves on the convolutional workload, from rocprofv3 --pmc runs
 # (FETCH_SIZE x 2 KiB, the factor a 256 MiB copy kernel calibrates, + WRITE_SIZE x 1 KiB, over 10,000 graphs).
-MEASURED_TRAFFIC_BYTES_PER_GRAPH = {"convolutional_images": (72096.1 * 2 + 406.2) * 1024 / 10000}
+MEASURED_TRAFFIC_BYTES_PER_GRAPH = {"convolutional_images": (131715.6 * 2 + 406.3) * 1024 / 10000}
 
 
 def parse():
@@ -49,7 +49,7 @@ OTHER_WORKLOADS = {
     "single_node_images": (20000, 10000),
     "convolutional_images": (5000, 2000),
     "sequence_chains": (1000, 500),
-    "colour_convolution": (48, 32),
+    "colour_convolution": (48, 256),
 }
 
 
@@ -197,7 +197,7 @@ def main():
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
         "traffic": (round(MEASURED_TRAFFIC_BYTES_PER_GRAPH[args.workload] * graphs_per_launch)
-                    if args.workload in MEASURED_TRAFFIC_BYTES_PER_GRAPH and kernel_name == "k_tile_layer<score>" else None),
+                    if args.workload in MEASURED_TRAFFIC_BYTES_PER_GRAPH and kernel_name == "k_tile_two_phase<score>" else None),
         "kernel": kernel_name, "kernel_ms": round(kernel_ms, 4), "launches": launches,
         "graphs_per_launch": graphs_per_launch,
         "algorithmic_bytes_per_graph": b_eval,

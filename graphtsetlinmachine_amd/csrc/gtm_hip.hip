@@ -668,11 +668,12 @@ int launch_tile_layer_lw(const TileLayerArgs &a, int n_tiles, int src, bool last
     if (src == ROWS_MESSAGES)
         return last ? launch_tile_layer_as<NW, LW, ROWS_MESSAGES, true>(a, n_tiles, nullptr, st)
                     : launch_tile_layer_as<NW, LW, ROWS_MESSAGES, false>(a, n_tiles, nullptr, st);
+    // the layer-0 kernel is the one the library times (gtm_profile_*)
     if (src == ROWS_GLOBAL)
-        return last ? launch_tile_layer_as<NW, LW, ROWS_GLOBAL, true>(a, n_tiles, nullptr, st)
-                    : launch_tile_layer_as<NW, LW, ROWS_GLOBAL, false>(a, n_tiles, nullptr, st);
+        return last ? launch_tile_layer_as<NW, LW, ROWS_GLOBAL, true>(a, n_tiles, "k_tile_layer<score>", st)
+                    : launch_tile_layer_as<NW, LW, ROWS_GLOBAL, false>(a, n_tiles, "k_tile_layer<layer0>", st);
     return last ? launch_tile_layer_as<NW, LW, ROWS_STAGED, true>(a, n_tiles, "k_tile_layer<score>", st)
-                : launch_tile_layer_as<NW, LW, ROWS_STAGED, false>(a, n_tiles, nullptr, st);
+                : launch_tile_layer_as<NW, LW, ROWS_STAGED, false>(a, n_tiles, "k_tile_layer<layer0>", st);
 }
 
 int launch_tile_layer(const TileLayerArgs &a, int n_tiles, int src, bool last, hipStream_t st) {
@@ -694,10 +695,10 @@ int launch_two_phase_as(const TileLayerArgs &a, int n_tiles, hipStream_t st) {
         if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
         lds_set = lds;
     }
-    if (LAST) profile_start("k_tile_two_phase<score>", st);
+    profile_start(LAST ? "k_tile_two_phase<score>" : "k_tile_two_phase<layer0>", st);
     hipLaunchKernelGGL((k_tile_two_phase<NW, LW, LA4, LAST, FULL>), dim3(n_tiles), dim3(NW * 64), lds, st, a);
     if (int rc = check_launch("tile_two_phase")) return rc;
-    if (LAST) profile_stop(st);
+    profile_stop(st);
     return GTM_OK;
 }
 
