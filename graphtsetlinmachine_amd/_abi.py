@@ -88,6 +88,10 @@ PROTOTYPES = {
     "gtm_select_clause_updates": (C.c_int, [_CFG, _U64, _P, _P, _P, _I, _P, _P, _P]),
     "gtm_update": (C.c_int, [_CFG, _GR, _I, _U64, _P, _P, _P, _P, _P]),
     "gtm_update_message": (C.c_int, [_CFG, _U64, _I, _P, _P, _P, _P, _P, _P]),
+    "gtm_get_ta_states": (C.c_int, [_CFG, _P, _I, _I, _P, _P]),
+    "gtm_get_hyperliterals": (C.c_int, [_CFG, _P, _I, _I, _P, _P]),
+    "gtm_transform_workspace_bytes": (_SZ, [_CFG, _GR, _I]),
+    "gtm_transform": (C.c_int, [_CFG, _GR, _ST, _I, _I, _I, _P, _SZ, _P, _P, _I, _P, _P]),
     "gtm_profile_enable": (C.c_int, [C.c_int]),
     "gtm_profile_read": (C.c_int, [C.POINTER(C.c_char_p), C.POINTER(C.c_int32), C.POINTER(C.c_double)]),
     "gtm_tiles_bytes": (_SZ, [_CFG, _GR]),

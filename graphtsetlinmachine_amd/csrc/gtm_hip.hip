@@ -429,6 +429,53 @@ __global__ void k_update(uint32_t *bank, int C, int chunks, int B, int K, int bo
                       thr16);
 }
 
+// `get_ta_states` / `get_hyperliterals` (kernels.py:718-790): one thread per (clause, literal).
+__global__ void k_read_bank(const uint32_t *__restrict__ bank, int C, int chunks, int B, int literals, int actions,
+                            uint32_t *__restrict__ out) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)C * literals) return;
+    int c = (int)(i / literals), k = (int)(i % literals);
+    const uint32_t *planes = bank + ((int64_t)c * chunks + (k >> 5)) * B;
+    uint32_t v;
+    if (actions) {
+        v = (planes[B - 1] >> (k & 31)) & 1u;
+    } else {
+        v = 0;
+        for (int b = 0; b < B; ++b) v |= ((planes[b] >> (k & 31)) & 1u) << b;
+    }
+    out[i] = v;
+}
+
+// `transform` (kernels.py:671-691): one thread per (graph of the batch, clause).
+__global__ void k_transform(const uint32_t *__restrict__ bitmap, int C, int NC,
+                            const uint32_t *__restrict__ n_nodes_arr, int first_graph, int64_t total,
+                            int32_t *__restrict__ out) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    int b = (int)(i / C);
+    int n = (int)n_nodes_arr[first_graph + b];
+    const uint32_t *row = bitmap + i * NC;
+    uint32_t any = 0;
+    if (n > 0) {  // the reference loops over the nodes, so a graph without nodes gives 0
+        int chunks = chunks_of(n);
+        for (int w = 0; w < chunks - 1; ++w) any |= row[w];
+        any |= row[chunks - 1] & node_filter_of(n);
+    }
+    out[i] = any != 0;
+}
+
+// `transform_nodewise` (kernels.py:693-710): one thread per (graph, clause, node < width).
+__global__ void k_transform_nodewise(const uint32_t *__restrict__ bitmap, int C, int NC, int width,
+                                     const uint32_t *__restrict__ n_nodes_arr, int first_graph, int64_t total,
+                                     int32_t *__restrict__ out) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    int node = (int)(i % width);
+    int64_t gc = i / width;  // (graph of the batch, clause)
+    int n = (int)n_nodes_arr[first_graph + (int)(gc / C)];
+    out[i] = node < n ? (bitmap[gc * NC + (node >> 5)] >> (node & 31)) & 1u : 0;
+}
+
 // ------------------------------------------------------------ launch helpers
 
 int launch_clause_node_bits(const Dims &d, const gtm_graphs *g, int first, int n_graphs, const uint32_t *inc_t,
@@ -993,6 +1040,73 @@ int gtm_update_message(const gtm_config *cfg, uint64_t step, int32_t bank, uint3
         return fail(GTM_ERR_INVALID, "NULL buffer");
     return op_update(d, cfg, step, bank, message_ta_state, d.MC, clause_node, number_of_include_actions, clause_X,
                      class_clause_update, (hipStream_t)stream);
+}
+
+static int read_bank(const gtm_config *cfg, const uint32_t *bank, int32_t chunks, int32_t literals, int actions,
+                     uint32_t *out, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (!bank || !out) return fail(GTM_ERR_INVALID, "NULL buffer");
+    if (chunks < 1 || literals < 1 || literals > chunks * 32)
+        return fail(GTM_ERR_INVALID, "chunks=%d literals=%d", chunks, literals);
+    int64_t total = (int64_t)d.C * literals;
+    hipLaunchKernelGGL(k_read_bank, dim3(blocks_for(total, TPB)), dim3(TPB), 0, (hipStream_t)stream, bank, d.C, chunks,
+                       d.B, literals, actions, out);
+    return check_launch("read_bank");
+}
+
+int gtm_get_ta_states(const gtm_config *cfg, const uint32_t *bank, int32_t chunks, int32_t literals, uint32_t *out,
+                      void *stream) {
+    return read_bank(cfg, bank, chunks, literals, 0, out, stream);
+}
+
+int gtm_get_hyperliterals(const gtm_config *cfg, const uint32_t *bank, int32_t chunks, int32_t literals,
+                          uint32_t *out, void *stream) {
+    return read_bank(cfg, bank, chunks, literals, 1, out, stream);
+}
+
+size_t gtm_transform_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs, int32_t batch) {
+    Dims d;
+    if (validate(cfg, &d) || batch < 1) return 0;
+    (void)graphs;
+    return carve_score(d, cfg, batch, nullptr).bytes;
+}
+
+int gtm_transform(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, int32_t first_graph,
+                  int32_t n_graphs, int32_t batch, void *workspace, size_t workspace_bytes, int32_t *transformed,
+                  int32_t *nodewise, int32_t width, int32_t *class_sum, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (int rc = validate_graphs(cfg, graphs, first_graph, n_graphs)) return rc;
+    if (int rc = validate_state(cfg, state)) return rc;
+    if (batch < 1) return fail(GTM_ERR_INVALID, "batch=%d", batch);
+    if (!transformed || !class_sum) return fail(GTM_ERR_INVALID, "NULL output");
+    if (nodewise && (width < 1 || width > cfg->max_nodes))
+        return fail(GTM_ERR_INVALID, "width=%d outside [1, max_nodes=%d]", width, cfg->max_nodes);
+    ScoreWs w = carve_score(d, cfg, batch, (char *)workspace);
+    if (!workspace || workspace_bytes < w.bytes)
+        return fail(GTM_ERR_INVALID, "workspace of %zu bytes needed, %zu given", w.bytes, workspace_bytes);
+    hipStream_t st = (hipStream_t)stream;
+    for (int done = 0; done < n_graphs; done += batch) {
+        int nb = n_graphs - done < batch ? n_graphs - done : batch;
+        uint32_t *final_bitmap = nullptr;
+        uint32_t *layers[1] = {w.clause_X};
+        if (int rc = run_evaluate(d, cfg, graphs, state, first_graph + done, nb, w.inc_t, w.bitmap_a, w.bitmap_b, layers,
+                                  false, nullptr, class_sum + (int64_t)done * d.K, &final_bitmap, st))
+            return rc;
+        int64_t total = (int64_t)nb * d.C;
+        hipLaunchKernelGGL(k_transform, dim3(blocks_for(total, TPB)), dim3(TPB), 0, st, final_bitmap, d.C, d.NC,
+                           graphs->number_of_graph_nodes, first_graph + done, total, transformed + (int64_t)done * d.C);
+        if (int rc = check_launch("transform")) return rc;
+        if (nodewise) {
+            int64_t cells = total * width;
+            hipLaunchKernelGGL(k_transform_nodewise, dim3(blocks_for(cells, TPB)), dim3(TPB), 0, st, final_bitmap, d.C,
+                               d.NC, width, graphs->number_of_graph_nodes, first_graph + done, cells,
+                               nodewise + (int64_t)done * d.C * width);
+            if (int rc = check_launch("transform_nodewise")) return rc;
+        }
+    }
+    return GTM_OK;
 }
 
 int gtm_profile_enable(int on) {

@@ -307,6 +307,37 @@ class CommonTsetlinMachine:
         )
         return out
 
+    def _transform(self, graphs, nodewise, batch=None):
+        """tm.py:814-900 as one gtm_transform call."""
+        dg = self._score_init(graphs)
+        cfg = self._config(max(dg.max_nodes, 1))
+        n, C = dg.number_of_graphs, self.number_of_clauses
+        width = max(int(np.max(graphs.number_of_graph_nodes)), 1) if nodewise else 0
+        if batch is None:
+            size = lambda b: _abi.lib.gtm_transform_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc), b)
+            fixed = size(1)
+            per_graph = max(1.0, (size(1025) - fixed) / 1024.0)
+            batch = int(max(1, min(n, ((1 << 30) - fixed) // per_graph, 1 << 16)))
+        need = _abi.lib.gtm_transform_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc), batch)
+        ws = self._workspace_of(need)
+        sums = torch.empty(n * self.number_of_outputs, dtype=torch.int32, device=_device())
+        flat = torch.empty(n * C, dtype=torch.int32, device=_device())
+        wide = torch.empty(n * C * width, dtype=torch.int32, device=_device()) if nodewise else None
+        _abi.call(
+            "gtm_transform", ctypes.byref(cfg), ctypes.byref(dg.desc), ctypes.byref(self._state), 0, n, batch,
+            _ptr(ws), ws.numel(), _ptr(flat), _ptr(wide) if nodewise else None, width, _ptr(sums), _stream(),
+        )
+        out = wide.cpu().numpy().reshape(n, C, width) if nodewise else flat.cpu().numpy().reshape(n, C)
+        return out, sums.cpu().numpy().reshape(n, self.number_of_outputs)
+
+    def transform(self, graphs):
+        """tm.py:814-851: (int32 [graphs][clauses] = the clause is true at some node, class sums)."""
+        return self._transform(graphs, False)
+
+    def transform_nodewise(self, graphs):
+        """tm.py:853-900: (int32 [graphs][clauses][largest graph] = the clause's truth per node, class sums)."""
+        return self._transform(graphs, True)
+
     # ------------------------------------------------------------- state I/O
 
     def _download(self):
@@ -324,6 +355,57 @@ class CommonTsetlinMachine:
         else:
             bank = self.message_ta_state[depth - 1].reshape(self.number_of_clauses, self.number_of_message_chunks, B)
         return (bank[clause, ta // 32, B - 1] & (1 << (ta % 32))) > 0
+
+    def _read_bank(self, entry, depth):
+        if depth == 0:
+            bank, chunks, literals = self.ta_state_gpu, self.number_of_ta_chunks, self.number_of_literals
+        else:
+            bank = self.message_ta_state_gpu[depth - 1]
+            chunks, literals = self.number_of_message_chunks, self.number_of_message_literals
+        cfg = self._config(max(self._max_nodes_seen(), 1))
+        out = torch.empty(self.number_of_clauses * literals, dtype=torch.int32, device=_device())
+        _abi.call(entry, ctypes.byref(cfg), _ptr(bank), chunks, literals, _ptr(out), _stream())
+        return out.cpu().numpy().view(np.uint32).reshape(self.number_of_clauses, literals)
+
+    def _max_nodes_seen(self):
+        return self._train_graphs.max_nodes if self._train_graphs is not None else 1
+
+    def get_hyperliterals(self, depth):
+        """tm.py:144-172: uint32 [clauses][literals of the layer], 1 where the automaton includes."""
+        return self._read_bank("gtm_get_hyperliterals", depth)
+
+    def get_ta_states(self, depth):
+        """tm.py:174-205: uint32 [clauses][literals of the layer], the automata's integer states."""
+        return self._read_bank("gtm_get_ta_states", depth)
+
+    def get_clause_literals(self, symbol_hv):
+        """tm.py:213-240: float [clauses][2 * symbols], how many of each symbol's hypervector
+        bits the clause includes (second half: their negations)."""
+        hv_clauses = self.get_hyperliterals(0)
+        half = self.number_of_literals // 2
+        n_symbols = symbol_hv.shape[0]
+        expanded = np.zeros((half, n_symbols), dtype=np.uint8)
+        for sym_id in range(n_symbols):
+            expanded[symbol_hv[sym_id].ravel(), sym_id] = 1
+        out = np.zeros((self.number_of_clauses, 2 * n_symbols))
+        out[:, :n_symbols] = hv_clauses[:, :half] @ expanded
+        out[:, n_symbols:] = hv_clauses[:, half:] @ expanded
+        return out
+
+    def get_messages(self, depth, edge_types):
+        """tm.py:242-279: float [edge types][clauses][2 * clauses], how many of each sending
+        clause's (rotated) hypervector bits a clause's message literals of layer `depth` include."""
+        assert depth > 0, f"Expected depth > 0, got {depth}. Depth <= 0 means surface, use get_clause_literals()"
+        hv_messages = self.get_hyperliterals(depth).astype(np.float32)
+        half, C = self.number_of_message_literals // 2, self.number_of_clauses
+        out = np.zeros((edge_types, C, 2 * C))
+        for edge_type in range(edge_types):
+            expanded = np.zeros((half, C))
+            for sym_id in range(C):
+                expanded[(self.hypervectors[sym_id].ravel() + edge_type) % self.message_size, sym_id] = 1
+            out[edge_type, :, :C] = hv_messages[:, :half] @ expanded
+            out[edge_type, :, C:] = hv_messages[:, half:] @ expanded
+        return out
 
     def get_weights(self):
         """tm.py:207-211."""

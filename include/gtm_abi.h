@@ -197,6 +197,28 @@ int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *st
 
 /* ---- measurement -------------------------------------------------------- */
 
+/* `get_ta_states` and `get_hyperliterals` (kernels.py:718-757, :761-790; called
+ * from tm.py:144-205): the integer state (resp. 1 for an include action) of
+ * every automaton of a bank, uint32 out[CLAUSES][literals].  `chunks` and
+ * `literals` are the bank's: LA_CHUNKS / LITERALS for ta_state, MESSAGE_CHUNKS /
+ * MESSAGE_LITERALS for a message bank. */
+int gtm_get_ta_states(const gtm_config *cfg, const uint32_t *bank, int32_t chunks, int32_t literals, uint32_t *out,
+                      void *stream);
+int gtm_get_hyperliterals(const gtm_config *cfg, const uint32_t *bank, int32_t chunks, int32_t literals,
+                          uint32_t *out, void *stream);
+
+/* The loops of `transform` and `transform_nodewise` (tm.py:814-900 with
+ * kernels.py:671-710) for graphs [first_graph, first_graph + n_graphs), `batch`
+ * graphs per launch: int32 transformed[n_graphs][CLAUSES] = 1 where the clause
+ * is true at some node of the graph; when `nodewise` is not NULL also int32
+ * nodewise[n_graphs][CLAUSES][width] = the clause's truth at every node (0 past
+ * the graph's nodes; width >= the largest graph of the range); and the class
+ * sums as gtm_score gives them.  Workspace: gtm_transform_workspace_bytes(). */
+size_t gtm_transform_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs, int32_t batch);
+int gtm_transform(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, int32_t first_graph,
+                  int32_t n_graphs, int32_t batch, void *workspace, size_t workspace_bytes, int32_t *transformed,
+                  int32_t *nodewise, int32_t width, int32_t *class_sum, void *stream);
+
 /* No counterpart in the reference.  While enabled, gtm_score / gtm_fit bracket
  * each launch of their clause-evaluation kernel (the dominant kernel) with HIP
  * events on the caller's stream (at most 512 launches are kept).

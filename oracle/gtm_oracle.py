@@ -548,6 +548,50 @@ def score(model, graphs, indices=None):
     return out
 
 
+def transform(model, graphs, indices=None, nodewise=False):
+    """tm.py:814-900 with kernels.py:671-710: per graph, 1 where the clause is true
+    at some node of the graph (``nodewise``: its truth at every node, zero-padded
+    to the largest graph), next to the class sums.  Unlike `evaluate`, the
+    transform kernels loop over the graph's nodes, so a graph without nodes
+    gives zeros."""
+    cfg = model.cfg
+    if indices is None:
+        indices = range(graphs.number_of_graphs)
+    width = int(graphs.number_of_graph_nodes.max()) if graphs.number_of_graphs else 0
+    shape = (len(indices), cfg.clauses, width) if nodewise else (len(indices), cfg.clauses)
+    out = np.zeros(shape, dtype=np.int32)
+    sums = np.zeros((len(indices), cfg.classes), dtype=np.int32)
+    for i, e in enumerate(indices):
+        n = int(graphs.number_of_graph_nodes[e])
+        bitmap, sums[i], _, _ = evaluate_graph(model, graphs, e)
+        if n == 0:
+            continue
+        truth = _unpack_bitmap(bitmap, n)
+        if nodewise:
+            out[i, :, :n] = truth
+        else:
+            out[i] = truth.any(axis=1)
+    return out, sums
+
+
+def get_ta_states(bank, state_bits, literals):
+    """kernels.py:718-757: the integer state of every automaton, uint32 [CLAUSES][literals]."""
+    bank = np.asarray(bank, dtype=U32)
+    clauses, chunks, _ = bank.shape
+    out = np.zeros((clauses, chunks * 32), dtype=U32)
+    for b in range(state_bits):
+        plane = np.unpackbits(np.ascontiguousarray(bank[:, :, b]).view(np.uint8), axis=1, bitorder="little")
+        out |= plane.astype(U32) << U32(b)
+    return out[:, :literals]
+
+
+def get_hyperliterals(bank, state_bits, literals):
+    """kernels.py:761-790: 1 where the automaton's action is include, uint32 [CLAUSES][literals]."""
+    bank = np.asarray(bank, dtype=U32)
+    plane = np.unpackbits(np.ascontiguousarray(bank[:, :, state_bits - 1]).view(np.uint8), axis=1, bitorder="little")
+    return plane[:, :literals].astype(U32)
+
+
 def fit_graph(model, graphs, encoded_Y, e):
     """One iteration of the loop at tm.py:669-747."""
     cfg = model.cfg

@@ -127,3 +127,54 @@ def test_score_before_fit_exits_like_the_reference():
     tm = MultiClassGraphTsetlinMachine(**wl.params, seed=1)
     with pytest.raises(SystemExit):
         tm.score(wl.graphs_test)
+
+
+def test_transform_and_read_outs_match_the_oracle():
+    """transform / transform_nodewise / get_ta_states / get_hyperliterals (bit-exact against the
+    oracle) and the two host read-outs built on them (against a literal-level recount)."""
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    train = helpers.random_graphs(60, n_graphs=30, hv_size=24, node_types=("a", "b"), edge_types=("l", "r"),
+                                  sizes=[5, 0, 33, 1, 40, 64] * 5)
+    rng = np.random.default_rng(2)
+    Y = rng.integers(0, 3, size=30)
+    np.random.seed(9)
+    tm = MultiClassGraphTsetlinMachine(40, 30, (2.0, 1.5), depth=2, message_size=40, message_bits=2, seed=11)
+    tm.fit(train, Y, epochs=2, incremental=True)
+    model = oracle_twin(tm, train)
+    o.fit(model, train, o.encode_labels(Y, 3, tm.T), epochs=2)
+    assert_same_state(tm, model)
+
+    got, sums = tm.transform(train)
+    want, want_sums = o.transform(model, train)
+    assert got.dtype == np.int32 and np.array_equal(got, want) and np.array_equal(sums, want_sums)
+    assert got.any() and not got[1].any()  # a graph without nodes transforms to zeros
+    wide, sums = tm.transform_nodewise(train)
+    want, _ = o.transform(model, train, nodewise=True)
+    assert wide.shape == (30, 40, 64) and np.array_equal(wide, want) and np.array_equal(sums, want_sums)
+
+    for depth, bank, literals in ((0, model.ta_state, tm.number_of_literals),
+                                  (1, model.message_ta_state[0], tm.number_of_message_literals)):
+        assert np.array_equal(tm.get_ta_states(depth), o.get_ta_states(bank, 8, literals))
+        assert np.array_equal(tm.get_hyperliterals(depth), o.get_hyperliterals(bank, 8, literals))
+
+    # get_clause_literals: per clause and symbol, the number of the symbol's bits among the included literals
+    included = o.get_hyperliterals(model.ta_state, 8, tm.number_of_literals)
+    table = tm.get_clause_literals(train.hypervectors)
+    n_symbols, half = train.hypervectors.shape[0], tm.number_of_literals // 2
+    assert table.shape == (40, 2 * n_symbols)
+    for c in (0, 7, 39):
+        for sym in range(n_symbols):
+            bits = [int(b) for b in train.hypervectors[sym]]
+            assert table[c, sym] == sum(int(included[c, b]) for b in bits)
+            assert table[c, n_symbols + sym] == sum(int(included[c, half + b]) for b in bits)
+    # get_messages: the same count for the sending clauses' hypervector bits rotated by the edge type
+    included = o.get_hyperliterals(model.message_ta_state[0], 8, tm.number_of_message_literals)
+    messages = tm.get_messages(1, 2)
+    assert messages.shape == (2, 40, 80)
+    for edge_type in (0, 1):
+        for c in (0, 13):
+            for sender in (0, 5, 39):
+                bits = [(int(b) + edge_type) % 40 for b in tm.hypervectors[sender]]
+                assert messages[edge_type, c, sender] == sum(int(included[c, b]) for b in bits)
+                assert messages[edge_type, c, 40 + sender] == sum(int(included[c, 40 + b]) for b in bits)
