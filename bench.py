@@ -22,6 +22,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+VALU_PEAK_LANE_OPS = 256 * 64 * 2.4e9  # 32-bit integer lane operations per second
 
 # HBM bytes per graph that the scoring kernel moves on the convolutional workload, from rocprofv3 --pmc runs
 # (FETCH_SIZE x 2 KiB, the factor a 256 MiB copy kernel calibrates, + WRITE_SIZE x 1 KiB, over 10,000 graphs).
@@ -202,6 +203,10 @@ def main():
         "graphs_per_launch": graphs_per_launch,
         "algorithmic_bytes_per_graph": b_eval,
         "compulsory_GBs": round(compulsory / (kernel_ms * 1e-3) / 1e9, 1),
+        # the dense formulation (one word test per clause, node and literal word) against the integer
+        # VALU peak of 256 CUs x 64 lanes x 2.4 GHz: what a kernel that does not skip work could reach
+        "dense_word_ops_per_graph": tm.number_of_clauses * n_nodes * la,
+        "dense_valu_ceiling_graphs_per_s": round(VALU_PEAK_LANE_OPS / (tm.number_of_clauses * n_nodes * la), 1),
     }
 
     cpu = None
@@ -218,9 +223,18 @@ def main():
         if not np.array_equal(want, sums_host[:sample]):
             print("bench.py: GPU class sums differ from the CPU oracle on the sample", file=sys.stderr)
             sys.exit(1)
+        # training: the same oracle, continuing from the GPU model's state on a few training graphs
+        train_sample = max(2, min(sample // 8, args.train_graphs))
+        encoded = o.encode_labels(wl.Y_train[:train_sample], tm.number_of_outputs, tm.T)
+        train_model = oracle_twin(tm, int(wl.graphs_train.max_number_of_graph_nodes))
+        t0 = time.perf_counter()
+        o.fit(train_model, wl.graphs_train, encoded, indices=range(train_sample))
+        t_cpu_train = time.perf_counter() - t0
         cpu = {"value": round(sample / t_cpu, 2), "unit": "graphs/s", "cores": 1, "kind": "port",
                "sample": "NumPy oracle, inference on the first %d test graphs (%.1f s), checked equal to the GPU sums"
-                         % (sample, t_cpu)}
+                         % (sample, t_cpu),
+               "train_value": round(train_sample / t_cpu_train, 2),
+               "train_sample": "NumPy oracle, one training pass over %d graphs (%.1f s)" % (train_sample, t_cpu_train)}
 
     others = {}
     if not args.only_main:
