@@ -514,6 +514,9 @@ struct ScoreWs {
     uint32_t *message_lists;  // [depth-1][C][message_list_stride]  (tile path, depth > 1)
     int message_list_stride;
     uint32_t *tile_bitmap;    // [tiles per launch][C][tw]  (tile path, depth > 1)
+    uint32_t *sent, *got;     // [tiles per launch][tw * 32 node slots][ceil(M / 32)]  (tile path, depth > 1)
+    uint32_t *message_rows;   // [tiles per launch][M + 2][tw]  (tile path, depth > 1)
+    size_t vector_words;      // words of sent (and of got)
     uint32_t *inc_t;          // [max(LA,MC)][C]
     uint32_t *bitmap_a;       // [batch][C][NC]
     uint32_t *bitmap_b;       // [batch][C][NC] (depth > 1)
@@ -548,7 +551,12 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base,
     if (tg) {
         w.message_list_stride = clause_list_stride(2 * d.M);
         w.message_lists = (uint32_t *)take((size_t)(cfg->depth - 1) * d.C * w.message_list_stride * 4);
-        w.tile_bitmap = (uint32_t *)take((size_t)tiles_per_batch(*tg, batch) * d.C * tg->tw * 4);
+        const size_t n_tiles = tiles_per_batch(*tg, batch);
+        w.tile_bitmap = (uint32_t *)take(n_tiles * d.C * tg->tw * 4);
+        w.vector_words = n_tiles * tg->tw * 32 * ((d.M + 31) / 32);
+        w.sent = (uint32_t *)take(w.vector_words * 4);
+        w.got = (uint32_t *)take(w.vector_words * 4);
+        w.message_rows = (uint32_t *)take(n_tiles * tile_message_rows(d.M) * tg->tw * 4);
         w.bytes = off;
         return w;
     }
@@ -848,6 +856,17 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         return fail(GTM_ERR_INVALID, "graphs with edges need number_of_graph_node_edges, edge and edge_index");
     const int tiles_per_launch = tiles_per_batch(tg, batch);
     const int tile_first = first / tg.gpt, tile_last = (first + n_graphs - 1) / tg.gpt;
+    const int MW = (d.M + 31) / 32;
+    int group = 16;  // words of a truth row per k_tile_node_messages block: its vectors must fit in 64 KB of LDS
+    while (group > 1 && (size_t)32 * group * MW * 4 > 64 * 1024) group >>= 1;
+    a.message_rows = w.message_rows;
+    static thread_local bool node_messages_lds_raised = false;
+    if (!node_messages_lds_raised) {
+        hipError_t e = hipFuncSetAttribute((const void *)k_tile_node_messages,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit: %s", hipGetErrorString(e));
+        node_messages_lds_raised = true;
+    }
     for (int t0 = tile_first; t0 <= tile_last; t0 += tiles_per_launch) {
         const int n_tiles = tile_last - t0 + 1 < tiles_per_launch ? tile_last - t0 + 1 : tiles_per_launch;
         a.tile0 = t0;
@@ -856,6 +875,25 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         a.class_sum = class_sum;
         if (int rc = layer0(n_tiles, false)) return rc;
         for (int l = 1; l < layers; ++l) {
+            // the layer's message rows for these tiles (score_tiles.h)
+            hipLaunchKernelGGL(k_tile_node_messages, dim3((tg.tw + group - 1) / group, n_tiles),
+                               dim3(TILE_MESSAGES_BLOCK), (size_t)32 * group * MW * 4, st, w.tile_bitmap, d.C, tg.tw,
+                               group, s->hypervectors, d.MB, MW, w.sent);
+            if (int rc = check_launch("tile_node_messages")) return rc;
+            const int64_t vector_words = (int64_t)n_tiles * tg.tw * 32 * MW;
+            hipLaunchKernelGGL(k_fill_i32, dim3(blocks_for(vector_words, TPB)), dim3(TPB), 0, st, (int32_t *)w.got,
+                               vector_words, 0);
+            if (int rc = check_launch("fill")) return rc;
+            if (g->total_edges > 0) {
+                hipLaunchKernelGGL(k_tile_edge_messages, dim3(blocks_for(vector_words, TPB)), dim3(TPB), 0, st, w.sent, tg,
+                                   t0, g->number_of_graphs, d.M, MW, g->node_index, g->number_of_graph_nodes,
+                                   g->number_of_graph_node_edges, g->edge_index, g->edge, vector_words, w.got);
+                if (int rc = check_launch("tile_edge_messages")) return rc;
+            }
+            hipLaunchKernelGGL(k_tile_pack_messages, dim3((tg.tw + 1) / 2, n_tiles), dim3(256),
+                               (size_t)64 * (MW + 1) * 4, st, w.got, tg, t0, g->number_of_graphs, d.M, MW,
+                               g->number_of_graph_nodes, w.message_rows);
+            if (int rc = check_launch("tile_pack_messages")) return rc;
             a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
             a.stride = w.message_list_stride;
             if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1, st)) return rc;
@@ -1170,6 +1208,8 @@ int gtm_build_tiles(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *t
 static bool score_uses_tiles(const gtm_config *cfg, const gtm_graphs *graphs, int classes, TileGeom *tg) {
     if (!graphs || !graphs->tiles || graphs->number_of_graphs < 1 || graphs->number_of_node_types < 1) return false;
     *tg = geometry_for(cfg, graphs, classes);
+    // with message layers a 64-slot block of message vectors has to fit in 64 KB of LDS
+    if (cfg->depth > 1 && (size_t)64 * ((cfg->message_size + 31) / 32 + 1) * 4 > 64 * 1024) return false;
     return tg->ok != 0;
 }
 

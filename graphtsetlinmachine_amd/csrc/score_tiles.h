@@ -298,6 +298,7 @@ struct TileLayerArgs {
     const uint32_t *hv;     // [C][MB]
     const uint32_t *node_index, *n_nodes, *n_edges, *edge_index, *edge;
     const uint32_t *X;      // [nodes][LA] node-major literal words (two-phase layer 0)
+    const uint32_t *message_rows;  // [tiles of the launch][M + 2][tw] (message layers, built by k_tile_pack_messages)
 };
 
 // Rows a message layer keeps in LDS: M message rows, the all-ones row, the row of graphs without nodes.
@@ -307,17 +308,167 @@ inline size_t tile_layer_lds_bytes(const TileGeom &g, int classes, int src, int 
     return tile_lds_bytes(src == ROWS_STAGED ? g.rows : src == ROWS_MESSAGES ? tile_message_rows(M) : 0, g, classes);
 }
 
+// ---- the message rows of a layer, for all tiles of a launch ------------------
+//
+// A message factors: the bits a node sends are the OR of the hypervector bits
+// of the clauses true at it; what a neighbour receives along an edge of type t
+// is that bit vector rotated by t (kernels.py:581).  Node slots are addressed
+// by their position in the tile, so padding slots simply stay empty.
+//   k_tile_node_messages  sent[tile][slot][MW] from the truth rows [tile][C][tw]
+//   k_tile_edge_messages  got[tile][dst slot] |= rotate(sent[tile][slot], type)
+//   k_tile_pack_messages  rows[tile][M + 2][tw]: got turned literal-major, the
+//                         all-ones row, the row of graphs without nodes
+// (got is cleared before every layer's k_tile_edge_messages)
+// MW = ceil(M / 32) words per vector.
+
+constexpr int TILE_MESSAGES_BLOCK = 256;
+
+// grid (ceil(tw / group), tiles); `group` consecutive words of every truth row of the tile per
+// block (a power of two <= 16: one cache line per clause), dynamic LDS 32 * group * MW words.
+// Every word of sent is written (no clearing needed).
+__global__ __launch_bounds__(TILE_MESSAGES_BLOCK) void k_tile_node_messages(
+    const uint32_t *__restrict__ bitmap, int C, int tw, int group, const uint32_t *__restrict__ hv, int MB, int MW,
+    uint32_t *__restrict__ sent) {
+    extern __shared__ uint32_t vec[];  // [32 * group slots][MW]
+    const int tid = threadIdx.x;
+    const int w0 = blockIdx.x * group, tile = blockIdx.y;
+    const int n_vec = 32 * group * MW;
+    for (int i = tid; i < n_vec; i += TILE_MESSAGES_BLOCK) vec[i] = 0u;
+    __syncthreads();
+    const int wl = tid & (group - 1), w = w0 + wl;
+    const uint32_t *rows = bitmap + (int64_t)tile * C * tw;
+    constexpr int AHEAD = 4;  // truth words in flight per thread
+    const int step = TILE_MESSAGES_BLOCK / group;
+    if (w < tw)
+        for (int c0 = tid / group; c0 < C; c0 += AHEAD * step) {
+            uint32_t words[AHEAD];
+#pragma unroll
+            for (int u = 0; u < AHEAD; ++u) {
+                const int c = c0 + u * step;
+                words[u] = c < C ? rows[(int64_t)c * tw + w] : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < AHEAD; ++u) {
+                uint32_t word = words[u];
+                if (!word) continue;
+                const int c = c0 + u * step;
+                for (int j = 0; j < MB; ++j) {
+                    const uint32_t h = hv[(int64_t)c * MB + j];
+                    const uint32_t bit = 1u << (h & 31);
+                    uint32_t *column = vec + (wl * 32) * MW + (h >> 5);
+                    for (uint32_t m = word; m; m &= m - 1) atomicOr(&column[(__ffs(m) - 1) * MW], bit);
+                }
+            }
+        }
+    __syncthreads();
+    uint32_t *out = sent + ((int64_t)tile * tw + w0) * 32 * MW;
+    const int n_out = (min(tw, w0 + group) - w0) * 32 * MW;
+    for (int i = tid; i < n_out; i += TILE_MESSAGES_BLOCK) out[i] = vec[i];
+}
+
+// One thread per (tile of the launch, node slot, vector word).
+__global__ void k_tile_edge_messages(const uint32_t *__restrict__ sent, TileGeom tg, int tile0, int G, int M, int MW,
+                                     const uint32_t *__restrict__ node_index, const uint32_t *__restrict__ n_nodes,
+                                     const uint32_t *__restrict__ n_edges, const uint32_t *__restrict__ edge_index,
+                                     const uint32_t *__restrict__ edge, int64_t total, uint32_t *got) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int j = (int)(i % MW);
+    const int64_t slot_id = i / MW;  // tile of the launch * slots per tile + slot
+    const int slots = tg.tw * 32;
+    const int tile_local = (int)(slot_id / slots), pos = (int)(slot_id % slots);
+    const int gj = pos / tg.slot_bits, n = pos - gj * tg.slot_bits;
+    const int64_t g = (int64_t)(tile0 + tile_local) * tg.gpt + gj;
+    if (gj >= tg.gpt || g >= G || (uint32_t)n >= n_nodes[g]) return;
+    const uint32_t *v = sent + slot_id * MW;
+    const int64_t row = (int64_t)node_index[g] + n;
+    const uint32_t ne = n_edges[row];
+    const int64_t e0 = edge_index[row];
+    for (uint32_t e = 0; e < ne; ++e) {
+        const uint32_t dst = edge[(e0 + e) * 2], shift = edge[(e0 + e) * 2 + 1] % (uint32_t)M;
+        uint32_t word = 0;
+        if ((M & 31) == 0) {
+            // bit p of the result is bit (p - shift) mod M of v
+            const int q = (int)(shift >> 5), r = (int)(shift & 31u);
+            const int a = (j - q + MW) % MW, below = (a - 1 + MW) % MW;
+            word = r ? (v[a] << r) | (v[below] >> (32 - r)) : v[a];
+        } else {
+            for (int b = 0; b < 32; ++b) {
+                const int p = j * 32 + b;
+                if (p >= M) break;
+                const int from = (p + M - (int)shift) % M;
+                word |= ((v[from >> 5] >> (from & 31)) & 1u) << b;
+            }
+        }
+        if (word) atomicOr(&got[((int64_t)tile_local * slots + gj * tg.slot_bits + dst) * MW + j], word);
+    }
+}
+
+// grid (ceil(tw / 2), tiles), 256 threads: the received vectors of 64 node slots go through LDS
+// (read row by row, coalesced) and come out literal-major: wave v turns vector words v, v + 4, ...
+// into rows 32 j .. 32 j + 31 (lane = slot, one ballot per bit).  Wave 0 also writes the all-ones
+// row M and row M + 1 (slot bit 0 of the graphs without nodes: the reference's chunk arithmetic
+// leaves every clause true for such a graph at every layer, kernels.py:443-466,505-527, which the
+// message literals must not undo).  Dynamic LDS 64 * (MW + 1) words.
+__global__ __launch_bounds__(256) void k_tile_pack_messages(const uint32_t *__restrict__ got, TileGeom tg, int tile0,
+                                                             int G, int M, int MW,
+                                                             const uint32_t *__restrict__ n_nodes,
+                                                             uint32_t *__restrict__ rows) {
+    extern __shared__ uint32_t block[];  // [64 slots][MW + 1]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nb = blockIdx.x, tile_local = blockIdx.y;
+    const int tw = tg.tw, slots = tw * 32;
+    const int n_here = min(64, slots - nb * 64);
+    const uint32_t *src = got + ((int64_t)tile_local * slots + nb * 64) * MW;
+    for (int i = tid; i < n_here * MW; i += 256) block[(i / MW) * (MW + 1) + i % MW] = src[i];
+    __syncthreads();
+    uint32_t *out = rows + (int64_t)tile_local * (M + 2) * tw;
+    const bool lo_ok = nb * 2 < tw, hi_ok = nb * 2 + 1 < tw;
+    for (int j = wave; j < MW; j += 4) {
+        const uint32_t word = lane < n_here ? block[lane * (MW + 1) + j] : 0u;
+        unsigned long long mine = 0;
+#pragma unroll
+        for (int b = 0; b < 32; ++b) {
+            const unsigned long long column = __ballot((word >> b) & 1u);
+            if (lane == b) mine = column;
+        }
+        const int p = j * 32 + lane;
+        if (lane < 32 && p < M) {
+            if (lo_ok) out[(int64_t)p * tw + nb * 2] = (uint32_t)mine;
+            if (hi_ok) out[(int64_t)p * tw + nb * 2 + 1] = (uint32_t)(mine >> 32);
+        }
+    }
+    if (wave == 0) {
+        const int pos = nb * 64 + lane;
+        const int used = tg.slot_words == 0 ? tw : tg.gpt * tg.slot_words;
+        const int gj = pos / tg.slot_bits, n = pos - gj * tg.slot_bits;
+        const int64_t g = (int64_t)(tile0 + tile_local) * tg.gpt + gj;
+        const bool empty = pos < slots && n == 0 && gj < tg.gpt && g < G && n_nodes[g] == 0u;
+        const unsigned long long e = __ballot(empty);
+        if (lane == 0) {
+            if (lo_ok) {
+                out[(int64_t)M * tw + nb * 2] = nb * 2 < used ? 0xFFFFFFFFu : 0u;
+                out[(int64_t)(M + 1) * tw + nb * 2] = (uint32_t)e;
+            }
+            if (hi_ok) {
+                out[(int64_t)M * tw + nb * 2 + 1] = nb * 2 + 1 < used ? 0xFFFFFFFFu : 0u;
+                out[(int64_t)(M + 1) * tw + nb * 2 + 1] = (uint32_t)(e >> 32);
+            }
+        }
+    }
+}
+
 // One layer of clause evaluation for one tile per workgroup.
 //
 // Layer 0 (ROWS_STAGED / ROWS_GLOBAL): a clause's truth over the tile's node
 // slots is the AND of the node-type row and the rows of its included literals
-// (kernels.py:443-466).  Message layers (ROWS_MESSAGES): first the workgroup
-// builds the layer's message rows in LDS - row p has the bit of node slot n set
-// iff some clause that is true at a neighbour s with an edge s -> n of type t
-// has (h + t) mod M == p for one of its hypervector bits h (kernels.py:565-588;
-// the negated message literal p + M is the complement of row p) - then a
-// clause's truth is its previous truth AND the rows of its included message
-// literals (kernels.py:505-527).
+// (kernels.py:443-466).  Message layers (ROWS_MESSAGES): the layer's message
+// rows (k_tile_*_messages below; row p has the bit of node slot n set iff some
+// clause that is true at a neighbour s with an edge s -> n of type t has
+// (h + t) mod M == p for one of its hypervector bits h, kernels.py:565-588; the
+// negated message literal p + M is the complement of row p) are staged in LDS,
+// and a clause's truth is its previous truth AND the rows of its included
+// message literals (kernels.py:505-527).
 //
 // A wave owns a clause at a time.  The clause's row list is wave-uniform: its
 // first 32 entries arrive by scalar loads issued while the previous clause is
@@ -342,10 +493,12 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     uint32_t *bitmap = a.bitmap + (int64_t)blockIdx.x * C * tw;  // this tile's truth rows
 
-    if (SRC == ROWS_STAGED) {  // tile -> LDS, 16 bytes per thread and trip, several loads in flight
-        const uint4 *src = reinterpret_cast<const uint4 *>(a.tiles + (int64_t)tile * tg.rows * tw);
+    if (SRC == ROWS_STAGED || SRC == ROWS_MESSAGES) {  // rows -> LDS, 16 bytes per thread and trip, several loads in flight
+        const uint4 *src = reinterpret_cast<const uint4 *>(
+            SRC == ROWS_STAGED ? a.tiles + (int64_t)tile * tg.rows * tw
+                               : a.message_rows + (int64_t)blockIdx.x * n_rows_lds * tw);
         uint4 *dst = reinterpret_cast<uint4 *>(bt);
-        const int n4 = (tg.rows * tw) >> 2;  // tw is a multiple of 4
+        const int n4 = (n_rows_lds * tw) >> 2;  // tw is a multiple of 4
         for (int i = tid; i < n4; i += NT * 4) {
             uint4 v[4];
 #pragma unroll
@@ -360,57 +513,8 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
             }
         }
     }
-    if (SRC == ROWS_MESSAGES) {
-        // rows 0..M-1 empty, row M all ones over the graph slots (pads the lists), row M+1 empty
-        const int used = tg.slot_words == 0 ? tw : tg.gpt * tg.slot_words;
-        for (int i = tid; i < a.M * tw; i += NT) bt[i] = 0u;
-        for (int i = tid; i < tw; i += NT) {
-            bt[a.M * tw + i] = i < used ? 0xFFFFFFFFu : 0u;
-            bt[(a.M + 1) * tw + i] = 0u;
-        }
-    }
     for (int i = tid; i < TILE_LDS_PAD_WORDS + tg.gpt * K; i += NT) bt[(size_t)n_rows_lds * tw + i] = 0;
     __syncthreads();
-
-    if (SRC == ROWS_MESSAGES) {
-        // Row M+1: slot bit 0 of the graphs without nodes.  The reference's chunk arithmetic leaves
-        // every clause true for such a graph at every layer (kernels.py:443-466,505-527 never
-        // enter their node loop); the tile carries that in slot bit 0, which message literals
-        // therefore must not clear.
-        for (int j = tid; j < tg.gpt; j += NT) {
-            const int64_t g = (int64_t)tile * tg.gpt + j;
-            if (g < a.G && a.n_nodes[g] == 0u) {
-                const int pos = j * tg.slot_bits;
-                atomicOr(&bt[(a.M + 1) * tw + (pos >> 5)], 1u << (pos & 31));
-            }
-        }
-        // every true (clause, node slot) marks its clause's rotated hypervector bits at the node's out-neighbours
-        for (int c = wave; c < C; c += NWAVES) {
-            const uint32_t *truth = bitmap + (int64_t)c * tw;
-            for (int w = lane; w < tw; w += 64) {
-                uint32_t word = truth[w];
-                while (word) {
-                    const int pos = (w << 5) + __ffs(word) - 1;
-                    word &= word - 1;
-                    const int j = pos / tg.slot_bits, n = pos - j * tg.slot_bits;
-                    const int64_t g = (int64_t)tile * tg.gpt + j;
-                    if (g >= a.G || (uint32_t)n >= a.n_nodes[g]) continue;
-                    const int64_t row = (int64_t)a.node_index[g] + n;
-                    const uint32_t ne = a.n_edges[row];
-                    const int64_t e0 = a.edge_index[row];
-                    for (uint32_t e = 0; e < ne; ++e) {
-                        const uint32_t dst = a.edge[(e0 + e) * 2], type = a.edge[(e0 + e) * 2 + 1];
-                        const int dpos = j * tg.slot_bits + (int)dst;
-                        for (int b = 0; b < a.MB; ++b) {
-                            const uint32_t p = (a.hv[(int64_t)c * a.MB + b] + type) % (uint32_t)a.M;
-                            atomicOr(&bt[p * tw + (dpos >> 5)], 1u << (dpos & 31));
-                        }
-                    }
-                }
-            }
-        }
-        __syncthreads();
-    }
 
     // Lanes past the row width: their running AND starts at 0 and stays 0.  In LDS they read the
     // words after the row (inside the allocation) so that they fall on banks no other lane of
@@ -536,36 +640,60 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
         }
     };
 
-    // Two clauses per trip so that the chunk fetched ahead never has to be copied.  Pointers step
-    // by NWAVES clauses; past the end they stay on the wave's last clause (a valid address whose
-    // data is not used).
-    const int64_t list_step = (int64_t)NWAVES * a.stride;
-    const int wt_step = NWAVES * K;
-    const int64_t truth_step = (int64_t)NWAVES * tw * 4;
-    const int first = wave < C ? wave : 0;
-    const uint32_t *list_a = a.lists + (int64_t)first * a.stride;
-    const int32_t *wt_a = LAST ? a.wt + (int64_t)first * K : nullptr;
-    char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
-    Chunk32 ca = *reinterpret_cast<const Chunk32 *>(list_a);
-    LaneWords<LW> ta, tb;
+    if (SRC == ROWS_MESSAGES) {
+        // Message layers: most clauses are already false at every node slot of the tile.  A wave
+        // reads the truth rows of 8 of its clauses at once and fetches the list of, and evaluates,
+        // only those that are still true somewhere.
+        constexpr int GROUP = 8;
+        for (int c0 = wave; c0 < C; c0 += GROUP * NWAVES) {
+            LaneWords<LW> t[GROUP];
 #pragma unroll
-    for (int u = 0; u < LW; ++u) ta.w[u] = tb.w[u] = 0u;
-    if (SRC == ROWS_MESSAGES && active) ta.load(truth_a);
-    for (int c = wave; c < C; c += 2 * NWAVES) {
-        const bool has_b = c + NWAVES < C;
-        const uint32_t *list_b = has_b ? list_a + list_step : list_a;
-        const int32_t *wt_b = LAST ? (has_b ? wt_a + wt_step : wt_a) : nullptr;
-        char *truth_b = has_b ? truth_a + truth_step : truth_a;
-        const Chunk32 cb = *reinterpret_cast<const Chunk32 *>(list_b);
-        if (SRC == ROWS_MESSAGES && active) tb.load(truth_b);
-        evaluate(ca, list_a, wt_a, ta, truth_a);
-        const bool has_a = c + 2 * NWAVES < C;
-        list_a = has_a ? list_b + list_step : list_b;
-        if (LAST) wt_a = has_a ? wt_b + wt_step : wt_b;
-        truth_a = has_a ? truth_b + truth_step : truth_b;
-        ca = *reinterpret_cast<const Chunk32 *>(list_a);
-        if (SRC == ROWS_MESSAGES && active) ta.load(truth_a);
-        if (has_b) evaluate(cb, list_b, wt_b, tb, truth_b);
+            for (int g = 0; g < GROUP; ++g) {
+                const int c = c0 + g * NWAVES;
+#pragma unroll
+                for (int u = 0; u < LW; ++u) t[g].w[u] = 0u;
+                if (c < C && active) t[g].load(reinterpret_cast<const char *>(bitmap + (int64_t)c * tw + lane * LW));
+            }
+#pragma unroll
+            for (int g = 0; g < GROUP; ++g) {
+                const int c = c0 + g * NWAVES;
+                if (c < C && __ballot(any_bit(t[g])) != 0) {
+                    const uint32_t *list = a.lists + (int64_t)c * a.stride;
+                    const Chunk32 head = *reinterpret_cast<const Chunk32 *>(list);
+                    evaluate(head, list, LAST ? a.wt + (int64_t)c * K : nullptr, t[g],
+                             reinterpret_cast<char *>(bitmap + (int64_t)c * tw + (active ? lane * LW : 0)));
+                }
+            }
+        }
+    } else {
+        // Two clauses per trip so that the chunk fetched ahead never has to be copied.  Pointers step
+        // by NWAVES clauses; past the end they stay on the wave's last clause (a valid address whose
+        // data is not used).
+        const int64_t list_step = (int64_t)NWAVES * a.stride;
+        const int wt_step = NWAVES * K;
+        const int64_t truth_step = (int64_t)NWAVES * tw * 4;
+        const int first = wave < C ? wave : 0;
+        const uint32_t *list_a = a.lists + (int64_t)first * a.stride;
+        const int32_t *wt_a = LAST ? a.wt + (int64_t)first * K : nullptr;
+        char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
+        Chunk32 ca = *reinterpret_cast<const Chunk32 *>(list_a);
+        LaneWords<LW> none;
+#pragma unroll
+        for (int u = 0; u < LW; ++u) none.w[u] = 0u;
+        for (int c = wave; c < C; c += 2 * NWAVES) {
+            const bool has_b = c + NWAVES < C;
+            const uint32_t *list_b = has_b ? list_a + list_step : list_a;
+            const int32_t *wt_b = LAST ? (has_b ? wt_a + wt_step : wt_a) : nullptr;
+            char *truth_b = has_b ? truth_a + truth_step : truth_a;
+            const Chunk32 cb = *reinterpret_cast<const Chunk32 *>(list_b);
+            evaluate(ca, list_a, wt_a, none, truth_a);
+            const bool has_a = c + 2 * NWAVES < C;
+            list_a = has_a ? list_b + list_step : list_b;
+            if (LAST) wt_a = has_a ? wt_b + wt_step : wt_b;
+            truth_a = has_a ? truth_b + truth_step : truth_b;
+            ca = *reinterpret_cast<const Chunk32 *>(list_a);
+            if (has_b) evaluate(cb, list_b, wt_b, none, truth_b);
+        }
     }
     if (!LAST) return;
     __syncthreads();
