@@ -383,29 +383,6 @@ __global__ void k_select_clause_updates(int32_t *weights, const int32_t *__restr
     }
 }
 
-// kernels.py:55-96 on one word of 32 automata held as B bit planes.
-__device__ __forceinline__ void ta_inc(uint32_t *ta, int B, uint32_t active) {
-    uint32_t carry = active;
-    for (int b = 0; b < B && carry; ++b) {
-        uint32_t v = ta[b];
-        ta[b] = v ^ carry;
-        carry &= v;
-    }
-    if (carry)
-        for (int b = 0; b < B; ++b) ta[b] |= carry;
-}
-
-__device__ __forceinline__ void ta_dec(uint32_t *ta, int B, uint32_t active) {
-    uint32_t carry = active;
-    for (int b = 0; b < B && carry; ++b) {
-        uint32_t v = ta[b];
-        ta[b] = v ^ carry;
-        carry &= ~v;
-    }
-    if (carry)
-        for (int b = 0; b < B; ++b) ta[b] &= ~carry;
-}
-
 #include "fit_fused.h"
 #include "fit_deep.h"
 #include "fit_persistent.h"
@@ -786,6 +763,48 @@ int launch_two_phase(const TileLayerArgs &a, int n_tiles, int la4, bool last, hi
     }
 }
 
+template <int NW, int LW, int SRC, bool LAST>
+int launch_two_phase_wide_as(const TileLayerArgs &a, int n_tiles, int LA, hipStream_t st) {
+    // rows (if staged), padding, class sums, and the first node and node count of the tile's graphs
+    size_t lds = tile_layer_lds_bytes(a.tg, a.K, SRC, a.M) + (size_t)a.tg.gpt * 8;
+    static thread_local size_t lds_set = 0;
+    if (lds > lds_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)k_tile_two_phase_wide<NW, LW, SRC, LAST>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
+        lds_set = lds;
+    }
+    // rows read in place and no votes: several workgroups share a tile's clauses until the chip is full
+    int splits = 1;
+    if (SRC == ROWS_GLOBAL && !LAST) {
+        splits = 2048 / (n_tiles > 0 ? n_tiles : 1);
+        splits = splits < 1 ? 1 : (splits > 16 ? 16 : splits);
+    }
+    profile_start(LAST ? "k_tile_two_phase_wide<score>" : "k_tile_two_phase_wide<layer0>", st);
+    hipLaunchKernelGGL((k_tile_two_phase_wide<NW, LW, SRC, LAST>), dim3(n_tiles, splits), dim3(NW * 64), lds, st, a, LA);
+    if (int rc = check_launch("tile_two_phase_wide")) return rc;
+    profile_stop(st);
+    return GTM_OK;
+}
+
+template <int NW, int LW>
+int launch_two_phase_wide_lw(const TileLayerArgs &a, int n_tiles, int LA, bool staged, bool last, hipStream_t st) {
+    if (staged)
+        return last ? launch_two_phase_wide_as<NW, LW, ROWS_STAGED, true>(a, n_tiles, LA, st)
+                    : launch_two_phase_wide_as<NW, LW, ROWS_STAGED, false>(a, n_tiles, LA, st);
+    return last ? launch_two_phase_wide_as<NW, LW, ROWS_GLOBAL, true>(a, n_tiles, LA, st)
+                : launch_two_phase_wide_as<NW, LW, ROWS_GLOBAL, false>(a, n_tiles, LA, st);
+}
+
+int launch_two_phase_wide(const TileLayerArgs &a, int n_tiles, int LA, bool staged, bool last, hipStream_t st) {
+    constexpr int NW = 16;
+    switch (a.tg.lw) {
+        case 1: return launch_two_phase_wide_lw<NW, 1>(a, n_tiles, LA, staged, last, st);
+        case 2: return launch_two_phase_wide_lw<NW, 2>(a, n_tiles, LA, staged, last, st);
+        default: return launch_two_phase_wide_lw<NW, 4>(a, n_tiles, LA, staged, last, st);
+    }
+}
+
 // Layer 0 can run in two phases (k_tile_two_phase) on tiles of whole-word graph slots staged in
 // LDS when a node has 4, 8, 12 or 16 literal words.  GTM_NO_TWO_PHASE (tuning aid) turns it off.
 bool two_phase_layer0(const Dims &d, const gtm_graphs *g, const TileGeom &tg) {
@@ -800,7 +819,10 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                    const ScoreWs &w, int first, int n_graphs, int batch, int32_t *class_sum, hipStream_t st) {
     const uint32_t *order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
     const int layers = cfg->depth;
-    const bool two_phase = two_phase_layer0(d, g, tg);
+    const bool narrow = two_phase_layer0(d, g, tg);
+    // any other tile of whole-word slots whose row offsets fit the 16-bit entries: k_tile_two_phase_wide
+    const bool wide = !narrow && tg.slot_words > 0 && (int64_t)tg.rows * tg.tw / 4 < 65536 && !getenv("GTM_NO_TWO_PHASE");
+    const bool two_phase = narrow || wide;
     const int stride0 = two_phase ? 8 + d.LA : w.list_stride;
     if (two_phase)
         hipLaunchKernelGGL(k_compile_clauses_two_phase, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state,
@@ -828,20 +850,16 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     a.wt = w.wt;
     a.bitmap = w.tile_bitmap;
     a.M = d.M;
-    a.MB = d.MB;
     a.G = g->number_of_graphs;
-    a.hv = s->hypervectors;
     a.node_index = g->node_index;
     a.n_nodes = g->number_of_graph_nodes;
-    a.n_edges = g->number_of_graph_node_edges;
-    a.edge_index = g->edge_index;
-    a.edge = g->edge;
     a.X = g->X;
     auto layer0 = [&](int n_tiles, bool last) {
         a.lists = w.lists;
         a.stride = stride0;
-        return two_phase ? launch_two_phase(a, n_tiles, d.LA / 4, last, st)
-                         : launch_tile_layer(a, n_tiles, tg.stage0 ? ROWS_STAGED : ROWS_GLOBAL, last, st);
+        if (narrow) return launch_two_phase(a, n_tiles, d.LA / 4, last, st);
+        if (wide) return launch_two_phase_wide(a, n_tiles, d.LA, tg.stage0 != 0, last, st);
+        return launch_tile_layer(a, n_tiles, tg.stage0 ? ROWS_STAGED : ROWS_GLOBAL, last, st);
     };
     if (layers == 1) {
         // no truth rows are kept: every tile of the range in one launch

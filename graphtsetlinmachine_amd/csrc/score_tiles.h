@@ -1,4 +1,4 @@
-// Batched depth-1 inference on literal-major tiles.
+// Batched inference on literal-major tiles.
 //
 // The dense form of clause evaluation tests every clause against every word
 // of every node (CLAUSES x nodes x LA_CHUNKS word operations per graph) and is
@@ -7,9 +7,11 @@
 // one bit-row per LITERAL (bit n of the row = that literal at node slot n of
 // the tile), staged in LDS, and a clause's truth over all node slots of the
 // tile is the AND of the rows of its included literals only.  The result is
-// the same bits as kernels.py:443-466 computes; no clause/node bitmap is
-// written because `evaluate` (kernels.py:297-315) only needs "true at some
-// node of the graph".
+// the same bits as kernels.py:443-466 computes.  At depth 1 no clause/node
+// bitmap is written because `evaluate` (kernels.py:297-315) only needs "true
+// at some node of the graph"; with message layers the truth rows of a launch's
+// tiles pass from layer to layer in the same slot layout, and each layer's
+// messages are built literal-major as well.
 //
 // Tile layout in HBM (built once per data set by k_build_tiles):
 //   tiles[tile][row][tw] uint32, rows = LITERALS + node_types + 1
@@ -293,10 +295,8 @@ struct TileLayerArgs {
     int tile0, first_graph, n_graphs;
     int32_t *class_sum;     // [n_graphs][K] (last layer)
     uint32_t *bitmap;       // [tiles of the launch][C][tw]: clause truth per node slot, read and written in place
-    // message layers
-    int M, MB, G;
-    const uint32_t *hv;     // [C][MB]
-    const uint32_t *node_index, *n_nodes, *n_edges, *edge_index, *edge;
+    int M, G;               // message size; graphs in the data set
+    const uint32_t *node_index, *n_nodes;
     const uint32_t *X;      // [nodes][LA] node-major literal words (two-phase layer 0)
     const uint32_t *message_rows;  // [tiles of the launch][M + 2][tw] (message layers, built by k_tile_pack_messages)
 };
@@ -1011,6 +1011,154 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
         finish(pa, ma);
     }
     finish(pb, mb);
+    if (!LAST) return;
+    __syncthreads();
+    const int64_t g0 = (int64_t)tile * tg.gpt;
+    for (int i = tid; i < tg.gpt * K; i += NT) {
+        int64_t g = g0 + i / K;
+        if (g >= a.first_graph && g < (int64_t)a.first_graph + a.n_graphs)
+            a.class_sum[(g - a.first_graph) * K + (i % K)] = sums[i];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// The two-phase layer 0 for nodes with many literal words (any LA), tiles of
+// whole-word slots whose rows are staged in LDS or read in place.  Phase 1 as
+// above; in phase 2 the surviving node slots are walked on the scalar unit, 8 at
+// a time, and for each one lane w compares include word w with the node's
+// literal word w (one coalesced load per node and 64 words).  With the rows
+// read in place nothing ties a tile to one workgroup, so gridDim.y workgroups
+// share a tile's clauses (truth rows only: the votes of LAST need one
+// workgroup per tile).
+template <int NWAVES, int LW, int SRC, bool LAST>
+__global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerArgs a, int LA) {
+    extern __shared__ uint32_t lds[];
+    const TileGeom &tg = a.tg;
+    const int tw = tg.tw, C = a.C, K = a.K;
+    constexpr int NT = NWAVES * 64;
+    const int n_rows_lds = SRC == ROWS_STAGED ? tg.rows : 0;
+    uint32_t *bt = lds;
+    int32_t *sums = (int32_t *)(lds + (size_t)n_rows_lds * tw + TILE_LDS_PAD_WORDS);
+    uint32_t *first_node = (uint32_t *)(sums + tg.gpt * K);  // [gpt] row of X of each graph's node 0
+    uint32_t *node_count = first_node + tg.gpt;              // [gpt]
+    const int tile = a.tile0 + blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    uint32_t *bitmap = a.bitmap + (int64_t)blockIdx.x * C * tw;
+
+    if (SRC == ROWS_STAGED) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.tiles + (int64_t)tile * tg.rows * tw);
+        uint4 *dst = reinterpret_cast<uint4 *>(bt);
+        const int n4 = (tg.rows * tw) >> 2;
+        for (int i = tid; i < n4; i += NT) dst[i] = src[i];
+    }
+    for (int i = tid; i < TILE_LDS_PAD_WORDS + tg.gpt * K; i += NT) bt[(size_t)n_rows_lds * tw + i] = 0;
+    for (int j = tid; j < tg.gpt; j += NT) {
+        const int64_t g = (int64_t)tile * tg.gpt + j;
+        first_node[j] = g < a.G ? a.node_index[g] : 0u;
+        node_count[j] = g < a.G ? a.n_nodes[g] : 0u;
+    }
+    __syncthreads();
+
+    const bool active = lane * LW < tw;
+    const char *col = SRC == ROWS_GLOBAL
+                          ? reinterpret_cast<const char *>(a.tiles + (int64_t)tile * tg.rows * tw + (active ? lane * LW : 0))
+                          : reinterpret_cast<const char *>(bt + lane * LW);
+    const int pairs = tg.gpt * K;
+    const int my_shift = (lane < tg.gpt ? lane : 0) * tg.lanes_per_graph;
+    const unsigned long long slot_lanes = tg.lanes_per_graph >= 64 ? ~0ull : (1ull << tg.lanes_per_graph) - 1ull;
+
+    auto any_bit = [](const LaneWords<LW> &x) {
+        uint32_t m = x.w[0];
+#pragma unroll
+        for (int u = 1; u < LW; ++u) m |= x.w[u];
+        return m != 0;
+    };
+    auto entry_of = [](const Packed8 &rec, int i) { return ((rec.v[i >> 1] >> ((i & 1) * 16)) & 0xFFFFu) << 4; };
+
+    const int c_step = NWAVES * gridDim.y;
+    const int c_first = wave + NWAVES * blockIdx.y;
+    const int valid = c_first < C ? c_first : 0;
+    Packed8 next = *reinterpret_cast<const Packed8 *>(a.lists + (int64_t)valid * a.stride);
+    for (int c = c_first; c < C; c += c_step) {
+        const uint32_t *record = a.lists + (int64_t)c * a.stride;
+        const Packed8 rec = next;
+        next = *reinterpret_cast<const Packed8 *>(a.lists + (int64_t)(c + c_step < C ? c + c_step : valid) * a.stride);
+        const uint32_t header = rec.v[0] & 0xFFFFu;
+        // the first 64 include words travel with the rows (phase 2 would otherwise wait for them alone)
+        const uint32_t include0 = lane < LA ? record[8 + lane] : 0u;
+        LaneWords<LW> acc;
+#pragma unroll
+        for (int u = 0; u < LW; ++u) acc.w[u] = active ? 0xFFFFFFFFu : 0u;
+        {
+            LaneWords<LW> r[15];
+            if ((header & 0xFFu) > 7u) {
+#pragma unroll
+                for (int i = 0; i < 15; ++i) r[i].load(col + entry_of(rec, i + 1));
+#pragma unroll
+                for (int i = 0; i < 15; ++i)
+#pragma unroll
+                    for (int u = 0; u < LW; ++u) acc.w[u] &= r[i].w[u];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 7; ++i) r[i].load(col + entry_of(rec, i + 1));
+#pragma unroll
+                for (int i = 0; i < 7; ++i)
+#pragma unroll
+                    for (int u = 0; u < LW; ++u) acc.w[u] &= r[i].w[u];
+            }
+        }
+        unsigned long long nz = __ballot(any_bit(acc));
+        if ((header & 0x100u) && nz != 0) {
+            for (int w0 = 0; w0 < LA; w0 += 64) {
+                const bool in_row = w0 + lane < LA;
+                const uint32_t include = w0 == 0 ? include0 : (in_row ? record[8 + w0 + lane] : 0u);
+                unsigned long long live = __ballot(any_bit(acc));
+                while (live) {
+                    const int L = __ffsll((long long)live) - 1;
+                    live &= live - 1;
+#pragma unroll
+                    for (int u = 0; u < LW; ++u) {
+                        uint32_t word = __builtin_amdgcn_readlane(acc.w[u], L);
+                        const int tile_word = L * LW + u;                 // word of the tile row
+                        const int gj = tile_word / tg.slot_words;         // graph of the tile
+                        const int node0 = (tile_word - gj * tg.slot_words) * 32;
+                        if (node_count[gj] == 0u) continue;               // a graph without nodes keeps its bit
+                        const uint32_t *x = a.X + ((int64_t)first_node[gj] + node0) * LA + w0 + (in_row ? lane : 0);
+                        uint32_t cleared = 0;
+                        while (word) {
+                            int bit[8];
+#pragma unroll
+                            for (int q = 0; q < 8; ++q) {
+                                bit[q] = word ? __builtin_ctz(word) : -1;
+                                word &= word - 1;
+                            }
+                            uint32_t xs[8];
+#pragma unroll
+                            for (int q = 0; q < 8; ++q) xs[q] = x[(int64_t)(bit[q] < 0 ? 0 : bit[q]) * LA];
+#pragma unroll
+                            for (int q = 0; q < 8; ++q)
+                                if (bit[q] >= 0 && __ballot((include & ~xs[q]) != 0) != 0) cleared |= 1u << bit[q];
+                        }
+                        if (lane == L) acc.w[u] &= ~cleared;
+                    }
+                }
+            }
+            nz = __ballot(any_bit(acc));
+        }
+        if (!LAST) {
+            if (active) acc.store(reinterpret_cast<char *>(bitmap + (int64_t)c * tw + lane * LW));
+            continue;
+        }
+        if (nz == 0) continue;
+        const int32_t *weights_of_clause = a.wt + (int64_t)c * K;
+        const unsigned long long gm = __ballot(lane < tg.gpt && ((nz >> my_shift) & slot_lanes) != 0);
+        for (int p = lane; p < pairs; p += 64) {
+            int j = p / K, k = p - j * K;
+            if ((gm >> j) & 1ull) atomicAdd(&sums[p], weights_of_clause[k]);
+        }
+    }
     if (!LAST) return;
     __syncthreads();
     const int64_t g0 = (int64_t)tile * tg.gpt;

@@ -227,6 +227,9 @@ TILE_SHAPES = [
     dict(seed=15, g=dict(n_graphs=23, max_nodes=361, min_nodes=300, hv_size=128, max_degree=0), classes=10, clauses=120),
     dict(seed=16, g=dict(n_graphs=5, max_nodes=2048, min_nodes=1990, hv_size=16, max_degree=0, node_types=("a", "b", "c")),
          classes=2, clauses=40),
+    # 5 literal words per node (layer 0 in two phases, nodes tested word-parallel)
+    dict(seed=19, g=dict(n_graphs=25, max_nodes=90, min_nodes=30, hv_size=80, n_symbols=12, node_types=("a", "b")),
+         classes=3, clauses=70),
     # 12 and 16 literal words per node (layer 0 in two phases)
     dict(seed=17, g=dict(n_graphs=30, max_nodes=100, min_nodes=20, hv_size=192, n_symbols=12), classes=3, clauses=90),
     dict(seed=18, g=dict(n_graphs=20, max_nodes=50, hv_size=256, n_symbols=12, node_types=("a", "b")), classes=4,
