@@ -1,0 +1,82 @@
+"""The 361-node convolutional configuration at its full test size (10,000 graphs, 2,500 clauses):
+properties that do not need the oracle to finish a 10,000-graph run.
+
+* a sample of the class sums equals the oracle;
+* scoring is a per-graph function: a shuffled subset of the graphs scores to the same rows, whatever
+  tile a graph lands in;
+* transform (per-operator kernels, clause/node bitmaps materialised) and score (tile kernels) agree:
+  class sums identical, and the sums recomputed from the transformed clause outputs and the
+  weights equal both;
+* scoring twice gives the same result."""
+
+import numpy as np
+import pytest
+
+from graphtsetlinmachine_amd import workloads
+from oracle import gtm_oracle as o
+from tests.test_gpu_model import oracle_twin
+
+pytestmark = pytest.mark.gpu
+
+
+def test_convolutional_configuration_at_full_test_size():
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    wl = workloads.convolutional_images(n_train=8000, n_test=10000)
+    np.random.seed(42)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
+    test = wl.graphs_test
+    sums = tm.score(test)
+    assert sums.shape == (10000, 10)
+    assert np.array_equal(tm.score(test), sums)
+    assert (sums.argmax(axis=1) == wl.Y_test).mean() > 0.9
+
+    # the oracle on a sample spread over the set (first and last tile included)
+    model = oracle_twin(tm, wl.graphs_train)
+    model.ta_state = tm.get_state()[0].reshape(model.ta_state.shape).copy()
+    model.clause_weights = tm.get_weights().copy()
+    model.cfg = oracle_twin(tm, test).cfg
+    sample = [0, 1, 9, 10, 4999, 5003, 9989, 9999]
+    assert np.array_equal(sums[sample], o.score(model, test, sample))
+
+    # a shuffled subset lands in other tiles and other slots
+    rng = np.random.default_rng(7)
+    picked = rng.permutation(10000)[:3001]
+    assert np.array_equal(tm.score(test[picked]), sums[picked])
+
+    # the bitmap path: same sums, and clause outputs that reproduce them through the weights
+    part = test[np.arange(2000, 3000)]
+    fired, part_sums = tm.transform(part)
+    assert np.array_equal(part_sums, sums[2000:3000])
+    assert np.array_equal(fired.astype(np.int64) @ tm.get_weights().T.astype(np.int64), part_sums)
+
+
+def test_sequence_chains_at_full_test_size():
+    """The same properties for a model with a message layer: 5,000 chains of 1,000 nodes."""
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    wl = workloads.sequence_chains(n_train=300, n_test=5000)
+    np.random.seed(42)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
+    test = wl.graphs_test
+    sums = tm.score(test)
+    assert sums.shape == (5000, 2) and np.array_equal(tm.score(test), sums)
+
+    state = tm.get_state()
+    model = oracle_twin(tm, test)
+    model.ta_state = state[0].reshape(model.ta_state.shape).copy()
+    model.message_ta_state = [b.reshape(model.message_ta_state[0].shape).copy() for b in tm.save()["message_ta_state"]]
+    model.clause_weights = tm.get_weights().copy()
+    sample = [0, 1, 2, 2499, 4998, 4999]
+    assert np.array_equal(sums[sample], o.score(model, test, sample))
+
+    rng = np.random.default_rng(8)
+    picked = rng.permutation(5000)[:1001]
+    assert np.array_equal(tm.score(test[picked]), sums[picked])
+
+    part = test[np.arange(1000, 1300)]
+    fired, part_sums = tm.transform(part)
+    assert np.array_equal(part_sums, sums[1000:1300])
+    assert np.array_equal(fired.astype(np.int64) @ tm.get_weights().T.astype(np.int64), part_sums)
