@@ -109,7 +109,8 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
     int32_t *votes = sums + K;                                 // [K] this group's share of the class sums
     uint32_t *gate = (uint32_t *)(votes + K);                  // [own][K][2] random words of the feedback gates
     uint32_t *fbits = gate + 2 * (size_t)own_max * K;          // [own][LA][K] Type I feedback bits
-    __shared__ int go_on;
+    int32_t *pair_list = (int32_t *)(fbits + (size_t)own_max * LA * K);  // [own * K] (clause, class) pairs with Type I feedback
+    __shared__ int go_on, n_pairs;
 
     // own state -> LDS
     for (int k = tid; k < K; k += FITP_BLOCK) votes[k] = 0;
@@ -133,6 +134,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
     __syncthreads();
 
     const int ones_row = p.literals + p.n_types;
+    int div_words = 0, div_dr = 0, div_r0 = 0;
     for (int i = 0; i < p.n_examples; ++i) {
         const int ex = p.first_example + i;
         const uint32_t step = p.first_step + (uint32_t)i;
@@ -149,8 +151,13 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         {
             // element at = row * words + w; a thread's elements are FITP_BLOCK apart: step (row, w) without dividing
             const uint32_t *tile = p.tiles + (int64_t)fn.tile * p.tg.rows * p.tg.tw + fn.word0;
-            const int dr = FITP_BLOCK / fn.words, dw = FITP_BLOCK - dr * fn.words;
-            int r = tid / fn.words, w = tid - r * fn.words;
+            if (fn.words != div_words) {  // the divisions are redone only when the slot width changes
+                div_words = fn.words;
+                div_dr = FITP_BLOCK / fn.words;
+                div_r0 = tid / fn.words;
+            }
+            const int dr = div_dr, dw = FITP_BLOCK - dr * fn.words;
+            int r = div_r0, w = tid - r * fn.words;
 #pragma unroll
             for (int u = 0; u < FITP_PREFETCH; ++u) {
                 pre[u] = tid + u * FITP_BLOCK < next_total ? tile[(int64_t)r * p.tg.tw + w] : 0u;
@@ -255,14 +262,16 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             gate[2 * j] = r.v[0];
             gate[2 * j + 1] = r.v[1];
         }
-        uint32_t x_mine = 0;  // literals word of this thread's (clause, word) item, first pass of the update loop
+        if (tid == 0) go_on = 1;
+        __syncthreads();
+        // requested now, so that it travels while the sums are polled: the literals word of this
+        // thread's (clause, word) item in the first pass of the update loop
+        uint32_t x_mine = 0;
         if (tid < n_own * LA) {
             const int cl = tid / LA, w = tid - cl * LA;
             const int node = node_of[cl];
             if (node != -1) x_mine = p.X[((int64_t)base_now + node) * LA + w];
         }
-        if (tid == 0) go_on = 1;
-        __syncthreads();
         for (int k = tid; k < K; k += FITP_BLOCK) {
             uint32_t polls = 0;
             unsigned long long word;
@@ -314,12 +323,26 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             upd[j] = u;
         }
         __syncthreads();
-        // Type I feedback bits, one thread per (clause, word, class) that needs them
-        for (int j = tid; j < n_own * LA * K; j += FITP_BLOCK) {
-            const int k = j % K, cw = j / K;
-            const int cl = cw / LA, w = cw - cl * LA;
-            if (upd[cl * K + k] > 0)
-                fbits[j] = gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
+        // Type I feedback bits for the (clause, class) pairs that need them: the pairs are listed
+        // first (wave 0, ballots), then one thread per (listed pair, word) draws the bits, so that
+        // the lanes that run the generator are (nearly) all busy
+        if (wave == 0) {
+            int n_listed = 0;
+            for (int j0 = 0; j0 < n_own * K; j0 += 64) {
+                const int j = j0 + lane;
+                const bool need = j < n_own * K && upd[j] > 0;
+                const unsigned long long m = __ballot(need);
+                if (need) pair_list[n_listed + __popcll(m & ((1ull << lane) - 1ull))] = j;
+                n_listed += __popcll(m);
+            }
+            if (lane == 0) n_pairs = n_listed;
+        }
+        __syncthreads();
+        for (int t = tid; t < n_pairs * LA; t += FITP_BLOCK) {
+            const int j = pair_list[t / LA], w = t % LA;
+            const int cl = j / K, k = j - cl * K;
+            fbits[((size_t)cl * LA + w) * K + k] =
+                gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
         }
         __syncthreads();
         const uint32_t *X_rows = p.X + (int64_t)base_now * LA;

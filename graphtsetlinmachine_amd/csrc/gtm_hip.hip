@@ -1292,7 +1292,7 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     const int waves = FITP_BLOCK / 64;
     auto lds_bytes = [&](int per_group) {
         return (2 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group +
-                2 * (size_t)d.K + 4 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K) * 4;
+                2 * (size_t)d.K + 5 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K) * 4;
     };
     const size_t lds_limit = 150 * 1024;
     int per_group = (d.C + cus - 1) / cus;
