@@ -50,6 +50,8 @@ struct FitPersistParams {
     int clauses_per_group;
     int rows_words;       // LDS words of one staged graph: (literals + n_types + 1) * max slot words
     int max_words;        // words per graph slot that can hold nodes
+    const uint32_t *order;  // literals sorted by how often they hold in the data set, rarest first
+    int x_words;          // LDS words of one graph's node-major literal words: max nodes * LA
 };
 
 __device__ __forceinline__ void fitp_stage_rows(const FitPersistParams &p, const FitGraph &fg, uint32_t *dst, int tid) {
@@ -80,6 +82,9 @@ __device__ __forceinline__ void fitp_stage_rows(const FitPersistParams &p, const
 constexpr unsigned long long FITP_BIAS = 1ull << 47;      // a class sum s is stored as s + FITP_BIAS in bits 0..47
 constexpr unsigned long long FITP_ARRIVED = 1ull << 48;   // one arrival in bits 48..63
 constexpr int FITP_PREFETCH = 8;  // words of the next graph's rows a thread holds in registers while evaluating
+constexpr int FITP_PREFETCH_X = 4;  // the same for the next graph's node-major literal words
+constexpr int FITP_WALK_ALL = 24;   // clauses with at most this many literals AND all their rows
+constexpr int FITP_FILTER_ROWS = 16;  // rows the others AND before testing the surviving nodes
 
 // Address of element `i` of the staged rows (i = row * words + w) inside the graph's tile.
 __device__ __forceinline__ const uint32_t *fitp_row_word(const FitPersistParams &p, const FitGraph &fg, int i) {
@@ -110,6 +115,9 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
     uint32_t *gate = (uint32_t *)(votes + K);                  // [own][K][2] random words of the feedback gates
     uint32_t *fbits = gate + 2 * (size_t)own_max * K;          // [own][LA][K] Type I feedback bits
     int32_t *pair_list = (int32_t *)(fbits + (size_t)own_max * LA * K);  // [own * K] (clause, class) pairs with Type I feedback
+    uint32_t *x_buf[2] = {(uint32_t *)(pair_list + (size_t)own_max * K),
+                          (uint32_t *)(pair_list + (size_t)own_max * K) + p.x_words};  // [nodes][LA] of the graph
+    uint32_t *order_lds = x_buf[1] + p.x_words;                 // [literals]
     __shared__ int go_on, n_pairs;
 
     // own state -> LDS
@@ -130,7 +138,9 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         base_next = p.node_index[e1];
         FitGraph fg0 = fit_graph_slot(p.tg, p.first_example, n_now);
         fitp_stage_rows(p, fg0, rows_buf[0], tid);
+        for (int at = tid; at < n_now * LA; at += FITP_BLOCK) x_buf[0][at] = p.X[(int64_t)base_now * LA + at];
     }
+    for (int l = tid; l < p.literals; l += FITP_BLOCK) order_lds[l] = p.order[l];
     __syncthreads();
 
     const int ones_row = p.literals + p.n_types;
@@ -169,6 +179,15 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 }
             }
         }
+        uint32_t pre_x[FITP_PREFETCH_X];
+        const int next_x_total = has_next ? n_next * LA : 0;
+        {
+            const uint32_t *src = p.X + (int64_t)base_next * LA;
+#pragma unroll
+            for (int u = 0; u < FITP_PREFETCH_X; ++u)
+                pre_x[u] = tid + u * FITP_BLOCK < next_x_total ? src[tid + u * FITP_BLOCK] : 0u;
+        }
+        const uint32_t *x_now = x_buf[i & 1];
         const int e2 = min(ex + 2, last);
         const int n_after = (int)p.n_nodes[e2];
         const uint32_t base_after = p.node_index[e2];
@@ -182,32 +201,92 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             const uint32_t *inc = ta + (size_t)cl * LA * B + (B - 1);
             uint32_t acc = active ? col[(p.literals + c % p.n_types) * stride] : 0u;
             int included = 0;
+            uint32_t first_words = 0;
             for (int w0 = 0; w0 < LA; w0 += 64) {
                 uint32_t mine = w0 + lane < LA ? inc[(w0 + lane) * B] : 0u;
                 if (w0 + lane == LA - 1) mine &= p.filter;
-                unsigned long long nonzero = __ballot(mine != 0);
-                while (nonzero) {
-                    const int wl = __ffsll((long long)nonzero) - 1;
-                    nonzero &= nonzero - 1;
-                    uint32_t m = __builtin_amdgcn_readlane(mine, wl);
-                    included += __popc(m);
-                    const int base = (w0 + wl) << 5;
-                    while (m) {
+                if (w0 == 0) first_words = mine;
+                included += __popc(mine);
+            }
+            for (int off = 32; off > 0; off >>= 1) included += __shfl_xor(included, off);
+            // A clause with many literals ANDs only the rows of its FITP_FILTER_ROWS rarest ones and then
+            // tests the few nodes that are left against its whole include mask on the nodes' own words.
+            const bool filter_only = included > FITP_WALK_ALL && n_now > 0;
+            if (filter_only) {
+                int budget = FITP_FILTER_ROWS;
+                for (int r0 = 0; r0 < p.literals && budget > 0; r0 += 64) {
+                    const int r = r0 + lane;
+                    const uint32_t lit = r < p.literals ? order_lds[r] : 0u;
+                    uint32_t word = inc[(lit >> 5) * B];
+                    if ((int)(lit >> 5) == LA - 1) word &= p.filter;
+                    unsigned long long picked = __ballot(r < p.literals && ((word >> (lit & 31u)) & 1u));
+                    while (picked && budget > 0) {
                         int row[8];
 #pragma unroll
                         for (int u = 0; u < 8; ++u) {
-                            row[u] = m ? base + __builtin_ctz(m) : ones_row;
-                            m &= m - 1;
+                            row[u] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
+                            picked &= picked - 1;
                         }
-                        uint32_t r[8];
+                        uint32_t r8[8];
 #pragma unroll
-                        for (int u = 0; u < 8; ++u) r[u] = col[row[u] * stride];
+                        for (int u = 0; u < 8; ++u) r8[u] = col[row[u] * stride];
 #pragma unroll
-                        for (int u = 0; u < 8; ++u) acc &= r[u];
+                        for (int u = 0; u < 8; ++u) acc &= r8[u];
+                        budget -= 8;
+                    }
+                }
+            } else {
+                for (int w0 = 0; w0 < LA; w0 += 64) {
+                    uint32_t mine = w0 == 0 ? first_words : (w0 + lane < LA ? inc[(w0 + lane) * B] : 0u);
+                    if (w0 != 0 && w0 + lane == LA - 1) mine &= p.filter;
+                    unsigned long long nonzero = __ballot(mine != 0);
+                    while (nonzero) {
+                        const int wl = __ffsll((long long)nonzero) - 1;
+                        nonzero &= nonzero - 1;
+                        uint32_t m = __builtin_amdgcn_readlane(mine, wl);
+                        const int base = (w0 + wl) << 5;
+                        while (m) {
+                            int row[8];
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) {
+                                row[u] = m ? base + __builtin_ctz(m) : ones_row;
+                                m &= m - 1;
+                            }
+                            uint32_t r[8];
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) r[u] = col[row[u] * stride];
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) acc &= r[u];
+                        }
                     }
                 }
             }
-            const uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
+            uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
+            if (filter_only) {
+                // lane L holds nodes 32 L .. 32 L + 31: the surviving ones are walked on the scalar unit; lane w
+                // compares include word w with the node's literal word w (LDS copy of the graph's X rows)
+                unsigned long long live = __ballot(v != 0);
+                while (live) {
+                    const int L = __ffsll((long long)live) - 1;
+                    live &= live - 1;
+                    uint32_t word = __builtin_amdgcn_readlane(v, L);
+                    uint32_t cleared = 0;
+                    while (word) {
+                        const int b = __builtin_ctz(word);
+                        word &= word - 1;
+                        const uint32_t *x = x_now + (L * 32 + b) * LA;
+                        bool violated = false;
+                        for (int w0 = 0; w0 < LA; w0 += 64) {
+                            uint32_t mine = w0 == 0 ? first_words : (w0 + lane < LA ? inc[(w0 + lane) * B] : 0u);
+                            if (w0 != 0 && w0 + lane == LA - 1) mine &= p.filter;
+                            const uint32_t xs = w0 + lane < LA ? x[w0 + lane] : 0xFFFFFFFFu;
+                            violated |= __ballot((mine & ~xs) != 0) != 0;
+                        }
+                        if (violated) cleared |= 1u << b;
+                    }
+                    if (lane == L) v &= ~cleared;
+                }
+            }
             const int pc = __popc(v);
             int true_nodes, before;
             wave_count_scan(pc, lane, &true_nodes, &before);
@@ -255,6 +334,14 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             }
             for (int at = tid + FITP_PREFETCH * FITP_BLOCK; at < next_total; at += FITP_BLOCK)
                 dst[at] = *fitp_row_word(p, fn, at);
+            uint32_t *dst_x = x_buf[(i + 1) & 1];
+#pragma unroll
+            for (int u = 0; u < FITP_PREFETCH_X; ++u) {
+                const int at = tid + u * FITP_BLOCK;
+                if (at < next_x_total) dst_x[at] = pre_x[u];
+            }
+            for (int at = tid + FITP_PREFETCH_X * FITP_BLOCK; at < next_x_total; at += FITP_BLOCK)
+                dst_x[at] = p.X[(int64_t)base_next * LA + at];
         }
         for (int j = tid; j < n_own * K; j += FITP_BLOCK) {
             const int cl = j / K, k = j - cl * K;
@@ -264,14 +351,6 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         }
         if (tid == 0) go_on = 1;
         __syncthreads();
-        // requested now, so that it travels while the sums are polled: the literals word of this
-        // thread's (clause, word) item in the first pass of the update loop
-        uint32_t x_mine = 0;
-        if (tid < n_own * LA) {
-            const int cl = tid / LA, w = tid - cl * LA;
-            const int node = node_of[cl];
-            if (node != -1) x_mine = p.X[((int64_t)base_now + node) * LA + w];
-        }
         for (int k = tid; k < K; k += FITP_BLOCK) {
             uint32_t polls = 0;
             unsigned long long word;
@@ -345,7 +424,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
         }
         __syncthreads();
-        const uint32_t *X_rows = p.X + (int64_t)base_now * LA;
+        const uint32_t *X_rows = x_now;  // the graph's literal words, node-major, in LDS
         for (int j = tid; j < n_own * LA; j += FITP_BLOCK) {
             const int cl = j / LA, w = j - cl * LA;
             const int32_t *u_of = upd + cl * K;
@@ -355,7 +434,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             const int node = node_of[cl];
             const bool fired = node != -1;
             const bool within = incl_of[cl] <= p.max_included;
-            const uint32_t x = !fired ? 0u : (j == tid ? x_mine : X_rows[(int64_t)node * LA + w]);
+            const uint32_t x = fired ? X_rows[node * LA + w] : 0u;
             feedback_word_any(ta + (size_t)j * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1,
                               (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, p.thr16, fbits + (size_t)j * K);
         }

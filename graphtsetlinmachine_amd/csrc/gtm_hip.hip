@@ -1287,12 +1287,15 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     FitPersistParams p{};
     p.max_words = tg.slot_words > 0 ? tg.slot_words : 1;
     p.rows_words = (cfg->literals + g->number_of_node_types + 1) * p.max_words;
+    p.x_words = (g->max_number_of_graph_nodes > 0 ? g->max_number_of_graph_nodes : 1) * d.LA;
+    p.order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
     // One clause per wave and step (16 per group) where that fits; fewer per group when the
     // automata of 16 clauses do not fit in LDS and the chip has room for more groups.
     const int waves = FITP_BLOCK / 64;
     auto lds_bytes = [&](int per_group) {
         return (2 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group +
-                2 * (size_t)d.K + 5 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K) * 4;
+                2 * (size_t)d.K + 5 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K + 2 * (size_t)p.x_words +
+                (size_t)cfg->literals) * 4;
     };
     const size_t lds_limit = 150 * 1024;
     int per_group = (d.C + cus - 1) / cus;

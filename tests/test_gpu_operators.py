@@ -385,12 +385,16 @@ def test_fused_fit_on_every_tile_geometry(shape, boost, max_included, state_bits
     (38, dict(n_graphs=6, hv_size=2200, n_symbols=30, sizes=[3, 70, 0, 1, 33, 64]), dict(classes=2, clauses=30, depth=1)),
 ], ids=lambda v: str(v) if isinstance(v, int) else "")
 @pytest.mark.parametrize("density", [0.3, 0.9])
-def test_fused_fit_with_many_literals(seed, g, m, density, monkeypatch):
-    """Clauses with many included literals (the training kernel ANDs a few of their rows and
-    tests the surviving nodes against the whole include mask) == the oracle."""
+@pytest.mark.parametrize("persistent", [True, False], ids=["one-launch", "per-example"])
+def test_fused_fit_with_many_literals(seed, g, m, density, persistent, monkeypatch):
+    """Clauses with many included literals (the training kernels AND a few of their rows and
+    test the surviving nodes against the whole include mask) == the oracle."""
     from tests.gpu_harness import Device
 
-    monkeypatch.setenv("GTM_NO_PERSISTENT_FIT", "1")
+    if not persistent:
+        monkeypatch.setenv("GTM_NO_PERSISTENT_FIT", "1")
+    elif m["depth"] > 1:
+        pytest.skip("models with message layers have one training path")
     graphs = helpers.random_graphs(seed, **g)
     m = dict(m)
     depth = m.pop("depth")
