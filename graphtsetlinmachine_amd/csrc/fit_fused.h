@@ -304,8 +304,16 @@ __device__ __forceinline__ uint32_t feedback_word(uint32_t *ta_global, int B, in
                                                   uint32_t k1, uint32_t c, uint32_t w, uint32_t step, uint32_t bank_id,
                                                   uint32_t thr16, const uint32_t *fb_of = nullptr) {
     uint32_t ta[MAXB];
+    // 8 planes (the default): the word's planes are 32 contiguous, 32-byte aligned bytes
+    const bool vector8 = MAXB == 8 && B == 8 && (reinterpret_cast<uintptr_t>(ta_global) & 31u) == 0;
+    if (vector8) {
+        const uint4 lo = reinterpret_cast<const uint4 *>(ta_global)[0], hi = reinterpret_cast<const uint4 *>(ta_global)[1];
+        ta[0] = lo.x, ta[1] = lo.y, ta[2] = lo.z, ta[3] = lo.w;
+        if (MAXB >= 8) ta[4 % MAXB] = hi.x, ta[5 % MAXB] = hi.y, ta[6 % MAXB] = hi.z, ta[7 % MAXB] = hi.w;
+    } else {
 #pragma unroll
-    for (int b = 0; b < MAXB; ++b) ta[b] = b < B ? ta_global[b] : 0u;
+        for (int b = 0; b < MAXB; ++b) ta[b] = b < B ? ta_global[b] : 0u;
+    }
     for (int k = 0; k < K; ++k) {
         const int u = u_of[(int64_t)k * u_stride];
         if (u > 0) {
@@ -325,6 +333,11 @@ __device__ __forceinline__ uint32_t feedback_word(uint32_t *ta_global, int B, in
         }
     }
     uint32_t top = 0;
+    if (vector8) {
+        reinterpret_cast<uint4 *>(ta_global)[0] = make_uint4(ta[0], ta[1], ta[2], ta[3]);
+        reinterpret_cast<uint4 *>(ta_global)[1] = make_uint4(ta[4 % MAXB], ta[5 % MAXB], ta[6 % MAXB], ta[7 % MAXB]);
+        return ta[7 % MAXB];
+    }
 #pragma unroll
     for (int b = 0; b < MAXB; ++b)
         if (b < B) {

@@ -1450,8 +1450,9 @@ int fit_deep_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g,
     const int cpb = per_clause >= TPB ? 1 : TPB / per_clause;
     const uint64_t q_thr = q_threshold(cfg->q, cfg->classes);
     const int waves_per_block = FIT_EVAL_BLOCK / 64;
-    int eval_blocks = (d.C + 2 * waves_per_block - 1) / (2 * waves_per_block);
-    if (eval_blocks > 1024) eval_blocks = 1024;
+    // one clause per wave while the chip has room (the evaluation is a chain of memory round trips)
+    int eval_blocks = (d.C + waves_per_block - 1) / waves_per_block;
+    if (eval_blocks > 2048) eval_blocks = 2048;
     static thread_local size_t lds_set = 0;
     // Messages by per-node bit vectors (fit_deep.h) when MESSAGE_SIZE is a multiple of 32 and the
     // graph is big enough for the saved atomics to pay for the extra pass.
