@@ -112,6 +112,10 @@ def _load():
             "`python -c 'import __graft_entry__ as g; g.build()'` at the repository root "
             "(or graphtsetlinmachine_amd/build.py)." % LIBRARY_PATH
         )
+    # torch brings its own HIP runtime; loading it first makes this library bind to the same
+    # one (two runtimes in a process do not see each other's device state)
+    import torch  # noqa: F401
+
     lib = C.CDLL(LIBRARY_PATH)
     for name, (restype, argtypes) in PROTOTYPES.items():
         fn = getattr(lib, name)

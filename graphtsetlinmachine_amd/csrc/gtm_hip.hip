@@ -385,6 +385,7 @@ __global__ void k_select_clause_updates(int32_t *weights, const int32_t *__restr
 
 #include "fit_fused.h"
 #include "fit_deep.h"
+#include "fit_small.h"
 #include "fit_persistent.h"
 
 // K9 / K10: one thread per (clause, automaton word); the classes are applied
@@ -681,7 +682,7 @@ TileGeom geometry_for(const gtm_config *cfg, const gtm_graphs *g, int classes) {
 template <int NW, int LW, int SRC, bool LAST>
 int launch_tile_layer_as(const TileLayerArgs &a, int n_tiles, const char *profile_name, hipStream_t st) {
     size_t lds = tile_layer_lds_bytes(a.tg, a.K, SRC, a.M);
-    static thread_local size_t lds_set = 0;
+    static thread_local size_t lds_set = 48 * 1024;
     if (lds > lds_set) {
         hipError_t e = hipFuncSetAttribute((const void *)k_tile_layer<NW, LW, SRC, LAST>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -720,7 +721,7 @@ int launch_tile_layer(const TileLayerArgs &a, int n_tiles, int src, bool last, h
 template <int NW, int LW, int LA4, bool LAST, bool FULL>
 int launch_two_phase_as(const TileLayerArgs &a, int n_tiles, hipStream_t st) {
     size_t lds = tile_layer_lds_bytes(a.tg, a.K, ROWS_STAGED, a.M);
-    static thread_local size_t lds_set = 0;
+    static thread_local size_t lds_set = 48 * 1024;
     if (lds > lds_set) {
         hipError_t e = hipFuncSetAttribute((const void *)k_tile_two_phase<NW, LW, LA4, LAST, FULL>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -767,7 +768,7 @@ template <int NW, int LW, int SRC, bool LAST>
 int launch_two_phase_wide_as(const TileLayerArgs &a, int n_tiles, int LA, hipStream_t st) {
     // rows (if staged), padding, class sums, and the first node and node count of the tile's graphs
     size_t lds = tile_layer_lds_bytes(a.tg, a.K, SRC, a.M) + (size_t)a.tg.gpt * 8;
-    static thread_local size_t lds_set = 0;
+    static thread_local size_t lds_set = 48 * 1024;
     if (lds > lds_set) {
         hipError_t e = hipFuncSetAttribute((const void *)k_tile_two_phase_wide<NW, LW, SRC, LAST>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1304,7 +1305,7 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     const int groups = (d.C + per_group - 1) / per_group;
     p.clauses_per_group = per_group;
     const size_t lds = lds_bytes(per_group);
-    static thread_local size_t lds_set = 0;
+    static thread_local size_t lds_set = 48 * 1024;
     if (lds > lds_set) {
         if (hipFuncSetAttribute((const void *)k_fit_persistent, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
             hipSuccess) {
@@ -1429,6 +1430,77 @@ int fit_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, cons
                            cfg->max_included_literals, q_thr, key.k0, key.k1, step, w.clause_node, w.n_incl, cpb);
         if (int rc = check_launch("fit_feedback")) return rc;
     }
+    return GTM_OK;
+}
+
+// A small model with message layers on tiny graphs trains inside one workgroup (fit_small.h).
+// Sets *done = false when the shape does not qualify.
+int fit_small(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const int32_t *encoded_Y,
+              int first_example, int n_examples, uint64_t first_step, hipStream_t st, bool *done) {
+    *done = false;
+    if (getenv("GTM_NO_SMALL_FIT")) return GTM_OK;
+    if (cfg->depth < 2 || d.M % 32 != 0 || g->max_number_of_graph_nodes > FITS_MAX_NODES ||
+        g->number_of_node_types < 1)
+        return GTM_OK;
+    const int MW = d.M / 32;
+    const size_t lds = fit_small_lds_words(cfg->depth, d.C, d.LA, d.MC, MW, d.B, d.K) * 4;
+    if (lds > FITS_MAX_LDS_BYTES) return GTM_OK;
+    if (g->total_edges > 0 && (!g->number_of_graph_node_edges || !g->edge || !g->edge_index))
+        return fail(GTM_ERR_INVALID, "graphs with edges need number_of_graph_node_edges, edge and edge_index");
+    Key key = key_of(cfg);
+    FitSmallParams p{};
+    p.X = g->X;
+    p.node_type = g->node_type;
+    p.node_index = g->node_index;
+    p.n_nodes = g->number_of_graph_nodes;
+    p.n_edges = g->number_of_graph_node_edges;
+    p.edge_index = g->edge_index;
+    p.edge = g->edge;
+    p.encoded_Y = encoded_Y;
+    p.first_example = first_example;
+    p.n_examples = n_examples;
+    p.first_step = (uint32_t)first_step;
+    p.n_types = g->number_of_node_types;
+    p.has_edges = g->total_edges > 0;
+    p.bank[0] = s->ta_state;
+    p.filter[0] = d.filter;
+    p.thr16[0] = feedback_threshold(cfg->s[0]);
+    for (int l = 1; l < cfg->depth; ++l) {
+        p.bank[l] = s->message_ta_state[l - 1];
+        p.filter[l] = d.mfilter;
+        p.thr16[l] = feedback_threshold(cfg->s[l]);
+    }
+    p.weights = s->clause_weights;
+    p.hv = s->hypervectors;
+    p.depth = cfg->depth;
+    p.C = d.C;
+    p.LA = d.LA;
+    p.MC = d.MC;
+    p.MW = MW;
+    p.MB = d.MB;
+    p.B = d.B;
+    p.K = d.K;
+    p.T = cfg->threshold;
+    p.negative = cfg->negative_clauses;
+    p.boost = cfg->boost_true_positive_feedback;
+    p.max_included = cfg->max_included_literals;
+    p.k0 = key.k0;
+    p.k1 = key.k1;
+    p.q_thr = q_threshold(cfg->q, cfg->classes);
+    static thread_local size_t lds_set = 48 * 1024;
+    if (lds > lds_set) {
+        if (hipFuncSetAttribute((const void *)k_fit_small, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+            hipSuccess) {
+            (void)hipGetLastError();
+            return GTM_OK;
+        }
+        lds_set = lds;
+    }
+    profile_start("k_fit_small", st);
+    hipLaunchKernelGGL(k_fit_small, dim3(1), dim3(FITS_BLOCK), lds, st, p);
+    profile_stop(st);
+    if (int rc = check_launch("fit_small")) return rc;
+    *done = true;
     return GTM_OK;
 }
 
@@ -1610,6 +1682,11 @@ int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *st
             return fit_on_tiles(d, cfg, graphs, state, tg, w, encoded_Y, first_example, n_examples, first_step, h_n,
                                 h_base, st);
         }
+    }
+    if (cfg->depth > 1) {
+        bool done = false;
+        if (int rc = fit_small(d, cfg, graphs, state, encoded_Y, first_example, n_examples, first_step, st, &done)) return rc;
+        if (done) return GTM_OK;
     }
     if (cfg->depth > 1 && graphs->tiles && graphs->number_of_node_types >= 1 && !getenv("GTM_NO_DEEP_FIT")) {
         TileGeom tg = geometry_for(cfg, graphs, d.K);

@@ -3,10 +3,12 @@
 Bar: bit-exact (everything here is integer / bitwise work)."""
 
 import copy
+import ctypes
 
 import numpy as np
 import pytest
 
+from graphtsetlinmachine_amd import _abi
 from oracle import gtm_oracle as o
 from tests import helpers
 
@@ -318,6 +320,7 @@ def test_fused_fit_with_message_layers(shape, boost, max_included, state_bits, m
     from tests.gpu_harness import Device
 
     monkeypatch.setenv("GTM_FIT_FACTOR_MIN", "0" if messages == "by-node-vectors" else str(1 << 60))
+    monkeypatch.setenv("GTM_NO_SMALL_FIT", "1")  # the one-workgroup kernel has its own test
 
     g = dict(shape["g"])
     if "sizes" not in g:
@@ -337,6 +340,62 @@ def test_fused_fit_with_message_layers(shape, boost, max_included, state_bits, m
     for epoch in range(2):
         o.fit(model, graphs, Y)
         dev.fit(Y, 0, G, epoch * G)
+        ta, banks, w = dev.download()
+        assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
+        assert np.array_equal(ta, model.ta_state), "layer-0 automata after epoch %d" % epoch
+        for layer in range(depth - 1):
+            assert np.array_equal(banks[layer], model.message_ta_state[layer]), "bank %d epoch %d" % (layer, epoch)
+    assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
+
+
+SMALL_DEEP_SHAPES = [
+    # two-node graphs with two edge types; 9..16 nodes, three layers; exactly 64 nodes (two truth
+    # words) and four edge types; graphs without nodes among small ones; single nodes with self-loops;
+    # several classes on graphs without edges
+    dict(seed=41, g=dict(n_graphs=40, max_nodes=2, min_nodes=2, hv_size=8, edge_types=("x", "y")),
+         m=dict(classes=2, clauses=10, depth=2, message_size=256, message_bits=2)),
+    dict(seed=42, g=dict(n_graphs=24, max_nodes=16, min_nodes=9, hv_size=20),
+         m=dict(classes=4, clauses=100, depth=3, message_size=64, message_bits=3)),
+    dict(seed=43, g=dict(n_graphs=10, max_nodes=64, min_nodes=64, hv_size=40, edge_types=("l", "r", "u", "d"),
+                         node_types=("a", "b")),
+         m=dict(classes=3, clauses=70, depth=2, message_size=96)),
+    dict(seed=44, g=dict(n_graphs=7, hv_size=16, sizes=[5, 0, 33, 1, 0, 40, 64]),
+         m=dict(classes=3, clauses=20, depth=4, message_size=32, message_bits=1)),
+    dict(seed=45, g=dict(n_graphs=30, max_nodes=1, hv_size=40), m=dict(classes=3, clauses=50, depth=2, message_size=32)),
+    dict(seed=46, g=dict(n_graphs=12, max_nodes=40, min_nodes=20, hv_size=100, max_degree=0),
+         m=dict(classes=5, clauses=64, depth=2, message_size=128)),
+]
+
+
+@pytest.mark.parametrize("shape", SMALL_DEEP_SHAPES, ids=lambda s: "small%d" % s["seed"])
+@pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 9, 5), (1, None, 12)])
+def test_one_workgroup_fit_with_message_layers(shape, boost, max_included, state_bits):
+    """Small models with message layers on graphs of at most 64 nodes train inside one workgroup
+    (k_fit_small): automata of every bank and the weights after each of two epochs == the oracle,
+    and the run is split into two calls so the state's round trip through memory is covered."""
+    from tests.gpu_harness import Device
+
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    m = dict(shape["m"])
+    depth = m.pop("depth")
+    cfg = helpers.oracle_config(graphs, **m, depth=depth, T=30, boost=boost, max_included=max_included,
+                                state_bits=state_bits)
+    model = helpers.random_model(shape["seed"], cfg, depth, s=(3.0, 2.0, 1.5, 1.2)[:depth],
+                                 include_density=shape.get("density", 0.02), message_density=0.02)
+    dev = Device(model, graphs)
+    dev.build_tiles()
+    rng = np.random.default_rng(shape["seed"])
+    G = graphs.number_of_graphs
+    Y = o.encode_labels(rng.integers(0, cfg.classes, size=G), cfg.classes, cfg.threshold)
+    name, launches, total = ctypes.c_char_p(), ctypes.c_int32(), ctypes.c_double()
+    for epoch in range(2):
+        o.fit(model, graphs, Y)
+        _abi.call("gtm_profile_enable", 1)
+        dev.fit(Y, 0, G // 2, epoch * G)
+        dev.fit(Y, G // 2, G - G // 2, epoch * G + G // 2)
+        _abi.call("gtm_profile_read", ctypes.byref(name), ctypes.byref(launches), ctypes.byref(total))
+        _abi.call("gtm_profile_enable", 0)
+        assert (name.value, launches.value) == (b"k_fit_small", 2), "the one-workgroup kernel should have run"
         ta, banks, w = dev.download()
         assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
         assert np.array_equal(ta, model.ta_state), "layer-0 automata after epoch %d" % epoch
