@@ -1443,7 +1443,7 @@ int fit_small(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const g
         g->number_of_node_types < 1)
         return GTM_OK;
     const int MW = d.M / 32;
-    const size_t lds = fit_small_lds_words(cfg->depth, d.C, d.LA, d.MC, MW, d.B, d.K) * 4;
+    const size_t lds = fit_small_lds_words(cfg->depth, d.C, d.LA, d.MC, MW, d.MB, d.B, d.K) * 4;
     if (lds > FITS_MAX_LDS_BYTES) return GTM_OK;
     if (g->total_edges > 0 && (!g->number_of_graph_node_edges || !g->edge || !g->edge_index))
         return fail(GTM_ERR_INVALID, "graphs with edges need number_of_graph_node_edges, edge and edge_index");
