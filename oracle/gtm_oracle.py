@@ -526,7 +526,7 @@ def evaluate_graph(model, graphs, e):
     layers = []
     if model.depth > 1:
         n_edges = graphs.number_of_graph_node_edges[base : base + n]
-        e0 = int(graphs.edge_index[base])
+        e0 = int(graphs.edge_index[base]) if n > 0 else 0  # a trailing graph without nodes has no entry
         edge = graphs.edge[e0 : e0 + int(n_edges.astype(np.int64).sum())]
     for d in range(model.depth - 1):
         clause_X = build_messages(cfg, n, model.hypervectors, bitmap, n_edges, edge)

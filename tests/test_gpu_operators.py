@@ -276,7 +276,7 @@ DEEP_TILE_SHAPES = [
          m=dict(classes=10, clauses=80, depth=2, message_size=256)),
     dict(seed=35, g=dict(n_graphs=5, sizes=[3, 520, 40, 1, 200], hv_size=1500, n_symbols=30),
          m=dict(classes=2, clauses=60, depth=2, message_size=32), density=0.0007),
-    dict(seed=36, g=dict(n_graphs=6, hv_size=16, sizes=[5, 0, 33, 1, 0, 40]),
+    dict(seed=36, g=dict(n_graphs=7, hv_size=16, sizes=[5, 0, 33, 1, 0, 40, 0]),
          m=dict(classes=3, clauses=20, depth=3, message_size=16, message_bits=1)),
     dict(seed=37, g=dict(n_graphs=200, max_nodes=1, hv_size=40), m=dict(classes=3, clauses=50, depth=2, message_size=8)),
 ]
@@ -350,7 +350,7 @@ def test_fused_fit_with_message_layers(shape, boost, max_included, state_bits, m
 
 SMALL_DEEP_SHAPES = [
     # two-node graphs with two edge types; 9..16 nodes, three layers; exactly 64 nodes (two truth
-    # words) and four edge types; graphs without nodes among small ones; single nodes with self-loops;
+    # words) and four edge types; graphs without nodes among small ones and at the end; single nodes with self-loops;
     # several classes on graphs without edges
     dict(seed=41, g=dict(n_graphs=40, max_nodes=2, min_nodes=2, hv_size=8, edge_types=("x", "y")),
          m=dict(classes=2, clauses=10, depth=2, message_size=256, message_bits=2)),
@@ -359,7 +359,7 @@ SMALL_DEEP_SHAPES = [
     dict(seed=43, g=dict(n_graphs=10, max_nodes=64, min_nodes=64, hv_size=40, edge_types=("l", "r", "u", "d"),
                          node_types=("a", "b")),
          m=dict(classes=3, clauses=70, depth=2, message_size=96)),
-    dict(seed=44, g=dict(n_graphs=7, hv_size=16, sizes=[5, 0, 33, 1, 0, 40, 64]),
+    dict(seed=44, g=dict(n_graphs=8, hv_size=16, sizes=[5, 0, 33, 1, 0, 40, 64, 0]),
          m=dict(classes=3, clauses=20, depth=4, message_size=32, message_bits=1)),
     dict(seed=45, g=dict(n_graphs=30, max_nodes=1, hv_size=40), m=dict(classes=3, clauses=50, depth=2, message_size=32)),
     dict(seed=46, g=dict(n_graphs=12, max_nodes=40, min_nodes=20, hv_size=100, max_degree=0),
