@@ -47,10 +47,10 @@ def parse():
 # (train graphs, test graphs) for the short runs of the configurations that are not the main one
 OTHER_WORKLOADS = {
     "noisy_xor": (10000, 10000),
-    "single_node_images": (20000, 10000),
+    "single_node_images": (60000, 10000),
     "convolutional_images": (5000, 2000),
-    "sequence_chains": (1000, 500),
-    "colour_convolution": (48, 256),
+    "sequence_chains": (5000, 2000),
+    "colour_convolution": (256, 256),
 }
 
 

@@ -1,4 +1,4 @@
-"""Seeded synthetic workloads: the five benchmark configurations.
+"""Seeded synthetic workloads: the five benchmark configurations and the README's sequence task.
 
 Each builder returns a ``Workload`` with encoded train/test ``Graphs``, labels
 and the constructor arguments of ``MultiClassGraphTsetlinMachine`` for that
@@ -288,10 +288,58 @@ def colour_convolution(n_train=50000, n_test=10000, seed=1239, patch=4, levels=8
     return Workload("colour_convolution", gtr, ytr, gte, yte, params, 10)
 
 
+# ----------------------------------------------- the README's sequence task
+
+
+def runs_of_a(n_train=40000, n_test=40000, seed=1240, classes=3, max_length=10, noise=0.01):
+    """The task of the reference's sequence demo (README.md:194-208,
+    examples/SequenceClassificationDemo.py:48-84): chains of 3..max_length nodes
+    with 'Left'/'Right' edges, one run of y + 1 consecutive 'A's somewhere, the
+    class is y.  A node sees only its own symbol, so the classes can only be told
+    apart through the messages: learning it needs every part of a model with
+    message layers to work."""
+    rng = np.random.default_rng(seed)
+
+    def build(n, parent, flip):
+        if parent is None:
+            g = _seeded_graphs(seed, n, symbols=["A"], hypervector_size=256, hypervector_bits=2)
+        else:
+            g = Graphs(n, init_with=parent)
+        lengths = rng.integers(classes, max_length + 1, size=n)
+        g.number_of_graph_nodes[:] = lengths
+        g.prepare_node_configuration()
+        local = np.concatenate([np.arange(m) for m in lengths])
+        gid = np.repeat(np.arange(n), lengths)
+        last = np.repeat(lengths, lengths) - 1
+        degree = np.where((local > 0) & (local < last), 2, 1).astype(np.uint32)
+        g.add_graph_nodes(degree)
+        g.prepare_edge_configuration()
+        # per node the reference adds 'Left' before 'Right' (examples/SequenceClassificationDemo.py:64-72)
+        has_left, has_right = local > 0, local < last
+        g.add_graph_node_edges(gid[has_left], local[has_left], local[has_left] - 1, "Left")
+        g.add_graph_node_edges(gid[has_right], local[has_right], local[has_right] + 1, "Right")
+        y = rng.integers(0, classes, size=n).astype(np.uint32)
+        end = rng.integers(y, lengths)  # the run ends at node `end`, inclusive
+        rows = np.concatenate([g.node_index[i] + np.arange(end[i] - y[i], end[i] + 1) for i in range(n)])
+        g.add_graph_node_properties(rows, np.zeros(rows.size, dtype=np.int64))
+        if flip:
+            wrong = rng.random(n) <= noise
+            y = np.where(wrong, (y + rng.integers(1, classes, size=n)) % classes, y).astype(np.uint32)
+        g.encode()
+        return g, y
+
+    gtr, ytr = build(n_train, None, True)
+    gte, yte = build(n_test, gtr, False)
+    params = dict(number_of_clauses=60, T=600, s=1.0, depth=3, message_size=256, message_bits=2,
+                  max_included_literals=4)
+    return Workload("runs_of_a", gtr, ytr, gte, yte, params, classes)
+
+
 BUILDERS = {
     "noisy_xor": noisy_xor,
     "single_node_images": single_node_images,
     "convolutional_images": convolutional_images,
     "sequence_chains": sequence_chains,
     "colour_convolution": colour_convolution,
+    "runs_of_a": runs_of_a,
 }
