@@ -11,14 +11,21 @@
 //   2. meets the other workgroups at a device-wide barrier (the class sums are
 //      the only thing that crosses clause boundaries, kernels.py:310-315);
 //   3. decides the feedback and updates its automata and weights in LDS.
-// Class sums and barrier are one thing: the sum of class k is a 64-bit word whose
-// low 48 bits hold the (biased) sum and whose high 16 bits count the workgroups
-// that have added their share.  A workgroup adds (1 << 48) + share with one
-// device-scope atomic per class and then polls the words until the count equals
-// the number of workgroups: when it does, the low bits are the final sum.  One
-// atomic per class carries both, so nothing has to be ordered against a separate
-// barrier word and no cache is flushed or invalidated.  The words live in a ring
-// of three slots so that no slot is reset while someone may still read it.
+// Class sums and barrier are one thing: class k has a 64-bit word to which every
+// workgroup adds (1 << 48) + its share with one device-scope atomic, and which it
+// then polls.  Nothing else is ever done to the word - no reset, no store - so
+// per-location coherence is all the protocol needs: nothing has to be ordered
+// against a separate barrier word and no cache is flushed or invalidated.  What an
+// example contributed is the word now minus the word as it stood when its last use
+// was complete (each polling thread remembers that value): modulo 2^64 that
+// difference is arrivals * 2^48 + sum, whatever borrows negative shares caused, so
+// with |sum| < 2^47 the arrivals are (difference + 2^47) >> 48 and, once they equal
+// the number of workgroups, the sum is the rest.  The words live in a ring of three
+// slots, each in a cache line of its own (the adds and polls of different classes
+// go to different memory channels): a workgroup can be one example ahead of the
+// slowest one, never three.  While waiting, all of a workgroup's polling threads
+// watch the word of class 0 (one request per poll) and look at their own only when
+// that one is complete.
 //
 // The wait is bounded: after `spin_limit` polls a workgroup raises the abort
 // flag and every workgroup leaves the loop at its next check, so the grid always
@@ -44,7 +51,7 @@ struct FitPersistParams {
     uint32_t filter, thr16, k0, k1;
     uint64_t q_thr;
     // coordination
-    unsigned long long *class_sum;  // [3][K], every word FITP_BIAS on entry
+    unsigned long long *class_sum;  // [3][K] words FITP_SUM_STRIDE apart, zero on entry (K <= FITP_BLOCK)
     uint32_t *abort_flag;           // [1], zero on entry
     uint32_t spin_limit;
     int clauses_per_group;
@@ -79,8 +86,9 @@ __device__ __forceinline__ void fitp_stage_rows(const FitPersistParams &p, const
     }
 }
 
-constexpr unsigned long long FITP_BIAS = 1ull << 47;      // a class sum s is stored as s + FITP_BIAS in bits 0..47
+constexpr unsigned long long FITP_HALF = 1ull << 47;      // class sums are smaller than this in magnitude
 constexpr unsigned long long FITP_ARRIVED = 1ull << 48;   // one arrival in bits 48..63
+constexpr int FITP_SUM_STRIDE = 16;                      // 64-bit words between two class-sum words (one per 128-byte line)
 constexpr int FITP_PREFETCH = 8;  // words of the next graph's rows a thread holds in registers while evaluating
 constexpr int FITP_PREFETCH_X = 4;  // the same for the next graph's node-major literal words
 constexpr int FITP_WALK_ALL = 24;   // clauses with at most this many literals AND all their rows
@@ -145,12 +153,15 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
 
     const int ones_row = p.literals + p.n_types;
     int div_words = 0, div_dr = 0, div_r0 = 0;
+    // thread k < K: its class-sum word and the word of class 0 as they stood when the slots of
+    // examples i, i + 1, i + 2 were last complete (all zero before their first use)
+    unsigned long long seen_own[3] = {0ull, 0ull, 0ull}, seen_first[3] = {0ull, 0ull, 0ull};
     for (int i = 0; i < p.n_examples; ++i) {
         const int ex = p.first_example + i;
         const uint32_t step = p.first_step + (uint32_t)i;
         const FitGraph fg = fit_graph_slot(p.tg, ex, n_now);
         const uint32_t *rows = rows_buf[i & 1];
-        unsigned long long *slot_now = p.class_sum + (size_t)(i % 3) * K;
+        unsigned long long *slot_now = p.class_sum + (size_t)(i % 3) * K * FITP_SUM_STRIDE;
 
         // ---- 0. requests that can be in flight while this example is evaluated: the next graph's
         // rows (into registers) and the sizes of the graph after it
@@ -318,7 +329,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         // ---- 2. class sums across the device (see the header comment)
         __syncthreads();  // the group's votes are complete
         for (int k = tid; k < K; k += FITP_BLOCK) {
-            __hip_atomic_fetch_add(&slot_now[k], FITP_ARRIVED + (unsigned long long)(long long)votes[k], __ATOMIC_RELAXED,
+            __hip_atomic_fetch_add(&slot_now[k * FITP_SUM_STRIDE], FITP_ARRIVED + (unsigned long long)(long long)votes[k], __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
             votes[k] = 0;
         }
@@ -351,12 +362,30 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         }
         if (tid == 0) go_on = 1;
         __syncthreads();
-        for (int k = tid; k < K; k += FITP_BLOCK) {
+        if (tid < K) {
+            const int k = tid;
+            const unsigned long long everyone = (unsigned long long)gridDim.x;
+            auto arrivals = [](unsigned long long now, unsigned long long before) {
+                return ((now - before + FITP_HALF) >> 48) & 0xFFFFull;
+            };
             uint32_t polls = 0;
-            unsigned long long word;
-            bool ok = true;
-            while (((word = __hip_atomic_load(&slot_now[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 48) <
-                   (unsigned long long)gridDim.x) {
+            unsigned long long word = 0ull, first = 0ull;
+            bool ok = true, mine = false;
+            for (;;) {
+                if (!mine) {
+                    first = __hip_atomic_load(&slot_now[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (arrivals(first, seen_first[0]) == everyone) {
+                        mine = true;
+                        if (k == 0) {
+                            word = first;
+                            break;
+                        }
+                        continue;
+                    }
+                } else {
+                    word = __hip_atomic_load(&slot_now[k * FITP_SUM_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (arrivals(word, seen_own[0]) == everyone) break;
+                }
                 if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
                     ++polls > p.spin_limit) {
                     __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -366,15 +395,13 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 __builtin_amdgcn_s_sleep(1);
             }
             if (!ok) go_on = 0;
-            sums[k] = (int32_t)(long long)((word & (FITP_ARRIVED - 1)) - FITP_BIAS);
+            sums[k] = (int32_t)(long long)(word - seen_own[0] - (everyone << 48));
+            // the slot's next use is three examples on
+            seen_own[0] = seen_own[1], seen_own[1] = seen_own[2], seen_own[2] = word;
+            seen_first[0] = seen_first[1], seen_first[1] = seen_first[2], seen_first[2] = first;
         }
         __syncthreads();
         if (!go_on) break;  // uniform over the group; every group leaves at its next check
-        // slot (i+2)%3 was last read for example i-1; everybody is past that: reset it for example i+2
-        if (blockIdx.x == 0)
-            for (int k = tid; k < K; k += FITP_BLOCK)
-                __hip_atomic_store(&p.class_sum[(size_t)((i + 2) % 3) * K + k], FITP_BIAS, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
 
         // ---- 3. feedback (K8) and automaton updates (K9) on the LDS copies
         const int32_t *y = p.encoded_Y + (int64_t)ex * K;
