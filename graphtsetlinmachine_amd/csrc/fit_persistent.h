@@ -127,6 +127,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                           (uint32_t *)(pair_list + (size_t)own_max * K) + p.x_words};  // [nodes][LA] of the graph
     uint32_t *order_lds = x_buf[1] + p.x_words;                 // [literals]
     __shared__ int go_on, n_pairs;
+    __shared__ uint32_t after_lds[2];
 
     // own state -> LDS
     for (int k = tid; k < K; k += FITP_BLOCK) votes[k] = 0;
@@ -199,9 +200,12 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 pre_x[u] = tid + u * FITP_BLOCK < next_x_total ? src[tid + u * FITP_BLOCK] : 0u;
         }
         const uint32_t *x_now = x_buf[i & 1];
+        // node count and first node of the graph after the next, fetched by two threads with vector
+        // loads (scalar loads share their counter with LDS: the evaluation's first LDS read would wait
+        // for them) and handed over through LDS at the end of the step
         const int e2 = min(ex + 2, last);
-        const int n_after = (int)p.n_nodes[e2];
-        const uint32_t base_after = p.node_index[e2];
+        uint32_t after = 0u;
+        if (tid < 2) after = (tid == 0 ? p.n_nodes : p.node_index)[e2];
 
         // ---- 1. evaluate own clauses (K1 + K7), votes (K6)
         const bool active = lane < fg.words;
@@ -465,11 +469,12 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             feedback_word_any(ta + (size_t)j * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1,
                               (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, p.thr16, fbits + (size_t)j * K);
         }
+        if (tid < 2) after_lds[tid] = after;
         __syncthreads();
         n_now = n_next;
         base_now = base_next;
-        n_next = n_after;
-        base_next = base_after;
+        n_next = (int)after_lds[0];
+        base_next = after_lds[1];
     }
     // own state -> global memory (also after an abort: every clause is left as of some whole step)
     for (int i = tid; i < n_own * LA * B; i += FITP_BLOCK) p.bank[(int64_t)c0 * LA * B + i] = ta[i];
