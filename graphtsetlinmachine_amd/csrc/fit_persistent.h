@@ -89,10 +89,11 @@ __device__ __forceinline__ void fitp_stage_rows(const FitPersistParams &p, const
 constexpr unsigned long long FITP_HALF = 1ull << 47;      // class sums are smaller than this in magnitude
 constexpr unsigned long long FITP_ARRIVED = 1ull << 48;   // one arrival in bits 48..63
 constexpr int FITP_SUM_STRIDE = 16;                      // 64-bit words between two class-sum words (one per 128-byte line)
-constexpr int FITP_PREFETCH = 8;  // words of the next graph's rows a thread holds in registers while evaluating
-constexpr int FITP_PREFETCH_X = 4;  // the same for the next graph's node-major literal words
+constexpr int FITP_PREFETCH = 5;  // words of the next graph's rows a thread holds in registers while evaluating
+constexpr int FITP_PREFETCH_X = 3;  // the same for the next graph's node-major literal words
 constexpr int FITP_WALK_ALL = 24;   // clauses with at most this many literals AND all their rows
 constexpr int FITP_FILTER_ROWS = 16;  // rows the others AND before testing the surviving nodes
+constexpr int FITP_FEW_NODES = 2;     // up to this many surviving nodes are tested one by one, more are filtered further
 
 // Address of element `i` of the staged rows (i = row * words + w) inside the graph's tile.
 __device__ __forceinline__ const uint32_t *fitp_row_word(const FitPersistParams &p, const FitGraph &fg, int i) {
@@ -100,6 +101,8 @@ __device__ __forceinline__ const uint32_t *fitp_row_word(const FitPersistParams 
     return p.tiles + ((int64_t)fg.tile * p.tg.rows + r) * p.tg.tw + fg.word0 + w;
 }
 
+// MAXB: bit planes of an automaton the kernel keeps in registers while updating a word (>= B).
+template <int MAXB>
 __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams p) {
     extern __shared__ uint32_t lds[];
     const int tid = threadIdx.x;
@@ -126,6 +129,9 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
     uint32_t *x_buf[2] = {(uint32_t *)(pair_list + (size_t)own_max * K),
                           (uint32_t *)(pair_list + (size_t)own_max * K) + p.x_words};  // [nodes][LA] of the graph
     uint32_t *order_lds = x_buf[1] + p.x_words;                 // [literals]
+    // thread k < K: its class-sum word and the word of class 0 as they stood when each of the three
+    // slots was last complete (all zero before the first use): [slot][own, first][low, high][K]
+    uint32_t *seen = order_lds + p.literals;
     __shared__ int go_on, n_pairs;
     __shared__ uint32_t after_lds[2];
 
@@ -150,13 +156,11 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         for (int at = tid; at < n_now * LA; at += FITP_BLOCK) x_buf[0][at] = p.X[(int64_t)base_now * LA + at];
     }
     for (int l = tid; l < p.literals; l += FITP_BLOCK) order_lds[l] = p.order[l];
+    for (int j = tid; j < 12 * K; j += FITP_BLOCK) seen[j] = 0u;
     __syncthreads();
 
     const int ones_row = p.literals + p.n_types;
     int div_words = 0, div_dr = 0, div_r0 = 0;
-    // thread k < K: its class-sum word and the word of class 0 as they stood when the slots of
-    // examples i, i + 1, i + 2 were last complete (all zero before their first use)
-    unsigned long long seen_own[3] = {0ull, 0ull, 0ull}, seen_first[3] = {0ull, 0ull, 0ull};
     for (int i = 0; i < p.n_examples; ++i) {
         const int ex = p.first_example + i;
         const uint32_t step = p.first_step + (uint32_t)i;
@@ -227,28 +231,48 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             // A clause with many literals ANDs only the rows of its FITP_FILTER_ROWS rarest ones and then
             // tests the few nodes that are left against its whole include mask on the nodes' own words.
             const bool filter_only = included > FITP_WALK_ALL && n_now > 0;
+            bool all_rows = false;  // every included literal's row has been applied: acc is the clause's truth
             if (filter_only) {
                 int budget = FITP_FILTER_ROWS;
-                for (int r0 = 0; r0 < p.literals && budget > 0; r0 += 64) {
-                    const int r = r0 + lane;
-                    const uint32_t lit = r < p.literals ? order_lds[r] : 0u;
-                    uint32_t word = inc[(lit >> 5) * B];
-                    if ((int)(lit >> 5) == LA - 1) word &= p.filter;
-                    unsigned long long picked = __ballot(r < p.literals && ((word >> (lit & 31u)) & 1u));
-                    while (picked && budget > 0) {
-                        int row[8];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) {
-                            row[u] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
-                            picked &= picked - 1;
-                        }
-                        uint32_t r8[8];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) r8[u] = col[row[u] * stride];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) acc &= r8[u];
-                        budget -= 8;
+                int r0 = 0;
+                unsigned long long picked = 0ull;  // lanes whose literal (in rarest-first order) is included and not applied yet
+                uint32_t lit = 0u;
+                for (;;) {
+                    if (budget <= 0) {
+                        // a few surviving nodes are cheapest tested one by one; more than that, and 8 more
+                        // rows (one LDS round trip) remove most of them at the price of testing one
+                        // (counted as lanes with a survivor, twice those with several: an estimate is enough)
+                        if (n_now <= FITP_FEW_NODES) break;
+                        const int mine = active ? __popc((acc >> fg.shift) & fg.mask) : 0;
+                        const int left = __popcll(__ballot(mine > 0)) + __popcll(__ballot(mine > 1));
+                        if (left <= FITP_FEW_NODES) break;
+                        budget = 8;
                     }
+                    if (picked == 0ull) {
+                        if (r0 >= p.literals) {
+                            all_rows = true;
+                            break;
+                        }
+                        const int r = r0 + lane;
+                        lit = r < p.literals ? order_lds[r] : 0u;
+                        uint32_t word = inc[(lit >> 5) * B];
+                        if ((int)(lit >> 5) == LA - 1) word &= p.filter;
+                        picked = __ballot(r < p.literals && ((word >> (lit & 31u)) & 1u));
+                        r0 += 64;
+                        continue;
+                    }
+                    int row[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        row[u] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
+                        picked &= picked - 1;
+                    }
+                    uint32_t r8[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) r8[u] = col[row[u] * stride];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc &= r8[u];
+                    budget -= 8;
                 }
             } else {
                 for (int w0 = 0; w0 < LA; w0 += 64) {
@@ -277,7 +301,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 }
             }
             uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
-            if (filter_only) {
+            if (filter_only && !all_rows) {
                 // lane L holds nodes 32 L .. 32 L + 31: the surviving ones are walked on the scalar unit; lane w
                 // compares include word w with the node's literal word w (LDS copy of the graph's X rows)
                 unsigned long long live = __ballot(v != 0);
@@ -372,13 +396,16 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             auto arrivals = [](unsigned long long now, unsigned long long before) {
                 return ((now - before + FITP_HALF) >> 48) & 0xFFFFull;
             };
+            uint32_t *seen_slot = seen + (size_t)(i % 3) * 4 * K;
+            const unsigned long long seen_own = ((unsigned long long)seen_slot[K + k] << 32) | seen_slot[k];
+            const unsigned long long seen_first = ((unsigned long long)seen_slot[3 * K + k] << 32) | seen_slot[2 * K + k];
             uint32_t polls = 0;
             unsigned long long word = 0ull, first = 0ull;
             bool ok = true, mine = false;
             for (;;) {
                 if (!mine) {
                     first = __hip_atomic_load(&slot_now[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (arrivals(first, seen_first[0]) == everyone) {
+                    if (arrivals(first, seen_first) == everyone) {
                         mine = true;
                         if (k == 0) {
                             word = first;
@@ -388,7 +415,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                     }
                 } else {
                     word = __hip_atomic_load(&slot_now[k * FITP_SUM_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (arrivals(word, seen_own[0]) == everyone) break;
+                    if (arrivals(word, seen_own) == everyone) break;
                 }
                 if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
                     ++polls > p.spin_limit) {
@@ -399,10 +426,10 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 __builtin_amdgcn_s_sleep(1);
             }
             if (!ok) go_on = 0;
-            sums[k] = (int32_t)(long long)(word - seen_own[0] - (everyone << 48));
-            // the slot's next use is three examples on
-            seen_own[0] = seen_own[1], seen_own[1] = seen_own[2], seen_own[2] = word;
-            seen_first[0] = seen_first[1], seen_first[1] = seen_first[2], seen_first[2] = first;
+            sums[k] = (int32_t)(long long)(word - seen_own - (everyone << 48));
+            // for the slot's next use, three examples on
+            seen_slot[k] = (uint32_t)word, seen_slot[K + k] = (uint32_t)(word >> 32);
+            seen_slot[2 * K + k] = (uint32_t)first, seen_slot[3 * K + k] = (uint32_t)(first >> 32);
         }
         __syncthreads();
         if (!go_on) break;  // uniform over the group; every group leaves at its next check
@@ -466,7 +493,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             const bool fired = node != -1;
             const bool within = incl_of[cl] <= p.max_included;
             const uint32_t x = fired ? X_rows[node * LA + w] : 0u;
-            feedback_word_any(ta + (size_t)j * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1,
+            feedback_word<MAXB>(ta + (size_t)j * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1,
                               (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, p.thr16, fbits + (size_t)j * K);
         }
         if (tid < 2) after_lds[tid] = after;

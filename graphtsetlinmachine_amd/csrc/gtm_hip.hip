@@ -1296,7 +1296,7 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     auto lds_bytes = [&](int per_group) {
         return (2 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group +
                 2 * (size_t)d.K + 5 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K + 2 * (size_t)p.x_words +
-                (size_t)cfg->literals) * 4;
+                (size_t)cfg->literals + 12 * (size_t)d.K) * 4;
     };
     const size_t lds_limit = 150 * 1024;
     int per_group = (d.C + cus - 1) / cus;
@@ -1305,9 +1305,15 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     const int groups = (d.C + per_group - 1) / per_group;
     p.clauses_per_group = per_group;
     const size_t lds = lds_bytes(per_group);
-    static thread_local size_t lds_set = 48 * 1024;
+    // one instance per width of the automata in registers (the widest would cost the others registers)
+    const int variant = d.B <= 8 ? 0 : d.B <= 16 ? 1 : 2;
+    const void *kernel = variant == 0   ? (const void *)k_fit_persistent<8>
+                         : variant == 1 ? (const void *)k_fit_persistent<16>
+                                        : (const void *)k_fit_persistent<32>;
+    static thread_local size_t lds_set_of[3] = {48 * 1024, 48 * 1024, 48 * 1024};
+    size_t &lds_set = lds_set_of[variant];
     if (lds > lds_set) {
-        if (hipFuncSetAttribute((const void *)k_fit_persistent, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+        if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
             hipSuccess) {
             (void)hipGetLastError();
             return GTM_OK;
@@ -1315,7 +1321,7 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         lds_set = lds;
     }
     int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_fit_persistent, FITP_BLOCK, lds) != hipSuccess ||
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, FITP_BLOCK, lds) != hipSuccess ||
         per_cu < 1 || groups > per_cu * cus) {
         (void)hipGetLastError();
         return GTM_OK;
@@ -1358,7 +1364,7 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     if (int rc = check_launch("fill")) return rc;
     void *args[] = {&p};
     profile_start("k_fit_persistent", st);
-    hipError_t e = hipLaunchCooperativeKernel((const void *)k_fit_persistent, dim3(groups), dim3(FITP_BLOCK), args,
+    hipError_t e = hipLaunchCooperativeKernel(kernel, dim3(groups), dim3(FITP_BLOCK), args,
                                               (unsigned)lds, st);
     if (e != hipSuccess) return fail(GTM_ERR_HIP, "cooperative launch of the training kernel: %s", hipGetErrorString(e));
     profile_stop(st);
