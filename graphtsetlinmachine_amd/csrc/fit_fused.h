@@ -20,6 +20,7 @@ constexpr int FIT_EVAL_BLOCK = 256;
 constexpr int FIT_WALK_ALL = 40;      // clauses with at most this many literals AND all their rows (rows in global memory)
 constexpr int FIT_WALK_ALL_LDS = 512; // the same with the rows staged in LDS
 constexpr int FIT_FILTER_ROWS = 16;  // rows the others AND before testing nodes
+constexpr int FIT_FEW_NODES = 2;    // up to this many surviving nodes (estimate) are tested one by one, more are filtered further
 
 struct FitGraph {
     int tile;        // tile holding the graph
@@ -169,29 +170,47 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
         // few nodes that are left against its whole include mask on the nodes' own literal words.
         const bool filter_only = included > (STAGE ? FIT_WALK_ALL_LDS : FIT_WALK_ALL) && n_nodes > 0;
         uint32_t acc = active ? col[(int64_t)(literals + c % n_types) * stride] : 0u;
+        bool all_rows = false;  // every included literal's row has been applied: acc is the clause's truth
         if (filter_only && order) {
-            // the first FIT_FILTER_ROWS included literals in `order` (the ones that hold least often in the data set)
+            // the first FIT_FILTER_ROWS included literals in `order` (the ones that hold least often in the
+            // data set); while more than a few nodes survive, 8 more at a time: one round trip of row
+            // reads removes most of them, testing them costs a round trip per word of nodes
             int budget = FIT_FILTER_ROWS;
-            for (int r0 = 0; r0 < literals && budget > 0; r0 += 64) {
-                const int r = r0 + lane;
-                const uint32_t lit = r < literals ? order[r] : 0u;
-                uint32_t word = inc[(int64_t)(lit >> 5) * B];
-                if ((int)(lit >> 5) == LA - 1) word &= filter;
-                unsigned long long picked = __ballot(r < literals && ((word >> (lit & 31u)) & 1u));
-                while (picked && budget > 0) {
-                    int row[8];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) {
-                        row[u] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
-                        picked &= picked - 1;
-                    }
-                    uint32_t r8[8];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) r8[u] = col[(int64_t)row[u] * stride];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) acc &= r8[u];
-                    budget -= 8;
+            int r0 = 0;
+            unsigned long long picked = 0ull;  // lanes whose literal (in `order`) is included and not applied yet
+            uint32_t lit = 0u;
+            for (;;) {
+                if (budget <= 0) {
+                    const int mine = active ? __popc((acc >> fg.shift) & fg.mask) : 0;
+                    const int left = __popcll(__ballot(mine > 0)) + __popcll(__ballot(mine > 1));
+                    if (left <= FIT_FEW_NODES) break;
+                    budget = 8;
                 }
+                if (picked == 0ull) {
+                    if (r0 >= literals) {
+                        all_rows = true;
+                        break;
+                    }
+                    const int r = r0 + lane;
+                    lit = r < literals ? order[r] : 0u;
+                    uint32_t word = inc[(int64_t)(lit >> 5) * B];
+                    if ((int)(lit >> 5) == LA - 1) word &= filter;
+                    picked = __ballot(r < literals && ((word >> (lit & 31u)) & 1u));
+                    r0 += 64;
+                    continue;
+                }
+                int row[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    row[u] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
+                    picked &= picked - 1;
+                }
+                uint32_t r8[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) r8[u] = col[(int64_t)row[u] * stride];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) acc &= r8[u];
+                budget -= 8;
             }
         } else {
             int budget = filter_only ? FIT_FILTER_ROWS : 0x7FFFFFFF;
@@ -221,7 +240,7 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
             }
         }
         uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
-        if (filter_only) {
+        if (filter_only && !all_rows) {
             // Lane L holds nodes 32 L .. 32 L + 31.  The surviving nodes are walked on the scalar unit, 8 at
             // a time; for each, lane w compares include word w with the node's literal word w (one
             // coalesced load per node and 64 words), and a node with any violated word is cleared.
