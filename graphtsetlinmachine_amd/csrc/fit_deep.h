@@ -167,7 +167,9 @@ __global__ __launch_bounds__(64) void k_fit_pack_messages(uint32_t *sent, uint32
 //   by node     64 nodes at a time, lane = node: the node's packed message words
 //               against the clause's include words, (include & ~words) == 0, for
 //               the blocks of nodes where the clause is still true.
-__global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
+constexpr int FIT_MESSAGE_EVAL_BLOCK = 1024;  // at most 16 waves: a graph of up to 1,024 nodes has a wave per block of 64 nodes
+
+__global__ __launch_bounds__(FIT_MESSAGE_EVAL_BLOCK) void k_fit_message_eval(
     const uint32_t *__restrict__ rows, int row_words, const uint32_t *__restrict__ clause_X, int words, int n_nodes,
     int M, int C, int MC, int B, int K, int NC, uint32_t filter, const uint32_t *__restrict__ bank,
     const int32_t *__restrict__ weights, uint32_t k0, uint32_t k1, uint32_t step, int finish,
@@ -179,9 +181,10 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    constexpr int WAVES = FIT_EVAL_BLOCK / 64;
+    const int WAVES = (int)(blockDim.x >> 6);  // chosen by the host: few clauses -> many waves per clause
     const bool active = lane < words;
     const uint32_t *col = rows + (active ? lane : 0);
+    const bool rows_of_16_bytes = (MC & 3) == 0;  // a node's packed words can be read four at a time
     int partial = 0;
     for (int c = blockIdx.x; c < C; c += gridDim.x) {
         const uint32_t *inc = bank + (int64_t)c * MC * B + (B - 1);
@@ -200,7 +203,9 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
             const int live_blocks = __popcll((live_words | (live_words >> 1)) & 0x5555555555555555ull);
             for (int off = 32; off > 0; off >>= 1) here += __shfl_xor(here, off);
             const int trips_by_literal = (here + 7) >> 3;
-            const int trips_by_node = ((live_blocks + WAVES - 1) / WAVES) * ((__popcll(nonzero) + 7) >> 3);
+            const int chunk_words = MC - w0 < 64 ? MC - w0 : 64;
+            const int trips_by_node = ((live_blocks + WAVES - 1) / WAVES) *
+                                      (rows_of_16_bytes ? (chunk_words + 31) >> 5 : (__popcll(nonzero) + 7) >> 3);
             if (trips_by_node < trips_by_literal) {
                 if (tid < 64) handed[tid] = 0u;
                 __syncthreads();
@@ -214,6 +219,26 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_message_eval(
                     const uint32_t *x = clause_X + (int64_t)(node < n_nodes ? node : 0) * MC + w0;
                     unsigned long long todo = nonzero;
                     uint32_t violated = 0;
+                    if (rows_of_16_bytes) {
+                        // the node's words of this chunk, 32 per round trip, against the include words
+                        // (zero past the bank's last word, so words read for nothing change nothing)
+                        todo = 0ull;
+                        const uint4 *x4 = reinterpret_cast<const uint4 *>(x);
+                        for (int q0 = 0; q0 * 4 < chunk_words; q0 += 8) {
+                            uint4 xs[8];
+#pragma unroll
+                            for (int u = 0; u < 8; ++u)
+                                xs[u] = (q0 + u) * 4 < chunk_words ? x4[q0 + u] : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) {
+                                const int wl = ((q0 + u) * 4) & 63;
+                                violated |= (__builtin_amdgcn_readlane(mine, wl) & ~xs[u].x) |
+                                            (__builtin_amdgcn_readlane(mine, (wl + 1) & 63) & ~xs[u].y) |
+                                            (__builtin_amdgcn_readlane(mine, (wl + 2) & 63) & ~xs[u].z) |
+                                            (__builtin_amdgcn_readlane(mine, (wl + 3) & 63) & ~xs[u].w);
+                            }
+                        }
+                    }
                     while (todo) {
                         uint32_t xs[8], is[8];
 #pragma unroll

@@ -1611,7 +1611,11 @@ int fit_deep_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g,
                                    cx, n_nodes, d.M, d.MC, w.message_row_words, w.message_rows);
                 if (int rc = check_launch("fit_message_rows")) return rc;
             }
-            hipLaunchKernelGGL(k_fit_message_eval, dim3(d.C < 4096 ? d.C : 4096), dim3(FIT_EVAL_BLOCK), 0, st, w.message_rows,
+            // waves per clause: one per block of 64 nodes while the chip has room for that many
+            int eval_waves = (n_nodes + 63) / 64;
+            eval_waves = eval_waves < 4 ? 4 : eval_waves > FIT_MESSAGE_EVAL_BLOCK / 64 ? FIT_MESSAGE_EVAL_BLOCK / 64 : eval_waves;
+            if ((int64_t)d.C * eval_waves > 16384) eval_waves = 4;
+            hipLaunchKernelGGL(k_fit_message_eval, dim3(d.C < 4096 ? d.C : 4096), dim3(eval_waves * 64), 0, st, w.message_rows,
                                w.message_row_words, cx, words, n_nodes, d.M, d.C, d.MC, d.B, d.K, d.NC, d.mfilter,
                                s->message_ta_state[l], s->clause_weights, key.k0, key.k1, step, l == layers - 1 ? 1 : 0,
                                cur, nxt, w.n_incl, w.clause_node, sum_now);
