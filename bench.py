@@ -73,7 +73,7 @@ def oracle_twin(tm, n_nodes):
 
 def short_run(name, n_train, n_test, check_graphs):
     """Train one epoch and score once on a reduced copy of a configuration; check a few class sums
-    against the CPU oracle."""
+    against the NumPy oracle and all of them against the C one."""
     import numpy as np
     import torch
 
@@ -99,11 +99,25 @@ def short_run(name, n_train, n_test, check_graphs):
     sums = sums.cpu().numpy().reshape(n_test, -1)
     model = oracle_twin(tm, int(wl.graphs_test.max_number_of_graph_nodes))
     want = o.score(model, wl.graphs_test, range(check_graphs))
+    # the C restatement checks every test graph (16 host threads at most)
+    from oracle import gtm_oracle_c as oc
+
+    threads = max(1, min(16, oc.threads_available()))
+    t0 = time.perf_counter()
+    checked, same = 0, True
+    while checked < n_test and time.perf_counter() - t0 < 8.0:  # bounded: the colour workload costs ~0.5 s per graph
+        upto = min(n_test, checked + max(4 * threads, checked))
+        same = same and np.array_equal(oc.score(model, wl.graphs_test, range(checked, upto), threads=threads),
+                                       sums[checked:upto])
+        checked = upto
+    t_c = time.perf_counter() - t0
     return {
         "train_graphs": n_train, "test_graphs": n_test, "train_graphs_per_s": round(n_train / t_train, 1),
         "inference_graphs_per_s": round(n_test / t_test, 1),
         "test_accuracy": round(float((sums.argmax(axis=1) == wl.Y_test).mean()), 4),
         "class_sums_equal_oracle_on": check_graphs if np.array_equal(want, sums[:check_graphs]) else "MISMATCH",
+        "class_sums_equal_c_oracle_on": checked if same else "MISMATCH",
+        "c_oracle_graphs_per_s": round(checked / t_c, 1),
     }
 
 
@@ -212,27 +226,51 @@ def main():
     cpu = None
     if not args.no_cpu:
         from oracle import gtm_oracle as o
+        from oracle import gtm_oracle_c as oc
 
-        # the NumPy oracle costs ~3.5 ns per clause x node x word; aim at ~15 s
-        sample = args.cpu_sample or max(8, int(15.0 / (tm.number_of_clauses * n_nodes * la * tm.depth * 3.5e-9)))
-        sample = min(sample, args.graphs)
         model = oracle_twin(tm, n_nodes)
-        t0 = time.perf_counter()
-        want = o.score(model, test, range(sample))
-        t_cpu = time.perf_counter() - t0
-        if not np.array_equal(want, sums_host[:sample]):
-            print("bench.py: GPU class sums differ from the CPU oracle on the sample", file=sys.stderr)
+        # the C restatement of the reference's kernels on the box's host cores: whole passes over the
+        # step's graphs for about 10 s, every class sum compared with the GPU's
+        threads = max(1, min(16, oc.threads_available()))
+        passes, t0 = 0, time.perf_counter()
+        while True:
+            want = oc.score(model, test, threads=threads)
+            passes += 1
+            t_cpu = time.perf_counter() - t0
+            if t_cpu >= 10.0 or passes >= 200:
+                break
+        if not np.array_equal(want, sums_host):
+            print("bench.py: GPU class sums differ from the C oracle", file=sys.stderr)
             sys.exit(1)
-        # training: the same oracle, continuing from the GPU model's state on a few training graphs
-        train_sample = max(2, min(sample // 8, args.train_graphs))
+        rate = passes * args.graphs / t_cpu
+        # one thread, about 3 s
+        one = max(8, min(args.graphs, int(3.0 * rate / threads)))
+        t0 = time.perf_counter()
+        oc.score(model, test, range(one), threads=1)
+        t_one = time.perf_counter() - t0
+        # the NumPy oracle (~3.5 ns per clause x node x word) as a second opinion, about 3 s
+        sample = args.cpu_sample or max(8, int(3.0 / (tm.number_of_clauses * n_nodes * la * tm.depth * 3.5e-9)))
+        sample = min(sample, args.graphs)
+        t0 = time.perf_counter()
+        want_np = o.score(model, test, range(sample))
+        t_np = time.perf_counter() - t0
+        if not np.array_equal(want_np, sums_host[:sample]):
+            print("bench.py: GPU class sums differ from the NumPy oracle on the sample", file=sys.stderr)
+            sys.exit(1)
+        # training: the NumPy oracle, continuing from the GPU model's state on a few training graphs
+        train_sample = max(2, min(sample // 2, args.train_graphs))
         encoded = o.encode_labels(wl.Y_train[:train_sample], tm.number_of_outputs, tm.T)
         train_model = oracle_twin(tm, int(wl.graphs_train.max_number_of_graph_nodes))
         t0 = time.perf_counter()
         o.fit(train_model, wl.graphs_train, encoded, indices=range(train_sample))
         t_cpu_train = time.perf_counter() - t0
-        cpu = {"value": round(sample / t_cpu, 2), "unit": "graphs/s", "cores": 1, "kind": "port",
-               "sample": "NumPy oracle, inference on the first %d test graphs (%.1f s), checked equal to the GPU sums"
-                         % (sample, t_cpu),
+        cpu = {"value": round(rate, 1), "unit": "graphs/s", "cores": threads, "kind": "port",
+               "sample": "C restatement of the reference's kernels (oracle/gtm_oracle.c, OpenMP over graphs): %d "
+                         "pass(es) over the step's %d graphs in %.1f s, every class sum equal to the GPU's"
+                         % (passes, args.graphs, t_cpu),
+               "one_core_value": round(one / t_one, 1),
+               "numpy_value": round(sample / t_np, 2),
+               "numpy_sample": "NumPy oracle on the first %d graphs (%.1f s), equal to the GPU sums" % (sample, t_np),
                "train_value": round(train_sample / t_cpu_train, 2),
                "train_sample": "NumPy oracle, one training pass over %d graphs (%.1f s)" % (train_sample, t_cpu_train)}
 
