@@ -1,7 +1,8 @@
 """The 361-node convolutional configuration at its full test size (10,000 graphs, 2,500 clauses):
-properties that do not need the oracle to finish a 10,000-graph run.
+the C oracle on every graph, and properties that need no oracle at all.
 
-* a sample of the class sums equals the oracle;
+* every class sum equals the C restatement's (a few thousand graphs/s on the host cores), a sample
+  also the NumPy oracle's;
 * scoring is a per-graph function: a shuffled subset of the graphs scores to the same rows, whatever
   tile a graph lands in;
 * transform (per-operator kernels, clause/node bitmaps materialised) and score (tile kernels) agree:
@@ -14,6 +15,7 @@ import pytest
 
 from graphtsetlinmachine_amd import workloads
 from oracle import gtm_oracle as o
+from oracle import gtm_oracle_c as oc
 from tests.test_gpu_model import oracle_twin
 
 pytestmark = pytest.mark.gpu
@@ -39,6 +41,7 @@ def test_convolutional_configuration_at_full_test_size():
     model.cfg = oracle_twin(tm, test).cfg
     sample = [0, 1, 9, 10, 4999, 5003, 9989, 9999]
     assert np.array_equal(sums[sample], o.score(model, test, sample))
+    assert np.array_equal(sums, oc.score(model, test, threads=min(16, oc.threads_available())))
 
     # a shuffled subset lands in other tiles and other slots
     rng = np.random.default_rng(7)
@@ -71,6 +74,8 @@ def test_sequence_chains_at_full_test_size():
     model.clause_weights = tm.get_weights().copy()
     sample = [0, 1, 2, 2499, 4998, 4999]
     assert np.array_equal(sums[sample], o.score(model, test, sample))
+    every_fifth = list(range(0, 5000, 5))
+    assert np.array_equal(sums[every_fifth], oc.score(model, test, every_fifth, threads=min(16, oc.threads_available())))
 
     rng = np.random.default_rng(8)
     picked = rng.permutation(5000)[:1001]
