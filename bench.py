@@ -257,12 +257,21 @@ def main():
         if not np.array_equal(want_np, sums_host[:sample]):
             print("bench.py: GPU class sums differ from the NumPy oracle on the sample", file=sys.stderr)
             sys.exit(1)
-        # training: the NumPy oracle, continuing from the GPU model's state on a few training graphs
+        # training: the C restatement continuing from the GPU model's state for about 5 s (16 threads at
+        # most: clauses of one example in parallel, examples one after the other), and the NumPy oracle
+        # on a few graphs
+        train_model = oracle_twin(tm, int(wl.graphs_train.max_number_of_graph_nodes))
+        encoded_all = o.encode_labels(wl.Y_train, tm.number_of_outputs, tm.T)
+        trained, t0 = 0, time.perf_counter()
+        while trained < args.train_graphs and time.perf_counter() - t0 < 5.0:
+            upto = min(args.train_graphs, trained + 64)
+            oc.fit(train_model, wl.graphs_train, encoded_all, indices=range(trained, upto), threads=threads)
+            trained = upto
+        t_c_train = time.perf_counter() - t0
         train_sample = max(2, min(sample // 2, args.train_graphs))
-        encoded = o.encode_labels(wl.Y_train[:train_sample], tm.number_of_outputs, tm.T)
         train_model = oracle_twin(tm, int(wl.graphs_train.max_number_of_graph_nodes))
         t0 = time.perf_counter()
-        o.fit(train_model, wl.graphs_train, encoded, indices=range(train_sample))
+        o.fit(train_model, wl.graphs_train, encoded_all, indices=range(train_sample))
         t_cpu_train = time.perf_counter() - t0
         cpu = {"value": round(rate, 1), "unit": "graphs/s", "cores": threads, "kind": "port",
                "sample": "C restatement of the reference's kernels (oracle/gtm_oracle.c, OpenMP over graphs): %d "
@@ -271,8 +280,12 @@ def main():
                "one_core_value": round(one / t_one, 1),
                "numpy_value": round(sample / t_np, 2),
                "numpy_sample": "NumPy oracle on the first %d graphs (%.1f s), equal to the GPU sums" % (sample, t_np),
-               "train_value": round(train_sample / t_cpu_train, 2),
-               "train_sample": "NumPy oracle, one training pass over %d graphs (%.1f s)" % (train_sample, t_cpu_train)}
+               "train_value": round(trained / t_c_train, 1),
+               "train_sample": "C restatement, %d threads, %d training graphs one after the other (%.1f s)"
+                               % (threads, trained, t_c_train),
+               "numpy_train_value": round(train_sample / t_cpu_train, 2),
+               "numpy_train_sample": "NumPy oracle, one training pass over %d graphs (%.1f s)"
+                                     % (train_sample, t_cpu_train)}
 
     others = {}
     if not args.only_main:

@@ -1,9 +1,10 @@
-/* CPU restatement in plain C of the Graph Tsetlin Machine's inference path.
+/* CPU restatement in plain C of the Graph Tsetlin Machine's hot path.
  *
  * TEST INFRASTRUCTURE ONLY: nothing in the shipped package links or loads this
  * file.  It is a second, independent checker next to oracle/gtm_oracle.py (the
  * two are compared with each other in tests/test_oracle_c.py) and the CPU
- * baseline that bench.py times beside the GPU.
+ * baseline that bench.py times beside the GPU: inference (gtmc_score) and
+ * training (gtmc_fit).
  *
  * It follows the reference's CUDA kernels loop for loop, one graph at a time,
  * on the reference's own memory layouts:
@@ -54,6 +55,7 @@ static void clause_node_bits(int clauses, int node_chunks, int chunks, int state
                              const uint32_t *literal_words, const uint32_t *condition, uint32_t *out) {
     const int n_chunks = (n_nodes - 1) / 32 + 1; /* C division: 1 for a graph without nodes */
     const uint32_t node_filter = n_nodes % 32 != 0 ? ~(0xFFFFFFFFu << (n_nodes % 32)) : 0xFFFFFFFFu;
+#pragma omp parallel for schedule(static) /* (serial inside gtmc_score's own parallel region) */
     for (int clause = 0; clause < clauses; ++clause) {
         const uint32_t *ta = bank + (size_t)clause * chunks * state_bits + (state_bits - 1);
         for (int node_chunk = 0; node_chunk < node_chunks; ++node_chunk) {
@@ -180,6 +182,227 @@ int gtmc_score(const gtmc_config *cfg, const gtmc_graphs *g, const uint32_t *ta_
         free(packed);
     }
     return failed ? -1 : 0;
+}
+
+/* ---------------------------------------------------------------------------
+ * Training (tm.py:664-752): K7 select_clause_node (kernels.py:319-354), K8
+ * select_clause_updates (kernels.py:356-405), K9/K10 update and update_message
+ * (kernels.py:55-242), one example after the other.  The random numbers are the
+ * counter-based Philox4x32-10 ones that the NumPy oracle and the HIP kernels
+ * share (the reference's cuRAND stream depends on its launch shape and cannot be
+ * restated): which counter feeds which decision is stated at each use. */
+
+enum { TAG_CLAUSE_NODE = 2, TAG_CLAUSE_UPDATES = 3, TAG_FEEDBACK = 4 };
+
+static void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1, uint32_t out[4]) {
+    for (int round = 0; round < 10; ++round) { /* Salmon et al., SC'11; Random123 philox.h */
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1,
+                       n3 = (uint32_t)p0;
+        c0 = n0, c1 = n1, c2 = n2, c3 = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c0, out[1] = c1, out[2] = c2, out[3] = c3;
+}
+
+typedef struct {
+    int32_t threshold, boost_true_positive_feedback, max_included_literals, negative_clauses;
+    uint64_t q_threshold;   /* a negative target is kept when its 32-bit draw is below this */
+    uint64_t seed;
+    uint32_t feedback_threshold[8]; /* per bank: a Type I bit is set when its 16-bit draw is below this */
+} gtmc_training;
+
+/* kernels.py:55-74 / :77-96 on one word of automata: saturating +1 / -1 on the automata in `active`. */
+static void inc_word(uint32_t *ta, int state_bits, uint32_t active) {
+    uint32_t carry = active;
+    for (int b = 0; b < state_bits; ++b) {
+        const uint32_t next = ta[b] & carry;
+        ta[b] ^= carry;
+        carry = next;
+    }
+    for (int b = 0; b < state_bits; ++b) ta[b] |= carry;
+}
+
+static void dec_word(uint32_t *ta, int state_bits, uint32_t active) {
+    uint32_t carry = active;
+    for (int b = 0; b < state_bits; ++b) {
+        const uint32_t next = ~ta[b] & carry;
+        ta[b] ^= carry;
+        carry = next;
+    }
+    for (int b = 0; b < state_bits; ++b) ta[b] &= ~carry;
+}
+
+/* The 32 Type I feedback bits of word `w` of clause `c` for one class: four Philox blocks at
+ * counters (c, 4 w + j, step, TAG_FEEDBACK | bank << 8 | class << 16); bit b takes block b / 8,
+ * output word (b % 8) / 2, its low half for even b and its high half for odd b. */
+static uint32_t feedback_bits(const gtmc_training *t, uint32_t step, int bank, int class_id, int c, int w) {
+    const uint32_t k0 = (uint32_t)t->seed, k1 = (uint32_t)(t->seed >> 32);
+    const uint32_t c3 = (uint32_t)TAG_FEEDBACK | ((uint32_t)bank << 8) | ((uint32_t)class_id << 16);
+    uint32_t bits = 0;
+    for (int j = 0; j < 4; ++j) {
+        uint32_t r[4];
+        philox4x32_10((uint32_t)c, (uint32_t)(4 * w + j), step, c3, k0, k1, r);
+        for (int q = 0; q < 8; ++q) {
+            const uint32_t half = (q & 1) ? r[q >> 1] >> 16 : r[q >> 1] & 0xFFFFu;
+            if (half < t->feedback_threshold[bank]) bits |= 1u << (8 * j + q);
+        }
+    }
+    return bits;
+}
+
+/* K9 / K10 for one bank: classes in ascending order on the same automata (kernels.py:205-207, 236-238). */
+static void feedback(const gtmc_config *cfg, const gtmc_training *t, uint32_t step, int bank_id, uint32_t *bank,
+                     int chunks, const int32_t *clause_node, const int32_t *n_incl, const uint32_t *literal_words,
+                     const int32_t *updates) {
+    const int B = cfg->state_bits;
+#pragma omp parallel for schedule(static)
+    for (int c = 0; c < cfg->clauses; ++c) {
+        const int fired = clause_node[c] != -1;
+        const int within = n_incl[c] <= t->max_included_literals;
+        for (int w = 0; w < chunks; ++w) {
+            uint32_t *ta = bank + ((size_t)c * chunks + w) * B;
+            const uint32_t x = fired ? literal_words[(size_t)clause_node[c] * chunks + w] : 0u;
+            for (int k = 0; k < cfg->classes; ++k) {
+                const int32_t u = updates[(size_t)k * cfg->clauses + c];
+                if (u > 0) {
+                    const uint32_t fb = feedback_bits(t, step, bank_id, k, c, w);
+                    if (fired && within) {
+                        inc_word(ta, B, t->boost_true_positive_feedback == 1 ? x : x & ~fb);
+                        dec_word(ta, B, ~x & fb);
+                    } else {
+                        dec_word(ta, B, fb);
+                    }
+                } else if (u < 0 && fired) {
+                    inc_word(ta, B, ~x & ~ta[B - 1]);
+                }
+            }
+        }
+    }
+}
+
+static int include_count(const uint32_t *bank, int clause, int chunks, int state_bits, uint32_t filter) {
+    int n = 0; /* kernels.py:244-277 */
+    for (int w = 0; w < chunks; ++w) {
+        uint32_t include = bank[((size_t)clause * chunks + w) * state_bits + state_bits - 1];
+        if (w == chunks - 1) include &= filter;
+        n += __builtin_popcount(include);
+    }
+    return n;
+}
+
+/* One pass over the examples graph_ids[0..n) in that order; example i is training step
+ * first_step + i.  encoded_Y is [graphs][classes] (+T / -T, tm.py:949-951).  The banks and the
+ * weights are updated in place.  Returns 0, or -1 when memory runs out. */
+int gtmc_fit(const gtmc_config *cfg, const gtmc_training *t, const gtmc_graphs *g, uint32_t *ta_state,
+             uint32_t *const *message_ta_state, int32_t *clause_weights, const uint32_t *hypervectors,
+             const int32_t *encoded_Y, const int32_t *graph_ids, int32_t n, uint64_t first_step, int32_t threads) {
+    const int la_chunks = chunks_of(cfg->literals), message_chunks = chunks_of(2 * cfg->message_size);
+    const int node_chunks = chunks_of(cfg->max_nodes > 0 ? cfg->max_nodes : 1);
+    const uint32_t filter = tail_filter(cfg->literals), message_filter = tail_filter(2 * cfg->message_size);
+    const uint32_t k0 = (uint32_t)t->seed, k1 = (uint32_t)(t->seed >> 32);
+    const int C = cfg->clauses, K = cfg->classes, T = t->threshold, layers = cfg->depth - 1;
+    const size_t nodes = (size_t)(cfg->max_nodes > 0 ? cfg->max_nodes : 1);
+#ifdef _OPENMP
+    if (threads > 0) omp_set_num_threads(threads);
+#else
+    (void)threads;
+#endif
+    uint32_t *bitmap_a = malloc((size_t)C * node_chunks * 4), *bitmap_b = malloc((size_t)C * node_chunks * 4);
+    uint8_t *x_int = layers > 0 ? malloc(nodes * 2 * (size_t)cfg->message_size) : NULL;
+    uint32_t *packed = layers > 0 ? malloc((size_t)layers * nodes * message_chunks * 4) : NULL; /* kept per layer for K10 */
+    int32_t *n_incl = malloc((size_t)C * 4), *clause_node = malloc((size_t)C * 4), *updates = malloc((size_t)K * C * 4);
+    int32_t *sums = malloc((size_t)K * 4);
+    int rc = 0;
+    if (!bitmap_a || !bitmap_b || !n_incl || !clause_node || !updates || !sums || (layers > 0 && (!x_int || !packed))) rc = -1;
+    for (int32_t i = 0; rc == 0 && i < n; ++i) {
+        const int32_t e = graph_ids[i];
+        const uint32_t step = (uint32_t)(first_step + (uint64_t)i);
+        const int n_nodes = (int)g->number_of_graph_nodes[e];
+        const size_t base = g->node_index[e];
+        const uint32_t *types = g->node_type + base;
+        /* evaluation, keeping every layer's messages (tm.py:563-662) */
+        uint32_t *now = bitmap_a, *next = bitmap_b;
+        clause_node_bits(C, node_chunks, la_chunks, cfg->state_bits, filter, ta_state, types, g->number_of_node_types,
+                         n_nodes, g->X + base * la_chunks, NULL, now);
+        for (int c = 0; c < C; ++c) n_incl[c] = include_count(ta_state, c, la_chunks, cfg->state_bits, filter);
+        for (int layer = 0; layer < layers; ++layer) {
+            uint32_t *messages = packed + (size_t)layer * nodes * message_chunks;
+            const uint32_t *n_edges = g->number_of_graph_node_edges + base;
+            const uint32_t *edges = n_nodes > 0 ? g->edge + (size_t)g->edge_index[base] * 2 : g->edge;
+            build_messages(cfg, node_chunks, n_nodes, hypervectors, now, n_edges, edges, x_int, messages);
+            clause_node_bits(C, node_chunks, message_chunks, cfg->state_bits, message_filter, message_ta_state[layer],
+                             types, g->number_of_node_types, n_nodes, messages, now, next);
+            for (int c = 0; c < C; ++c)
+                n_incl[c] += include_count(message_ta_state[layer], c, message_chunks, cfg->state_bits, message_filter);
+            uint32_t *swap = now;
+            now = next;
+            next = swap;
+        }
+        class_sums(cfg, node_chunks, n_nodes, now, clause_weights, sums);
+        /* K7: a uniformly drawn true node per clause, -1 without one.  Draw: word 0 at counter
+         * (clause, 0, step, TAG_CLAUSE_NODE); index = (draw * count) >> 32 among the true nodes. */
+#pragma omp parallel for schedule(static)
+        for (int c = 0; c < C; ++c) {
+            int count = 0;
+            for (int node = 0; node < n_nodes; ++node) count += (now[(size_t)c * node_chunks + node / 32] >> (node % 32)) & 1u;
+            clause_node[c] = -1;
+            if (count > 0) {
+                uint32_t r[4];
+                philox4x32_10((uint32_t)c, 0u, step, TAG_CLAUSE_NODE, k0, k1, r);
+                int pick = (int)(((uint64_t)r[0] * (uint64_t)count) >> 32);
+                for (int node = 0; node < n_nodes; ++node)
+                    if ((now[(size_t)c * node_chunks + node / 32] >> (node % 32)) & 1u) {
+                        if (pick == 0) {
+                            clause_node[c] = node;
+                            break;
+                        }
+                        --pick;
+                    }
+            }
+        }
+        /* K8.  Draws at counter (clause, class, step, TAG_CLAUSE_UPDATES): word 0 gates negative
+         * targets, word 1 gates on the error, kept when draw * 2T < |y - sum| * 2^32. */
+        const int32_t *y = encoded_Y + (size_t)e * K;
+        for (int k = 0; k < K; ++k) {
+            const int64_t cs = sums[k] > T ? T : sums[k] < -T ? -T : sums[k];
+            const int target = 1 - 2 * (cs > y[k]);
+            const int64_t err = y[k] > cs ? y[k] - cs : cs - y[k];
+            for (int c = 0; c < C; ++c) {
+                int32_t *w = clause_weights + (size_t)k * C + c;
+                const int sign = *w >= 0 ? 1 : -1;
+                uint32_t r[4];
+                philox4x32_10((uint32_t)c, (uint32_t)k, step, TAG_CLAUSE_UPDATES, k0, k1, r);
+                const int skip = (target == -1 && (uint64_t)r[0] >= t->q_threshold) ||
+                                 ((uint64_t)r[1] * (uint64_t)(2 * (int64_t)T) >= ((uint64_t)err << 32));
+                const int u = skip ? 0 : target * sign;
+                const int fired = clause_node[c] != -1;
+                if (u > 0 && fired && (*w < 0 ? -(int64_t)*w : (int64_t)*w) < 2147483647) {
+                    *w += sign;
+                } else if (u < 0 && fired) {
+                    int64_t moved = (int64_t)*w - sign;
+                    if (t->negative_clauses == 0 && moved < 1) moved = 1;
+                    *w = (int32_t)moved;
+                }
+                updates[(size_t)k * C + c] = u;
+            }
+        }
+        /* K9, K10 */
+        feedback(cfg, t, step, 0, ta_state, la_chunks, clause_node, n_incl, g->X + base * la_chunks, updates);
+        for (int layer = 0; layer < layers; ++layer)
+            feedback(cfg, t, step, layer + 1, message_ta_state[layer], message_chunks, clause_node, n_incl,
+                     packed + (size_t)layer * nodes * message_chunks, updates);
+    }
+    free(bitmap_a);
+    free(bitmap_b);
+    free(x_int);
+    free(packed);
+    free(n_incl);
+    free(clause_node);
+    free(updates);
+    free(sums);
+    return rc;
 }
 
 int gtmc_threads_available(void) {

@@ -85,3 +85,49 @@ def test_sequence_chains_at_full_test_size():
     fired, part_sums = tm.transform(part)
     assert np.array_equal(part_sums, sums[1000:1300])
     assert np.array_equal(fired.astype(np.int64) @ tm.get_weights().T.astype(np.int64), part_sums)
+
+
+def test_training_at_full_model_size_follows_the_c_oracle():
+    """2,500 clauses on 361-node graphs: the state after 400 examples from the initial state, bit for
+    bit (the C restatement trains ~500 graphs/s on the host cores; the NumPy oracle needs minutes)."""
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    wl = workloads.convolutional_images(n_train=400, n_test=64)
+    np.random.seed(42)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=0, incremental=True)  # initial state only
+    model = oracle_twin(tm, wl.graphs_train)
+    state = tm.get_state()
+    assert np.array_equal(state[0], model.ta_state.reshape(-1)) and np.array_equal(
+        state[1].reshape(model.clause_weights.shape), model.clause_weights)
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
+    oc.fit(model, wl.graphs_train, o.encode_labels(wl.Y_train, tm.number_of_outputs, tm.T),
+           threads=min(16, oc.threads_available()))
+    state = tm.get_state()
+    assert np.array_equal(state[1].reshape(model.clause_weights.shape), model.clause_weights)
+    assert np.array_equal(state[0], model.ta_state.reshape(-1))
+    assert np.array_equal(tm.score(wl.graphs_test), oc.score(model, wl.graphs_test))
+
+
+@pytest.mark.parametrize("name,n_train", [("sequence_chains", 600), ("colour_convolution", 16), ("single_node_images", 600),
+                                          ("noisy_xor", 3000), ("runs_of_a", 3000)])
+def test_training_of_every_configuration_follows_the_c_oracle(name, n_train):
+    """Each configuration at its full model size (the colour one: 8,000 clauses, three banks of
+    2,048 literals, 841 nodes): the state after n_train examples from the initial state, bit for bit."""
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    wl = workloads.BUILDERS[name](n_train=n_train, n_test=8)
+    np.random.seed(42)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=0, incremental=True)  # initial state only
+    model = oracle_twin(tm, wl.graphs_train)
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
+    oc.fit(model, wl.graphs_train, o.encode_labels(wl.Y_train, tm.number_of_outputs, tm.T),
+           threads=min(16, oc.threads_available()))
+    saved = tm.save()
+    assert np.array_equal(saved["clause_weights"].reshape(model.clause_weights.shape), model.clause_weights)
+    assert np.array_equal(saved["ta_state"], model.ta_state.reshape(-1))
+    for got, want in zip(saved["message_ta_state"], model.message_ta_state):
+        assert np.array_equal(got, want.reshape(-1))
+    model.cfg = oracle_twin(tm, wl.graphs_test).cfg
+    assert np.array_equal(tm.score(wl.graphs_test), oc.score(model, wl.graphs_test))

@@ -50,3 +50,34 @@ def test_c_oracle_on_a_model_trained_by_the_numpy_oracle():
     Y = o.encode_labels(rng.integers(0, 3, size=30), 3, cfg.threshold)
     o.fit(model, graphs, Y, epochs=2)
     assert np.array_equal(oc.score(model, graphs), o.score(model, graphs))
+
+
+@pytest.mark.parametrize("shape", SHAPES[:6], ids=lambda s: "seed%d" % s["seed"])
+@pytest.mark.parametrize("boost,max_included,state_bits,negative", [(1, None, 8, 1), (0, 9, 5, 1), (1, None, 12, 0)])
+def test_c_and_numpy_oracles_train_alike(shape, boost, max_included, state_bits, negative):
+    """Two epochs, the second split into two calls and run on three threads: banks, weights and step."""
+    import copy
+
+    g = dict(shape["g"])
+    graphs = helpers.random_graphs(shape["seed"], **g)
+    m = dict(shape["m"])
+    depth = m.pop("depth")
+    m.pop("state_bits", None)
+    cfg = helpers.oracle_config(graphs, **m, depth=depth, T=30, boost=boost, max_included=max_included,
+                                state_bits=state_bits)
+    cfg.negative_clauses = negative
+    model = helpers.random_model(shape["seed"], cfg, depth, s=(3.0, 2.0, 1.0)[:depth] if depth > 1 else 3.0,
+                                 include_density=0.03, message_density=0.02)
+    twin = copy.deepcopy(model)
+    rng = np.random.default_rng(shape["seed"])
+    G = graphs.number_of_graphs
+    Y = o.encode_labels(rng.integers(0, cfg.classes, size=G), cfg.classes, cfg.threshold)
+    o.fit(model, graphs, Y, epochs=2)
+    oc.fit(twin, graphs, Y)
+    oc.fit(twin, graphs, Y, indices=range(G // 2), threads=3)
+    oc.fit(twin, graphs, Y, indices=range(G // 2, G), threads=3)
+    assert twin.step == model.step
+    assert np.array_equal(twin.clause_weights, model.clause_weights)
+    assert np.array_equal(twin.ta_state, model.ta_state)
+    for a, b in zip(twin.message_ta_state, model.message_ta_state):
+        assert np.array_equal(a, b)
