@@ -879,6 +879,20 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     int group = 16;  // words of a truth row per k_tile_node_messages block: its vectors must fit in 64 KB of LDS
     while (group > 1 && (size_t)32 * group * MW * 4 > 64 * 1024) group >>= 1;
     a.message_rows = w.message_rows;
+    const size_t fused_lds = tg.slot_words > 0 ? tile_fused_messages_lds_bytes(tg, MW) : 0;
+    bool fused_messages = tg.slot_words > 0 && d.M % 32 == 0 && fused_lds <= 150 * 1024 && !getenv("GTM_NO_FUSED_MESSAGES");
+    if (fused_messages) {
+        static thread_local size_t fused_lds_set = 48 * 1024;
+        if (fused_lds > fused_lds_set) {
+            if (hipFuncSetAttribute((const void *)k_tile_messages_fused, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)fused_lds) != hipSuccess) {
+                (void)hipGetLastError();
+                fused_messages = false;
+            } else {
+                fused_lds_set = fused_lds;
+            }
+        }
+    }
     static thread_local bool node_messages_lds_raised = false;
     if (!node_messages_lds_raised) {
         hipError_t e = hipFuncSetAttribute((const void *)k_tile_node_messages,
@@ -894,7 +908,19 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         a.class_sum = class_sum;
         if (int rc = layer0(n_tiles, false)) return rc;
         for (int l = 1; l < layers; ++l) {
-            // the layer's message rows for these tiles (score_tiles.h)
+            // the layer's message rows for these tiles (score_tiles.h): one graph per workgroup with its
+            // vectors in LDS when they fit, else three launches with the vectors in global memory
+            if (fused_messages) {
+                hipLaunchKernelGGL(k_tile_messages_fused, dim3(tg.gpt, n_tiles), dim3(TILE_FUSED_MESSAGES_BLOCK),
+                                   fused_lds, st, w.tile_bitmap, d.C, tg, t0, g->number_of_graphs, d.M, MW, s->hypervectors,
+                                   d.MB, g->node_index, g->number_of_graph_nodes, g->number_of_graph_node_edges,
+                                   g->edge_index, g->edge, g->total_edges > 0 ? 1 : 0, w.message_rows);
+                if (int rc = check_launch("tile_messages_fused")) return rc;
+                a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
+                a.stride = w.message_list_stride;
+                if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1, st)) return rc;
+                continue;
+            }
             hipLaunchKernelGGL(k_tile_node_messages, dim3((tg.tw + group - 1) / group, n_tiles),
                                dim3(TILE_MESSAGES_BLOCK), (size_t)32 * group * MW * 4, st, w.tile_bitmap, d.C, tg.tw,
                                group, s->hypervectors, d.MB, MW, w.sent);

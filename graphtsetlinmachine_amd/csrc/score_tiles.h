@@ -458,6 +458,149 @@ __global__ __launch_bounds__(256) void k_tile_pack_messages(const uint32_t *__re
     }
 }
 
+// The three steps above for one graph per workgroup with the vectors in LDS (no sent / got in
+// global memory, no global atomics): tiles of whole-word slots, M a multiple of 32, and a graph's
+// vectors small enough - 2 * slot_bits * (MW | 1) words of LDS.  grid (graphs per tile,
+// tiles of the launch), 1,024 threads.
+//   1. sent[slot] |= hypervector bits of every clause true at the slot (LDS atomics)
+//   2. got[destination] |= rotate(sent[slot], edge type) along every out-edge (LDS atomics)
+//   3. got turned literal-major, 64 slots at a time by ballots; a wave collects 32 rows in LDS (in
+//      the space of sent, which is no longer needed) and writes them whole: rows[tile][M + 2][tw],
+//      the graph's words of each; plus the all-ones row and the row of graphs without nodes.
+// The workgroup of a tile's last graph also clears the words past the last slot of every row.
+constexpr int TILE_FUSED_MESSAGES_BLOCK = 1024;
+
+inline size_t tile_fused_messages_lds_bytes(const TileGeom &g, int MW) {
+    return 2 * (size_t)g.slot_bits * (MW | 1) * 4;  // vectors are MW | 1 words apart: lanes on different slots hit different banks
+}
+
+__global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fused(
+    const uint32_t *__restrict__ bitmap, int C, TileGeom tg, int tile0, int G, int M, int MW,
+    const uint32_t *__restrict__ hv, int MB, const uint32_t *__restrict__ node_index,
+    const uint32_t *__restrict__ n_nodes, const uint32_t *__restrict__ n_edges, const uint32_t *__restrict__ edge_index,
+    const uint32_t *__restrict__ edge, int has_edges, uint32_t *__restrict__ rows) {
+    extern __shared__ uint32_t lds[];
+    constexpr int NT = TILE_FUSED_MESSAGES_BLOCK;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int gj = blockIdx.x, tile_local = blockIdx.y;
+    const int tw = tg.tw, sw = tg.slot_words, slots = tg.slot_bits, MWP = MW | 1;
+    uint32_t *sent = lds;               // [slots][MWP]
+    uint32_t *got = lds + slots * MWP;  // [slots][MWP]
+    const int64_t g = (int64_t)(tile0 + tile_local) * tg.gpt + gj;
+    const int nodes = g < G ? (int)n_nodes[g] : 0;
+    const int w_first = gj * sw;        // the graph's first word of a tile row
+    uint32_t *out = rows + (int64_t)tile_local * (M + 2) * tw;
+
+    for (int i = tid; i < 2 * slots * MWP; i += NT) lds[i] = 0u;
+    __syncthreads();
+
+    // 1. what every node slot sends
+    if (nodes > 0) {
+        const uint32_t *truth = bitmap + (int64_t)tile_local * C * tw + w_first;
+        const int used = (nodes + 31) >> 5;  // words of a truth row that can hold a true node
+        constexpr int AHEAD = 4;
+        for (int i0 = tid; i0 < C * used; i0 += AHEAD * NT) {
+            uint32_t words[AHEAD], h01[AHEAD][2];  // the clause's first two hypervector bits travel with the word
+            int cs[AHEAD], wls[AHEAD];
+#pragma unroll
+            for (int u = 0; u < AHEAD; ++u) {
+                const int i = i0 + u * NT;
+                const bool in_range = i < C * used;
+                cs[u] = in_range ? i / used : 0;
+                wls[u] = i - cs[u] * used;
+                words[u] = in_range ? truth[(int64_t)cs[u] * tw + wls[u]] : 0u;
+                h01[u][0] = hv[(int64_t)cs[u] * MB];
+                h01[u][1] = MB > 1 ? hv[(int64_t)cs[u] * MB + 1] : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < AHEAD; ++u) {
+                const uint32_t word = words[u];
+                if (!word) continue;
+                for (int j = 0; j < MB; ++j) {
+                    const uint32_t h = j < 2 ? h01[u][j] : hv[(int64_t)cs[u] * MB + j];
+                    const uint32_t bit = 1u << (h & 31);
+                    uint32_t *column = sent + (wls[u] * 32) * MWP + (h >> 5);
+                    for (uint32_t m = word; m; m &= m - 1) atomicOr(&column[(__ffs(m) - 1) * MWP], bit);
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // 2. along the edges: bit p of what arrives is bit (p - type) mod M of what was sent
+    // (one thread per node: its edge list is two dependent memory round trips, paid once for all
+    // the vector words)
+    if (has_edges && nodes > 0) {
+        const int64_t row0 = node_index[g];
+        for (int n = tid; n < nodes; n += NT) {
+            const uint32_t *v = sent + n * MWP;
+            const uint32_t ne = n_edges[row0 + n];
+            const uint2 *out_edges = reinterpret_cast<const uint2 *>(edge) + edge_index[row0 + n];
+            for (uint32_t e0 = 0; e0 < ne; e0 += 4) {
+                uint2 pair[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) pair[u] = e0 + u < ne ? out_edges[e0 + u] : make_uint2(0u, 0u);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (e0 + u >= ne) break;
+                    const uint32_t dst = pair[u].x, shift = pair[u].y % (uint32_t)M;
+                    const int q = (int)(shift >> 5), r = (int)(shift & 31u);
+                    int a = (int)((MW - q) % MW);  // word of v that feeds word 0
+                    for (int j = 0; j < MW; ++j) {
+                        const int below = a == 0 ? MW - 1 : a - 1;
+                        const uint32_t word = r ? (v[a] << r) | (v[below] >> (32 - r)) : v[a];
+                        if (word) atomicOr(&got[dst * MWP + j], word);
+                        a = a + 1 == MW ? 0 : a + 1;
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // 3. literal-major rows: wave v turns vector words v, v + 16, ... (32 rows each) and writes
+    // the graph's words of those rows; its 32 x sw words of staging live where sent was
+    const int pack_waves = MW < NT / 64 ? MW : NT / 64;
+    if (wave < pack_waves) {
+        uint32_t *stage = sent + wave * 32 * sw;  // [32 rows][sw]
+        for (int j = wave; j < MW; j += pack_waves) {
+            for (int nb = 0; nb * 2 < sw; ++nb) {
+                const int slot = nb * 64 + lane;
+                const uint32_t word = slot < slots ? got[slot * MWP + j] : 0u;
+                unsigned long long mine = 0;
+#pragma unroll
+                for (int b = 0; b < 32; ++b) {
+                    const unsigned long long column = __ballot((word >> b) & 1u);
+                    if (lane == b) mine = column;
+                }
+                if (lane < 32) {
+                    stage[lane * sw + nb * 2] = (uint32_t)mine;
+                    if (nb * 2 + 1 < sw) stage[lane * sw + nb * 2 + 1] = (uint32_t)(mine >> 32);
+                }
+            }
+            // (a wave's LDS writes are visible to its own later reads: same wave, in order)
+            for (int i = lane; i < 32 * sw; i += 64) {
+                const int r = i / sw, w = i - r * sw;
+                out[(int64_t)(j * 32 + r) * tw + w_first + w] = stage[i];
+            }
+        }
+    }
+    // the all-ones row and the row of graphs without nodes (kernels.py:443-466,505-527 leave every
+    // clause true for such a graph at every layer, which the message literals must not undo)
+    for (int w = tid; w < sw; w += NT) {
+        out[(int64_t)M * tw + w_first + w] = 0xFFFFFFFFu;
+        out[(int64_t)(M + 1) * tw + w_first + w] = (w == 0 && g < G && nodes == 0) ? 1u : 0u;
+    }
+    // words past the tile's last slot
+    if (gj == tg.gpt - 1) {
+        const int from = tg.gpt * sw, extra = tw - from;
+        for (int i = tid; i < (M + 2) * extra; i += NT) {
+            const int r = i / extra, w = i - r * extra;
+            out[(int64_t)r * tw + from + w] = 0u;
+        }
+    }
+}
+
 // One layer of clause evaluation for one tile per workgroup.
 //
 // Layer 0 (ROWS_STAGED / ROWS_GLOBAL): a clause's truth over the tile's node
