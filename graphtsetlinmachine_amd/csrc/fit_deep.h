@@ -75,14 +75,15 @@ __global__ __launch_bounds__(64) void k_fit_message_rows(const uint32_t *__restr
 constexpr int FIT_NODE_MESSAGES_BLOCK = 256;
 constexpr int FIT_NODE_MESSAGES_CLAUSES = 1024;  // clauses per block
 
-// grid (node words in use, ceil(C / FIT_NODE_MESSAGES_CLAUSES)); dynamic LDS 32 * MW words
+// grid (node words in use, ceil(C / FIT_NODE_MESSAGES_CLAUSES)); dynamic LDS 32 * (MW | 1) words
 __global__ __launch_bounds__(FIT_NODE_MESSAGES_BLOCK) void k_fit_node_messages(
     const uint32_t *__restrict__ bitmap, int C, int NC, int n_nodes, const uint32_t *__restrict__ hv, int MB, int MW,
     uint32_t *sent) {
-    extern __shared__ uint32_t vec[];  // [32 nodes][MW]
+    extern __shared__ uint32_t vec[];  // [32 nodes][MW | 1]: lanes on different nodes hit different banks
     const int tid = threadIdx.x;
     const int nw = blockIdx.x;
-    for (int i = tid; i < 32 * MW; i += FIT_NODE_MESSAGES_BLOCK) vec[i] = 0u;
+    const int MWP = MW | 1;
+    for (int i = tid; i < 32 * MWP; i += FIT_NODE_MESSAGES_BLOCK) vec[i] = 0u;
     __syncthreads();
     const int c_end = min(C, (int)(blockIdx.y + 1) * FIT_NODE_MESSAGES_CLAUSES);
     const uint32_t valid = n_nodes - nw * 32 >= 32 ? 0xFFFFFFFFu : (1u << (n_nodes - nw * 32)) - 1u;
@@ -93,14 +94,15 @@ __global__ __launch_bounds__(FIT_NODE_MESSAGES_BLOCK) void k_fit_node_messages(
             word &= word - 1;
             for (int j = 0; j < MB; ++j) {
                 const uint32_t h = hv[(int64_t)c * MB + j];
-                atomicOr(&vec[n * MW + (h >> 5)], 1u << (h & 31));
+                atomicOr(&vec[n * MWP + (h >> 5)], 1u << (h & 31));
             }
         }
     }
     __syncthreads();
     for (int i = tid; i < 32 * MW; i += FIT_NODE_MESSAGES_BLOCK) {
         const int n = nw * 32 + i / MW;
-        if (vec[i] != 0u && n < n_nodes) atomicOr(&sent[(int64_t)n * MW + (i % MW)], vec[i]);
+        const uint32_t word = vec[(i / MW) * MWP + i % MW];
+        if (word != 0u && n < n_nodes) atomicOr(&sent[(int64_t)n * MW + (i % MW)], word);
     }
 }
 

@@ -324,15 +324,16 @@ inline size_t tile_layer_lds_bytes(const TileGeom &g, int classes, int src, int 
 constexpr int TILE_MESSAGES_BLOCK = 256;
 
 // grid (ceil(tw / group), tiles); `group` consecutive words of every truth row of the tile per
-// block (a power of two <= 16: one cache line per clause), dynamic LDS 32 * group * MW words.
+// block (a power of two <= 16: one cache line per clause), dynamic LDS 32 * group * (MW | 1) words.
 // Every word of sent is written (no clearing needed).
 __global__ __launch_bounds__(TILE_MESSAGES_BLOCK) void k_tile_node_messages(
     const uint32_t *__restrict__ bitmap, int C, int tw, int group, const uint32_t *__restrict__ hv, int MB, int MW,
     uint32_t *__restrict__ sent) {
-    extern __shared__ uint32_t vec[];  // [32 * group slots][MW]
+    extern __shared__ uint32_t vec[];  // [32 * group slots][MW | 1]: lanes on different slots hit different banks
     const int tid = threadIdx.x;
     const int w0 = blockIdx.x * group, tile = blockIdx.y;
-    const int n_vec = 32 * group * MW;
+    const int MWP = MW | 1;
+    const int n_vec = 32 * group * MWP;
     for (int i = tid; i < n_vec; i += TILE_MESSAGES_BLOCK) vec[i] = 0u;
     __syncthreads();
     const int wl = tid & (group - 1), w = w0 + wl;
@@ -355,15 +356,15 @@ __global__ __launch_bounds__(TILE_MESSAGES_BLOCK) void k_tile_node_messages(
                 for (int j = 0; j < MB; ++j) {
                     const uint32_t h = hv[(int64_t)c * MB + j];
                     const uint32_t bit = 1u << (h & 31);
-                    uint32_t *column = vec + (wl * 32) * MW + (h >> 5);
-                    for (uint32_t m = word; m; m &= m - 1) atomicOr(&column[(__ffs(m) - 1) * MW], bit);
+                    uint32_t *column = vec + (wl * 32) * MWP + (h >> 5);
+                    for (uint32_t m = word; m; m &= m - 1) atomicOr(&column[(__ffs(m) - 1) * MWP], bit);
                 }
             }
         }
     __syncthreads();
     uint32_t *out = sent + ((int64_t)tile * tw + w0) * 32 * MW;
     const int n_out = (min(tw, w0 + group) - w0) * 32 * MW;
-    for (int i = tid; i < n_out; i += TILE_MESSAGES_BLOCK) out[i] = vec[i];
+    for (int i = tid; i < n_out; i += TILE_MESSAGES_BLOCK) out[i] = vec[(i / MW) * MWP + i % MW];
 }
 
 // One thread per (tile of the launch, node slot, vector word).
