@@ -146,16 +146,8 @@ __global__ __launch_bounds__(64) void k_fit_pack_messages(uint32_t *sent, uint32
         clause_X[(int64_t)n * 2 * MW + j] = word;
         clause_X[(int64_t)n * 2 * MW + MW + j] = ~word;
     }
-    unsigned long long mine = 0;
-#pragma unroll
-    for (int b = 0; b < 32; ++b) {
-        const unsigned long long column = __ballot((word >> b) & 1u);
-        if (lane == b) mine = column;
-    }
-    if (lane < 32) {
-        rows[(int64_t)(j * 32 + lane) * row_words + nb * 2] = (uint32_t)mine;
-        rows[(int64_t)(j * 32 + lane) * row_words + nb * 2 + 1] = (uint32_t)(mine >> 32);
-    }
+    // each half of the wave transposes its 32 nodes x 32 bits: lane b of a half holds one word of row 32 j + b
+    rows[(int64_t)(j * 32 + (lane & 31)) * row_words + nb * 2 + (lane >> 5)] = tile_transpose32(word, lane);
 }
 
 // K2 (+ K6 + K7 when `finish`) for one graph and one message layer.  Each block

@@ -323,6 +323,21 @@ inline size_t tile_layer_lds_bytes(const TileGeom &g, int classes, int src, int 
 
 constexpr int TILE_MESSAGES_BLOCK = 256;
 
+// Transposes the 32 x 32 bit matrix whose row i is the word of lane i (of each half of the wave):
+// afterwards bit i of lane b's word is what bit b of lane i's word was.  Five exchanges of
+// half-blocks with the lane 16, 8, 4, 2, 1 away.
+__device__ __forceinline__ uint32_t tile_transpose32(uint32_t v, int lane) {
+#pragma unroll
+    for (int j = 16; j >= 1; j >>= 1) {
+        // columns whose index has bit j clear
+        const uint32_t m = j == 16 ? 0x0000FFFFu : j == 8 ? 0x00FF00FFu : j == 4 ? 0x0F0F0F0Fu : j == 2 ? 0x33333333u : 0x55555555u;
+        const uint32_t p = (uint32_t)__shfl_xor((int)v, j);
+        v = (lane & j) ? ((p >> j) & m) | (v & ~m) : (v & m) | ((p & m) << j);
+    }
+    return v;
+}
+
+
 // grid (ceil(tw / group), tiles); `group` consecutive words of every truth row of the tile per
 // block (a power of two <= 16: one cache line per clause), dynamic LDS 32 * group * (MW | 1) words.
 // Every word of sent is written (no clearing needed).
@@ -407,7 +422,7 @@ __global__ void k_tile_edge_messages(const uint32_t *__restrict__ sent, TileGeom
 
 // grid (ceil(tw / 2), tiles), 256 threads: the received vectors of 64 node slots go through LDS
 // (read row by row, coalesced) and come out literal-major: wave v turns vector words v, v + 4, ...
-// into rows 32 j .. 32 j + 31 (lane = slot, one ballot per bit).  Wave 0 also writes the all-ones
+// into rows 32 j .. 32 j + 31 (lane = slot, a 32 x 32 bit transposition across the lanes of each half).  Wave 0 also writes the all-ones
 // row M and row M + 1 (slot bit 0 of the graphs without nodes: the reference's chunk arithmetic
 // leaves every clause true for such a graph at every layer, kernels.py:443-466,505-527, which the
 // message literals must not undo).  Dynamic LDS 64 * (MW + 1) words.
@@ -427,17 +442,10 @@ __global__ __launch_bounds__(256) void k_tile_pack_messages(const uint32_t *__re
     const bool lo_ok = nb * 2 < tw, hi_ok = nb * 2 + 1 < tw;
     for (int j = wave; j < MW; j += 4) {
         const uint32_t word = lane < n_here ? block[lane * (MW + 1) + j] : 0u;
-        unsigned long long mine = 0;
-#pragma unroll
-        for (int b = 0; b < 32; ++b) {
-            const unsigned long long column = __ballot((word >> b) & 1u);
-            if (lane == b) mine = column;
-        }
-        const int p = j * 32 + lane;
-        if (lane < 32 && p < M) {
-            if (lo_ok) out[(int64_t)p * tw + nb * 2] = (uint32_t)mine;
-            if (hi_ok) out[(int64_t)p * tw + nb * 2 + 1] = (uint32_t)(mine >> 32);
-        }
+        // each half of the wave transposes its 32 slots x 32 bits: lane b of a half holds one word of row 32 j + b
+        const uint32_t column = tile_transpose32(word, lane);
+        const int p = j * 32 + (lane & 31);
+        if (p < M && (lane < 32 ? lo_ok : hi_ok)) out[(int64_t)p * tw + nb * 2 + (lane >> 5)] = column;
     }
     if (wave == 0) {
         const int pos = nb * 64 + lane;
@@ -465,7 +473,8 @@ __global__ __launch_bounds__(256) void k_tile_pack_messages(const uint32_t *__re
 // tiles of the launch), 1,024 threads.
 //   1. sent[slot] |= hypervector bits of every clause true at the slot (LDS atomics)
 //   2. got[destination] |= rotate(sent[slot], edge type) along every out-edge (LDS atomics)
-//   3. got turned literal-major, 64 slots at a time by ballots; a wave collects 32 rows in LDS (in
+//   3. got turned literal-major, 64 slots at a time (two 32 x 32 bit transpositions across the
+//      lanes); a wave collects 32 rows in LDS (in
 //      the space of sent, which is no longer needed) and writes them whole: rows[tile][M + 2][tw],
 //      the graph's words of each; plus the all-ones row and the row of graphs without nodes.
 // The workgroup of a tile's last graph also clears the words past the last slot of every row.
@@ -568,16 +577,10 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
             for (int nb = 0; nb * 2 < sw; ++nb) {
                 const int slot = nb * 64 + lane;
                 const uint32_t word = slot < slots ? got[slot * MWP + j] : 0u;
-                unsigned long long mine = 0;
-#pragma unroll
-                for (int b = 0; b < 32; ++b) {
-                    const unsigned long long column = __ballot((word >> b) & 1u);
-                    if (lane == b) mine = column;
-                }
-                if (lane < 32) {
-                    stage[lane * sw + nb * 2] = (uint32_t)mine;
-                    if (nb * 2 + 1 < sw) stage[lane * sw + nb * 2 + 1] = (uint32_t)(mine >> 32);
-                }
+                // lanes 0..31 and 32..63 each transpose their 32 x 32 bits: lane b of a half ends up
+                // with bit b of the half's 32 slots, i.e. one word of row 32 j + b
+                const uint32_t column = tile_transpose32(word, lane);
+                if (nb * 2 + (lane >> 5) < sw) stage[(lane & 31) * sw + nb * 2 + (lane >> 5)] = column;
             }
             // (a wave's LDS writes are visible to its own later reads: same wave, in order)
             for (int i = lane; i < 32 * sw; i += 64) {
