@@ -679,9 +679,24 @@ TileGeom geometry_for(const gtm_config *cfg, const gtm_graphs *g, int classes) {
                          classes, max_lane_words(), cfg->depth > 1 ? tile_message_rows(cfg->message_size) : 0);
 }
 
+// Workgroups that share a tile's clauses when layer 0 reads its rows in place and the tiles are few.
+int tile_layer_splits(const TileLayerArgs &a, int n_tiles, int src) {
+    if (src != ROWS_GLOBAL) return 1;
+    int splits = (512 + n_tiles - 1) / n_tiles;
+    const int most = (a.C + 15) / 16;  // at least one clause per wave
+    splits = splits > most ? most : splits;
+    return splits < 1 ? 1 : splits > 64 ? 64 : splits;
+}
+
 template <int NW, int LW, int SRC, bool LAST>
 int launch_tile_layer_as(const TileLayerArgs &a, int n_tiles, const char *profile_name, hipStream_t st) {
     size_t lds = tile_layer_lds_bytes(a.tg, a.K, SRC, a.M);
+    const int splits = tile_layer_splits(a, n_tiles, SRC);
+    if (LAST && splits > 1) {  // the workgroups of a tile add their shares
+        const int64_t n = (int64_t)a.n_graphs * a.K;
+        hipLaunchKernelGGL(k_fill_i32, dim3(blocks_for(n, TPB)), dim3(TPB), 0, st, a.class_sum, n, 0);
+        if (int rc = check_launch("fill")) return rc;
+    }
     static thread_local size_t lds_set = 48 * 1024;
     if (lds > lds_set) {
         hipError_t e = hipFuncSetAttribute((const void *)k_tile_layer<NW, LW, SRC, LAST>,
@@ -690,7 +705,7 @@ int launch_tile_layer_as(const TileLayerArgs &a, int n_tiles, const char *profil
         lds_set = lds;
     }
     if (profile_name) profile_start(profile_name, st);
-    hipLaunchKernelGGL((k_tile_layer<NW, LW, SRC, LAST>), dim3(n_tiles), dim3(NW * 64), lds, st, a);
+    hipLaunchKernelGGL((k_tile_layer<NW, LW, SRC, LAST>), dim3(n_tiles, splits), dim3(NW * 64), lds, st, a);
     if (int rc = check_launch("tile_layer")) return rc;
     if (profile_name) profile_stop(st);
     return GTM_OK;

@@ -107,7 +107,16 @@ inline TileGeom tile_geometry(int literals, int n_types, int max_nodes, int n_gr
             // (1 + lw) / gpt, compared without division; ties go to the wider lanes
             if (!best.ok || (int64_t)(1 + g.lw) * best.gpt < (int64_t)(1 + best.lw) * g.gpt) best = g;
         }
-        if (best.ok) return best;
+        if (best.ok) {
+            // Tiny graphs (several per word) whose many literal rows fit in LDS only at a fraction of the
+            // 64 lanes' width: full-width rows read in place (global memory, L2) keep every lane busy
+            // and leave few, large tiles, whose clauses several workgroups then share.
+            if (message_rows == 0 && best.slot_words == 0 && best.tw < 64 * best.lw) {
+                TileGeom wide = tile_geometry_lw(literals, n_types, max_nodes, n_graphs, classes, best.lw, 0);
+                if (wide.ok && wide.tw > best.tw) return wide;
+            }
+            return best;
+        }
     }
     best.ok = 0;
     return best;
@@ -816,10 +825,12 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
         // Two clauses per trip so that the chunk fetched ahead never has to be copied.  Pointers step
         // by NWAVES clauses; past the end they stay on the wave's last clause (a valid address whose
         // data is not used).
-        const int64_t list_step = (int64_t)NWAVES * a.stride;
-        const int wt_step = NWAVES * K;
-        const int64_t truth_step = (int64_t)NWAVES * tw * 4;
-        const int first = wave < C ? wave : 0;
+        // gridDim.y workgroups share the tile's clauses (rows read in place: nothing ties a tile to one)
+        const int c_step = NWAVES * (int)gridDim.y, c_first = wave + NWAVES * (int)blockIdx.y;
+        const int64_t list_step = (int64_t)c_step * a.stride;
+        const int wt_step = c_step * K;
+        const int64_t truth_step = (int64_t)c_step * tw * 4;
+        const int first = c_first < C ? c_first : 0;
         const uint32_t *list_a = a.lists + (int64_t)first * a.stride;
         const int32_t *wt_a = LAST ? a.wt + (int64_t)first * K : nullptr;
         char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
@@ -827,14 +838,14 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
         LaneWords<LW> none;
 #pragma unroll
         for (int u = 0; u < LW; ++u) none.w[u] = 0u;
-        for (int c = wave; c < C; c += 2 * NWAVES) {
-            const bool has_b = c + NWAVES < C;
+        for (int c = c_first; c < C; c += 2 * c_step) {
+            const bool has_b = c + c_step < C;
             const uint32_t *list_b = has_b ? list_a + list_step : list_a;
             const int32_t *wt_b = LAST ? (has_b ? wt_a + wt_step : wt_a) : nullptr;
             char *truth_b = has_b ? truth_a + truth_step : truth_a;
             const Chunk32 cb = *reinterpret_cast<const Chunk32 *>(list_b);
             evaluate(ca, list_a, wt_a, none, truth_a);
-            const bool has_a = c + 2 * NWAVES < C;
+            const bool has_a = c + 2 * c_step < C;
             list_a = has_a ? list_b + list_step : list_b;
             if (LAST) wt_a = has_a ? wt_b + wt_step : wt_b;
             truth_a = has_a ? truth_b + truth_step : truth_b;
@@ -847,8 +858,14 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
     const int64_t g0 = (int64_t)tile * tg.gpt;
     for (int i = tid; i < tg.gpt * K; i += NT) {
         int64_t g = g0 + i / K;
-        if (g >= a.first_graph && g < (int64_t)a.first_graph + a.n_graphs)
-            a.class_sum[(g - a.first_graph) * K + (i % K)] = sums[i];
+        if (g >= a.first_graph && g < (int64_t)a.first_graph + a.n_graphs) {
+            // workgroups that share a tile add their shares (the host cleared the sums)
+            if (gridDim.y > 1) {
+                if (sums[i] != 0) atomicAdd(&a.class_sum[(g - a.first_graph) * K + (i % K)], sums[i]);
+            } else {
+                a.class_sum[(g - a.first_graph) * K + (i % K)] = sums[i];
+            }
+        }
     }
 }
 
