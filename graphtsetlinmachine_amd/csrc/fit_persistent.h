@@ -59,6 +59,8 @@ struct FitPersistParams {
     int max_words;        // words per graph slot that can hold nodes
     const uint32_t *order;  // literals sorted by how often they hold in the data set, rarest first
     int x_words;          // LDS words of one graph's node-major literal words: max nodes * LA
+    const uint32_t *node_type;  // [total nodes]
+    int direct;           // graphs of at most FITP_DIRECT_NODES nodes: every node is tested on its own literal words, no rows are staged
 };
 
 __device__ __forceinline__ void fitp_stage_rows(const FitPersistParams &p, const FitGraph &fg, uint32_t *dst, int tid) {
@@ -93,6 +95,7 @@ constexpr int FITP_PREFETCH = 5;  // words of the next graph's rows a thread hol
 constexpr int FITP_PREFETCH_X = 3;  // the same for the next graph's node-major literal words
 constexpr int FITP_WALK_ALL = 24;   // clauses with at most this many literals AND all their rows
 constexpr int FITP_FILTER_ROWS = 16;  // rows the others AND before testing the surviving nodes
+constexpr int FITP_DIRECT_NODES = 2;  // data sets whose graphs have at most this many nodes skip the literal rows altogether
 constexpr int FITP_FEW_NODES = 2;     // up to this many surviving nodes are tested one by one, more are filtered further
 
 // Address of element `i` of the staged rows (i = row * words + w) inside the graph's tile.
@@ -134,6 +137,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
     uint32_t *seen = order_lds + p.literals;
     __shared__ int go_on, n_pairs;
     __shared__ uint32_t after_lds[2];
+    __shared__ uint32_t types_lds[2][FITP_DIRECT_NODES];  // node types of this and the next graph (direct evaluation)
 
     // own state -> LDS
     for (int k = tid; k < K; k += FITP_BLOCK) votes[k] = 0;
@@ -152,8 +156,9 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         n_next = (int)p.n_nodes[e1];
         base_next = p.node_index[e1];
         FitGraph fg0 = fit_graph_slot(p.tg, p.first_example, n_now);
-        fitp_stage_rows(p, fg0, rows_buf[0], tid);
+        if (!p.direct) fitp_stage_rows(p, fg0, rows_buf[0], tid);
         for (int at = tid; at < n_now * LA; at += FITP_BLOCK) x_buf[0][at] = p.X[(int64_t)base_now * LA + at];
+        if (p.direct && tid < n_now) types_lds[0][tid] = p.node_type[base_now + tid];
     }
     for (int l = tid; l < p.literals; l += FITP_BLOCK) order_lds[l] = p.order[l];
     for (int j = tid; j < 12 * K; j += FITP_BLOCK) seen[j] = 0u;
@@ -172,7 +177,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         // rows (into registers) and the sizes of the graph after it
         const bool has_next = i + 1 < p.n_examples;
         const FitGraph fn = fit_graph_slot(p.tg, has_next ? ex + 1 : ex, has_next ? n_next : n_now);
-        const int next_total = has_next ? (p.literals + p.n_types + 1) * fn.words : 0;
+        const int next_total = has_next && !p.direct ? (p.literals + p.n_types + 1) * fn.words : 0;
         uint32_t pre[FITP_PREFETCH];
         {
             // element at = row * words + w; a thread's elements are FITP_BLOCK apart: step (row, w) without dividing
@@ -210,6 +215,8 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         const int e2 = min(ex + 2, last);
         uint32_t after = 0u;
         if (tid < 2) after = (tid == 0 ? p.n_nodes : p.node_index)[e2];
+        uint32_t type_ahead = 0u;
+        if (p.direct && has_next && tid < n_next) type_ahead = p.node_type[base_next + tid];
 
         // ---- 1. evaluate own clauses (K1 + K7), votes (K6)
         const bool active = lane < fg.words;
@@ -218,7 +225,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         for (int cl = wave; cl < n_own; cl += WAVES) {
             const int c = c0 + cl;
             const uint32_t *inc = ta + (size_t)cl * LA * B + (B - 1);
-            uint32_t acc = active ? col[(p.literals + c % p.n_types) * stride] : 0u;
+            uint32_t acc = active && !p.direct ? col[(p.literals + c % p.n_types) * stride] : 0u;
             int included = 0;
             uint32_t first_words = 0;
             for (int w0 = 0; w0 < LA; w0 += 64) {
@@ -230,7 +237,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             for (int off = 32; off > 0; off >>= 1) included += __shfl_xor(included, off);
             // A clause with many literals ANDs only the rows of its FITP_FILTER_ROWS rarest ones and then
             // tests the few nodes that are left against its whole include mask on the nodes' own words.
-            const bool filter_only = included > FITP_WALK_ALL && n_now > 0;
+            const bool filter_only = included > FITP_WALK_ALL && n_now > 0 && !p.direct;
             bool all_rows = false;  // every included literal's row has been applied: acc is the clause's truth
             if (filter_only) {
                 int budget = FITP_FILTER_ROWS;
@@ -274,7 +281,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                     for (int u = 0; u < 8; ++u) acc &= r8[u];
                     budget -= 8;
                 }
-            } else {
+            } else if (!p.direct) {
                 for (int w0 = 0; w0 < LA; w0 += 64) {
                     uint32_t mine = w0 == 0 ? first_words : (w0 + lane < LA ? inc[(w0 + lane) * B] : 0u);
                     if (w0 != 0 && w0 + lane == LA - 1) mine &= p.filter;
@@ -301,6 +308,22 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 }
             }
             uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
+            if (p.direct) {
+                // one or two nodes: the clause against each node's own literal words (kernels.py:443-466 as
+                // it stands), lane w on word w; no literal-major rows are read or staged
+                uint32_t bits = 0u;
+                for (int node = 0; node < n_now; ++node) {
+                    bool violated = false;
+                    for (int w0 = 0; w0 < LA; w0 += 64) {
+                        uint32_t mine = w0 == 0 ? first_words : (w0 + lane < LA ? inc[(w0 + lane) * B] : 0u);
+                        if (w0 != 0 && w0 + lane == LA - 1) mine &= p.filter;
+                        const uint32_t xs = w0 + lane < LA ? x_now[node * LA + w0 + lane] : 0xFFFFFFFFu;
+                        violated |= __ballot((mine & ~xs) != 0) != 0;
+                    }
+                    if (!violated && (int)types_lds[i & 1][node] == c % p.n_types) bits |= 1u << node;
+                }
+                v = lane == 0 ? bits : 0u;
+            }
             if (filter_only && !all_rows) {
                 // lane L holds nodes 32 L .. 32 L + 31: the surviving ones are walked on the scalar unit; lane w
                 // compares include word w with the node's literal word w (LDS copy of the graph's X rows)
@@ -381,6 +404,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             }
             for (int at = tid + FITP_PREFETCH_X * FITP_BLOCK; at < next_x_total; at += FITP_BLOCK)
                 dst_x[at] = p.X[(int64_t)base_next * LA + at];
+            if (p.direct && has_next && tid < n_next) types_lds[(i + 1) & 1][tid] = type_ahead;
         }
         for (int j = tid; j < n_own * K; j += FITP_BLOCK) {
             const int cl = j / K, k = j - cl * K;

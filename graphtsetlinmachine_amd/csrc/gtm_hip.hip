@@ -1328,7 +1328,10 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
 
     FitPersistParams p{};
     p.max_words = tg.slot_words > 0 ? tg.slot_words : 1;
-    p.rows_words = (cfg->literals + g->number_of_node_types + 1) * p.max_words;
+    // graphs of one or two nodes: the nodes are tested on their own literal words, no rows are staged
+    p.direct = g->max_number_of_graph_nodes <= FITP_DIRECT_NODES && !getenv("GTM_NO_DIRECT_FIT");
+    p.node_type = g->node_type;
+    p.rows_words = p.direct ? 0 : (cfg->literals + g->number_of_node_types + 1) * p.max_words;
     p.x_words = (g->max_number_of_graph_nodes > 0 ? g->max_number_of_graph_nodes : 1) * d.LA;
     p.order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
     // One clause per wave and step (16 per group) where that fits; fewer per group when the
