@@ -16,6 +16,16 @@
 // needs a single device-wide dependency per graph.
 #pragma once
 
+// Sum over the wave of a small per-lane count (< 64) from ballots of the count's bits: scalar
+// population counts, no cross-lane data movement (a shuffle reduction is six dependent LDS-pipe
+// round trips).
+__device__ __forceinline__ int wave_sum_small(int count) {
+    int t = 0;
+#pragma unroll
+    for (int bit = 0; bit < 6; ++bit) t += __popcll(__ballot((count >> bit) & 1)) << bit;
+    return t;
+}
+
 constexpr int FIT_EVAL_BLOCK = 256;
 constexpr int FIT_WALK_ALL = 40;      // clauses with at most this many literals AND all their rows (rows in global memory)
 constexpr int FIT_WALK_ALL_LDS = 512; // the same with the rows staged in LDS
@@ -163,9 +173,8 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
         for (int w0 = 0; w0 < LA; w0 += 64) {
             const uint32_t mine = include_words(w0);
             if (w0 == 0) first_words = mine;
-            included += __popc(mine);
+            included += wave_sum_small(__popc(mine));
         }
-        for (int off = 32; off > 0; off >>= 1) included += __shfl_xor(included, off);
         // A clause with many literals ANDs the rows of its first FIT_FILTER_ROWS only and then tests the
         // few nodes that are left against its whole include mask on the nodes' own literal words.
         const bool filter_only = included > (STAGE ? FIT_WALK_ALL_LDS : FIT_WALK_ALL) && n_nodes > 0;

@@ -232,9 +232,8 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 uint32_t mine = w0 + lane < LA ? inc[(w0 + lane) * B] : 0u;
                 if (w0 + lane == LA - 1) mine &= p.filter;
                 if (w0 == 0) first_words = mine;
-                included += __popc(mine);
+                included += wave_sum_small(__popc(mine));
             }
-            for (int off = 32; off > 0; off >>= 1) included += __shfl_xor(included, off);
             // A clause with many literals ANDs only the rows of its FITP_FILTER_ROWS rarest ones and then
             // tests the few nodes that are left against its whole include mask on the nodes' own words.
             const bool filter_only = included > FITP_WALK_ALL && n_now > 0 && !p.direct;
