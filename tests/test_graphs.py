@@ -196,3 +196,26 @@ def test_subsetting_matches_direct_construction_and_shares_vocabulary():
     child.prepare_node_configuration()
     child.add_graph_node(0, "n", 0, "brand-new-type")
     assert "brand-new-type" in g.node_type_id  # shared dict, as in the reference
+
+
+def test_print_graph_writes_the_reference_format(capsys):
+    """graphs.py:164-206: one line of nodes with the symbols each holds ('*' for the others), one
+    line per edge with its global slot, a blank line after each node's edges."""
+    from graphtsetlinmachine_amd.graphs import Graphs
+
+    g = Graphs(1, symbols=["A", "B"], hypervector_size=8, hypervector_bits=1, one_hot_encoding=True)
+    g.set_number_of_graph_nodes(0, 2)
+    g.prepare_node_configuration()
+    g.add_graph_node(0, "n0", 1)
+    g.add_graph_node(0, "n1", 1)
+    g.prepare_edge_configuration()
+    g.add_graph_node_edge(0, "n0", "n1", "Plain")
+    g.add_graph_node_edge(0, "n1", "n0", "Other")
+    g.add_graph_node_property(0, "n0", "A")
+    g.add_graph_node_property(0, "n1", "B")
+    g.encode()
+    g.print_graph(0)
+    out = capsys.readouterr().out
+    assert out == ("Printing nodes of Graph#0:\nNode#0( A * ) Node#1( * B ) \n\n"
+                   "Printing edges of Graph#0:\nEdge#0 SrcNode#0 DestNode#1 EdgeType#0\n\n"
+                   "Edge#1 SrcNode#1 DestNode#0 EdgeType#1\n\n\n\n")
