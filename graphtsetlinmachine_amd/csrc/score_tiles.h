@@ -335,15 +335,19 @@ constexpr int TILE_MESSAGES_BLOCK = 256;
 // Transposes the 32 x 32 bit matrix whose row i is the word of lane i (of each half of the wave):
 // afterwards bit i of lane b's word is what bit b of lane i's word was.  Five exchanges of
 // half-blocks with the lane 16, 8, 4, 2, 1 away.
+template <int J, uint32_t M>
+__device__ __forceinline__ uint32_t tile_transpose_step(uint32_t v, int lane) {
+    // M: the columns whose index has bit J clear
+    const uint32_t p = (uint32_t)__shfl_xor((int)v, J);
+    return (lane & J) ? ((p >> J) & M) | (v & ~M) : (v & M) | ((p & M) << J);
+}
+
 __device__ __forceinline__ uint32_t tile_transpose32(uint32_t v, int lane) {
-#pragma unroll
-    for (int j = 16; j >= 1; j >>= 1) {
-        // columns whose index has bit j clear
-        const uint32_t m = j == 16 ? 0x0000FFFFu : j == 8 ? 0x00FF00FFu : j == 4 ? 0x0F0F0F0Fu : j == 2 ? 0x33333333u : 0x55555555u;
-        const uint32_t p = (uint32_t)__shfl_xor((int)v, j);
-        v = (lane & j) ? ((p >> j) & m) | (v & ~m) : (v & m) | ((p & m) << j);
-    }
-    return v;
+    v = tile_transpose_step<16, 0x0000FFFFu>(v, lane);
+    v = tile_transpose_step<8, 0x00FF00FFu>(v, lane);
+    v = tile_transpose_step<4, 0x0F0F0F0Fu>(v, lane);
+    v = tile_transpose_step<2, 0x33333333u>(v, lane);
+    return tile_transpose_step<1, 0x55555555u>(v, lane);
 }
 
 
