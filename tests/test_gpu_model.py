@@ -202,3 +202,38 @@ def test_transform_and_read_outs_match_the_oracle():
                 bits = [(int(b) + edge_type) % 40 for b in tm.hypervectors[sender]]
                 assert messages[edge_type, c, sender] == sum(int(included[c, b]) for b in bits)
                 assert messages[edge_type, c, 40 + sender] == sum(int(included[c, 40 + b]) for b in bits)
+
+
+def test_multi_output_and_single_output_heads_follow_the_oracle():
+    """tm.py:961-1072: several independent outputs (Y in {0, 1} per output, prediction sum >= 0) and
+    the single-output machine (one 'class', score is a vector): states, sums and predictions."""
+    from graphtsetlinmachine_amd.tm import GraphTsetlinMachine, MultiOutputGraphTsetlinMachine
+
+    wl = workloads.noisy_xor(1200, 300)
+    x_train = wl.Y_train.astype(np.int64)
+    Y3 = np.stack([x_train, 1 - x_train, np.ones_like(x_train)], axis=1)
+    params = dict(wl.params)
+    tm = MultiOutputGraphTsetlinMachine(**params, seed=5)
+    tm.fit(wl.graphs_train, Y3, epochs=0, incremental=True)
+    model = oracle_twin(tm, wl.graphs_train)
+    assert model.cfg.classes == 3
+    tm.fit(wl.graphs_train, Y3, epochs=2, incremental=True)
+    o.fit(model, wl.graphs_train, np.where(Y3 == 1, tm.T, -tm.T).astype(np.int32), epochs=2)
+    assert_same_state(tm, model)
+    sums = tm.score(wl.graphs_test)
+    assert np.array_equal(sums, o.score(model, wl.graphs_test))
+    pred = tm.predict(wl.graphs_test)
+    assert pred.dtype == np.uint32 and np.array_equal(pred, (sums >= 0).astype(np.uint32))
+    assert (pred[:, 0] == wl.Y_test).mean() == 1.0 and (pred[:, 1] == 1 - wl.Y_test).mean() == 1.0 and pred[:, 2].all()
+
+    one = GraphTsetlinMachine(**params, seed=6)
+    one.fit(wl.graphs_train, wl.Y_train, epochs=0, incremental=True)
+    model = oracle_twin(one, wl.graphs_train)
+    assert model.cfg.classes == 1
+    one.fit(wl.graphs_train, wl.Y_train, epochs=2, incremental=True)
+    o.fit(model, wl.graphs_train, np.where(wl.Y_train == 1, one.T, -one.T).astype(np.int32).reshape(-1, 1), epochs=2)
+    assert_same_state(one, model)
+    score = one.score(wl.graphs_test)
+    assert score.shape == (300,) and np.array_equal(score, o.score(model, wl.graphs_test)[:, 0])
+    assert np.array_equal(one.predict(wl.graphs_test), score >= 0)
+    assert (one.predict(wl.graphs_test) == (wl.Y_test == 1)).mean() == 1.0
