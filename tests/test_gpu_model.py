@@ -237,3 +237,71 @@ def test_multi_output_and_single_output_heads_follow_the_oracle():
     assert score.shape == (300,) and np.array_equal(score, o.score(model, wl.graphs_test)[:, 0])
     assert np.array_equal(one.predict(wl.graphs_test), score >= 0)
     assert (one.predict(wl.graphs_test) == (wl.Y_test == 1)).mean() == 1.0
+
+
+def test_the_call_sequence_of_the_noisy_xor_demo_runs_unchanged():
+    """A user's script written against the reference (the calls and attributes of
+    examples/NoisyXORDemo.py: per-call graph building, `init_with`, grid/block arguments, one
+    epoch per fit call, the clause read-out loop at the end) works with the import swapped."""
+    from graphtsetlinmachine_amd.graphs import Graphs
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    rng = np.random.default_rng(3)
+    np.random.seed(3)
+
+    def build(n, init_with=None, noise=0.0):
+        if init_with is None:
+            graphs = Graphs(n, symbols=["A", "B"], hypervector_size=32, hypervector_bits=2)
+        else:
+            graphs = Graphs(n, init_with=init_with)
+        for graph_id in range(n):
+            graphs.set_number_of_graph_nodes(graph_id, 2)
+        graphs.prepare_node_configuration()
+        for graph_id in range(n):
+            graphs.add_graph_node(graph_id, "Node 1", 1)
+            graphs.add_graph_node(graph_id, "Node 2", 1)
+        graphs.prepare_edge_configuration()
+        Y = np.empty(n, dtype=np.uint32)
+        for graph_id in range(n):
+            graphs.add_graph_node_edge(graph_id, "Node 1", "Node 2", "Plain")
+            graphs.add_graph_node_edge(graph_id, "Node 2", "Node 1", "Plain")
+            x1, x2 = rng.integers(0, 2, size=2)
+            graphs.add_graph_node_property(graph_id, "Node 1", "A" if x1 else "B")
+            graphs.add_graph_node_property(graph_id, "Node 2", "A" if x2 else "B")
+            Y[graph_id] = x1 ^ x2
+            if rng.random() <= noise:
+                Y[graph_id] = 1 - Y[graph_id]
+        graphs.encode()
+        return graphs, Y
+
+    graphs_train, Y_train = build(2000, noise=0.01)
+    graphs_test, Y_test = build(500, init_with=graphs_train)
+    assert graphs_test.hypervectors is graphs_train.hypervectors or np.array_equal(graphs_test.hypervectors,
+                                                                                  graphs_train.hypervectors)
+    assert graphs_train.signature != graphs_test.signature and len(graphs_train) == 2000
+
+    # (the demo's default limit of 4 included literals makes learning depend on the seed, in the CPU
+    # oracle as well: the limit is left at its constructor default here)
+    tm = MultiClassGraphTsetlinMachine(10, 100, 1.0, depth=2, message_size=256, message_bits=2,
+                                       max_included_literals=None, grid=(16 * 13, 1, 1), block=(128, 1, 1))
+    for _ in range(3):
+        tm.fit(graphs_train, Y_train, epochs=1, incremental=True)
+        result_test = 100 * (tm.predict(graphs_test) == Y_test).mean()
+        result_train = 100 * (tm.predict(graphs_train) == Y_train).mean()
+    assert result_test == 100.0 and result_train >= 97.0
+
+    weights = tm.get_state()[1].reshape(2, -1)
+    assert weights.shape == (2, tm.number_of_clauses)
+    described = []
+    for i in range(tm.number_of_clauses):
+        literals = []
+        for k in range(graphs_train.hypervector_size * 2):
+            if tm.ta_action(0, i, k):
+                literals.append(("x%d" if k < graphs_train.hypervector_size else "NOT x%d")
+                                % (k % graphs_train.hypervector_size))
+        for k in range(tm.message_size * 2):
+            if tm.ta_action(1, i, k):
+                literals.append(("c%d" if k < tm.message_size else "NOT c%d") % (k % tm.message_size))
+        described.append(" AND ".join(literals))
+    assert any(described) and tm.hypervectors.shape == (10, 2)
+    assert graphs_train.edge_type_id == {"Plain": 0} and set(graphs_train.symbol_id) == {"A", "B"}
