@@ -51,7 +51,7 @@ struct FitPersistParams {
     uint32_t filter, thr16, k0, k1;
     uint64_t q_thr;
     // coordination
-    unsigned long long *class_sum;  // [3][K] words FITP_SUM_STRIDE apart, zero on entry (K <= FITP_BLOCK)
+    unsigned long long *class_sum;  // [3][K][FITP_SUM_PARTS] words FITP_SUM_STRIDE apart, zero on entry (K <= FITP_BLOCK)
     uint32_t *abort_flag;           // [1], zero on entry
     uint32_t spin_limit;
     int clauses_per_group;
@@ -91,8 +91,10 @@ __device__ __forceinline__ void fitp_stage_rows(const FitPersistParams &p, const
 constexpr unsigned long long FITP_HALF = 1ull << 47;      // class sums are smaller than this in magnitude
 constexpr unsigned long long FITP_ARRIVED = 1ull << 48;   // one arrival in bits 48..63
 constexpr int FITP_SUM_STRIDE = 16;                      // 64-bit words between two class-sum words (one per 128-byte line)
-constexpr int FITP_PREFETCH = 5;  // words of the next graph's rows a thread holds in registers while evaluating
-constexpr int FITP_PREFETCH_X = 3;  // the same for the next graph's node-major literal words
+// A class sum is kept as this many partial words; group g adds to part g % FITP_SUM_PARTS and the
+// reader adds the parts up (the protocol is linear in the word). Adds to one word are carried out
+// one after the other by the memory system, so fewer groups per word shorten the exchange.
+constexpr int FITP_SUM_PARTS = 16;
 constexpr int FITP_WALK_ALL = 24;   // clauses with at most this many literals AND all their rows
 constexpr int FITP_FILTER_ROWS = 16;  // rows the others AND before testing the surviving nodes
 constexpr int FITP_DIRECT_NODES = 2;  // data sets whose graphs have at most this many nodes skip the literal rows altogether
@@ -103,6 +105,15 @@ __device__ __forceinline__ const uint32_t *fitp_row_word(const FitPersistParams 
     const int r = i / fg.words, w = i - r * fg.words;
     return p.tiles + ((int64_t)fg.tile * p.tg.rows + r) * p.tg.tw + fg.word0 + w;
 }
+
+// One 32-bit word per lane from global memory straight into LDS (no register holds it meanwhile):
+// lane l's word lands at dst_of_wave[l]; dst_of_wave must be the same for the whole wave. The words
+// are there once the wave has waited for its vector-memory counter (FITP_WAIT_VMEM) and, for other
+// waves, after the barrier that follows.
+__device__ __forceinline__ void fitp_load_to_lds(const uint32_t *src, uint32_t *dst_of_wave) {
+    __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) uint32_t *)dst_of_wave, 4, 0, 0);
+}
+constexpr int FITP_WAIT_VMEM = 0x0F70;  // s_waitcnt vmcnt(0) (export and LDS counters left alone)
 
 // MAXB: bit planes of an automaton the kernel keeps in registers while updating a word (>= B).
 template <int MAXB>
@@ -171,14 +182,13 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         const uint32_t step = p.first_step + (uint32_t)i;
         const FitGraph fg = fit_graph_slot(p.tg, ex, n_now);
         const uint32_t *rows = rows_buf[i & 1];
-        unsigned long long *slot_now = p.class_sum + (size_t)(i % 3) * K * FITP_SUM_STRIDE;
+        unsigned long long *slot_now = p.class_sum + (size_t)(i % 3) * K * FITP_SUM_PARTS * FITP_SUM_STRIDE;
 
         // ---- 0. requests that can be in flight while this example is evaluated: the next graph's
-        // rows (into registers) and the sizes of the graph after it
+        // rows and literal words (straight into the other LDS buffers) and the sizes of the graph after it
         const bool has_next = i + 1 < p.n_examples;
         const FitGraph fn = fit_graph_slot(p.tg, has_next ? ex + 1 : ex, has_next ? n_next : n_now);
         const int next_total = has_next && !p.direct ? (p.literals + p.n_types + 1) * fn.words : 0;
-        uint32_t pre[FITP_PREFETCH];
         {
             // element at = row * words + w; a thread's elements are FITP_BLOCK apart: step (row, w) without dividing
             const uint32_t *tile = p.tiles + (int64_t)fn.tile * p.tg.rows * p.tg.tw + fn.word0;
@@ -189,9 +199,9 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             }
             const int dr = div_dr, dw = FITP_BLOCK - dr * fn.words;
             int r = div_r0, w = tid - r * fn.words;
-#pragma unroll
-            for (int u = 0; u < FITP_PREFETCH; ++u) {
-                pre[u] = tid + u * FITP_BLOCK < next_total ? tile[(int64_t)r * p.tg.tw + w] : 0u;
+            uint32_t *dst = rows_buf[(i + 1) & 1] + wave * 64;
+            for (int at0 = 0; at0 < next_total; at0 += FITP_BLOCK) {
+                if (at0 + tid < next_total) fitp_load_to_lds(tile + (int64_t)r * p.tg.tw + w, dst + at0);
                 r += dr;
                 w += dw;
                 if (w >= fn.words) {
@@ -200,13 +210,12 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 }
             }
         }
-        uint32_t pre_x[FITP_PREFETCH_X];
         const int next_x_total = has_next ? n_next * LA : 0;
         {
-            const uint32_t *src = p.X + (int64_t)base_next * LA;
-#pragma unroll
-            for (int u = 0; u < FITP_PREFETCH_X; ++u)
-                pre_x[u] = tid + u * FITP_BLOCK < next_x_total ? src[tid + u * FITP_BLOCK] : 0u;
+            const uint32_t *src = p.X + (int64_t)base_next * LA + tid;
+            uint32_t *dst = x_buf[(i + 1) & 1] + wave * 64;
+            for (int at0 = 0; at0 < next_x_total; at0 += FITP_BLOCK)
+                if (at0 + tid < next_x_total) fitp_load_to_lds(src + at0, dst + at0);
         }
         const uint32_t *x_now = x_buf[i & 1];
         // node count and first node of the graph after the next, fetched by two threads with vector
@@ -377,45 +386,56 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         }
 
         // ---- 2. class sums across the device (see the header comment)
+        if (tid == 0) go_on = 1;
         __syncthreads();  // the group's votes are complete
         for (int k = tid; k < K; k += FITP_BLOCK) {
-            __hip_atomic_fetch_add(&slot_now[k * FITP_SUM_STRIDE], FITP_ARRIVED + (unsigned long long)(long long)votes[k], __ATOMIC_RELAXED,
+            __hip_atomic_fetch_add(&slot_now[(k * FITP_SUM_PARTS + (int)(blockIdx.x % FITP_SUM_PARTS)) * FITP_SUM_STRIDE], FITP_ARRIVED + (unsigned long long)(long long)votes[k], __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
             votes[k] = 0;
         }
-        // Work that does not need the class sums is done while the other groups arrive: the next
-        // graph's rows go to LDS, the random numbers of the feedback gates, the literals of the
-        // picked nodes.
-        {
-            uint32_t *dst = rows_buf[(i + 1) & 1];
-#pragma unroll
-            for (int u = 0; u < FITP_PREFETCH; ++u) {
-                const int at = tid + u * FITP_BLOCK;
-                if (at < next_total) dst[at] = pre[u];
+        // Work that does not need the class sums is done while the other groups arrive
+        if (p.direct && has_next && tid < n_next) types_lds[(i + 1) & 1][tid] = type_ahead;
+        // With few (clause, class, word) triples the waves that do not poll draw the Type I feedback
+        // bits of all of them while the class sums are on their way; otherwise the bits are drawn
+        // afterwards, for the pairs that turn out to need them.
+        const int pollers = (K + 63) & ~63, helpers = FITP_BLOCK - pollers;
+        const bool ahead = helpers >= FITP_BLOCK / 2 && n_own * K * LA <= 2 * helpers;
+        if (ahead) {
+            if (tid >= pollers) {
+                for (int j = tid - pollers; j < n_own * K; j += helpers) {
+                    const int cl = j / K, k = j - cl * K;
+                    philox_out r = philox4x32_10((uint32_t)(c0 + cl), (uint32_t)k, step, GTM_TAG_CLAUSE_UPDATES, p.k0, p.k1);
+                    gate[2 * j] = r.v[0];
+                    gate[2 * j + 1] = r.v[1];
+                }
+                for (int t = tid - pollers; t < n_own * K * LA; t += helpers) {
+                    const int j = t / LA, w = t - j * LA;
+                    const int cl = j / K, k = j - cl * K;
+                    fbits[((size_t)cl * LA + w) * K + k] =
+                        gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
+                }
             }
-            for (int at = tid + FITP_PREFETCH * FITP_BLOCK; at < next_total; at += FITP_BLOCK)
-                dst[at] = *fitp_row_word(p, fn, at);
-            uint32_t *dst_x = x_buf[(i + 1) & 1];
-#pragma unroll
-            for (int u = 0; u < FITP_PREFETCH_X; ++u) {
-                const int at = tid + u * FITP_BLOCK;
-                if (at < next_x_total) dst_x[at] = pre_x[u];
+        } else {
+            for (int j = tid; j < n_own * K; j += FITP_BLOCK) {
+                const int cl = j / K, k = j - cl * K;
+                philox_out r = philox4x32_10((uint32_t)(c0 + cl), (uint32_t)k, step, GTM_TAG_CLAUSE_UPDATES, p.k0, p.k1);
+                gate[2 * j] = r.v[0];
+                gate[2 * j + 1] = r.v[1];
             }
-            for (int at = tid + FITP_PREFETCH_X * FITP_BLOCK; at < next_x_total; at += FITP_BLOCK)
-                dst_x[at] = p.X[(int64_t)base_next * LA + at];
-            if (p.direct && has_next && tid < n_next) types_lds[(i + 1) & 1][tid] = type_ahead;
+            __syncthreads();
         }
-        for (int j = tid; j < n_own * K; j += FITP_BLOCK) {
-            const int cl = j / K, k = j - cl * K;
-            philox_out r = philox4x32_10((uint32_t)(c0 + cl), (uint32_t)k, step, GTM_TAG_CLAUSE_UPDATES, p.k0, p.k1);
-            gate[2 * j] = r.v[0];
-            gate[2 * j + 1] = r.v[1];
-        }
-        if (tid == 0) go_on = 1;
-        __syncthreads();
         if (tid < K) {
             const int k = tid;
             const unsigned long long everyone = (unsigned long long)gridDim.x;
+            auto read_sum = [](const unsigned long long *slot, int k) {
+                unsigned long long part[FITP_SUM_PARTS], all = 0ull;
+#pragma unroll
+                for (int s = 0; s < FITP_SUM_PARTS; ++s)
+                    part[s] = __hip_atomic_load(&slot[(k * FITP_SUM_PARTS + s) * FITP_SUM_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                for (int s = 0; s < FITP_SUM_PARTS; ++s) all += part[s];
+                return all;
+            };
             auto arrivals = [](unsigned long long now, unsigned long long before) {
                 return ((now - before + FITP_HALF) >> 48) & 0xFFFFull;
             };
@@ -427,7 +447,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             bool ok = true, mine = false;
             for (;;) {
                 if (!mine) {
-                    first = __hip_atomic_load(&slot_now[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    first = read_sum(slot_now, 0);
                     if (arrivals(first, seen_first) == everyone) {
                         mine = true;
                         if (k == 0) {
@@ -437,7 +457,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                         continue;
                     }
                 } else {
-                    word = __hip_atomic_load(&slot_now[k * FITP_SUM_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    word = read_sum(slot_now, k);
                     if (arrivals(word, seen_own) == everyone) break;
                 }
                 if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
@@ -486,7 +506,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         // Type I feedback bits for the (clause, class) pairs that need them: the pairs are listed
         // first (wave 0, ballots), then one thread per (listed pair, word) draws the bits, so that
         // the lanes that run the generator are (nearly) all busy
-        if (wave == 0) {
+        if (!ahead && wave == 0) {
             int n_listed = 0;
             for (int j0 = 0; j0 < n_own * K; j0 += 64) {
                 const int j = j0 + lane;
@@ -497,14 +517,16 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             }
             if (lane == 0) n_pairs = n_listed;
         }
-        __syncthreads();
-        for (int t = tid; t < n_pairs * LA; t += FITP_BLOCK) {
-            const int j = pair_list[t / LA], w = t % LA;
-            const int cl = j / K, k = j - cl * K;
-            fbits[((size_t)cl * LA + w) * K + k] =
-                gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
+        if (!ahead) {
+            __syncthreads();
+            for (int t = tid; t < n_pairs * LA; t += FITP_BLOCK) {
+                const int j = pair_list[t / LA], w = t % LA;
+                const int cl = j / K, k = j - cl * K;
+                fbits[((size_t)cl * LA + w) * K + k] =
+                    gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
+            }
+            __syncthreads();
         }
-        __syncthreads();
         const uint32_t *X_rows = x_now;  // the graph's literal words, node-major, in LDS
         for (int j = tid; j < n_own * LA; j += FITP_BLOCK) {
             const int cl = j / LA, w = j - cl * LA;
@@ -519,6 +541,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             feedback_word<MAXB>(ta + (size_t)j * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1,
                               (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, p.thr16, fbits + (size_t)j * K);
         }
+        __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);  // the next graph's words are in LDS
         if (tid < 2) after_lds[tid] = after;
         __syncthreads();
         n_now = n_next;
@@ -526,6 +549,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         n_next = (int)after_lds[0];
         base_next = after_lds[1];
     }
+    __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);  // no load into LDS is left in flight when the group ends
     // own state -> global memory (also after an abort: every clause is left as of some whole step)
     for (int i = tid; i < n_own * LA * B; i += FITP_BLOCK) p.bank[(int64_t)c0 * LA * B + i] = ta[i];
     for (int i = tid; i < n_own * K; i += FITP_BLOCK) {

@@ -577,7 +577,7 @@ FitWs carve_fit(const Dims &d, const gtm_config *cfg, char *base) {
     for (int l = 0; l < GTM_MAX_DEPTH - 1; ++l)
         w.clause_X[l] = l < cfg->depth - 1 ? (uint32_t *)take((size_t)cfg->max_nodes * d.MC * 4) : nullptr;
     // the fused paths rotate class-sum buffers: 2 x int32 [K], or 3 x 64-bit [K] followed by an abort flag
-    w.class_sum = (int32_t *)take(((size_t)d.K * 3 * FITP_SUM_STRIDE + 1) * 8);  // the persistent kernel's ring is the largest user
+    w.class_sum = (int32_t *)take(((size_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE + 1) * 8);  // the persistent kernel's ring is the largest user
     w.clause_node = (int32_t *)take((size_t)d.C * 4);
     w.n_incl = (int32_t *)take((size_t)d.C * 4);
     w.update = (int32_t *)take((size_t)d.K * d.C * 4);
@@ -1399,12 +1399,12 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     p.k1 = key.k1;
     p.q_thr = q_threshold(cfg->q, cfg->classes);
     p.class_sum = (unsigned long long *)w.class_sum;
-    p.abort_flag = (uint32_t *)((unsigned long long *)w.class_sum + (size_t)d.K * 3 * FITP_SUM_STRIDE);
+    p.abort_flag = (uint32_t *)((unsigned long long *)w.class_sum + (size_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE);
     p.spin_limit = 4000000u;  // a few seconds of polling at the very most
     if (const char *e = getenv("GTM_FIT_SPIN_LIMIT")) p.spin_limit = (uint32_t)strtoul(e, nullptr, 10);  // tests force the give-up path
 
-    hipLaunchKernelGGL(k_fill_u64, dim3(blocks_for((int64_t)d.K * 3 * FITP_SUM_STRIDE + 1, TPB)), dim3(TPB), 0, st,
-                       (unsigned long long *)w.class_sum, (int64_t)0, 0ull, (int64_t)d.K * 3 * FITP_SUM_STRIDE + 1);
+    hipLaunchKernelGGL(k_fill_u64, dim3(blocks_for((int64_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE + 1, TPB)), dim3(TPB), 0, st,
+                       (unsigned long long *)w.class_sum, (int64_t)0, 0ull, (int64_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE + 1);
     if (int rc = check_launch("fill")) return rc;
     void *args[] = {&p};
     profile_start("k_fit_persistent", st);
