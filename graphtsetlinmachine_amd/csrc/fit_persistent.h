@@ -146,6 +146,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
     // thread k < K: its class-sum word and the word of class 0 as they stood when each of the three
     // slots was last complete (all zero before the first use): [slot][own, first][low, high][K]
     uint32_t *seen = order_lds + p.literals;
+    uint32_t *y_buf[2] = {seen + 12 * K, seen + 13 * K};        // [K] labels of this and the next example
     __shared__ int go_on, n_pairs;
     __shared__ uint32_t after_lds[2];
     __shared__ uint32_t types_lds[2][FITP_DIRECT_NODES];  // node types of this and the next graph (direct evaluation)
@@ -170,10 +171,11 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         if (!p.direct) fitp_stage_rows(p, fg0, rows_buf[0], tid);
         for (int at = tid; at < n_now * LA; at += FITP_BLOCK) x_buf[0][at] = p.X[(int64_t)base_now * LA + at];
         if (p.direct && tid < n_now) types_lds[0][tid] = p.node_type[base_now + tid];
+        for (int k = tid; k < K; k += FITP_BLOCK) y_buf[0][k] = (uint32_t)p.encoded_Y[(int64_t)p.first_example * K + k];
     }
     for (int l = tid; l < p.literals; l += FITP_BLOCK) order_lds[l] = p.order[l];
     for (int j = tid; j < 12 * K; j += FITP_BLOCK) seen[j] = 0u;
-    __syncthreads();
+    lds_barrier();
 
     const int ones_row = p.literals + p.n_types;
     int div_words = 0, div_dr = 0, div_r0 = 0;
@@ -216,6 +218,12 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             uint32_t *dst = x_buf[(i + 1) & 1] + wave * 64;
             for (int at0 = 0; at0 < next_x_total; at0 += FITP_BLOCK)
                 if (at0 + tid < next_x_total) fitp_load_to_lds(src + at0, dst + at0);
+        }
+        if (has_next) {
+            const uint32_t *src = (const uint32_t *)p.encoded_Y + (int64_t)(ex + 1) * K + tid;
+            uint32_t *dst = y_buf[(i + 1) & 1] + wave * 64;
+            for (int at0 = 0; at0 < K; at0 += FITP_BLOCK)
+                if (at0 + tid < K) fitp_load_to_lds(src + at0, dst + at0);
         }
         const uint32_t *x_now = x_buf[i & 1];
         // node count and first node of the graph after the next, fetched by two threads with vector
@@ -387,7 +395,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
 
         // ---- 2. class sums across the device (see the header comment)
         if (tid == 0) go_on = 1;
-        __syncthreads();  // the group's votes are complete
+        lds_barrier();  // the group's votes are complete
         for (int k = tid; k < K; k += FITP_BLOCK) {
             __hip_atomic_fetch_add(&slot_now[(k * FITP_SUM_PARTS + (int)(blockIdx.x % FITP_SUM_PARTS)) * FITP_SUM_STRIDE], FITP_ARRIVED + (unsigned long long)(long long)votes[k], __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
@@ -395,26 +403,19 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         }
         // Work that does not need the class sums is done while the other groups arrive
         if (p.direct && has_next && tid < n_next) types_lds[(i + 1) & 1][tid] = type_ahead;
-        // With few (clause, class, word) triples the waves that do not poll draw the Type I feedback
-        // bits of all of them while the class sums are on their way; otherwise the bits are drawn
-        // afterwards, for the pairs that turn out to need them.
+        // The random words of the feedback gates are drawn by the waves that do not poll, while the
+        // class sums are on their way. (Drawing the Type I feedback bits of every (clause, class,
+        // word) here as well costs more generator work than the exchange hides: they are drawn
+        // afterwards, for the pairs that turn out to need them.)
         const int pollers = (K + 63) & ~63, helpers = FITP_BLOCK - pollers;
-        const bool ahead = helpers >= FITP_BLOCK / 2 && n_own * K * LA <= 2 * helpers;
-        if (ahead) {
-            if (tid >= pollers) {
+        if (helpers >= FITP_BLOCK / 2) {
+            if (tid >= pollers)
                 for (int j = tid - pollers; j < n_own * K; j += helpers) {
                     const int cl = j / K, k = j - cl * K;
                     philox_out r = philox4x32_10((uint32_t)(c0 + cl), (uint32_t)k, step, GTM_TAG_CLAUSE_UPDATES, p.k0, p.k1);
                     gate[2 * j] = r.v[0];
                     gate[2 * j + 1] = r.v[1];
                 }
-                for (int t = tid - pollers; t < n_own * K * LA; t += helpers) {
-                    const int j = t / LA, w = t - j * LA;
-                    const int cl = j / K, k = j - cl * K;
-                    fbits[((size_t)cl * LA + w) * K + k] =
-                        gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
-                }
-            }
         } else {
             for (int j = tid; j < n_own * K; j += FITP_BLOCK) {
                 const int cl = j / K, k = j - cl * K;
@@ -422,7 +423,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 gate[2 * j] = r.v[0];
                 gate[2 * j + 1] = r.v[1];
             }
-            __syncthreads();
+            lds_barrier();
         }
         if (tid < K) {
             const int k = tid;
@@ -474,11 +475,11 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             seen_slot[k] = (uint32_t)word, seen_slot[K + k] = (uint32_t)(word >> 32);
             seen_slot[2 * K + k] = (uint32_t)first, seen_slot[3 * K + k] = (uint32_t)(first >> 32);
         }
-        __syncthreads();
+        lds_barrier();
         if (!go_on) break;  // uniform over the group; every group leaves at its next check
 
         // ---- 3. feedback (K8) and automaton updates (K9) on the LDS copies
-        const int32_t *y = p.encoded_Y + (int64_t)ex * K;
+        const int32_t *y = (const int32_t *)y_buf[i & 1];
         for (int j = tid; j < n_own * K; j += FITP_BLOCK) {
             const int cl = j / K, k = j - cl * K;
             int cs = sums[k];
@@ -502,11 +503,11 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             }
             upd[j] = u;
         }
-        __syncthreads();
+        lds_barrier();
         // Type I feedback bits for the (clause, class) pairs that need them: the pairs are listed
         // first (wave 0, ballots), then one thread per (listed pair, word) draws the bits, so that
         // the lanes that run the generator are (nearly) all busy
-        if (!ahead && wave == 0) {
+        if (wave == 0) {
             int n_listed = 0;
             for (int j0 = 0; j0 < n_own * K; j0 += 64) {
                 const int j = j0 + lane;
@@ -517,16 +518,14 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             }
             if (lane == 0) n_pairs = n_listed;
         }
-        if (!ahead) {
-            __syncthreads();
-            for (int t = tid; t < n_pairs * LA; t += FITP_BLOCK) {
-                const int j = pair_list[t / LA], w = t % LA;
-                const int cl = j / K, k = j - cl * K;
-                fbits[((size_t)cl * LA + w) * K + k] =
-                    gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
-            }
-            __syncthreads();
+        lds_barrier();
+        for (int t = tid; t < n_pairs * LA; t += FITP_BLOCK) {
+            const int j = pair_list[t / LA], w = t % LA;
+            const int cl = j / K, k = j - cl * K;
+            fbits[((size_t)cl * LA + w) * K + k] =
+                gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
         }
+        lds_barrier();
         const uint32_t *X_rows = x_now;  // the graph's literal words, node-major, in LDS
         for (int j = tid; j < n_own * LA; j += FITP_BLOCK) {
             const int cl = j / LA, w = j - cl * LA;
@@ -543,7 +542,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         }
         __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);  // the next graph's words are in LDS
         if (tid < 2) after_lds[tid] = after;
-        __syncthreads();
+        lds_barrier();
         n_now = n_next;
         base_now = base_next;
         n_next = (int)after_lds[0];

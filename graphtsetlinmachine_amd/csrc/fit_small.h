@@ -28,8 +28,9 @@
 // node types, edge counts and offsets, labels) and of the node count and offset
 // of example i + 2 are in flight into registers; they land in the other half of
 // double-buffered LDS arrays before the step's last barrier.  The edges of
-// example i are fetched at the top of its step and parked in LDS before the
-// first message layer needs them.  LDS loads inside a phase are issued in
+// example i are fetched at the top of its step and parked in LDS right before
+// the first message layer walks them.  The barriers order LDS traffic only, so
+// none of them waits for these loads.  LDS loads inside a phase are issued in
 // batches (no early exit inside a batch), since one thread's chain of dependent
 // LDS round trips is what a phase costs.
 #pragma once
@@ -150,7 +151,7 @@ __global__ __launch_bounds__(FITS_BLOCK) void k_fit_small(FitSmallParams p) {
         if (tid < 2 && p.n_examples > 1)
             labels[FITS_Y_LDS + tid] = (tid == 0 ? p.n_nodes : p.node_index)[p.first_example + 1];
     }
-    __syncthreads();
+    lds_barrier();
 
     for (int i = 0; i < p.n_examples; ++i) {
         const int ex = p.first_example + i;
@@ -227,11 +228,7 @@ __global__ __launch_bounds__(FITS_BLOCK) void k_fit_small(FitSmallParams p) {
                 draw_update[2 * ck + 1] = r.v[1];
             }
         }
-        if (edges_parked && tid < graph_edges) {
-            edges_lds[2 * tid] = edge_ahead.x;
-            edges_lds[2 * tid + 1] = edge_ahead.y;
-        }
-        __syncthreads();
+        lds_barrier();
 
         // ---- message layers; sent is all zero at the start of each
         for (int l = 0; l < layers; ++l) {
@@ -246,7 +243,12 @@ __global__ __launch_bounds__(FITS_BLOCK) void k_fit_small(FitSmallParams p) {
                         atomicOr(&sent[n * MW + (h >> 5)], 1u << (h & 31));
                     }
             }
-            __syncthreads();
+            // the edges requested at the top of the step are parked here, as late as their first use allows
+            if (l == 0 && edges_parked && tid < graph_edges) {
+                edges_lds[2 * tid] = edge_ahead.x;
+                edges_lds[2 * tid + 1] = edge_ahead.y;
+            }
+            lds_barrier();
             // along every edge: the vector rotated by the edge type (bit p of the result is bit (p - type) mod M)
             if (graph_edges > 0)
                 for (int j = tid; j < n_nodes * MW; j += FITS_BLOCK) {
@@ -270,7 +272,7 @@ __global__ __launch_bounds__(FITS_BLOCK) void k_fit_small(FitSmallParams p) {
                         if (word) atomicOr(&got[dst * MW + jw], word);
                     }
                 }
-            __syncthreads();
+            lds_barrier();
             // K2, one thread per (clause, node): include words 0 .. MW - 1 against the received
             // vector, MW .. 2 MW - 1 against its complement
             for (int j = tid; j < FITS_MAX_NODES * MW; j += FITS_BLOCK) sent[j] = 0u;
@@ -289,7 +291,7 @@ __global__ __launch_bounds__(FITS_BLOCK) void k_fit_small(FitSmallParams p) {
                         atomicOr(&nxt[2 * c + (n >> 5)], 1u << (n & 31));
                 }
             }
-            __syncthreads();
+            lds_barrier();
             uint32_t *swap = cur;
             cur = nxt;
             nxt = swap;
@@ -316,7 +318,7 @@ __global__ __launch_bounds__(FITS_BLOCK) void k_fit_small(FitSmallParams p) {
             if (fired)
                 for (int k = 0; k < K; ++k) atomicAdd(&sums[k], wts[k * C + c]);
         }
-        __syncthreads();
+        lds_barrier();
 
         // ---- K8: feedback decision and weight update, one thread per (clause, class)
         const int32_t *y_global = p.encoded_Y + (int64_t)ex * K;
@@ -345,7 +347,7 @@ __global__ __launch_bounds__(FITS_BLOCK) void k_fit_small(FitSmallParams p) {
             }
             upd[j] = u;
         }
-        __syncthreads();
+        lds_barrier();
 
         // ---- K9, K10: one thread per (clause, automaton word of any bank)
         const int per_clause = LA + layers * MC;
@@ -390,7 +392,7 @@ __global__ __launch_bounds__(FITS_BLOCK) void k_fit_small(FitSmallParams p) {
         field_next[tid] = field_ahead;
         if (tid < 2) field_next[3 * FITS_MAX_NODES + FITS_Y_LDS + tid] = header_ahead;
         n_nodes = n_next;
-        __syncthreads();
+        lds_barrier();
     }
 
     // state -> global memory

@@ -1334,17 +1334,23 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     p.rows_words = p.direct ? 0 : (cfg->literals + g->number_of_node_types + 1) * p.max_words;
     p.x_words = (g->max_number_of_graph_nodes > 0 ? g->max_number_of_graph_nodes : 1) * d.LA;
     p.order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
-    // One clause per wave and step (16 per group) where that fits; fewer per group when the
-    // automata of 16 clauses do not fit in LDS and the chip has room for more groups.
-    const int waves = FITP_BLOCK / 64;
+    // One clause per wave and step. Few clauses per group keep a step's feedback short, few groups
+    // keep the exchange of the class sums short: the clauses are spread over all CUs (8 to 12 per
+    // group measured best on 2,000 and 2,500 clauses), but a group gets at least 8 where their
+    // automata fit in LDS.
     auto lds_bytes = [&](int per_group) {
         return (2 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group +
                 2 * (size_t)d.K + 5 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K + 2 * (size_t)p.x_words +
-                (size_t)cfg->literals + 12 * (size_t)d.K) * 4;
+                (size_t)cfg->literals + 14 * (size_t)d.K) * 4;
     };
     const size_t lds_limit = 150 * 1024;
     int per_group = (d.C + cus - 1) / cus;
-    if (per_group < waves && lds_bytes(waves) <= lds_limit) per_group = waves;
+    const int preferred = 8;
+    if (per_group < preferred && lds_bytes(preferred) <= lds_limit) per_group = preferred;
+    if (const char *e = getenv("GTM_FIT_PER_GROUP")) {  // tuning: clauses per group, at least C / CUs
+        const int asked = atoi(e);
+        if (asked >= (d.C + cus - 1) / cus && asked <= FITP_BLOCK) per_group = asked;
+    }
     if (lds_bytes(per_group) > lds_limit) return GTM_OK;
     const int groups = (d.C + per_group - 1) / per_group;
     p.clauses_per_group = per_group;

@@ -23,6 +23,15 @@
 //   whole number of 32-bit words (a multiple of the words one lane holds).
 #pragma once
 
+// Workgroup barrier for exchanges through LDS only: earlier LDS accesses of the wave are complete
+// and visible to the group afterwards, but loads from (and atomics on) global memory stay in flight
+// across it, which __syncthreads() would wait for.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 struct TileGeom {
     int slot_bits;        // bits per graph slot
     int slot_words;       // words per graph slot (0 when slot_bits < 32)
