@@ -186,45 +186,10 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         const uint32_t *rows = rows_buf[i & 1];
         unsigned long long *slot_now = p.class_sum + (size_t)(i % 3) * K * FITP_SUM_PARTS * FITP_SUM_STRIDE;
 
-        // ---- 0. requests that can be in flight while this example is evaluated: the next graph's
-        // rows and literal words (straight into the other LDS buffers) and the sizes of the graph after it
+        // ---- 0. the next graph's slot; the sizes of the graph after it are requested
         const bool has_next = i + 1 < p.n_examples;
         const FitGraph fn = fit_graph_slot(p.tg, has_next ? ex + 1 : ex, has_next ? n_next : n_now);
         const int next_total = has_next && !p.direct ? (p.literals + p.n_types + 1) * fn.words : 0;
-        {
-            // element at = row * words + w; a thread's elements are FITP_BLOCK apart: step (row, w) without dividing
-            const uint32_t *tile = p.tiles + (int64_t)fn.tile * p.tg.rows * p.tg.tw + fn.word0;
-            if (fn.words != div_words) {  // the divisions are redone only when the slot width changes
-                div_words = fn.words;
-                div_dr = FITP_BLOCK / fn.words;
-                div_r0 = tid / fn.words;
-            }
-            const int dr = div_dr, dw = FITP_BLOCK - dr * fn.words;
-            int r = div_r0, w = tid - r * fn.words;
-            uint32_t *dst = rows_buf[(i + 1) & 1] + wave * 64;
-            for (int at0 = 0; at0 < next_total; at0 += FITP_BLOCK) {
-                if (at0 + tid < next_total) fitp_load_to_lds(tile + (int64_t)r * p.tg.tw + w, dst + at0);
-                r += dr;
-                w += dw;
-                if (w >= fn.words) {
-                    w -= fn.words;
-                    ++r;
-                }
-            }
-        }
-        const int next_x_total = has_next ? n_next * LA : 0;
-        {
-            const uint32_t *src = p.X + (int64_t)base_next * LA + tid;
-            uint32_t *dst = x_buf[(i + 1) & 1] + wave * 64;
-            for (int at0 = 0; at0 < next_x_total; at0 += FITP_BLOCK)
-                if (at0 + tid < next_x_total) fitp_load_to_lds(src + at0, dst + at0);
-        }
-        if (has_next) {
-            const uint32_t *src = (const uint32_t *)p.encoded_Y + (int64_t)(ex + 1) * K + tid;
-            uint32_t *dst = y_buf[(i + 1) & 1] + wave * 64;
-            for (int at0 = 0; at0 < K; at0 += FITP_BLOCK)
-                if (at0 + tid < K) fitp_load_to_lds(src + at0, dst + at0);
-        }
         const uint32_t *x_now = x_buf[i & 1];
         // node count and first node of the graph after the next, fetched by two threads with vector
         // loads (scalar loads share their counter with LDS: the evaluation's first LDS read would wait
@@ -401,7 +366,43 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                                    __HIP_MEMORY_SCOPE_AGENT);
             votes[k] = 0;
         }
-        // Work that does not need the class sums is done while the other groups arrive
+        // Work that does not need the class sums is done while the other groups arrive: the next
+        // graph's rows, literal words and labels are requested (straight into the other LDS
+        // buffers; they are waited for at the end of the step)
+        {
+            // element at = row * words + w; a thread's elements are FITP_BLOCK apart: step (row, w) without dividing
+            const uint32_t *tile = p.tiles + (int64_t)fn.tile * p.tg.rows * p.tg.tw + fn.word0;
+            if (fn.words != div_words) {  // the divisions are redone only when the slot width changes
+                div_words = fn.words;
+                div_dr = FITP_BLOCK / fn.words;
+                div_r0 = tid / fn.words;
+            }
+            const int dr = div_dr, dw = FITP_BLOCK - dr * fn.words;
+            int r = div_r0, w = tid - r * fn.words;
+            uint32_t *dst = rows_buf[(i + 1) & 1] + wave * 64;
+            for (int at0 = 0; at0 < next_total; at0 += FITP_BLOCK) {
+                if (at0 + tid < next_total) fitp_load_to_lds(tile + (int64_t)r * p.tg.tw + w, dst + at0);
+                r += dr;
+                w += dw;
+                if (w >= fn.words) {
+                    w -= fn.words;
+                    ++r;
+                }
+            }
+        }
+        const int next_x_total = has_next ? n_next * LA : 0;
+        {
+            const uint32_t *src = p.X + (int64_t)base_next * LA + tid;
+            uint32_t *dst = x_buf[(i + 1) & 1] + wave * 64;
+            for (int at0 = 0; at0 < next_x_total; at0 += FITP_BLOCK)
+                if (at0 + tid < next_x_total) fitp_load_to_lds(src + at0, dst + at0);
+        }
+        if (has_next) {
+            const uint32_t *src = (const uint32_t *)p.encoded_Y + (int64_t)(ex + 1) * K + tid;
+            uint32_t *dst = y_buf[(i + 1) & 1] + wave * 64;
+            for (int at0 = 0; at0 < K; at0 += FITP_BLOCK)
+                if (at0 + tid < K) fitp_load_to_lds(src + at0, dst + at0);
+        }
         if (p.direct && has_next && tid < n_next) types_lds[(i + 1) & 1][tid] = type_ahead;
         // The random words of the feedback gates are drawn by the waves that do not poll, while the
         // class sums are on their way. (Drawing the Type I feedback bits of every (clause, class,
