@@ -113,6 +113,13 @@ __device__ __forceinline__ const uint32_t *fitp_row_word(const FitPersistParams 
 __device__ __forceinline__ void fitp_load_to_lds(const uint32_t *src, uint32_t *dst_of_wave) {
     __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) uint32_t *)dst_of_wave, 4, 0, 0);
 }
+// Between LDS writes of some lanes of a wave and reads of them by other lanes of the same wave (the
+// hardware carries out a wave's LDS accesses in order; this keeps the compiler from reordering them).
+__device__ __forceinline__ void fitp_wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+}
 constexpr int FITP_WAIT_VMEM = 0x0F70;  // s_waitcnt vmcnt(0) (export and LDS counters left alone)
 
 // MAXB: bit planes of an automaton the kernel keeps in registers while updating a word (>= B).
@@ -481,8 +488,9 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
 
         // ---- 3. feedback (K8) and automaton updates (K9) on the LDS copies
         const int32_t *y = (const int32_t *)y_buf[i & 1];
-        for (int j = tid; j < n_own * K; j += FITP_BLOCK) {
-            const int cl = j / K, k = j - cl * K;
+        const uint32_t *X_rows = x_now;  // the graph's literal words, node-major, in LDS
+        auto decide = [&](int j, int k) {  // K8 for (clause, class) pair j = cl * K + k
+            const int cl = j / K;
             int cs = sums[k];
             cs = cs > p.T ? p.T : (cs < -p.T ? -p.T : cs);
             const int yk = y[k];
@@ -503,43 +511,81 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 wts[j] = w;
             }
             upd[j] = u;
-        }
-        lds_barrier();
-        // Type I feedback bits for the (clause, class) pairs that need them: the pairs are listed
-        // first (wave 0, ballots), then one thread per (listed pair, word) draws the bits, so that
-        // the lanes that run the generator are (nearly) all busy
-        if (wave == 0) {
-            int n_listed = 0;
-            for (int j0 = 0; j0 < n_own * K; j0 += 64) {
-                const int j = j0 + lane;
-                const bool need = j < n_own * K && upd[j] > 0;
-                const unsigned long long m = __ballot(need);
-                if (need) pair_list[n_listed + __popcll(m & ((1ull << lane) - 1ull))] = j;
-                n_listed += __popcll(m);
+            return u;
+        };
+        if (own_max <= WAVES && K * LA <= 256) {
+            // One clause per wave and few (class, word) pairs per clause: the wave decides for the clause's classes, draws the Type I feedback
+            // bits of the (class, word) pairs that need them and updates the clause's automata, with
+            // no barrier in between (a wave's LDS accesses are carried out in order).
+            if (wave < n_own) {
+                const int cl = wave;
+                bool any = false;
+                for (int k0 = 0; k0 < K; k0 += 64) {
+                    const int k = k0 + lane;
+                    const int u = k < K ? decide(cl * K + k, k) : 0;
+                    any |= __ballot(u != 0) != 0ull;
+                    const unsigned long long type1 = __ballot(u > 0);
+                    const int n_items = __popcll(type1) * LA;
+                    for (int t = lane; t < n_items; t += 64) {
+                        const int nth = t / LA, w = t - nth * LA;
+                        unsigned long long m = type1;
+                        for (int skip = 0; skip < nth; ++skip) m &= m - 1;
+                        const int kk = k0 + __ffsll((long long)m) - 1;
+                        fbits[((size_t)cl * LA + w) * K + kk] =
+                            gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)kk, p.thr16);
+                    }
+                }
+                fitp_wave_lds_sync();
+                if (any) {
+                    const int node = node_of[cl];
+                    const bool fired = node != -1;
+                    const bool within = incl_of[cl] <= p.max_included;
+                    for (int w = lane; w < LA; w += 64) {
+                        const uint32_t x = fired ? X_rows[node * LA + w] : 0u;
+                        feedback_word<MAXB>(ta + ((size_t)cl * LA + w) * B, B, K, upd + cl * K, 1, fired, within, p.boost, x, p.k0,
+                                            p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, p.thr16,
+                                            fbits + ((size_t)cl * LA + w) * K);
+                    }
+                }
             }
-            if (lane == 0) n_pairs = n_listed;
-        }
-        lds_barrier();
-        for (int t = tid; t < n_pairs * LA; t += FITP_BLOCK) {
-            const int j = pair_list[t / LA], w = t % LA;
-            const int cl = j / K, k = j - cl * K;
-            fbits[((size_t)cl * LA + w) * K + k] =
-                gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
-        }
-        lds_barrier();
-        const uint32_t *X_rows = x_now;  // the graph's literal words, node-major, in LDS
-        for (int j = tid; j < n_own * LA; j += FITP_BLOCK) {
-            const int cl = j / LA, w = j - cl * LA;
-            const int32_t *u_of = upd + cl * K;
-            bool any = false;
-            for (int k = 0; k < K; ++k) any |= u_of[k] != 0;
-            if (!any) continue;
-            const int node = node_of[cl];
-            const bool fired = node != -1;
-            const bool within = incl_of[cl] <= p.max_included;
-            const uint32_t x = fired ? X_rows[node * LA + w] : 0u;
-            feedback_word<MAXB>(ta + (size_t)j * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1,
-                              (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, p.thr16, fbits + (size_t)j * K);
+        } else {
+            for (int j = tid; j < n_own * K; j += FITP_BLOCK) decide(j, j % K);
+            lds_barrier();
+            // Type I feedback bits for the (clause, class) pairs that need them: the pairs are listed
+            // first (wave 0, ballots), then one thread per (listed pair, word) draws the bits, so that
+            // the lanes that run the generator are (nearly) all busy
+            if (wave == 0) {
+                int n_listed = 0;
+                for (int j0 = 0; j0 < n_own * K; j0 += 64) {
+                    const int j = j0 + lane;
+                    const bool need = j < n_own * K && upd[j] > 0;
+                    const unsigned long long m = __ballot(need);
+                    if (need) pair_list[n_listed + __popcll(m & ((1ull << lane) - 1ull))] = j;
+                    n_listed += __popcll(m);
+                }
+                if (lane == 0) n_pairs = n_listed;
+            }
+            lds_barrier();
+            for (int t = tid; t < n_pairs * LA; t += FITP_BLOCK) {
+                const int j = pair_list[t / LA], w = t % LA;
+                const int cl = j / K, k = j - cl * K;
+                fbits[((size_t)cl * LA + w) * K + k] =
+                    gtm_feedback_bits(p.k0, p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, (uint32_t)k, p.thr16);
+            }
+            lds_barrier();
+            for (int j = tid; j < n_own * LA; j += FITP_BLOCK) {
+                const int cl = j / LA, w = j - cl * LA;
+                const int32_t *u_of = upd + cl * K;
+                bool any = false;
+                for (int k = 0; k < K; ++k) any |= u_of[k] != 0;
+                if (!any) continue;
+                const int node = node_of[cl];
+                const bool fired = node != -1;
+                const bool within = incl_of[cl] <= p.max_included;
+                const uint32_t x = fired ? X_rows[node * LA + w] : 0u;
+                feedback_word<MAXB>(ta + (size_t)j * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1,
+                                  (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, p.thr16, fbits + (size_t)j * K);
+            }
         }
         __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);  // the next graph's words are in LDS
         if (tid < 2) after_lds[tid] = after;
