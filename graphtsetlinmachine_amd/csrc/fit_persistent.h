@@ -4,14 +4,16 @@
 // Each workgroup owns a contiguous range of clauses for the whole run and keeps
 // their automata (all bit planes) and weights in LDS; they go back to global
 // memory once, at the end.  Per example a workgroup
-//   1. evaluates its clauses on the graph's literal-major rows (staged in LDS,
-//      the next graph's rows are fetched while waiting at the barrier),
-//      picks the nodes, and adds its clauses' votes to the class sums in
-//      global memory;
+//   1. evaluates its clauses on the graph's literal-major rows (staged in LDS;
+//      the next graph's rows, literal words and labels are loaded straight into
+//      the other LDS buffers while waiting at the barrier), picks the nodes, and
+//      adds its clauses' votes to the class sums in global memory;
 //   2. meets the other workgroups at a device-wide barrier (the class sums are
 //      the only thing that crosses clause boundaries, kernels.py:310-315);
 //   3. decides the feedback and updates its automata and weights in LDS.
-// Class sums and barrier are one thing: class k has a 64-bit word to which every
+// Class sums and barrier are one thing: class k has a 64-bit word (kept as
+// FITP_SUM_PARTS partial words that a reader adds up, since the memory system
+// carries out the adds to one word one after the other) to which every
 // workgroup adds (1 << 48) + its share with one device-scope atomic, and which it
 // then polls.  Nothing else is ever done to the word - no reset, no store - so
 // per-location coherence is all the protocol needs: nothing has to be ordered
@@ -21,11 +23,11 @@
 // difference is arrivals * 2^48 + sum, whatever borrows negative shares caused, so
 // with |sum| < 2^47 the arrivals are (difference + 2^47) >> 48 and, once they equal
 // the number of workgroups, the sum is the rest.  The words live in a ring of three
-// slots, each in a cache line of its own (the adds and polls of different classes
-// go to different memory channels): a workgroup can be one example ahead of the
-// slowest one, never three.  While waiting, all of a workgroup's polling threads
-// watch the word of class 0 (one request per poll) and look at their own only when
-// that one is complete.
+// slots, each partial word in a cache line of its own (the adds and polls go to
+// different memory channels): a workgroup can be one example ahead of the
+// slowest one, never three.  Thread k of a workgroup polls the word of class k.
+// The workgroup's barriers order LDS traffic only, so none of them waits for the
+// adds or for the loads of the next graph.
 //
 // The wait is bounded: after `spin_limit` polls a workgroup raises the abort
 // flag and every workgroup leaves the loop at its next check, so the grid always
@@ -150,10 +152,10 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
     uint32_t *x_buf[2] = {(uint32_t *)(pair_list + (size_t)own_max * K),
                           (uint32_t *)(pair_list + (size_t)own_max * K) + p.x_words};  // [nodes][LA] of the graph
     uint32_t *order_lds = x_buf[1] + p.x_words;                 // [literals]
-    // thread k < K: its class-sum word and the word of class 0 as they stood when each of the three
-    // slots was last complete (all zero before the first use): [slot][own, first][low, high][K]
+    // thread k < K: its class-sum word as it stood when each of the three
+    // slots was last complete (all zero before the first use): [slot][low, high][K]
     uint32_t *seen = order_lds + p.literals;
-    uint32_t *y_buf[2] = {seen + 12 * K, seen + 13 * K};        // [K] labels of this and the next example
+    uint32_t *y_buf[2] = {seen + 6 * K, seen + 7 * K};        // [K] labels of this and the next example
     __shared__ int go_on, n_pairs;
     __shared__ uint32_t after_lds[2];
     __shared__ uint32_t types_lds[2][FITP_DIRECT_NODES];  // node types of this and the next graph (direct evaluation)
@@ -181,7 +183,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         for (int k = tid; k < K; k += FITP_BLOCK) y_buf[0][k] = (uint32_t)p.encoded_Y[(int64_t)p.first_example * K + k];
     }
     for (int l = tid; l < p.literals; l += FITP_BLOCK) order_lds[l] = p.order[l];
-    for (int j = tid; j < 12 * K; j += FITP_BLOCK) seen[j] = 0u;
+    for (int j = tid; j < 6 * K; j += FITP_BLOCK) seen[j] = 0u;
     lds_barrier();
 
     const int ones_row = p.literals + p.n_types;
@@ -448,27 +450,14 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             auto arrivals = [](unsigned long long now, unsigned long long before) {
                 return ((now - before + FITP_HALF) >> 48) & 0xFFFFull;
             };
-            uint32_t *seen_slot = seen + (size_t)(i % 3) * 4 * K;
+            uint32_t *seen_slot = seen + (size_t)(i % 3) * 2 * K;
             const unsigned long long seen_own = ((unsigned long long)seen_slot[K + k] << 32) | seen_slot[k];
-            const unsigned long long seen_first = ((unsigned long long)seen_slot[3 * K + k] << 32) | seen_slot[2 * K + k];
             uint32_t polls = 0;
-            unsigned long long word = 0ull, first = 0ull;
-            bool ok = true, mine = false;
+            unsigned long long word = 0ull;
+            bool ok = true;
             for (;;) {
-                if (!mine) {
-                    first = read_sum(slot_now, 0);
-                    if (arrivals(first, seen_first) == everyone) {
-                        mine = true;
-                        if (k == 0) {
-                            word = first;
-                            break;
-                        }
-                        continue;
-                    }
-                } else {
-                    word = read_sum(slot_now, k);
-                    if (arrivals(word, seen_own) == everyone) break;
-                }
+                word = read_sum(slot_now, k);
+                if (arrivals(word, seen_own) == everyone) break;
                 if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
                     ++polls > p.spin_limit) {
                     __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -481,7 +470,6 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             sums[k] = (int32_t)(long long)(word - seen_own - (everyone << 48));
             // for the slot's next use, three examples on
             seen_slot[k] = (uint32_t)word, seen_slot[K + k] = (uint32_t)(word >> 32);
-            seen_slot[2 * K + k] = (uint32_t)first, seen_slot[3 * K + k] = (uint32_t)(first >> 32);
         }
         lds_barrier();
         if (!go_on) break;  // uniform over the group; every group leaves at its next check

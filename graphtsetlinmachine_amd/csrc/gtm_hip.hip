@@ -1341,7 +1341,7 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     auto lds_bytes = [&](int per_group) {
         return (2 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group +
                 2 * (size_t)d.K + 5 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K + 2 * (size_t)p.x_words +
-                (size_t)cfg->literals + 14 * (size_t)d.K) * 4;
+                (size_t)cfg->literals + 8 * (size_t)d.K) * 4;
     };
     const size_t lds_limit = 150 * 1024;
     int per_group = (d.C + cus - 1) / cus;
