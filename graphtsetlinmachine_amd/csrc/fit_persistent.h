@@ -187,6 +187,8 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
     lds_barrier();
 
     const int ones_row = p.literals + p.n_types;
+    // one small clause per wave: the feedback of a step runs inside the clause's wave
+    const bool wave_local = own_max <= WAVES && K * LA <= 256;
     int div_words = 0, div_dr = 0, div_r0 = 0;
     for (int i = 0; i < p.n_examples; ++i) {
         const int ex = p.first_example + i;
@@ -471,6 +473,8 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             // for the slot's next use, three examples on
             seen_slot[k] = (uint32_t)word, seen_slot[K + k] = (uint32_t)(word >> 32);
         }
+        __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);  // the next graph's words are in LDS
+        if (tid < 2) after_lds[tid] = after;
         lds_barrier();
         if (!go_on) break;  // uniform over the group; every group leaves at its next check
 
@@ -501,7 +505,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             upd[j] = u;
             return u;
         };
-        if (own_max <= WAVES && K * LA <= 256) {
+        if (wave_local) {
             // One clause per wave and few (class, word) pairs per clause: the wave decides for the clause's classes, draws the Type I feedback
             // bits of the (class, word) pairs that need them and updates the clause's automata, with
             // no barrier in between (a wave's LDS accesses are carried out in order).
@@ -575,15 +579,16 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                                   (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, p.thr16, fbits + (size_t)j * K);
             }
         }
-        __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);  // the next graph's words are in LDS
-        if (tid < 2) after_lds[tid] = after;
-        lds_barrier();
+        // With the feedback inside the clause's wave, the wave goes on to evaluate its clause on the
+        // next graph (everything that evaluation reads was complete at the barrier above).
+        if (!wave_local) lds_barrier();
         n_now = n_next;
         base_now = base_next;
         n_next = (int)after_lds[0];
         base_next = after_lds[1];
     }
     __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);  // no load into LDS is left in flight when the group ends
+    lds_barrier();
     // own state -> global memory (also after an abort: every clause is left as of some whole step)
     for (int i = tid; i < n_own * LA * B; i += FITP_BLOCK) p.bank[(int64_t)c0 * LA * B + i] = ta[i];
     for (int i = tid; i < n_own * K; i += FITP_BLOCK) {
