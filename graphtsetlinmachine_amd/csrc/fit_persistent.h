@@ -233,46 +233,62 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             bool all_rows = false;  // every included literal's row has been applied: acc is the clause's truth
             if (filter_only) {
                 int budget = FITP_FILTER_ROWS;
-                int r0 = 0;
-                unsigned long long picked = 0ull;  // lanes whose literal (in rarest-first order) is included and not applied yet
-                uint32_t lit = 0u;
-                for (;;) {
-                    if (budget <= 0) {
-                        // a few surviving nodes are cheapest tested one by one; more than that, and 8 more
-                        // rows (one LDS round trip) remove most of them at the price of testing one
-                        // (counted as lanes with a survivor, twice those with several: an estimate is enough)
-                        if (n_now <= FITP_FEW_NODES) break;
-                        const int mine = active ? __popc((acc >> fg.shift) & fg.mask) : 0;
-                        const int left = __popcll(__ballot(mine > 0)) + __popcll(__ballot(mine > 1));
-                        if (left <= FITP_FEW_NODES) break;
-                        budget = 8;
+                bool stop = false;
+                // The included literals in rarest-first order, 256 ranks at a time: the four LDS reads
+                // of the ranks and the four of the include words are each issued together (a clause
+                // whose rare literals are few would otherwise pay two LDS round trips per 64 ranks).
+                for (int g0 = 0; g0 < p.literals && !stop; g0 += 256) {
+                    uint32_t lit4[4];
+                    unsigned long long m4[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int r = g0 + 64 * u + lane;
+                        lit4[u] = r < p.literals ? order_lds[r] : 0u;
                     }
-                    if (picked == 0ull) {
-                        if (r0 >= p.literals) {
-                            all_rows = true;
-                            break;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int r = g0 + 64 * u + lane;
+                        uint32_t word = inc[(lit4[u] >> 5) * B];
+                        if ((int)(lit4[u] >> 5) == LA - 1) word &= p.filter;
+                        m4[u] = __ballot(r < p.literals && ((word >> (lit4[u] & 31u)) & 1u));
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        unsigned long long picked = m4[u];  // lanes whose literal is included and not applied yet
+                        const uint32_t lit = lit4[u];
+                        while (picked != 0ull && !stop) {
+                            if (budget <= 0) {
+                                // a few surviving nodes are cheapest tested one by one; more than that, and 8 more
+                                // rows (one LDS round trip) remove most of them at the price of testing one
+                                // (counted as lanes with a survivor, twice those with several: an estimate is enough)
+                                if (n_now <= FITP_FEW_NODES) {
+                                    stop = true;
+                                    break;
+                                }
+                                const int mine = active ? __popc((acc >> fg.shift) & fg.mask) : 0;
+                                const int left = __popcll(__ballot(mine > 0)) + __popcll(__ballot(mine > 1));
+                                if (left <= FITP_FEW_NODES) {
+                                    stop = true;
+                                    break;
+                                }
+                                budget = 8;
+                            }
+                            int row[8];
+#pragma unroll
+                            for (int v8 = 0; v8 < 8; ++v8) {
+                                row[v8] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
+                                picked &= picked - 1;
+                            }
+                            uint32_t r8[8];
+#pragma unroll
+                            for (int v8 = 0; v8 < 8; ++v8) r8[v8] = col[row[v8] * stride];
+#pragma unroll
+                            for (int v8 = 0; v8 < 8; ++v8) acc &= r8[v8];
+                            budget -= 8;
                         }
-                        const int r = r0 + lane;
-                        lit = r < p.literals ? order_lds[r] : 0u;
-                        uint32_t word = inc[(lit >> 5) * B];
-                        if ((int)(lit >> 5) == LA - 1) word &= p.filter;
-                        picked = __ballot(r < p.literals && ((word >> (lit & 31u)) & 1u));
-                        r0 += 64;
-                        continue;
                     }
-                    int row[8];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) {
-                        row[u] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
-                        picked &= picked - 1;
-                    }
-                    uint32_t r8[8];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) r8[u] = col[row[u] * stride];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) acc &= r8[u];
-                    budget -= 8;
                 }
+                all_rows = !stop;  // every included literal's row has been applied
             } else if (!p.direct) {
                 for (int w0 = 0; w0 < LA; w0 += 64) {
                     uint32_t mine = w0 == 0 ? first_words : (w0 + lane < LA ? inc[(w0 + lane) * B] : 0u);
