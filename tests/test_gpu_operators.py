@@ -441,6 +441,35 @@ def test_fused_fit_on_every_tile_geometry(shape, boost, max_included, state_bits
     assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
 
 
+@pytest.mark.parametrize("shape", [TILE_SHAPES[3], TILE_SHAPES[5], TILE_SHAPES[6]], ids=lambda s: "tiles%d" % s["seed"])
+@pytest.mark.parametrize("per_group", [1, 3, 16, 20, 40])
+def test_one_launch_fit_with_any_number_of_clauses_per_workgroup(shape, per_group, monkeypatch):
+    """The cooperative training kernel gives a workgroup 8 or more clauses; GTM_FIT_PER_GROUP sets
+    the number.  Up to 16 (one clause per wave) a small clause's feedback runs inside its wave,
+    above that a wave evaluates several clauses and the feedback is shared out over the group:
+    every split == the oracle."""
+    from tests.gpu_harness import Device
+
+    monkeypatch.setenv("GTM_FIT_PER_GROUP", str(per_group))
+    g = dict(shape["g"])
+    g["n_graphs"] = min(g["n_graphs"], 24)
+    graphs = helpers.random_graphs(shape["seed"], **g)
+    cfg = helpers.oracle_config(graphs, classes=shape["classes"], clauses=shape["clauses"], T=30)
+    model = helpers.random_model(shape["seed"], cfg, 1, s=3.0, include_density=0.02)
+    dev = Device(model, graphs)
+    assert dev.build_tiles()
+    rng = np.random.default_rng(shape["seed"] + per_group)
+    G = graphs.number_of_graphs
+    Y = o.encode_labels(rng.integers(0, cfg.classes, size=G), cfg.classes, cfg.threshold)
+    for epoch in range(2):
+        o.fit(model, graphs, Y)
+        dev.fit(Y, 0, G, epoch * G)
+        ta, _, w = dev.download()
+        assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
+        assert np.array_equal(ta, model.ta_state), "automata after epoch %d" % epoch
+    assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
+
+
 @pytest.mark.parametrize("seed,g,m", [
     (15, dict(n_graphs=10, max_nodes=361, min_nodes=300, hv_size=128, max_degree=0), dict(classes=10, clauses=60, depth=1)),
     (18, dict(n_graphs=12, max_nodes=50, hv_size=256, n_symbols=12, node_types=("a", "b")), dict(classes=4, clauses=64, depth=1)),
