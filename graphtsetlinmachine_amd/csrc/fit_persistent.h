@@ -69,7 +69,7 @@ __device__ __forceinline__ void fitp_stage_rows(const FitPersistParams &p, const
     const uint32_t *tile = p.tiles + (int64_t)fg.tile * p.tg.rows * p.tg.tw + fg.word0;
     const int words = fg.words;
     const int total = (p.literals + p.n_types + 1) * words;
-    // element i = r * words + w; a thread visits i = tid, tid + 256, ...: (r, w) advance without dividing
+    // element i = r * words + w; a thread visits i = tid, tid + FITP_BLOCK, ...: (r, w) advance without dividing
     const int dr = FITP_BLOCK / words, dw = FITP_BLOCK - dr * words;
     int r = tid / words, w = tid - r * words;
     for (int base = tid; base < total; base += FITP_BLOCK * 8) {
@@ -101,12 +101,6 @@ constexpr int FITP_WALK_ALL = 24;   // clauses with at most this many literals A
 constexpr int FITP_FILTER_ROWS = 16;  // rows the others AND before testing the surviving nodes
 constexpr int FITP_DIRECT_NODES = 2;  // data sets whose graphs have at most this many nodes skip the literal rows altogether
 constexpr int FITP_FEW_NODES = 2;     // up to this many surviving nodes are tested one by one, more are filtered further
-
-// Address of element `i` of the staged rows (i = row * words + w) inside the graph's tile.
-__device__ __forceinline__ const uint32_t *fitp_row_word(const FitPersistParams &p, const FitGraph &fg, int i) {
-    const int r = i / fg.words, w = i - r * fg.words;
-    return p.tiles + ((int64_t)fg.tile * p.tg.rows + r) * p.tg.tw + fg.word0 + w;
-}
 
 // One 32-bit word per lane from global memory straight into LDS (no register holds it meanwhile):
 // lane l's word lands at dst_of_wave[l]; dst_of_wave must be the same for the whole wave. The words
