@@ -441,6 +441,47 @@ def test_fused_fit_on_every_tile_geometry(shape, boost, max_included, state_bits
     assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
 
 
+MANY_CLASSES_SHAPES = [
+    dict(seed=61, g=dict(n_graphs=40, max_nodes=1, hv_size=40, max_degree=0), depth=1, clauses=50),
+    dict(seed=62, g=dict(n_graphs=24, max_nodes=31, min_nodes=17, hv_size=64, max_degree=0), depth=1, clauses=90),
+    dict(seed=63, g=dict(n_graphs=8, max_nodes=361, min_nodes=300, hv_size=128, max_degree=0), depth=1, clauses=40),
+    dict(seed=64, g=dict(n_graphs=30, max_nodes=12, min_nodes=2, hv_size=16, max_degree=2), depth=2, clauses=30),
+    dict(seed=65, g=dict(n_graphs=10, max_nodes=150, min_nodes=70, hv_size=32, max_degree=2), depth=3, clauses=40),
+]
+
+
+@pytest.mark.parametrize("shape", MANY_CLASSES_SHAPES, ids=lambda s: "shape%d" % s["seed"])
+@pytest.mark.parametrize("classes", [65, 130])
+def test_more_classes_than_lanes(shape, classes):
+    """More classes than a wave has lanes (the kernels keep per-class values lane by lane up to 64
+    and loop beyond): inference without and with tiles, two epochs of training on whichever path
+    the shape takes, inference again == the oracle."""
+    from tests.gpu_harness import Device
+
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    depth = shape["depth"]
+    cfg = helpers.oracle_config(graphs, classes=classes, clauses=shape["clauses"], depth=depth, T=20, message_size=64)
+    model = helpers.random_model(shape["seed"], cfg, depth, s=(3.0,) * depth, include_density=0.03)
+    dev = Device(model, graphs)
+    G = graphs.number_of_graphs
+    want = o.score(model, graphs)
+    assert np.array_equal(dev.score(0, G, G), want)
+    if dev.build_tiles():
+        assert np.array_equal(dev.score(0, G, G), want)
+        assert np.array_equal(dev.score(0, G, 7), want)
+    rng = np.random.default_rng(shape["seed"])
+    Y = o.encode_labels(rng.integers(0, classes, size=G), classes, cfg.threshold)
+    for epoch in range(2):
+        o.fit(model, graphs, Y)
+        dev.fit(Y, 0, G, epoch * G)
+        ta, banks, w = dev.download()
+        assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
+        assert np.array_equal(ta, model.ta_state), "layer-0 automata after epoch %d" % epoch
+        for layer in range(depth - 1):
+            assert np.array_equal(banks[layer], model.message_ta_state[layer]), "bank %d epoch %d" % (layer, epoch)
+    assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
+
+
 @pytest.mark.parametrize("shape", [TILE_SHAPES[3], TILE_SHAPES[5], TILE_SHAPES[6]], ids=lambda s: "tiles%d" % s["seed"])
 @pytest.mark.parametrize("per_group", [1, 3, 16, 20, 40])
 def test_one_launch_fit_with_any_number_of_clauses_per_workgroup(shape, per_group, monkeypatch):
