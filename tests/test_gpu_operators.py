@@ -451,6 +451,35 @@ MANY_CLASSES_SHAPES = [
 
 
 @pytest.mark.parametrize("shape", MANY_CLASSES_SHAPES, ids=lambda s: "shape%d" % s["seed"])
+@pytest.mark.parametrize("state_bits", [1, 2, 16, 17, 32])
+def test_narrow_and_wide_automata(shape, state_bits):
+    """Automata of 1 to 32 bits (the training kernels keep 8, 16 or 32 planes of a word in
+    registers): two epochs on whichever path the shape takes == the oracle."""
+    from tests.gpu_harness import Device
+
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    depth = shape["depth"]
+    cfg = helpers.oracle_config(graphs, classes=4, clauses=shape["clauses"], depth=depth, T=20, message_size=64,
+                                state_bits=state_bits)
+    model = helpers.random_model(shape["seed"], cfg, depth, s=(3.0,) * depth, include_density=0.03)
+    dev = Device(model, graphs)
+    dev.build_tiles()
+    G = graphs.number_of_graphs
+    assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
+    rng = np.random.default_rng(shape["seed"])
+    Y = o.encode_labels(rng.integers(0, 4, size=G), 4, cfg.threshold)
+    for epoch in range(2):
+        o.fit(model, graphs, Y)
+        dev.fit(Y, 0, G, epoch * G)
+        ta, banks, w = dev.download()
+        assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
+        assert np.array_equal(ta, model.ta_state), "layer-0 automata after epoch %d" % epoch
+        for layer in range(depth - 1):
+            assert np.array_equal(banks[layer], model.message_ta_state[layer]), "bank %d epoch %d" % (layer, epoch)
+    assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
+
+
+@pytest.mark.parametrize("shape", MANY_CLASSES_SHAPES, ids=lambda s: "shape%d" % s["seed"])
 @pytest.mark.parametrize("classes", [65, 130])
 def test_more_classes_than_lanes(shape, classes):
     """More classes than a wave has lanes (the kernels keep per-class values lane by lane up to 64
