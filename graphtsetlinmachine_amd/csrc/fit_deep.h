@@ -72,10 +72,13 @@ __global__ __launch_bounds__(64) void k_fit_message_rows(const uint32_t *__restr
 // which needs (true pairs x MESSAGE_BITS) LDS atomics and (edges x words)
 // global ones instead of (true pairs x edges x MESSAGE_BITS x 2) global ones.
 
-constexpr int FIT_NODE_MESSAGES_BLOCK = 256;
+constexpr int FIT_NODE_MESSAGES_BLOCK = 1024;
 constexpr int FIT_NODE_MESSAGES_CLAUSES = 1024;  // clauses per block
+constexpr int FIT_NODE_MESSAGES_PARTS = 4;       // threads that share a clause's word of 32 nodes
 
-// grid (node words in use, ceil(C / FIT_NODE_MESSAGES_CLAUSES)); dynamic LDS 32 * (MW | 1) words
+// grid (node words in use, ceil(C / FIT_NODE_MESSAGES_CLAUSES)); dynamic LDS 32 * (MW | 1) words.
+// What a thread does is a chain of dependent LDS atomics, so a clause's 32 nodes are split over
+// FIT_NODE_MESSAGES_PARTS threads, and a hypervector bit is fetched once for all of a thread's nodes.
 __global__ __launch_bounds__(FIT_NODE_MESSAGES_BLOCK) void k_fit_node_messages(
     const uint32_t *__restrict__ bitmap, int C, int NC, int n_nodes, const uint32_t *__restrict__ hv, int MB, int MW,
     uint32_t *sent) {
@@ -83,19 +86,20 @@ __global__ __launch_bounds__(FIT_NODE_MESSAGES_BLOCK) void k_fit_node_messages(
     const int tid = threadIdx.x;
     const int nw = blockIdx.x;
     const int MWP = MW | 1;
+    constexpr int PARTS = FIT_NODE_MESSAGES_PARTS, BITS = 32 / PARTS;
     for (int i = tid; i < 32 * MWP; i += FIT_NODE_MESSAGES_BLOCK) vec[i] = 0u;
     __syncthreads();
     const int c_end = min(C, (int)(blockIdx.y + 1) * FIT_NODE_MESSAGES_CLAUSES);
     const uint32_t valid = n_nodes - nw * 32 >= 32 ? 0xFFFFFFFFu : (1u << (n_nodes - nw * 32)) - 1u;
-    for (int c = blockIdx.y * FIT_NODE_MESSAGES_CLAUSES + tid; c < c_end; c += FIT_NODE_MESSAGES_BLOCK) {
-        uint32_t word = bitmap[(int64_t)c * NC + nw] & valid;
-        while (word) {
-            const int n = __ffs(word) - 1;
-            word &= word - 1;
-            for (int j = 0; j < MB; ++j) {
-                const uint32_t h = hv[(int64_t)c * MB + j];
-                atomicOr(&vec[n * MWP + (h >> 5)], 1u << (h & 31));
-            }
+    const uint32_t mine = valid & (((1u << BITS) - 1u) << ((tid % PARTS) * BITS));
+    for (int c = blockIdx.y * FIT_NODE_MESSAGES_CLAUSES + tid / PARTS; c < c_end; c += FIT_NODE_MESSAGES_BLOCK / PARTS) {
+        const uint32_t word = bitmap[(int64_t)c * NC + nw] & mine;
+        if (!word) continue;
+        for (int j = 0; j < MB; ++j) {
+            const uint32_t h = hv[(int64_t)c * MB + j];
+            uint32_t *column = vec + (h >> 5);
+            const uint32_t bit = 1u << (h & 31);
+            for (uint32_t m = word; m; m &= m - 1) atomicOr(&column[(__ffs(m) - 1) * MWP], bit);
         }
     }
     __syncthreads();

@@ -339,7 +339,7 @@ inline size_t tile_layer_lds_bytes(const TileGeom &g, int classes, int src, int 
 // (got is cleared before every layer's k_tile_edge_messages)
 // MW = ceil(M / 32) words per vector.
 
-constexpr int TILE_MESSAGES_BLOCK = 256;
+constexpr int TILE_MESSAGES_BLOCK = 1024;
 
 // Transposes the 32 x 32 bit matrix whose row i is the word of lane i (of each half of the wave):
 // afterwards bit i of lane b's word is what bit b of lane i's word was.  Five exchanges of
