@@ -81,7 +81,8 @@ constexpr int FIT_NODE_MESSAGES_PARTS = 4;       // threads that share a clause'
 // FIT_NODE_MESSAGES_PARTS threads, and a hypervector bit is fetched once for all of a thread's nodes.
 __global__ __launch_bounds__(FIT_NODE_MESSAGES_BLOCK) void k_fit_node_messages(
     const uint32_t *__restrict__ bitmap, int C, int NC, int n_nodes, const uint32_t *__restrict__ hv, int MB, int MW,
-    uint32_t *sent) {
+    uint32_t *sent, const uint32_t *__restrict__ n_edges, const uint32_t *__restrict__ edge_index,
+    const uint32_t *__restrict__ edge, uint32_t *got) {
     extern __shared__ uint32_t vec[];  // [32 nodes][MW | 1]: lanes on different nodes hit different banks
     const int tid = threadIdx.x;
     const int nw = blockIdx.x;
@@ -103,6 +104,26 @@ __global__ __launch_bounds__(FIT_NODE_MESSAGES_BLOCK) void k_fit_node_messages(
         }
     }
     __syncthreads();
+    if (n_edges != nullptr) {
+        // One block holds every clause (the host passes the edges only then): its 32 vectors are
+        // complete and go along the edges from here, as k_fit_edge_messages would send them.
+        const uint32_t M = (uint32_t)MW * 32u;
+        for (int i = tid; i < 32 * MW; i += FIT_NODE_MESSAGES_BLOCK) {
+            const int nl = i / MW, j = i - nl * MW, n = nw * 32 + nl;
+            if (n >= n_nodes) continue;
+            const uint32_t *v = vec + nl * MWP;
+            const uint32_t ne = n_edges[n];
+            const int64_t e0 = edge_index[n];
+            for (uint32_t e = 0; e < ne; ++e) {
+                const uint32_t dst = edge[(e0 + e) * 2], shift = edge[(e0 + e) * 2 + 1] % M;
+                const int q = (int)(shift >> 5), r = (int)(shift & 31u);
+                const int a = (j - q + MW) % MW, below = (a - 1 + MW) % MW;
+                const uint32_t word = r ? (v[a] << r) | (v[below] >> (32 - r)) : v[a];
+                if (word) atomicOr(&got[(int64_t)dst * MW + j], word);
+            }
+        }
+        return;
+    }
     for (int i = tid; i < 32 * MW; i += FIT_NODE_MESSAGES_BLOCK) {
         const int n = nw * 32 + i / MW;
         const uint32_t word = vec[(i / MW) * MWP + i % MW];

@@ -1626,13 +1626,17 @@ int fit_deep_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g,
         for (int l = 0; l < layers; ++l) {
             uint32_t *cx = w.clause_X[l];
             if (factored && (int64_t)d.C * n_nodes >= factor_min) {
-                if (n_nodes > 0) {
-                    hipLaunchKernelGGL(k_fit_node_messages,
-                                       dim3(words, (d.C + FIT_NODE_MESSAGES_CLAUSES - 1) / FIT_NODE_MESSAGES_CLAUSES),
-                                       dim3(FIT_NODE_MESSAGES_BLOCK), (size_t)32 * (MW | 1) * 4, st, cur, d.C, d.NC, n_nodes,
-                                       s->hypervectors, d.MB, MW, w.sent);
+                if (n_nodes > 0 && g->total_edges > 0) {  // without edges nothing is received: the messages stay blank
+                    // with every clause in one block, that block also sends its vectors along the edges
+                    const int clause_blocks = (d.C + FIT_NODE_MESSAGES_CLAUSES - 1) / FIT_NODE_MESSAGES_CLAUSES;
+                    const bool and_edges = clause_blocks == 1;
+                    const uint32_t *no_edges = nullptr;
+                    hipLaunchKernelGGL(k_fit_node_messages, dim3(words, clause_blocks), dim3(FIT_NODE_MESSAGES_BLOCK),
+                                       (size_t)32 * (MW | 1) * 4, st, cur, d.C, d.NC, n_nodes, s->hypervectors, d.MB, MW,
+                                       w.sent, and_edges ? g->number_of_graph_node_edges + h_base[i] : no_edges,
+                                       and_edges ? g->edge_index + h_base[i] : no_edges, g->edge, w.got);
                     if (int rc = check_launch("fit_node_messages")) return rc;
-                    if (g->total_edges > 0) {
+                    if (!and_edges) {
                         hipLaunchKernelGGL(k_fit_edge_messages, dim3(blocks_for((int64_t)n_nodes * MW, TPB)), dim3(TPB), 0,
                                            st, w.sent, n_nodes, MW, g->number_of_graph_node_edges + h_base[i],
                                            g->edge_index + h_base[i], g->edge, w.got);
