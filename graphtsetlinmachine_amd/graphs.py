@@ -138,7 +138,8 @@ class Graphs:
         self.node_index = np.zeros(counts.shape[0], dtype=np.uint32)
         self.node_index[1:] = np.add.accumulate(counts[:-1])
         self.max_number_of_graph_nodes = counts.max()
-        self.max_number_of_graph_node_chunks = (self.max_number_of_graph_nodes - 1) // 32 + 1
+        # 0 for a data set without nodes (the reference's unsigned subtraction wraps there, graphs.py:105)
+        self.max_number_of_graph_node_chunks = np.uint32((int(self.max_number_of_graph_nodes) - 1) // 32 + 1)
         self.number_of_nodes = counts.sum()
         n = int(self.number_of_nodes)
         self.node_type = np.empty(n, dtype=np.uint32)

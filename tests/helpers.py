@@ -46,7 +46,7 @@ def oracle_config(graphs, classes, clauses, depth=1, message_size=37, message_bi
     return o.Config(
         classes=classes, clauses=clauses, literals=2 * graphs.hypervector_size, state_bits=state_bits,
         boost_true_positive_feedback=boost, threshold=T, q=q, max_included_literals=max_included,
-        negative_clauses=1, max_nodes=int(max_nodes or graphs.max_number_of_graph_nodes),
+        negative_clauses=1, max_nodes=max(1, int(max_nodes or graphs.max_number_of_graph_nodes)),  # as tm.py sizes a model for a data set without nodes
         message_size=message_size, message_bits=message_bits,
     )
 
