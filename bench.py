@@ -32,8 +32,8 @@ MEASURED_TRAFFIC_BYTES_PER_GRAPH = {"convolutional_images": (131715.6 * 2 + 406.
 def parse():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=20)
-    p.add_argument("--warmup", type=int, default=3)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--workload", default="convolutional_images")
     p.add_argument("--graphs", type=int, default=10000, help="test graphs scored per step")
     p.add_argument("--train-graphs", type=int, default=60000, help="training graphs used to produce the model state")
