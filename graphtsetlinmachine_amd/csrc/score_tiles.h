@@ -898,6 +898,8 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
 // units of 16 bytes, unused ones pointing at the all-ones row - followed by the
 // LA words of the include mask.
 
+constexpr int TWO_PHASE_WALK_FROM = 6;  // slots a lane has left besides its first from which a clause's rows are all walked instead
+
 struct alignas(32) Packed8 {
     uint32_t v[8];
 };
@@ -1117,14 +1119,47 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
                 acc.w[u] = failed ? rest.w[u] : acc.w[u];
             }
             if (__ballot(tested && any_bit(rest)) != 0) {
+                int others = 0;
 #pragma unroll
-                for (int u = 0; u < LW; ++u) {
-                    uint32_t todo = tested ? rest.w[u] : 0u;
-                    while (todo) {
-                        const int b = __ffs(todo) - 1;
-                        todo &= todo - 1;
-                        const uint4 *x = reinterpret_cast<const uint4 *>(x_base + (lane_x0 + (u * 32 + b) * (LA4 * 16u)));
-                        if (violates(include, x)) acc.w[u] &= ~(1u << b);
+                for (int u = 0; u < LW; ++u) others += __popc(tested ? rest.w[u] : 0u);
+                if (__builtin_expect(__ballot(others >= TWO_PHASE_WALK_FROM) != 0, 0)) {
+                    // Phase 1 has left some lane several slots (its literals hold nearly everywhere:
+                    // negated ones, mostly), and testing them costs a memory round trip each.  The
+                    // rows of ALL the clause's literals are ANDed instead, as k_tile_layer does
+                    // (row l belongs to literal l; unused reads take the all-ones row).
+                    acc = p.acc;
+                    const uint32_t row_bytes = (uint32_t)a.tg.tw * 4u, ones = (uint32_t)(a.tg.rows - 1);
+                    uint32_t include_of_lane = 0u;  // lane w holds include word w: one copy of the loop below
+#pragma unroll
+                    for (int w = 0; w < 4 * LA4; ++w) include_of_lane = lane == w ? include.v[w] : include_of_lane;
+#pragma unroll 1
+                    for (int w = 0; w < 4 * LA4; ++w) {
+                        uint32_t m = __builtin_amdgcn_readlane(include_of_lane, w);
+                        while (m) {
+                            LaneWords<LW> r[8];
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) {
+                                const uint32_t lit = m ? (uint32_t)(w * 32 + __builtin_ctz(m)) : ones;
+                                m &= m - 1u;
+                                r[u].load(col + lit * row_bytes);
+                            }
+#pragma unroll
+                            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                                for (int v = 0; v < LW; ++v) acc.w[v] &= r[u].w[v];
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < LW; ++u) {
+                        uint32_t todo = tested ? rest.w[u] : 0u;
+                        while (todo) {
+                            const int b = __ffs(todo) - 1;
+                            todo &= todo - 1;
+                            const uint4 *x =
+                                reinterpret_cast<const uint4 *>(x_base + (lane_x0 + (u * 32 + b) * (LA4 * 16u)));
+                            if (violates(include, x)) acc.w[u] &= ~(1u << b);
+                        }
                     }
                 }
             }

@@ -263,6 +263,35 @@ def test_tile_scoring_equals_oracle(shape, density):
         assert np.array_equal(dev.score(3, G - 5, G), plain[3:G - 2])
 
 
+@pytest.mark.parametrize("hv_size,sizes", [
+    (64, [40, 0, 2, 64, 1, 50, 3, 1, 2, 5]), (128, [361, 1, 300, 0, 2, 361, 3, 1]), (256, [100, 1, 31, 2, 90, 1, 3, 2, 1])])
+@pytest.mark.parametrize("depth", [1, 2])
+def test_tile_scoring_with_clauses_of_negated_literals(hv_size, sizes, depth):
+    """Clauses that include 16 to 40 negated literals and nothing else: each
+    of them holds at nearly every node, so the rarest literals of a clause
+    filter out almost nothing and the two-phase layer 0 is left with most node
+    slots (it then ANDs the rows of all the clause's literals instead)."""
+    from tests.gpu_harness import Device
+
+    graphs = helpers.random_graphs(41, n_graphs=len(sizes), hv_size=hv_size, n_symbols=24, sizes=sizes, max_degree=2)
+    cfg = helpers.oracle_config(graphs, classes=3, clauses=48, depth=depth, message_size=64)
+    model = helpers.random_model(41, cfg, depth, include_density=0.0, message_density=0.0)
+    rng = np.random.default_rng(41)
+    top = cfg.state_bits - 1
+    for c in range(cfg.clauses):
+        for k in rng.choice(hv_size, size=int(rng.integers(16, 41)), replace=False):
+            lit = hv_size + int(k)
+            model.ta_state[c, lit // 32, top] |= np.uint32(1 << (lit % 32))
+    G = graphs.number_of_graphs
+    want = o.score(model, graphs)
+    assert len(np.unique(want, axis=0)) > 1, "the clauses should tell some graphs apart"
+    dev = Device(model, graphs)
+    assert np.array_equal(dev.score(0, G, G), want)
+    assert dev.build_tiles()
+    assert np.array_equal(dev.score(0, G, G), want)
+    assert np.array_equal(dev.score(0, G, 2), want)
+
+
 DEEP_TILE_SHAPES = [
     # several graphs per word; one word per graph; several words; 361-node graphs; literal rows too
     # big for LDS (read in place); graphs without nodes; single-node graphs with self-loops
