@@ -892,7 +892,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     const int tile_first = first / tg.gpt, tile_last = (first + n_graphs - 1) / tg.gpt;
     const int MW = (d.M + 31) / 32;
     int group = 16;  // words of a truth row per k_tile_node_messages block: its vectors must fit in 64 KB of LDS
-    while (group > 1 && (size_t)32 * group * (MW | 1) * 4 > 64 * 1024) group >>= 1;
+    while (group > 1 && ((size_t)32 * group * (MW | 1) + group) * 4 > 64 * 1024) group >>= 1;
     a.message_rows = w.message_rows;
     const size_t fused_lds = tg.slot_words > 0 ? tile_fused_messages_lds_bytes(tg, MW) : 0;
     bool fused_messages = tg.slot_words > 0 && d.M % 32 == 0 && fused_lds <= 150 * 1024 && !getenv("GTM_NO_FUSED_MESSAGES");
@@ -937,7 +937,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                 continue;
             }
             hipLaunchKernelGGL(k_tile_node_messages, dim3((tg.tw + group - 1) / group, n_tiles),
-                               dim3(TILE_MESSAGES_BLOCK), (size_t)32 * group * (MW | 1) * 4, st, w.tile_bitmap, d.C, tg.tw,
+                               dim3(TILE_MESSAGES_BLOCK), ((size_t)32 * group * (MW | 1) + group) * 4, st, w.tile_bitmap, d.C, tg.tw,
                                group, s->hypervectors, d.MB, MW, w.sent);
             if (int rc = check_launch("tile_node_messages")) return rc;
             const int64_t vector_words = (int64_t)n_tiles * tg.tw * 32 * MW;

@@ -366,11 +366,13 @@ __device__ __forceinline__ uint32_t tile_transpose32(uint32_t v, int lane) {
 __global__ __launch_bounds__(TILE_MESSAGES_BLOCK) void k_tile_node_messages(
     const uint32_t *__restrict__ bitmap, int C, int tw, int group, const uint32_t *__restrict__ hv, int MB, int MW,
     uint32_t *__restrict__ sent) {
-    extern __shared__ uint32_t vec[];  // [32 * group slots][MW | 1]: lanes on different slots hit different banks
+    // [32 * group slots][MW | 1], slot s at s * (MW | 1) + s / 32: lanes on neighbouring slots hit different
+    // banks, and so do lanes on the same bit of different words of a row (32 slots apart)
+    extern __shared__ uint32_t vec[];
     const int tid = threadIdx.x;
     const int w0 = blockIdx.x * group, tile = blockIdx.y;
     const int MWP = MW | 1;
-    const int n_vec = 32 * group * MWP;
+    const int n_vec = 32 * group * MWP + group;
     for (int i = tid; i < n_vec; i += TILE_MESSAGES_BLOCK) vec[i] = 0u;
     __syncthreads();
     const int wl = tid & (group - 1), w = w0 + wl;
@@ -393,7 +395,7 @@ __global__ __launch_bounds__(TILE_MESSAGES_BLOCK) void k_tile_node_messages(
                 for (int j = 0; j < MB; ++j) {
                     const uint32_t h = hv[(int64_t)c * MB + j];
                     const uint32_t bit = 1u << (h & 31);
-                    uint32_t *column = vec + (wl * 32) * MWP + (h >> 5);
+                    uint32_t *column = vec + (wl * 32) * MWP + wl + (h >> 5);
                     for (uint32_t m = word; m; m &= m - 1) atomicOr(&column[(__ffs(m) - 1) * MWP], bit);
                 }
             }
@@ -401,7 +403,7 @@ __global__ __launch_bounds__(TILE_MESSAGES_BLOCK) void k_tile_node_messages(
     __syncthreads();
     uint32_t *out = sent + ((int64_t)tile * tw + w0) * 32 * MW;
     const int n_out = (min(tw, w0 + group) - w0) * 32 * MW;
-    for (int i = tid; i < n_out; i += TILE_MESSAGES_BLOCK) out[i] = vec[(i / MW) * MWP + i % MW];
+    for (int i = tid; i < n_out; i += TILE_MESSAGES_BLOCK) out[i] = vec[(i / MW) * MWP + ((i / MW) >> 5) + i % MW];
 }
 
 // One thread per (tile of the launch, node slot, vector word).
@@ -503,7 +505,9 @@ __global__ __launch_bounds__(256) void k_tile_pack_messages(const uint32_t *__re
 constexpr int TILE_FUSED_MESSAGES_BLOCK = 1024;
 
 inline size_t tile_fused_messages_lds_bytes(const TileGeom &g, int MW) {
-    return 2 * (size_t)g.slot_bits * (MW | 1) * 4;  // vectors are MW | 1 words apart: lanes on different slots hit different banks
+    // vectors are MW | 1 words apart plus one word per 32 slots: lanes on neighbouring slots hit different
+    // banks, and so do lanes on the same bit of different words of a truth row (32 slots apart)
+    return 2 * ((size_t)g.slot_bits * (MW | 1) + (size_t)g.slot_words) * 4;
 }
 
 __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fused(
@@ -516,14 +520,15 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int gj = blockIdx.x, tile_local = blockIdx.y;
     const int tw = tg.tw, sw = tg.slot_words, slots = tg.slot_bits, MWP = MW | 1;
-    uint32_t *sent = lds;               // [slots][MWP]
-    uint32_t *got = lds + slots * MWP;  // [slots][MWP]
+    const int VEC = slots * MWP + sw;   // slot n's vector starts at n * MWP + n / 32
+    uint32_t *sent = lds;
+    uint32_t *got = lds + VEC;
     const int64_t g = (int64_t)(tile0 + tile_local) * tg.gpt + gj;
     const int nodes = g < G ? (int)n_nodes[g] : 0;
     const int w_first = gj * sw;        // the graph's first word of a tile row
     uint32_t *out = rows + (int64_t)tile_local * (M + 2) * tw;
 
-    for (int i = tid; i < 2 * slots * MWP; i += NT) lds[i] = 0u;
+    for (int i = tid; i < 2 * VEC; i += NT) lds[i] = 0u;
     __syncthreads();
 
     // 1. what every node slot sends
@@ -551,7 +556,7 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
                 for (int j = 0; j < MB; ++j) {
                     const uint32_t h = j < 2 ? h01[u][j] : hv[(int64_t)cs[u] * MB + j];
                     const uint32_t bit = 1u << (h & 31);
-                    uint32_t *column = sent + (wls[u] * 32) * MWP + (h >> 5);
+                    uint32_t *column = sent + (wls[u] * 32) * MWP + wls[u] + (h >> 5);
                     for (uint32_t m = word; m; m &= m - 1) atomicOr(&column[(__ffs(m) - 1) * MWP], bit);
                 }
             }
@@ -565,7 +570,7 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
     if (has_edges && nodes > 0) {
         const int64_t row0 = node_index[g];
         for (int n = tid; n < nodes; n += NT) {
-            const uint32_t *v = sent + n * MWP;
+            const uint32_t *v = sent + n * MWP + (n >> 5);
             const uint32_t ne = n_edges[row0 + n];
             const uint2 *out_edges = reinterpret_cast<const uint2 *>(edge) + edge_index[row0 + n];
             for (uint32_t e0 = 0; e0 < ne; e0 += 4) {
@@ -581,7 +586,7 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
                     for (int j = 0; j < MW; ++j) {
                         const int below = a == 0 ? MW - 1 : a - 1;
                         const uint32_t word = r ? (v[a] << r) | (v[below] >> (32 - r)) : v[a];
-                        if (word) atomicOr(&got[dst * MWP + j], word);
+                        if (word) atomicOr(&got[dst * MWP + (dst >> 5) + j], word);
                         a = a + 1 == MW ? 0 : a + 1;
                     }
                 }
@@ -598,7 +603,7 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
         for (int j = wave; j < MW; j += pack_waves) {
             for (int nb = 0; nb * 2 < sw; ++nb) {
                 const int slot = nb * 64 + lane;
-                const uint32_t word = slot < slots ? got[slot * MWP + j] : 0u;
+                const uint32_t word = slot < slots ? got[slot * MWP + (slot >> 5) + j] : 0u;
                 // lanes 0..31 and 32..63 each transpose their 32 x 32 bits: lane b of a half ends up
                 // with bit b of the half's 32 slots, i.e. one word of row 32 j + b
                 const uint32_t column = tile_transpose32(word, lane);
