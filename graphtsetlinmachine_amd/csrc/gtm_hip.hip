@@ -494,6 +494,7 @@ struct ScoreWs {
     uint32_t *tile_bitmap;    // [tiles per launch][C][tw]  (tile path, depth > 1)
     uint32_t *sent, *got;     // [tiles per launch][tw * 32 node slots][ceil(M / 32)]  (tile path, depth > 1)
     uint32_t *message_rows;   // [tiles per launch][M + 2][tw]  (tile path, depth > 1)
+    uint32_t *bit_start, *bit_cursor, *bit_clauses;  // [M + 1], [M], [C * MB]: the clauses of every message bit (tile path, depth > 1)
     size_t vector_words;      // words of sent (and of got)
     uint32_t *inc_t;          // [max(LA,MC)][C]
     uint32_t *bitmap_a;       // [batch][C][NC]
@@ -535,6 +536,9 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base,
         w.sent = (uint32_t *)take(w.vector_words * 4);
         w.got = (uint32_t *)take(w.vector_words * 4);
         w.message_rows = (uint32_t *)take(n_tiles * tile_message_rows(d.M) * tg->tw * 4);
+        w.bit_start = (uint32_t *)take(((size_t)d.M + 1) * 4);
+        w.bit_cursor = (uint32_t *)take((size_t)d.M * 4);
+        w.bit_clauses = (uint32_t *)take((size_t)d.C * d.MB * 4);
         w.bytes = off;
         return w;
     }
@@ -908,6 +912,12 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             }
         }
     }
+    if (fused_messages) {
+        // the clauses of every message bit, for the kernel that builds what the nodes send
+        hipLaunchKernelGGL(k_message_bit_index, dim3(1), dim3(BIT_INDEX_BLOCK), 0, st, s->hypervectors, d.C, d.MB, d.M,
+                           w.bit_start, w.bit_cursor, w.bit_clauses);
+        if (int rc = check_launch("message_bit_index")) return rc;
+    }
     static thread_local bool node_messages_lds_raised = false;
     if (!node_messages_lds_raised) {
         hipError_t e = hipFuncSetAttribute((const void *)k_tile_node_messages,
@@ -927,8 +937,8 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             // vectors in LDS when they fit, else three launches with the vectors in global memory
             if (fused_messages) {
                 hipLaunchKernelGGL(k_tile_messages_fused, dim3(tg.gpt, n_tiles), dim3(TILE_FUSED_MESSAGES_BLOCK),
-                                   fused_lds, st, w.tile_bitmap, d.C, tg, t0, g->number_of_graphs, d.M, MW, s->hypervectors,
-                                   d.MB, g->node_index, g->number_of_graph_nodes, g->number_of_graph_node_edges,
+                                   fused_lds, st, w.tile_bitmap, d.C, tg, t0, g->number_of_graphs, d.M, MW, w.bit_start,
+                                   w.bit_clauses, g->node_index, g->number_of_graph_nodes, g->number_of_graph_node_edges,
                                    g->edge_index, g->edge, g->total_edges > 0 ? 1 : 0, w.message_rows);
                 if (int rc = check_launch("tile_messages_fused")) return rc;
                 a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;

@@ -360,6 +360,74 @@ __device__ __forceinline__ uint32_t tile_transpose32(uint32_t v, int lane) {
 }
 
 
+// What a node sends (kernels.py:565-588) is the OR of the hypervector bits of the clauses true at
+// it.  Turned round: bit p of the vectors of 32 nodes is the OR of the truth words of the clauses
+// whose hypervector holds p - plain ORs of whole words, however many clauses are true, instead of
+// one atomic per (true clause, node, bit); 32 such words (bits 32 j .. 32 j + 31) transposed are
+// word j of the 32 nodes' vectors.  k_message_bit_index lists the clauses of every bit.
+
+constexpr int BIT_INDEX_BLOCK = 1024;
+
+// One block.  start[p] .. start[p + 1] index `clauses` for message bit p; `cursor` is M words of scratch.
+__global__ __launch_bounds__(BIT_INDEX_BLOCK) void k_message_bit_index(const uint32_t *__restrict__ hv, int C, int MB,
+                                                                       int M, uint32_t *start, uint32_t *cursor,
+                                                                       uint32_t *clauses) {
+    __shared__ uint32_t chunk_sum[BIT_INDEX_BLOCK];
+    const int tid = threadIdx.x;
+    for (int p = tid; p <= M; p += BIT_INDEX_BLOCK) start[p] = 0u;
+    for (int p = tid; p < M; p += BIT_INDEX_BLOCK) cursor[p] = 0u;
+    __syncthreads();
+    for (int i = tid; i < C * MB; i += BIT_INDEX_BLOCK) {
+        const uint32_t h = hv[i];
+        if (h < (uint32_t)M) atomicAdd(&start[h + 1], 1u);
+    }
+    __syncthreads();
+    // running sums of start[1 .. M]: a run of `per` entries per thread, then the runs' totals
+    const int per = (M + BIT_INDEX_BLOCK - 1) / BIT_INDEX_BLOCK;
+    const int first = 1 + tid * per, last = first + per < M + 1 ? first + per : M + 1;
+    uint32_t sum = 0u;
+    for (int p = first; p < last; ++p) sum += start[p];
+    chunk_sum[tid] = sum;
+    __syncthreads();
+    for (int off = 1; off < BIT_INDEX_BLOCK; off <<= 1) {
+        const uint32_t v = tid >= off ? chunk_sum[tid - off] : 0u;
+        __syncthreads();
+        chunk_sum[tid] += v;
+        __syncthreads();
+    }
+    uint32_t run = tid ? chunk_sum[tid - 1] : 0u;
+    for (int p = first; p < last; ++p) {
+        run += start[p];
+        start[p] = run;
+    }
+    __syncthreads();
+    // start[p + 1] now counts the entries of bits 0 .. p, so bit p's entries begin at start[p]
+    for (int i = tid; i < C * MB; i += BIT_INDEX_BLOCK) {
+        const uint32_t h = hv[i];
+        if (h < (uint32_t)M) clauses[start[h] + atomicAdd(&cursor[h], 1u)] = (uint32_t)(i / MB);
+    }
+}
+
+constexpr int MESSAGE_WORDS_AT_ONCE = 8;  // truth words a lane ORs per clause of its bit: independent loads in flight
+
+// word[u] = OR over the clauses that hold message bit p of word u of their truth rows (`rows`:
+// word 0 of clause 0's row, `tw` words per row), for u < n_words.
+__device__ __forceinline__ void message_bit_words(const uint32_t *__restrict__ rows, int tw, int n_words,
+                                                  const uint32_t *__restrict__ bit_start,
+                                                  const uint32_t *__restrict__ bit_clauses, int p, int M,
+                                                  uint32_t (&word)[MESSAGE_WORDS_AT_ONCE]) {
+#pragma unroll
+    for (int u = 0; u < MESSAGE_WORDS_AT_ONCE; ++u) word[u] = 0u;
+    if (p >= M || n_words <= 0) return;
+    const uint32_t from = bit_start[p], to = bit_start[p + 1];
+    for (uint32_t i = from; i < to; ++i) {
+        const uint32_t *row = rows + (int64_t)bit_clauses[i] * tw;
+#pragma unroll
+        for (int u = 0; u < MESSAGE_WORDS_AT_ONCE; ++u)
+            if (u < n_words) word[u] |= row[u];
+    }
+}
+
 // grid (ceil(tw / group), tiles); `group` consecutive words of every truth row of the tile per
 // block (a power of two <= 16: one cache line per clause), dynamic LDS 32 * group * (MW | 1) words.
 // Every word of sent is written (no clearing needed).
@@ -512,7 +580,7 @@ inline size_t tile_fused_messages_lds_bytes(const TileGeom &g, int MW) {
 
 __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fused(
     const uint32_t *__restrict__ bitmap, int C, TileGeom tg, int tile0, int G, int M, int MW,
-    const uint32_t *__restrict__ hv, int MB, const uint32_t *__restrict__ node_index,
+    const uint32_t *__restrict__ bit_start, const uint32_t *__restrict__ bit_clauses, const uint32_t *__restrict__ node_index,
     const uint32_t *__restrict__ n_nodes, const uint32_t *__restrict__ n_edges, const uint32_t *__restrict__ edge_index,
     const uint32_t *__restrict__ edge, int has_edges, uint32_t *__restrict__ rows) {
     extern __shared__ uint32_t lds[];
@@ -531,34 +599,26 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
     for (int i = tid; i < 2 * VEC; i += NT) lds[i] = 0u;
     __syncthreads();
 
-    // 1. what every node slot sends
+    // 1. what every node slot sends: a half-wave takes 32 message bits and up to 8 words of the graph's
+    // truth rows at a time (lane = bit: the OR of the truth words of the bit's clauses), transposes,
+    // and lane = node stores word j of its vector - each word once, no atomics
     if (nodes > 0) {
+        constexpr int WB = MESSAGE_WORDS_AT_ONCE;
         const uint32_t *truth = bitmap + (int64_t)tile_local * C * tw + w_first;
         const int used = (nodes + 31) >> 5;  // words of a truth row that can hold a true node
-        constexpr int AHEAD = 4;
-        for (int i0 = tid; i0 < C * used; i0 += AHEAD * NT) {
-            uint32_t words[AHEAD], h01[AHEAD][2];  // the clause's first two hypervector bits travel with the word
-            int cs[AHEAD], wls[AHEAD];
+        const int hl = lane & 31, half = lane >> 5;
+        const int blocks_w = (used + WB - 1) / WB, tasks = MW * blocks_w;
+        for (int t0 = wave * 2; t0 < tasks; t0 += NT / 32) {
+            const int t = t0 + half;
+            const bool valid = t < tasks;
+            const int j = valid ? t / blocks_w : 0, wl0 = valid ? (t - j * blocks_w) * WB : 0;
+            const int n_words = valid ? (used - wl0 < WB ? used - wl0 : WB) : 0;
+            uint32_t word[WB];
+            message_bit_words(truth + wl0, tw, n_words, bit_start, bit_clauses, j * 32 + hl, M, word);
 #pragma unroll
-            for (int u = 0; u < AHEAD; ++u) {
-                const int i = i0 + u * NT;
-                const bool in_range = i < C * used;
-                cs[u] = in_range ? i / used : 0;
-                wls[u] = i - cs[u] * used;
-                words[u] = in_range ? truth[(int64_t)cs[u] * tw + wls[u]] : 0u;
-                h01[u][0] = hv[(int64_t)cs[u] * MB];
-                h01[u][1] = MB > 1 ? hv[(int64_t)cs[u] * MB + 1] : 0u;
-            }
-#pragma unroll
-            for (int u = 0; u < AHEAD; ++u) {
-                const uint32_t word = words[u];
-                if (!word) continue;
-                for (int j = 0; j < MB; ++j) {
-                    const uint32_t h = j < 2 ? h01[u][j] : hv[(int64_t)cs[u] * MB + j];
-                    const uint32_t bit = 1u << (h & 31);
-                    uint32_t *column = sent + (wls[u] * 32) * MWP + wls[u] + (h >> 5);
-                    for (uint32_t m = word; m; m &= m - 1) atomicOr(&column[(__ffs(m) - 1) * MWP], bit);
-                }
+            for (int u = 0; u < WB; ++u) {
+                const uint32_t column = tile_transpose32(word[u], lane);
+                if (u < n_words) sent[((wl0 + u) * 32 + hl) * MWP + (wl0 + u) + j] = column;
             }
         }
     }
