@@ -912,8 +912,9 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             }
         }
     }
-    if (fused_messages) {
-        // the clauses of every message bit, for the kernel that builds what the nodes send
+    const bool by_bit = !getenv("GTM_NODE_MESSAGES_BY_ATOMICS");  // tuning aid: the earlier kernel
+    if (fused_messages || by_bit) {
+        // the clauses of every message bit, for the kernels that build what the nodes send
         hipLaunchKernelGGL(k_message_bit_index, dim3(1), dim3(BIT_INDEX_BLOCK), 0, st, s->hypervectors, d.C, d.MB, d.M,
                            w.bit_start, w.bit_cursor, w.bit_clauses);
         if (int rc = check_launch("message_bit_index")) return rc;
@@ -946,6 +947,12 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                 if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1, st)) return rc;
                 continue;
             }
+            if (by_bit)
+                hipLaunchKernelGGL(k_tile_node_messages_by_bit,
+                                   dim3((MW + NODE_MESSAGES_BY_BIT_WAVES - 1) / NODE_MESSAGES_BY_BIT_WAVES, n_tiles),
+                                   dim3(64 * NODE_MESSAGES_BY_BIT_WAVES), 0, st, w.tile_bitmap, d.C, tg.tw, w.bit_start,
+                                   w.bit_clauses, d.M, MW, w.sent);
+            else
             hipLaunchKernelGGL(k_tile_node_messages, dim3((tg.tw + group - 1) / group, n_tiles),
                                dim3(TILE_MESSAGES_BLOCK), ((size_t)32 * group * (MW | 1) + group) * 4, st, w.tile_bitmap, d.C, tg.tw,
                                group, s->hypervectors, d.MB, MW, w.sent);

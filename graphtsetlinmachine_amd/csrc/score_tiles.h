@@ -428,6 +428,76 @@ __device__ __forceinline__ void message_bit_words(const uint32_t *__restrict__ r
     }
 }
 
+// What the node slots of a tile send, vectors in global memory (graphs too big for the kernel
+// below).  A wave takes 32 message bits (word j of every vector), lane = word of the tile's truth
+// rows: for each bit the rows of the bit's clauses are ORed (whole rows, coalesced; the clause
+// numbers come in by one load per bit and are handed round with readlane), the 32 resulting rows
+// are transposed inside each lane, 32 x 32 bits, and the lane stores word j of its 32 slots.
+// grid (ceil(MW / waves per block), tiles).  Every word of sent is written (no clearing needed).
+constexpr int NODE_MESSAGES_BY_BIT_WAVES = 4;
+
+__global__ __launch_bounds__(64 * NODE_MESSAGES_BY_BIT_WAVES) void k_tile_node_messages_by_bit(
+    const uint32_t *__restrict__ bitmap, int C, int tw, const uint32_t *__restrict__ bit_start,
+    const uint32_t *__restrict__ bit_clauses, int M, int MW, uint32_t *__restrict__ sent) {
+    __shared__ uint32_t stage_of_wave[NODE_MESSAGES_BY_BIT_WAVES][32][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = blockIdx.x * NODE_MESSAGES_BY_BIT_WAVES + wave, tile = blockIdx.y;
+    if (j >= MW) return;  // the block has no barrier
+    uint32_t(*stage)[64] = stage_of_wave[wave];
+    const uint32_t *rows = bitmap + (int64_t)tile * C * tw;
+    // lane i <= 32 holds where the clauses of bit 32 j + i begin (bits past M: nothing)
+    const int p_of_lane = 32 * j + lane < M ? 32 * j + lane : M;
+    const uint32_t start_of_lane = lane <= 32 ? bit_start[p_of_lane] : 0u;
+    for (int w0 = 0; w0 < tw; w0 += 64) {
+        const int w = w0 + lane;
+        const bool active = w < tw;
+        const uint32_t *col = rows + (active ? w : 0);
+#pragma unroll 1
+        for (int i = 0; i < 32; ++i) {
+            const uint32_t from = __builtin_amdgcn_readlane(start_of_lane, i);
+            const uint32_t to = __builtin_amdgcn_readlane(start_of_lane, i + 1);
+            uint32_t acc = 0u;
+            for (uint32_t k0 = from; k0 < to; k0 += 64u) {
+                const uint32_t n = to - k0 < 64u ? to - k0 : 64u;
+                const uint32_t clause_of_lane = (uint32_t)lane < n ? bit_clauses[k0 + lane] : 0u;
+                for (uint32_t e = 0; e < n; e += 8u) {
+                    uint32_t v[8];
+#pragma unroll
+                    for (uint32_t u = 0; u < 8u; ++u) {
+                        const uint32_t c = __builtin_amdgcn_readlane(clause_of_lane, (e + u) & 63u);
+                        v[u] = e + u < n ? col[(int64_t)c * tw] : 0u;
+                    }
+#pragma unroll
+                    for (uint32_t u = 0; u < 8u; ++u) acc |= v[u];
+                }
+            }
+            stage[i][lane] = active ? acc : 0u;
+        }
+        // (a wave's LDS writes are visible to its own later reads: same wave, in order)
+        uint32_t a[32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) a[i] = stage[i][lane];
+        // a[i] bit b -> a[b] bit i: blocks of s x s bits swap across the diagonal, s = 16 .. 1
+#pragma unroll
+        for (int s = 16; s >= 1; s >>= 1) {
+            const uint32_t m = s == 16 ? 0x0000FFFFu : s == 8 ? 0x00FF00FFu : s == 4 ? 0x0F0F0F0Fu : s == 2 ? 0x33333333u : 0x55555555u;
+#pragma unroll
+            for (int i = 0; i < 32; ++i)
+                if ((i & s) == 0) {
+                    const uint32_t t = ((a[i] >> s) ^ a[i + s]) & m;
+                    a[i + s] ^= t;
+                    a[i] ^= t << s;
+                }
+        }
+        if (active) {
+            uint32_t *out = sent + ((int64_t)tile * tw + w) * 32 * MW + j;
+#pragma unroll
+            for (int b = 0; b < 32; ++b) out[(int64_t)b * MW] = a[b];
+        }
+    }
+}
+
 // grid (ceil(tw / group), tiles); `group` consecutive words of every truth row of the tile per
 // block (a power of two <= 16: one cache line per clause), dynamic LDS 32 * group * (MW | 1) words.
 // Every word of sent is written (no clearing needed).

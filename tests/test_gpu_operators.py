@@ -313,15 +313,17 @@ DEEP_TILE_SHAPES = [
 
 @pytest.mark.parametrize("shape", DEEP_TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
 @pytest.mark.parametrize("message_density", [0.0, 0.01, 0.1])
-@pytest.mark.parametrize("messages", ["graph-per-workgroup", "three-launches"])
+@pytest.mark.parametrize("messages", ["graph-per-workgroup", "three-launches", "three-launches-atomics"])
 def test_tile_scoring_with_message_layers(shape, message_density, messages, monkeypatch):
     """gtm_score with message layers on literal-major tiles == oracle == the bitmap path, with the
     message rows built by one workgroup per graph (where the shape allows) and by the three
     launches that keep the vectors in global memory."""
     from tests.gpu_harness import Device
 
-    if messages == "three-launches":
+    if messages != "graph-per-workgroup":
         monkeypatch.setenv("GTM_NO_FUSED_MESSAGES", "1")
+    if messages == "three-launches-atomics":
+        monkeypatch.setenv("GTM_NODE_MESSAGES_BY_ATOMICS", "1")
 
     graphs = helpers.random_graphs(shape["seed"], **shape["g"])
     m = dict(shape["m"])
