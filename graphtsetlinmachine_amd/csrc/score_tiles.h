@@ -666,7 +666,7 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
     const int w_first = gj * sw;        // the graph's first word of a tile row
     uint32_t *out = rows + (int64_t)tile_local * (M + 2) * tw;
 
-    for (int i = tid; i < 2 * VEC; i += NT) lds[i] = 0u;
+    for (int i = tid; i < VEC; i += NT) got[i] = 0u;  // (every word of sent that is read is stored first)
     __syncthreads();
 
     // 1. what every node slot sends: a half-wave takes 32 message bits and up to 8 words of the graph's
