@@ -1457,7 +1457,49 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
             }
         }
         unsigned long long nz = __ballot(any_bit(acc));
+        // Phase 2 costs a memory round trip per 8 surviving slots, ANDing the rows of all the clause's
+        // literals one per 8 literals: when more slots survive than the clause has literals (its rarest
+        // literals hold nearly everywhere: negated ones, mostly), the rows are walked instead, as
+        // k_tile_layer does (row l belongs to literal l; unused reads take the all-ones row).
+        bool walk = false;
         if ((header & 0x100u) && nz != 0) {
+            int survivors = 0, literals = __popc(include0);
+#pragma unroll
+            for (int u = 0; u < LW; ++u) survivors += __popc(acc.w[u]);
+            for (int w0 = 64; w0 < LA; w0 += 64) literals += w0 + lane < LA ? __popc(record[8 + w0 + lane]) : 0;
+            for (int off = 32; off > 0; off >>= 1) {
+                survivors += __shfl_xor(survivors, off);
+                literals += __shfl_xor(literals, off);
+            }
+            walk = survivors > literals;
+        }
+        if (walk) {
+            const uint32_t row_bytes = (uint32_t)tw * 4u, ones = (uint32_t)(tg.rows - 1);
+            for (int w0 = 0; w0 < LA; w0 += 64) {
+                const uint32_t include = w0 == 0 ? include0 : (w0 + lane < LA ? record[8 + w0 + lane] : 0u);
+                unsigned long long has = __ballot(include != 0u);
+                while (has) {
+                    const int L = __ffsll((long long)has) - 1;
+                    has &= has - 1;
+                    uint32_t m = __builtin_amdgcn_readlane(include, L);
+                    const uint32_t base = (uint32_t)(w0 + L) * 32u;
+                    while (m) {
+                        LaneWords<LW> r[8];
+#pragma unroll
+                        for (int q = 0; q < 8; ++q) {
+                            const uint32_t lit = m ? base + (uint32_t)__builtin_ctz(m) : ones;
+                            m &= m - 1u;
+                            r[q].load(col + (size_t)lit * row_bytes);
+                        }
+#pragma unroll
+                        for (int q = 0; q < 8; ++q)
+#pragma unroll
+                            for (int u = 0; u < LW; ++u) acc.w[u] &= r[q].w[u];
+                    }
+                }
+            }
+            nz = __ballot(any_bit(acc));
+        } else if ((header & 0x100u) && nz != 0) {
             for (int w0 = 0; w0 < LA; w0 += 64) {
                 const bool in_row = w0 + lane < LA;
                 const uint32_t include = w0 == 0 ? include0 : (in_row ? record[8 + w0 + lane] : 0u);

@@ -264,7 +264,8 @@ def test_tile_scoring_equals_oracle(shape, density):
 
 
 @pytest.mark.parametrize("hv_size,sizes", [
-    (64, [40, 0, 2, 64, 1, 50, 3, 1, 2, 5]), (128, [361, 1, 300, 0, 2, 361, 3, 1]), (256, [100, 1, 31, 2, 90, 1, 3, 2, 1])])
+    (64, [40, 0, 2, 64, 1, 50, 3, 1, 2, 5]), (128, [361, 1, 300, 0, 2, 361, 3, 1]), (256, [100, 1, 31, 2, 90, 1, 3, 2, 1]),
+    (80, [70, 1, 0, 2, 33, 64, 1, 3]), (1100, [40, 1, 2, 35, 0, 1])])  # 5 and 69 literal words per node: the other two-phase kernel
 @pytest.mark.parametrize("depth", [1, 2])
 def test_tile_scoring_with_clauses_of_negated_literals(hv_size, sizes, depth):
     """Clauses that include 16 to 40 negated literals and nothing else: each
@@ -278,8 +279,13 @@ def test_tile_scoring_with_clauses_of_negated_literals(hv_size, sizes, depth):
     model = helpers.random_model(41, cfg, depth, include_density=0.0, message_density=0.0)
     rng = np.random.default_rng(41)
     top = cfg.state_bits - 1
+    used = np.unique(graphs.hypervectors)  # the bits that symbols set: their negations are what tells nodes apart
     for c in range(cfg.clauses):
-        for k in rng.choice(hv_size, size=int(rng.integers(16, 41)), replace=False):
+        n = int(rng.integers(16, 41))
+        bits = rng.permutation(used)[:n]
+        if len(bits) < n:
+            bits = np.concatenate([bits, rng.choice(np.setdiff1d(np.arange(hv_size), used), size=n - len(bits), replace=False)])
+        for k in bits:
             lit = hv_size + int(k)
             model.ta_state[c, lit // 32, top] |= np.uint32(1 << (lit % 32))
     G = graphs.number_of_graphs
