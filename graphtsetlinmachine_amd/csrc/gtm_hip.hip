@@ -801,7 +801,8 @@ int launch_two_phase_wide_as(const TileLayerArgs &a, int n_tiles, int LA, hipStr
         splits = splits < 1 ? 1 : (splits > 16 ? 16 : splits);
     }
     profile_start(LAST ? "k_tile_two_phase_wide<score>" : "k_tile_two_phase_wide<layer0>", st);
-    hipLaunchKernelGGL((k_tile_two_phase_wide<NW, LW, SRC, LAST>), dim3(n_tiles, splits), dim3(NW * 64), lds, st, a, LA);
+    hipLaunchKernelGGL((k_tile_two_phase_wide<NW, LW, SRC, LAST>), dim3((unsigned)((n_tiles + 7) / 8 * 8 * splits)),
+                       dim3(NW * 64), lds, st, a, LA, n_tiles, splits);
     if (int rc = check_launch("tile_two_phase_wide")) return rc;
     profile_stop(st);
     return GTM_OK;

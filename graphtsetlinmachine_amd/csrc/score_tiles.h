@@ -1374,12 +1374,19 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
 // above; in phase 2 the surviving node slots are walked on the scalar unit, 8 at
 // a time, and for each one lane w compares include word w with the node's
 // literal word w (one coalesced load per node and 64 words).  With the rows
-// read in place nothing ties a tile to one workgroup, so gridDim.y workgroups
+// read in place nothing ties a tile to one workgroup, so several workgroups
 // share a tile's clauses (truth rows only: the votes of LAST need one
 // workgroup per tile).
 template <int NWAVES, int LW, int SRC, bool LAST>
-__global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerArgs a, int LA) {
+__global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerArgs a, int LA, int n_tiles, int splits) {
     extern __shared__ uint32_t lds[];
+    // Workgroups go to the 8 XCDs in turn, and each XCD has its own L2: the workgroups that share a
+    // tile (its rows are read in place, again and again) are given to one XCD, one after the other,
+    // so that the few tiles an XCD works on at a time stay in its L2.  1-D grid of
+    // ceil(n_tiles / 8) * 8 * splits workgroups.
+    const int xcd = blockIdx.x & 7, turn = blockIdx.x >> 3;
+    const int split = turn % splits, tile_of_launch = (turn / splits) * 8 + xcd;
+    if (tile_of_launch >= n_tiles) return;
     const TileGeom &tg = a.tg;
     const int tw = tg.tw, C = a.C, K = a.K;
     constexpr int NT = NWAVES * 64;
@@ -1388,11 +1395,11 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
     int32_t *sums = (int32_t *)(lds + (size_t)n_rows_lds * tw + TILE_LDS_PAD_WORDS);
     uint32_t *first_node = (uint32_t *)(sums + tg.gpt * K);  // [gpt] row of X of each graph's node 0
     uint32_t *node_count = first_node + tg.gpt;              // [gpt]
-    const int tile = a.tile0 + blockIdx.x;
+    const int tile = a.tile0 + tile_of_launch;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    uint32_t *bitmap = a.bitmap + (int64_t)blockIdx.x * C * tw;
+    uint32_t *bitmap = a.bitmap + (int64_t)tile_of_launch * C * tw;
 
     if (SRC == ROWS_STAGED) {
         const uint4 *src = reinterpret_cast<const uint4 *>(a.tiles + (int64_t)tile * tg.rows * tw);
@@ -1424,37 +1431,38 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
     };
     auto entry_of = [](const Packed8 &rec, int i) { return ((rec.v[i >> 1] >> ((i & 1) * 16)) & 0xFFFFu) << 4; };
 
-    const int c_step = NWAVES * gridDim.y;
-    const int c_first = wave + NWAVES * blockIdx.y;
+    const int c_step = NWAVES * splits;
+    const int c_first = wave + NWAVES * split;
     const int valid = c_first < C ? c_first : 0;
-    Packed8 next = *reinterpret_cast<const Packed8 *>(a.lists + (int64_t)valid * a.stride);
-    for (int c = c_first; c < C; c += c_step) {
-        const uint32_t *record = a.lists + (int64_t)c * a.stride;
-        const Packed8 rec = next;
-        next = *reinterpret_cast<const Packed8 *>(a.lists + (int64_t)(c + c_step < C ? c + c_step : valid) * a.stride);
+    struct Rows {
+        LaneWords<LW> r[15];
+    };
+    // phase 1, first half: the reads of the clause's 7 or 15 rows are sent off
+    auto issue = [&](const Packed8 &rec, Rows &rows) {
+        if ((rec.v[0] & 0xFFu) > 7u) {
+#pragma unroll
+            for (int i = 0; i < 15; ++i) rows.r[i].load(col + entry_of(rec, i + 1));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 7; ++i) rows.r[i].load(col + entry_of(rec, i + 1));
+        }
+    };
+    // the rest of the clause
+    auto finish = [&](int c, const Packed8 &rec, const uint32_t *record, uint32_t include0, const Rows &rows) {
         const uint32_t header = rec.v[0] & 0xFFFFu;
-        // the first 64 include words travel with the rows (phase 2 would otherwise wait for them alone)
-        const uint32_t include0 = lane < LA ? record[8 + lane] : 0u;
         LaneWords<LW> acc;
 #pragma unroll
         for (int u = 0; u < LW; ++u) acc.w[u] = active ? 0xFFFFFFFFu : 0u;
-        {
-            LaneWords<LW> r[15];
-            if ((header & 0xFFu) > 7u) {
+        if ((header & 0xFFu) > 7u) {
 #pragma unroll
-                for (int i = 0; i < 15; ++i) r[i].load(col + entry_of(rec, i + 1));
+            for (int i = 0; i < 15; ++i)
 #pragma unroll
-                for (int i = 0; i < 15; ++i)
+                for (int u = 0; u < LW; ++u) acc.w[u] &= rows.r[i].w[u];
+        } else {
 #pragma unroll
-                    for (int u = 0; u < LW; ++u) acc.w[u] &= r[i].w[u];
-            } else {
+            for (int i = 0; i < 7; ++i)
 #pragma unroll
-                for (int i = 0; i < 7; ++i) r[i].load(col + entry_of(rec, i + 1));
-#pragma unroll
-                for (int i = 0; i < 7; ++i)
-#pragma unroll
-                    for (int u = 0; u < LW; ++u) acc.w[u] &= r[i].w[u];
-            }
+                for (int u = 0; u < LW; ++u) acc.w[u] &= rows.r[i].w[u];
         }
         unsigned long long nz = __ballot(any_bit(acc));
         // Phase 2 costs a memory round trip per 8 surviving slots, ANDing the rows of all the clause's
@@ -1538,15 +1546,38 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
         }
         if (!LAST) {
             if (active) acc.store(reinterpret_cast<char *>(bitmap + (int64_t)c * tw + lane * LW));
-            continue;
+            return;
         }
-        if (nz == 0) continue;
+        if (nz == 0) return;
         const int32_t *weights_of_clause = a.wt + (int64_t)c * K;
         const unsigned long long gm = __ballot(lane < tg.gpt && ((nz >> my_shift) & slot_lanes) != 0);
         for (int p = lane; p < pairs; p += 64) {
             int j = p / K, k = p - j * K;
             if ((gm >> j) & 1ull) atomicAdd(&sums[p], weights_of_clause[k]);
         }
+        };
+    // Two clauses of a wave are under way at a time: the rows of both are requested before either is
+    // ANDed (rows read in place come from L2 or further: a clause is a chain of memory round trips).
+    // Without a second clause the first is repeated and the result dropped.
+    const int64_t pair_step = 2 * (int64_t)c_step;
+    Packed8 next_a = *reinterpret_cast<const Packed8 *>(a.lists + (int64_t)valid * a.stride);
+    Packed8 next_b = *reinterpret_cast<const Packed8 *>(a.lists + (int64_t)(c_first + c_step < C ? c_first + c_step : valid) * a.stride);
+    for (int c = c_first; c < C; c += 2 * c_step) {
+        const bool has_b = c + c_step < C;
+        const int cb = has_b ? c + c_step : c;
+        const uint32_t *record_a = a.lists + (int64_t)c * a.stride, *record_b = a.lists + (int64_t)cb * a.stride;
+        const Packed8 rec_a = next_a, rec_b = next_b;
+        const int64_t na = c + pair_step < C ? c + pair_step : valid, nb = c + pair_step + c_step < C ? c + pair_step + c_step : na;
+        next_a = *reinterpret_cast<const Packed8 *>(a.lists + na * a.stride);
+        next_b = *reinterpret_cast<const Packed8 *>(a.lists + nb * a.stride);
+        // the first 64 include words travel with the rows (phase 2 would otherwise wait for them alone)
+        const uint32_t include0_a = lane < LA ? record_a[8 + lane] : 0u;
+        const uint32_t include0_b = lane < LA ? record_b[8 + lane] : 0u;
+        Rows rows_a, rows_b;
+        issue(rec_a, rows_a);
+        issue(rec_b, rows_b);
+        finish(c, rec_a, record_a, include0_a, rows_a);
+        if (has_b) finish(cb, rec_b, record_b, include0_b, rows_b);
     }
     if (!LAST) return;
     __syncthreads();
