@@ -1508,38 +1508,63 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
             }
             nz = __ballot(any_bit(acc));
         } else if ((header & 0x100u) && nz != 0) {
+            // Phase 2: the surviving slots, wherever in the wave they sit, are taken 8 at a time (one
+            // memory round trip per 8): a cursor on the scalar unit walks the lanes that hold some, the
+            // words of such a lane and the bits of such a word.
             for (int w0 = 0; w0 < LA; w0 += 64) {
                 const bool in_row = w0 + lane < LA;
                 const uint32_t include = w0 == 0 ? include0 : (in_row ? record[8 + w0 + lane] : 0u);
                 unsigned long long live = __ballot(any_bit(acc));
-                while (live) {
-                    const int L = __ffsll((long long)live) - 1;
-                    live &= live - 1;
-#pragma unroll
-                    for (int u = 0; u < LW; ++u) {
-                        uint32_t word = __builtin_amdgcn_readlane(acc.w[u], L);
-                        const int tile_word = L * LW + u;                 // word of the tile row
-                        const int gj = tile_word / tg.slot_words;         // graph of the tile
-                        const int node0 = (tile_word - gj * tg.slot_words) * 32;
-                        if (node_count[gj] == 0u) continue;               // a graph without nodes keeps its bit
-                        const uint32_t *x = a.X + ((int64_t)first_node[gj] + node0) * LA + w0 + (in_row ? lane : 0);
-                        uint32_t cleared = 0;
-                        while (word) {
-                            int bit[8];
-#pragma unroll
-                            for (int q = 0; q < 8; ++q) {
-                                bit[q] = word ? __builtin_ctz(word) : -1;
-                                word &= word - 1;
-                            }
-                            uint32_t xs[8];
-#pragma unroll
-                            for (int q = 0; q < 8; ++q) xs[q] = x[(int64_t)(bit[q] < 0 ? 0 : bit[q]) * LA];
-#pragma unroll
-                            for (int q = 0; q < 8; ++q)
-                                if (bit[q] >= 0 && __ballot((include & ~xs[q]) != 0) != 0) cleared |= 1u << bit[q];
+                int at_lane = 0, at_word = LW, next_word = LW;
+                uint32_t bits = 0u;
+                const uint32_t *x_of_word = a.X;  // literal words w0 + lane of the node at bit 0 of the cursor's word
+                // the next surviving slot as lane | word << 8 | bit << 16, or -1
+                auto next_slot = [&]() {
+                    while (bits == 0u) {
+                        if (next_word >= LW) {
+                            if (live == 0ull) return -1;
+                            at_lane = __ffsll((long long)live) - 1;
+                            live &= live - 1;
+                            next_word = 0;
                         }
-                        if (lane == L) acc.w[u] &= ~cleared;
+                        uint32_t word = 0u;
+#pragma unroll
+                        for (int u = 0; u < LW; ++u)
+                            if (u == next_word) word = __builtin_amdgcn_readlane(acc.w[u], at_lane);
+                        at_word = next_word++;
+                        const int tile_word = at_lane * LW + at_word;       // word of the tile row
+                        const int gj = tile_word / tg.slot_words;           // graph of the tile
+                        const int node0 = (tile_word - gj * tg.slot_words) * 32;
+                        // (LDS reads at a wave-uniform index: readfirstlane keeps the cursor on the scalar unit)
+                        if (__builtin_amdgcn_readfirstlane(node_count[gj]) == 0u) word = 0u;  // a graph without nodes keeps its bit
+                        x_of_word = a.X + ((int64_t)__builtin_amdgcn_readfirstlane(first_node[gj]) + node0) * LA + w0 +
+                                    (in_row ? lane : 0);
+                        bits = word;
                     }
+                    const int b = __builtin_ctz(bits);
+                    bits &= bits - 1u;
+                    return at_lane | at_word << 8 | b << 16;
+                };
+                for (;;) {
+                    int slot[8];
+                    uint32_t xs[8];
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        slot[q] = next_slot();
+                        const uint32_t *x = slot[q] >= 0 ? x_of_word + (int64_t)(slot[q] >> 16) * LA : a.X;
+                        xs[q] = *x;
+                    }
+                    if (slot[0] < 0) break;
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        if (slot[q] < 0) continue;
+                        if (__ballot((include & ~xs[q]) != 0u) == 0ull) continue;
+                        const uint32_t keep = ~(1u << (slot[q] >> 16));
+#pragma unroll
+                        for (int u = 0; u < LW; ++u)
+                            if (lane == (slot[q] & 0xFF) && u == ((slot[q] >> 8) & 0xFF)) acc.w[u] &= keep;
+                    }
+                    if (slot[7] < 0) break;
                 }
             }
             nz = __ballot(any_bit(acc));
