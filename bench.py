@@ -24,9 +24,17 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 VALU_PEAK_LANE_OPS = 256 * 64 * 2.4e9  # 32-bit integer lane operations per second
 
-# HBM bytes per graph that the scoring kernel moves on the convolutional workload, from rocprofv3 --pmc runs
-# (FETCH_SIZE x 2 KiB, the factor a 256 MiB copy kernel calibrates, + WRITE_SIZE x 1 KiB, over 10,000 graphs).
-MEASURED_TRAFFIC_BYTES_PER_GRAPH = {"convolutional_images": (131715.6 * 2 + 406.3) * 1024 / 10000}
+# Hardware counters of the scoring kernel on the convolutional workload (10,000 graphs per launch, state after
+# one epoch), from rocprofv3 --pmc runs of this file; the summaries and the commands are under profiles/.
+# FETCH_SIZE counts 2 KiB per unit and WRITE_SIZE 1 KiB per unit on this part (a 256 MiB copy kernel reads
+# 131,089 and writes 262,144).  valu_busy = SQ_ACTIVE_INST_VALU x 4 / SQ_BUSY_CU_CYCLES.  The figures belong
+# to the kernel as of `commit`; a run whose kernel differs reports them as stale by that name.
+MEASURED_COUNTERS = {
+    "convolutional_images": {
+        "kernel": "k_tile_two_phase<score>", "commit": "3237649",
+        "fetch_units": 131715.6, "write_units": 406.3, "valu_busy": 0.59, "graphs": 10000,
+    },
+}
 
 
 def parse():
@@ -41,6 +49,10 @@ def parse():
     p.add_argument("--cpu-sample", type=int, default=None, help="graphs timed on the CPU oracle")
     p.add_argument("--no-cpu", action="store_true")
     p.add_argument("--only-main", action="store_true", help="skip the short runs of the other four configurations")
+    p.add_argument("--one-state", action="store_true", help="time the kernel on the headline state only")
+    p.add_argument("--save-state", default="", help="write the trained model to this .npz file after the run")
+    p.add_argument("--load-state", default="", help="score a model saved by --save-state instead of training one "
+                   "(the process then runs the scoring path only: what a profiler should see)")
     return p.parse_args()
 
 
@@ -147,6 +159,33 @@ def mean_included_literals(tm):
     return float(np.unpackbits(plane.view(np.uint8)).sum()) / tm.number_of_clauses
 
 
+def time_scoring(tm, test, steps, warmup, graphs):
+    """`steps` timed passes of gtm_score over the resident test graphs after `warmup` untimed ones."""
+    import torch
+
+    from graphtsetlinmachine_amd import _abi
+
+    for _ in range(warmup):
+        tm.score_device(test)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    _abi.call("gtm_profile_enable", 1)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        sums = tm.score_device(test)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_name, launches, kernel_total_ms = read_kernel_profile()
+    _abi.call("gtm_profile_enable", 0)
+    return {
+        "wall": wall, "event_ms": start.elapsed_time(stop) / steps, "kernel": kernel_name, "launches": launches,
+        "kernel_ms": kernel_total_ms / max(launches, 1), "graphs_per_launch": graphs * steps / max(launches, 1),
+        "sums": sums.cpu().numpy().reshape(graphs, -1),
+    }
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -157,65 +196,102 @@ def main():
     import numpy as np
     import torch
 
-    from graphtsetlinmachine_amd import _abi, workloads
+    from graphtsetlinmachine_amd import workloads
     from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
 
     torch.cuda.set_device(0)
     t0 = time.time()
     wl = workloads.BUILDERS[args.workload](n_train=args.train_graphs, n_test=args.graphs)
     t_data = time.time() - t0
+    test = wl.graphs_test
+    n_nodes = int(test.max_number_of_graph_nodes)
 
     np.random.seed(42)
     tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
-    # training throughput (also produces the state that inference is timed on)
-    tm.fit(wl.graphs_train, wl.Y_train, epochs=0, incremental=True)  # allocate + upload only
-    torch.cuda.synchronize()
-    t0 = time.time()
-    tm.fit(wl.graphs_train, wl.Y_train, epochs=args.train_epochs, incremental=True)
-    torch.cuda.synchronize()
-    t_train = time.time() - t0
-    train_gps = args.train_graphs * args.train_epochs / t_train
-
-    test = wl.graphs_test
+    if args.load_state:
+        tm.load(fname=args.load_state)
+        args.one_state, args.train_epochs = True, 0
+    else:
+        tm.fit(wl.graphs_train, wl.Y_train, epochs=0, incremental=True)  # allocate + upload only
     tm.score_device(test)  # uploads the test graphs
-    for _ in range(args.warmup):
-        tm.score_device(test)
     torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    _abi.call("gtm_profile_enable", 1)
-    t0 = time.perf_counter()
-    start.record()
-    for _ in range(args.steps):
-        sums = tm.score_device(test)
-    stop.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    kernel_name, launches, kernel_total_ms = read_kernel_profile()
-    _abi.call("gtm_profile_enable", 0)
-    ms_per_step = wall * 1000.0 / args.steps
-    event_ms = start.elapsed_time(stop) / args.steps
-    value = args.graphs * args.steps / wall
-
-    sums_host = sums.cpu().numpy().reshape(args.graphs, -1)
-    accuracy = float((sums_host.argmax(axis=1) == wl.Y_test).mean())
-
-    # roofline of the clause-evaluation kernel: algorithmic bytes / kernel time
-    n_nodes = int(test.max_number_of_graph_nodes)
     la = tm.number_of_ta_chunks
     b_eval = eval_bytes_per_graph(n_nodes, la, tm.number_of_clauses, (n_nodes - 1) // 32 + 1)
-    # every launch of the kernel inside the timed region; a step may split its graphs over several launches
-    kernel_ms = kernel_total_ms / max(launches, 1)
-    graphs_per_launch = args.graphs * args.steps / max(launches, 1)
+
+    def frac_of(run):
+        return b_eval * run["graphs_per_launch"] / (run["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+
+    def c_oracle_agrees(run):
+        from oracle import gtm_oracle_c as oc
+
+        model = oracle_twin(tm, n_nodes)
+        return bool(np.array_equal(oc.score(model, test, threads=max(1, min(16, oc.threads_available()))), run["sums"]))
+
+    def state_entry(label, run, checked):
+        return {"state": label, "frac": round(frac_of(run), 4), "kernel_ms": round(run["kernel_ms"], 4),
+                "graphs_per_s": round(args.graphs * args.steps / run["wall"], 1),
+                "mean_included_literals": round(mean_included_literals(tm), 2),
+                "class_sums_equal_c_oracle": checked}
+
+    # The include density of the state decides how much the sparse kernel can skip, so the kernel is
+    # timed on three states of the same run: early in the first epoch, after the configured epochs
+    # (the headline, `value`), and after two epochs more.
+    states = []
+    early = min(5000, args.train_graphs // 2)
+    t_train = 0.0
+    if early > 0 and args.train_epochs >= 1 and not args.one_state:
+        t0 = time.time()
+        tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True, examples=(0, early))
+        torch.cuda.synchronize()
+        t_train += time.time() - t0
+        run = time_scoring(tm, test, args.steps, args.warmup, args.graphs)
+        states.append(state_entry("after %d training graphs" % early, run, None if args.no_cpu else c_oracle_agrees(run)))
+        t0 = time.time()
+        tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True, examples=(early, args.train_graphs - early))
+        if args.train_epochs > 1:
+            tm.fit(wl.graphs_train, wl.Y_train, epochs=args.train_epochs - 1, incremental=True)
+    elif not args.load_state:
+        t0 = time.time()
+        tm.fit(wl.graphs_train, wl.Y_train, epochs=args.train_epochs, incremental=True)
+    else:
+        t0 = time.time()
+    torch.cuda.synchronize()
+    t_train += time.time() - t0
+    train_gps = args.train_graphs * args.train_epochs / max(t_train, 1e-9)
+    if args.save_state:
+        tm.save(args.save_state)
+
+    main_run = time_scoring(tm, test, args.steps, args.warmup, args.graphs)
+    wall, kernel_name, launches = main_run["wall"], main_run["kernel"], main_run["launches"]
+    kernel_ms, graphs_per_launch, event_ms = main_run["kernel_ms"], main_run["graphs_per_launch"], main_run["event_ms"]
+    sums_host = main_run["sums"]
+    ms_per_step = wall * 1000.0 / args.steps
+    value = args.graphs * args.steps / wall
+    accuracy = float((sums_host.argmax(axis=1) == wl.Y_test).mean())
+    included_main = mean_included_literals(tm)
+
+    # roofline of the clause-evaluation kernel: algorithmic bytes / kernel time
     achieved = b_eval * graphs_per_launch / (kernel_ms * 1e-3) / 1e9
     compulsory = (n_nodes * la * 4 + n_nodes * 4 + tm.number_of_outputs * 4) * graphs_per_launch
+    counters = MEASURED_COUNTERS.get(args.workload)
+    if counters and counters["kernel"] != kernel_name:
+        counters = None
+    traffic = (round((counters["fetch_units"] * 2 + counters["write_units"]) * 1024 / counters["graphs"] * graphs_per_launch)
+               if counters else None)
     roofline = {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": (round(MEASURED_TRAFFIC_BYTES_PER_GRAPH[args.workload] * graphs_per_launch)
-                    if args.workload in MEASURED_TRAFFIC_BYTES_PER_GRAPH and kernel_name == "k_tile_two_phase<score>" else None),
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
         "kernel": kernel_name, "kernel_ms": round(kernel_ms, 4), "launches": launches,
         "graphs_per_launch": graphs_per_launch,
         "algorithmic_bytes_per_graph": b_eval,
+        # the same bytes over the whole timed step (kernel + clause compilation + launch gaps)
+        "frac_whole_step": round(b_eval * args.graphs / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        # what the memory system really moved (rocprofv3 FETCH_SIZE + WRITE_SIZE) over this run's kernel time,
+        # and the share of cycles in which the vector ALUs issued (both from the counter runs named above)
+        "hbm_measured_GBs": round(traffic / (kernel_ms * 1e-3) / 1e9, 1) if traffic else None,
+        "hbm_measured_frac": round(traffic / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if traffic else None,
+        "valu_busy": counters["valu_busy"] if counters else None,
+        "counters_measured_at_commit": counters["commit"] if counters else None,
         "compulsory_GBs": round(compulsory / (kernel_ms * 1e-3) / 1e9, 1),
         # the dense formulation (one word test per clause, node and literal word) against the integer
         # VALU peak of 256 CUs x 64 lanes x 2.4 GHz: what a kernel that does not skip work could reach
@@ -287,6 +363,22 @@ def main():
                "numpy_train_sample": "NumPy oracle, one training pass over %d graphs (%.1f s)"
                                      % (train_sample, t_cpu_train)}
 
+    if states:
+        states.append({"state": "after %d epoch(s) (the headline)" % args.train_epochs, "frac": roofline["frac"],
+                       "kernel_ms": roofline["kernel_ms"], "graphs_per_s": round(value, 1),
+                       "mean_included_literals": round(included_main, 2),
+                       "class_sums_equal_c_oracle": None if args.no_cpu else True})
+        tm.fit(wl.graphs_train, wl.Y_train, epochs=2, incremental=True)
+        torch.cuda.synchronize()
+        run = time_scoring(tm, test, args.steps, args.warmup, args.graphs)
+        states.append(state_entry("after %d epochs" % (args.train_epochs + 2), run,
+                                  None if args.no_cpu else c_oracle_agrees(run)))
+        roofline["states"] = states
+        roofline["frac_worst_state"] = min(e["frac"] for e in states)
+        if any(e["class_sums_equal_c_oracle"] is False for e in states):
+            print("bench.py: GPU class sums differ from the C oracle on a state: %s" % json.dumps(states), file=sys.stderr)
+            sys.exit(1)
+
     others = {}
     if not args.only_main:
         for name, (n_train, n_test) in OTHER_WORKLOADS.items():
@@ -298,9 +390,12 @@ def main():
             # graphs, hardware not stated): 1.52-1.55 s per training epoch, 0.88 s per test pass
             others["noisy_xor"]["reference_readme_train_graphs_per_s"] = 6500
             others["noisy_xor"]["reference_readme_test_graphs_per_s"] = 11400
-            if others[name]["class_sums_equal_oracle_on"] == "MISMATCH":
-                print("bench.py: GPU class sums differ from the CPU oracle on %s" % name, file=sys.stderr)
-                sys.exit(1)
+        wrong = [name for name, r in others.items()
+                 if "MISMATCH" in (r["class_sums_equal_oracle_on"], r["class_sums_equal_c_oracle_on"])]
+        if wrong:
+            print("bench.py: GPU class sums differ from a CPU oracle on %s: %s"
+                  % (", ".join(wrong), json.dumps({n: others[n] for n in wrong})), file=sys.stderr)
+            sys.exit(1)
 
     line = {
         "metric": "inference graphs/sec on 1 MI355X (%s)" % args.workload,
@@ -309,15 +404,23 @@ def main():
         "dtype": "u32", "data": "synthetic",
         "config": {"workload": args.workload, "graphs_per_step": args.graphs, "nodes_per_graph": n_nodes,
                    "clauses": tm.number_of_clauses, "literals": tm.number_of_literals, "depth": tm.depth,
-                   "classes": tm.number_of_outputs, "state": "trained %d epoch(s) on %d graphs on the GPU"
-                   % (args.train_epochs, args.train_graphs),
-                   "mean_included_literals": round(mean_included_literals(tm), 2)},
+                   "classes": tm.number_of_outputs,
+                   "state": ("loaded from %s" % args.load_state) if args.load_state else
+                            "trained %d epoch(s) on %d graphs on the GPU" % (args.train_epochs, args.train_graphs),
+                   "mean_included_literals": round(included_main, 2)},
         "roofline": roofline, "cpu_baseline": cpu,
         "train_graphs_per_s": round(train_gps, 1), "test_accuracy": round(accuracy, 4),
         "event_ms_per_step": round(event_ms, 4), "data_build_s": round(t_data, 1),
         "other_workloads": others,
     }
-    print(json.dumps(line))
+    print(json.dumps(line), flush=True)
+    # nothing of this process's is left on the device when the interpreter starts to shut down
+    del tm, wl, test
+    import gc
+
+    gc.collect()
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
 
 
 if __name__ == "__main__":

@@ -56,6 +56,7 @@ struct FitPersistParams {
     unsigned long long *class_sum;  // [3][K][FITP_SUM_PARTS] words FITP_SUM_STRIDE apart, zero on entry (K <= FITP_BLOCK)
     uint32_t *abort_flag;           // [1], zero on entry
     uint32_t spin_limit;
+    int force_abort;      // give up at the first wait without looking (exercises the drain path)
     int clauses_per_group;
     int rows_words;       // LDS words of one staged graph: (literals + n_types + 1) * max slot words
     int max_words;        // words per graph slot that can hold nodes
@@ -466,8 +467,9 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             const unsigned long long seen_own = ((unsigned long long)seen_slot[K + k] << 32) | seen_slot[k];
             uint32_t polls = 0;
             unsigned long long word = 0ull;
-            bool ok = true;
-            for (;;) {
+            bool ok = !p.force_abort;
+            if (!ok) __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            while (ok) {
                 word = read_sum(slot_now, k);
                 if (arrivals(word, seen_own) == everyone) break;
                 if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||

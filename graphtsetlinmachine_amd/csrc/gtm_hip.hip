@@ -9,7 +9,9 @@
 #include <cstdio>
 #include <cstring>
 #include <cstdlib>
+#include <mutex>
 #include <string>
+#include <unordered_map>
 
 #include "../../include/gtm_abi.h"
 #include "philox.h"
@@ -19,15 +21,14 @@ namespace {
 
 // ------------------------------------------------------------------ errors
 
-thread_local std::string g_error;
+// Plain storage: nothing of this library's has a destructor that runs at thread or process exit.
+thread_local char g_error[512] = "";
 
 int fail(int code, const char *fmt, ...) {
-    char buf[512];
     va_list ap;
     va_start(ap, fmt);
-    vsnprintf(buf, sizeof buf, fmt, ap);
+    vsnprintf(g_error, sizeof g_error, fmt, ap);
     va_end(ap);
-    g_error = buf;
     return code;
 }
 
@@ -54,7 +55,10 @@ void profile_start(const char *name, hipStream_t st) {
     if (!g_prof.on || g_prof.used >= Profile::MAX) return;
     if (g_prof.used >= g_prof.created) {
         if (hipEventCreate(&g_prof.start[g_prof.created]) != hipSuccess) return;
-        if (hipEventCreate(&g_prof.stop[g_prof.created]) != hipSuccess) return;
+        if (hipEventCreate(&g_prof.stop[g_prof.created]) != hipSuccess) {
+            (void)hipEventDestroy(g_prof.start[g_prof.created]);
+            return;
+        }
         ++g_prof.created;
     }
     g_prof.name = name;
@@ -563,6 +567,8 @@ struct FitWs {
     uint32_t *message_rows;                 // [M][message_row_words] literal-major messages of one layer (depth > 1)
     int message_row_words;
     uint32_t *sent, *got;                   // [max_nodes][M / 32] bit vectors sent / received per node (depth > 1)
+    uint32_t *bank_backup;                  // [C][LA][B]: the layer-0 bank as it was before a cooperative run (depth 1)
+    int32_t *weights_backup;                // [K][C]
     size_t bytes;
 };
 
@@ -590,6 +596,8 @@ FitWs carve_fit(const Dims &d, const gtm_config *cfg, char *base) {
     const size_t vector_bytes = (size_t)cfg->max_nodes * ((d.M + 31) / 32) * 4;
     w.sent = cfg->depth > 1 ? (uint32_t *)take(vector_bytes) : nullptr;
     w.got = cfg->depth > 1 ? (uint32_t *)take(vector_bytes) : nullptr;
+    w.bank_backup = cfg->depth == 1 ? (uint32_t *)take((size_t)d.C * d.LA * d.B * 4) : nullptr;
+    w.weights_backup = cfg->depth == 1 ? (int32_t *)take((size_t)d.K * d.C * 4) : nullptr;
     w.bytes = off;
     return w;
 }
@@ -681,6 +689,40 @@ int max_lane_words() {
 TileGeom geometry_for(const gtm_config *cfg, const gtm_graphs *g, int classes) {
     return tile_geometry(cfg->literals, g->number_of_node_types, g->max_number_of_graph_nodes, g->number_of_graphs,
                          classes, max_lane_words(), cfg->depth > 1 ? tile_message_rows(cfg->message_size) : 0);
+}
+
+// The geometry every tile buffer of this process was built for, by address.  The driver loops
+// recompute the geometry from their arguments on every call; a buffer built for other arguments
+// (another number of classes, depth, message size or lane-width setting) would be read with the
+// wrong row width, so such a call is refused.  (Leaked on purpose: no destructor runs at exit.)
+struct TilesTag {
+    TileGeom tg;
+    int literals, n_types, n_graphs;
+};
+std::mutex g_tiles_mutex;
+std::unordered_map<const void *, TilesTag> &tiles_registry() {
+    static auto *m = new std::unordered_map<const void *, TilesTag>();
+    return *m;
+}
+
+void remember_tiles(const void *tiles, const TileGeom &tg, const gtm_config *cfg, const gtm_graphs *g) {
+    std::lock_guard<std::mutex> lock(g_tiles_mutex);
+    tiles_registry()[tiles] = TilesTag{tg, cfg->literals, g->number_of_node_types, g->number_of_graphs};
+}
+
+int check_tiles(const TileGeom &tg, const gtm_config *cfg, const gtm_graphs *g) {
+    std::lock_guard<std::mutex> lock(g_tiles_mutex);
+    auto it = tiles_registry().find(g->tiles);
+    if (it == tiles_registry().end())
+        return fail(GTM_ERR_INVALID, "graphs->tiles was not filled by gtm_build_tiles in this process");
+    const TilesTag &t = it->second;
+    if (memcmp(&t.tg, &tg, sizeof tg) != 0 || t.literals != cfg->literals || t.n_types != g->number_of_node_types ||
+        t.n_graphs != g->number_of_graphs)
+        return fail(GTM_ERR_INVALID,
+                    "graphs->tiles was built for another configuration (rows of %d words x %d rows, %d graphs per "
+                    "tile; this call needs %d x %d, %d): build the tiles again with this configuration",
+                    t.tg.tw, t.tg.rows, t.tg.gpt, tg.tw, tg.rows, tg.gpt);
+    return GTM_OK;
 }
 
 // Workgroups that share a tile's clauses when layer 0 reads its rows in place and the tiles are few.
@@ -988,7 +1030,7 @@ extern "C" {
 
 int gtm_abi_version(void) { return GTM_ABI_VERSION; }
 
-const char *gtm_last_error(void) { return g_error.c_str(); }
+const char *gtm_last_error(void) { return g_error; }
 
 int gtm_prepare(const gtm_config *cfg, uint64_t step, uint32_t *ta_state, int32_t *clause_weights, void *stream) {
     Dims d;
@@ -1228,6 +1270,14 @@ int gtm_transform(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_sta
 int gtm_profile_enable(int on) {
     g_prof.on = on != 0;
     g_prof.used = 0;
+    if (!on) {
+        // no HIP object of this library's outlives the measurement (none is left for process exit)
+        for (int i = 0; i < g_prof.created; ++i) {
+            (void)hipEventDestroy(g_prof.start[i]);
+            (void)hipEventDestroy(g_prof.stop[i]);
+        }
+        g_prof.created = 0;
+    }
     return GTM_OK;
 }
 
@@ -1279,7 +1329,9 @@ int gtm_build_tiles(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *t
     if (int rc = check_launch("row_counts")) return rc;
     hipLaunchKernelGGL(k_row_order, dim3(blocks_for(cfg->literals, TPB)), dim3(TPB), 0, st,
                        (const unsigned long long *)counts, cfg->literals, (uint32_t *)(counts + (size_t)tg.rows * 2));
-    return check_launch("row_order");
+    if (int rc = check_launch("row_order")) return rc;
+    remember_tiles(tiles, tg, cfg, graphs);
+    return GTM_OK;
 }
 
 // The tile path runs when the data set carries tiles (gtm_build_tiles) of a supported shape.
@@ -1315,7 +1367,10 @@ int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *
         return fail(GTM_ERR_INVALID, "workspace of %zu bytes needed, %zu given", w.bytes, workspace_bytes);
     hipStream_t st = (hipStream_t)stream;
     if (n_graphs == 0) return GTM_OK;
-    if (tiles) return score_on_tiles(d, cfg, graphs, state, tg, w, first_graph, n_graphs, batch, class_sum, st);
+    if (tiles) {
+        if (int rc = check_tiles(tg, cfg, graphs)) return rc;
+        return score_on_tiles(d, cfg, graphs, state, tg, w, first_graph, n_graphs, batch, class_sum, st);
+    }
     for (int done = 0; done < n_graphs; done += batch) {
         int nb = n_graphs - done < batch ? n_graphs - done : batch;
         uint32_t *final_bitmap = nullptr;
@@ -1425,24 +1480,40 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     p.class_sum = (unsigned long long *)w.class_sum;
     p.abort_flag = (uint32_t *)((unsigned long long *)w.class_sum + (size_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE);
     p.spin_limit = 4000000u;  // a few seconds of polling at the very most
-    if (const char *e = getenv("GTM_FIT_SPIN_LIMIT")) p.spin_limit = (uint32_t)strtoul(e, nullptr, 10);  // tests force the give-up path
+    if (const char *e = getenv("GTM_FIT_SPIN_LIMIT")) {  // tests force the give-up path
+        // "abort": every workgroup gives up at its first wait, whatever it reads there
+        p.force_abort = strcmp(e, "abort") == 0;
+        if (!p.force_abort) p.spin_limit = (uint32_t)strtoul(e, nullptr, 10);
+    }
+    // A run that gives up leaves the workgroups at different examples.  The bank and the weights
+    // are kept as they were, so that a failed call leaves the model as it found it.
+    const size_t bank_bytes = (size_t)d.C * d.LA * d.B * 4, weights_bytes = (size_t)d.K * d.C * 4;
+    hipError_t e = hipMemcpyAsync(w.bank_backup, s->ta_state, bank_bytes, hipMemcpyDeviceToDevice, st);
+    if (e == hipSuccess) e = hipMemcpyAsync(w.weights_backup, s->clause_weights, weights_bytes, hipMemcpyDeviceToDevice, st);
+    if (e != hipSuccess) return fail(GTM_ERR_HIP, "keeping a copy of the model state: %s", hipGetErrorString(e));
 
     hipLaunchKernelGGL(k_fill_u64, dim3(blocks_for((int64_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE + 1, TPB)), dim3(TPB), 0, st,
                        (unsigned long long *)w.class_sum, (int64_t)0, 0ull, (int64_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE + 1);
     if (int rc = check_launch("fill")) return rc;
     void *args[] = {&p};
     profile_start("k_fit_persistent", st);
-    hipError_t e = hipLaunchCooperativeKernel(kernel, dim3(groups), dim3(FITP_BLOCK), args,
-                                              (unsigned)lds, st);
+    e = hipLaunchCooperativeKernel(kernel, dim3(groups), dim3(FITP_BLOCK), args, (unsigned)lds, st);
     if (e != hipSuccess) return fail(GTM_ERR_HIP, "cooperative launch of the training kernel: %s", hipGetErrorString(e));
     profile_stop(st);
     uint32_t flag = 0;
     e = hipMemcpyAsync(&flag, p.abort_flag, 4, hipMemcpyDeviceToHost, st);
     if (e == hipSuccess) e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(GTM_ERR_HIP, "training kernel: %s", hipGetErrorString(e));
-    if (flag != 0)
+    if (flag != 0) {
+        e = hipMemcpyAsync(s->ta_state, w.bank_backup, bank_bytes, hipMemcpyDeviceToDevice, st);
+        if (e == hipSuccess) e = hipMemcpyAsync(s->clause_weights, w.weights_backup, weights_bytes, hipMemcpyDeviceToDevice, st);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        if (e != hipSuccess)
+            return fail(GTM_ERR_HIP, "training kernel gave up waiting at its device-wide barrier (%d workgroups) and "
+                                     "the model state could not be restored: %s", groups, hipGetErrorString(e));
         return fail(GTM_ERR_HIP, "training kernel gave up waiting at its device-wide barrier (%d workgroups); "
-                                 "the model state is inconsistent", groups);
+                                 "the model state is as it was before the call", groups);
+    }
     *done = true;
     return GTM_OK;
 }
@@ -1753,6 +1824,11 @@ int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *st
     if (e == hipSuccess) e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(GTM_ERR_HIP, "reading graph sizes: %s", hipGetErrorString(e));
 
+    if (graphs->tiles) {
+        TileGeom tg = geometry_for(cfg, graphs, d.K);
+        if (tg.ok)
+            if (int rc = check_tiles(tg, cfg, graphs)) return rc;
+    }
     if (cfg->depth == 1 && graphs->tiles) {
         TileGeom tg = geometry_for(cfg, graphs, d.K);
         if (tg.ok && tg.slot_words <= 64) {  // one lane per word of the graph's slot

@@ -157,6 +157,9 @@ class Graphs:
         type_id = self._node_type(node_type_name)
         names = self.graph_node_id[graph_id]
         if node_name not in names:
+            if isinstance(names, _RangeNames):
+                # a name outside 0..n-1 after the bulk builder: fall back to the reference's dict
+                names = self.graph_node_id[graph_id] = dict(names.items())
             names[node_name] = len(names)
         row = int(self.node_index[graph_id]) + names[node_name]
         self.node_type[row] = type_id
@@ -454,10 +457,15 @@ class Graphs:
         subset.X[:] = self.X[old_rows]
         subset.prepare_edge_configuration()
 
-        e_counts = self.number_of_graph_node_edges[old_rows].astype(np.int64)
+        # per node the edges added so far (graphs.py:288-296 copies graph_node_edge_counter of them);
+        # for a complete data set that is every declared edge
+        e_counts = self.graph_node_edge_counter[old_rows].astype(np.int64)
         e_starts = self.edge_index[old_rows].astype(np.int64)
         e_within = np.arange(int(e_counts.sum())) - np.repeat(np.cumsum(e_counts) - e_counts, e_counts)
-        subset.edge[:] = self.edge[np.repeat(e_starts, e_counts) + e_within]
+        if int(e_counts.sum()) != subset.edge.shape[0]:
+            subset.edge[:] = 0  # slots of edges not yet added (encode() below reports them)
+        new_starts = subset.edge_index.astype(np.int64)
+        subset.edge[np.repeat(new_starts, e_counts) + e_within] = self.edge[np.repeat(e_starts, e_counts) + e_within]
         subset.encode()
         return subset
 

@@ -17,6 +17,7 @@ accepted and ignored: launch shapes are chosen by the library.
 """
 
 import ctypes
+import os
 import pickle
 import sys
 
@@ -75,21 +76,84 @@ class _DeviceGraphs:
         d.tiles = None
         self.desc = d
         self.tiles = None
-        self._tiles_tried = False
+        self._tiles_key = None
 
     def ensure_tiles(self, cfg):
-        """Build the literal-major tile layout once per data set (used by
-        inference and depth-1 training); shapes without such a layout keep
-        tiles = NULL."""
-        if self._tiles_tried:
+        """Build the literal-major tile layout once per data set and tile
+        geometry (used by inference and training); shapes without such a
+        layout keep tiles = NULL.  The geometry depends on the model's
+        sizes, so a data set handed to a model of another shape is tiled
+        again."""
+        key = (cfg.classes, cfg.literals, cfg.depth, cfg.message_size, os.environ.get("GTM_TILE_LANE_WORDS"))
+        if self._tiles_key == key:
             return
-        self._tiles_tried = True
+        self._tiles_key = key
+        self.tiles = None
+        self.desc.tiles = None
         nbytes = _abi.lib.gtm_tiles_bytes(ctypes.byref(cfg), ctypes.byref(self.desc))
         if nbytes == 0:
             return
         self.tiles = torch.empty(nbytes // 4, dtype=torch.int32, device=_device())
         _abi.call("gtm_build_tiles", ctypes.byref(cfg), ctypes.byref(self.desc), _ptr(self.tiles), _stream())
         self.desc.tiles = self.tiles.data_ptr()
+
+
+class ModelState(tuple):
+    """The 10-tuple of ``get_state`` (tm.py:287) with the message banks riding
+    along as an attribute; indexes, unpacks and compares as the plain tuple."""
+
+    message_ta_state = None
+
+
+_NPZ_ARRAYS = ("ta_state", "clause_weights", "hypervectors")
+_NPZ_SCALARS = (
+    "number_of_outputs", "number_of_literals", "number_of_message_literals", "min_y", "max_y", "negative_clauses",
+    "max_number_of_graph_nodes", "number_of_clauses", "T", "q", "max_included_literals",
+    "boost_true_positive_feedback", "number_of_state_bits", "depth", "message_size", "message_bits",
+    "double_hashing", "one_hot_encoding", "rng_seed", "rng_step",
+)
+
+
+def write_state_npz(state_dict, fname):
+    """The dict of ``save`` (tm.py:328-354) as a NumPy archive of plain arrays:
+    nothing in it is pickled, so ``numpy.load(allow_pickle=False)`` reads it.
+    Message banks become ``message_ta_state_<i>``, ``s`` a float array, scalars
+    0-d arrays; a value of None is left out."""
+    out = {name: np.asarray(state_dict[name]) for name in _NPZ_ARRAYS}
+    for i, bank in enumerate(state_dict["message_ta_state"]):
+        out["message_ta_state_%d" % i] = np.asarray(bank, dtype=np.uint32)
+    out["s"] = np.asarray(state_dict["s"], dtype=np.float64).reshape(-1)
+    for name in _NPZ_SCALARS:
+        value = state_dict.get(name)
+        if value is None:
+            continue
+        out[name] = np.asarray(value, dtype=np.uint64 if name == "rng_seed" else None)
+    with open(fname, "wb") as f:
+        np.savez(f, **out)
+
+
+def read_state_npz(fname):
+    """Inverse of ``write_state_npz``: the dict ``load`` takes."""
+    with np.load(fname, allow_pickle=False) as z:
+        d = {name: z[name] for name in _NPZ_ARRAYS}
+        banks = []
+        while "message_ta_state_%d" % len(banks) in z.files:
+            banks.append(z["message_ta_state_%d" % len(banks)])
+        d["message_ta_state"] = banks
+        d["s"] = tuple(float(v) for v in z["s"])
+        for name in _NPZ_SCALARS:
+            if name not in z.files:
+                if name not in ("rng_seed", "rng_step"):
+                    d[name] = None
+                continue
+            v = z[name][()]
+            if name in ("double_hashing", "one_hot_encoding"):
+                d[name] = bool(v)
+            elif name == "q":
+                d[name] = float(v)
+            else:
+                d[name] = int(v)
+    return d
 
 
 class CommonTsetlinMachine:
@@ -193,6 +257,7 @@ class CommonTsetlinMachine:
             for _ in range(self.depth - 1)
         ]
         self.clause_weights_gpu = torch.empty(self.number_of_outputs * C, dtype=torch.int32, device=dev)
+        self._allocated_outputs = int(self.number_of_outputs)
         self.hypervectors_gpu = _to_device(self.hypervectors)
         st = _abi.State()
         st.ta_state = _ptr(self.ta_state_gpu)
@@ -202,7 +267,29 @@ class CommonTsetlinMachine:
         st.hypervectors = _ptr(self.hypervectors_gpu)
         self._state = st
 
+    def _outputs_for(self, seen):
+        """Number of outputs for a ``fit`` whose labels show ``seen`` of them.
+
+        The weight buffer and the tile geometry are sized for the outputs of
+        the first ``fit`` (the reference compiles CLASSES in then,
+        tm.py:452).  A later batch may hold fewer labels - the model keeps
+        its size - but never more: that would index past the buffers."""
+        allocated = getattr(self, "_allocated_outputs", None)
+        if not self.initialized or allocated is None:
+            return int(seen)
+        if seen > allocated:
+            raise _abi.GtmError(
+                "this model was sized for %d outputs at its first fit; the labels passed now need %d"
+                % (allocated, seen)
+            )
+        return allocated
+
     def _config(self, max_nodes):
+        if getattr(self, "_allocated_outputs", self.number_of_outputs) != self.number_of_outputs:
+            raise _abi.GtmError(
+                "number_of_outputs=%d differs from the %d outputs the device buffers were allocated for"
+                % (self.number_of_outputs, self._allocated_outputs)
+            )
         return _abi.make_config(
             classes=self.number_of_outputs,
             clauses=self.number_of_clauses,
@@ -248,20 +335,25 @@ class CommonTsetlinMachine:
             self.encoded_Y = encoded_Y
             self._encoded_Y_gpu = _to_device(np.ascontiguousarray(encoded_Y, dtype=np.int32))
 
-    def _fit(self, graphs, encoded_Y, epochs=100, incremental=False):
-        """tm.py:664-752; each epoch is one gtm_fit call."""
+    def _fit(self, graphs, encoded_Y, epochs=100, incremental=False, examples=None):
+        """tm.py:664-752; each epoch is one gtm_fit call.  ``examples=(first, count)`` (not in
+        the reference) restricts an epoch to that run of the data set's graphs, so that a
+        resident data set can be trained on piece by piece without being cut up."""
         self._init_fit(graphs, encoded_Y, incremental)
         dg = self._train_graphs
         cfg = self._config(max(dg.max_nodes, 1))
         dg.ensure_tiles(cfg)
         need = _abi.lib.gtm_fit_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc))
         ws = self._workspace_of(need)
+        first, count = (0, dg.number_of_graphs) if examples is None else (int(examples[0]), int(examples[1]))
+        if first < 0 or count < 0 or first + count > dg.number_of_graphs:
+            raise _abi.GtmError("examples=(%d, %d) outside the data set's %d graphs" % (first, count, dg.number_of_graphs))
         for _ in range(epochs):
             _abi.call(
                 "gtm_fit", ctypes.byref(cfg), ctypes.byref(dg.desc), ctypes.byref(self._state),
-                _ptr(self._encoded_Y_gpu), 0, dg.number_of_graphs, self.step, _ptr(ws), ws.numel(), _stream(),
+                _ptr(self._encoded_Y_gpu), first, count, self.step, _ptr(ws), ws.numel(), _stream(),
             )
-            self.step += dg.number_of_graphs
+            self.step += count
         torch.cuda.current_stream().synchronize()
         self.ta_state = np.array([])
         self.clause_weights = np.array([])
@@ -414,24 +506,90 @@ class CommonTsetlinMachine:
         return self.clause_weights.reshape((self.number_of_outputs, self.number_of_clauses))
 
     def get_state(self):
-        """tm.py:281-287: the 10-tuple, always read fresh from the device."""
+        """tm.py:281-287: the 10-tuple, always read fresh from the device.  The
+        tuple also carries the message banks as the attribute
+        ``message_ta_state`` (the reference's tuple leaves them out), so that
+        ``set_state(get_state())`` restores a model with message layers
+        completely."""
         self._download()
-        return (
+        state = ModelState((
             self.ta_state, self.clause_weights, self.number_of_outputs, self.number_of_clauses,
             self.number_of_literals, self.depth, self.number_of_state_bits, self.number_of_ta_chunks,
             self.min_y, self.max_y,
-        )
+        ))
+        state.message_ta_state = list(self.message_ta_state)
+        return state
 
     def set_state(self, state):
-        """tm.py:289-310.  Restores the layer-0 bank and the weights into an
-        initialised model of the same shape (the reference's version leaves
-        message banks and kernels unset)."""
-        (ta_state, weights, self.number_of_outputs, self.number_of_clauses, self.number_of_literals,
-         self.depth, self.number_of_state_bits, self.number_of_ta_chunks, self.min_y, self.max_y) = state
-        if not self.initialized:
-            raise _abi.GtmError("set_state needs an initialised model; use load() to build one from a saved state")
-        self.ta_state_gpu.copy_(_to_device(np.asarray(ta_state, dtype=np.uint32)))
-        self.clause_weights_gpu.copy_(_to_device(np.asarray(weights, dtype=np.int32)))
+        """tm.py:289-310, made to leave a usable model: works on a model that
+        has never been trained (every buffer is allocated here), restores the
+        layer-0 bank and the weights from the tuple and the message banks from
+        its ``message_ta_state`` attribute when it has one (tuples made by
+        this class's ``get_state``).  A plain 10-tuple, as the reference makes
+        them, holds no message banks: those keep their contents on an
+        initialised model of the same shape and start from the initial state
+        otherwise."""
+        (ta_state, weights, outputs, clauses, literals, depth, state_bits, ta_chunks, min_y, max_y) = tuple(state)
+        same_shape = self.initialized and (
+            int(outputs), int(clauses), int(literals), int(depth), int(state_bits)
+        ) == (
+            getattr(self, "_allocated_outputs", -1), self.number_of_clauses, self.number_of_literals, self.depth,
+            self.number_of_state_bits,
+        )
+        if int(depth) != self.depth and self.one_hot_encoding:
+            raise _abi.GtmError("set_state cannot change the depth of a one-hot model; use load()")
+        if not same_shape and self.one_hot_encoding and int(depth) > 1 and not self.initialized:
+            raise _abi.GtmError(
+                "a one-hot model takes its message size from the first data set's edge types; "
+                "use load() to build it from a saved state"
+            )
+        ta_state = np.ascontiguousarray(ta_state, dtype=np.uint32).reshape(-1)
+        weights = np.ascontiguousarray(weights, dtype=np.int32).reshape(-1)
+        chunks = int((int(literals) - 1) // 32 + 1)
+        bank_words = int(clauses) * chunks * int(state_bits)
+        # the reference allocates depth x the layer-0 bank (tm.py:299) and copies the whole array:
+        # only the first bank's worth is the layer-0 state
+        if ta_state.size < bank_words or weights.size != int(outputs) * int(clauses) or int(ta_chunks) != chunks:
+            raise _abi.GtmError("set_state: array sizes do not match the sizes in the tuple")
+        banks = getattr(state, "message_ta_state", None)
+        if not same_shape:
+            if int(clauses) != self.number_of_clauses and int(depth) > 1:
+                raise _abi.GtmError("set_state cannot change the number of clauses of a model with message layers "
+                                    "(its hypervectors have one row per clause); use load()")
+            self.number_of_outputs = int(outputs)
+            self.number_of_clauses = int(clauses)
+            self.number_of_clause_chunks = (self.number_of_clauses - 1) // 32 + 1
+            self.number_of_literals = int(literals)
+            if int(depth) != self.depth:
+                self.s = tuple(self.s[i] if i < len(self.s) else self.s[-1] for i in range(int(depth)))
+            self.depth = int(depth)
+            self.number_of_state_bits = int(state_bits)
+            self.number_of_ta_chunks = chunks
+            self.number_of_features = self.number_of_literals // 2
+            self.number_of_message_features = self.message_size
+            self.number_of_message_literals = self.message_size * 2
+            self.number_of_message_chunks = int((self.number_of_message_literals - 1) // 32 + 1)
+            if self.max_included_literals is None:
+                self.max_included_literals = self.number_of_literals
+            if not hasattr(self, "max_number_of_graph_nodes"):
+                self.max_number_of_graph_nodes = 0  # taken from the data set of every call
+            self._allocate()
+            self.initialized = True
+            if banks is None and self.depth > 1:
+                cfg = self._config(1)
+                for t in self.message_ta_state_gpu:
+                    _abi.call("gtm_prepare_message_ta_state", ctypes.byref(cfg), _ptr(t), _stream())
+        self.min_y, self.max_y = min_y, max_y
+        self.ta_state_gpu.copy_(_to_device(ta_state[:bank_words]))
+        self.clause_weights_gpu.copy_(_to_device(weights))
+        if banks is not None:
+            if len(banks) != self.depth - 1:
+                raise _abi.GtmError("set_state: %d message banks for depth %d" % (len(banks), self.depth))
+            for t, host in zip(self.message_ta_state_gpu, banks):
+                host = np.ascontiguousarray(host, dtype=np.uint32).reshape(-1)
+                if host.size != t.numel():
+                    raise _abi.GtmError("set_state: a message bank has %d words, expected %d" % (host.size, t.numel()))
+                t.copy_(_to_device(host))
         self.graphs_signature_train = np.array([])
         self.graphs_signature_test = np.array([])
         self._train_graphs = self._test_graphs = None
@@ -473,8 +631,11 @@ class CommonTsetlinMachine:
         }
         if len(fname) > 0:
             print(f"Saving model to {fname}.")
-            with open(fname, "wb") as f:
-                pickle.dump(state_dict, f)
+            if fname.endswith(".npz"):
+                write_state_npz(state_dict, fname)
+            else:
+                with open(fname, "wb") as f:
+                    pickle.dump(state_dict, f)
         return state_dict
 
     def load(self, state_dict={}, fname=""):
@@ -484,8 +645,20 @@ class CommonTsetlinMachine:
             return
         if len(fname) > 0:
             print(f"Loading model from {fname}.")
-            with open(fname, "rb") as f:
-                state_dict = pickle.load(f)
+            if fname.endswith(".npz"):
+                state_dict = read_state_npz(fname)
+            else:
+                with open(fname, "rb") as f:
+                    state_dict = pickle.load(f)
+        # the constructor arguments travel with the state (tm.py:341-353 saves them; the reference's
+        # load leaves them to the caller's constructor call): a model built with other arguments
+        # must not run a loaded state with the wrong clause count, depth or automaton width
+        for key in ("number_of_clauses", "T", "s", "q", "max_included_literals", "boost_true_positive_feedback",
+                    "number_of_state_bits", "depth", "message_bits", "double_hashing", "one_hot_encoding"):
+            if key in state_dict:
+                setattr(self, key, state_dict[key])
+        self.number_of_clause_chunks = (self.number_of_clauses - 1) // 32 + 1
+        self.s = tuple(self.s) if isinstance(self.s, (tuple, list)) else (self.s,) * self.depth
         self.ta_state = state_dict["ta_state"]
         self.message_ta_state = state_dict["message_ta_state"]
         self.clause_weights = state_dict["clause_weights"]
@@ -508,12 +681,26 @@ class CommonTsetlinMachine:
         if self.max_included_literals is None:
             self.max_included_literals = self.number_of_literals
 
+        C, B = self.number_of_clauses, self.number_of_state_bits
+        expected = [("ta_state", self.ta_state, C * self.number_of_ta_chunks * B),
+                    ("clause_weights", self.clause_weights, self.number_of_outputs * C),
+                    ("hypervectors", self.hypervectors, C * self.message_bits)]
+        if len(self.message_ta_state) != self.depth - 1:
+            raise _abi.GtmError("state has %d message banks for depth %d" % (len(self.message_ta_state), self.depth))
+        expected += [("message_ta_state[%d]" % i, b, C * self.number_of_message_chunks * B)
+                     for i, b in enumerate(self.message_ta_state)]
+        for name, array, size in expected:
+            if np.asarray(array).size != size:
+                raise _abi.GtmError("state's %s has %d elements, expected %d" % (name, np.asarray(array).size, size))
+        self.hypervectors = np.ascontiguousarray(self.hypervectors, dtype=np.uint32).reshape(C, self.message_bits)
         self._allocate()
         self.ta_state_gpu.copy_(_to_device(np.asarray(self.ta_state, dtype=np.uint32)))
         for t, host in zip(self.message_ta_state_gpu, self.message_ta_state):
             t.copy_(_to_device(np.asarray(host, dtype=np.uint32)))
         self.clause_weights_gpu.copy_(_to_device(np.asarray(self.clause_weights, dtype=np.int32)))
         self._train_graphs = self._test_graphs = None
+        self.encoded_Y = np.array([])
+        self._encoded_Y_gpu = None
         self.graphs_signature_train = np.array([])
         self.graphs_signature_test = np.array([])
         self.initialized = True
@@ -526,15 +713,15 @@ class MultiClassGraphTsetlinMachine(CommonTsetlinMachine):
         super().__init__(*args, **kwargs)
         self.negative_clauses = 1
 
-    def fit(self, graphs, Y, epochs=100, incremental=False):
+    def fit(self, graphs, Y, epochs=100, incremental=False, examples=None):
         Y = np.asarray(Y)
-        self.number_of_outputs = int(np.max(Y) + 1)
+        self.number_of_outputs = self._outputs_for(int(np.max(Y) + 1))
         self.max_y = None
         self.min_y = None
         encoded_Y = np.empty((Y.shape[0], self.number_of_outputs), dtype=np.int32)
         for i in range(self.number_of_outputs):
             encoded_Y[:, i] = np.where(Y == i, self.T, -self.T)
-        self._fit(graphs, encoded_Y, epochs=epochs, incremental=incremental)
+        self._fit(graphs, encoded_Y, epochs=epochs, incremental=incremental, examples=examples)
 
     def score(self, graphs):
         return self._score(graphs)
@@ -552,6 +739,8 @@ class MultiOutputGraphTsetlinMachine(CommonTsetlinMachine):
 
     def fit(self, graphs, Y, epochs=100, incremental=False):
         Y = np.asarray(Y)
+        if self._outputs_for(Y.shape[1]) != Y.shape[1]:
+            raise _abi.GtmError("this model has %d outputs; Y has %d columns" % (self._allocated_outputs, Y.shape[1]))
         self.number_of_outputs = Y.shape[1]
         self.max_y = None
         self.min_y = None

@@ -305,3 +305,183 @@ def test_the_call_sequence_of_the_noisy_xor_demo_runs_unchanged():
         described.append(" AND ".join(literals))
     assert any(described) and tm.hypervectors.shape == (10, 2)
     assert graphs_train.edge_type_id == {"Plain": 0} and set(graphs_train.symbol_id) == {"A", "B"}
+
+
+@pytest.mark.parametrize("encoding, clauses, edge_types, depth", [
+    ("one_hot_encoding", 30, ("l", "r", "u"), 2),     # message size 90: not a multiple of 32
+    ("one_hot_encoding", 32, ("l", "r"), 3),          # message size 64: the factored message kernels
+    ("one_hot_encoding", 12, ("l",), 2),
+    ("double_hashing", 40, ("l", "r", "u"), 3),
+    ("double_hashing", 70, ("l", "r"), 2),   # more clauses than message bits: hypervectors repeat
+])
+def test_one_hot_and_double_hashed_clause_messages_follow_the_oracle(encoding, clauses, edge_types, depth):
+    """tm.py:90-106,415-418: the two deterministic clause hypervector tables.  One-hot sizes the
+    messages at the first fit (clauses x edge types), after the constructor made the table.
+    Training trajectories and class sums are compared with the oracle given the same table."""
+    from sympy import prevprime
+
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    train = helpers.random_graphs(70, n_graphs=36, max_nodes=50, hv_size=24, node_types=("a", "b"),
+                                  edge_types=edge_types, max_degree=3)
+    test = helpers.random_graphs(71, n_graphs=20, max_nodes=70, parent=train, node_types=("a", "b"),
+                                 edge_types=edge_types, max_degree=3)
+    Y = np.random.default_rng(5).integers(0, 3, size=36)
+    kwargs = {encoding: True}
+    tm = MultiClassGraphTsetlinMachine(clauses, 40, (2.0, 1.5, 3.0)[:depth], depth=depth, message_size=64,
+                                       message_bits=3, max_included_literals=14, seed=31, **kwargs)
+    tm.fit(train, Y, epochs=2, incremental=True)
+    n_types = len(train.edge_type_id)
+    if encoding == "one_hot_encoding":
+        assert tm.message_size == clauses * n_types and tm.message_bits == 1
+        assert np.array_equal(tm.hypervectors[:, 0], np.arange(clauses) * n_types)
+    else:
+        p = int(prevprime(64))
+        ids = np.arange(clauses)
+        assert tm.message_size == 64 and tm.message_bits == 2
+        assert np.array_equal(tm.hypervectors, np.stack([ids % 64, p - ids % p], axis=1))
+    model = oracle_twin(tm, train)
+    assert model.cfg.message_size == tm.message_size and model.cfg.message_bits == tm.message_bits
+    o.fit(model, train, o.encode_labels(Y, 3, tm.T), epochs=2)
+    assert_same_state(tm, model)
+    model.cfg = oracle_twin(tm, test).cfg
+    assert np.array_equal(tm.score(test), o.score(model, test))
+    saved = tm.save()
+    assert saved["message_size"] == tm.message_size and saved[encoding] is True
+    again = MultiClassGraphTsetlinMachine(clauses, 40, (2.0, 1.5, 3.0)[:depth], depth=depth, **kwargs)
+    again.load(saved)
+    assert np.array_equal(again.score(test), tm.score(test))
+
+
+def _reference_dict(state):
+    """The dict exactly as the reference's save() writes it: its 23 keys (tm.py:328-354), no generator position."""
+    from tests.test_model_host import REFERENCE_KEYS
+
+    return {key: state[key] for key in REFERENCE_KEYS}
+
+
+def test_a_state_dict_shaped_like_the_references_loads_scores_and_resumes(tmp_path):
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    train = helpers.random_graphs(80, n_graphs=30, max_nodes=40, hv_size=20, edge_types=("l", "r"), max_degree=2)
+    Y = np.random.default_rng(6).integers(0, 2, size=30)
+    np.random.seed(12)
+    a = MultiClassGraphTsetlinMachine(24, 30, (1.5, 2.5), depth=2, message_size=40, message_bits=2, seed=77)
+    a.fit(train, Y, epochs=1, incremental=True)
+    model = oracle_twin(a, train)
+    o.fit(model, train, o.encode_labels(Y, 2, a.T))
+    assert_same_state(a, model)
+    state = _reference_dict(a.save())
+    assert len(state) == 23 and "rng_seed" not in state
+
+    # a model constructed with other arguments takes its shape from the dict
+    b = MultiClassGraphTsetlinMachine(5, 7, 9.0, seed=77)
+    b.load(state)
+    assert (b.number_of_clauses, b.depth, b.T, b.s) == (24, 2, 30, (1.5, 2.5))
+    assert np.array_equal(b.score(train), o.score(model, train))
+    # resuming: without a generator position the loaded model starts its draws at step 0 of its own seed
+    b.fit(train, Y, epochs=1, incremental=True)
+    resumed = oracle_twin(b, train)
+    resumed.ta_state, resumed.message_ta_state = model.ta_state.copy(), [m.copy() for m in model.message_ta_state]
+    resumed.clause_weights = model.clause_weights.copy()
+    resumed.step = 0
+    o.fit(resumed, train, o.encode_labels(Y, 2, b.T))
+    assert_same_state(b, resumed)
+
+    # the archive without pickle: same state, generator position included, so both go on identically
+    path = str(tmp_path / "model.npz")
+    a.save(path)
+    with np.load(path, allow_pickle=False) as z:
+        assert "ta_state" in z.files and "message_ta_state_0" in z.files
+    c = MultiClassGraphTsetlinMachine(24, 30, (1.5, 2.5), depth=2, message_size=40, message_bits=2, seed=1)
+    c.load(fname=path)
+    assert c.seed == 77 and c.step == a.step
+    assert np.array_equal(c.score(train), a.score(train))
+    a.fit(train, Y, epochs=1, incremental=True)
+    c.fit(train, Y, epochs=1, incremental=True)
+    sa, sc = a.save(), c.save()
+    assert np.array_equal(sa["ta_state"], sc["ta_state"]) and np.array_equal(sa["clause_weights"], sc["clause_weights"])
+    assert np.array_equal(sa["message_ta_state"][0], sc["message_ta_state"][0])
+
+    # a state whose arrays do not fit its sizes is refused before anything is copied to the device
+    bad = dict(state)
+    bad["ta_state"] = state["ta_state"][:-1]
+    with pytest.raises(Exception, match="ta_state"):
+        MultiClassGraphTsetlinMachine(24, 30, 1.0).load(bad)
+
+
+def test_set_state_builds_a_usable_model_from_a_state_tuple():
+    """tm.py:289-310 made functional: on a model that never trained, with message banks."""
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    train = helpers.random_graphs(81, n_graphs=30, max_nodes=40, hv_size=20, edge_types=("l", "r"), max_degree=2)
+    Y = np.random.default_rng(7).integers(0, 3, size=30)
+    np.random.seed(13)
+    a = MultiClassGraphTsetlinMachine(24, 30, (1.5, 2.5), depth=2, message_size=40, message_bits=2, seed=5)
+    a.fit(train, Y, epochs=1, incremental=True)
+    state = a.get_state()
+    assert len(state) == 10 and isinstance(state, tuple) and state[2:8] == (3, 24, 40, 2, 8, 2)
+    assert len(state.message_ta_state) == 1
+
+    np.random.seed(13)  # same clause hypervectors
+    b = MultiClassGraphTsetlinMachine(24, 30, (1.5, 2.5), depth=2, message_size=40, message_bits=2, seed=5)
+    b.set_state(state)
+    assert np.array_equal(b.score(train), a.score(train))
+    back = b.get_state()
+    assert np.array_equal(back[0], state[0]) and np.array_equal(back[1], state[1])
+    assert np.array_equal(back.message_ta_state[0], state.message_ta_state[0])
+
+    # a plain tuple (the reference's) carries no message banks: a fresh model starts them from the initial state
+    np.random.seed(13)
+    c = MultiClassGraphTsetlinMachine(24, 30, (1.5, 2.5), depth=2, message_size=40, message_bits=2, seed=5)
+    c.set_state(tuple(state))
+    model = oracle_twin(a, train)
+    cfg = model.cfg
+    model.ta_state = state[0].reshape(cfg.clauses, cfg.la_chunks, cfg.state_bits).copy()
+    model.clause_weights = state[1].reshape(cfg.classes, cfg.clauses).copy()  # message bank: as new_model left it
+    assert np.array_equal(c.score(train), o.score(model, train))
+    # on an initialised model of the same shape they keep their contents
+    a.set_state(tuple(state))
+    assert np.array_equal(a.get_state().message_ta_state[0], state.message_ta_state[0])
+    # and training goes on from the restored state
+    c.step = a.step
+    c.set_state(state)
+    a.fit(train, Y, epochs=1, incremental=True)
+    c.fit(train, Y, epochs=1, incremental=True)
+    assert np.array_equal(a.get_state()[0], c.get_state()[0])
+
+    # depth 1: the reference's allocation of depth x the bank; only the first bank is the state
+    d1 = MultiClassGraphTsetlinMachine(16, 20, 2.0, seed=3)
+    d1.fit(train, Y, epochs=1, incremental=True)
+    s1 = d1.get_state()
+    e1 = MultiClassGraphTsetlinMachine(16, 20, 2.0, seed=3)
+    e1.set_state(tuple(s1))
+    assert np.array_equal(e1.score(train), d1.score(train))
+    with pytest.raises(Exception, match="sizes"):
+        e1.set_state((s1[0][:-1],) + tuple(s1[1:]))
+
+
+def test_a_later_fit_with_more_labels_than_the_first_is_refused_and_fewer_keep_the_size():
+    from graphtsetlinmachine_amd import _abi
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    wl = workloads.noisy_xor(200, 50)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=2)
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
+    before = tm.save()
+    with pytest.raises(_abi.GtmError, match="sized for 2 outputs"):
+        tm.fit(wl.graphs_train, np.where(wl.Y_train == 1, 4, 0), epochs=1, incremental=True)
+    after = tm.save()
+    assert np.array_equal(before["ta_state"], after["ta_state"]) and tm.number_of_outputs == 2
+    # a batch that happens to hold only label 0 trains the same two-output model
+    tm.fit(wl.graphs_train, np.zeros_like(wl.Y_train), epochs=1, incremental=True)
+    assert tm.number_of_outputs == 2 and tm.score(wl.graphs_test).shape == (50, 2)
+    model = oracle_twin(tm, wl.graphs_train)
+    cfg = model.cfg
+    model.ta_state = before["ta_state"].reshape(cfg.clauses, cfg.la_chunks, cfg.state_bits).copy()
+    model.message_ta_state = [b.reshape(cfg.clauses, cfg.message_chunks, cfg.state_bits).copy()
+                              for b in before["message_ta_state"]]
+    model.clause_weights = before["clause_weights"].reshape(2, -1).copy()
+    model.step = 200
+    o.fit(model, wl.graphs_train, o.encode_labels(np.zeros_like(wl.Y_train), 2, tm.T))
+    assert_same_state(tm, model)

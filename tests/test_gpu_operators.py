@@ -658,8 +658,10 @@ def test_empty_graphs_score_like_the_reference_arithmetic(hv_size, density):
 
 def test_training_kernel_gives_up_instead_of_hanging(monkeypatch):
     """The one-launch training kernel waits for the other workgroups with a
-    bounded number of polls.  A limit of 0 makes every wait give up at once: the
-    kernel must still drain and the call must report it."""
+    bounded number of polls.  GTM_FIT_SPIN_LIMIT=abort makes every workgroup give up at
+    its first wait whatever it reads there (no dependence on timing or on the number of
+    workgroups): the kernel must still drain, the call must report it, and the model must
+    be left as it was before the call."""
     from tests.gpu_harness import Device
     from graphtsetlinmachine_amd import _abi
 
@@ -670,15 +672,58 @@ def test_training_kernel_gives_up_instead_of_hanging(monkeypatch):
     dev = Device(model, graphs)
     assert dev.build_tiles()
     Y = o.encode_labels(np.zeros(graphs.number_of_graphs, dtype=np.int64), cfg.classes, cfg.threshold)
-    monkeypatch.setenv("GTM_FIT_SPIN_LIMIT", "0")
-    with pytest.raises(_abi.GtmError, match="gave up waiting"):
+    monkeypatch.setenv("GTM_FIT_SPIN_LIMIT", "abort")
+    with pytest.raises(_abi.GtmError, match="gave up waiting.*as it was before the call"):
         dev.fit(Y, 0, graphs.number_of_graphs, 0)
     monkeypatch.delenv("GTM_FIT_SPIN_LIMIT")
-    # the device and the library are still usable afterwards
-    model2 = helpers.random_model(shape["seed"] + 1, cfg, 1, s=3.0, include_density=0.02)
-    dev2 = Device(model2, graphs)
-    assert dev2.build_tiles()
-    o.fit(model2, graphs, Y)
-    dev2.fit(Y, 0, graphs.number_of_graphs, 0)
-    ta, _, w = dev2.download()
-    assert np.array_equal(w, model2.clause_weights) and np.array_equal(ta, model2.ta_state)
+    ta, _, w = dev.download()
+    assert np.array_equal(w, model.clause_weights) and np.array_equal(ta, model.ta_state)
+    # the same model trains normally afterwards
+    o.fit(model, graphs, Y)
+    dev.fit(Y, 0, graphs.number_of_graphs, 0)
+    ta, _, w = dev.download()
+    assert np.array_equal(w, model.clause_weights) and np.array_equal(ta, model.ta_state)
+    # a limit of 0 polls: whoever does not see every arrival at its first look gives up
+    monkeypatch.setenv("GTM_FIT_SPIN_LIMIT", "0")
+    try:
+        dev.fit(Y, 0, graphs.number_of_graphs, graphs.number_of_graphs)
+        o.fit(model, graphs, Y)  # nobody had to wait: the run went through
+    except _abi.GtmError as e:
+        assert "gave up waiting" in str(e)
+    monkeypatch.delenv("GTM_FIT_SPIN_LIMIT")
+    ta, _, w = dev.download()
+    assert np.array_equal(w, model.clause_weights) and np.array_equal(ta, model.ta_state)
+
+
+def test_tiles_built_for_another_configuration_are_refused():
+    """The driver loops recompute the tile geometry from their arguments; a buffer built for other
+    arguments would be read with the wrong row width."""
+    from tests.gpu_harness import Device
+    from graphtsetlinmachine_amd import _abi
+
+    shape = TILE_SHAPES[3]
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    cfg = helpers.oracle_config(graphs, classes=shape["classes"], clauses=shape["clauses"], T=30)
+    model = helpers.random_model(shape["seed"], cfg, 1, s=3.0, include_density=0.02)
+    dev = Device(model, graphs)
+    assert dev.build_tiles()
+    want = o.score(model, graphs)
+    assert np.array_equal(dev.score(0, graphs.number_of_graphs, 8), want)
+    # the same buffer handed to a model with message layers (other rows per tile)
+    deep_cfg = helpers.oracle_config(graphs, classes=shape["classes"], clauses=shape["clauses"], T=30, depth=2,
+                                     message_size=4096)
+    deep = Device(helpers.random_model(shape["seed"], deep_cfg, 2), graphs)
+    deep.dg.desc.tiles = dev.tiles.data_ptr()
+    geometry_differs = _abi.lib.gtm_tiles_bytes(ctypes.byref(deep.acfg), ctypes.byref(deep.dg.desc)) != dev.tiles.numel() * 4
+    if geometry_differs:
+        with pytest.raises(_abi.GtmError, match="another configuration"):
+            deep.score(0, graphs.number_of_graphs, 8)
+    # a buffer the library never filled
+    import torch
+
+    stray = torch.zeros(dev.tiles.numel(), dtype=torch.int32, device="cuda")
+    dev.dg.desc.tiles = stray.data_ptr()
+    with pytest.raises(_abi.GtmError, match="not filled by gtm_build_tiles"):
+        dev.score(0, graphs.number_of_graphs, 8)
+    dev.dg.desc.tiles = dev.tiles.data_ptr()
+    assert np.array_equal(dev.score(0, graphs.number_of_graphs, 8), want)
