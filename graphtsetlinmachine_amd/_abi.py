@@ -98,6 +98,8 @@ PROTOTYPES = {
     "gtm_build_tiles": (C.c_int, [_CFG, _GR, _P, _P]),
     "gtm_score_workspace_bytes": (_SZ, [_CFG, _GR, _I]),
     "gtm_score": (C.c_int, [_CFG, _GR, _ST, _I, _I, _I, _P, _SZ, _P, _P]),
+    "gtm_score_static_scratch_bytes": (_SZ, []),
+    "gtm_score_static": (C.c_int, [_CFG, _GR, _ST, _I, _I, _I, _P, _P]),
     "gtm_fit_workspace_bytes": (_SZ, [_CFG, _GR]),
     "gtm_fit": (C.c_int, [_CFG, _GR, _ST, _P, _I, _I, _U64, _P, _SZ, _P]),
 }

@@ -1382,6 +1382,58 @@ int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *
     return GTM_OK;
 }
 
+// ---- gtm_score for callers that cannot allocate -----------------------------------------------
+// The workspace of gtm_score lives in a file-scope device array instead of a caller's buffer.
+// Every GPU the library runs on holds its own copy of the array, at its own address, until the
+// process ends; the address is looked up once per device and only that pointer is ever handed to
+// kernels (the array's name is a host-side stand-in, not a device address).
+constexpr size_t GTM_STATIC_SCRATCH_BYTES = (size_t)16 << 20;
+constexpr int GTM_STATIC_SCRATCH_DEVICES = 64;
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[GTM_STATIC_SCRATCH_BYTES];
+static void *g_scratch_of_device[GTM_STATIC_SCRATCH_DEVICES];  // filled on a device's first call
+static std::mutex g_scratch_mutex;
+
+static int static_scratch(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(GTM_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= GTM_STATIC_SCRATCH_DEVICES) return fail(GTM_ERR_INVALID, "device %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_of_device[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));  // with `dev` current: that device's copy
+        if (e != hipSuccess || !ptr)
+            return fail(GTM_ERR_HIP, "address of the static scratch array on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_of_device[dev] = ptr;
+    }
+    *out = g_scratch_of_device[dev];
+    return GTM_OK;
+}
+
+size_t gtm_score_static_scratch_bytes(void) { return GTM_STATIC_SCRATCH_BYTES; }
+
+int gtm_score_static(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, int32_t first_graph,
+                     int32_t n_graphs, int32_t batch, int32_t *class_sum, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (batch < 1) return fail(GTM_ERR_INVALID, "batch=%d", batch);
+    const size_t need = gtm_score_workspace_bytes(cfg, graphs, batch);
+    if (need == 0) return fail(GTM_ERR_INVALID, "invalid configuration");
+    if (need > GTM_STATIC_SCRATCH_BYTES)
+        return fail(GTM_ERR_INVALID,
+                    "this model and batch need %zu bytes of scratch; the allocation-free entry point has %zu "
+                    "(use a smaller batch, or gtm_score with a workspace of the caller's)",
+                    need, GTM_STATIC_SCRATCH_BYTES);
+    void *ptr = nullptr;
+    if (int rc = static_scratch(&ptr)) return rc;
+    // the launch timing of gtm_profile_enable creates events: not on this path
+    const bool profiling = g_prof.on;
+    g_prof.on = false;
+    const int rc = gtm_score(cfg, graphs, state, first_graph, n_graphs, batch, ptr, GTM_STATIC_SCRATCH_BYTES, class_sum, stream);
+    g_prof.on = profiling;
+    return rc;
+}
+
 }  // extern "C"
 
 namespace {

@@ -180,6 +180,20 @@ int gtm_score(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *
               int32_t n_graphs, int32_t batch, void *workspace, size_t workspace_bytes, int32_t *class_sum,
               void *stream);
 
+/* No counterpart in the reference.  gtm_score for callers that cannot allocate
+ * device memory or hand over a workspace of their own: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  Same
+ * arguments and results as gtm_score, minus the workspace: the scratch is a
+ * fixed array inside the library's device image (gtm_score_static_scratch_bytes()
+ * = 16 MiB on every GPU the library runs on, held until the process ends).  A
+ * model and batch whose gtm_score_workspace_bytes() exceeds that is refused
+ * with GTM_ERR_INVALID.  The call allocates and frees nothing.  All calls on
+ * one GPU share the array: calls that overlap on one GPU (other streams, other
+ * threads) race; calls one after the other need nothing cleared between them. */
+size_t gtm_score_static_scratch_bytes(void);
+int gtm_score_static(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, int32_t first_graph,
+                     int32_t n_graphs, int32_t batch, int32_t *class_sum, void *stream);
+
 /* Scratch needed by gtm_fit. */
 size_t gtm_fit_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs);
 
