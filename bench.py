@@ -50,6 +50,8 @@ def parse():
     p.add_argument("--no-cpu", action="store_true")
     p.add_argument("--only-main", action="store_true", help="skip the short runs of the other four configurations")
     p.add_argument("--one-state", action="store_true", help="time the kernel on the headline state only")
+    p.add_argument("--copy-probe", action="store_true", help="only copy 256 MiB three times with a library copy kernel: "
+                   "calibrates the units of the FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc")
     p.add_argument("--save-state", default="", help="write the trained model to this .npz file after the run")
     p.add_argument("--load-state", default="", help="score a model saved by --save-state instead of training one "
                    "(the process then runs the scoring path only: what a profiler should see)")
@@ -195,6 +197,15 @@ def main():
 
     import numpy as np
     import torch
+
+    if args.copy_probe:
+        a = torch.empty(256 * 1024 * 1024 // 4, dtype=torch.int32, device="cuda").fill_(1)
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print("copied %d bytes three times" % (a.numel() * 4))
+        return
 
     from graphtsetlinmachine_amd import workloads
     from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine

@@ -8,7 +8,8 @@ import ctypes as C
 import os
 
 GTM_MAX_DEPTH = 8
-GTM_ABI_VERSION = 1
+GTM_ABI_VERSION = 2
+GTM_GRAPHS_COMPLEMENTARY = 1
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIBRARY_PATH = os.path.join(_HERE, "libgtm_hip.so")
@@ -50,7 +51,7 @@ class GraphsDesc(C.Structure):
         ("number_of_graphs", C.c_int32),
         ("number_of_node_types", C.c_int32),
         ("max_number_of_graph_nodes", C.c_int32),
-        ("reserved", C.c_int32),
+        ("flags", C.c_int32),
         ("total_nodes", C.c_int64),
         ("total_edges", C.c_int64),
         ("tiles", C.c_void_p),
@@ -94,6 +95,7 @@ PROTOTYPES = {
     "gtm_transform": (C.c_int, [_CFG, _GR, _ST, _I, _I, _I, _P, _SZ, _P, _P, _I, _P, _P]),
     "gtm_profile_enable": (C.c_int, [C.c_int]),
     "gtm_profile_read": (C.c_int, [C.POINTER(C.c_char_p), C.POINTER(C.c_int32), C.POINTER(C.c_double)]),
+    "gtm_graphs_properties": (C.c_int, [_CFG, _GR, _P, _P]),
     "gtm_tiles_bytes": (_SZ, [_CFG, _GR]),
     "gtm_build_tiles": (C.c_int, [_CFG, _GR, _P, _P]),
     "gtm_score_workspace_bytes": (_SZ, [_CFG, _GR, _I]),

@@ -291,6 +291,29 @@ __global__ void k_messages_scatter(const uint32_t *__restrict__ bitmap, int C, i
     }
 }
 
+// out[0] |= 1 if on some node a negated literal is not the complement of its positive literal
+// (literal k + hv against literal k, hv = literals / 2; bits past the literals are not looked at);
+// out[1] |= 1 if some graph has no nodes.  One thread per node, then one per graph.
+__global__ void k_graphs_properties(const uint32_t *__restrict__ X, int64_t total_nodes, int LA, int literals,
+                                    const uint32_t *__restrict__ n_nodes_arr, int G, uint32_t *out) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total_nodes) {
+        const uint32_t *row = X + i * LA;
+        const int hv = literals / 2;
+        bool bad = false;
+        if ((hv & 31) == 0) {
+            for (int w = 0; w < hv / 32; ++w) bad |= (row[w] ^ row[w + hv / 32]) != 0xFFFFFFFFu;
+        } else {
+            for (int k = 0; k < hv; ++k) {
+                const uint32_t pos = (row[k >> 5] >> (k & 31)) & 1u, neg = (row[(k + hv) >> 5] >> ((k + hv) & 31)) & 1u;
+                bad |= pos == neg;
+            }
+        }
+        if (bad) atomicOr(&out[0], 1u);
+    }
+    if (i < G && n_nodes_arr[i] == 0u) atomicOr(&out[1], 1u);
+}
+
 // p[0..n) = v, p[n..total) = 0
 __global__ void k_fill_u64(unsigned long long *p, int64_t n, unsigned long long v, int64_t total) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -679,6 +702,18 @@ int validate_state(const gtm_config *cfg, const gtm_state *s) {
 // Words of bit rows in a tile buffer, padded so that the row counts after them are 8-byte aligned.
 size_t tiles_words(const TileGeom &tg) { return ((size_t)tg.n_tiles * tg.rows * tg.tw + 1) & ~(size_t)1; }
 
+// Half tiles carry a fourth part after the rows, the row counts and the literal order: the positive
+// half of every node's literal words, by node SLOT ([tile][slot of the tile][LA / 2] words, zeros in
+// slots without a node), 16-byte aligned.  Phase 2 of k_tile_two_phase_half reads it instead of X:
+// half the bytes per candidate node, no lookup of the graph's first node, and a tile's share of it
+// stays in the XCD's L2 while the tile's clauses are worked through.
+size_t tiles_xpos_offset_words(const TileGeom &tg, int literals) {
+    return (tiles_words(tg) + (size_t)tg.rows * 2 + (size_t)literals + 3) & ~(size_t)3;
+}
+size_t tiles_xpos_words(const TileGeom &tg, int literals) {
+    return tg.half ? (size_t)tg.n_tiles * tg.tw * 32 * (size_t)(literals / 64) : 0;
+}
+
 // Inference on literal-major tiles (see score_tiles.h).
 int max_lane_words() {
     const char *e = getenv("GTM_TILE_LANE_WORDS");  // 1, 2 or 4: upper bound on words per lane (tuning aid)
@@ -686,9 +721,19 @@ int max_lane_words() {
     return v == 1 || v == 2 ? v : 4;
 }
 
+// Half tiles (positive rows only in LDS, k_tile_two_phase_half): a depth-1 model on a data set that
+// the caller has declared complementary, with word-aligned halves of 4 to 16 literal words per node.
+// GTM_NO_HALF_TILES (tuning aid) turns them off.
+bool half_tiles_allowed(const gtm_config *cfg, const gtm_graphs *g) {
+    const int LA = (cfg->literals - 1) / 32 + 1;
+    return cfg->depth == 1 && (g->flags & GTM_GRAPHS_COMPLEMENTARY) && cfg->literals % 64 == 0 && LA % 4 == 0 &&
+           LA <= 16 && !getenv("GTM_NO_HALF_TILES") && !getenv("GTM_NO_TWO_PHASE");
+}
+
 TileGeom geometry_for(const gtm_config *cfg, const gtm_graphs *g, int classes) {
     return tile_geometry(cfg->literals, g->number_of_node_types, g->max_number_of_graph_nodes, g->number_of_graphs,
-                         classes, max_lane_words(), cfg->depth > 1 ? tile_message_rows(cfg->message_size) : 0);
+                         classes, max_lane_words(), cfg->depth > 1 ? tile_message_rows(cfg->message_size) : 0,
+                         half_tiles_allowed(cfg, g), getenv("GTM_HALF_LANE_WORDS") ? atoi(getenv("GTM_HALF_LANE_WORDS")) : 0);
 }
 
 // The geometry every tile buffer of this process was built for, by address.  The driver loops
@@ -825,6 +870,52 @@ int launch_two_phase(const TileLayerArgs &a, int n_tiles, int la4, bool last, hi
     }
 }
 
+template <int NW, int LW, int LA4, bool LAST, bool FULL>
+int launch_two_phase_half_as(const TileLayerArgs &a, int n_tiles, hipStream_t st) {
+    const size_t lds = tile_lds_bytes(a.tg.rows - LA4 * 64, a.tg, a.K);  // the rows of the negated literals stay out
+    static thread_local size_t lds_set = 48 * 1024;
+    if (lds > lds_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)k_tile_two_phase_half<NW, LW, LA4, LAST, FULL>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
+        lds_set = lds;
+    }
+    profile_start(LAST ? "k_tile_two_phase_half<score>" : "k_tile_two_phase_half<layer0>", st);
+    hipLaunchKernelGGL((k_tile_two_phase_half<NW, LW, LA4, LAST, FULL>), dim3(n_tiles), dim3(NW * 64), lds, st, a);
+    if (int rc = check_launch("tile_two_phase_half")) return rc;
+    profile_stop(st);
+    return GTM_OK;
+}
+
+template <int NW, int LW, int LA4>
+int launch_two_phase_half_la(const TileLayerArgs &a, int n_tiles, bool last, hipStream_t st) {
+    const bool full = a.tg.tw == 64 * LW;
+    if (last)
+        return full ? launch_two_phase_half_as<NW, LW, LA4, true, true>(a, n_tiles, st)
+                    : launch_two_phase_half_as<NW, LW, LA4, true, false>(a, n_tiles, st);
+    return full ? launch_two_phase_half_as<NW, LW, LA4, false, true>(a, n_tiles, st)
+                : launch_two_phase_half_as<NW, LW, LA4, false, false>(a, n_tiles, st);
+}
+
+template <int NW, int LW>
+int launch_two_phase_half_lw(const TileLayerArgs &a, int n_tiles, int la4, bool last, hipStream_t st) {
+    switch (la4) {
+        case 1: return launch_two_phase_half_la<NW, LW, 1>(a, n_tiles, last, st);
+        case 2: return launch_two_phase_half_la<NW, LW, 2>(a, n_tiles, last, st);
+        case 3: return launch_two_phase_half_la<NW, LW, 3>(a, n_tiles, last, st);
+        default: return launch_two_phase_half_la<NW, LW, 4>(a, n_tiles, last, st);
+    }
+}
+
+int launch_two_phase_half(const TileLayerArgs &a, int n_tiles, int la4, bool last, hipStream_t st) {
+    constexpr int NW = 16;
+    switch (a.tg.lw) {
+        case 1: return launch_two_phase_half_lw<NW, 1>(a, n_tiles, la4, last, st);
+        case 2: return launch_two_phase_half_lw<NW, 2>(a, n_tiles, la4, last, st);
+        default: return launch_two_phase_half_lw<NW, 4>(a, n_tiles, la4, last, st);
+    }
+}
+
 template <int NW, int LW, int SRC, bool LAST>
 int launch_two_phase_wide_as(const TileLayerArgs &a, int n_tiles, int LA, hipStream_t st) {
     // rows (if staged), padding, class sums, and the first node and node count of the tile's graphs
@@ -871,7 +962,8 @@ int launch_two_phase_wide(const TileLayerArgs &a, int n_tiles, int LA, bool stag
 // Layer 0 can run in two phases (k_tile_two_phase) on tiles of whole-word graph slots staged in
 // LDS when a node has 4, 8, 12 or 16 literal words.  GTM_NO_TWO_PHASE (tuning aid) turns it off.
 bool two_phase_layer0(const Dims &d, const gtm_graphs *g, const TileGeom &tg) {
-    // the kernel addresses X with 32-bit byte offsets
+    if (tg.half) return true;  // such a geometry is only chosen for k_tile_two_phase_half (64-bit offsets into X)
+    // k_tile_two_phase addresses X with 32-bit byte offsets
     const bool x_fits = (uint64_t)g->total_nodes * d.LA * 4 < (1ull << 32);
     return tg.slot_words > 0 && tg.stage0 && d.LA % 4 == 0 && d.LA <= 16 && x_fits && !getenv("GTM_NO_TWO_PHASE");
 }
@@ -887,7 +979,11 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     const bool wide = !narrow && tg.slot_words > 0 && (int64_t)tg.rows * tg.tw / 4 < 65536 && !getenv("GTM_NO_TWO_PHASE");
     const bool two_phase = narrow || wide;
     const int stride0 = two_phase ? 8 + d.LA : w.list_stride;
-    if (two_phase)
+    if (tg.half)
+        hipLaunchKernelGGL(k_compile_clauses_half, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C,
+                           d.LA, d.B, d.filter, cfg->literals, g->number_of_node_types, tg.tw, order, w.lists, stride0,
+                           d.K, layers == 1 ? s->clause_weights : nullptr, w.wt);
+    else if (two_phase)
         hipLaunchKernelGGL(k_compile_clauses_two_phase, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state,
                            d.C, d.LA, d.B, d.filter, cfg->literals, g->number_of_node_types, cfg->literals,
                            tg.rows - 1, tg.tw, order, w.lists, stride0, d.K,
@@ -917,9 +1013,11 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     a.node_index = g->node_index;
     a.n_nodes = g->number_of_graph_nodes;
     a.X = g->X;
+    a.xpos = tg.half ? g->tiles + tiles_xpos_offset_words(tg, cfg->literals) : nullptr;
     auto layer0 = [&](int n_tiles, bool last) {
         a.lists = w.lists;
         a.stride = stride0;
+        if (tg.half) return launch_two_phase_half(a, n_tiles, d.LA / 4, last, st);
         if (narrow) return launch_two_phase(a, n_tiles, d.LA / 4, last, st);
         if (wide) return launch_two_phase_wide(a, n_tiles, d.LA, tg.stage0 != 0, last, st);
         return launch_tile_layer(a, n_tiles, tg.stage0 ? ROWS_STAGED : ROWS_GLOBAL, last, st);
@@ -1298,12 +1396,28 @@ int gtm_profile_read(const char **kernel_name, int32_t *launches, double *total_
     return GTM_OK;
 }
 
+int gtm_graphs_properties(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *properties, void *stream) {
+    Dims d;
+    if (int rc = validate(cfg, &d)) return rc;
+    if (int rc = validate_graphs(cfg, graphs, 0, 0)) return rc;
+    if (!properties) return fail(GTM_ERR_INVALID, "properties is NULL");
+    if (cfg->literals % 2 != 0) return fail(GTM_ERR_INVALID, "literals=%d is odd", cfg->literals);
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(k_fill_i32, dim3(1), dim3(TPB), 0, st, (int32_t *)properties, (int64_t)2, 0);
+    if (int rc = check_launch("fill")) return rc;
+    const int64_t items = graphs->total_nodes > graphs->number_of_graphs ? graphs->total_nodes : graphs->number_of_graphs;
+    hipLaunchKernelGGL(k_graphs_properties, dim3(blocks_for(items, TPB)), dim3(TPB), 0, st, graphs->X, graphs->total_nodes,
+                       d.LA, cfg->literals, graphs->number_of_graph_nodes, graphs->number_of_graphs, properties);
+    return check_launch("graphs_properties");
+}
+
 size_t gtm_tiles_bytes(const gtm_config *cfg, const gtm_graphs *graphs) {
     Dims d;
     if (validate(cfg, &d) || !graphs || graphs->number_of_graphs < 1 || graphs->number_of_node_types < 1) return 0;
     TileGeom tg = geometry_for(cfg, graphs, d.K);
     if (!tg.ok) return 0;
     // bit rows, one 64-bit population count per row, the literal order
+    if (tg.half) return (tiles_xpos_offset_words(tg, cfg->literals) + tiles_xpos_words(tg, cfg->literals)) * 4;
     return tiles_words(tg) * 4 + (size_t)tg.rows * 8 + (size_t)cfg->literals * 4;
 }
 
@@ -1330,6 +1444,13 @@ int gtm_build_tiles(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *t
     hipLaunchKernelGGL(k_row_order, dim3(blocks_for(cfg->literals, TPB)), dim3(TPB), 0, st,
                        (const unsigned long long *)counts, cfg->literals, (uint32_t *)(counts + (size_t)tg.rows * 2));
     if (int rc = check_launch("row_order")) return rc;
+    if (tg.half) {
+        const int64_t slots = (int64_t)tg.n_tiles * tg.tw * 32;
+        hipLaunchKernelGGL(k_build_xpos, dim3(blocks_for(slots, TPB)), dim3(TPB), 0, st, graphs->X, graphs->node_index,
+                           graphs->number_of_graph_nodes, graphs->number_of_graphs, d.LA, tg, slots,
+                           tiles + tiles_xpos_offset_words(tg, cfg->literals));
+        if (int rc = check_launch("build_xpos")) return rc;
+    }
     remember_tiles(tiles, tg, cfg, graphs);
     return GTM_OK;
 }

@@ -43,6 +43,8 @@ struct TileGeom {
     int lanes_per_graph;  // slot_words / lw (0 when slot_bits < 32)
     int ok;               // geometry supported by the tile kernels
     int stage0;           // the literal rows of layer 0 fit in LDS (else they are read from global memory)
+    int half;             // layer 0 keeps only the rows of the positive literals in LDS and evaluates a negated
+                          // literal as the complement of its positive row (k_tile_two_phase_half)
 };
 
 constexpr size_t TILE_LDS_BUDGET = 156 * 1024;  // of the 160 KB per CU
@@ -99,10 +101,35 @@ inline TileGeom tile_geometry_lw(int literals, int n_types, int max_nodes, int n
 // `gpt` graphs.  `message_rows` > 0 (models with message layers) asks that that many rows fit too;
 // if the literal rows of layer 0 and the message rows cannot both fit, the message rows win and
 // layer 0 reads its rows from global memory.
+// Rows of layer 0 that a half tile keeps in LDS: the positive literals, the node types, all ones.
+inline int tile_half_rows(int literals, int n_types) { return literals / 2 + n_types + 1; }
+
+// `allow_half`: the data set's negated literals are the complements of its positive ones on every
+// node and no graph is empty, so a tile may keep the positive rows only (TileGeom::half) - half the
+// LDS per graph, which buys twice the graphs per tile.
 inline TileGeom tile_geometry(int literals, int n_types, int max_nodes, int n_graphs, int classes, int max_lw = 4,
-                              int message_rows = 0) {
+                              int message_rows = 0, bool allow_half = false, int half_lw = 0) {
     if (max_nodes < 1) max_nodes = 1;
     const int rows0 = literals + n_types + 1;
+    if (allow_half && message_rows == 0 && max_nodes > 16) {
+        TileGeom full = tile_geometry(literals, n_types, max_nodes, n_graphs, classes, max_lw, 0, false);
+        TileGeom best_half{};
+        for (int lw = max_lw; lw >= 1; lw >>= 1) {
+            if (half_lw && lw != half_lw) continue;  // tuning aid: only this lane width, and then always taken
+            TileGeom g = tile_geometry_lw(literals, n_types, max_nodes, n_graphs, classes, lw,
+                                          tile_half_rows(literals, n_types));
+            if (!g.ok) continue;
+            if (!best_half.ok || (int64_t)(1 + g.lw) * best_half.gpt < (int64_t)(1 + best_half.lw) * g.gpt) best_half = g;
+        }
+        // taken when it covers more graphs per wave instruction than the tile of all rows
+        if (best_half.ok && (!full.ok || !full.stage0 || half_lw ||
+                             (int64_t)(1 + best_half.lw) * full.gpt < (int64_t)(1 + full.lw) * best_half.gpt)) {
+            best_half.half = 1;
+            best_half.stage0 = 1;
+            return best_half;
+        }
+        return full;
+    }
     TileGeom best{};
     for (int pass = 0; pass < 2; ++pass) {
         const int fit_rows = pass == 0 ? (rows0 > message_rows ? rows0 : message_rows) : message_rows;
@@ -171,6 +198,24 @@ __global__ void k_build_tiles(const uint32_t *__restrict__ X, const uint32_t *__
         }
     }
     tiles[i] = out;
+}
+
+// Half tiles: the positive half of the literal words of the node in every slot (zeros where the slot
+// holds no node).  One thread per slot.
+__global__ void k_build_xpos(const uint32_t *__restrict__ X, const uint32_t *__restrict__ node_index,
+                             const uint32_t *__restrict__ n_nodes_arr, int G, int LA, TileGeom tg, int64_t slots,
+                             uint32_t *__restrict__ xpos) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= slots) return;
+    const int per_tile = tg.tw * 32;
+    const int64_t tile = i / per_tile;
+    const int pos = (int)(i - tile * per_tile);
+    const int j = pos / tg.slot_bits, n = pos - j * tg.slot_bits;
+    const int64_t g = tile * tg.gpt + j;
+    const int half = LA / 2;
+    const bool has_node = j < tg.gpt && g < G && (uint32_t)n < n_nodes_arr[g];
+    const uint32_t *row = has_node ? X + ((int64_t)node_index[g] + n) * LA : X;
+    for (int w = 0; w < half; ++w) xpos[i * half + w] = has_node ? row[w] : 0u;
 }
 
 // Number of set bits of every row over all tiles (how often a literal holds in
@@ -317,6 +362,7 @@ struct TileLayerArgs {
     const uint32_t *node_index, *n_nodes;
     const uint32_t *X;      // [nodes][LA] node-major literal words (two-phase layer 0)
     const uint32_t *message_rows;  // [tiles of the launch][M + 2][tw] (message layers, built by k_tile_pack_messages)
+    const uint32_t *xpos;   // [tiles][tw * 32 slots][LA / 2]: the positive literal words by node slot (half tiles)
 };
 
 // Rows a message layer keeps in LDS: M message rows, the all-ones row, the row of graphs without nodes.
@@ -1352,6 +1398,433 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
         // without a second clause this repeats the first one and drops the result: keeping the
         // sequence of loads the same on every trip lets the waits stay partial
         mb = *reinterpret_cast<const Words<4 * LA4> *>(rec_b + 8);
+        ea = *reinterpret_cast<const Packed8 *>(rec_a);
+        begin(pb, eb, wt_b, truth_b);
+        pb.live = has_b;
+        finish(pa, ma);
+    }
+    finish(pb, mb);
+    if (!LAST) return;
+    __syncthreads();
+    const int64_t g0 = (int64_t)tile * tg.gpt;
+    for (int i = tid; i < tg.gpt * K; i += NT) {
+        int64_t g = g0 + i / K;
+        if (g >= a.first_graph && g < (int64_t)a.first_graph + a.n_graphs)
+            a.class_sum[(g - a.first_graph) * K + (i % K)] = sums[i];
+    }
+}
+
+
+// ---------------------------------------------------------------------------
+// The two-phase layer 0 on HALF tiles: LDS holds only the rows of the positive
+// literals (plus the node-type rows and the all-ones row), and a negated literal
+// l + hv is evaluated as the complement of row l.  That is exact where the data
+// set's negated literals are the complements of its positive ones on every node
+// (graphs.py:91-98,148-159 build them so; the caller asserts it, GTM_GRAPHS_COMPLEMENTARY)
+// and no graph is empty: on node slots past a graph's nodes the complement is 1, but the
+// node-type row, which every clause ANDs first, is 0 there.  Half the rows per graph buy
+// twice the graphs per tile: the scalar work, the address arithmetic and the phase-2 loads
+// of a (clause, tile) pair are spread over twice as many graphs.
+//
+// Compiled clause (same 8 + LA words as k_compile_clauses_two_phase): entry 0 =
+// variant (7 or 15 rows) | needs-phase-2 << 8 | positive pairs << 12; entry 1 = the
+// node-type row; then literal rows in PAIRS, 3 or 7 of them: first the pairs of positive
+// literals (an odd one out is paired with the all-ones row), then the pairs of negated
+// ones (padded with the all-zero words that follow the rows in LDS).  With the signs fixed
+// per pair, a pair costs one 3-input bit operation per word of the lane - acc & a & b or
+// acc & ~(a | b) - and the clause's pattern (how many positive pairs) selects one of 8
+// straight-line variants with a single scalar jump.
+// The filter takes the clause's rarest literals, at most 14, as many as fit the pairs.
+
+__global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C, int chunks, int B, uint32_t filter,
+                                       int literals, int n_types, int tw, const uint32_t *__restrict__ order,
+                                       uint32_t *__restrict__ records, int record_words, int K,
+                                       const int32_t *__restrict__ weights, int32_t *__restrict__ wt) {
+    __shared__ uint32_t chosen_of_wave[4][16];
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (c >= C) return;  // whole waves leave; no barrier below
+    uint32_t *chosen = chosen_of_wave[(threadIdx.x >> 6) & 3];
+    const int hv = literals >> 1;
+    const uint32_t row16 = (uint32_t)tw >> 2;  // a row in units of 16 bytes (tw is a multiple of 4)
+    const uint32_t ones_row = (uint32_t)(hv + n_types), zero_row = ones_row + 1u;  // the zeroed words after the rows
+    uint32_t *rec = records + (int64_t)c * record_words;
+    uint16_t *e = reinterpret_cast<uint16_t *>(rec);
+    const uint32_t *inc = bank + (int64_t)c * chunks * B + (B - 1);
+    // the clause's 14 rarest included literals, in `order`
+    int n = 0;
+    for (int r0 = 0; r0 < literals; r0 += 64) {
+        const int r = r0 + lane;
+        const uint32_t lit = r < literals ? order[r] : 0u;
+        const uint32_t w = lit >> 5;
+        uint32_t word = inc[(int64_t)w * B];
+        if ((int)w == chunks - 1) word &= filter;
+        const bool included = r < literals && ((word >> (lit & 31)) & 1u);
+        const unsigned long long mask = __ballot(included);
+        const int at = n + __popcll(mask & ((1ull << lane) - 1ull));
+        if (included && at < 14) chosen[at] = lit;
+        n += __popcll(mask);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+    int taken = n < 14 ? n : 14;
+    const uint32_t lit = lane < taken ? chosen[lane] : 0u;
+    bool positive = lane < taken && (int)lit < hv, negative = lane < taken && (int)lit >= hv;
+    int p = __popcll(__ballot(positive)), q = __popcll(__ballot(negative));
+    // 7 pairs hold p positives and q negatives if ceil(p / 2) + ceil(q / 2) <= 7: 14 literals with an
+    // odd number of each sign do not fit, and then the least rare of the 14 is left to phase 2
+    if (p + q == 14 && (p & 1)) {
+        --taken;
+        if (lane == taken) positive = negative = false;
+        p = __popcll(__ballot(positive)), q = __popcll(__ballot(negative));
+    }
+    const int a = (p + 1) >> 1, b = (q + 1) >> 1;
+    const int pairs = a + b <= 3 ? 3 : 7;
+    const int pos_rank = __popcll(__ballot(positive) & ((1ull << lane) - 1ull));
+    const int neg_rank = __popcll(__ballot(negative) & ((1ull << lane) - 1ull));
+    // the 16 entries are put together in LDS (a wave's LDS accesses are carried out in order) and
+    // written out once: unused positive slots take the all-ones row, unused negative ones the zeros
+    uint32_t *slots = chosen;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    if (lane < 16) {
+        uint32_t v = (lane >= 2 && lane < 2 + 2 * a ? ones_row : zero_row) * row16;
+        if (lane == 0) v = (uint32_t)((pairs == 3 ? 7 : 15) | (n > taken ? 0x100 : 0) | (a << 12));
+        if (lane == 1) v = (uint32_t)(hv + c % n_types) * row16;
+        slots[lane] = v;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    if (positive) slots[2 + pos_rank] = lit * row16;
+    if (negative) slots[2 + 2 * a + neg_rank] = (lit - (uint32_t)hv) * row16;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+    if (lane < 16) e[lane] = (uint16_t)slots[lane];
+    for (int w = lane; w < chunks; w += 64) {
+        uint32_t word = inc[(int64_t)w * B];
+        if (w == chunks - 1) word &= filter;
+        rec[8 + w] = word;
+    }
+    if (weights)
+        for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
+}
+
+// acc &= the PAIRS row pairs in r, the first A of them positive, the others negated
+template <int LW, int PAIRS, int A>
+__device__ __forceinline__ void half_combine(LaneWords<LW> &acc, const LaneWords<LW> *r) {
+#pragma unroll
+    for (int j = 0; j < PAIRS; ++j)
+#pragma unroll
+        for (int u = 0; u < LW; ++u)
+            acc.w[u] = j < A ? acc.w[u] & r[2 * j].w[u] & r[2 * j + 1].w[u] : acc.w[u] & ~(r[2 * j].w[u] | r[2 * j + 1].w[u]);
+}
+
+template <int NWAVES, int LW, int LA4, bool LAST, bool FULL>
+__global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerArgs a) {
+    extern __shared__ uint32_t lds[];
+    const TileGeom &tg = a.tg;
+    const int tw = tg.tw, C = a.C, K = a.K;
+    constexpr int NT = NWAVES * 64;
+    constexpr int LA = 4 * LA4;
+    const int hv = LA * 16;                      // positive literals = LDS rows 0 .. hv - 1
+    const int rows_lds = tg.rows - hv;           // + node types + all ones
+    uint32_t *bt = lds;
+    int32_t *sums = (int32_t *)(lds + (size_t)rows_lds * tw + TILE_LDS_PAD_WORDS);
+    const int tile = a.tile0 + blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    uint32_t *bitmap = a.bitmap + (int64_t)blockIdx.x * C * tw;
+
+    {  // the tile's positive rows, then its node-type rows and the all-ones row -> LDS
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.tiles + (int64_t)tile * tg.rows * tw);
+        uint4 *dst = reinterpret_cast<uint4 *>(bt);
+        const int n4 = (rows_lds * tw) >> 2, first4 = (hv * tw) >> 2, skip4 = (hv * tw) >> 2;  // rows hv .. 2 hv - 1 stay out
+        for (int i = tid; i < n4; i += NT * 4) {
+            uint4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int at = i + u * NT;
+                v[u] = at < n4 ? src[at < first4 ? at : at + skip4] : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int at = i + u * NT;
+                if (at < n4) dst[at] = v[u];
+            }
+        }
+        for (int i = tid; i < TILE_LDS_PAD_WORDS + tg.gpt * K; i += NT) bt[(size_t)rows_lds * tw + i] = 0;
+    }
+    __syncthreads();
+
+    const bool active = FULL || lane * LW < tw;
+    const char *col = reinterpret_cast<const char *>(bt + lane * LW);
+
+    // the graph whose slot this lane's words belong to, and the literal words of the node at the lane's first bit
+    const int lpg = tg.lanes_per_graph;
+    const int lane_j = lane / lpg;
+    const int64_t lane_g = (int64_t)tile * tg.gpt + lane_j;
+    const bool has_graph = active && lane_j < tg.gpt && lane_g < a.G;
+    // the positive literal words of the node slots of this lane's words (LA / 2 words per slot)
+    const char *x_base = reinterpret_cast<const char *>(a.xpos) + (int64_t)tile * tw * 32 * (LA * 2);
+    const char *x_lane = x_base + (active ? lane * LW * 32 : 0) * (LA * 2);
+
+    // lane p adds weight k = p % K to graph j = p / K of the tile, for p = lane, lane + 64, lane + 128, lane + 192
+    const int pairs = tg.gpt * K;
+    constexpr int VOTES = 4;
+    uint32_t vote_k_bytes[VOTES], vote_shift[VOTES];
+    bool vote_on[VOTES];
+#pragma unroll
+    for (int v = 0; v < VOTES; ++v) {
+        const int q = lane + 64 * v, j = q / K;
+        vote_on[v] = LAST && q < pairs;
+        vote_k_bytes[v] = vote_on[v] ? (uint32_t)(q - j * K) * 4u : 0u;
+        vote_shift[v] = vote_on[v] ? (uint32_t)(j * lpg) : 0u;  // first lane of the pair's graph
+    }
+    const int my_shift = (lane < tg.gpt ? lane : 0) * lpg;
+    const unsigned long long slot_lanes = lpg >= 64 ? ~0ull : (1ull << lpg) - 1ull;
+
+    auto any_bit = [](const LaneWords<LW> &x) {
+        uint32_t m = x.w[0];
+#pragma unroll
+        for (int u = 1; u < LW; ++u) m |= x.w[u];
+        return m != 0;
+    };
+    auto entry_of = [](const Packed8 &rec, int i) { return ((rec.v[i >> 1] >> ((i & 1) * 16)) & 0xFFFFu) << 4; };
+    // a positive literal is violated where the node lacks it, a negated one (include words LA / 2 ..)
+    // where the node has it: (include_pos & ~x) | (include_neg & x), one 3-input operation per word
+    auto violates = [](const Words<LA> &include, const uint2 *x) {
+        uint32_t violated = 0;
+#pragma unroll
+        for (int q = 0; q < LA4; ++q) {
+            const uint2 v = x[q];
+            violated |= (include.v[2 * q] & ~v.x) | (include.v[2 * q + LA / 2] & v.x) | (include.v[2 * q + 1] & ~v.y) |
+                        (include.v[2 * q + 1 + LA / 2] & v.y);
+        }
+        return violated != 0;
+    };
+    // the word set with only `bit` set (bit < 32 * LW)
+    auto one_hot = [](uint32_t bit) {
+        LaneWords<LW> m;
+#pragma unroll
+        for (int u = 0; u < LW; ++u) m.w[u] = (int)(bit >> 5) == u ? 1u << (bit & 31u) : 0u;
+        return m;
+    };
+
+    struct Pending {
+        LaneWords<LW> acc;
+        uint2 x[LA4];
+        uint32_t bit;            // the node slot this lane has under test (index into its LW words), ~0 if none
+        bool live, test;         // wave-uniform: a clause is pending / its phase 2 runs
+        unsigned long long nz;   // lanes with a surviving slot after phase 1
+        int weight[VOTES];
+        const int32_t *weights;
+        char *truth_out;
+    };
+
+    // Phase 1 and the loads of phase 2.  Every load is issued by all lanes whatever the clause
+    // does, so that the number of loads in flight is known when the pending clause is finished.
+    auto begin = [&](Pending &p, const Packed8 &rec, const int32_t *weights_of_clause, char *truth_out) {
+        p.live = true;
+        p.weights = weights_of_clause;
+        p.truth_out = truth_out;
+        if (LAST) {  // needed only if the clause fires
+            const char *wb = reinterpret_cast<const char *>(weights_of_clause);
+#pragma unroll
+            for (int v = 0; v < VOTES; ++v) p.weight[v] = *reinterpret_cast<const int32_t *>(wb + vote_k_bytes[v]);
+        }
+        const uint32_t header = rec.v[0] & 0xFFFFu;
+        const uint32_t positive_pairs = header >> 12;
+        LaneWords<LW> acc, r[14];
+        acc.load(col + entry_of(rec, 1));  // the node-type row: zero past the graphs' nodes and in unused lanes
+        if (!FULL && !active)
+#pragma unroll
+            for (int u = 0; u < LW; ++u) acc.w[u] = 0u;
+        if ((header & 0xFFu) > 7u) {
+#pragma unroll
+            for (int i = 0; i < 14; ++i) r[i].load(col + entry_of(rec, i + 2));
+            switch (positive_pairs) {
+                case 0: half_combine<LW, 7, 0>(acc, r); break;
+                case 1: half_combine<LW, 7, 1>(acc, r); break;
+                case 2: half_combine<LW, 7, 2>(acc, r); break;
+                case 3: half_combine<LW, 7, 3>(acc, r); break;
+                case 4: half_combine<LW, 7, 4>(acc, r); break;
+                case 5: half_combine<LW, 7, 5>(acc, r); break;
+                case 6: half_combine<LW, 7, 6>(acc, r); break;
+                default: half_combine<LW, 7, 7>(acc, r); break;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 6; ++i) r[i].load(col + entry_of(rec, i + 2));
+            switch (positive_pairs) {
+                case 0: half_combine<LW, 3, 0>(acc, r); break;
+                case 1: half_combine<LW, 3, 1>(acc, r); break;
+                case 2: half_combine<LW, 3, 2>(acc, r); break;
+                default: half_combine<LW, 3, 3>(acc, r); break;
+            }
+        }
+        p.nz = __ballot(any_bit(acc));
+        p.test = (header & 0x100u) && p.nz != 0;
+        // lowest surviving slot of the lane: the lowest set bit of its first word that has one
+        // (__ffs(0) - 1 is ~0, which survives the OR: no slot)
+        uint32_t first_word = acc.w[LW - 1], first_base = (uint32_t)(LW - 1) * 32u;
+#pragma unroll
+        for (int u = LW - 2; u >= 0; --u) {
+            const bool here = acc.w[u] != 0u;
+            first_word = here ? acc.w[u] : first_word;
+            first_base = here ? (uint32_t)u * 32u : first_base;
+        }
+        const uint32_t bit = (uint32_t)(__ffs(first_word) - 1) | first_base;
+        p.bit = has_graph ? bit : ~0u;
+        // lanes with nothing to test all read the tile's first slot (one cache line for the wave)
+        const uint2 *x = reinterpret_cast<const uint2 *>(p.bit != ~0u ? x_lane + p.bit * (LA * 2u) : x_base);
+#pragma unroll
+        for (int q = 0; q < LA4; ++q) p.x[q] = x[q];
+        p.acc = acc;
+    };
+
+    // The rest of phase 2, then the clause's votes (or its truth row).
+    auto finish = [&](Pending &p, const Words<LA> &include) {
+        if (!p.live) return;
+        p.live = false;
+        LaneWords<LW> acc = p.acc;
+        unsigned long long nz = p.nz;
+        bool settled = false;
+        if (LAST && p.test) {
+            // Class sums only ask whether the clause is true at SOME node of a graph
+            // (kernels.py:297-308): a lane whose first candidate holds has settled that for its graph.
+            // Only a lane whose first candidate failed and that has others needs more tests (rare: then
+            // the exact path below runs).
+            const bool tested = p.bit != ~0u;
+            const bool failed = violates(include, p.x) && tested;
+            int slots_left = 0;
+#pragma unroll
+            for (int u = 0; u < LW; ++u) slots_left += __popc(acc.w[u]);
+            if (__ballot(failed && slots_left > 1) == 0ull) {
+                nz = __ballot(tested && !failed);
+                settled = true;
+            }
+        }
+        if (p.test && !settled) {
+            const bool tested = p.bit != ~0u;
+            const bool failed = violates(include, p.x) && tested;
+            // the lane's other surviving slots
+            const LaneWords<LW> hot = one_hot(p.bit);
+            LaneWords<LW> rest;
+#pragma unroll
+            for (int u = 0; u < LW; ++u) {
+                rest.w[u] = tested ? acc.w[u] & ~hot.w[u] : 0u;
+                acc.w[u] = failed ? rest.w[u] : acc.w[u];
+            }
+            if (__ballot(any_bit(rest)) != 0) {
+                int others = 0;
+#pragma unroll
+                for (int u = 0; u < LW; ++u) others += __popc(rest.w[u]);
+                if (__builtin_expect(__ballot(others >= TWO_PHASE_WALK_FROM) != 0, 0)) {
+                    // Phase 1 has left some lane several slots (its literals hold nearly everywhere), and
+                    // testing them costs a memory round trip each.  The rows of ALL the clause's literals are
+                    // ANDed instead (row l is literal l's; a negated literal l + hv takes the complement of
+                    // row l; unused reads take the all-ones row, resp. the zeroed words after the rows).
+                    acc = p.acc;
+                    const uint32_t row_bytes = (uint32_t)tw * 4u;
+                    const uint32_t ones = (uint32_t)(rows_lds - 1), zeros = (uint32_t)rows_lds;
+                    uint32_t include_of_lane = 0u;  // lane w holds include word w: one copy of the loop below
+#pragma unroll
+                    for (int w = 0; w < LA; ++w) include_of_lane = lane == w ? include.v[w] : include_of_lane;
+#pragma unroll 1
+                    for (int w = 0; w < LA; ++w) {
+                        uint32_t m = __builtin_amdgcn_readlane(include_of_lane, w);
+                        const bool negated = w >= LA / 2;
+                        const uint32_t first = (uint32_t)((negated ? w - LA / 2 : w) * 32), unused = negated ? zeros : ones;
+                        while (m) {
+                            LaneWords<LW> r[8];
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) {
+                                const uint32_t row = m ? first + (uint32_t)__builtin_ctz(m) : unused;
+                                m &= m - 1u;
+                                r[u].load(col + row * row_bytes);
+                            }
+                            if (negated) {
+#pragma unroll
+                                for (int u = 0; u < 8; ++u)
+#pragma unroll
+                                    for (int v = 0; v < LW; ++v) acc.w[v] &= ~r[u].w[v];
+                            } else {
+#pragma unroll
+                                for (int u = 0; u < 8; ++u)
+#pragma unroll
+                                    for (int v = 0; v < LW; ++v) acc.w[v] &= r[u].w[v];
+                            }
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < LW; ++u) {
+                        uint32_t todo = rest.w[u];
+                        while (todo) {
+                            const int b = __ffs(todo) - 1;
+                            todo &= todo - 1;
+                            const uint2 *x = reinterpret_cast<const uint2 *>(x_lane + (u * 32 + b) * (LA * 2u));
+                            if (violates(include, x)) acc.w[u] &= ~(1u << b);
+                        }
+                    }
+                }
+            }
+            nz = __ballot(any_bit(acc));
+        }
+        if (!LAST) {
+            if (active) acc.store(p.truth_out);
+            return;
+        }
+        if (nz == 0) return;
+        // graph j owns lanes [j * lanes_per_graph, (j + 1) * lanes_per_graph)
+        if (lpg <= 32 && pairs <= 64 * VOTES) {
+            const uint32_t m = (uint32_t)slot_lanes;
+#pragma unroll
+            for (int v = 0; v < VOTES; ++v)
+                if (vote_on[v] && ((uint32_t)(nz >> vote_shift[v]) & m) != 0) atomicAdd(&sums[lane + 64 * v], p.weight[v]);
+        } else {
+            const unsigned long long gm = __ballot(lane < tg.gpt && ((nz >> my_shift) & slot_lanes) != 0);
+            for (int q = lane; q < pairs; q += 64) {
+                const int j = q / K, k = q - j * K;
+                if ((gm >> j) & 1ull) atomicAdd(&sums[q], p.weights[k]);
+            }
+        }
+    };
+
+    // Clause records: the 8 words of row entries are fetched one clause ahead of phase 1, the
+    // include mask at the start of the clause's phase 1 (it is first needed when the clause is
+    // finished, one phase 1 later).  Pointers step by NWAVES clauses; past the end they stay on
+    // the wave's last clause (a valid address whose data is not used).
+    const int64_t rec_step = (int64_t)NWAVES * a.stride;
+    const int wt_step = NWAVES * K;
+    const int64_t truth_step = (int64_t)NWAVES * tw * 4;
+    const int first = wave < C ? wave : 0;
+    const uint32_t *rec_a = a.lists + (int64_t)first * a.stride;
+    const int32_t *wt_a = LAST ? a.wt + (int64_t)first * K : nullptr;
+    char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
+    Packed8 ea = *reinterpret_cast<const Packed8 *>(rec_a);
+    Words<LA> ma, mb;
+    Pending pa, pb;
+    pa.live = pb.live = false;
+    for (int c = wave; c < C; c += 2 * NWAVES) {
+        const bool has_b = c + NWAVES < C;
+        const uint32_t *rec_b = has_b ? rec_a + rec_step : rec_a;
+        const int32_t *wt_b = LAST ? (has_b ? wt_a + wt_step : wt_a) : nullptr;
+        char *truth_b = has_b ? truth_a + truth_step : truth_a;
+        ma = *reinterpret_cast<const Words<LA> *>(rec_a + 8);
+        const Packed8 eb = *reinterpret_cast<const Packed8 *>(rec_b);
+        begin(pa, ea, wt_a, truth_a);
+        finish(pb, mb);
+        const bool has_a = c + 2 * NWAVES < C;
+        rec_a = has_a ? rec_b + rec_step : rec_b;
+        if (LAST) wt_a = has_a ? wt_b + wt_step : wt_b;
+        truth_a = has_a ? truth_b + truth_step : truth_b;
+        // without a second clause this repeats the first one and drops the result: keeping the
+        // sequence of loads the same on every trip lets the waits stay partial
+        mb = *reinterpret_cast<const Words<LA> *>(rec_b + 8);
         ea = *reinterpret_cast<const Packed8 *>(rec_a);
         begin(pb, eb, wt_b, truth_b);
         pb.live = has_b;

@@ -77,6 +77,7 @@ class _DeviceGraphs:
         self.desc = d
         self.tiles = None
         self._tiles_key = None
+        self._complementary = None  # not looked at yet
 
     def ensure_tiles(self, cfg):
         """Build the literal-major tile layout once per data set and tile
@@ -84,12 +85,22 @@ class _DeviceGraphs:
         layout keep tiles = NULL.  The geometry depends on the model's
         sizes, so a data set handed to a model of another shape is tiled
         again."""
-        key = (cfg.classes, cfg.literals, cfg.depth, cfg.message_size, os.environ.get("GTM_TILE_LANE_WORDS"))
+        key = (cfg.classes, cfg.literals, cfg.depth, cfg.message_size, os.environ.get("GTM_TILE_LANE_WORDS"),
+               os.environ.get("GTM_NO_HALF_TILES"), os.environ.get("GTM_NO_TWO_PHASE"),
+               os.environ.get("GTM_HALF_LANE_WORDS"))
         if self._tiles_key == key:
             return
         self._tiles_key = key
         self.tiles = None
         self.desc.tiles = None
+        if self._complementary is None and cfg.literals % 2 == 0:
+            # one look at the data on the device: are the negated literals the complements of the
+            # positive ones everywhere, and has every graph a node?  (What Graphs builds - but X is a
+            # public array.)  Then the tile kernels may keep half the rows on chip.
+            found = torch.zeros(2, dtype=torch.int32, device=_device())
+            _abi.call("gtm_graphs_properties", ctypes.byref(cfg), ctypes.byref(self.desc), _ptr(found), _stream())
+            self._complementary = not found.cpu().numpy().any()
+        self.desc.flags = _abi.GTM_GRAPHS_COMPLEMENTARY if self._complementary else 0
         nbytes = _abi.lib.gtm_tiles_bytes(ctypes.byref(cfg), ctypes.byref(self.desc))
         if nbytes == 0:
             return

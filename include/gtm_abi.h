@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define GTM_ABI_VERSION 1
+#define GTM_ABI_VERSION 2
 #define GTM_MAX_DEPTH 8
 
 #define GTM_OK 0
@@ -63,6 +63,13 @@ typedef struct gtm_config {
     uint64_t seed;                        /* Philox key */
 } gtm_config;
 
+/* gtm_graphs.flags: on every node, literal k + LITERALS/2 is the complement of
+ * literal k (what Graphs builds, graphs.py:91-98,148-159: a property sets k and
+ * clears its negation), and every graph has at least one node.  With it the
+ * tile kernels may keep only the positive literals' rows on chip.  Check with
+ * gtm_graphs_properties(); never set it for data the check has not passed. */
+#define GTM_GRAPHS_COMPLEMENTARY 1
+
 /* Device copies of the arrays of a Graphs object (graphs.py:38,101-112,128-129). */
 typedef struct gtm_graphs {
     const uint32_t *X;                          /* [total_nodes][LA_CHUNKS] */
@@ -75,7 +82,7 @@ typedef struct gtm_graphs {
     int32_t number_of_graphs;
     int32_t number_of_node_types;      /* Graphs.number_of_node_types() */
     int32_t max_number_of_graph_nodes; /* must be <= gtm_config.max_nodes */
-    int32_t reserved;
+    int32_t flags;                     /* GTM_GRAPHS_* bits the caller vouches for; 0 is always valid */
     int64_t total_nodes;
     int64_t total_edges;
     const uint32_t *tiles; /* optional: literal-major tiles from gtm_build_tiles, or NULL */
@@ -167,6 +174,14 @@ int gtm_update_message(const gtm_config *cfg, uint64_t step, int32_t bank, uint3
  * has no such layout (then leave gtm_graphs.tiles NULL); gtm_build_tiles()
  * fills a caller-owned buffer of that size from X / node_type. */
 size_t gtm_tiles_bytes(const gtm_config *cfg, const gtm_graphs *graphs);
+
+/* No counterpart in the reference (its kernels read X as it is).  Looks at the
+ * data set once on the device: properties[0] = 1 if on some node a negated
+ * literal is not the complement of its positive one, properties[1] = 1 if
+ * some graph has no nodes (two uint32 in device memory).  Both 0 entitles the
+ * caller to set GTM_GRAPHS_COMPLEMENTARY before gtm_tiles_bytes /
+ * gtm_build_tiles and in every later call with that data set. */
+int gtm_graphs_properties(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *properties, void *stream);
 int gtm_build_tiles(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *tiles, void *stream);
 
 /* Scratch needed by gtm_score for sub-batches of `batch` graphs. */

@@ -110,6 +110,18 @@ class Device:
                   _ptr(clause_node), _ptr(n_incl), _ptr(cx), _ptr(updates), _stream())
 
     # --- driver loops ----------------------------------------------------
+    def properties(self):
+        """(some negated literal is not its positive one's complement, some graph has no nodes)"""
+        found = torch.full((2,), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+        _abi.call("gtm_graphs_properties", ctypes.byref(self.acfg), ctypes.byref(self.dg.desc), _ptr(found), _stream())
+        return tuple(int(v) for v in found.cpu().numpy())
+
+    def declare_complementary(self):
+        """Set GTM_GRAPHS_COMPLEMENTARY if the data set passes the library's check."""
+        ok = self.properties() == (0, 0)
+        self.dg.desc.flags = _abi.GTM_GRAPHS_COMPLEMENTARY if ok else 0
+        return ok
+
     def build_tiles(self):
         nbytes = _abi.lib.gtm_tiles_bytes(ctypes.byref(self.acfg), ctypes.byref(self.dg.desc))
         if nbytes == 0:

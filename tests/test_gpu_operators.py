@@ -727,3 +727,106 @@ def test_tiles_built_for_another_configuration_are_refused():
         dev.score(0, graphs.number_of_graphs, 8)
     dev.dg.desc.tiles = dev.tiles.data_ptr()
     assert np.array_equal(dev.score(0, graphs.number_of_graphs, 8), want)
+
+
+HALF_TILE_SHAPES = [
+    # 4, 8, 12, 16 literal words per node; one word per graph up to 64; one to three node types
+    dict(seed=51, g=dict(n_graphs=90, max_nodes=31, min_nodes=17, hv_size=64), classes=10, clauses=200, half=False),
+    dict(seed=52, g=dict(n_graphs=47, max_nodes=361, min_nodes=300, hv_size=128, max_degree=0), classes=10, clauses=150),
+    dict(seed=53, g=dict(n_graphs=45, max_nodes=100, min_nodes=20, hv_size=192, n_symbols=12), classes=3, clauses=90),
+    dict(seed=54, g=dict(n_graphs=60, max_nodes=50, min_nodes=17, hv_size=256, n_symbols=12, node_types=("a", "b")),
+         classes=4, clauses=64),
+    dict(seed=55, g=dict(n_graphs=7, max_nodes=2048, min_nodes=1500, hv_size=64, max_degree=0, node_types=("a", "b", "c")),
+         classes=2, clauses=40, half=False),
+    # more (graph, class) pairs per tile than four per lane
+    dict(seed=56, g=dict(n_graphs=30, max_nodes=361, min_nodes=200, hv_size=128, n_symbols=20, max_degree=0), classes=70,
+         clauses=50),
+]
+
+
+@pytest.mark.parametrize("shape", HALF_TILE_SHAPES, ids=lambda s: "half%d" % s["seed"])
+@pytest.mark.parametrize("density", [0.0, 0.02, 0.2])
+def test_half_tile_scoring_equals_oracle(shape, density):
+    """Depth-1 gtm_score on tiles whose LDS copy holds the positive literals' rows only (negated
+    literals as complements; data declared complementary after the library's own check) == oracle
+    == the bitmap path == the tiles of all rows."""
+    from tests.gpu_harness import Device
+
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    cfg = helpers.oracle_config(graphs, classes=shape["classes"], clauses=shape["clauses"])
+    model = helpers.random_model(shape["seed"], cfg, 1, include_density=density)
+    top = cfg.state_bits - 1
+    model.ta_state[3, :, top] = 0  # an empty clause among the random ones
+    rng = np.random.default_rng(shape["seed"])
+    used = np.unique(graphs.hypervectors)
+    hv = graphs.hypervector_size
+    # clauses of positive literals only, of negated literals only (each holds at nearly every node), of one
+    # literal, of exactly 7 + 7 (one of the 14 rarest is left to phase 2), and with x and NOT x together
+    def include(c, literals):
+        model.ta_state[c, :, top] = 0
+        for l in literals:
+            model.ta_state[c, l // 32, top] |= np.uint32(1 << (l % 32))
+    include(4, rng.choice(used, size=min(5, used.size), replace=False))
+    include(5, hv + rng.choice(hv, size=30, replace=False))
+    include(6, [int(used[0])])
+    include(7, [hv + int(used[0])])
+    include(8, list(rng.choice(used, size=min(7, used.size), replace=False)) + list(hv + rng.choice(hv, size=7, replace=False)))
+    include(9, [int(used[1]), hv + int(used[1])])
+    include(10, hv + rng.choice(hv, size=3, replace=False))
+    include(11, list(rng.choice(used, size=min(3, used.size), replace=False)) + list(hv + rng.choice(hv, size=2, replace=False)))
+    dev = Device(model, graphs)
+    G = graphs.number_of_graphs
+    plain = dev.score(0, G, G)
+    assert dev.build_tiles()
+    full = dev.score(0, G, G)
+    assert dev.declare_complementary()
+    assert dev.build_tiles()
+    _abi.call("gtm_profile_enable", 1)
+    half = dev.score(0, G, G)
+    name, launches, total = ctypes.c_char_p(), ctypes.c_int32(), ctypes.c_double()
+    _abi.call("gtm_profile_read", ctypes.byref(name), ctypes.byref(launches), ctypes.byref(total))
+    _abi.call("gtm_profile_enable", 0)
+    # the half tiles are taken where they hold more graphs than the tiles of all rows
+    expected = "k_tile_two_phase_half<score>" if shape.get("half", True) else "k_tile_two_phase<score>"
+    assert name.value.decode() == expected
+    assert np.array_equal(full, plain) and np.array_equal(half, plain)
+    sample = sorted(set([0, 1, G // 2, G - 1]))
+    assert np.array_equal(half[sample], o.score(model, graphs, sample))
+    assert np.array_equal(dev.score(3, G - 5, G), plain[3:G - 2])  # a range that starts and ends inside tiles
+    # one-launch training on the same tiles follows the oracle
+    Y = o.encode_labels(rng.integers(0, cfg.classes, size=G), cfg.classes, cfg.threshold)
+    o.fit(model, graphs, Y)
+    dev.fit(Y, 0, G, 0)
+    ta, _, w = dev.download()
+    assert np.array_equal(w, model.clause_weights) and np.array_equal(ta, model.ta_state)
+    assert np.array_equal(dev.score(0, G, G)[sample], o.score(model, graphs, sample))
+
+
+def test_data_that_is_not_complementary_is_detected_and_keeps_all_rows():
+    from tests.gpu_harness import Device
+
+    graphs = helpers.random_graphs(57, n_graphs=20, max_nodes=60, min_nodes=20, hv_size=64)
+    cfg = helpers.oracle_config(graphs, classes=3, clauses=40)
+    model = helpers.random_model(57, cfg, 1, include_density=0.03)
+    assert Device(model, graphs).properties() == (0, 0)
+    # a node whose literal 5 and its negation are both set (X is a public array: a user can do this)
+    broken = copy.deepcopy(graphs)
+    row = int(broken.node_index[7]) + 3
+    broken.X[row, 0] |= np.uint32(1 << 5)
+    broken.X[row, 2] |= np.uint32(1 << 5)
+    dev = Device(model, broken)
+    assert dev.properties() == (1, 0) and not dev.declare_complementary()
+    assert dev.build_tiles()
+    assert np.array_equal(dev.score(0, 20, 20), o.score(model, broken))
+    # a graph without nodes rules the half tiles out as well
+    sizes = [30, 0, 40, 25]
+    empty = helpers.random_graphs(58, n_graphs=4, hv_size=64, sizes=sizes)
+    dev = Device(model, empty)
+    assert dev.properties() == (0, 1) and not dev.declare_complementary()
+    # a width of the literal halves that is not a multiple of 32 is compared bit by bit
+    odd = helpers.random_graphs(59, n_graphs=6, max_nodes=20, hv_size=20)
+    odd_cfg = helpers.oracle_config(odd, classes=2, clauses=10)
+    dev = Device(helpers.random_model(59, odd_cfg, 1), odd)
+    assert dev.properties() == (0, 0)
+    odd.X[2, 1] ^= np.uint32(1 << 3)  # literal 35 = the negation of literal 15
+    assert Device(helpers.random_model(59, odd_cfg, 1), odd).properties() == (1, 0)
