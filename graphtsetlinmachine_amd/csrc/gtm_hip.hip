@@ -978,7 +978,8 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     // any other tile of whole-word slots whose row offsets fit the 16-bit entries: k_tile_two_phase_wide
     const bool wide = !narrow && tg.slot_words > 0 && (int64_t)tg.rows * tg.tw / 4 < 65536 && !getenv("GTM_NO_TWO_PHASE");
     const bool two_phase = narrow || wide;
-    const int stride0 = two_phase ? 8 + d.LA : w.list_stride;
+    // compiled clause: 8 words of packed 16-bit row entries (16 words of byte offsets on half tiles) + the include words
+    const int stride0 = tg.half ? 16 + d.LA : two_phase ? 8 + d.LA : w.list_stride;
     if (tg.half)
         hipLaunchKernelGGL(k_compile_clauses_half, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C,
                            d.LA, d.B, d.filter, cfg->literals, g->number_of_node_types, tg.tw, order, w.lists, stride0,

@@ -1426,8 +1426,9 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
 // twice the graphs per tile: the scalar work, the address arithmetic and the phase-2 loads
 // of a (clause, tile) pair are spread over twice as many graphs.
 //
-// Compiled clause (same 8 + LA words as k_compile_clauses_two_phase): entry 0 =
-// variant (7 or 15 rows) | needs-phase-2 << 8 | positive pairs << 12; entry 1 = the
+// Compiled clause, 16 + LA words: 16 entries of 32 bits, then the include words.  Entry 0 =
+// variant (7 or 15 rows) | needs-phase-2 << 8 | positive pairs << 12; the others are rows as
+// LDS byte offsets, ready for use (a scalar load puts them in registers): entry 1 = the
 // node-type row; then literal rows in PAIRS, 3 or 7 of them: first the pairs of positive
 // literals (an odd one out is paired with the all-ones row), then the pairs of negated
 // ones (padded with the all-zero words that follow the rows in LDS).  With the signs fixed
@@ -1435,6 +1436,10 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
 // acc & ~(a | b) - and the clause's pattern (how many positive pairs) selects one of 8
 // straight-line variants with a single scalar jump.
 // The filter takes the clause's rarest literals, at most 14, as many as fit the pairs.
+
+struct alignas(16) Entries16 {
+    uint32_t v[16];
+};
 
 __global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C, int chunks, int B, uint32_t filter,
                                        int literals, int n_types, int tw, const uint32_t *__restrict__ order,
@@ -1449,7 +1454,6 @@ __global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C,
     const uint32_t row16 = (uint32_t)tw >> 2;  // a row in units of 16 bytes (tw is a multiple of 4)
     const uint32_t ones_row = (uint32_t)(hv + n_types), zero_row = ones_row + 1u;  // the zeroed words after the rows
     uint32_t *rec = records + (int64_t)c * record_words;
-    uint16_t *e = reinterpret_cast<uint16_t *>(rec);
     const uint32_t *inc = bank + (int64_t)c * chunks * B + (B - 1);
     // the clause's 14 rarest included literals, in `order`
     int n = 0;
@@ -1501,11 +1505,11 @@ __global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C,
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-    if (lane < 16) e[lane] = (uint16_t)slots[lane];
+    if (lane < 16) rec[lane] = lane == 0 ? slots[0] : slots[lane] << 4;  // rows as byte offsets: nothing to unpack
     for (int w = lane; w < chunks; w += 64) {
         uint32_t word = inc[(int64_t)w * B];
         if (w == chunks - 1) word &= filter;
-        rec[8 + w] = word;
+        rec[16 + w] = word;
     }
     if (weights)
         for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
@@ -1592,7 +1596,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         for (int u = 1; u < LW; ++u) m |= x.w[u];
         return m != 0;
     };
-    auto entry_of = [](const Packed8 &rec, int i) { return ((rec.v[i >> 1] >> ((i & 1) * 16)) & 0xFFFFu) << 4; };
+    auto entry_of = [](const Entries16 &rec, int i) { return rec.v[i]; };
     // a positive literal is violated where the node lacks it, a negated one (include words LA / 2 ..)
     // where the node has it: (include_pos & ~x) | (include_neg & x), one 3-input operation per word
     auto violates = [](const Words<LA> &include, const uint2 *x) {
@@ -1626,7 +1630,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
 
     // Phase 1 and the loads of phase 2.  Every load is issued by all lanes whatever the clause
     // does, so that the number of loads in flight is known when the pending clause is finished.
-    auto begin = [&](Pending &p, const Packed8 &rec, const int32_t *weights_of_clause, char *truth_out) {
+    auto begin = [&](Pending &p, const Entries16 &rec, const int32_t *weights_of_clause, char *truth_out) {
         p.live = true;
         p.weights = weights_of_clause;
         p.truth_out = truth_out;
@@ -1805,7 +1809,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
     const uint32_t *rec_a = a.lists + (int64_t)first * a.stride;
     const int32_t *wt_a = LAST ? a.wt + (int64_t)first * K : nullptr;
     char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
-    Packed8 ea = *reinterpret_cast<const Packed8 *>(rec_a);
+    Entries16 ea = *reinterpret_cast<const Entries16 *>(rec_a);
     Words<LA> ma, mb;
     Pending pa, pb;
     pa.live = pb.live = false;
@@ -1814,8 +1818,8 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         const uint32_t *rec_b = has_b ? rec_a + rec_step : rec_a;
         const int32_t *wt_b = LAST ? (has_b ? wt_a + wt_step : wt_a) : nullptr;
         char *truth_b = has_b ? truth_a + truth_step : truth_a;
-        ma = *reinterpret_cast<const Words<LA> *>(rec_a + 8);
-        const Packed8 eb = *reinterpret_cast<const Packed8 *>(rec_b);
+        ma = *reinterpret_cast<const Words<LA> *>(rec_a + 16);
+        const Entries16 eb = *reinterpret_cast<const Entries16 *>(rec_b);
         begin(pa, ea, wt_a, truth_a);
         finish(pb, mb);
         const bool has_a = c + 2 * NWAVES < C;
@@ -1824,8 +1828,8 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         truth_a = has_a ? truth_b + truth_step : truth_b;
         // without a second clause this repeats the first one and drops the result: keeping the
         // sequence of loads the same on every trip lets the waits stay partial
-        mb = *reinterpret_cast<const Words<LA> *>(rec_b + 8);
-        ea = *reinterpret_cast<const Packed8 *>(rec_a);
+        mb = *reinterpret_cast<const Words<LA> *>(rec_b + 16);
+        ea = *reinterpret_cast<const Entries16 *>(rec_a);
         begin(pb, eb, wt_b, truth_b);
         pb.live = has_b;
         finish(pa, ma);

@@ -405,9 +405,18 @@ int gtmc_fit(const gtmc_config *cfg, const gtmc_training *t, const gtmc_graphs *
     return rc;
 }
 
+/* Threads a call may use: the processors OpenMP sees, capped by OMP_NUM_THREADS.  (Not
+ * omp_get_max_threads(): the entry points above set the calling thread's team size, and that
+ * setting outlives the call.) */
 int gtmc_threads_available(void) {
 #ifdef _OPENMP
-    return omp_get_max_threads();
+    int n = omp_get_num_procs();
+    const char *env = getenv("OMP_NUM_THREADS");
+    if (env) {
+        const int k = atoi(env);
+        if (k > 0 && k < n) n = k;
+    }
+    return n > 0 ? n : 1;
 #else
     return 1;
 #endif

@@ -131,3 +131,53 @@ def test_training_of_every_configuration_follows_the_c_oracle(name, n_train):
         assert np.array_equal(got, want.reshape(-1))
     model.cfg = oracle_twin(tm, wl.graphs_test).cfg
     assert np.array_equal(tm.score(wl.graphs_test), oc.score(model, wl.graphs_test))
+
+
+def test_a_whole_epoch_of_the_convolutional_configuration_follows_the_c_oracle(capsys):
+    """All 60,000 training graphs of the 361-node configuration, one after the other: the state the
+    benchmark times its scoring kernel on.  The GPU trains the epoch in 48 runs of 1,250 examples and
+    its state is read back after each; the C restatement then goes from every one of those states
+    over the next 1,250 examples (single-threaded, 16 runs side by side) and must arrive at the next
+    state bit for bit.  The first state is the common initial one, so by induction the whole GPU
+    trajectory is the oracle's - without the oracle having to do 60,000 examples in sequence."""
+    import copy
+    from concurrent.futures import ThreadPoolExecutor
+
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    n, run = 60000, 1250
+    wl = workloads.convolutional_images(n_train=n, n_test=512)
+    np.random.seed(42)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=0, incremental=True)  # initial state only
+    first = oracle_twin(tm, wl.graphs_train)
+    states = [tm.get_state()]
+    assert np.array_equal(states[0][0], first.ta_state.reshape(-1))
+    assert np.array_equal(states[0][1].reshape(first.clause_weights.shape), first.clause_weights)
+    for start in range(0, n, run):
+        tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True, examples=(start, run))
+        states.append(tm.get_state())
+    assert tm.step == n
+    encoded = o.encode_labels(wl.Y_train, tm.number_of_outputs, tm.T)
+
+    def follow(i):
+        model = copy.copy(first)
+        model.ta_state = states[i][0].reshape(first.ta_state.shape).copy()
+        model.clause_weights = states[i][1].reshape(first.clause_weights.shape).copy()
+        model.step = i * run
+        oc.fit(model, wl.graphs_train, encoded, indices=range(i * run, (i + 1) * run), threads=1)
+        return (np.array_equal(model.ta_state.reshape(-1), states[i + 1][0]) and
+                np.array_equal(model.clause_weights.reshape(-1), states[i + 1][1].reshape(-1)))
+
+    with ThreadPoolExecutor(max_workers=max(1, min(16, oc.threads_available()))) as pool:
+        for i, same in enumerate(pool.map(follow, range(n // run))):
+            assert same, "the GPU and the oracle part ways between examples %d and %d" % (i * run, (i + 1) * run)
+            if i % 8 == 7:
+                with capsys.disabled():
+                    print(" [%d examples followed]" % ((i + 1) * run), end="", flush=True)
+    last = copy.copy(first)
+    last.ta_state = states[-1][0].reshape(first.ta_state.shape).copy()
+    last.clause_weights = states[-1][1].reshape(first.clause_weights.shape).copy()
+    sums = tm.score(wl.graphs_test)
+    assert np.array_equal(sums, oc.score(last, wl.graphs_test, threads=min(16, oc.threads_available())))
+    assert (sums.argmax(axis=1) == wl.Y_test).mean() > 0.95
