@@ -50,6 +50,9 @@ def parse():
     p.add_argument("--no-cpu", action="store_true")
     p.add_argument("--only-main", action="store_true", help="skip the short runs of the other four configurations")
     p.add_argument("--one-state", action="store_true", help="time the kernel on the headline state only")
+    p.add_argument("--full-size", action="store_true", help="the chosen workload at its full data-set size: one epoch "
+                   "of training on every training graph, every test graph scored, a sample spread over the set "
+                   "(first and last tile, graphs on both sides of the 4 GiB mark of X) checked against the C oracle")
     p.add_argument("--copy-probe", action="store_true", help="only copy 256 MiB three times with a library copy kernel: "
                    "calibrates the units of the FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc")
     p.add_argument("--save-state", default="", help="write the trained model to this .npz file after the run")
@@ -135,6 +138,100 @@ def short_run(name, n_train, n_test, check_graphs):
     }
 
 
+FULL_SIZES = {  # (training graphs, test graphs) the configurations are stated with
+    "noisy_xor": (10000, 10000), "single_node_images": (60000, 10000), "convolutional_images": (60000, 10000),
+    "sequence_chains": (20000, 5000), "colour_convolution": (50000, 10000),
+}
+
+
+def full_size_run(name, check_seconds=60.0):
+    """One epoch over every training graph and one scoring pass over every test graph of a configuration
+    at its stated data-set size; the trained state goes to the C oracle, which scores a sample spread
+    over both sets (first and last graphs, and graphs around every multiple of 4 GiB of X)."""
+    import numpy as np
+    import torch
+
+    from graphtsetlinmachine_amd import workloads
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+    from oracle import gtm_oracle_c as oc
+
+    import threading
+
+    n_train, n_test = FULL_SIZES[name]
+    t0 = time.time()
+    building = threading.Event()
+
+    def heartbeat():  # building the largest data set takes minutes: say so while it lasts
+        while not building.wait(30.0):
+            print("bench.py: building %s ... %.0f s" % (name, time.time() - t0), file=sys.stderr, flush=True)
+
+    threading.Thread(target=heartbeat, daemon=True).start()
+    try:
+        wl = workloads.BUILDERS[name](n_train=n_train, n_test=n_test)
+    finally:
+        building.set()
+    t_data = time.time() - t0
+    print("bench.py: %s built in %.0f s (X: %.2f GB train, %.2f GB test)"
+          % (name, t_data, wl.graphs_train.X.nbytes / 1e9, wl.graphs_test.X.nbytes / 1e9), file=sys.stderr, flush=True)
+    np.random.seed(42)
+    tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
+    t0 = time.perf_counter()
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=0, incremental=True)  # upload, tiles, initial state
+    torch.cuda.synchronize()
+    t_upload = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
+    torch.cuda.synchronize()
+    t_train = time.perf_counter() - t0
+    print("bench.py: trained %d graphs in %.1f s" % (n_train, t_train), file=sys.stderr, flush=True)
+    tm.score_device(wl.graphs_test)  # uploads the test graphs
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    sums_test = tm.score_device(wl.graphs_test)
+    torch.cuda.synchronize()
+    t_test = time.perf_counter() - t0
+    sums_test = sums_test.cpu().numpy().reshape(n_test, -1)
+    t0 = time.perf_counter()
+    sums_train = tm.score_device(wl.graphs_train)  # the training set is the one that crosses 4 GiB
+    torch.cuda.synchronize()
+    t_score_train = time.perf_counter() - t0
+    sums_train = sums_train.cpu().numpy().reshape(n_train, -1)
+
+    def spread(graphs):
+        n = graphs.number_of_graphs
+        picks = {0, 1, n // 2, n - 2, n - 1}
+        words = graphs.X.shape[1]
+        mark = (1 << 32) // (words * 4)  # nodes per 4 GiB of literal words
+        for k in range(1, int(graphs.X.shape[0] // mark) + 1):
+            g = int(np.searchsorted(graphs.node_index, k * mark, side="right")) - 1
+            picks.update(e for e in (g - 1, g, g + 1) if 0 <= e < n)
+        return sorted(picks)
+
+    threads = max(1, min(16, oc.threads_available()))
+    checked, same, t0 = {}, True, time.perf_counter()
+    for label, graphs, sums in (("test", wl.graphs_test, sums_test), ("train", wl.graphs_train, sums_train)):
+        model = oracle_twin(tm, int(graphs.max_number_of_graph_nodes))
+        picks = spread(graphs)
+        done = []
+        for at in range(0, len(picks), threads):  # bounded: a colour graph costs about half a second
+            if time.perf_counter() - t0 > check_seconds and done:
+                break
+            part = picks[at:at + threads]
+            same = same and bool(np.array_equal(oc.score(model, graphs, part, threads=threads), sums[part]))
+            done += part
+        checked[label] = done
+    return {
+        "workload": name, "train_graphs": n_train, "test_graphs": n_test,
+        "X_train_bytes": int(wl.graphs_train.X.nbytes), "X_test_bytes": int(wl.graphs_test.X.nbytes),
+        "total_train_nodes": int(wl.graphs_train.X.shape[0]),
+        "train_graphs_per_s": round(n_train / t_train, 1), "inference_graphs_per_s": round(n_test / t_test, 1),
+        "inference_graphs_per_s_on_the_training_set": round(n_train / t_score_train, 1),
+        "test_accuracy": round(float((sums_test.argmax(axis=1) == wl.Y_test).mean()), 4),
+        "class_sums_equal_c_oracle_on": checked if same else "MISMATCH",
+        "data_build_s": round(t_data, 1), "upload_and_tiles_s": round(t_upload, 1),
+    }
+
+
 def eval_bytes_per_graph(n_nodes, la_chunks, clauses, node_chunks):
     """Algorithmic bytes of one layer-0 clause evaluation of one graph: its X
     rows, node types and the include plane in; the clause x node bitmap and the
@@ -211,6 +308,16 @@ def main():
     from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
 
     torch.cuda.set_device(0)
+    if args.full_size:
+        result = full_size_run(args.workload)
+        print(json.dumps({"metric": "train & inference graphs/sec on 1 MI355X (%s at full data-set size)" % args.workload,
+                          "value": result["inference_graphs_per_s"], "unit": "graphs/s", "n_gpus": 1,
+                          "higher_is_better": True, "dtype": "u32", "data": "synthetic",
+                          "config": {"workload": args.workload}, "full_size": result}), flush=True)
+        if result["class_sums_equal_c_oracle_on"] == "MISMATCH":
+            print("bench.py: GPU class sums differ from the C oracle", file=sys.stderr)
+            sys.exit(1)
+        return
     t0 = time.time()
     wl = workloads.BUILDERS[args.workload](n_train=args.train_graphs, n_test=args.graphs)
     t_data = time.time() - t0

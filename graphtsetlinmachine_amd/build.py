@@ -19,7 +19,23 @@ FLAGS = [
 ]
 
 
+ENCODER_SOURCE = os.path.join(HERE, "csrc", "encode.c")
+ENCODER_OUTPUT = os.path.join(HERE, "libgtm_encode.so")
+
+
+def build_encoder(verbose=True):
+    """The host-side property encoder (plain C, OpenMP) that graphs.py loads through ctypes."""
+    cmd = [os.environ.get("CC", "gcc"), "-O3", "-fopenmp", "-shared", "-fPIC", "-o", ENCODER_OUTPUT, ENCODER_SOURCE]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("gcc failed:\n" + proc.stdout)
+    return ENCODER_OUTPUT
+
+
 def build(verbose=True):
+    build_encoder(verbose)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     cmd = [hipcc] + FLAGS + ["-o", OUTPUT] + SOURCES
     if verbose:

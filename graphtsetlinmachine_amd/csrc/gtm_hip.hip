@@ -32,8 +32,17 @@ int fail(int code, const char *fmt, ...) {
     return code;
 }
 
+// Set by blocks_for() when a work size does not fit the grid of one launch; the launch that follows
+// runs one block (harmless) and check_launch() reports the call as failed.
+thread_local bool g_grid_overflow = false;
+
 int check_launch(const char *what) {
     hipError_t e = hipGetLastError();
+    if (g_grid_overflow) {
+        g_grid_overflow = false;
+        return fail(GTM_ERR_INVALID, "%s: the work size exceeds what one launch can cover (2^31 - 1 blocks); "
+                                     "pass fewer graphs per call", what);
+    }
     if (e != hipSuccess) return fail(GTM_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
     return GTM_OK;
 }
@@ -134,7 +143,14 @@ uint64_t q_threshold(double q, int classes) {
     return (uint64_t)(p * 4294967296.0);
 }
 
-inline unsigned blocks_for(int64_t items, int per_block) { return (unsigned)((items + per_block - 1) / per_block); }
+inline unsigned blocks_for(int64_t items, int per_block) {
+    const int64_t blocks = (items + per_block - 1) / per_block;
+    if (blocks > 0x7FFFFFFF) {  // never truncated silently
+        g_grid_overflow = true;
+        return 1u;
+    }
+    return (unsigned)blocks;
+}
 
 constexpr int TPB = 256;
 
@@ -963,8 +979,9 @@ int launch_two_phase_wide(const TileLayerArgs &a, int n_tiles, int LA, bool stag
 // LDS when a node has 4, 8, 12 or 16 literal words.  GTM_NO_TWO_PHASE (tuning aid) turns it off.
 bool two_phase_layer0(const Dims &d, const gtm_graphs *g, const TileGeom &tg) {
     if (tg.half) return true;  // such a geometry is only chosen for k_tile_two_phase_half (64-bit offsets into X)
-    // k_tile_two_phase addresses X with 32-bit byte offsets
-    const bool x_fits = (uint64_t)g->total_nodes * d.LA * 4 < (1ull << 32);
+    // k_tile_two_phase addresses X with 32-bit byte offsets: beyond 4 GiB of literal words (or with
+    // GTM_NO_NARROW_TWO_PHASE, which lets tests take that way with small data) k_tile_two_phase_wide runs
+    const bool x_fits = (uint64_t)g->total_nodes * d.LA * 4 < (1ull << 32) && !getenv("GTM_NO_NARROW_TWO_PHASE");
     return tg.slot_words > 0 && tg.stage0 && d.LA % 4 == 0 && d.LA <= 16 && x_fits && !getenv("GTM_NO_TWO_PHASE");
 }
 

@@ -91,7 +91,8 @@ inline TileGeom tile_geometry_lw(int literals, int n_types, int max_nodes, int n
         }
     }
     g.n_tiles = g.gpt > 0 ? (n_graphs + g.gpt - 1) / g.gpt : 0;
-    g.ok = g.gpt > 0 && tile_lds_bytes(fit_rows, g, classes) <= TILE_LDS_BUDGET;
+    // (compiled clauses address a tile's rows by 31-bit byte offsets: bit 31 marks a negated message literal)
+    g.ok = g.gpt > 0 && tile_lds_bytes(fit_rows, g, classes) <= TILE_LDS_BUDGET && (int64_t)g.rows * g.tw * 4 < (1ll << 31);
     g.stage0 = g.ok && tile_lds_bytes(g.rows, g, classes) <= TILE_LDS_BUDGET;
     return g;
 }

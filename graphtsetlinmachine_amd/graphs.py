@@ -26,9 +26,33 @@ variants (``add_graph_nodes``, ``add_graph_node_edges``,
 insertions cannot be built one Python call at a time.
 """
 
+import ctypes
 import hashlib
+import os
 
 import numpy as np
+
+_ENCODER_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libgtm_encode.so")
+_encoder = None
+
+
+def _native_encoder():
+    """The C encoder of csrc/encode.c (built by build.py), or None when it has not been built or
+    GTM_NO_NATIVE_ENCODER is set: the NumPy forms below give the same arrays, more slowly."""
+    global _encoder
+    if os.environ.get("GTM_NO_NATIVE_ENCODER"):
+        return None
+    if _encoder is None:
+        if not os.path.exists(_ENCODER_PATH):
+            return None
+        lib = ctypes.CDLL(_ENCODER_PATH)
+        p, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32
+        lib.gtm_encode_membership.restype = None
+        lib.gtm_encode_membership.argtypes = [p, i64, i32, p, i32, i32, i32, p]
+        lib.gtm_encode_pairs.restype = None
+        lib.gtm_encode_pairs.argtypes = [p, p, i64, p, i32, i32, i32, p]
+        _encoder = lib
+    return _encoder
 
 
 class GraphsError(SystemExit):
@@ -131,7 +155,9 @@ class Graphs:
         lit = np.arange(self.number_of_hypervector_chunks * 32, dtype=np.int64).reshape(-1, 32)
         negated = (lit >= hv) & (lit < 2 * hv)
         row = (negated.astype(np.uint64) << np.arange(32, dtype=np.uint64)).sum(axis=1)
-        return np.tile(row.astype(np.uint32), (n_rows, 1))
+        rows = np.empty((n_rows, row.shape[0]), dtype=np.uint32)
+        rows[:] = row.astype(np.uint32)  # (a broadcast store: np.tile goes through repeat, ten times slower)
+        return rows
 
     def prepare_node_configuration(self):
         counts = self.number_of_graph_nodes
@@ -277,6 +303,13 @@ class Graphs:
             n = k + hv
             x[n >> 5] &= np.uint32(~(1 << (n & 31)) & 0xFFFFFFFF)
 
+    def _encodable(self):
+        """The arrays are as the C encoder addresses them: contiguous uint32, every hypervector index
+        inside the hypervector."""
+        return (self.X.dtype == np.uint32 and self.X.flags.c_contiguous and self.hypervectors.dtype == np.uint32 and
+                self.hypervectors.flags.c_contiguous and self.hypervectors.ndim == 2 and
+                (self.hypervectors.size == 0 or int(self.hypervectors.max()) < self.hypervector_size))
+
     def add_graph_node_properties(self, node_rows, symbol_ids, chunk_rows=1 << 18):
         """Bulk form of ``add_graph_node_property``.
 
@@ -290,6 +323,14 @@ class Graphs:
         if rows.shape != syms.shape:
             raise ValueError("node_rows and symbol_ids must have the same length")
         if rows.size == 0:
+            return
+        if rows.min() < 0 or rows.max() >= self.X.shape[0] or syms.min() < 0 or syms.max() >= self.hypervectors.shape[0]:
+            raise IndexError("node row or symbol id out of range")
+        native = _native_encoder()
+        if native is not None and self._encodable():
+            native.gtm_encode_pairs(rows.ctypes.data, syms.ctypes.data, rows.size, self.hypervectors.ctypes.data,
+                                    self.hypervectors.shape[1], self.hypervector_size,
+                                    self.number_of_hypervector_chunks, self.X.ctypes.data)
             return
         hv = self.hypervector_size
         chunks = self.number_of_hypervector_chunks
@@ -329,6 +370,16 @@ class Graphs:
         n_rows, n_symbols = membership.shape
         if n_symbols != len(self.symbol_id):
             raise ValueError("membership needs one column per symbol")
+        if first_node_row < 0 or first_node_row + n_rows > self.X.shape[0]:
+            raise IndexError("node rows out of range")
+        native = _native_encoder()
+        if native is not None and self._encodable() and n_rows > 0:
+            flags = np.ascontiguousarray(membership if membership.dtype == np.uint8 else membership != 0).view(np.uint8)
+            target = self.X[first_node_row:first_node_row + n_rows]
+            native.gtm_encode_membership(flags.ctypes.data, n_rows, n_symbols, self.hypervectors.ctypes.data,
+                                         self.hypervectors.shape[1], self.hypervector_size,
+                                         self.number_of_hypervector_chunks, target.ctypes.data)
+            return
         hv = self.hypervector_size
         chunks = self.number_of_hypervector_chunks
         # symbol -> hypervector index incidence; small-integer float32 products are exact

@@ -76,3 +76,53 @@ def test_product_package_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+
+
+def _desc(n_graphs, max_nodes, n_types=1, edges_per_graph=0, tiles=0):
+    from graphtsetlinmachine_amd import _abi
+
+    d = _abi.GraphsDesc()
+    d.number_of_graphs = n_graphs
+    d.number_of_node_types = n_types
+    d.max_number_of_graph_nodes = max_nodes
+    d.total_nodes = n_graphs * max_nodes
+    d.total_edges = n_graphs * edges_per_graph
+    d.tiles = tiles
+    return d
+
+
+def test_buffer_sizes_are_computed_in_64_bits_at_and_beyond_the_largest_configuration():
+    """The colour configuration at its full data-set size (50,000 graphs of 841 nodes, 2,048 literals, 8,000
+    clauses, depth 3: X alone is 10.8 GB) and ten times that: every size the host hands out is the
+    product it should be, far beyond 2^32 - no offset of the driver loops is formed in 32 bits.  (Host
+    arithmetic only: nothing is launched.)"""
+    from graphtsetlinmachine_amd import _abi
+
+    cfg = _abi.make_config(classes=10, clauses=8000, literals=2048, state_bits=8, boost_true_positive_feedback=1,
+                           threshold=10000, q=1.0, max_included_literals=2048, negative_clauses=1, max_nodes=841,
+                           message_size=1024, message_bits=2, depth=3, s=(15.0,) * 3, seed=1)
+    for n_graphs in (50000, 500000):
+        d = _desc(n_graphs, 841, edges_per_graph=3248)
+        # message rows (1,026) rule the tile: one 841-node graph (27 -> 28 words per row) per tile
+        rows, tw = 2048 + 1 + 1, 28
+        want = n_graphs * rows * tw * 4 + rows * 8 + 2048 * 4
+        got = _abi.lib.gtm_tiles_bytes(ctypes.byref(cfg), ctypes.byref(d))
+        assert got == want and got > 2**33
+        # the dense path's workspace grows with the batch: [batch][CLAUSES][NODE_CHUNKS] bitmaps twice and
+        # [batch][max_nodes][MESSAGE_CHUNKS] packed messages
+        small = _abi.lib.gtm_score_workspace_bytes(ctypes.byref(cfg), ctypes.byref(d), 1)
+        big = _abi.lib.gtm_score_workspace_bytes(ctypes.byref(cfg), ctypes.byref(d), 1 << 16)
+        per_graph = 2 * 8000 * 27 * 4 + 841 * 64 * 4
+        assert big - small == ((1 << 16) - 1) * per_graph and big > 2**36
+    # the 361-node configuration with 6 million graphs: X = 69 GB, tiles of all rows 10 graphs each
+    conv = _abi.make_config(classes=10, clauses=2500, literals=256, state_bits=8, boost_true_positive_feedback=1,
+                            threshold=3125, q=1.0, max_included_literals=256, negative_clauses=1, max_nodes=361,
+                            message_size=256, message_bits=2, depth=1, s=(10.0,), seed=1)
+    d = _desc(6_000_000, 361)
+    assert _abi.lib.gtm_tiles_bytes(ctypes.byref(conv), ctypes.byref(d)) == 600_000 * 258 * 128 * 4 + 258 * 8 + 256 * 4
+    # and declared complementary: 21 graphs per tile of 256-word rows, plus 16 bytes per node slot
+    d.flags = _abi.GTM_GRAPHS_COMPLEMENTARY
+    n_tiles = (6_000_000 + 20) // 21
+    rows_part = n_tiles * 258 * 256 * 4 + 258 * 8 + 256 * 4
+    assert rows_part % 16 == 0
+    assert _abi.lib.gtm_tiles_bytes(ctypes.byref(conv), ctypes.byref(d)) == rows_part + n_tiles * 256 * 32 * 16

@@ -830,3 +830,25 @@ def test_data_that_is_not_complementary_is_detected_and_keeps_all_rows():
     assert dev.properties() == (0, 0)
     odd.X[2, 1] ^= np.uint32(1 << 3)  # literal 35 = the negation of literal 15
     assert Device(helpers.random_model(59, odd_cfg, 1), odd).properties() == (1, 0)
+
+
+@pytest.mark.parametrize("shape", [s for s in TILE_SHAPES if s["seed"] in (14, 15, 16, 17, 18)], ids=lambda s: "tiles%d" % s["seed"])
+def test_the_kernel_that_takes_over_beyond_4_gib_of_literal_words_follows_the_oracle(shape, monkeypatch):
+    """k_tile_two_phase addresses X with 32-bit byte offsets and hands data sets of 4 GiB and more to
+    k_tile_two_phase_wide (64-bit offsets).  GTM_NO_NARROW_TWO_PHASE takes that way with small data."""
+    from tests.gpu_harness import Device
+
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    cfg = helpers.oracle_config(graphs, classes=shape["classes"], clauses=shape["clauses"])
+    model = helpers.random_model(shape["seed"], cfg, 1, include_density=0.05)
+    dev = Device(model, graphs)
+    G = graphs.number_of_graphs
+    assert dev.build_tiles()
+    monkeypatch.setenv("GTM_NO_NARROW_TWO_PHASE", "1")
+    _abi.call("gtm_profile_enable", 1)
+    got = dev.score(0, G, G)
+    name, launches, total = ctypes.c_char_p(), ctypes.c_int32(), ctypes.c_double()
+    _abi.call("gtm_profile_read", ctypes.byref(name), ctypes.byref(launches), ctypes.byref(total))
+    _abi.call("gtm_profile_enable", 0)
+    assert name.value.decode() == "k_tile_two_phase_wide<score>"
+    assert np.array_equal(got, o.score(model, graphs))

@@ -99,7 +99,15 @@ def test_tutorial_graph_layout():
     assert len(g) == 3
 
 
-def test_bulk_builders_equal_single_calls():
+@pytest.mark.parametrize("encoder", ["native", "numpy"])
+def test_bulk_builders_equal_single_calls(encoder, monkeypatch):
+    from graphtsetlinmachine_amd import graphs as graphs_module
+
+    if encoder == "numpy":
+        monkeypatch.setenv("GTM_NO_NATIVE_ENCODER", "1")
+        assert graphs_module._native_encoder() is None
+    else:
+        assert graphs_module._native_encoder() is not None, "libgtm_encode.so has not been built"
     rng = np.random.default_rng(0)
     n, nodes = 7, 5
     np.random.seed(9)
@@ -219,3 +227,50 @@ def test_print_graph_writes_the_reference_format(capsys):
     assert out == ("Printing nodes of Graph#0:\nNode#0( A * ) Node#1( * B ) \n\n"
                    "Printing edges of Graph#0:\nEdge#0 SrcNode#0 DestNode#1 EdgeType#0\n\n"
                    "Edge#1 SrcNode#1 DestNode#0 EdgeType#1\n\n\n\n")
+
+
+@pytest.mark.parametrize("hv_size, hv_bits", [(20, 3), (64, 2), (1024, 2), (37, 1)])
+def test_the_native_encoder_and_the_numpy_forms_build_the_same_rows(hv_size, hv_bits, monkeypatch):
+    """csrc/encode.c (the reference's per-property loop, graphs.py:148-162, over whole arrays) against
+    the vectorised NumPy forms: repeated pairs, rows that already hold properties, both entry points."""
+    from graphtsetlinmachine_amd import graphs as graphs_module
+
+    assert graphs_module._native_encoder() is not None, "libgtm_encode.so has not been built"
+    rng = np.random.default_rng(hv_size)
+    n_symbols, n_graphs, nodes = 23, 40, 50
+
+    def build():
+        np.random.seed(hv_size)
+        g = Graphs(n_graphs, symbols=list(range(n_symbols)), hypervector_size=hv_size, hypervector_bits=hv_bits)
+        g.number_of_graph_nodes[:] = nodes
+        g.prepare_node_configuration()
+        g.add_graph_nodes(0)
+        g.prepare_edge_configuration()
+        return g
+
+    rows = rng.integers(0, n_graphs * nodes, size=6000)
+    syms = rng.integers(0, n_symbols, size=6000)
+    member = rng.random((700, n_symbols)) < 0.2
+    native, plain = build(), build()
+    native.add_graph_node_properties(rows, syms)
+    native.add_graph_node_property_matrix(300, member)
+    native.add_graph_node_property_matrix(900, member.astype(np.uint8) * 7)  # any non-zero value counts
+    monkeypatch.setenv("GTM_NO_NATIVE_ENCODER", "1")
+    plain.add_graph_node_properties(rows, syms)
+    plain.add_graph_node_property_matrix(300, member)
+    plain.add_graph_node_property_matrix(900, member.astype(np.uint8) * 7)
+    assert np.array_equal(native.X, plain.X)
+    # and both equal the single calls on a few rows
+    single = build()
+    for r, s_ in zip(rows[:300].tolist(), syms[:300].tolist()):
+        single.add_graph_node_property(r // nodes, r % nodes, s_)
+    check = build()
+    monkeypatch.delenv("GTM_NO_NATIVE_ENCODER")
+    check.add_graph_node_properties(rows[:300], syms[:300])
+    assert np.array_equal(check.X, single.X)
+    with pytest.raises(IndexError):
+        check.add_graph_node_properties([n_graphs * nodes], [0])
+    with pytest.raises(IndexError):
+        check.add_graph_node_properties([0], [n_symbols])
+    with pytest.raises(IndexError):
+        check.add_graph_node_property_matrix(n_graphs * nodes - 10, member)
