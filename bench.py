@@ -27,12 +27,12 @@ VALU_PEAK_LANE_OPS = 256 * 64 * 2.4e9  # 32-bit integer lane operations per seco
 # Hardware counters of the scoring kernel on the convolutional workload (10,000 graphs per launch, state after
 # one epoch), from rocprofv3 --pmc runs of this file; the summaries and the commands are under profiles/.
 # FETCH_SIZE counts 2 KiB per unit and WRITE_SIZE 1 KiB per unit on this part (a 256 MiB copy kernel reads
-# 131,089 and writes 262,144).  valu_busy = SQ_ACTIVE_INST_VALU x 4 / SQ_BUSY_CU_CYCLES.  The figures belong
-# to the kernel as of `commit`; a run whose kernel differs reports them as stale by that name.
+# 131,085 and writes 262,144).  valu_busy = SQ_INSTS_VALU / (1,024 SIMDs x the launch's 4-clock issue slots at
+# 2.4 GHz).  The figures belong to the kernel as of `commit`; a run on another kernel reports none.
 MEASURED_COUNTERS = {
     "convolutional_images": {
-        "kernel": "k_tile_two_phase<score>", "commit": "3237649",
-        "fetch_units": 131715.6, "write_units": 406.3, "valu_busy": 0.59, "graphs": 10000,
+        "kernel": "k_tile_two_phase_half<score>", "commit": "9ca7f4a",
+        "fetch_units": 81892.2, "write_units": 401.8, "valu_busy": 0.65, "graphs": 10000,
     },
 }
 
@@ -327,7 +327,10 @@ def main():
     np.random.seed(42)
     tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
     if args.load_state:
-        tm.load(fname=args.load_state)
+        import contextlib
+
+        with contextlib.redirect_stdout(sys.stderr):  # load() announces the file, as the reference's does
+            tm.load(fname=args.load_state)
         args.one_state, args.train_epochs = True, 0
     else:
         tm.fit(wl.graphs_train, wl.Y_train, epochs=0, incremental=True)  # allocate + upload only
@@ -377,7 +380,10 @@ def main():
     t_train += time.time() - t0
     train_gps = args.train_graphs * args.train_epochs / max(t_train, 1e-9)
     if args.save_state:
-        tm.save(args.save_state)
+        import contextlib
+
+        with contextlib.redirect_stdout(sys.stderr):
+            tm.save(args.save_state)
 
     main_run = time_scoring(tm, test, args.steps, args.warmup, args.graphs)
     wall, kernel_name, launches = main_run["wall"], main_run["kernel"], main_run["launches"]
