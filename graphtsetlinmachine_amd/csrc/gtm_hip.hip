@@ -430,6 +430,7 @@ __global__ void k_select_clause_updates(int32_t *weights, const int32_t *__restr
 #include "fit_deep.h"
 #include "fit_small.h"
 #include "fit_persistent.h"
+#include "fit_deep_persistent.h"
 
 // K9 / K10: one thread per (clause, automaton word); the classes are applied
 // in ascending order to that word, as kernels.py:205-207,236-238 do per clause
@@ -606,8 +607,11 @@ struct FitWs {
     uint32_t *message_rows;                 // [M][message_row_words] literal-major messages of one layer (depth > 1)
     int message_row_words;
     uint32_t *sent, *got;                   // [max_nodes][M / 32] bit vectors sent / received per node (depth > 1)
-    uint32_t *bank_backup;                  // [C][LA][B]: the layer-0 bank as it was before a cooperative run (depth 1)
+    uint32_t *bank_backup;                  // every bank as it was before a cooperative run: [C][LA][B], then [C][MC][B] per message bank
     int32_t *weights_backup;                // [K][C]
+    uint32_t *coop_got;                     // [3][depth - 1][M][NC] rows exchanged by k_fit_deep_persistent (depth > 1)
+    unsigned long long *coop_arrived;       // [depth - 1][FITD_PARTS * FITD_STRIDE]
+    size_t coop_words;                      // words of coop_got
     size_t bytes;
 };
 
@@ -635,8 +639,11 @@ FitWs carve_fit(const Dims &d, const gtm_config *cfg, char *base) {
     const size_t vector_bytes = (size_t)cfg->max_nodes * ((d.M + 31) / 32) * 4;
     w.sent = cfg->depth > 1 ? (uint32_t *)take(vector_bytes) : nullptr;
     w.got = cfg->depth > 1 ? (uint32_t *)take(vector_bytes) : nullptr;
-    w.bank_backup = cfg->depth == 1 ? (uint32_t *)take((size_t)d.C * d.LA * d.B * 4) : nullptr;
-    w.weights_backup = cfg->depth == 1 ? (int32_t *)take((size_t)d.K * d.C * 4) : nullptr;
+    w.bank_backup = (uint32_t *)take(((size_t)d.C * d.LA + (size_t)(cfg->depth - 1) * d.C * d.MC) * d.B * 4);
+    w.weights_backup = (int32_t *)take((size_t)d.K * d.C * 4);
+    w.coop_words = cfg->depth > 1 ? (size_t)3 * (cfg->depth - 1) * d.M * d.NC : 0;
+    w.coop_got = cfg->depth > 1 ? (uint32_t *)take(w.coop_words * 4) : nullptr;
+    w.coop_arrived = cfg->depth > 1 ? (unsigned long long *)take((size_t)(cfg->depth - 1) * FITD_PARTS * FITD_STRIDE * 8) : nullptr;
     w.bytes = off;
     return w;
 }
@@ -1709,6 +1716,179 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     return GTM_OK;
 }
 
+// `_fit`'s inner loop of a model with message layers as one cooperative launch (fit_deep_persistent.h).
+// Returns GTM_OK with *done = false when this device or shape cannot run it, so that the caller
+// falls back to the launches per example.  GTM_NO_DEEP_PERSISTENT_FIT (tuning aid) turns it off.
+int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
+                        const FitWs &w, const int32_t *encoded_Y, int first_example, int n_examples, uint64_t first_step,
+                        hipStream_t st, bool *done) {
+    *done = false;
+    if (getenv("GTM_NO_DEEP_PERSISTENT_FIT") || getenv("GTM_NO_PERSISTENT_FIT") || cfg->depth < 2 || d.K > FITD_BLOCK) return GTM_OK;
+    if (d.M % 32 != 0 || d.NC > 64) return GTM_OK;  // whole words of message bits; one lane per word of a truth row
+    int dev = 0, coop = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return GTM_OK;
+    if (hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) != hipSuccess || !coop) return GTM_OK;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) return GTM_OK;
+    if (g->total_edges > 0 && (!g->number_of_graph_node_edges || !g->edge || !g->edge_index))
+        return fail(GTM_ERR_INVALID, "graphs with edges need number_of_graph_node_edges, edge and edge_index");
+
+    const int layers = cfg->depth - 1, MW = d.M / 32;
+    int per_group = (d.C + cus - 1) / cus;
+    if (const char *e = getenv("GTM_FIT_DEEP_CLAUSES_PER_GROUP")) per_group = std::max(per_group, atoi(e));  // tuning aid
+    const int groups = (d.C + per_group - 1) / per_group;
+    const int NW = d.NC;
+    const int rows_words = (cfg->literals + g->number_of_node_types + 1) * NW;
+    // the edges of the run's examples: most per graph, largest type, stored node after node?
+    uint32_t limits[3] = {0u, 0u, 0u};
+    if (g->total_edges > 0) {
+        hipLaunchKernelGGL(k_fill_i32, dim3(1), dim3(TPB), 0, st, (int32_t *)w.coop_got, (int64_t)3, 0);
+        if (int rc = check_launch("fill")) return rc;
+        hipLaunchKernelGGL(k_edge_limits, dim3(n_examples), dim3(256), 0, st, g->number_of_graph_nodes, g->node_index,
+                           g->number_of_graph_node_edges, g->edge_index, g->edge, first_example, w.coop_got);
+        if (int rc = check_launch("k_edge_limits")) return rc;
+        hipError_t e = hipMemcpyAsync(limits, w.coop_got, sizeof(limits), hipMemcpyDeviceToHost, st);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "reading the edge limits: %s", hipGetErrorString(e));
+        if (limits[2] != 0u || limits[1] >= (uint32_t)FITD_MAX_EDGE_TYPES || limits[0] > (1u << 20)) return GTM_OK;
+    }
+    const int edge_cap = (int)limits[0], edge_types = (int)limits[1] + 1;
+    const size_t lds = fit_deep_lds_words(cfg->depth, per_group, d.LA, d.MC, d.M, d.MB, d.B, d.K, NW, rows_words, cfg->max_nodes, edge_cap,
+                                          edge_types) * 4;
+    if (lds > 150 * 1024) return GTM_OK;
+    const int variant = d.B <= 8 ? 0 : d.B <= 16 ? 1 : 2;
+    const void *kernel = variant == 0   ? (const void *)k_fit_deep_persistent<8>
+                         : variant == 1 ? (const void *)k_fit_deep_persistent<16>
+                                        : (const void *)k_fit_deep_persistent<32>;
+    static thread_local size_t lds_set_of[3] = {48 * 1024, 48 * 1024, 48 * 1024};
+    if (lds > lds_set_of[variant]) {
+        if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return GTM_OK;
+        }
+        lds_set_of[variant] = lds;
+    }
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, FITD_BLOCK, lds) != hipSuccess || per_cu < 1 ||
+        groups > per_cu * cus) {
+        (void)hipGetLastError();
+        return GTM_OK;
+    }
+
+    Key key = key_of(cfg);
+    FitDeepParams p{};
+    p.tiles = g->tiles;
+    p.X = g->X;
+    p.node_index = g->node_index;
+    p.n_nodes = g->number_of_graph_nodes;
+    p.n_edges = g->number_of_graph_node_edges;
+    p.edge_index = g->edge_index;
+    p.edge = g->edge;
+    p.encoded_Y = encoded_Y;
+    p.tg = tg;
+    p.first_example = first_example;
+    p.n_examples = n_examples;
+    p.first_step = (uint32_t)first_step;
+    p.bank[0] = s->ta_state;
+    p.thr16[0] = feedback_threshold(cfg->s[0]);
+    for (int l = 1; l < cfg->depth; ++l) {
+        p.bank[l] = s->message_ta_state[l - 1];
+        p.thr16[l] = feedback_threshold(cfg->s[l]);
+    }
+    p.weights = s->clause_weights;
+    p.hv = s->hypervectors;
+    p.depth = cfg->depth;
+    p.literals = cfg->literals;
+    p.n_types = g->number_of_node_types;
+    p.C = d.C;
+    p.LA = d.LA;
+    p.MC = d.MC;
+    p.MW = MW;
+    p.M = d.M;
+    p.MB = d.MB;
+    p.B = d.B;
+    p.K = d.K;
+    p.T = cfg->threshold;
+    p.negative = cfg->negative_clauses;
+    p.boost = cfg->boost_true_positive_feedback;
+    p.max_included = cfg->max_included_literals;
+    p.has_edges = g->total_edges > 0;
+    p.filter = d.filter;
+    p.k0 = key.k0;
+    p.k1 = key.k1;
+    p.q_thr = q_threshold(cfg->q, cfg->classes);
+    p.got = w.coop_got;
+    p.arrived = w.coop_arrived;
+    p.class_sum = (unsigned long long *)w.class_sum;
+    p.abort_flag = (uint32_t *)((unsigned long long *)w.class_sum + (size_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE);
+    p.spin_limit = 4000000u;
+    if (const char *e = getenv("GTM_FIT_SPIN_LIMIT")) {  // tests force the give-up path
+        p.force_abort = strcmp(e, "abort") == 0;
+        if (!p.force_abort) p.spin_limit = (uint32_t)strtoul(e, nullptr, 10);
+    }
+    p.clauses_per_group = per_group;
+    p.NW = NW;
+    p.rows_words = rows_words;
+    p.max_nodes = cfg->max_nodes;
+    p.edge_cap = edge_cap;
+    p.edge_types = edge_types;
+
+    // the exchange buffers start at zero; the model is kept as it was in case the run gives up
+    hipLaunchKernelGGL(k_fill_u64, dim3(blocks_for((int64_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE + 1, TPB)), dim3(TPB), 0, st,
+                       (unsigned long long *)w.class_sum, (int64_t)0, 0ull, (int64_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE + 1);
+    if (int rc = check_launch("fill")) return rc;
+    hipLaunchKernelGGL(k_fill_u64, dim3(blocks_for((int64_t)layers * FITD_PARTS * FITD_STRIDE, TPB)), dim3(TPB), 0, st,
+                       w.coop_arrived, (int64_t)0, 0ull, (int64_t)layers * FITD_PARTS * FITD_STRIDE);
+    if (int rc = check_launch("fill")) return rc;
+    hipLaunchKernelGGL(k_fill_i32, dim3(blocks_for((int64_t)w.coop_words, TPB)), dim3(TPB), 0, st, (int32_t *)w.coop_got,
+                       (int64_t)w.coop_words, 0);
+    if (int rc = check_launch("fill")) return rc;
+    const size_t bank0_bytes = (size_t)d.C * d.LA * d.B * 4, bankm_bytes = (size_t)d.C * d.MC * d.B * 4;
+    const size_t weights_bytes = (size_t)d.K * d.C * 4;
+    hipError_t e = hipMemcpyAsync(w.bank_backup, s->ta_state, bank0_bytes, hipMemcpyDeviceToDevice, st);
+    for (int l = 0; l < layers && e == hipSuccess; ++l)
+        e = hipMemcpyAsync((char *)w.bank_backup + bank0_bytes + (size_t)l * bankm_bytes, s->message_ta_state[l], bankm_bytes,
+                           hipMemcpyDeviceToDevice, st);
+    if (e == hipSuccess) e = hipMemcpyAsync(w.weights_backup, s->clause_weights, weights_bytes, hipMemcpyDeviceToDevice, st);
+    if (e != hipSuccess) return fail(GTM_ERR_HIP, "keeping a copy of the model state: %s", hipGetErrorString(e));
+
+#ifdef FITD_CLOCKS
+    p.clocks = (unsigned long long *)w.bank_backup;  // (development builds only: an aborted run is not restored correctly)
+#endif
+    void *args[] = {&p};
+    profile_start("k_fit_deep_persistent", st);
+    e = hipLaunchCooperativeKernel(kernel, dim3(groups), dim3(FITD_BLOCK), args, (unsigned)lds, st);
+    if (e != hipSuccess) return fail(GTM_ERR_HIP, "cooperative launch of the training kernel: %s", hipGetErrorString(e));
+    profile_stop(st);
+    uint32_t flag = 0;
+    e = hipMemcpyAsync(&flag, p.abort_flag, 4, hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return fail(GTM_ERR_HIP, "training kernel: %s", hipGetErrorString(e));
+#ifdef FITD_CLOCKS
+    {
+        unsigned long long clk[16];
+        (void)hipMemcpy(clk, w.bank_backup, sizeof(clk), hipMemcpyDeviceToHost);
+        fprintf(stderr, "fitd clocks (us per example, %d groups):", groups);
+        for (int k = 0; k < 13; ++k) fprintf(stderr, " %d:%.2f", k, clk[k] * 0.01 / n_examples);
+        fprintf(stderr, "\n");
+    }
+#endif
+    if (flag != 0) {
+        e = hipMemcpyAsync(s->ta_state, w.bank_backup, bank0_bytes, hipMemcpyDeviceToDevice, st);
+        for (int l = 0; l < layers && e == hipSuccess; ++l)
+            e = hipMemcpyAsync(s->message_ta_state[l], (char *)w.bank_backup + bank0_bytes + (size_t)l * bankm_bytes, bankm_bytes,
+                               hipMemcpyDeviceToDevice, st);
+        if (e == hipSuccess) e = hipMemcpyAsync(s->clause_weights, w.weights_backup, weights_bytes, hipMemcpyDeviceToDevice, st);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        if (e != hipSuccess)
+            return fail(GTM_ERR_HIP, "training kernel gave up waiting at a device-wide barrier (%d workgroups) and the "
+                                     "model state could not be restored: %s", groups, hipGetErrorString(e));
+        return fail(GTM_ERR_HIP, "training kernel gave up waiting at a device-wide barrier (%d workgroups); "
+                                 "the model state is as it was before the call", groups);
+    }
+    *done = true;
+    return GTM_OK;
+}
+
 // `_fit`'s inner loop for a depth-1 model on a data set that has tiles: two
 // launches per example (fit_fused.h).
 int fit_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
@@ -2039,7 +2219,14 @@ int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *st
     }
     if (cfg->depth > 1 && graphs->tiles && graphs->number_of_node_types >= 1 && !getenv("GTM_NO_DEEP_FIT")) {
         TileGeom tg = geometry_for(cfg, graphs, d.K);
-        if (tg.ok && tg.slot_words <= 64 && cfg->max_nodes <= 2048)  // one lane per word of the graph's nodes
+        if (tg.ok && tg.slot_words <= 64 && cfg->max_nodes <= 2048) {  // one lane per word of the graph's nodes
+            bool done = false;
+            if (int rc = fit_deep_persistent(d, cfg, graphs, state, tg, w, encoded_Y, first_example, n_examples, first_step, st,
+                                             &done))
+                return rc;
+            if (done) return GTM_OK;
+        }
+        if (tg.ok && tg.slot_words <= 64 && cfg->max_nodes <= 2048)
             return fit_deep_on_tiles(d, cfg, graphs, state, tg, w, encoded_Y, first_example, n_examples, first_step, h_n,
                                      h_base, st);
     }

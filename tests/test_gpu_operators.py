@@ -364,6 +364,7 @@ def test_fused_fit_with_message_layers(shape, boost, max_included, state_bits, m
 
     monkeypatch.setenv("GTM_FIT_FACTOR_MIN", "0" if messages == "by-node-vectors" else str(1 << 60))
     monkeypatch.setenv("GTM_NO_SMALL_FIT", "1")  # the one-workgroup kernel has its own test
+    monkeypatch.setenv("GTM_NO_DEEP_PERSISTENT_FIT", "1")  # and so has the one-launch kernel
 
     g = dict(shape["g"])
     if "sizes" not in g:
@@ -389,6 +390,107 @@ def test_fused_fit_with_message_layers(shape, boost, max_included, state_bits, m
         for layer in range(depth - 1):
             assert np.array_equal(banks[layer], model.message_ta_state[layer]), "bank %d epoch %d" % (layer, epoch)
     assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
+
+
+ONE_LAUNCH_DEEP_SHAPES = [
+    # (every MESSAGE_SIZE a multiple of 32) several graphs per word with node and edge types; three layers;
+    # two truth words per graph; 361-node graphs with four edge types, more clauses than one workgroup
+    # per clause can hold; graphs without nodes among others, four layers; single nodes with self-loops;
+    # no edges at all; several messages bits per clause and a large hypervector
+    dict(seed=61, g=dict(n_graphs=40, max_nodes=3, hv_size=16, node_types=("a", "b"), edge_types=("x", "y", "z")),
+         m=dict(classes=2, clauses=33, depth=2, message_size=64)),
+    dict(seed=62, g=dict(n_graphs=24, max_nodes=16, min_nodes=9, hv_size=20),
+         m=dict(classes=4, clauses=100, depth=3, message_size=64, message_bits=3)),
+    dict(seed=63, g=dict(n_graphs=10, max_nodes=64, min_nodes=40, hv_size=40, edge_types=("l", "r", "u", "d"),
+                         node_types=("a", "b")),
+         m=dict(classes=3, clauses=70, depth=2, message_size=96)),
+    dict(seed=64, g=dict(n_graphs=6, max_nodes=361, min_nodes=300, hv_size=128, edge_types=("l", "r", "u", "d")),
+         m=dict(classes=10, clauses=700, depth=2, message_size=256)),
+    dict(seed=65, g=dict(n_graphs=8, hv_size=16, sizes=[5, 0, 33, 1, 0, 40, 64, 0]),
+         m=dict(classes=3, clauses=20, depth=4, message_size=32, message_bits=1)),
+    dict(seed=66, g=dict(n_graphs=30, max_nodes=1, hv_size=40), m=dict(classes=3, clauses=50, depth=2, message_size=32)),
+    dict(seed=67, g=dict(n_graphs=12, max_nodes=40, min_nodes=20, hv_size=100, max_degree=0),
+         m=dict(classes=5, clauses=64, depth=2, message_size=128)),
+    dict(seed=68, g=dict(n_graphs=16, max_nodes=30, min_nodes=2, hv_size=24, edge_types=("p", "q")),
+         m=dict(classes=2, clauses=300, depth=3, message_size=512, message_bits=4)),
+]
+
+
+@pytest.mark.parametrize("shape", ONE_LAUNCH_DEEP_SHAPES, ids=lambda s: "deep%d" % s["seed"])
+@pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 9, 5), (1, None, 12)])
+def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bits, monkeypatch):
+    """A run of training examples of a model with message layers in one cooperative launch
+    (k_fit_deep_persistent: clauses spread over workgroups, the nodes' messages and the class sums
+    exchanged through device memory): automata of every bank and the weights after each of two
+    epochs == the oracle; each epoch is split into two calls, so the state's round trip
+    through memory and the restart of the exchange buffers are covered."""
+    import ctypes
+    from tests.gpu_harness import Device
+    from graphtsetlinmachine_amd import _abi
+
+    monkeypatch.setenv("GTM_NO_SMALL_FIT", "1")
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    m = dict(shape["m"])
+    depth = m.pop("depth")
+    cfg = helpers.oracle_config(graphs, **m, depth=depth, T=30, boost=boost, max_included=max_included,
+                                state_bits=state_bits)
+    model = helpers.random_model(shape["seed"], cfg, depth, s=(3.0, 2.0, 1.5, 1.2)[:depth],
+                                 include_density=shape.get("density", 0.02), message_density=0.02)
+    dev = Device(model, graphs)
+    assert dev.build_tiles()
+    rng = np.random.default_rng(shape["seed"])
+    G = graphs.number_of_graphs
+    Y = o.encode_labels(rng.integers(0, cfg.classes, size=G), cfg.classes, cfg.threshold)
+    name, launches, total = ctypes.c_char_p(), ctypes.c_int32(), ctypes.c_double()
+    for epoch in range(2):
+        o.fit(model, graphs, Y)
+        _abi.call("gtm_profile_enable", 1)
+        dev.fit(Y, 0, G // 3, epoch * G)
+        dev.fit(Y, G // 3, G - G // 3, epoch * G + G // 3)
+        _abi.call("gtm_profile_read", ctypes.byref(name), ctypes.byref(launches), ctypes.byref(total))
+        _abi.call("gtm_profile_enable", 0)
+        assert (name.value, launches.value) == (b"k_fit_deep_persistent", 2), "the one-launch kernel should have run"
+        ta, banks, w = dev.download()
+        assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
+        assert np.array_equal(ta, model.ta_state), "layer-0 automata after epoch %d" % epoch
+        for layer in range(depth - 1):
+            assert np.array_equal(banks[layer], model.message_ta_state[layer]), "bank %d epoch %d" % (layer, epoch)
+    assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
+
+
+def test_one_launch_fit_with_message_layers_gives_up_instead_of_hanging(monkeypatch):
+    """As for the depth-1 kernel: GTM_FIT_SPIN_LIMIT=abort makes every workgroup give up at its first
+    device-wide wait; the kernel drains, the call reports it, every bank and the weights are as
+    they were, and the same model trains normally afterwards."""
+    from tests.gpu_harness import Device
+    from graphtsetlinmachine_amd import _abi
+
+    monkeypatch.setenv("GTM_NO_SMALL_FIT", "1")
+    shape = ONE_LAUNCH_DEEP_SHAPES[1]
+    graphs = helpers.random_graphs(shape["seed"], **shape["g"])
+    m = dict(shape["m"])
+    depth = m.pop("depth")
+    cfg = helpers.oracle_config(graphs, **m, depth=depth, T=30)
+    model = helpers.random_model(shape["seed"], cfg, depth, s=(3.0, 2.0, 1.5)[:depth], include_density=0.02,
+                                 message_density=0.02)
+    dev = Device(model, graphs)
+    assert dev.build_tiles()
+    G = graphs.number_of_graphs
+    Y = o.encode_labels(np.arange(G) % cfg.classes, cfg.classes, cfg.threshold)
+
+    def same_as_oracle():
+        ta, banks, w = dev.download()
+        return (np.array_equal(w, model.clause_weights) and np.array_equal(ta, model.ta_state) and
+                all(np.array_equal(banks[l], model.message_ta_state[l]) for l in range(depth - 1)))
+
+    monkeypatch.setenv("GTM_FIT_SPIN_LIMIT", "abort")
+    with pytest.raises(_abi.GtmError, match="gave up waiting.*as it was before the call"):
+        dev.fit(Y, 0, G, 0)
+    monkeypatch.delenv("GTM_FIT_SPIN_LIMIT")
+    assert same_as_oracle()
+    o.fit(model, graphs, Y)
+    dev.fit(Y, 0, G, 0)
+    assert same_as_oracle()
 
 
 SMALL_DEEP_SHAPES = [
