@@ -27,9 +27,10 @@
 // received rows of layer l for bank l.
 //
 // Nothing is exchanged through ordinary stores and no cache is flushed: every
-// word another workgroup reads is written with a device-scope atomic whose
-// returned value the writer waits for before it announces its arrival, and read
-// with a device-scope atomic load after the reader has seen every arrival.  The
+// word another workgroup reads is written with a device-scope atomic (carried out
+// where all workgroups see it) that the writer waits for - its wave's count of
+// outstanding memory operations falls to zero - before it announces its arrival,
+// and read with a device-scope atomic load after the reader has seen every arrival.  The
 // received rows live in a ring of three slots (example i uses slot i mod 3).  A
 // workgroup clears its share of slot (i + 1) mod 3 during example i: whoever is in
 // example i has seen every workgroup arrive at the class sums of example i - 1, so
@@ -37,6 +38,15 @@
 // contribution of example i + 1 cannot precede this workgroup's arrival at the
 // class sums of example i, which it makes after the clearing.  Arrival counters
 // only ever grow.
+//
+// Two layouts (template flag BIG).  Small models keep the automata of the own clauses in LDS, next to
+// the layer-0 rows of the graph and all M received rows.  Where that does not fit (8000 clauses on
+// 841-node graphs with 2048 literals), the automata stay in global memory - a workgroup only ever
+// touches those of its own clauses, with ordinary loads and stores - and LDS holds a copy of their
+// include planes; layer 0 reads the literal rows it needs from the tiles in place; the received rows
+// pass through LDS a window of rows at a time; and what each node received is also published
+// node-major (`vec`: every workgroup turns the bits of its share of the nodes while a window is in
+// LDS), so that the message literals of a picked node are words to load, not bits to collect.
 //
 // Every wait is bounded (`spin_limit` polls); a workgroup that gives up raises the
 // abort flag and every workgroup leaves at its next wait, so the grid always drains.
@@ -63,6 +73,7 @@ constexpr int FITD_MAX_EDGE_TYPES = 16;
 struct FitDeepParams {
     // data set
     const uint32_t *tiles, *X, *node_index, *n_nodes, *n_edges, *edge_index, *edge;
+    const uint32_t *order;  // the literals, the ones that hold least often in the data set first
     const int32_t *encoded_Y;
     TileGeom tg;
     int first_example, n_examples;
@@ -76,6 +87,7 @@ struct FitDeepParams {
     uint64_t q_thr;
     // exchange (device memory, zero on entry)
     uint32_t *got;                  // [3][depth - 1][M][NW]
+    uint32_t *vec;                  // [depth - 1][max_nodes][MW] what each node received, node-major (BIG only)
     unsigned long long *arrived;    // [depth - 1][FITD_PARTS * FITD_STRIDE]
     unsigned long long *class_sum;  // [3][K][FITP_SUM_PARTS] words FITP_SUM_STRIDE apart
     uint32_t *abort_flag;
@@ -83,7 +95,9 @@ struct FitDeepParams {
     int force_abort;
     int clauses_per_group;
     int NW;          // words of a row over the nodes of the largest graph
-    int rows_words;  // LDS words of the staged layer-0 rows: (literals + n_types + 1) * NW
+    int rows_words;  // LDS words of the staged layer-0 rows: (literals + n_types + 1) * NW; 0 when they are read in place (BIG)
+    int window_rows; // received rows that pass through LDS at a time: a multiple of 32, M unless BIG
+    int by_masks;    // phase a goes over the edges once for 32 clauses (the window's LDS is large enough for that)
     int max_nodes;   // nodes of the largest graph
     int edge_cap;    // edges of the graph that has most (0 without edges)
     int edge_types;  // largest edge type + 1 (at most FITD_MAX_EDGE_TYPES)
@@ -92,13 +106,14 @@ struct FitDeepParams {
 #endif
 };
 
-inline size_t fit_deep_lds_words(int depth, int per_group, int LA, int MC, int M, int MB, int B, int K, int NW, int rows_words,
-                                 int max_nodes, int edge_cap, int edge_types) {
+// LDS words of the kernel.  big: rows_words == 0 and window_rows <= M; else window_rows == M.
+inline size_t fit_deep_lds_words(bool big, int depth, int literals, int per_group, int LA, int MC, int MB, int B, int K, int NW, int rows_words,
+                                 int window_rows, int max_nodes, int edge_cap, int edge_types) {
     const size_t per_clause = (size_t)LA + (size_t)(depth - 1) * MC;
-    return 2 * ((size_t)rows_words + 2 * (size_t)max_nodes + (size_t)edge_cap + (size_t)K) + (size_t)M * NW +
-           (size_t)per_group * edge_types * NW + (size_t)per_group * per_clause * B + 2 * (size_t)per_group * K +
+    return 2 * ((size_t)rows_words + 2 * (size_t)max_nodes + (size_t)edge_cap + (size_t)K) + (size_t)window_rows * NW +
+           (size_t)per_group * edge_types * NW + (size_t)per_group * per_clause * (big ? 1 : B) + 2 * (size_t)per_group * K +
            2 * (size_t)per_group + (size_t)per_group * NW + 2 * (size_t)K + 6 * (size_t)K +
-           (size_t)per_group * (depth - 1) * MC + (size_t)per_group * MB + 64;
+           (big ? (size_t)literals : (size_t)per_group * (depth - 1) * MC) + (size_t)per_group * MB + 64;
 }
 
 // What the cooperative kernel has to know about the edges of a run of examples: [0] most edges of
@@ -154,36 +169,51 @@ __device__ __forceinline__ bool fitd_wait(const unsigned long long *parts, unsig
     }
 }
 
+// A 32 x 32 bit matrix held one row per lane (both halves of a wave hold one each): afterwards lane b
+// holds column b, i.e. bit k of its word = bit b of what lane k (of the same half) held.
+__device__ __forceinline__ uint32_t fitd_transpose32(uint32_t a, int lane) {
+    uint32_t m = 0x0000FFFFu;
+#pragma unroll
+    for (int j = 16; j != 0; j >>= 1) {
+        const uint32_t other = __shfl_xor(a, j);
+        a = (lane & j) ? (a & ~m) | ((other >> j) & m) : (a & m) | ((other << j) & ~m);
+        m ^= m << (j >> 1);
+    }
+    return a;
+}
+
 // truth[cl] &= the rows of the literals that words [w_lo, w_hi) of an include plane hold; returns how many
-// they hold.  `inc` points at the include plane's word 0 (words B apart); row r of the literal rows is at
-// col[r * stride] for this lane; literals >= `half` are negated: the complement of row (literal - half)
-// when `complement`, else a row of their own.  One wave.
-__device__ __forceinline__ int fitd_and_rows(const uint32_t *inc, int B, int w_lo, int w_hi, int last_word, uint32_t filter,
-                                             const uint32_t *col, int stride, int half, bool complement, int ones_row,
-                                             uint32_t &acc, int lane) {
+// they hold.  `inc` points at the include plane's word 0 (words inc_stride apart); row r of the literal rows
+// is at col[(r - row_base) * stride] for this lane; literals >= `half` are negated: the complement of row
+// (literal - half) when `complement`, else a row of their own.  One wave.
+template <typename Rows>
+__device__ __forceinline__ int fitd_and_rows(const uint32_t *inc, int inc_stride, int w_lo, int w_hi, int last_word,
+                                             uint32_t filter, Rows col, int stride, int row_base, int half, bool complement,
+                                             int ones_row, uint32_t &acc, int lane) {
     int included = 0;
     for (int w0 = w_lo; w0 < w_hi; w0 += 64) {
-        uint32_t mine = w0 + lane < w_hi ? inc[(w0 + lane) * B] : 0u;
+        uint32_t mine = w0 + lane < w_hi ? inc[(w0 + lane) * inc_stride] : 0u;
         if (w0 + lane == last_word) mine &= filter;
         included += wave_sum_small(__popc(mine));
         unsigned long long nonzero = __ballot(mine != 0);
         if (__ballot(acc != 0u) == 0ull) continue;  // false everywhere stays false: only the count matters
         while (nonzero) {
+            if (__ballot(acc != 0u) == 0ull) break;
             const int wl = __ffsll((long long)nonzero) - 1;
             nonzero &= nonzero - 1;
             uint32_t m = __builtin_amdgcn_readlane(mine, wl);
             const int first = (w0 + wl) << 5;
             const bool negated = complement && first >= half;  // (a word holds positive or negated literals, never both)
-            const int row0 = negated ? first - half : first;
+            const int row0 = (negated ? first - half : first) - row_base;
             const uint32_t flip = negated ? 0xFFFFFFFFu : 0u;
             while (m) {
                 uint32_t r[8];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     const bool used = m != 0;
-                    const int row = used ? row0 + __builtin_ctz(m) : ones_row;
+                    const int row = used ? row0 + __builtin_ctz(m) : ones_row - row_base;
                     m &= m - 1;
-                    r[u] = (col[row * stride] ^ flip) | (used ? 0u : 0xFFFFFFFFu);
+                    r[u] = (col[(int64_t)row * stride] ^ flip) | (used ? 0u : 0xFFFFFFFFu);
                 }
 #pragma unroll
                 for (int u = 0; u < 8; ++u) acc &= r[u];
@@ -194,7 +224,8 @@ __device__ __forceinline__ int fitd_and_rows(const uint32_t *inc, int B, int w_l
 }
 
 // MAXB: bit planes of an automaton kept in registers while a word is updated (>= B).
-template <int MAXB>
+// BIG: automata in global memory, layer-0 rows read in place, received rows in windows (see the top).
+template <int MAXB, bool BIG>
 __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParams p) {
     extern __shared__ uint32_t lds[];
     const int tid = threadIdx.x;
@@ -206,18 +237,20 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
     const int c0 = g * own_max;
     const int n_own = min(own_max, p.C - c0);
     const int LA = p.LA, MC = p.MC, MW = p.MW, M = p.M, B = p.B, K = p.K, NW = p.NW, L = p.depth - 1, TE = p.edge_types;
+    const int WR = p.window_rows;
     const int per_clause = LA + L * MC;  // automaton words of a clause over all banks
+    const int SB = BIG ? 1 : B;          // LDS words per automaton word: the include plane, or every plane
 
     // LDS carve-up
-    // per example, twice (the next example's are fetched while this one waits for the class sums):
+    // per example, twice (the next example's are fetched while this one waits):
     //   [rows_words] staged layer-0 rows of the graph, [max_nodes] first edge of a node counted from the
     //   graph's first, [max_nodes] edges of a node, [edge_cap] destination | type << 16, [K] encoded labels
     const size_t staged_words = (size_t)p.rows_words + 2 * (size_t)p.max_nodes + (size_t)p.edge_cap + (size_t)K;
-    uint32_t *mrows = lds + 2 * staged_words;                     // [M][NW] received rows of the current layer
-    uint32_t *reach = mrows + (size_t)M * NW;                     // [own][TE][NW] nodes reached from a clause's true nodes, per edge type
-    // [own][per_clause][B]: bank 0 words, then bank 1 ...; 32-byte aligned (a word's 8 planes are moved as two vectors)
+    uint32_t *mrows = lds + 2 * staged_words;                     // [WR][NW] received rows of the current layer (a window of them)
+    uint32_t *reach = mrows + (size_t)WR * NW;                    // [own][TE][NW] nodes reached from a clause's true nodes, per edge type
+    // [own][per_clause][SB]: bank 0 words, then bank 1 ...; 32-byte aligned (a word's 8 planes are moved as two vectors)
     uint32_t *ta = lds + ((size_t)(reach + (size_t)own_max * TE * NW - lds + 7) & ~(size_t)7);
-    int32_t *wts = (int32_t *)(ta + (size_t)own_max * per_clause * B);  // [own][K]
+    int32_t *wts = (int32_t *)(ta + (size_t)own_max * per_clause * SB);  // [own][K]
     int32_t *upd = wts + (size_t)own_max * K;                     // [own][K]
     int32_t *node_of = upd + (size_t)own_max * K;                 // [own]
     int32_t *incl_of = node_of + own_max;                         // [own]
@@ -225,26 +258,35 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
     int32_t *sums = (int32_t *)(truth + (size_t)own_max * NW);    // [K]
     int32_t *votes = sums + K;                                    // [K]
     uint32_t *seen = (uint32_t *)(votes + K);                     // [3][2][K] (see fit_persistent.h)
-    uint32_t *mlit = seen + 6 * K;                                // [own][L][MC] message literal words of the picked node
-    uint32_t *hv_own = mlit + (size_t)own_max * L * MC;           // [own][MB] hypervector bits of the own clauses
+    uint32_t *hv_own = seen + 6 * K;                              // [own][MB] hypervector bits of the own clauses
+    uint32_t *mlit = hv_own + (size_t)own_max * p.MB;             // [own][L][MC] message literal words of the picked node (not BIG)
+    uint32_t *order = mlit;                                       // [literals] the literals, the ones that seldom hold first (BIG)
     __shared__ int go_on;
+    __shared__ int next_unit[2];  // waves take their units of work (a clause, or some words of one) from here: [0] layer 0, [1] a message layer
+
+    // where the automata of own clause cl, word w of all its banks' words, live in global memory
+    auto word_in_memory = [&](int cl, int w) -> uint32_t * {
+        const int bank = w < LA ? 0 : 1 + (w - LA) / MC;
+        const int wl = w < LA ? w : (w - LA) % MC, chunks = bank == 0 ? LA : MC;
+        return p.bank[bank] + ((int64_t)(c0 + cl) * chunks + wl) * B;
+    };
 
     // own state -> LDS
     for (int k = tid; k < K; k += FITD_BLOCK) votes[k] = 0;
     for (int j = tid; j < 6 * K; j += FITD_BLOCK) seen[j] = 0u;
-    for (int i = tid; i < n_own * per_clause * B; i += FITD_BLOCK) {
-        const int cl = i / (per_clause * B), r = i - cl * per_clause * B;
-        const int w = r / B, b = r - w * B;
-        const int bank = w < LA ? 0 : 1 + (w - LA) / MC;
-        const int wl = w < LA ? w : (w - LA) % MC, chunks = bank == 0 ? LA : MC;
-        ta[i] = p.bank[bank][((int64_t)(c0 + cl) * chunks + wl) * B + b];
+    for (int i = tid; i < n_own * per_clause * SB; i += FITD_BLOCK) {
+        const int cl = i / (per_clause * SB), r = i - cl * per_clause * SB;
+        const int w = r / SB, b = BIG ? B - 1 : r - w * SB;
+        ta[i] = word_in_memory(cl, w)[b];
     }
     for (int i = tid; i < n_own * K; i += FITD_BLOCK) {
         const int cl = i / K, k = i - cl * K;
         wts[i] = p.weights[(int64_t)k * p.C + c0 + cl];
     }
     for (int i = tid; i < n_own * p.MB; i += FITD_BLOCK) hv_own[i] = p.hv[(int64_t)c0 * p.MB + i];
-    if (tid == 0) go_on = 1;
+    if constexpr (BIG)
+        for (int i = tid; i < p.literals; i += FITD_BLOCK) order[i] = p.order[i];
+    if (tid == 0) go_on = 1, next_unit[0] = 0;
     lds_barrier();
 
     const int ones_row = p.literals + p.n_types;
@@ -252,25 +294,25 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
     const size_t share_lo = (size_t)g * layer_words / G, share_hi = (size_t)(g + 1) * layer_words / G;
     // how the automaton words of the own clauses are spread over the waves: `parts` waves per clause
     const int parts0 = max(1, min(LA, WAVES / max(1, n_own))), chunk0 = (LA + parts0 - 1) / parts0;
-    const int parts1 = max(1, min(MC, WAVES / max(1, n_own))), chunk1 = (MC + parts1 - 1) / parts1;
-    uint32_t sink = 0u;  // keeps the returned values of the exchange atomics alive
 #ifdef FITD_CLOCKS
     unsigned long long clk[16] = {}, last_ = wall_clock64();
 #endif
 
-    // the layer-0 rows of a graph (only the words that hold its nodes) and its edges -> LDS
+    // the layer-0 rows of a graph (only the words that hold its nodes; not BIG), its edges and labels -> LDS
     // (threads t of nt take part)
     auto stage = [&](int ex_s, uint32_t *to, int t, int nt) {
         const int n_s = (int)p.n_nodes[ex_s];
         const int64_t base_s = (int64_t)p.node_index[ex_s];
-        const FitGraph fg_s = fit_graph_slot(p.tg, ex_s, n_s);
-        const uint32_t *tile = p.tiles + (int64_t)fg_s.tile * p.tg.rows * p.tg.tw + fg_s.word0;
-        const int words_s = fg_s.words, total = (p.literals + p.n_types + 1) * words_s;
         int32_t *y_s = (int32_t *)(to + p.rows_words + 2 * p.max_nodes + p.edge_cap);
         for (int k = t; k < K; k += nt) y_s[k] = p.encoded_Y[(int64_t)ex_s * K + k];
-        for (int at = t; at < total; at += nt) {
-            const int r = at / words_s, w = at - r * words_s;
-            to[at] = tile[(int64_t)r * p.tg.tw + w];
+        if constexpr (!BIG) {
+            const FitGraph fg_s = fit_graph_slot(p.tg, ex_s, n_s);
+            const uint32_t *tile = p.tiles + (int64_t)fg_s.tile * p.tg.rows * p.tg.tw + fg_s.word0;
+            const int words_s = fg_s.words, total = (p.literals + p.n_types + 1) * words_s;
+            for (int at = t; at < total; at += nt) {
+                const int r = at / words_s, w = at - r * words_s;
+                to[at] = tile[(int64_t)r * p.tg.tw + w];
+            }
         }
         if (p.has_edges && n_s > 0) {
             uint32_t *first_s = to + p.rows_words, *count_s = first_s + p.max_nodes, *pack_s = count_s + p.max_nodes;
@@ -287,7 +329,12 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
             }
         }
     };
-
+    // the next unit of work for this wave (clauses differ a lot in what they cost: a fixed share per wave leaves most waves idle)
+    auto take_unit = [&](int which) {
+        int u = 0;
+        if (lane == 0) u = atomicAdd(&next_unit[which], 1);
+        return __builtin_amdgcn_readfirstlane(u);
+    };
     if (p.n_examples > 0) stage(p.first_example, lds, tid, FITD_BLOCK);
     lds_barrier();
 
@@ -302,39 +349,55 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
         uint32_t *got_now = p.got + (size_t)slot * slot_words, *got_next = p.got + (size_t)slot_next * slot_words;
         unsigned long long *slot_sum = p.class_sum + (size_t)slot * K * FITP_SUM_PARTS * FITP_SUM_STRIDE;
 
-        // ---- 0. the graph's layer-0 rows and edges are in LDS (fetched during the previous example)
+        // ---- 0. the graph's edges (and layer-0 rows) are in LDS, fetched during the previous example
         uint32_t *rows0 = lds + (size_t)(i & 1) * staged_words;   // row r at rows0[r * words]
         const uint32_t *e_first = rows0 + p.rows_words, *e_count = e_first + p.max_nodes, *e_pack = e_count + p.max_nodes;
         const int32_t *y = (const int32_t *)(e_pack + p.edge_cap);
+        const uint32_t *tile = p.tiles + (int64_t)fg.tile * p.tg.rows * p.tg.tw + fg.word0;  // (BIG: the rows in place)
+        const int row_stride = BIG ? p.tg.tw : words;
         for (int at = tid; at < n_own * TE * NW; at += FITD_BLOCK) reach[at] = 0u;
         for (int cl = tid; cl < n_own; cl += FITD_BLOCK) incl_of[cl] = 0;
         // ---- 1. layer 0 (K1): truth of own clauses over the graph's nodes, lane = word; the include
         //         words of a clause are shared out over `parts0` waves, whose results meet in LDS.
         //         Truth starts as the clause's node-type row (K1 looks at nodes of the clause's type only).
-        for (int at = tid; at < n_own * NW; at += FITD_BLOCK) {
-            const int cl = at / NW, w = at - cl * NW;
-            truth[at] = w < words ? rows0[(p.literals + (c0 + cl) % p.n_types) * words + w] : 0u;
-        }
-        lds_barrier();
-        FITD_TICK(0)
-        {
+        if constexpr (BIG) {
+            // (clauses with many literals: the rows of a few literals that seldom hold, then the surviving
+            // nodes against the whole include mask, as k_fit_eval does)
             const bool active = lane < words;
-            const uint32_t *col = rows0 + (active ? lane : 0);
+            for (int cl = take_unit(0); cl < n_own; cl = take_unit(0)) {
+                int included;
+                const uint32_t v = fit_clause_truth(ta + (size_t)cl * per_clause, 1, LA, p.filter, tile + (active ? lane : 0), row_stride,
+                                                    p.literals, p.literals + (c0 + cl) % p.n_types, ones_row, fg, n, FIT_WALK_ALL,
+                                                    p.X + base * LA, order, active, lane, &included);
+                if (lane < NW) truth[cl * NW + lane] = v;
+                if (lane == 0) incl_of[cl] = included;
+            }
+            lds_barrier();
+            FITD_TICK(0)
+        } else {
+            for (int at = tid; at < n_own * NW; at += FITD_BLOCK) {
+                const int cl = at / NW, w = at - cl * NW;
+                truth[at] = w < words ? rows0[(int64_t)(p.literals + (c0 + cl) % p.n_types) * row_stride + w] : 0u;
+            }
+            lds_barrier();
+            FITD_TICK(0)
+            const bool active = lane < words;
             for (int u = wave; u < n_own * parts0; u += WAVES) {
                 const int cl = u / parts0, part = u - cl * parts0;
                 uint32_t acc = active ? truth[cl * NW + lane] : 0u;
                 const uint32_t before = acc;
-                const int included = fitd_and_rows(ta + (size_t)cl * per_clause * B + (B - 1), B, part * chunk0,
-                                                   min(LA, (part + 1) * chunk0), LA - 1, p.filter, col, words, 0, false,
-                                                   ones_row, acc, lane);
+                const int included = fitd_and_rows(ta + (size_t)cl * per_clause * SB + (SB - 1), SB, part * chunk0,
+                                                   min(LA, (part + 1) * chunk0), LA - 1, p.filter,
+                                                   (const uint32_t *)rows0 + (active ? lane : 0), row_stride, 0, 0, false, ones_row,
+                                                   acc, lane);
                 if (active && acc != before) atomicAnd(&truth[cl * NW + lane], acc);
                 if (lane == 0 && included) atomicAdd(&incl_of[cl], included);
             }
-        }
-        lds_barrier();
-        if (fg.shift != 0 || fg.mask != 0xFFFFFFFFu) {  // several graphs share a word: keep this graph's bits
-            for (int cl = tid; cl < n_own; cl += FITD_BLOCK) truth[cl * NW] = (truth[cl * NW] >> fg.shift) & fg.mask;
             lds_barrier();
+            if (fg.shift != 0 || fg.mask != 0xFFFFFFFFu) {  // several graphs share a word: keep this graph's bits
+                for (int cl = tid; cl < n_own; cl += FITD_BLOCK) truth[cl * NW] = (truth[cl * NW] >> fg.shift) & fg.mask;
+                lds_barrier();
+            }
         }
         FITD_TICK(1)
 
@@ -346,16 +409,51 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
             const unsigned long long everyone = (unsigned long long)(i + 1) * (unsigned long long)G;
             // a. what the own clauses make the nodes receive
             if (p.has_edges && n > 0) {
-                for (int at = tid; at < n_own * n; at += FITD_BLOCK) {
-                    const int cl = at / n, src = at - cl * n;
-                    if (!((truth[cl * NW + (src >> 5)] >> (src & 31)) & 1u)) continue;
-                    const uint32_t first = e_first[src], count = e_count[src];
-                    for (uint32_t e = 0; e < count; ++e) {
-                        const uint32_t d = e_pack[first + e], dst = d & 0xFFFFu, type = d >> 16;
-                        atomicOr(&reach[(cl * TE + (int)type) * NW + (dst >> 5)], 1u << (dst & 31));
+                if (p.by_masks && n_own > 2) {
+                    // 32 clauses at a time: per node the clauses that are true there as a mask, the masks carried
+                    // along the edges (one pass over the edges whatever the number of clauses), and the masks that
+                    // arrived turned back into a row of nodes per clause and edge type.  (The masks use the
+                    // LDS of the received rows, which are not there yet.)
+                    uint32_t *mask_at = mrows, *mask_in = mrows + p.max_nodes;  // [max_nodes], [TE][max_nodes]
+                    for (int first_cl = 0; first_cl < n_own; first_cl += 32) {
+                        const int nb = min(32, n_own - first_cl);
+                        for (int u = tid >> 5; u < words; u += FITD_BLOCK / 32) {  // half a wave per word of nodes
+                            const int b = lane & 31;
+                            const uint32_t t = fitd_transpose32(b < nb ? truth[(first_cl + b) * NW + u] : 0u, lane);
+                            if (u * 32 + b < n) mask_at[u * 32 + b] = t;
+                        }
+                        for (int at = tid; at < TE * p.max_nodes; at += FITD_BLOCK) mask_in[at] = 0u;
+                        lds_barrier();
+                        for (int src = tid; src < n; src += FITD_BLOCK) {
+                            const uint32_t mask = mask_at[src];
+                            if (mask == 0u) continue;
+                            const uint32_t first = e_first[src], count = e_count[src];
+                            for (uint32_t e = 0; e < count; ++e) {
+                                const uint32_t d = e_pack[first + e], dst = d & 0xFFFFu, type = d >> 16;
+                                atomicOr(&mask_in[type * p.max_nodes + dst], mask);
+                            }
+                        }
+                        lds_barrier();
+                        for (int u = tid >> 5; u < TE * words; u += FITD_BLOCK / 32) {  // half a wave per type and word of nodes
+                            const int type = u / words, w = u - type * words, k = lane & 31;
+                            const uint32_t t = fitd_transpose32(w * 32 + k < n ? mask_in[type * p.max_nodes + w * 32 + k] : 0u, lane);
+                            if (k < nb) reach[((first_cl + k) * TE + type) * NW + w] = t;
+                        }
+                        lds_barrier();
                     }
+                } else {
+                    for (int at = tid; at < n_own * n; at += FITD_BLOCK) {
+                        const int cl = at / n, src = at - cl * n;
+                        if (!((truth[cl * NW + (src >> 5)] >> (src & 31)) & 1u)) continue;
+                        const uint32_t first = e_first[src], count = e_count[src];
+                        for (uint32_t e = 0; e < count; ++e) {
+                            const uint32_t d = e_pack[first + e], dst = d & 0xFFFFu, type = d >> 16;
+                            atomicOr(&reach[(cl * TE + (int)type) * NW + (dst >> 5)], 1u << (dst & 31));
+                        }
+                    }
+                    lds_barrier();
                 }
-                lds_barrier();
+                FITD_TICK(6)
                 for (int at = tid; at < n_own * TE * words; at += FITD_BLOCK) {
                     const int cl = at / (TE * words), r = at - cl * TE * words;
                     const int type = r / words, w = r - type * words;
@@ -363,12 +461,13 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                     if (v != 0u)
                         for (int j = 0; j < p.MB; ++j) {
                             const uint32_t row = (hv_own[cl * p.MB + j] + (uint32_t)type) % (uint32_t)M;
-                            sink |= __hip_atomic_fetch_or(&got_l[(size_t)row * NW + w], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            __hip_atomic_fetch_or(&got_l[(size_t)row * NW + w], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         }
                 }
             }
-            __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);  // every returned value is here: the ORs have been carried out
-            asm volatile("" ::"v"(sink) : "memory");
+            FITD_TICK(7)
+            __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);  // the ORs have been carried out where every workgroup sees them
+            asm volatile("" ::: "memory");
             lds_barrier();
             FITD_TICK(2)
             if (tid == 0)
@@ -380,8 +479,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                 // (meanwhile) this group's share of the slot the next example will send into; the next
                 // example's rows and edges
                 for (size_t at = share_lo + (size_t)(tid - 64); at < share_hi; at += FITD_BLOCK - 64)
-                    sink |= __hip_atomic_exchange(&got_next[(size_t)l * layer_words + at], 0u, __ATOMIC_RELAXED,
-                                                  __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(&got_next[(size_t)l * layer_words + at], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 for (int at = tid - 64; at < n_own * TE * NW; at += FITD_BLOCK - 64) reach[at] = 0u;
                 if (l == 0 && i + 1 < p.n_examples) stage(ex + 1, lds + (size_t)((i + 1) & 1) * staged_words, tid - 64, FITD_BLOCK - 64);
             }
@@ -391,42 +489,62 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                 alive = false;
                 break;
             }
-            // b. all received rows -> LDS, then K2 for own clauses
-            {
-                const unsigned long long *from = (const unsigned long long *)got_l;  // (M NW is even, the rows 8-byte aligned)
-                unsigned long long *to = (unsigned long long *)mrows;
-                const int pairs = M * NW / 2;
-                for (int at0 = tid; at0 < pairs; at0 += 8 * FITD_BLOCK) {
-                    unsigned long long v[8];
+            // b. the received rows -> LDS, a window at a time, and K2 for own clauses on the window's literals
+            for (int r0 = 0; r0 < M; r0 += WR) {
+                const int r1 = min(M, r0 + WR), w_first = r0 >> 5, window_words = (r1 - r0) >> 5;
+                {
+                    const unsigned long long *from = (const unsigned long long *)(got_l + (size_t)r0 * NW);  // (32 NW is even, the rows 8-byte aligned)
+                    unsigned long long *to = (unsigned long long *)mrows;
+                    const int pairs = (r1 - r0) * NW / 2;
+                    for (int at0 = tid; at0 < pairs; at0 += 8 * FITD_BLOCK) {
+                        unsigned long long v[8];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                        v[u] = at0 + u * FITD_BLOCK < pairs
-                                   ? __hip_atomic_load(&from[at0 + u * FITD_BLOCK], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                   : 0ull;
+                        for (int u = 0; u < 8; ++u)
+                            v[u] = at0 + u * FITD_BLOCK < pairs
+                                       ? __hip_atomic_load(&from[at0 + u * FITD_BLOCK], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                       : 0ull;
 #pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                        if (at0 + u * FITD_BLOCK < pairs) to[at0 + u * FITD_BLOCK] = v[u];
+                        for (int u = 0; u < 8; ++u)
+                            if (at0 + u * FITD_BLOCK < pairs) to[at0 + u * FITD_BLOCK] = v[u];
+                    }
+                    if (tid == 0) next_unit[1] = 0;
                 }
-            }
-            lds_barrier();
-            FITD_TICK(4)
-            {
-                const bool active = lane < NW;
-                const uint32_t *col = mrows + (active ? lane : 0);
-                for (int u = wave; u < n_own * parts1; u += WAVES) {
-                    const int cl = u / parts1, part = u - cl * parts1;
-                    uint32_t acc = active ? truth[cl * NW + lane] : 0u;
-                    const uint32_t before = acc;
-                    // (2 M is a multiple of 32: the last word has no tail to mask)
-                    const int included = fitd_and_rows(ta + ((size_t)cl * per_clause + LA + (size_t)l * MC) * B + (B - 1), B,
-                                                       part * chunk1, min(MC, (part + 1) * chunk1), -1, 0u, col, NW, M, true, 0,
-                                                       acc, lane);
-                    if (active && acc != before) atomicAnd(&truth[cl * NW + lane], acc);
-                    if (lane == 0 && included) atomicAdd(&incl_of[cl], included);
+                lds_barrier();
+                FITD_TICK(4)
+                {
+                    const bool active = lane < NW;
+                    const uint32_t *col = mrows + (active ? lane : 0);
+                    const int parts1 = max(1, min(window_words, WAVES / max(1, n_own)));
+                    const int chunk1 = (window_words + parts1 - 1) / parts1;
+                    const int units = n_own * parts1;
+                    const bool queued = units > WAVES;  // (a unit per wave at most: nothing to balance)
+                    for (int u = queued ? take_unit(1) : wave; u < units; u = queued ? take_unit(1) : units) {
+                        const int cl = u / parts1, part = u - cl * parts1;
+                        uint32_t acc = active ? truth[cl * NW + lane] : 0u;
+                        const uint32_t before = acc;
+                        const uint32_t *inc = ta + ((size_t)cl * per_clause + LA + (size_t)l * MC) * SB + (SB - 1);
+                        const int lo = w_first + part * chunk1, hi = min(w_first + window_words, lo + chunk1);
+                        // (2 M is a multiple of 32: the last word has no tail to mask) positive literals, then negated
+                        int included = fitd_and_rows(inc, SB, lo, hi, -1, 0u, col, NW, r0, M, true, r0, acc, lane);
+                        included += fitd_and_rows(inc, SB, MW + lo, MW + hi, -1, 0u, col, NW, r0, M, true, r0, acc, lane);
+                        if (active && acc != before) atomicAnd(&truth[cl * NW + lane], acc);
+                        if (lane == 0 && included) atomicAdd(&incl_of[cl], included);
+                    }
                 }
+                if constexpr (BIG) {
+                    // what the nodes of this group's share received, node-major: bit b of word j of node v = bit v of row 32 j + b
+                    const int v_lo = (int)((int64_t)g * n / G), v_hi = (int)((int64_t)(g + 1) * n / G);
+                    uint32_t *vec_l = p.vec + (size_t)l * p.max_nodes * MW;
+                    for (int at = tid; at < (v_hi - v_lo) * window_words; at += FITD_BLOCK) {
+                        const int v = v_lo + at / window_words, j = at % window_words;
+                        uint32_t word = 0u;
+                        for (int b = 0; b < 32; ++b) word |= ((mrows[(j * 32 + b) * NW + (v >> 5)] >> (v & 31)) & 1u) << b;
+                        __hip_atomic_store(&vec_l[(size_t)v * MW + w_first + j], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
+                lds_barrier();
+                FITD_TICK(5)
             }
-            lds_barrier();
-            FITD_TICK(5)
         }
         if (!alive) break;
 
@@ -458,8 +576,9 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
             if (fired)
                 for (int k = lane; k < K; k += 64) atomicAdd(&votes[k], wts[cl * K + k]);  // LDS
         }
-        __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);  // the next slot's share is cleared before this group arrives
-        asm volatile("" ::"v"(sink) : "memory");
+        // the next slot's share is cleared (and the node-major words are out) before this group arrives
+        __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);
+        asm volatile("" ::: "memory");
         lds_barrier();
         FITD_TICK(9)
 
@@ -470,30 +589,32 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                                    __HIP_MEMORY_SCOPE_AGENT);
             votes[k] = 0;
         }
-        // the message literals of the picked nodes: bit `node` of the layer's received rows, packed as
-        // kernels.py:592-615 packs them (the negated half is the complement); done, like the fetch of the
-        // picked nodes' literal words, while the sums travel
-        for (int at = FITD_BLOCK - 1 - tid; at < n_own * L * MW; at += FITD_BLOCK) {
-            const int cl = at / (L * MW), r = at - cl * L * MW;
-            const int l = r / MW, j = r - l * MW;
-            const int node = node_of[cl];
-            uint32_t word = 0u;
-            if (node >= 0) {
-                if (l == L - 1) {
-                    for (int b = 0; b < 32; ++b) word |= ((mrows[(j * 32 + b) * NW + (node >> 5)] >> (node & 31)) & 1u) << b;
-                } else {
-                    const uint32_t *rows_l = got_now + (size_t)l * layer_words;
-                    for (int b = 0; b < 32; ++b)
-                        word |= ((fitd_load(&rows_l[(size_t)(j * 32 + b) * NW + (node >> 5)]) >> (node & 31)) & 1u) << b;
-                }
-            }
-            mlit[((size_t)cl * L + l) * MC + j] = word;
-            mlit[((size_t)cl * L + l) * MC + MW + j] = ~word;
-        }
         uint32_t x_first = 0u;  // the literal word of this thread's first automaton word of bank 0 (see step 6)
-        if (tid < n_own * per_clause) {
-            const int cl = tid / per_clause, w = tid - cl * per_clause;
-            if (w < LA && node_of[cl] >= 0) x_first = p.X[(base + node_of[cl]) * LA + w];
+        if constexpr (!BIG) {
+            // the message literals of the picked nodes: bit `node` of the layer's received rows, packed as
+            // kernels.py:592-615 packs them (the negated half is the complement); done, like the fetch of the
+            // picked nodes' literal words, while the sums travel
+            for (int at = FITD_BLOCK - 1 - tid; at < n_own * L * MW; at += FITD_BLOCK) {
+                const int cl = at / (L * MW), r = at - cl * L * MW;
+                const int l = r / MW, j = r - l * MW;
+                const int node = node_of[cl];
+                uint32_t word = 0u;
+                if (node >= 0) {
+                    if (l == L - 1) {
+                        for (int b = 0; b < 32; ++b) word |= ((mrows[(j * 32 + b) * NW + (node >> 5)] >> (node & 31)) & 1u) << b;
+                    } else {
+                        const uint32_t *rows_l = got_now + (size_t)l * layer_words;
+                        for (int b = 0; b < 32; ++b)
+                            word |= ((fitd_load(&rows_l[(size_t)(j * 32 + b) * NW + (node >> 5)]) >> (node & 31)) & 1u) << b;
+                    }
+                }
+                mlit[((size_t)cl * L + l) * MC + j] = word;
+                mlit[((size_t)cl * L + l) * MC + MW + j] = ~word;
+            }
+            if (tid < n_own * per_clause) {
+                const int cl = tid / per_clause, w = tid - cl * per_clause;
+                if (w < LA && node_of[cl] >= 0) x_first = p.X[(base + node_of[cl]) * LA + w];
+            }
         }
         if (tid < K) {
             const int k = tid;
@@ -556,22 +677,62 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
         FITD_TICK(11)
 
         // ---- 6. Type I / II feedback on every bank (K9, K10), one thread per automaton word
-        for (int at = tid; at < n_own * per_clause; at += FITD_BLOCK) {
-            const int cl = at / per_clause, w = at - cl * per_clause;
-            const int32_t *u_of = upd + cl * K;
-            bool any = false;
-            for (int k = 0; k < K; ++k) any |= u_of[k] != 0;
-            if (!any) continue;
-            const int node = node_of[cl];
-            const bool fired = node != -1;
-            const bool within = incl_of[cl] <= p.max_included;
-            const int bank = w < LA ? 0 : 1 + (w - LA) / MC;
-            const int wl = w < LA ? w : (w - LA) % MC;
-            uint32_t x = 0u;
-            if (fired) x = bank != 0 ? mlit[((size_t)cl * L + (bank - 1)) * MC + wl] : at == tid ? x_first : p.X[(base + node) * LA + wl];
-            feedback_word<MAXB>(ta + (size_t)at * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1, (uint32_t)(c0 + cl),
-                                (uint32_t)wl, step, (uint32_t)bank, p.thr16[bank]);
+        if constexpr (!BIG) {
+            for (int at = tid; at < n_own * per_clause; at += FITD_BLOCK) {
+                const int cl = at / per_clause, w = at - cl * per_clause;
+                const int32_t *u_of = upd + cl * K;
+                bool any = false;
+                for (int k = 0; k < K; ++k) any |= u_of[k] != 0;
+                if (!any) continue;
+                const int node = node_of[cl];
+                const bool fired = node != -1;
+                const bool within = incl_of[cl] <= p.max_included;
+                const int bank = w < LA ? 0 : 1 + (w - LA) / MC;
+                const int wl = w < LA ? w : (w - LA) % MC;
+                uint32_t x = 0u;
+                if (fired) x = bank != 0 ? mlit[((size_t)cl * L + (bank - 1)) * MC + wl] : at == tid ? x_first : p.X[(base + node) * LA + wl];
+                feedback_word<MAXB>(ta + (size_t)at * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1, (uint32_t)(c0 + cl),
+                                    (uint32_t)wl, step, (uint32_t)bank, p.thr16[bank]);
+            }
+        } else {
+            // eight words at a time: their literal words are fetched first (from X, or node-major from `vec`), so that
+            // the fetches travel together
+            for (int at0 = tid; at0 < n_own * per_clause; at0 += 8 * FITD_BLOCK) {
+                uint32_t x[8];
+                bool busy[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int at = at0 + u * FITD_BLOCK;
+                    x[u] = 0u, busy[u] = false;
+                    if (at >= n_own * per_clause) continue;
+                    const int cl = at / per_clause, w = at - cl * per_clause;
+                    const int32_t *u_of = upd + cl * K;
+                    for (int k = 0; k < K; ++k) busy[u] |= u_of[k] != 0;
+                    const int node = node_of[cl];
+                    if (!busy[u] || node < 0) continue;
+                    if (w < LA) {
+                        x[u] = p.X[(base + node) * LA + w];
+                    } else {
+                        const int bank = 1 + (w - LA) / MC, wl = (w - LA) % MC;
+                        const uint32_t word = fitd_load(&p.vec[((size_t)(bank - 1) * p.max_nodes + node) * MW + (wl < MW ? wl : wl - MW)]);
+                        x[u] = wl < MW ? word : ~word;
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (!busy[u]) continue;
+                    const int at = at0 + u * FITD_BLOCK;
+                    const int cl = at / per_clause, w = at - cl * per_clause;
+                    const int bank = w < LA ? 0 : 1 + (w - LA) / MC;
+                    const int wl = w < LA ? w : (w - LA) % MC;
+                    // (the include plane's copy in LDS follows)
+                    ta[at] = feedback_word<MAXB>(word_in_memory(cl, w), B, K, upd + cl * K, 1, node_of[cl] != -1,
+                                                 incl_of[cl] <= p.max_included, p.boost, x[u], p.k0, p.k1, (uint32_t)(c0 + cl),
+                                                 (uint32_t)wl, step, (uint32_t)bank, p.thr16[bank]);
+                }
+            }
         }
+        if (tid == 0) next_unit[0] = 0;
         lds_barrier();
         FITD_TICK(12)
     }
@@ -581,13 +742,12 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
 #endif
     lds_barrier();
     // own state -> global memory (also after an abort: the host puts the model back as it was)
-    for (int i = tid; i < n_own * per_clause * B; i += FITD_BLOCK) {
-        const int cl = i / (per_clause * B), r = i - cl * per_clause * B;
-        const int w = r / B, b = r - w * B;
-        const int bank = w < LA ? 0 : 1 + (w - LA) / MC;
-        const int wl = w < LA ? w : (w - LA) % MC, chunks = bank == 0 ? LA : MC;
-        p.bank[bank][((int64_t)(c0 + cl) * chunks + wl) * B + b] = ta[i];
-    }
+    if constexpr (!BIG)
+        for (int i = tid; i < n_own * per_clause * B; i += FITD_BLOCK) {
+            const int cl = i / (per_clause * B), r = i - cl * per_clause * B;
+            const int w = r / B, b = r - w * B;
+            word_in_memory(cl, w)[b] = ta[i];
+        }
     for (int i = tid; i < n_own * K; i += FITD_BLOCK) {
         const int cl = i / K, k = i - cl * K;
         p.weights[(int64_t)k * p.C + c0 + cl] = wts[i];

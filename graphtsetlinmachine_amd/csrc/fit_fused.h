@@ -111,6 +111,151 @@ __device__ __forceinline__ void fit_clause_tail(uint32_t v, int lane, int words,
     }
 }
 
+// Truth of one clause over the nodes of a graph from literal-major rows: lane L of the wave gets the
+// nodes of word L (`active` lanes hold a word of the graph; col = the lane's column of the rows, rows
+// `stride` words apart).  inc = word 0 of the clause's include plane (words inc_stride apart).  A
+// clause with more than `walk_all` literals ANDs the rows of its first FIT_FILTER_ROWS literals in
+// `order` (the ones that hold least often in the data set) and then tests the few nodes that are
+// left against its whole include mask on the nodes' own literal words (X_rows: the graph's
+// node-major literal words, its first node's row).  Returns the lane's word of node bits (already
+// shifted and masked for graphs that share a word); *included_out = the clause's literal count.
+__device__ __forceinline__ uint32_t fit_clause_truth(const uint32_t *inc, int inc_stride, int LA, uint32_t filter,
+                                                     const uint32_t *col, int stride, int literals, int type_row, int ones_row,
+                                                     const FitGraph &fg, int n_nodes, int walk_all,
+                                                     const uint32_t *__restrict__ X_rows, const uint32_t *__restrict__ order,
+                                                     bool active, int lane, int *included_out) {
+    // lane w fetches include word w0 + w: one memory latency for up to 64 words
+    auto include_words = [&](int w0) {
+        uint32_t mine = w0 + lane < LA ? inc[(int64_t)(w0 + lane) * inc_stride] : 0u;
+        if (w0 + lane == LA - 1) mine &= filter;
+        return mine;
+    };
+    int included = 0;
+    uint32_t first_words = 0;
+    for (int w0 = 0; w0 < LA; w0 += 64) {
+        const uint32_t mine = include_words(w0);
+        if (w0 == 0) first_words = mine;
+        included += wave_sum_small(__popc(mine));
+    }
+    // A clause with many literals ANDs the rows of its first FIT_FILTER_ROWS only and then tests the
+    // few nodes that are left against its whole include mask on the nodes' own literal words.
+    const bool filter_only = included > walk_all && n_nodes > 0;
+    uint32_t acc = active ? col[(int64_t)type_row * stride] : 0u;
+    bool all_rows = false;  // every included literal's row has been applied: acc is the clause's truth
+    if (filter_only && order) {
+        // the first FIT_FILTER_ROWS included literals in `order` (the ones that hold least often in the
+        // data set), 16 row reads in flight; while more than a few nodes survive, 16 more: one round
+        // trip of row reads removes most of them, testing them costs a round trip per word of nodes.
+        // A clause that still holds at many nodes after 32 rows is not one that a few rows decide:
+        // it takes all its rows, and stops early only when no node is left.
+        int budget = FIT_FILTER_ROWS, applied = 0;
+        int r0 = 0;
+        unsigned long long picked = 0ull;  // lanes whose literal (in `order`) is included and not applied yet
+        uint32_t lit = 0u;
+        for (;;) {
+            if (budget <= 0) {
+                const int mine = active ? __popc((acc >> fg.shift) & fg.mask) : 0;
+                const int left = __popcll(__ballot(mine > 0)) + __popcll(__ballot(mine > 1));
+                if (left <= FIT_FEW_NODES) break;
+                budget = applied >= 32 ? 0x7FFFFFFF : 16;
+            }
+            if (picked == 0ull) {
+                if (r0 >= literals) {
+                    all_rows = true;
+                    break;
+                }
+                const int r = r0 + lane;
+                lit = r < literals ? order[r] : 0u;
+                uint32_t word = inc[(int64_t)(lit >> 5) * inc_stride];
+                if ((int)(lit >> 5) == LA - 1) word &= filter;
+                picked = __ballot(r < literals && ((word >> (lit & 31u)) & 1u));
+                r0 += 64;
+                continue;
+            }
+            int row[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                row[u] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
+                picked &= picked - 1;
+            }
+            uint32_t r16[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) r16[u] = col[(int64_t)row[u] * stride];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) acc &= r16[u];
+            budget -= 16, applied += 16;
+            if (applied > 32 && __ballot(acc != 0u) == 0ull) {  // (all the rows are wanted, but no node is left)
+                all_rows = true;
+                break;
+            }
+        }
+    } else {
+        int budget = filter_only ? FIT_FILTER_ROWS : 0x7FFFFFFF;
+        for (int w0 = 0; w0 < LA && budget > 0; w0 += 64) {
+            const uint32_t mine = w0 == 0 ? first_words : include_words(w0);
+            unsigned long long nonzero = __ballot(mine != 0);
+            while (nonzero && budget > 0) {
+                const int wl = __ffsll((long long)nonzero) - 1;
+                nonzero &= nonzero - 1;
+                uint32_t m = __builtin_amdgcn_readlane(mine, wl);
+                const int base = (w0 + wl) << 5;
+                while (m && budget > 0) {
+                    int row[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        row[u] = m ? base + __builtin_ctz(m) : ones_row;
+                        m &= m - 1;
+                    }
+                    uint32_t r[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) r[u] = col[(int64_t)row[u] * stride];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc &= r[u];
+                    budget -= 8;
+                }
+            }
+        }
+    }
+    uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
+    if (filter_only && !all_rows) {
+        // Lane L holds nodes 32 L .. 32 L + 31.  The surviving nodes are walked on the scalar unit, 8 at
+        // a time; for each, lane w compares include word w with the node's literal word w (one
+        // coalesced load per node and 64 words), and a node with any violated word is cleared.
+        unsigned long long live = __ballot(v != 0);
+        while (live) {
+            const int L = __ffsll((long long)live) - 1;
+            live &= live - 1;
+            uint32_t word = __builtin_amdgcn_readlane(v, L);
+            uint32_t cleared = 0;
+            while (word) {
+                int bit[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    bit[u] = word ? __builtin_ctz(word) : -1;
+                    word &= word - 1;
+                }
+                uint32_t violated[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                for (int w0 = 0; w0 < LA; w0 += 64) {
+                    const uint32_t mine = w0 == 0 ? first_words : include_words(w0);
+                    const bool in_row = w0 + lane < LA;
+                    uint32_t xs[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        xs[u] = in_row ? X_rows[(int64_t)(L * 32 + (bit[u] < 0 ? 0 : bit[u])) * LA + w0 + lane] : 0xFFFFFFFFu;
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) violated[u] |= mine & ~xs[u];
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (bit[u] >= 0 && __ballot(violated[u] != 0) != 0) cleared |= 1u << bit[u];
+            }
+            if (lane == L) v &= ~cleared;
+        }
+    }
+    *included_out = included;
+    return v;
+}
+
 // K1 + K6 + K7 for one graph.  A block stages the graph's literal-major rows
 // (plus an all-ones row) in LDS; each wave then takes clauses in turn.  The
 // clause is wave-uniform: its include words come in by scalar loads straight
@@ -161,129 +306,10 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
     const uint32_t *col = rows + (active ? lane : 0);
     int partial = 0;  // lane k < K: this wave's contribution to class k
     for (int c = blockIdx.x * WAVES + wave; c < C; c += gridDim.x * WAVES) {
-        const uint32_t *inc = bank + (int64_t)c * LA * B + (B - 1);
-        // lane w fetches include word w0 + w: one memory latency for up to 64 words
-        auto include_words = [&](int w0) {
-            uint32_t mine = w0 + lane < LA ? inc[(int64_t)(w0 + lane) * B] : 0u;
-            if (w0 + lane == LA - 1) mine &= filter;
-            return mine;
-        };
-        int included = 0;
-        uint32_t first_words = 0;
-        for (int w0 = 0; w0 < LA; w0 += 64) {
-            const uint32_t mine = include_words(w0);
-            if (w0 == 0) first_words = mine;
-            included += wave_sum_small(__popc(mine));
-        }
-        // A clause with many literals ANDs the rows of its first FIT_FILTER_ROWS only and then tests the
-        // few nodes that are left against its whole include mask on the nodes' own literal words.
-        const bool filter_only = included > (STAGE ? FIT_WALK_ALL_LDS : FIT_WALK_ALL) && n_nodes > 0;
-        uint32_t acc = active ? col[(int64_t)(literals + c % n_types) * stride] : 0u;
-        bool all_rows = false;  // every included literal's row has been applied: acc is the clause's truth
-        if (filter_only && order) {
-            // the first FIT_FILTER_ROWS included literals in `order` (the ones that hold least often in the
-            // data set); while more than a few nodes survive, 8 more at a time: one round trip of row
-            // reads removes most of them, testing them costs a round trip per word of nodes
-            int budget = FIT_FILTER_ROWS;
-            int r0 = 0;
-            unsigned long long picked = 0ull;  // lanes whose literal (in `order`) is included and not applied yet
-            uint32_t lit = 0u;
-            for (;;) {
-                if (budget <= 0) {
-                    const int mine = active ? __popc((acc >> fg.shift) & fg.mask) : 0;
-                    const int left = __popcll(__ballot(mine > 0)) + __popcll(__ballot(mine > 1));
-                    if (left <= FIT_FEW_NODES) break;
-                    budget = 8;
-                }
-                if (picked == 0ull) {
-                    if (r0 >= literals) {
-                        all_rows = true;
-                        break;
-                    }
-                    const int r = r0 + lane;
-                    lit = r < literals ? order[r] : 0u;
-                    uint32_t word = inc[(int64_t)(lit >> 5) * B];
-                    if ((int)(lit >> 5) == LA - 1) word &= filter;
-                    picked = __ballot(r < literals && ((word >> (lit & 31u)) & 1u));
-                    r0 += 64;
-                    continue;
-                }
-                int row[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    row[u] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
-                    picked &= picked - 1;
-                }
-                uint32_t r8[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) r8[u] = col[(int64_t)row[u] * stride];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) acc &= r8[u];
-                budget -= 8;
-            }
-        } else {
-            int budget = filter_only ? FIT_FILTER_ROWS : 0x7FFFFFFF;
-            for (int w0 = 0; w0 < LA && budget > 0; w0 += 64) {
-                const uint32_t mine = w0 == 0 ? first_words : include_words(w0);
-                unsigned long long nonzero = __ballot(mine != 0);
-                while (nonzero && budget > 0) {
-                    const int wl = __ffsll((long long)nonzero) - 1;
-                    nonzero &= nonzero - 1;
-                    uint32_t m = __builtin_amdgcn_readlane(mine, wl);
-                    const int base = (w0 + wl) << 5;
-                    while (m && budget > 0) {
-                        int row[8];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) {
-                            row[u] = m ? base + __builtin_ctz(m) : ones_row;
-                            m &= m - 1;
-                        }
-                        uint32_t r[8];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) r[u] = col[(int64_t)row[u] * stride];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) acc &= r[u];
-                        budget -= 8;
-                    }
-                }
-            }
-        }
-        uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
-        if (filter_only && !all_rows) {
-            // Lane L holds nodes 32 L .. 32 L + 31.  The surviving nodes are walked on the scalar unit, 8 at
-            // a time; for each, lane w compares include word w with the node's literal word w (one
-            // coalesced load per node and 64 words), and a node with any violated word is cleared.
-            unsigned long long live = __ballot(v != 0);
-            while (live) {
-                const int L = __ffsll((long long)live) - 1;
-                live &= live - 1;
-                uint32_t word = __builtin_amdgcn_readlane(v, L);
-                uint32_t cleared = 0;
-                while (word) {
-                    int bit[8];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) {
-                        bit[u] = word ? __builtin_ctz(word) : -1;
-                        word &= word - 1;
-                    }
-                    uint32_t violated[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-                    for (int w0 = 0; w0 < LA; w0 += 64) {
-                        const uint32_t mine = w0 == 0 ? first_words : include_words(w0);
-                        const bool in_row = w0 + lane < LA;
-                        uint32_t xs[8];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u)
-                            xs[u] = in_row ? X_rows[(int64_t)(L * 32 + (bit[u] < 0 ? 0 : bit[u])) * LA + w0 + lane] : 0xFFFFFFFFu;
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) violated[u] |= mine & ~xs[u];
-                    }
-#pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                        if (bit[u] >= 0 && __ballot(violated[u] != 0) != 0) cleared |= 1u << bit[u];
-                }
-                if (lane == L) v &= ~cleared;
-            }
-        }
+        int included;
+        const uint32_t v = fit_clause_truth(bank + (int64_t)c * LA * B + (B - 1), B, LA, filter, col, stride, literals,
+                                            literals + c % n_types, ones_row, fg, n_nodes,
+                                            STAGE ? FIT_WALK_ALL_LDS : FIT_WALK_ALL, X_rows, order, active, lane, &included);
         if (lane == 0) n_incl[c] = included;
         fit_clause_tail(v, lane, fg.words, NC, n_nodes, c, C, K, weights, k0, k1, step, finish != 0,
                         bitmap + (int64_t)c * NC, clause_node, class_sum, &partial);

@@ -610,6 +610,7 @@ struct FitWs {
     uint32_t *bank_backup;                  // every bank as it was before a cooperative run: [C][LA][B], then [C][MC][B] per message bank
     int32_t *weights_backup;                // [K][C]
     uint32_t *coop_got;                     // [3][depth - 1][M][NC] rows exchanged by k_fit_deep_persistent (depth > 1)
+    uint32_t *coop_vec;                     // [depth - 1][max_nodes][M / 32] the same, node-major
     unsigned long long *coop_arrived;       // [depth - 1][FITD_PARTS * FITD_STRIDE]
     size_t coop_words;                      // words of coop_got
     size_t bytes;
@@ -643,6 +644,7 @@ FitWs carve_fit(const Dims &d, const gtm_config *cfg, char *base) {
     w.weights_backup = (int32_t *)take((size_t)d.K * d.C * 4);
     w.coop_words = cfg->depth > 1 ? (size_t)3 * (cfg->depth - 1) * d.M * d.NC : 0;
     w.coop_got = cfg->depth > 1 ? (uint32_t *)take(w.coop_words * 4) : nullptr;
+    w.coop_vec = cfg->depth > 1 ? (uint32_t *)take((size_t)(cfg->depth - 1) * cfg->max_nodes * d.MC * 2) : nullptr;
     w.coop_arrived = cfg->depth > 1 ? (unsigned long long *)take((size_t)(cfg->depth - 1) * FITD_PARTS * FITD_STRIDE * 8) : nullptr;
     w.bytes = off;
     return w;
@@ -1752,14 +1754,29 @@ int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *
         if (limits[2] != 0u || limits[1] >= (uint32_t)FITD_MAX_EDGE_TYPES || limits[0] > (1u << 20)) return GTM_OK;
     }
     const int edge_cap = (int)limits[0], edge_types = (int)limits[1] + 1;
-    const size_t lds = fit_deep_lds_words(cfg->depth, per_group, d.LA, d.MC, d.M, d.MB, d.B, d.K, NW, rows_words, cfg->max_nodes, edge_cap,
-                                          edge_types) * 4;
-    if (lds > 150 * 1024) return GTM_OK;
-    const int variant = d.B <= 8 ? 0 : d.B <= 16 ? 1 : 2;
-    const void *kernel = variant == 0   ? (const void *)k_fit_deep_persistent<8>
-                         : variant == 1 ? (const void *)k_fit_deep_persistent<16>
-                                        : (const void *)k_fit_deep_persistent<32>;
-    static thread_local size_t lds_set_of[3] = {48 * 1024, 48 * 1024, 48 * 1024};
+    // automata, layer-0 rows and all received rows in LDS where they fit; else automata in memory, rows in
+    // place and as wide a window of received rows as fits
+    const size_t lds_cap = 158 * 1024;  // of 160 KiB; the kernel has a few words of its own
+    bool big = getenv("GTM_FIT_DEEP_IN_MEMORY") != nullptr;  // tuning aid: take the second layout anyway
+    int window_rows = d.M;
+    size_t lds = fit_deep_lds_words(false, cfg->depth, cfg->literals, per_group, d.LA, d.MC, d.MB, d.B, d.K, NW, rows_words, d.M, cfg->max_nodes,
+                                    edge_cap, edge_types) * 4;
+    if (lds > lds_cap) big = true;
+    if (big) {
+        if (const char *e = getenv("GTM_FIT_DEEP_WINDOW_ROWS")) window_rows = std::max(32, std::min(d.M, atoi(e) / 32 * 32));
+        for (;; window_rows = (window_rows / 2 + 31) / 32 * 32) {
+            lds = fit_deep_lds_words(true, cfg->depth, cfg->literals, per_group, d.LA, d.MC, d.MB, d.B, d.K, NW, 0, window_rows, cfg->max_nodes,
+                                     edge_cap, edge_types) * 4;
+            if (lds <= lds_cap || window_rows == 32) break;
+        }
+        if (lds > lds_cap) return GTM_OK;
+    }
+    const int variant = (d.B <= 8 ? 0 : d.B <= 16 ? 1 : 2) + (big ? 3 : 0);
+    const void *kernels[6] = {(const void *)k_fit_deep_persistent<8, false>,  (const void *)k_fit_deep_persistent<16, false>,
+                              (const void *)k_fit_deep_persistent<32, false>, (const void *)k_fit_deep_persistent<8, true>,
+                              (const void *)k_fit_deep_persistent<16, true>,  (const void *)k_fit_deep_persistent<32, true>};
+    const void *kernel = kernels[variant];
+    static thread_local size_t lds_set_of[6] = {48 * 1024, 48 * 1024, 48 * 1024, 48 * 1024, 48 * 1024, 48 * 1024};
     if (lds > lds_set_of[variant]) {
         if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
             (void)hipGetLastError();
@@ -1817,6 +1834,7 @@ int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *
     p.k1 = key.k1;
     p.q_thr = q_threshold(cfg->q, cfg->classes);
     p.got = w.coop_got;
+    p.vec = w.coop_vec;
     p.arrived = w.coop_arrived;
     p.class_sum = (unsigned long long *)w.class_sum;
     p.abort_flag = (uint32_t *)((unsigned long long *)w.class_sum + (size_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE);
@@ -1827,7 +1845,10 @@ int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *
     }
     p.clauses_per_group = per_group;
     p.NW = NW;
-    p.rows_words = rows_words;
+    p.rows_words = big ? 0 : rows_words;
+    p.window_rows = window_rows;
+    p.by_masks = (size_t)window_rows * NW >= (size_t)(1 + edge_types) * cfg->max_nodes && !getenv("GTM_FIT_DEEP_NO_MASKS");
+    p.order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
     p.max_nodes = cfg->max_nodes;
     p.edge_cap = edge_cap;
     p.edge_types = edge_types;
@@ -1855,7 +1876,7 @@ int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *
     p.clocks = (unsigned long long *)w.bank_backup;  // (development builds only: an aborted run is not restored correctly)
 #endif
     void *args[] = {&p};
-    profile_start("k_fit_deep_persistent", st);
+    profile_start(big ? "k_fit_deep_persistent<in memory>" : "k_fit_deep_persistent", st);
     e = hipLaunchCooperativeKernel(kernel, dim3(groups), dim3(FITD_BLOCK), args, (unsigned)lds, st);
     if (e != hipSuccess) return fail(GTM_ERR_HIP, "cooperative launch of the training kernel: %s", hipGetErrorString(e));
     profile_stop(st);

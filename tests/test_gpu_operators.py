@@ -418,17 +418,29 @@ ONE_LAUNCH_DEEP_SHAPES = [
 
 @pytest.mark.parametrize("shape", ONE_LAUNCH_DEEP_SHAPES, ids=lambda s: "deep%d" % s["seed"])
 @pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 9, 5), (1, None, 12)])
-def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bits, monkeypatch):
+@pytest.mark.parametrize("layout", ["in-lds", "in-lds-40-clauses-per-workgroup", "in-memory", "in-memory-32-row-windows",
+                                    "in-memory-40-clauses-per-workgroup"])
+def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bits, layout, monkeypatch):
     """A run of training examples of a model with message layers in one cooperative launch
     (k_fit_deep_persistent: clauses spread over workgroups, the nodes' messages and the class sums
     exchanged through device memory): automata of every bank and the weights after each of two
     epochs == the oracle; each epoch is split into two calls, so the state's round trip
-    through memory and the restart of the exchange buffers are covered."""
+    through memory and the restart of the exchange buffers are covered.  Both layouts: automata
+    and all rows in LDS; automata in memory with the received rows passing through LDS in windows
+    (as wide as fits, and 32 rows wide, so that every layer takes several).  With 40 clauses per
+    workgroup what the clauses send is worked out 32 clauses at a time, in two passes."""
     import ctypes
     from tests.gpu_harness import Device
     from graphtsetlinmachine_amd import _abi
 
     monkeypatch.setenv("GTM_NO_SMALL_FIT", "1")
+    if layout.startswith("in-memory"):
+        monkeypatch.setenv("GTM_FIT_DEEP_IN_MEMORY", "1")
+    if layout == "in-memory-32-row-windows":
+        monkeypatch.setenv("GTM_FIT_DEEP_WINDOW_ROWS", "32")
+    if layout.endswith("40-clauses-per-workgroup"):
+        monkeypatch.setenv("GTM_FIT_DEEP_CLAUSES_PER_GROUP", "40")
+    kernel = b"k_fit_deep_persistent<in memory>" if layout.startswith("in-memory") else b"k_fit_deep_persistent"
     graphs = helpers.random_graphs(shape["seed"], **shape["g"])
     m = dict(shape["m"])
     depth = m.pop("depth")
@@ -449,7 +461,7 @@ def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bi
         dev.fit(Y, G // 3, G - G // 3, epoch * G + G // 3)
         _abi.call("gtm_profile_read", ctypes.byref(name), ctypes.byref(launches), ctypes.byref(total))
         _abi.call("gtm_profile_enable", 0)
-        assert (name.value, launches.value) == (b"k_fit_deep_persistent", 2), "the one-launch kernel should have run"
+        assert (name.value, launches.value) == (kernel, 2), "the one-launch kernel should have run"
         ta, banks, w = dev.download()
         assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
         assert np.array_equal(ta, model.ta_state), "layer-0 automata after epoch %d" % epoch
@@ -458,7 +470,8 @@ def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bi
     assert np.array_equal(dev.score(0, G, G), o.score(model, graphs))
 
 
-def test_one_launch_fit_with_message_layers_gives_up_instead_of_hanging(monkeypatch):
+@pytest.mark.parametrize("layout", ["in-lds", "in-memory"])
+def test_one_launch_fit_with_message_layers_gives_up_instead_of_hanging(layout, monkeypatch):
     """As for the depth-1 kernel: GTM_FIT_SPIN_LIMIT=abort makes every workgroup give up at its first
     device-wide wait; the kernel drains, the call reports it, every bank and the weights are as
     they were, and the same model trains normally afterwards."""
@@ -466,6 +479,8 @@ def test_one_launch_fit_with_message_layers_gives_up_instead_of_hanging(monkeypa
     from graphtsetlinmachine_amd import _abi
 
     monkeypatch.setenv("GTM_NO_SMALL_FIT", "1")
+    if layout == "in-memory":
+        monkeypatch.setenv("GTM_FIT_DEEP_IN_MEMORY", "1")
     shape = ONE_LAUNCH_DEEP_SHAPES[1]
     graphs = helpers.random_graphs(shape["seed"], **shape["g"])
     m = dict(shape["m"])
