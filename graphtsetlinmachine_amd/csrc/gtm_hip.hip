@@ -498,6 +498,56 @@ __global__ void k_transform_nodewise(const uint32_t *__restrict__ bitmap, int C,
     out[i] = node < n ? (bitmap[gc * NC + (node >> 5)] >> (node & 31)) & 1u : 0;
 }
 
+// `transform` and `transform_nodewise` (kernels.py:666-710) from the truth rows that the tile kernels
+// leave behind ([tiles of the launch][C][tw]), and the class sums (kernels.py:297-315) from the same
+// rows: one workgroup per graph.  A graph without nodes gives zeros in both outputs (the reference
+// loops over the nodes) while its class sums count every clause, as `evaluate` does.
+constexpr int TILE_TRANSFORM_BLOCK = 256;
+__global__ __launch_bounds__(TILE_TRANSFORM_BLOCK) void k_tile_transform(
+    const uint32_t *__restrict__ bitmap, TileGeom tg, int tile0, int graph0, int first_graph, int C, int K,
+    const uint32_t *__restrict__ n_nodes_arr, const int32_t *__restrict__ weights, int32_t *__restrict__ transformed,
+    int32_t *__restrict__ nodewise, int width, int32_t *__restrict__ class_sum) {
+    extern __shared__ uint32_t fired[];  // one bit per clause, then a partial sum per wave
+    int32_t *partial = (int32_t *)(fired + (C + 31) / 32);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = graph0 + (int)blockIdx.x;
+    const int n = (int)n_nodes_arr[g];
+    const FitGraph f = fit_graph_slot(tg, g, n);
+    const uint32_t *rows = bitmap + (int64_t)(f.tile - tile0) * C * tg.tw + f.word0;
+    const int64_t out0 = (int64_t)(g - first_graph) * C;
+    for (int i = tid; i < (C + 31) / 32; i += TILE_TRANSFORM_BLOCK) fired[i] = 0u;
+    __syncthreads();
+    for (int c = tid; c < C; c += TILE_TRANSFORM_BLOCK) {
+        uint32_t any = 0u;
+        for (int w = 0; w < f.words; ++w) any |= (rows[(int64_t)c * tg.tw + w] >> f.shift) & f.mask;
+        if (any) atomicOr(&fired[c >> 5], 1u << (c & 31));
+        transformed[out0 + c] = n > 0 && any != 0u;
+    }
+    if (nodewise)
+        for (int64_t i = tid; i < (int64_t)C * width; i += TILE_TRANSFORM_BLOCK) {
+            const int c = (int)(i / width), node = (int)(i - (int64_t)c * width);
+            uint32_t bit = 0u;
+            if (node < n) bit = (((rows[(int64_t)c * tg.tw + (node >> 5)] >> f.shift) & f.mask) >> (node & 31)) & 1u;
+            nodewise[out0 * width + i] = (int32_t)bit;
+        }
+    __syncthreads();
+    for (int k = 0; k < K; ++k) {
+        int sum = 0;
+        for (int c = tid; c < C; c += TILE_TRANSFORM_BLOCK)
+            if ((fired[c >> 5] >> (c & 31)) & 1u) sum += weights[(int64_t)k * C + c];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+        if (lane == 0) partial[wave] = sum;
+        __syncthreads();
+        if (tid == 0) {
+            int total = 0;
+            for (int w = 0; w < TILE_TRANSFORM_BLOCK / 64; ++w) total += partial[w];
+            class_sum[(int64_t)(g - first_graph) * K + k] = total;
+        }
+        __syncthreads();
+    }
+}
+
 // ------------------------------------------------------------ launch helpers
 
 int launch_clause_node_bits(const Dims &d, const gtm_graphs *g, int first, int n_graphs, const uint32_t *inc_t,
@@ -555,7 +605,9 @@ int clause_list_stride(int literals) { return ((literals + 2 + 31) & ~31) + 32; 
 int tiles_per_batch(const TileGeom &tg, int batch) { return (batch + tg.gpt - 1) / tg.gpt; }
 
 // `tg`: the data set's tile geometry when the tile path will run (its buffers replace the dense ones).
-ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base, const TileGeom *tg = nullptr) {
+// `keep_rows` (gtm_transform): the truth rows of the last layer are wanted, also without message layers.
+ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base, const TileGeom *tg = nullptr,
+                    bool keep_rows = false) {
     ScoreWs w{};
     size_t off = 0;
     int chunks = cfg->depth > 1 && d.MC > d.LA ? d.MC : d.LA;
@@ -567,7 +619,12 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base,
     w.list_stride = clause_list_stride(cfg->literals);
     w.lists = (uint32_t *)take((size_t)d.C * w.list_stride * 4);
     w.wt = (int32_t *)take((size_t)d.C * d.K * 4);
+    if (tg && cfg->depth == 1 && !keep_rows) {
+        w.bytes = off;
+        return w;
+    }
     if (tg && cfg->depth == 1) {
+        w.tile_bitmap = (uint32_t *)take((size_t)tiles_per_batch(*tg, batch) * d.C * tg->tw * 4);
         w.bytes = off;
         return w;
     }
@@ -996,8 +1053,16 @@ bool two_phase_layer0(const Dims &d, const gtm_graphs *g, const TileGeom &tg) {
 
 // `_score`'s loop (tm.py:786-812) on tiles: per launch group of tiles, layer 0 and then one
 // launch per message layer; the clause truth rows between layers stay in w.tile_bitmap.
+// With `tr` (gtm_transform; tm.py:814-900) every layer leaves its truth rows, and k_tile_transform
+// makes the per-clause outputs and the class sums from the last layer's.
+struct TransformOut {
+    int32_t *transformed, *nodewise;
+    int width;
+};
+
 int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
-                   const ScoreWs &w, int first, int n_graphs, int batch, int32_t *class_sum, hipStream_t st) {
+                   const ScoreWs &w, int first, int n_graphs, int batch, int32_t *class_sum, hipStream_t st,
+                   const TransformOut *tr = nullptr) {
     const uint32_t *order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
     const int layers = cfg->depth;
     const bool narrow = two_phase_layer0(d, g, tg);
@@ -1049,7 +1114,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         if (wide) return launch_two_phase_wide(a, n_tiles, d.LA, tg.stage0 != 0, last, st);
         return launch_tile_layer(a, n_tiles, tg.stage0 ? ROWS_STAGED : ROWS_GLOBAL, last, st);
     };
-    if (layers == 1) {
+    if (layers == 1 && !tr) {
         // no truth rows are kept: every tile of the range in one launch
         a.tile0 = first / tg.gpt;
         a.first_graph = first;
@@ -1058,7 +1123,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         int n_tiles = (first + n_graphs - 1) / tg.gpt - a.tile0 + 1;
         return layer0(n_tiles, true);
     }
-    if (g->total_edges > 0 && (!g->number_of_graph_node_edges || !g->edge || !g->edge_index))
+    if (layers > 1 && g->total_edges > 0 && (!g->number_of_graph_node_edges || !g->edge || !g->edge_index))
         return fail(GTM_ERR_INVALID, "graphs with edges need number_of_graph_node_edges, edge and edge_index");
     const int tiles_per_launch = tiles_per_batch(tg, batch);
     const int tile_first = first / tg.gpt, tile_last = (first + n_graphs - 1) / tg.gpt;
@@ -1067,7 +1132,8 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     while (group > 1 && ((size_t)32 * group * (MW | 1) + group) * 4 > 64 * 1024) group >>= 1;
     a.message_rows = w.message_rows;
     const size_t fused_lds = tg.slot_words > 0 ? tile_fused_messages_lds_bytes(tg, MW) : 0;
-    bool fused_messages = tg.slot_words > 0 && d.M % 32 == 0 && fused_lds <= 150 * 1024 && !getenv("GTM_NO_FUSED_MESSAGES");
+    bool fused_messages = layers > 1 && tg.slot_words > 0 && d.M % 32 == 0 && fused_lds <= 150 * 1024 &&
+                          !getenv("GTM_NO_FUSED_MESSAGES");
     if (fused_messages) {
         static thread_local size_t fused_lds_set = 48 * 1024;
         if (fused_lds > fused_lds_set) {
@@ -1081,14 +1147,14 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         }
     }
     const bool by_bit = !getenv("GTM_NODE_MESSAGES_BY_ATOMICS");  // tuning aid: the earlier kernel
-    if (fused_messages || by_bit) {
+    if (layers > 1 && (fused_messages || by_bit)) {
         // the clauses of every message bit, for the kernels that build what the nodes send
         hipLaunchKernelGGL(k_message_bit_index, dim3(1), dim3(BIT_INDEX_BLOCK), 0, st, s->hypervectors, d.C, d.MB, d.M,
                            w.bit_start, w.bit_cursor, w.bit_clauses);
         if (int rc = check_launch("message_bit_index")) return rc;
     }
     static thread_local bool node_messages_lds_raised = false;
-    if (!node_messages_lds_raised) {
+    if (layers > 1 && !node_messages_lds_raised) {
         hipError_t e = hipFuncSetAttribute((const void *)k_tile_node_messages,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
         if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit: %s", hipGetErrorString(e));
@@ -1112,7 +1178,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                 if (int rc = check_launch("tile_messages_fused")) return rc;
                 a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
                 a.stride = w.message_list_stride;
-                if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1, st)) return rc;
+                if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1 && !tr, st)) return rc;
                 continue;
             }
             if (by_bit)
@@ -1141,10 +1207,36 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             if (int rc = check_launch("tile_pack_messages")) return rc;
             a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
             a.stride = w.message_list_stride;
-            if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1, st)) return rc;
+            if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1 && !tr, st)) return rc;
+        }
+        if (tr) {
+            const int g_lo = std::max(first, t0 * tg.gpt), g_hi = std::min(first + n_graphs, (t0 + n_tiles) * tg.gpt);
+            if (g_hi > g_lo) {
+                profile_start("k_tile_transform", st);
+                hipLaunchKernelGGL(k_tile_transform, dim3(g_hi - g_lo), dim3(TILE_TRANSFORM_BLOCK),
+                                   ((size_t)(d.C + 31) / 32 + TILE_TRANSFORM_BLOCK / 64) * 4, st, w.tile_bitmap, tg, t0, g_lo, first,
+                                   d.C, d.K, g->number_of_graph_nodes, s->clause_weights, tr->transformed, tr->nodewise, tr->width,
+                                   class_sum);
+                if (int rc = check_launch("tile_transform")) return rc;
+                profile_stop(st);
+            }
         }
     }
     return GTM_OK;
+}
+
+// The tile path of gtm_score / gtm_transform needs a data set with tiles of a usable geometry.
+// GTM_NO_TILE_TRANSFORM (tuning aid) keeps gtm_transform on the dense path.
+bool tiles_usable(const gtm_config *cfg, const gtm_graphs *graphs, int classes, TileGeom *tg) {
+    if (!graphs || !graphs->tiles || graphs->number_of_graphs < 1 || graphs->number_of_node_types < 1) return false;
+    *tg = geometry_for(cfg, graphs, classes);
+    // with message layers a 64-slot block of message vectors has to fit in 64 KB of LDS
+    if (cfg->depth > 1 && (size_t)64 * ((cfg->message_size + 31) / 32 + 1) * 4 > 64 * 1024) return false;
+    return tg->ok != 0;
+}
+
+bool transform_uses_tiles(const gtm_config *cfg, const gtm_graphs *graphs, int classes, TileGeom *tg) {
+    return !getenv("GTM_NO_TILE_TRANSFORM") && tiles_usable(cfg, graphs, classes, tg);
 }
 
 }  // namespace
@@ -1351,8 +1443,9 @@ int gtm_get_hyperliterals(const gtm_config *cfg, const uint32_t *bank, int32_t c
 size_t gtm_transform_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs, int32_t batch) {
     Dims d;
     if (validate(cfg, &d) || batch < 1) return 0;
-    (void)graphs;
-    return carve_score(d, cfg, batch, nullptr).bytes;
+    TileGeom tg;
+    const bool tiles = transform_uses_tiles(cfg, graphs, d.K, &tg);
+    return carve_score(d, cfg, batch, nullptr, tiles ? &tg : nullptr, true).bytes;
 }
 
 int gtm_transform(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, int32_t first_graph,
@@ -1366,10 +1459,19 @@ int gtm_transform(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_sta
     if (!transformed || !class_sum) return fail(GTM_ERR_INVALID, "NULL output");
     if (nodewise && (width < 1 || width > cfg->max_nodes))
         return fail(GTM_ERR_INVALID, "width=%d outside [1, max_nodes=%d]", width, cfg->max_nodes);
-    ScoreWs w = carve_score(d, cfg, batch, (char *)workspace);
+    TileGeom tg;
+    const bool tiles = transform_uses_tiles(cfg, graphs, d.K, &tg);
+    ScoreWs w = carve_score(d, cfg, batch, (char *)workspace, tiles ? &tg : nullptr, true);
     if (!workspace || workspace_bytes < w.bytes)
         return fail(GTM_ERR_INVALID, "workspace of %zu bytes needed, %zu given", w.bytes, workspace_bytes);
     hipStream_t st = (hipStream_t)stream;
+    if (n_graphs == 0) return GTM_OK;
+    if (tiles) {
+        // the truth rows that the tile kernels of gtm_score compute, kept for the last layer too
+        if (int rc = check_tiles(tg, cfg, graphs)) return rc;
+        const TransformOut out{transformed, nodewise, width};
+        return score_on_tiles(d, cfg, graphs, state, tg, w, first_graph, n_graphs, batch, class_sum, st, &out);
+    }
     for (int done = 0; done < n_graphs; done += batch) {
         int nb = n_graphs - done < batch ? n_graphs - done : batch;
         uint32_t *final_bitmap = nullptr;
@@ -1484,11 +1586,7 @@ int gtm_build_tiles(const gtm_config *cfg, const gtm_graphs *graphs, uint32_t *t
 
 // The tile path runs when the data set carries tiles (gtm_build_tiles) of a supported shape.
 static bool score_uses_tiles(const gtm_config *cfg, const gtm_graphs *graphs, int classes, TileGeom *tg) {
-    if (!graphs || !graphs->tiles || graphs->number_of_graphs < 1 || graphs->number_of_node_types < 1) return false;
-    *tg = geometry_for(cfg, graphs, classes);
-    // with message layers a 64-slot block of message vectors has to fit in 64 KB of LDS
-    if (cfg->depth > 1 && (size_t)64 * ((cfg->message_size + 31) / 32 + 1) * 4 > 64 * 1024) return false;
-    return tg->ok != 0;
+    return tiles_usable(cfg, graphs, classes, tg);
 }
 
 size_t gtm_score_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs, int32_t batch) {

@@ -415,6 +415,7 @@ class CommonTsetlinMachine:
         dg = self._score_init(graphs)
         cfg = self._config(max(dg.max_nodes, 1))
         n, C = dg.number_of_graphs, self.number_of_clauses
+        dg.ensure_tiles(cfg)
         width = max(int(np.max(graphs.number_of_graph_nodes)), 1) if nodewise else 0
         if batch is None:
             size = lambda b: _abi.lib.gtm_transform_workspace_bytes(ctypes.byref(cfg), ctypes.byref(dg.desc), b)

@@ -204,6 +204,58 @@ def test_transform_and_read_outs_match_the_oracle():
                 assert messages[edge_type, c, 40 + sender] == sum(int(included[c, 40 + b]) for b in bits)
 
 
+@pytest.mark.parametrize("case", [
+    # 361-node graphs, one layer (tiles of positive rows only); tiny graphs that share words of a tile row;
+    # two and three layers with edge types and graphs without nodes
+    dict(g=dict(n_graphs=23, max_nodes=361, min_nodes=300, hv_size=128), m=dict(depth=1), clauses=70, classes=10),
+    dict(g=dict(n_graphs=90, max_nodes=3, hv_size=16, node_types=("a", "b")), m=dict(depth=1), clauses=33, classes=2),
+    dict(g=dict(n_graphs=30, hv_size=24, node_types=("a", "b"), edge_types=("l", "r"), sizes=[5, 0, 33, 1, 40, 64] * 5),
+         m=dict(depth=2, message_size=64, message_bits=2), clauses=40, classes=3),
+    dict(g=dict(n_graphs=20, max_nodes=20, min_nodes=4, hv_size=20, edge_types=("x", "y", "z")),
+         m=dict(depth=3, message_size=37, message_bits=3), clauses=50, classes=4),
+], ids=["361-nodes", "tiny-graphs", "two-layers", "three-layers"])
+def test_transform_on_tiles(case, monkeypatch):
+    """gtm_transform from the truth rows of the tile kernels (k_tile_transform) == the dense path ==
+    the oracle: per-clause outputs, per-node outputs and class sums, in one launch group and in groups
+    of 7 graphs (which start and end inside tiles)."""
+    import ctypes
+    from graphtsetlinmachine_amd import _abi
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    graphs = helpers.random_graphs(77, **case["g"])
+    n = graphs.number_of_graphs
+    depth = case["m"]["depth"]
+    rng = np.random.default_rng(3)
+    Y = rng.integers(0, case["classes"], size=n)
+    np.random.seed(5)
+    tm = MultiClassGraphTsetlinMachine(case["clauses"], 30, (2.0, 1.5, 1.2)[:depth] if depth > 1 else 2.0, seed=13, **case["m"])
+    tm.fit(graphs, Y, epochs=2, incremental=True)
+    model = oracle_twin(tm, graphs)  # an untrained oracle model of the same shape, given the trained state
+    state = tm.save()
+    model.ta_state = state["ta_state"].reshape(model.ta_state.shape).copy()
+    model.clause_weights = state["clause_weights"].reshape(model.clause_weights.shape).copy()
+    model.message_ta_state = [bank.reshape(init.shape).copy() for bank, init in zip(state["message_ta_state"], model.message_ta_state)]
+    want, want_sums = o.transform(model, graphs)
+    want_wide, _ = o.transform(model, graphs, nodewise=True)
+    assert want.any() and not want.all()
+
+    name, launches, total = ctypes.c_char_p(), ctypes.c_int32(), ctypes.c_double()
+    _abi.call("gtm_profile_enable", 1)
+    got, sums = tm._transform(graphs, False)
+    _abi.call("gtm_profile_read", ctypes.byref(name), ctypes.byref(launches), ctypes.byref(total))
+    _abi.call("gtm_profile_enable", 0)
+    assert name.value == b"k_tile_transform", "the tile path should have run"
+    assert np.array_equal(got, want) and np.array_equal(sums, want_sums)
+    assert np.array_equal(sums, tm.score_device(graphs).cpu().numpy().reshape(n, -1))
+    wide, sums = tm._transform(graphs, True, batch=7)
+    assert np.array_equal(wide, want_wide) and np.array_equal(sums, want_sums)
+    got, sums = tm._transform(graphs, False, batch=7)
+    assert np.array_equal(got, want) and np.array_equal(sums, want_sums)
+    monkeypatch.setenv("GTM_NO_TILE_TRANSFORM", "1")
+    dense, dense_sums = tm._transform(graphs, False)
+    assert np.array_equal(dense, want) and np.array_equal(dense_sums, want_sums)
+
+
 def test_multi_output_and_single_output_heads_follow_the_oracle():
     """tm.py:961-1072: several independent outputs (Y in {0, 1} per output, prediction sum >= 0) and
     the single-output machine (one 'class', score is a vector): states, sums and predictions."""
