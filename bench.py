@@ -250,6 +250,28 @@ def read_kernel_profile():
     return name.value.decode(), launches.value, total.value
 
 
+def read_kernel_breakdown():
+    """[(kernel name, launches, total ms)] for every kernel bracketed since profiling was enabled
+    (read before read_kernel_profile(), which clears the record)."""
+    from graphtsetlinmachine_amd import _abi
+
+    out = []
+    for index in range(64):
+        name, launches, total = ctypes.c_char_p(), ctypes.c_int32(), ctypes.c_double()
+        _abi.call("gtm_profile_read_kernel", index, ctypes.byref(name), ctypes.byref(launches), ctypes.byref(total))
+        if not name.value:
+            break
+        out.append((name.value.decode(), launches.value, total.value))
+    return out
+
+
+def message_layer_bytes_per_graph(n_nodes, message_chunks, clauses, node_chunks, edges):
+    """Algorithmic bytes of one message layer of one graph: the nodes' message literal words and the
+    include plane of the layer's bank in, the edges walked once, the previous layer's clause x node
+    bitmap in and the new one out."""
+    return n_nodes * message_chunks * 4 + clauses * message_chunks * 4 + 2 * clauses * node_chunks * 4 + edges * 8
+
+
 def mean_included_literals(tm):
     import numpy as np
 
@@ -276,9 +298,14 @@ def time_scoring(tm, test, steps, warmup, graphs):
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    breakdown = read_kernel_breakdown()
     kernel_name, launches, kernel_total_ms = read_kernel_profile()
     _abi.call("gtm_profile_enable", 0)
+    if len(breakdown) > 1:  # several kernels share the work: the roofline kernel is the one that takes longest
+        kernel_name, launches, kernel_total_ms = max(breakdown, key=lambda k: k[2])
     return {
+        "kernels": [{"kernel": k, "launches_per_step": round(n / steps, 2), "ms_per_step": round(ms / steps, 4)}
+                    for k, n, ms in breakdown],
         "wall": wall, "event_ms": start.elapsed_time(stop) / steps, "kernel": kernel_name, "launches": launches,
         "kernel_ms": kernel_total_ms / max(launches, 1), "graphs_per_launch": graphs * steps / max(launches, 1),
         "sums": sums.cpu().numpy().reshape(graphs, -1),
@@ -394,6 +421,30 @@ def main():
     accuracy = float((sums_host.argmax(axis=1) == wl.Y_test).mean())
     included_main = mean_included_literals(tm)
 
+    # models with message layers: the step's kernels in two groups - layer 0 and the message layers (building
+    # the messages and evaluating the clauses on them) - each with its algorithmic bytes per graph; the
+    # roofline below is then that of the group that takes longer
+    layer_groups, step_bytes = None, b_eval
+    if tm.depth > 1:
+        edges_per_graph = int(test.edge.shape[0]) // max(int(test.number_of_graphs), 1)
+        b_msg = message_layer_bytes_per_graph(n_nodes, tm.number_of_message_chunks, tm.number_of_clauses,
+                                              (n_nodes - 1) // 32 + 1, edges_per_graph)
+        layer_groups = []
+        for label, wanted, group_bytes in (("layer 0", lambda k: "messages" not in k, b_eval),
+                                          ("message layers (%d)" % (tm.depth - 1), lambda k: "messages" in k,
+                                           b_msg * (tm.depth - 1))):
+            members = [k for k in main_run["kernels"] if wanted(k["kernel"])]
+            ms = sum(k["ms_per_step"] for k in members)
+            gbs = group_bytes * args.graphs / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+            layer_groups.append({"layers": label, "kernels": [k["kernel"] for k in members], "ms_per_step": round(ms, 4),
+                                 "algorithmic_bytes_per_graph": group_bytes, "achieved_GBs": round(gbs, 1),
+                                 "frac": round(gbs / HBM_PEAK_GBS, 4)})
+        step_bytes = sum(e["algorithmic_bytes_per_graph"] for e in layer_groups)
+        slowest = max(layer_groups, key=lambda e: e["ms_per_step"])
+        if slowest["ms_per_step"] > 0:
+            b_eval, kernel_name = slowest["algorithmic_bytes_per_graph"], " + ".join(slowest["kernels"])
+            kernel_ms, graphs_per_launch = slowest["ms_per_step"], float(args.graphs)
+
     # roofline of the clause-evaluation kernel: algorithmic bytes / kernel time
     achieved = b_eval * graphs_per_launch / (kernel_ms * 1e-3) / 1e9
     compulsory = (n_nodes * la * 4 + n_nodes * 4 + tm.number_of_outputs * 4) * graphs_per_launch
@@ -408,8 +459,9 @@ def main():
         "kernel": kernel_name, "kernel_ms": round(kernel_ms, 4), "launches": launches,
         "graphs_per_launch": graphs_per_launch,
         "algorithmic_bytes_per_graph": b_eval,
+        "kernels": main_run["kernels"], "layer_groups": layer_groups,
         # the same bytes over the whole timed step (kernel + clause compilation + launch gaps)
-        "frac_whole_step": round(b_eval * args.graphs / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "frac_whole_step": round(step_bytes * args.graphs / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         # what the memory system really moved (rocprofv3 FETCH_SIZE + WRITE_SIZE) over this run's kernel time,
         # and the share of cycles in which the vector ALUs issued (both from the counter runs named above)
         "hbm_measured_GBs": round(traffic / (kernel_ms * 1e-3) / 1e9, 1) if traffic else None,

@@ -95,6 +95,7 @@ PROTOTYPES = {
     "gtm_transform": (C.c_int, [_CFG, _GR, _ST, _I, _I, _I, _P, _SZ, _P, _P, _I, _P, _P]),
     "gtm_profile_enable": (C.c_int, [C.c_int]),
     "gtm_profile_read": (C.c_int, [C.POINTER(C.c_char_p), C.POINTER(C.c_int32), C.POINTER(C.c_double)]),
+    "gtm_profile_read_kernel": (C.c_int, [C.c_int32, C.POINTER(C.c_char_p), C.POINTER(C.c_int32), C.POINTER(C.c_double)]),
     "gtm_graphs_properties": (C.c_int, [_CFG, _GR, _P, _P]),
     "gtm_tiles_bytes": (_SZ, [_CFG, _GR]),
     "gtm_build_tiles": (C.c_int, [_CFG, _GR, _P, _P]),

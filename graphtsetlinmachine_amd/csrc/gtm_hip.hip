@@ -48,14 +48,15 @@ int check_launch(const char *what) {
 }
 
 // --------------------------------------------------------------- profiling
-// When enabled (gtm_profile_enable), the launch of the dominant kernel of a
-// driver loop is bracketed by HIP events on the caller's stream.
+// When enabled (gtm_profile_enable), the launches of the kernels that do the work of a
+// driver loop are bracketed by HIP events on the caller's stream, each under its kernel's name.
 
 struct Profile {
     bool on = false;
     const char *name = "";
-    static constexpr int MAX = 512;
+    static constexpr int MAX = 4096;
     hipEvent_t start[MAX], stop[MAX];
+    const char *name_of[MAX];
     int created = 0, used = 0;
 };
 Profile g_prof;
@@ -71,6 +72,7 @@ void profile_start(const char *name, hipStream_t st) {
         ++g_prof.created;
     }
     g_prof.name = name;
+    g_prof.name_of[g_prof.used] = name;
     (void)hipEventRecord(g_prof.start[g_prof.used], st);
 }
 
@@ -887,9 +889,8 @@ int launch_tile_layer_as(const TileLayerArgs &a, int n_tiles, const char *profil
 template <int NW, int LW>
 int launch_tile_layer_lw(const TileLayerArgs &a, int n_tiles, int src, bool last, hipStream_t st) {
     if (src == ROWS_MESSAGES)
-        return last ? launch_tile_layer_as<NW, LW, ROWS_MESSAGES, true>(a, n_tiles, nullptr, st)
-                    : launch_tile_layer_as<NW, LW, ROWS_MESSAGES, false>(a, n_tiles, nullptr, st);
-    // the layer-0 kernel is the one the library times (gtm_profile_*)
+        return last ? launch_tile_layer_as<NW, LW, ROWS_MESSAGES, true>(a, n_tiles, "k_tile_layer<messages, score>", st)
+                    : launch_tile_layer_as<NW, LW, ROWS_MESSAGES, false>(a, n_tiles, "k_tile_layer<messages>", st);
     if (src == ROWS_GLOBAL)
         return last ? launch_tile_layer_as<NW, LW, ROWS_GLOBAL, true>(a, n_tiles, "k_tile_layer<score>", st)
                     : launch_tile_layer_as<NW, LW, ROWS_GLOBAL, false>(a, n_tiles, "k_tile_layer<layer0>", st);
@@ -1171,16 +1172,19 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             // the layer's message rows for these tiles (score_tiles.h): one graph per workgroup with its
             // vectors in LDS when they fit, else three launches with the vectors in global memory
             if (fused_messages) {
+                profile_start("k_tile_messages_fused", st);
                 hipLaunchKernelGGL(k_tile_messages_fused, dim3(tg.gpt, n_tiles), dim3(TILE_FUSED_MESSAGES_BLOCK),
                                    fused_lds, st, w.tile_bitmap, d.C, tg, t0, g->number_of_graphs, d.M, MW, w.bit_start,
                                    w.bit_clauses, g->node_index, g->number_of_graph_nodes, g->number_of_graph_node_edges,
                                    g->edge_index, g->edge, g->total_edges > 0 ? 1 : 0, w.message_rows);
                 if (int rc = check_launch("tile_messages_fused")) return rc;
+                profile_stop(st);
                 a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
                 a.stride = w.message_list_stride;
                 if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1 && !tr, st)) return rc;
                 continue;
             }
+            profile_start("k_tile_node_messages + k_tile_edge_messages + k_tile_pack_messages", st);
             if (by_bit)
                 hipLaunchKernelGGL(k_tile_node_messages_by_bit,
                                    dim3((MW + NODE_MESSAGES_BY_BIT_WAVES - 1) / NODE_MESSAGES_BY_BIT_WAVES, n_tiles),
@@ -1205,6 +1209,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                                (size_t)64 * (MW + 1) * 4, st, w.got, tg, t0, g->number_of_graphs, d.M, MW,
                                g->number_of_graph_nodes, w.message_rows);
             if (int rc = check_launch("tile_pack_messages")) return rc;
+            profile_stop(st);
             a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
             a.stride = w.message_list_stride;
             if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1 && !tr, st)) return rc;
@@ -1522,6 +1527,33 @@ int gtm_profile_read(const char **kernel_name, int32_t *launches, double *total_
     *launches = g_prof.used;
     *total_ms = total;
     g_prof.used = 0;
+    return GTM_OK;
+}
+
+int gtm_profile_read_kernel(int32_t index, const char **kernel_name, int32_t *launches, double *total_ms) {
+    if (!kernel_name || !launches || !total_ms || index < 0) return fail(GTM_ERR_INVALID, "NULL output or negative index");
+    *kernel_name = nullptr, *launches = 0, *total_ms = 0.0;
+    // the index-th distinct name in the order of first use (names are string literals of this file)
+    const char *wanted = nullptr;
+    int seen = 0;
+    for (int i = 0; i < g_prof.used && !wanted; ++i) {
+        bool earlier = false;
+        for (int j = 0; j < i && !earlier; ++j) earlier = strcmp(g_prof.name_of[j], g_prof.name_of[i]) == 0;
+        if (!earlier && seen++ == index) wanted = g_prof.name_of[i];
+    }
+    if (!wanted) return GTM_OK;
+    double total = 0.0;
+    int count = 0;
+    for (int i = 0; i < g_prof.used; ++i) {
+        if (strcmp(g_prof.name_of[i], wanted) != 0) continue;
+        hipError_t e = hipEventSynchronize(g_prof.stop[i]);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, g_prof.start[i], g_prof.stop[i]);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "reading profile events: %s", hipGetErrorString(e));
+        total += ms;
+        ++count;
+    }
+    *kernel_name = wanted, *launches = count, *total_ms = total;
     return GTM_OK;
 }
 

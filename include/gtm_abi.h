@@ -248,14 +248,20 @@ int gtm_transform(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_sta
                   int32_t n_graphs, int32_t batch, void *workspace, size_t workspace_bytes, int32_t *transformed,
                   int32_t *nodewise, int32_t width, int32_t *class_sum, void *stream);
 
-/* No counterpart in the reference.  While enabled, gtm_score / gtm_fit bracket
- * each launch of their clause-evaluation kernel (the dominant kernel) with HIP
- * events on the caller's stream (at most 512 launches are kept).
- * gtm_profile_read() waits for those events, returns the kernel's name, the
- * number of launches seen and their summed duration, and clears the record.
- * Not thread-safe; meant for the benchmark. */
+/* No counterpart in the reference.  While enabled, gtm_score / gtm_transform /
+ * gtm_fit bracket the launches of the kernels that do their work (clause
+ * evaluation per layer, message construction, the one-launch training kernels)
+ * with HIP events on the caller's stream, each under its kernel's name (at most
+ * 4096 launches are kept).  gtm_profile_read() waits for those events, returns
+ * the name of the kernel launched last, the number of launches seen and their
+ * summed duration (all kernels together: a model without message layers has one),
+ * and clears the record.  Not thread-safe; meant for the benchmark. */
 int gtm_profile_enable(int on);
 int gtm_profile_read(const char **kernel_name, int32_t *launches, double *total_ms);
+/* The same measurement kernel by kernel, without ending it: the index-th distinct kernel name in
+ * the order of first launch, the number of its launches and their total duration.  An index past
+ * the last name gives *kernel_name = NULL and zeros.  (No counterpart in the reference.) */
+int gtm_profile_read_kernel(int32_t index, const char **kernel_name, int32_t *launches, double *total_ms);
 
 #ifdef __cplusplus
 }
