@@ -1015,6 +1015,7 @@ int launch_two_phase_wide_as(const TileLayerArgs &a, int n_tiles, int LA, hipStr
     if (SRC == ROWS_GLOBAL && !LAST) {
         splits = 2048 / (n_tiles > 0 ? n_tiles : 1);
         splits = splits < 1 ? 1 : (splits > 16 ? 16 : splits);
+        if (const char *e = getenv("GTM_WIDE_SPLITS")) splits = std::max(1, std::min(64, atoi(e)));
     }
     profile_start(LAST ? "k_tile_two_phase_wide<score>" : "k_tile_two_phase_wide<layer0>", st);
     hipLaunchKernelGGL((k_tile_two_phase_wide<NW, LW, SRC, LAST>), dim3((unsigned)((n_tiles + 7) / 8 * 8 * splits)),
