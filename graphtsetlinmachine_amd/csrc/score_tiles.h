@@ -1909,6 +1909,21 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
     };
     auto entry_of = [](const Packed8 &rec, int i) { return ((rec.v[i >> 1] >> ((i & 1) * 16)) & 0xFFFFu) << 4; };
 
+    // Per word of this lane: where in X the literal words of the node at the word's bit 0 are, and whether the
+    // word belongs to a graph with nodes (a graph without nodes keeps its bit 0 untested).  Phase 2 hands
+    // these round with readlane instead of dividing and looking the graph up for every word it visits.
+    uint32_t x_lo[LW], x_hi[LW], testable[LW];
+#pragma unroll
+    for (int u = 0; u < LW; ++u) {
+        const int tile_word = lane * LW + u;
+        const int gj = tg.slot_words > 0 ? tile_word / tg.slot_words : 0;
+        const bool owned = tg.slot_words > 0 && gj < tg.gpt;
+        const int node0 = owned ? (tile_word - gj * tg.slot_words) * 32 : 0;
+        const uint64_t at = (uint64_t)(((int64_t)(owned ? first_node[gj] : 0u) + node0) * LA);  // in words from X
+        x_lo[u] = (uint32_t)at, x_hi[u] = (uint32_t)(at >> 32);
+        testable[u] = owned && node_count[gj] != 0u ? 0xFFFFFFFFu : 0u;
+    }
+
     const int c_step = NWAVES * splits;
     const int c_first = wave + NWAVES * split;
     const int valid = c_first < C ? c_first : 0;
@@ -2005,18 +2020,16 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
                             live &= live - 1;
                             next_word = 0;
                         }
-                        uint32_t word = 0u;
+                        uint32_t word = 0u, lo = 0u, hi = 0u;
 #pragma unroll
                         for (int u = 0; u < LW; ++u)
-                            if (u == next_word) word = __builtin_amdgcn_readlane(acc.w[u], at_lane);
+                            if (u == next_word) {
+                                word = __builtin_amdgcn_readlane(acc.w[u] & testable[u], at_lane);
+                                lo = __builtin_amdgcn_readlane(x_lo[u], at_lane);
+                                hi = __builtin_amdgcn_readlane(x_hi[u], at_lane);
+                            }
                         at_word = next_word++;
-                        const int tile_word = at_lane * LW + at_word;       // word of the tile row
-                        const int gj = tile_word / tg.slot_words;           // graph of the tile
-                        const int node0 = (tile_word - gj * tg.slot_words) * 32;
-                        // (LDS reads at a wave-uniform index: readfirstlane keeps the cursor on the scalar unit)
-                        if (__builtin_amdgcn_readfirstlane(node_count[gj]) == 0u) word = 0u;  // a graph without nodes keeps its bit
-                        x_of_word = a.X + ((int64_t)__builtin_amdgcn_readfirstlane(first_node[gj]) + node0) * LA + w0 +
-                                    (in_row ? lane : 0);
+                        x_of_word = a.X + (int64_t)(((uint64_t)hi << 32) | lo) + w0 + (in_row ? lane : 0);
                         bits = word;
                     }
                     const int b = __builtin_ctz(bits);
