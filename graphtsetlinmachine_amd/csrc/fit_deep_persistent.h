@@ -182,27 +182,30 @@ __device__ __forceinline__ uint32_t fitd_transpose32(uint32_t a, int lane) {
     return a;
 }
 
-// truth[cl] &= the rows of the literals that words [w_lo, w_hi) of an include plane hold; returns how many
-// they hold.  `inc` points at the include plane's word 0 (words inc_stride apart); row r of the literal rows
-// is at col[(r - row_base) * stride] for this lane; literals >= `half` are negated: the complement of row
-// (literal - half) when `complement`, else a row of their own.  One wave.
+// acc &= the rows of the literals that words [w_lo, w_hi) of an include plane hold - and, with `twin` >= 0,
+// words [twin + w_lo, twin + w_hi) as well, in the same pass (the negated halves of a message bank's words; at
+// most 32 words then) - and adds how many they hold to *included (an LDS counter).  `inc` points at the include
+// plane's word 0 (words inc_stride apart); row r of the literal rows is at col[(r - row_base) * stride] for this
+// lane; literals >= `half` are negated: the complement of row (literal - half) when `complement`, else a row of
+// their own.  One wave.
 template <typename Rows>
-__device__ __forceinline__ int fitd_and_rows(const uint32_t *inc, int inc_stride, int w_lo, int w_hi, int last_word,
-                                             uint32_t filter, Rows col, int stride, int row_base, int half, bool complement,
-                                             int ones_row, uint32_t &acc, int lane) {
-    int included = 0;
+__device__ __forceinline__ void fitd_and_rows(const uint32_t *inc, int inc_stride, int w_lo, int w_hi, int twin, int last_word,
+                                              uint32_t filter, Rows col, int stride, int row_base, int half, bool complement,
+                                              int ones_row, uint32_t &acc, int *included, int lane) {
+    const int span = twin >= 0 ? w_hi - w_lo : 64;  // lanes [0, span): the words themselves; [span, 2 span): their twins
     for (int w0 = w_lo; w0 < w_hi; w0 += 64) {
-        uint32_t mine = w0 + lane < w_hi ? inc[(w0 + lane) * inc_stride] : 0u;
-        if (w0 + lane == last_word) mine &= filter;
-        included += wave_sum_small(__popc(mine));
+        const int mine_is = lane < span ? w0 + lane : twin + w0 + lane - span;  // the include word this lane holds
+        const bool holds = lane < span ? w0 + lane < w_hi : lane < 2 * span;
+        uint32_t mine = holds ? inc[mine_is * inc_stride] : 0u;
+        if (mine_is == last_word) mine &= filter;
+        if (mine != 0u) atomicAdd(included, __popc(mine));
         unsigned long long nonzero = __ballot(mine != 0);
-        if (__ballot(acc != 0u) == 0ull) continue;  // false everywhere stays false: only the count matters
         while (nonzero) {
-            if (__ballot(acc != 0u) == 0ull) break;
+            if (__ballot(acc != 0u) == 0ull) break;  // false everywhere stays false: only the count matters
             const int wl = __ffsll((long long)nonzero) - 1;
             nonzero &= nonzero - 1;
             uint32_t m = __builtin_amdgcn_readlane(mine, wl);
-            const int first = (w0 + wl) << 5;
+            const int first = (wl < span ? w0 + wl : twin + w0 + wl - span) << 5;
             const bool negated = complement && first >= half;  // (a word holds positive or negated literals, never both)
             const int row0 = (negated ? first - half : first) - row_base;
             const uint32_t flip = negated ? 0xFFFFFFFFu : 0u;
@@ -220,7 +223,6 @@ __device__ __forceinline__ int fitd_and_rows(const uint32_t *inc, int inc_stride
             }
         }
     }
-    return included;
 }
 
 // MAXB: bit planes of an automaton kept in registers while a word is updated (>= B).
@@ -386,12 +388,10 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                 const int cl = u / parts0, part = u - cl * parts0;
                 uint32_t acc = active ? truth[cl * NW + lane] : 0u;
                 const uint32_t before = acc;
-                const int included = fitd_and_rows(ta + (size_t)cl * per_clause * SB + (SB - 1), SB, part * chunk0,
-                                                   min(LA, (part + 1) * chunk0), LA - 1, p.filter,
-                                                   (const uint32_t *)rows0 + (active ? lane : 0), row_stride, 0, 0, false, ones_row,
-                                                   acc, lane);
+                fitd_and_rows(ta + (size_t)cl * per_clause * SB + (SB - 1), SB, part * chunk0, min(LA, (part + 1) * chunk0), -1,
+                              LA - 1, p.filter, (const uint32_t *)rows0 + (active ? lane : 0), row_stride, 0, 0, false, ones_row, acc,
+                              &incl_of[cl], lane);
                 if (active && acc != before) atomicAnd(&truth[cl * NW + lane], acc);
-                if (lane == 0 && included) atomicAdd(&incl_of[cl], included);
             }
             lds_barrier();
             if (fg.shift != 0 || fg.mask != 0xFFFFFFFFu) {  // several graphs share a word: keep this graph's bits
@@ -524,11 +524,10 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                         const uint32_t before = acc;
                         const uint32_t *inc = ta + ((size_t)cl * per_clause + LA + (size_t)l * MC) * SB + (SB - 1);
                         const int lo = w_first + part * chunk1, hi = min(w_first + window_words, lo + chunk1);
-                        // (2 M is a multiple of 32: the last word has no tail to mask) positive literals, then negated
-                        int included = fitd_and_rows(inc, SB, lo, hi, -1, 0u, col, NW, r0, M, true, r0, acc, lane);
-                        included += fitd_and_rows(inc, SB, MW + lo, MW + hi, -1, 0u, col, NW, r0, M, true, r0, acc, lane);
+                        // (2 M is a multiple of 32: the last word has no tail to mask) the words of the positive literals and,
+                        // in the same pass, those of the negated ones (MW words further on)
+                        fitd_and_rows(inc, SB, lo, hi, MW, -1, 0u, col, NW, r0, M, true, r0, acc, &incl_of[cl], lane);
                         if (active && acc != before) atomicAnd(&truth[cl * NW + lane], acc);
-                        if (lane == 0 && included) atomicAdd(&incl_of[cl], included);
                     }
                 }
                 if constexpr (BIG) {
