@@ -1002,7 +1002,12 @@ int launch_two_phase_half(const TileLayerArgs &a, int n_tiles, int la4, bool las
 template <int NW, int LW, int SRC, bool LAST>
 int launch_two_phase_wide_as(const TileLayerArgs &a, int n_tiles, int LA, hipStream_t st) {
     // rows (if staged), padding, class sums, and the first node and node count of the tile's graphs
-    size_t lds = tile_layer_lds_bytes(a.tg, a.K, SRC, a.M) + (size_t)a.tg.gpt * 8;
+    // several narrow tiles per wave (rows read in place, truth rows only, one word per lane): see the kernel
+    int pack = 1;
+    if (SRC == ROWS_GLOBAL && !LAST && LW == 1 && a.tg.tw <= 32 && !getenv("GTM_NO_TILE_PACK"))
+        pack = 64 / a.tg.tw;
+    const int n_groups = (n_tiles + pack - 1) / pack;
+    size_t lds = tile_layer_lds_bytes(a.tg, a.K, SRC, a.M) + (size_t)pack * a.tg.gpt * 8;
     static thread_local size_t lds_set = 48 * 1024;
     if (lds > lds_set) {
         hipError_t e = hipFuncSetAttribute((const void *)k_tile_two_phase_wide<NW, LW, SRC, LAST>,
@@ -1013,13 +1018,13 @@ int launch_two_phase_wide_as(const TileLayerArgs &a, int n_tiles, int LA, hipStr
     // rows read in place and no votes: several workgroups share a tile's clauses until the chip is full
     int splits = 1;
     if (SRC == ROWS_GLOBAL && !LAST) {
-        splits = 2048 / (n_tiles > 0 ? n_tiles : 1);
+        splits = 2048 / (n_groups > 0 ? n_groups : 1);
         splits = splits < 1 ? 1 : (splits > 16 ? 16 : splits);
         if (const char *e = getenv("GTM_WIDE_SPLITS")) splits = std::max(1, std::min(64, atoi(e)));
     }
     profile_start(LAST ? "k_tile_two_phase_wide<score>" : "k_tile_two_phase_wide<layer0>", st);
-    hipLaunchKernelGGL((k_tile_two_phase_wide<NW, LW, SRC, LAST>), dim3((unsigned)((n_tiles + 7) / 8 * 8 * splits)),
-                       dim3(NW * 64), lds, st, a, LA, n_tiles, splits);
+    hipLaunchKernelGGL((k_tile_two_phase_wide<NW, LW, SRC, LAST>), dim3((unsigned)((n_groups + 7) / 8 * 8 * splits)),
+                       dim3(NW * 64), lds, st, a, LA, n_tiles, splits, pack);
     if (int rc = check_launch("tile_two_phase_wide")) return rc;
     profile_stop(st);
     return GTM_OK;
@@ -1186,11 +1191,14 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                 continue;
             }
             profile_start("k_tile_node_messages + k_tile_edge_messages + k_tile_pack_messages", st);
-            if (by_bit)
+            if (by_bit) {
+                const int pack = tg.tw <= 32 && !getenv("GTM_NO_TILE_PACK") ? 64 / tg.tw : 1;  // narrow tiles share a wave
                 hipLaunchKernelGGL(k_tile_node_messages_by_bit,
-                                   dim3((MW + NODE_MESSAGES_BY_BIT_WAVES - 1) / NODE_MESSAGES_BY_BIT_WAVES, n_tiles),
+                                   dim3((MW + NODE_MESSAGES_BY_BIT_WAVES - 1) / NODE_MESSAGES_BY_BIT_WAVES,
+                                        (n_tiles + pack - 1) / pack),
                                    dim3(64 * NODE_MESSAGES_BY_BIT_WAVES), 0, st, w.tile_bitmap, d.C, tg.tw, w.bit_start,
-                                   w.bit_clauses, d.M, MW, w.sent);
+                                   w.bit_clauses, d.M, MW, n_tiles, pack, w.sent);
+            }
             else
             hipLaunchKernelGGL(k_tile_node_messages, dim3((tg.tw + group - 1) / group, n_tiles),
                                dim3(TILE_MESSAGES_BLOCK), ((size_t)32 * group * (MW | 1) + group) * 4, st, w.tile_bitmap, d.C, tg.tw,

@@ -480,25 +480,30 @@ __device__ __forceinline__ void message_bit_words(const uint32_t *__restrict__ r
 // rows: for each bit the rows of the bit's clauses are ORed (whole rows, coalesced; the clause
 // numbers come in by one load per bit and are handed round with readlane), the 32 resulting rows
 // are transposed inside each lane, 32 x 32 bits, and the lane stores word j of its 32 slots.
-// grid (ceil(MW / waves per block), tiles).  Every word of sent is written (no clearing needed).
+// grid (ceil(MW / waves per block), ceil(tiles / pack)).  Every word of sent is written (no clearing
+// needed).  Tiles of at most 32 words are taken `pack` = 64 / tw at a time, lane l on word l % tw of tile
+// l / tw of the group (the clause numbers of a bit are the same for every tile).
 constexpr int NODE_MESSAGES_BY_BIT_WAVES = 4;
 
 __global__ __launch_bounds__(64 * NODE_MESSAGES_BY_BIT_WAVES) void k_tile_node_messages_by_bit(
     const uint32_t *__restrict__ bitmap, int C, int tw, const uint32_t *__restrict__ bit_start,
-    const uint32_t *__restrict__ bit_clauses, int M, int MW, uint32_t *__restrict__ sent) {
+    const uint32_t *__restrict__ bit_clauses, int M, int MW, int n_tiles, int pack, uint32_t *__restrict__ sent) {
     __shared__ uint32_t stage_of_wave[NODE_MESSAGES_BY_BIT_WAVES][32][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int j = blockIdx.x * NODE_MESSAGES_BY_BIT_WAVES + wave, tile = blockIdx.y;
+    const int j = blockIdx.x * NODE_MESSAGES_BY_BIT_WAVES + wave;
     if (j >= MW) return;  // the block has no barrier
     uint32_t(*stage)[64] = stage_of_wave[wave];
-    const uint32_t *rows = bitmap + (int64_t)tile * C * tw;
+    const int sub = pack > 1 ? lane / tw : 0, word_of_lane = pack > 1 ? lane - sub * tw : lane;
+    const int tile = (int)blockIdx.y * pack + sub;
+    const bool tile_exists = sub < pack && tile < n_tiles;
+    const uint32_t *rows = bitmap + (int64_t)(tile_exists ? tile : (int)blockIdx.y * pack) * C * tw;
     // lane i <= 32 holds where the clauses of bit 32 j + i begin (bits past M: nothing)
     const int p_of_lane = 32 * j + lane < M ? 32 * j + lane : M;
     const uint32_t start_of_lane = lane <= 32 ? bit_start[p_of_lane] : 0u;
-    for (int w0 = 0; w0 < tw; w0 += 64) {
-        const int w = w0 + lane;
-        const bool active = w < tw;
+    for (int w0 = 0; w0 < (pack > 1 ? 1 : tw); w0 += 64) {
+        const int w = pack > 1 ? word_of_lane : w0 + lane;
+        const bool active = tile_exists && w < tw;
         const uint32_t *col = rows + (active ? w : 0);
 #pragma unroll 1
         for (int i = 0; i < 32; ++i) {
@@ -1856,14 +1861,19 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
 // share a tile's clauses (truth rows only: the votes of LAST need one
 // workgroup per tile).
 template <int NWAVES, int LW, int SRC, bool LAST>
-__global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerArgs a, int LA, int n_tiles, int splits) {
+__global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerArgs a, int LA, int n_tiles, int splits,
+                                                                      int pack) {
     extern __shared__ uint32_t lds[];
     // Workgroups go to the 8 XCDs in turn, and each XCD has its own L2: the workgroups that share a
     // tile (its rows are read in place, again and again) are given to one XCD, one after the other,
     // so that the few tiles an XCD works on at a time stay in its L2.  1-D grid of
-    // ceil(n_tiles / 8) * 8 * splits workgroups.
+    // ceil(groups / 8) * 8 * splits workgroups, a group being `pack` consecutive tiles: a narrow tile
+    // (rows of at most 32 words, rows read in place, truth rows only) leaves half of a wave's lanes or more
+    // without a word, so a wave takes 64 / tw tiles at once, lane l on word l % tw of tile l / tw of the
+    // group - the clause's row offsets are the same for every tile, and everything else is per lane.
     const int xcd = blockIdx.x & 7, turn = blockIdx.x >> 3;
-    const int split = turn % splits, tile_of_launch = (turn / splits) * 8 + xcd;
+    const int split = turn % splits, group_of_launch = (turn / splits) * 8 + xcd;
+    const int tile_of_launch = group_of_launch * pack;  // the group's first tile
     if (tile_of_launch >= n_tiles) return;
     const TileGeom &tg = a.tg;
     const int tw = tg.tw, C = a.C, K = a.K;
@@ -1871,13 +1881,16 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
     const int n_rows_lds = SRC == ROWS_STAGED ? tg.rows : 0;
     uint32_t *bt = lds;
     int32_t *sums = (int32_t *)(lds + (size_t)n_rows_lds * tw + TILE_LDS_PAD_WORDS);
-    uint32_t *first_node = (uint32_t *)(sums + tg.gpt * K);  // [gpt] row of X of each graph's node 0
-    uint32_t *node_count = first_node + tg.gpt;              // [gpt]
+    uint32_t *first_node = (uint32_t *)(sums + tg.gpt * K);  // [pack][gpt] row of X of each graph's node 0
+    uint32_t *node_count = first_node + pack * tg.gpt;       // [pack][gpt]
     const int tile = a.tile0 + tile_of_launch;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    uint32_t *bitmap = a.bitmap + (int64_t)tile_of_launch * C * tw;
+    // this lane's tile of the group and its first word there
+    const int sub = pack > 1 ? lane / tw : 0, word_of_lane = pack > 1 ? lane - sub * tw : lane * LW;
+    const bool tile_exists = sub < pack && tile_of_launch + sub < n_tiles;  // (the last lanes may be left over)
+    uint32_t *bitmap = a.bitmap + (int64_t)(tile_of_launch + (tile_exists ? sub : 0)) * C * tw;
 
     if (SRC == ROWS_STAGED) {
         const uint4 *src = reinterpret_cast<const uint4 *>(a.tiles + (int64_t)tile * tg.rows * tw);
@@ -1886,16 +1899,17 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
         for (int i = tid; i < n4; i += NT) dst[i] = src[i];
     }
     for (int i = tid; i < TILE_LDS_PAD_WORDS + tg.gpt * K; i += NT) bt[(size_t)n_rows_lds * tw + i] = 0;
-    for (int j = tid; j < tg.gpt; j += NT) {
-        const int64_t g = (int64_t)tile * tg.gpt + j;
+    for (int j = tid; j < pack * tg.gpt; j += NT) {
+        const int64_t g = (int64_t)tile * tg.gpt + j;  // (the tiles of a group follow each other: so do their graphs)
         first_node[j] = g < a.G ? a.node_index[g] : 0u;
         node_count[j] = g < a.G ? a.n_nodes[g] : 0u;
     }
     __syncthreads();
 
-    const bool active = lane * LW < tw;
+    const bool active = pack > 1 ? tile_exists : lane * LW < tw;
     const char *col = SRC == ROWS_GLOBAL
-                          ? reinterpret_cast<const char *>(a.tiles + (int64_t)tile * tg.rows * tw + (active ? lane * LW : 0))
+                          ? reinterpret_cast<const char *>(a.tiles + (int64_t)(tile + (active ? sub : 0)) * tg.rows * tw +
+                                                           (active ? word_of_lane : 0))
                           : reinterpret_cast<const char *>(bt + lane * LW);
     const int pairs = tg.gpt * K;
     const int my_shift = (lane < tg.gpt ? lane : 0) * tg.lanes_per_graph;
@@ -1915,13 +1929,14 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
     uint32_t x_lo[LW], x_hi[LW], testable[LW];
 #pragma unroll
     for (int u = 0; u < LW; ++u) {
-        const int tile_word = lane * LW + u;
+        const int tile_word = word_of_lane + u;
         const int gj = tg.slot_words > 0 ? tile_word / tg.slot_words : 0;
-        const bool owned = tg.slot_words > 0 && gj < tg.gpt;
+        const bool owned = tg.slot_words > 0 && gj < tg.gpt && active;
         const int node0 = owned ? (tile_word - gj * tg.slot_words) * 32 : 0;
-        const uint64_t at = (uint64_t)(((int64_t)(owned ? first_node[gj] : 0u) + node0) * LA);  // in words from X
+        const int graph_of_group = sub * tg.gpt + gj;
+        const uint64_t at = (uint64_t)(((int64_t)(owned ? first_node[graph_of_group] : 0u) + node0) * LA);  // in words from X
         x_lo[u] = (uint32_t)at, x_hi[u] = (uint32_t)(at >> 32);
-        testable[u] = owned && node_count[gj] != 0u ? 0xFFFFFFFFu : 0u;
+        testable[u] = owned && node_count[graph_of_group] != 0u ? 0xFFFFFFFFu : 0u;
     }
 
     const int c_step = NWAVES * splits;
@@ -2061,7 +2076,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
             nz = __ballot(any_bit(acc));
         }
         if (!LAST) {
-            if (active) acc.store(reinterpret_cast<char *>(bitmap + (int64_t)c * tw + lane * LW));
+            if (active) acc.store(reinterpret_cast<char *>(bitmap + (int64_t)c * tw + word_of_lane));
             return;
         }
         if (nz == 0) return;
