@@ -171,16 +171,7 @@ __device__ __forceinline__ bool fitd_wait(const unsigned long long *parts, unsig
 
 // A 32 x 32 bit matrix held one row per lane (both halves of a wave hold one each): afterwards lane b
 // holds column b, i.e. bit k of its word = bit b of what lane k (of the same half) held.
-__device__ __forceinline__ uint32_t fitd_transpose32(uint32_t a, int lane) {
-    uint32_t m = 0x0000FFFFu;
-#pragma unroll
-    for (int j = 16; j != 0; j >>= 1) {
-        const uint32_t other = __shfl_xor(a, j);
-        a = (lane & j) ? (a & ~m) | ((other >> j) & m) : (a & m) | ((other << j) & ~m);
-        m ^= m << (j >> 1);
-    }
-    return a;
-}
+__device__ __forceinline__ uint32_t fitd_transpose32(uint32_t a, int lane) { return tile_transpose32(a, lane); }
 
 // acc &= the rows of the literals that words [w_lo, w_hi) of an include plane hold - and, with `twin` >= 0,
 // words [twin + w_lo, twin + w_hi) as well, in the same pass (the negated halves of a message bank's words; at

@@ -388,13 +388,37 @@ inline size_t tile_layer_lds_bytes(const TileGeom &g, int classes, int src, int 
 
 constexpr int TILE_MESSAGES_BLOCK = 1024;
 
+// The word of the lane whose index differs in bit J (1 .. 16): lane moves on the vector unit (within quads,
+// within rows of 16 lanes, and the swap of neighbouring rows of 16), which do not queue behind the LDS
+// traffic of the other waves the way a shuffle through the LDS crossbar does.  Every lane of the 32 that
+// exchange must be active.
+template <int J>
+__device__ __forceinline__ uint32_t tile_lane_xor(uint32_t v, int lane) {
+    static_assert(J == 1 || J == 2 || J == 4 || J == 8 || J == 16, "one bit of the lane index");
+    if constexpr (J == 1) {
+        return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);  // quad_perm [1, 0, 3, 2]
+    } else if constexpr (J == 2) {
+        return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xF, 0xF, true);  // quad_perm [2, 3, 0, 1]
+    } else if constexpr (J == 4) {
+        // lane ^ 7 (the 8 lanes mirrored), then lane ^ 3 (the quad reversed)
+        const int mirrored = __builtin_amdgcn_mov_dpp((int)v, 0x141, 0xF, 0xF, true);  // row_half_mirror
+        return (uint32_t)__builtin_amdgcn_mov_dpp(mirrored, 0x1B, 0xF, 0xF, true);     // quad_perm [3, 2, 1, 0]
+    } else if constexpr (J == 8) {
+        return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x128, 0xF, 0xF, true);  // row_ror 8
+    } else {
+        // the odd rows of 16 lanes of the first copy and the even rows of the second change places
+        const auto swapped = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+        return (lane & 16) ? swapped[0] : swapped[1];
+    }
+}
+
 // Transposes the 32 x 32 bit matrix whose row i is the word of lane i (of each half of the wave):
 // afterwards bit i of lane b's word is what bit b of lane i's word was.  Five exchanges of
 // half-blocks with the lane 16, 8, 4, 2, 1 away.
 template <int J, uint32_t M>
 __device__ __forceinline__ uint32_t tile_transpose_step(uint32_t v, int lane) {
     // M: the columns whose index has bit J clear
-    const uint32_t p = (uint32_t)__shfl_xor((int)v, J);
+    const uint32_t p = tile_lane_xor<J>(v, lane);
     return (lane & J) ? ((p >> J) & M) | (v & ~M) : (v & M) | ((p & M) << J);
 }
 
@@ -718,16 +742,30 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
     const int w_first = gj * sw;        // the graph's first word of a tile row
     uint32_t *out = rows + (int64_t)tile_local * (M + 2) * tw;
 
-    for (int i = tid; i < VEC; i += NT) got[i] = 0u;  // (every word of sent that is read is stored first)
-    __syncthreads();
-
     // 1. what every node slot sends: a half-wave takes 32 message bits and up to 8 words of the graph's
     // truth rows at a time (lane = bit: the OR of the truth words of the bit's clauses), transposes,
-    // and lane = node stores word j of its vector - each word once, no atomics
+    // and lane = node stores word j of its vector - each word once, no atomics.  A lane's work is a chain
+    // of dependent reads (where the bit's clauses start, which they are, their truth words): the index
+    // and the graph's truth rows are first copied into the space of `got`, which is not needed yet, when
+    // they fit there, so that the chain runs on LDS.
     if (nodes > 0) {
         constexpr int WB = MESSAGE_WORDS_AT_ONCE;
         const uint32_t *truth = bitmap + (int64_t)tile_local * C * tw + w_first;
         const int used = (nodes + 31) >> 5;  // words of a truth row that can hold a true node
+        const uint32_t n_listed = bit_start[M];  // (clause, bit) pairs in the index
+        // (staged rows an odd number of words apart: the lanes of a half-wave read words of different clauses)
+        const int ts = used | 1;
+        const bool staged = (size_t)(M + 1) + n_listed + (size_t)C * ts <= (size_t)VEC;
+        uint32_t *s_start = got, *s_clauses = got + (M + 1), *s_truth = s_clauses + n_listed;
+        if (staged) {
+            for (int i = tid; i <= M; i += NT) s_start[i] = bit_start[i];
+            for (uint32_t i = tid; i < n_listed; i += NT) s_clauses[i] = bit_clauses[i];
+            for (int i = tid; i < C * used; i += NT) {
+                const int c = i / used, w = i - c * used;
+                s_truth[c * ts + w] = truth[(int64_t)c * tw + w];
+            }
+            __syncthreads();
+        }
         const int hl = lane & 31, half = lane >> 5;
         const int blocks_w = (used + WB - 1) / WB, tasks = MW * blocks_w;
         for (int t0 = wave * 2; t0 < tasks; t0 += NT / 32) {
@@ -736,7 +774,11 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
             const int j = valid ? t / blocks_w : 0, wl0 = valid ? (t - j * blocks_w) * WB : 0;
             const int n_words = valid ? (used - wl0 < WB ? used - wl0 : WB) : 0;
             uint32_t word[WB];
-            message_bit_words(truth + wl0, tw, n_words, bit_start, bit_clauses, j * 32 + hl, M, word);
+            // (two calls, so that the copies are read with LDS instructions and not through generic pointers)
+            if (staged)
+                message_bit_words(s_truth + wl0, ts, n_words, s_start, s_clauses, j * 32 + hl, M, word);
+            else
+                message_bit_words(truth + wl0, tw, n_words, bit_start, bit_clauses, j * 32 + hl, M, word);
 #pragma unroll
             for (int u = 0; u < WB; ++u) {
                 const uint32_t column = tile_transpose32(word[u], lane);
@@ -744,6 +786,8 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
             }
         }
     }
+    __syncthreads();
+    for (int i = tid; i < VEC; i += NT) got[i] = 0u;  // (every word of sent that is read has been stored)
     __syncthreads();
 
     // 2. along the edges: bit p of what arrives is bit (p - type) mod M of what was sent
@@ -781,7 +825,10 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
     // the graph's words of those rows; its 32 x sw words of staging live where sent was
     const int pack_waves = MW < NT / 64 ? MW : NT / 64;
     if (wave < pack_waves) {
-        uint32_t *stage = sent + wave * 32 * sw;  // [32 rows][sw]
+        // (rows an odd number of words apart where there is room: the 32 lanes that store a column of 32 rows
+        // then hit 32 banks, not 2)
+        const int ss = pack_waves * 32 * (sw | 1) <= VEC ? sw | 1 : sw;
+        uint32_t *stage = sent + wave * 32 * ss;  // [32 rows][ss]
         for (int j = wave; j < MW; j += pack_waves) {
             for (int nb = 0; nb * 2 < sw; ++nb) {
                 const int slot = nb * 64 + lane;
@@ -789,12 +836,16 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
                 // lanes 0..31 and 32..63 each transpose their 32 x 32 bits: lane b of a half ends up
                 // with bit b of the half's 32 slots, i.e. one word of row 32 j + b
                 const uint32_t column = tile_transpose32(word, lane);
-                if (nb * 2 + (lane >> 5) < sw) stage[(lane & 31) * sw + nb * 2 + (lane >> 5)] = column;
+                if (nb * 2 + (lane >> 5) < sw) stage[(lane & 31) * ss + nb * 2 + (lane >> 5)] = column;
             }
             // (a wave's LDS writes are visible to its own later reads: same wave, in order)
-            for (int i = lane; i < 32 * sw; i += 64) {
-                const int r = i / sw, w = i - r * sw;
-                out[(int64_t)(j * 32 + r) * tw + w_first + w] = stage[i];
+            if (sw <= 32) {  // two rows per trip, a half-wave each
+                const int w = lane & 31;
+                for (int r = lane >> 5; r < 32; r += 2)
+                    if (w < sw) out[(int64_t)(j * 32 + r) * tw + w_first + w] = stage[r * ss + w];
+            } else {
+                for (int r = 0; r < 32; ++r)
+                    for (int w = lane; w < sw; w += 64) out[(int64_t)(j * 32 + r) * tw + w_first + w] = stage[r * ss + w];
             }
         }
     }
