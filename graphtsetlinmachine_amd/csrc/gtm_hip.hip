@@ -599,9 +599,9 @@ struct ScoreWs {
     size_t bytes;
 };
 
-// Length of a compiled clause: header + type row + literals, padded to 32 entries, + 32 entries
-// that the kernel may fetch ahead unused.
-int clause_list_stride(int literals) { return ((literals + 2 + 31) & ~31) + 32; }
+// Length of a compiled clause: header + type row + literals + what fills its two parts up to whole
+// 8-entry blocks, padded to 32 entries, + 32 entries that the kernel may fetch ahead unused.
+int clause_list_stride(int literals) { return ((literals + 2 + 14 + 31) & ~31) + 32; }
 
 // Tiles one launch group covers when the caller asks for `batch` graphs at a time.
 int tiles_per_batch(const TileGeom &tg, int batch) { return (batch + tg.gpt - 1) / tg.gpt; }
@@ -864,8 +864,15 @@ int tile_layer_splits(const TileLayerArgs &a, int n_tiles, int src) {
 }
 
 template <int NW, int LW, int SRC, bool LAST>
-int launch_tile_layer_as(const TileLayerArgs &a, int n_tiles, const char *profile_name, hipStream_t st) {
+int launch_tile_layer_as(const TileLayerArgs &a_in, int n_tiles, const char *profile_name, hipStream_t st) {
+    TileLayerArgs a = a_in;
     size_t lds = tile_layer_lds_bytes(a.tg, a.K, SRC, a.M);
+    // message layers: room for every wave's clause list where LDS has it (GTM_NO_LISTS_IN_LDS: tuning and test aid)
+    a.lists_in_lds = 0;
+    if (SRC == ROWS_MESSAGES && lds + (size_t)NW * TILE_LIST_LDS_WORDS * 4 <= 160 * 1024 && !getenv("GTM_NO_LISTS_IN_LDS")) {
+        a.lists_in_lds = 1;
+        lds += (size_t)NW * TILE_LIST_LDS_WORDS * 4;
+    }
     const int splits = tile_layer_splits(a, n_tiles, SRC);
     if (LAST && splits > 1) {  // the workgroups of a tile add their shares
         const int64_t n = (int64_t)a.n_graphs * a.K;

@@ -249,17 +249,16 @@ __global__ void k_row_order(const unsigned long long *__restrict__ row_count, in
 }
 
 // Per call, one wave per clause: the rows the clause ANDs together, as 32-bit
-// LDS byte offsets (row * tw * 4).  Entry 0 = number of 8-entry blocks in use;
-// with n_types > 0 entry 1 = the row of the clause's node type
-// (kernels.py:447); then the clause's included literals, in `order` when
-// given: the ones that hold least often come first, so the running AND dies
-// (and the walk stops) as early as it can; the order does not change the
+// LDS byte offsets (row * tw * 4).  Entry 0 = the 8-entry blocks in use (see
+// the end of the kernel); with n_types > 0 entry 1 = the row of the clause's
+// node type (kernels.py:447); then the clause's included literals, in `order`
+// when given: the ones that hold least often come first, so the running AND
+// dies (and the walk stops) as early as it can; the order does not change the
 // result.  With half > 0 (message banks) literal l >= half is the negation of
-// literal l - half and is stored as that row's offset with bit 31 set.  The
-// list starts with a chunk of 32 entries that the evaluating kernel fetches
-// one clause ahead; unused entries point at the all-ones row.  Also, when
-// `weights` is given, the weights clause-major.
-constexpr uint32_t TILE_NEGATED = 0x80000000u;
+// literal l - half: those come in a second part, as the offsets of the rows
+// whose complements are ANDed.  The list starts with a chunk of 32 entries;
+// unused entries point at the all-ones row.  Also, when `weights` is given,
+// the weights clause-major.
 
 __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int chunks, int B, uint32_t filter,
                                   int literals, int half, int n_types, int type_base_row, int ones_row, int tw,
@@ -277,25 +276,45 @@ __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int 
         if (lane == 0) list[1] = (uint32_t)(type_base_row + c % n_types) * row_bytes;
         n = 2;
     }
+    // With negated literals as complements of rows (half > 0: message layers) the list comes in two parts, each a
+    // whole number of 8-entry blocks: the rows to AND, then the rows whose complements to AND - a block is all of
+    // one kind, so the evaluation needs no per-entry flag.  `plain`: entries of the first part.
+    int plain = n;
+    for (int r0 = 0; r0 < literals; r0 += 64) {
+        const int r = r0 + lane;
+        const uint32_t lit = r < literals ? (order ? order[r] : (uint32_t)r) : 0u;
+        uint32_t word = inc[(int64_t)(lit >> 5) * B];
+        if ((int)(lit >> 5) == chunks - 1) word &= filter;
+        plain += __popcll(__ballot(r < literals && (half == 0 || (int)lit < half) && ((word >> (lit & 31)) & 1u)));
+    }
+    const int plain_padded = (plain + 7) & ~7;
+    int n_neg = 0;
     for (int r0 = 0; r0 < literals; r0 += 64) {
         int r = r0 + lane;
         uint32_t lit = r < literals ? (order ? order[r] : (uint32_t)r) : 0u;
         uint32_t w = lit >> 5;
         uint32_t word = inc[(int64_t)w * B];
         if ((int)w == chunks - 1) word &= filter;
-        bool included = r < literals && ((word >> (lit & 31)) & 1u);
-        unsigned long long mask = __ballot(included);
-        if (included) {
-            uint32_t entry = (half > 0 && (int)lit >= half) ? ((lit - (uint32_t)half) * row_bytes) | TILE_NEGATED
-                                                            : lit * row_bytes;
-            list[n + __popcll(mask & ((1ull << lane) - 1ull))] = entry;
-        }
-        n += __popcll(mask);
+        const bool included = r < literals && ((word >> (lit & 31)) & 1u);
+        const bool negated = included && half > 0 && (int)lit >= half;
+        const unsigned long long below = (1ull << lane) - 1ull;
+        const unsigned long long plain_mask = __ballot(included && !negated), neg_mask = __ballot(negated);
+        if (included && !negated) list[n + __popcll(plain_mask & below)] = lit * row_bytes;
+        if (negated) list[plain_padded + n_neg + __popcll(neg_mask & below)] = (lit - (uint32_t)half) * row_bytes;
+        n += __popcll(plain_mask);
+        n_neg += __popcll(neg_mask);
     }
-    const int padded = (n + 7) & ~7;
+    for (int i = n + lane; i < plain_padded; i += 64) list[i] = ones;
+    // The last block of complements is filled up with the row after the all-ones row: in a message layer's rows
+    // that is the row of the graphs without nodes, zero at every node slot of every other graph - and what its
+    // complement takes from a graph without nodes the evaluation puts back (such a graph keeps every clause true).
+    const int neg_padded = (n_neg + 7) & ~7;
+    for (int i = n_neg + lane; i < neg_padded; i += 64) list[plain_padded + i] = ones + row_bytes;
+    const int padded = plain_padded + neg_padded;
     const int fill_to = padded < 32 ? 32 : (padded + 15) & ~15;
-    for (int i = n + lane; i < fill_to; i += 64) list[i] = ones;
-    if (lane == 0) list[0] = (uint32_t)(padded >> 3);
+    for (int i = padded + lane; i < fill_to; i += 64) list[i] = ones;
+    // entry 0: blocks of rows to AND | blocks of rows whose complements to AND << 16
+    if (lane == 0) list[0] = (uint32_t)(plain_padded >> 3) | ((uint32_t)(neg_padded >> 3) << 16);
     if (weights)
         for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
 }
@@ -364,7 +383,13 @@ struct TileLayerArgs {
     const uint32_t *X;      // [nodes][LA] node-major literal words (two-phase layer 0)
     const uint32_t *message_rows;  // [tiles of the launch][M + 2][tw] (message layers, built by k_tile_pack_messages)
     const uint32_t *xpos;   // [tiles][tw * 32 slots][LA / 2]: the positive literal words by node slot (half tiles)
+    int lists_in_lds;       // message layers: LDS holds TILE_LIST_LDS_WORDS more words per wave for the clause lists
 };
+
+// A wave of k_tile_layer keeps the list of the clause it evaluates in LDS when it has at most this many entries
+// (+ 8 words that the walk reads ahead).
+constexpr int TILE_LIST_ENTRIES = 256;
+constexpr int TILE_LIST_LDS_WORDS = TILE_LIST_ENTRIES + 8;
 
 // Rows a message layer keeps in LDS: M message rows, the all-ones row, the row of graphs without nodes.
 inline int tile_message_rows(int M) { return M + 2; }
@@ -944,17 +969,24 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
         for (int u = 1; u < LW; ++u) m |= x.w[u];
         return m != 0;
     };
-    auto and_row = [&](LaneWords<LW> &acc, uint32_t entry) {
-        LaneWords<LW> r;
-        if (SRC == ROWS_MESSAGES) {
-            r.load(col + (entry & ~TILE_NEGATED));
-            const uint32_t flip = (uint32_t)((int32_t)entry >> 31);  // all ones for a negated literal
+    // acc &= the rows of entries e[from .. 7] of an 8-entry block (their complements: a block is all of one kind)
+    auto and_block = [&](LaneWords<LW> &acc, const uint32_t *e, int from, bool complements) {
+        LaneWords<LW> r[8];
 #pragma unroll
-            for (int u = 0; u < LW; ++u) acc.w[u] &= r.w[u] ^ flip;
+        for (int i = 0; i < 8; ++i)
+            if (i >= from) r[i].load(col + e[i]);
+        if (SRC == ROWS_MESSAGES && complements) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (i >= from)
+#pragma unroll
+                    for (int u = 0; u < LW; ++u) acc.w[u] &= ~r[i].w[u];
         } else {
-            r.load(col + entry);
 #pragma unroll
-            for (int u = 0; u < LW; ++u) acc.w[u] &= r.w[u];
+            for (int i = 0; i < 8; ++i)
+                if (i >= from)
+#pragma unroll
+                    for (int u = 0; u < LW; ++u) acc.w[u] &= r[i].w[u];
         }
     };
 
@@ -968,50 +1000,10 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
         any_empty = __ballot(any_bit(empties)) != 0;
     }
 
-    // `truth_in` is the clause's truth from the previous layer (message layers only)
-    auto evaluate = [&](const Chunk32 &head, const uint32_t *list, const int32_t *weights_of_clause,
-                        const LaneWords<LW> &truth_in, char *truth_out) {
-        const int my_weight = pair_lane ? weights_of_clause[my_k] : 0;  // needed only if the clause fires
-        const int nb = (int)head.v[0];
-        LaneWords<LW> acc;
-        bool alive = true;
-        if (SRC == ROWS_MESSAGES) {
-            acc = truth_in;
-            alive = __ballot(any_bit(acc)) != 0;
-        } else {
-#pragma unroll
-            for (int u = 0; u < LW; ++u) acc.w[u] = active ? 0xFFFFFFFFu : 0u;
-        }
-        if (alive) {
-#pragma unroll
-            for (int i = 1; i < 8; ++i) and_row(acc, head.v[i]);
-            // stop as soon as the clause is false at every node slot of the tile
-            if (nb > 1 && __ballot(any_bit(acc)) != 0) {
-                // entries past the first chunk, 16 at a time, requested one step before they are needed
-                const Chunk16 *tp = reinterpret_cast<const Chunk16 *>(list) + 2;
-                Chunk16 tail = *tp;
-#pragma unroll
-                for (int i = 8; i < 16; ++i) and_row(acc, head.v[i]);
-                if (nb > 2 && __ballot(any_bit(acc)) != 0) {
-#pragma unroll
-                    for (int i = 16; i < 24; ++i) and_row(acc, head.v[i]);
-                    if (nb > 3 && __ballot(any_bit(acc)) != 0) {
-#pragma unroll
-                        for (int i = 24; i < 32; ++i) and_row(acc, head.v[i]);
-                        for (int j = 4; j < nb && __ballot(any_bit(acc)) != 0; j += 2) {
-                            const Chunk16 ahead = *++tp;
-#pragma unroll
-                            for (int i = 0; i < 8; ++i) and_row(acc, tail.v[i]);
-                            if (j + 1 < nb && __ballot(any_bit(acc)) != 0) {
-#pragma unroll
-                                for (int i = 8; i < 16; ++i) and_row(acc, tail.v[i]);
-                            }
-                            tail = ahead;
-                        }
-                    }
-                }
-            }
-        }
+    // What a clause's truth row `acc` adds to the class sums, or the row itself.  `alive`: the clause was true
+    // somewhere before this layer.
+    auto finish = [&](LaneWords<LW> &acc, bool alive, int my_weight, const int32_t *weights_of_clause,
+                      const LaneWords<LW> &truth_in, char *truth_out) {
         if (SRC == ROWS_MESSAGES && any_empty) {
 #pragma unroll
             for (int u = 0; u < LW; ++u) acc.w[u] |= truth_in.w[u] & empties.w[u];
@@ -1047,6 +1039,81 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
         }
     };
 
+    // `truth_in` is the clause's truth from the previous layer (message layers only)
+    auto evaluate = [&](const Chunk32 &head, const uint32_t *list, const int32_t *weights_of_clause,
+                        const LaneWords<LW> &truth_in, char *truth_out) {
+        const int my_weight = pair_lane ? weights_of_clause[my_k] : 0;  // needed only if the clause fires
+        const int plain = (int)(head.v[0] & 0xFFFFu);  // blocks of rows; the blocks after them: rows to complement
+        const int nb = plain + (int)(head.v[0] >> 16);
+        LaneWords<LW> acc;
+        bool alive = true;
+        if (SRC == ROWS_MESSAGES) {
+            acc = truth_in;
+            alive = __ballot(any_bit(acc)) != 0;
+        } else {
+#pragma unroll
+            for (int u = 0; u < LW; ++u) acc.w[u] = active ? 0xFFFFFFFFu : 0u;
+        }
+        if (alive) {
+            and_block(acc, head.v, 1, false);  // (block 0 starts with the header and is never of the second kind)
+            // stop as soon as the clause is false at every node slot of the tile
+            if (nb > 1 && __ballot(any_bit(acc)) != 0) {
+                // entries past the first chunk, 16 at a time, requested one step before they are needed
+                const Chunk16 *tp = reinterpret_cast<const Chunk16 *>(list) + 2;
+                Chunk16 tail = *tp;
+                and_block(acc, head.v + 8, 0, 1 >= plain);
+                if (nb > 2 && __ballot(any_bit(acc)) != 0) {
+                    and_block(acc, head.v + 16, 0, 2 >= plain);
+                    if (nb > 3 && __ballot(any_bit(acc)) != 0) {
+                        and_block(acc, head.v + 24, 0, 3 >= plain);
+                        for (int j = 4; j < nb && __ballot(any_bit(acc)) != 0; j += 2) {
+                            const Chunk16 ahead = *++tp;
+                            and_block(acc, tail.v, 0, j >= plain);
+                            if (j + 1 < nb && __ballot(any_bit(acc)) != 0) and_block(acc, tail.v + 8, 0, j + 1 >= plain);
+                            tail = ahead;
+                        }
+                    }
+                }
+            }
+        }
+        finish(acc, alive, my_weight, weights_of_clause, truth_in, truth_out);
+    };
+
+    // The same for a message layer with the clause's list in this wave's LDS.  A list that comes in by scalar loads
+    // is waited for with the counter that the row reads from LDS use as well, and scalar loads return in no fixed
+    // order: every wait for a row would also wait for the chunk of the list requested ahead, so nothing is hidden.
+    // Here lane l brings entries l, 64 + l, ... of the lists of 8 clauses along with their truth rows (vector loads,
+    // a counter of their own), a clause's entries are put into LDS when its turn comes, and the walk reads them back
+    // a block ahead of the rows (LDS returns in order): the four lanes of every quad read entries 0..3 and 4..7 of
+    // the block, and entry i reaches all lanes inside the add that forms the row's address (quad broadcast).
+    constexpr int LIST_REGS = TILE_LIST_ENTRIES / 64;
+    uint32_t *my_list = lds + (size_t)n_rows_lds * tw + TILE_LDS_PAD_WORDS + (size_t)tg.gpt * K + wave * TILE_LIST_LDS_WORDS;
+    auto evaluate_listed = [&](const uint32_t (&entries)[LIST_REGS], int plain, int nb, const int32_t *weights_of_clause,
+                               const LaneWords<LW> &truth_in, char *truth_out) {
+        const int my_weight = pair_lane ? weights_of_clause[my_k] : 0;
+        const uint32_t ones_entry = (uint32_t)a.M * (uint32_t)tw * 4u;  // in the place of the header
+#pragma unroll
+        for (int k = 0; k < LIST_REGS; ++k)
+            if (k * 64 < nb * 8) my_list[k * 64 + lane] = k == 0 && lane == 0 ? ones_entry : entries[k];
+        LaneWords<LW> acc = truth_in;
+        bool alive = true;
+        const uint32_t *quad_entry = my_list + (lane & 3);
+        uint32_t lo = quad_entry[0], hi = quad_entry[4];
+        for (int b = 0; b < nb && alive; ++b) {
+            const uint32_t next_lo = quad_entry[8 * (b + 1)], next_hi = quad_entry[8 * (b + 1) + 4];
+            const uint32_t e[8] = {
+                (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0x00, 0xF, 0xF, true), (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0x55, 0xF, 0xF, true),
+                (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0xAA, 0xF, 0xF, true), (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0xFF, 0xF, 0xF, true),
+                (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0x00, 0xF, 0xF, true), (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0x55, 0xF, 0xF, true),
+                (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0xAA, 0xF, 0xF, true), (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0xFF, 0xF, 0xF, true)};
+            and_block(acc, e, 0, b >= plain);
+            alive = __ballot(any_bit(acc)) != 0;
+            lo = next_lo;
+            hi = next_hi;
+        }
+        finish(acc, true, my_weight, weights_of_clause, truth_in, truth_out);
+    };
+
     if (SRC == ROWS_MESSAGES) {
         // Message layers: most clauses are already false at every node slot of the tile.  A wave
         // reads the truth rows of 8 of its clauses at once and fetches the list of, and evaluates,
@@ -1054,21 +1121,37 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
         constexpr int GROUP = 8;
         for (int c0 = wave; c0 < C; c0 += GROUP * NWAVES) {
             LaneWords<LW> t[GROUP];
+            uint32_t entries[GROUP][LIST_REGS];
 #pragma unroll
             for (int g = 0; g < GROUP; ++g) {
                 const int c = c0 + g * NWAVES;
 #pragma unroll
                 for (int u = 0; u < LW; ++u) t[g].w[u] = 0u;
                 if (c < C && active) t[g].load(reinterpret_cast<const char *>(bitmap + (int64_t)c * tw + lane * LW));
+#pragma unroll
+                for (int k = 0; k < LIST_REGS; ++k) {
+                    entries[g][k] = 0u;
+                    if (a.lists_in_lds && c < C && k * 64 + lane < a.stride)
+                        entries[g][k] = a.lists[(int64_t)c * a.stride + k * 64 + lane];
+                }
             }
 #pragma unroll
             for (int g = 0; g < GROUP; ++g) {
                 const int c = c0 + g * NWAVES;
                 if (c < C && __ballot(any_bit(t[g])) != 0) {
                     const uint32_t *list = a.lists + (int64_t)c * a.stride;
+                    const int32_t *weights_of_clause = LAST ? a.wt + (int64_t)c * K : nullptr;
+                    char *truth_out = reinterpret_cast<char *>(bitmap + (int64_t)c * tw + (active ? lane * LW : 0));
+                    if (a.lists_in_lds) {
+                        const uint32_t header = (uint32_t)__builtin_amdgcn_readlane((int)entries[g][0], 0);
+                        const int plain = (int)(header & 0xFFFFu), nb = plain + (int)(header >> 16);
+                        if (nb * 8 <= TILE_LIST_ENTRIES) {
+                            evaluate_listed(entries[g], plain, nb, weights_of_clause, t[g], truth_out);
+                            continue;
+                        }
+                    }
                     const Chunk32 head = *reinterpret_cast<const Chunk32 *>(list);
-                    evaluate(head, list, LAST ? a.wt + (int64_t)c * K : nullptr, t[g],
-                             reinterpret_cast<char *>(bitmap + (int64_t)c * tw + (active ? lane * LW : 0)));
+                    evaluate(head, list, weights_of_clause, t[g], truth_out);
                 }
             }
         }
