@@ -387,9 +387,9 @@ struct TileLayerArgs {
 };
 
 // A wave of k_tile_layer keeps the list of the clause it evaluates in LDS when it has at most this many entries
-// (+ 8 words that the walk reads ahead).
+// (+ 32 words that the walk reads ahead).
 constexpr int TILE_LIST_ENTRIES = 256;
-constexpr int TILE_LIST_LDS_WORDS = TILE_LIST_ENTRIES + 8;
+constexpr int TILE_LIST_LDS_WORDS = TILE_LIST_ENTRIES + 32;
 
 // Rows a message layer keeps in LDS: M message rows, the all-ones row, the row of graphs without nodes.
 inline int tile_message_rows(int M) { return M + 2; }
@@ -1098,19 +1098,52 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
         LaneWords<LW> acc = truth_in;
         bool alive = true;
         const uint32_t *quad_entry = my_list + (lane & 3);
-        uint32_t lo = quad_entry[0], hi = quad_entry[4];
-        for (int b = 0; b < nb && alive; ++b) {
-            const uint32_t next_lo = quad_entry[8 * (b + 1)], next_hi = quad_entry[8 * (b + 1) + 4];
-            const uint32_t e[8] = {
-                (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0x00, 0xF, 0xF, true), (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0x55, 0xF, 0xF, true),
-                (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0xAA, 0xF, 0xF, true), (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0xFF, 0xF, 0xF, true),
-                (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0x00, 0xF, 0xF, true), (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0x55, 0xF, 0xF, true),
-                (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0xAA, 0xF, 0xF, true), (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0xFF, 0xF, 0xF, true)};
-            and_block(acc, e, 0, b >= plain);
-            alive = __ballot(any_bit(acc)) != 0;
-            lo = next_lo;
-            hi = next_hi;
-        }
+        auto block_of = [&](uint32_t lo, uint32_t hi, uint32_t (&e)[8]) {
+            e[0] = (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0x00, 0xF, 0xF, true);
+            e[1] = (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0x55, 0xF, 0xF, true);
+            e[2] = (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0xAA, 0xF, 0xF, true);
+            e[3] = (uint32_t)__builtin_amdgcn_mov_dpp((int)lo, 0xFF, 0xF, 0xF, true);
+            e[4] = (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0x00, 0xF, 0xF, true);
+            e[5] = (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0x55, 0xF, 0xF, true);
+            e[6] = (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0xAA, 0xF, 0xF, true);
+            e[7] = (uint32_t)__builtin_amdgcn_mov_dpp((int)hi, 0xFF, 0xF, 0xF, true);
+        };
+        // blocks [from, to), all of one kind, two at a time (16 rows in flight, one test for an all-zero row)
+        auto walk = [&](int from, int to, bool complements) {
+            int b = from;
+            uint32_t lo0 = quad_entry[8 * b], hi0 = quad_entry[8 * b + 4];
+            uint32_t lo1 = quad_entry[8 * b + 8], hi1 = quad_entry[8 * b + 12];
+            for (; b + 1 < to && alive; b += 2) {
+                const uint32_t n_lo0 = quad_entry[8 * b + 16], n_hi0 = quad_entry[8 * b + 20];
+                const uint32_t n_lo1 = quad_entry[8 * b + 24], n_hi1 = quad_entry[8 * b + 28];
+                uint32_t e0[8], e1[8];
+                block_of(lo0, hi0, e0);
+                block_of(lo1, hi1, e1);
+                LaneWords<LW> r[16];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    r[i].load(col + e0[i]);
+                    r[8 + i].load(col + e1[i]);
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+#pragma unroll
+                    for (int u = 0; u < LW; ++u) acc.w[u] &= complements ? ~r[i].w[u] : r[i].w[u];
+                alive = __ballot(any_bit(acc)) != 0;
+                lo0 = n_lo0;
+                hi0 = n_hi0;
+                lo1 = n_lo1;
+                hi1 = n_hi1;
+            }
+            if (b < to && alive) {  // an odd block at the end
+                uint32_t e0[8];
+                block_of(lo0, hi0, e0);
+                and_block(acc, e0, 0, complements);
+                alive = __ballot(any_bit(acc)) != 0;
+            }
+        };
+        walk(0, plain, false);
+        if (alive && nb > plain) walk(plain, nb, true);
         finish(acc, true, my_weight, weights_of_clause, truth_in, truth_out);
     };
 
