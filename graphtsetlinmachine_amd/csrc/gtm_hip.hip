@@ -587,6 +587,7 @@ struct ScoreWs {
     int list_stride;
     uint32_t *message_lists;  // [depth-1][C][message_list_stride]  (tile path, depth > 1)
     int message_list_stride;
+    uint32_t *longest_list;   // [depth-1] entries of each message bank's longest compiled list
     uint32_t *tile_bitmap;    // [tiles per launch][C][tw]  (tile path, depth > 1)
     uint32_t *sent, *got;     // [tiles per launch][tw * 32 node slots][ceil(M / 32)]  (tile path, depth > 1)
     uint32_t *message_rows;   // [tiles per launch][M + 2][tw]  (tile path, depth > 1)
@@ -633,6 +634,7 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base,
     if (tg) {
         w.message_list_stride = clause_list_stride(2 * d.M);
         w.message_lists = (uint32_t *)take((size_t)(cfg->depth - 1) * d.C * w.message_list_stride * 4);
+        w.longest_list = (uint32_t *)take((size_t)(cfg->depth - 1) * 4);
         const size_t n_tiles = tiles_per_batch(*tg, batch);
         w.tile_bitmap = (uint32_t *)take(n_tiles * d.C * tg->tw * 4);
         w.vector_words = n_tiles * tg->tw * 32 * ((d.M + 31) / 32);
@@ -1099,12 +1101,16 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                            d.LA, d.B, d.filter, cfg->literals, 0, g->number_of_node_types, cfg->literals, tg.rows - 1,
                            tg.tw, w.list_stride, order, w.lists, d.K, layers == 1 ? s->clause_weights : nullptr, w.wt);
     if (int rc = check_launch("compile_clauses")) return rc;
+    if (layers > 1) {
+        hipLaunchKernelGGL(k_fill_i32, dim3(1), dim3(TPB), 0, st, (int32_t *)w.longest_list, (int64_t)(layers - 1), 0);
+        if (int rc = check_launch("fill")) return rc;
+    }
     for (int l = 1; l < layers; ++l) {
         hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st,
                            s->message_ta_state[l - 1], d.C, d.MC, d.B, d.mfilter, 2 * d.M, d.M, 0, 0, d.M, tg.tw,
                            w.message_list_stride, (const uint32_t *)nullptr,
                            w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride, d.K,
-                           l == layers - 1 ? s->clause_weights : nullptr, w.wt);
+                           l == layers - 1 ? s->clause_weights : nullptr, w.wt, w.longest_list + (l - 1));
         if (int rc = check_launch("compile_clauses")) return rc;
     }
     TileLayerArgs a{};
@@ -1194,6 +1200,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                 profile_stop(st);
                 a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
                 a.stride = w.message_list_stride;
+                a.longest_list = w.longest_list + (l - 1);
                 if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1 && !tr, st)) return rc;
                 continue;
             }
@@ -1228,6 +1235,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             profile_stop(st);
             a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
             a.stride = w.message_list_stride;
+            a.longest_list = w.longest_list + (l - 1);
             if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1 && !tr, st)) return rc;
         }
         if (tr) {

@@ -263,7 +263,8 @@ __global__ void k_row_order(const unsigned long long *__restrict__ row_count, in
 __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int chunks, int B, uint32_t filter,
                                   int literals, int half, int n_types, int type_base_row, int ones_row, int tw,
                                   int stride, const uint32_t *__restrict__ order, uint32_t *__restrict__ lists, int K,
-                                  const int32_t *__restrict__ weights, int32_t *__restrict__ wt) {
+                                  const int32_t *__restrict__ weights, int32_t *__restrict__ wt,
+                                  uint32_t *__restrict__ longest = nullptr) {
     const int lane = threadIdx.x & 63;
     const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (c >= C) return;
@@ -315,6 +316,7 @@ __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int 
     for (int i = padded + lane; i < fill_to; i += 64) list[i] = ones;
     // entry 0: blocks of rows to AND | blocks of rows whose complements to AND << 16
     if (lane == 0) list[0] = (uint32_t)(plain_padded >> 3) | ((uint32_t)(neg_padded >> 3) << 16);
+    if (longest && lane == 0) atomicMax(longest, (uint32_t)padded);  // entries of the longest list (cleared by the caller)
     if (weights)
         for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
 }
@@ -384,6 +386,7 @@ struct TileLayerArgs {
     const uint32_t *message_rows;  // [tiles of the launch][M + 2][tw] (message layers, built by k_tile_pack_messages)
     const uint32_t *xpos;   // [tiles][tw * 32 slots][LA / 2]: the positive literal words by node slot (half tiles)
     int lists_in_lds;       // message layers: LDS holds TILE_LIST_LDS_WORDS more words per wave for the clause lists
+    const uint32_t *longest_list;  // entries of the layer's longest list (message layers)
 };
 
 // A wave of k_tile_layer keeps the list of the clause it evaluates in LDS when it has at most this many entries
@@ -1087,6 +1090,8 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
     // a block ahead of the rows (LDS returns in order): the four lanes of every quad read entries 0..3 and 4..7 of
     // the block, and entry i reaches all lanes inside the add that forms the row's address (quad broadcast).
     constexpr int LIST_REGS = TILE_LIST_ENTRIES / 64;
+    // (the registers that the layer's longest list needs are requested for every clause, alive or not)
+    const int list_regs = SRC == ROWS_MESSAGES && a.lists_in_lds ? (int)((*a.longest_list + 63u) >> 6) : 0;
     uint32_t *my_list = lds + (size_t)n_rows_lds * tw + TILE_LDS_PAD_WORDS + (size_t)tg.gpt * K + wave * TILE_LIST_LDS_WORDS;
     auto evaluate_listed = [&](const uint32_t (&entries)[LIST_REGS], int plain, int nb, const int32_t *weights_of_clause,
                                const LaneWords<LW> &truth_in, char *truth_out) {
@@ -1164,27 +1169,54 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
 #pragma unroll
                 for (int k = 0; k < LIST_REGS; ++k) {
                     entries[g][k] = 0u;
-                    if (a.lists_in_lds && c < C && k * 64 + lane < a.stride)
+                    if (k < list_regs && c < C && k * 64 + lane < a.stride)
                         entries[g][k] = a.lists[(int64_t)c * a.stride + k * 64 + lane];
                 }
             }
-#pragma unroll
-            for (int g = 0; g < GROUP; ++g) {
-                const int c = c0 + g * NWAVES;
-                if (c < C && __ballot(any_bit(t[g])) != 0) {
-                    const uint32_t *list = a.lists + (int64_t)c * a.stride;
-                    const int32_t *weights_of_clause = LAST ? a.wt + (int64_t)c * K : nullptr;
-                    char *truth_out = reinterpret_cast<char *>(bitmap + (int64_t)c * tw + (active ? lane * LW : 0));
-                    if (a.lists_in_lds) {
-                        const uint32_t header = (uint32_t)__builtin_amdgcn_readlane((int)entries[g][0], 0);
-                        const int plain = (int)(header & 0xFFFFu), nb = plain + (int)(header >> 16);
-                        if (nb * 8 <= TILE_LIST_ENTRIES) {
-                            evaluate_listed(entries[g], plain, nb, weights_of_clause, t[g], truth_out);
-                            continue;
-                        }
+            auto one_clause = [&](int c, const LaneWords<LW> &truth_in, const uint32_t (&mine)[LIST_REGS]) {
+                const uint32_t *list = a.lists + (int64_t)c * a.stride;
+                const int32_t *weights_of_clause = LAST ? a.wt + (int64_t)c * K : nullptr;
+                char *truth_out = reinterpret_cast<char *>(bitmap + (int64_t)c * tw + (active ? lane * LW : 0));
+                if (a.lists_in_lds) {
+                    const uint32_t header = (uint32_t)__builtin_amdgcn_readlane((int)mine[0], 0);
+                    const int plain = (int)(header & 0xFFFFu), nb = plain + (int)(header >> 16);
+                    if (nb * 8 <= TILE_LIST_ENTRIES) {
+                        evaluate_listed(mine, plain, nb, weights_of_clause, truth_in, truth_out);
+                        return;
                     }
-                    const Chunk32 head = *reinterpret_cast<const Chunk32 *>(list);
-                    evaluate(head, list, weights_of_clause, t[g], truth_out);
+                }
+                const Chunk32 head = *reinterpret_cast<const Chunk32 *>(list);
+                evaluate(head, list, weights_of_clause, truth_in, truth_out);
+            };
+            if (LAST) {
+                // (with the scoring in it the evaluation is long: one copy in the instruction cache, the clause's
+                // registers picked out of the 8, measured faster than 8 copies; without it the other way round)
+#pragma unroll 1
+                for (int g = 0; g < GROUP; ++g) {
+                    const int c = c0 + g * NWAVES;
+                    LaneWords<LW> truth_in = t[0];
+#pragma unroll
+                    for (int h = 1; h < GROUP; ++h)
+                        if (g == h) truth_in = t[h];
+                    if (c < C && __ballot(any_bit(truth_in)) != 0) {
+                        uint32_t mine[LIST_REGS];
+#pragma unroll
+                        for (int k = 0; k < LIST_REGS; ++k) mine[k] = entries[0][k];
+#pragma unroll
+                        for (int h = 1; h < GROUP; ++h) {
+                            if (g == h) {
+#pragma unroll
+                                for (int k = 0; k < LIST_REGS; ++k) mine[k] = entries[h][k];
+                            }
+                        }
+                        one_clause(c, truth_in, mine);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int g = 0; g < GROUP; ++g) {
+                    const int c = c0 + g * NWAVES;
+                    if (c < C && __ballot(any_bit(t[g])) != 0) one_clause(c, t[g], entries[g]);
                 }
             }
         }
