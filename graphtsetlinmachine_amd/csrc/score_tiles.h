@@ -1191,26 +1191,26 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
             if (LAST) {
                 // (with the scoring in it the evaluation is long: one copy in the instruction cache, the clause's
                 // registers picked out of the 8, measured faster than 8 copies; without it the other way round)
+                uint32_t alive_of_8 = 0u;  // (a clause that is false everywhere costs no more than this test)
+#pragma unroll
+                for (int g = 0; g < GROUP; ++g)
+                    if (c0 + g * NWAVES < C && __ballot(any_bit(t[g])) != 0) alive_of_8 |= 1u << g;
 #pragma unroll 1
-                for (int g = 0; g < GROUP; ++g) {
-                    const int c = c0 + g * NWAVES;
+                for (; alive_of_8 != 0u; alive_of_8 &= alive_of_8 - 1u) {
+                    const int g = __builtin_ctz(alive_of_8);
                     LaneWords<LW> truth_in = t[0];
+                    uint32_t mine[LIST_REGS];
 #pragma unroll
-                    for (int h = 1; h < GROUP; ++h)
-                        if (g == h) truth_in = t[h];
-                    if (c < C && __ballot(any_bit(truth_in)) != 0) {
-                        uint32_t mine[LIST_REGS];
+                    for (int k = 0; k < LIST_REGS; ++k) mine[k] = entries[0][k];
 #pragma unroll
-                        for (int k = 0; k < LIST_REGS; ++k) mine[k] = entries[0][k];
+                    for (int h = 1; h < GROUP; ++h) {
+                        if (g == h) {
+                            truth_in = t[h];
 #pragma unroll
-                        for (int h = 1; h < GROUP; ++h) {
-                            if (g == h) {
-#pragma unroll
-                                for (int k = 0; k < LIST_REGS; ++k) mine[k] = entries[h][k];
-                            }
+                            for (int k = 0; k < LIST_REGS; ++k) mine[k] = entries[h][k];
                         }
-                        one_clause(c, truth_in, mine);
                     }
+                    one_clause(c0 + g * NWAVES, truth_in, mine);
                 }
             } else {
 #pragma unroll
