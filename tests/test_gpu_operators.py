@@ -318,16 +318,21 @@ DEEP_TILE_SHAPES = [
 
 
 @pytest.mark.parametrize("shape", DEEP_TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
-@pytest.mark.parametrize("message_density", [0.0, 0.01, 0.1])
-@pytest.mark.parametrize("messages", ["graph-per-workgroup", "three-launches", "three-launches-atomics"])
+@pytest.mark.parametrize("message_density", [0.0, 0.01, 0.1, 0.6])
+@pytest.mark.parametrize("messages", ["graph-per-workgroup", "graph-per-workgroup-lists-by-scalar-loads",
+                                      "three-launches", "three-launches-atomics"])
 def test_tile_scoring_with_message_layers(shape, message_density, messages, monkeypatch):
     """gtm_score with message layers on literal-major tiles == oracle == the bitmap path, with the
     message rows built by one workgroup per graph (where the shape allows) and by the three
-    launches that keep the vectors in global memory."""
+    launches that keep the vectors in global memory.  The clause lists of the message layers reach the
+    evaluating waves through LDS (lists of up to 256 entries: at density 0.6 the larger message sizes
+    have longer ones, which take scalar loads) or, switched off, all by scalar loads."""
     from tests.gpu_harness import Device
 
-    if messages != "graph-per-workgroup":
+    if not messages.startswith("graph-per-workgroup"):
         monkeypatch.setenv("GTM_NO_FUSED_MESSAGES", "1")
+    if messages == "graph-per-workgroup-lists-by-scalar-loads":
+        monkeypatch.setenv("GTM_NO_LISTS_IN_LDS", "1")
     if messages == "three-launches-atomics":
         monkeypatch.setenv("GTM_NODE_MESSAGES_BY_ATOMICS", "1")
 
