@@ -1157,22 +1157,35 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
         // reads the truth rows of 8 of its clauses at once and fetches the list of, and evaluates,
         // only those that are still true somewhere.
         constexpr int GROUP = 8;
+        // (every lane loads, from an address that is always valid - a clause past the last one repeats the wave's
+        // first, a lane past the row or the list reads its first word - and what must not count is dropped
+        // afterwards: no branch around any load, pointers that step by additions)
+        const int64_t truth_step = (int64_t)NWAVES * tw, list_step = (int64_t)NWAVES * a.stride;
+        const int my_word = active ? lane * LW : 0;
+        int my_entry[LIST_REGS];
+#pragma unroll
+        for (int k = 0; k < LIST_REGS; ++k) my_entry[k] = k * 64 + lane < a.stride ? k * 64 + lane : 0;
         for (int c0 = wave; c0 < C; c0 += GROUP * NWAVES) {
             LaneWords<LW> t[GROUP];
             uint32_t entries[GROUP][LIST_REGS];
+            const uint32_t *truth_of = bitmap + (int64_t)c0 * tw, *list_of = a.lists + (int64_t)c0 * a.stride;
 #pragma unroll
             for (int g = 0; g < GROUP; ++g) {
-                const int c = c0 + g * NWAVES;
-#pragma unroll
-                for (int u = 0; u < LW; ++u) t[g].w[u] = 0u;
-                if (c < C && active) t[g].load(reinterpret_cast<const char *>(bitmap + (int64_t)c * tw + lane * LW));
+                const bool there = c0 + g * NWAVES < C;
+                const uint32_t *truth_row = there ? truth_of + g * truth_step : truth_of;
+                const uint32_t *list = there ? list_of + g * list_step : list_of;
+                t[g].load(reinterpret_cast<const char *>(truth_row + my_word));
 #pragma unroll
                 for (int k = 0; k < LIST_REGS; ++k) {
                     entries[g][k] = 0u;
-                    if (k < list_regs && c < C && k * 64 + lane < a.stride)
-                        entries[g][k] = a.lists[(int64_t)c * a.stride + k * 64 + lane];
+                    if (k < list_regs) entries[g][k] = list[my_entry[k]];
                 }
             }
+#pragma unroll
+            for (int g = 0; g < GROUP; ++g)
+                if (!active || c0 + g * NWAVES >= C)
+#pragma unroll
+                    for (int u = 0; u < LW; ++u) t[g].w[u] = 0u;
             auto one_clause = [&](int c, const LaneWords<LW> &truth_in, const uint32_t (&mine)[LIST_REGS]) {
                 const uint32_t *list = a.lists + (int64_t)c * a.stride;
                 const int32_t *weights_of_clause = LAST ? a.wt + (int64_t)c * K : nullptr;
