@@ -827,6 +827,12 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
             const uint32_t *v = sent + n * MWP + (n >> 5);
             const uint32_t ne = n_edges[row0 + n];
             const uint2 *out_edges = reinterpret_cast<const uint2 *>(edge) + edge_index[row0 + n];
+            // (vectors of at most 16 words are read once, into registers, for all the node's edges)
+            constexpr int IN_REGISTERS = 16;
+            uint32_t mine[IN_REGISTERS];
+#pragma unroll
+            for (int j = 0; j < IN_REGISTERS; ++j) mine[j] = MW <= IN_REGISTERS && j < MW ? v[j] : 0u;
+            const uint32_t last = v[MW - 1];
             for (uint32_t e0 = 0; e0 < ne; e0 += 4) {
                 uint2 pair[4];
 #pragma unroll
@@ -836,12 +842,26 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
                     if (e0 + u >= ne) break;
                     const uint32_t dst = pair[u].x, shift = pair[u].y % (uint32_t)M;
                     const int q = (int)(shift >> 5), r = (int)(shift & 31u);
-                    int a = (int)((MW - q) % MW);  // word of v that feeds word 0
-                    for (int j = 0; j < MW; ++j) {
-                        const int below = a == 0 ? MW - 1 : a - 1;
-                        const uint32_t word = r ? (v[a] << r) | (v[below] >> (32 - r)) : v[a];
-                        if (word) atomicOr(&got[dst * MWP + (dst >> 5) + j], word);
-                        a = a + 1 == MW ? 0 : a + 1;
+                    uint32_t *to = got + dst * MWP + (dst >> 5);
+                    if (MW <= IN_REGISTERS) {
+                        int at = q;  // the word that word 0 of the vector goes to
+#pragma unroll
+                        for (int j = 0; j < IN_REGISTERS; ++j) {
+                            if (j < MW) {
+                                const uint32_t below = j == 0 ? last : mine[j > 0 ? j - 1 : 0];
+                                const uint32_t word = r ? (mine[j] << r) | (below >> (32 - r)) : mine[j];
+                                if (word) atomicOr(&to[at], word);
+                                at = at + 1 == MW ? 0 : at + 1;
+                            }
+                        }
+                    } else {
+                        int a = (int)((MW - q) % MW);  // word of v that feeds word 0
+                        for (int j = 0; j < MW; ++j) {
+                            const int below = a == 0 ? MW - 1 : a - 1;
+                            const uint32_t word = r ? (v[a] << r) | (v[below] >> (32 - r)) : v[a];
+                            if (word) atomicOr(&to[j], word);
+                            a = a + 1 == MW ? 0 : a + 1;
+                        }
                     }
                 }
             }
