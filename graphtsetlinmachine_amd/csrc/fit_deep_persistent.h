@@ -171,7 +171,20 @@ __device__ __forceinline__ bool fitd_wait(const unsigned long long *parts, unsig
 
 // A 32 x 32 bit matrix held one row per lane (both halves of a wave hold one each): afterwards lane b
 // holds column b, i.e. bit k of its word = bit b of what lane k (of the same half) held.
-__device__ __forceinline__ uint32_t fitd_transpose32(uint32_t a, int lane) { return tile_transpose32(a, lane); }
+// (the form with a choice per lane instead of tile_transpose32's per-lane constants: this kernel has no vector
+// registers to spare for them)
+template <int J, uint32_t M>
+__device__ __forceinline__ uint32_t fitd_transpose_step(uint32_t v, int lane) {
+    const uint32_t p = tile_lane_xor<J>(v, lane);
+    return (lane & J) ? ((p >> J) & M) | (v & ~M) : (v & M) | ((p & M) << J);
+}
+__device__ __forceinline__ uint32_t fitd_transpose32(uint32_t a, int lane) {
+    a = fitd_transpose_step<16, 0x0000FFFFu>(a, lane);
+    a = fitd_transpose_step<8, 0x00FF00FFu>(a, lane);
+    a = fitd_transpose_step<4, 0x0F0F0F0Fu>(a, lane);
+    a = fitd_transpose_step<2, 0x33333333u>(a, lane);
+    return fitd_transpose_step<1, 0x55555555u>(a, lane);
+}
 
 // acc &= the rows of the literals that words [w_lo, w_hi) of an include plane hold - and, with `twin` >= 0,
 // words [twin + w_lo, twin + w_hi) as well, in the same pass (the negated halves of a message bank's words; at

@@ -445,9 +445,16 @@ __device__ __forceinline__ uint32_t tile_lane_xor(uint32_t v, int lane) {
 // half-blocks with the lane 16, 8, 4, 2, 1 away.
 template <int J, uint32_t M>
 __device__ __forceinline__ uint32_t tile_transpose_step(uint32_t v, int lane) {
-    // M: the columns whose index has bit J clear
+    // M: the columns whose index has bit J clear.  A lane whose index has bit J clear keeps those columns and takes
+    // the partner's, moved up by J, for the others: (v & M) | ((p & M) << J); a lane with bit J set the other way
+    // round: (v & ~M) | ((p >> J) & M).  Both are (v & keep) | (rotate(p) & ~keep) with a rotation by J to the left
+    // resp. right - what the rotation carries round lands on columns that `keep` covers - so the two kinds of lanes
+    // run the same three instructions (lane exchange, rotate, bit select) on per-lane constants, no branch.
     const uint32_t p = tile_lane_xor<J>(v, lane);
-    return (lane & J) ? ((p >> J) & M) | (v & ~M) : (v & M) | ((p & M) << J);
+    const bool upper = (lane & J) != 0;
+    const uint32_t keep = upper ? ~M : M, left = upper ? 32u - J : (uint32_t)J;
+    const uint32_t turned = __builtin_rotateleft32(p, left);
+    return (v & keep) | (turned & ~keep);
 }
 
 __device__ __forceinline__ uint32_t tile_transpose32(uint32_t v, int lane) {
