@@ -1126,6 +1126,8 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     a.n_nodes = g->number_of_graph_nodes;
     a.X = g->X;
     a.xpos = tg.half ? g->tiles + tiles_xpos_offset_words(tg, cfg->literals) : nullptr;
+    a.walk_factor = 2;
+    if (const char *e = getenv("GTM_WIDE_WALK_FACTOR")) a.walk_factor = std::max(1, atoi(e));  // (tuning aid)
     auto layer0 = [&](int n_tiles, bool last) {
         a.lists = w.lists;
         a.stride = stride0;

@@ -385,6 +385,8 @@ struct TileLayerArgs {
     const uint32_t *X;      // [nodes][LA] node-major literal words (two-phase layer 0)
     const uint32_t *message_rows;  // [tiles of the launch][M + 2][tw] (message layers, built by k_tile_pack_messages)
     const uint32_t *xpos;   // [tiles][tw * 32 slots][LA / 2]: the positive literal words by node slot (half tiles)
+    int walk_factor;        // k_tile_two_phase_wide: a clause's rows are all walked when more than this many slots per
+                            // literal survive phase 1
     int lists_in_lds;       // message layers: LDS holds TILE_LIST_LDS_WORDS more words per wave for the clause lists
     const uint32_t *longest_list;  // entries of the layer's longest list (message layers)
 };
@@ -2213,9 +2215,11 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
         }
         unsigned long long nz = __ballot(any_bit(acc));
         // Phase 2 costs a memory round trip per 8 surviving slots, ANDing the rows of all the clause's
-        // literals one per 8 literals: when more slots survive than the clause has literals (its rarest
-        // literals hold nearly everywhere: negated ones, mostly), the rows are walked instead, as
-        // k_tile_layer does (row l belongs to literal l; unused reads take the all-ones row).
+        // literals one per 8 literals: when more than twice as many slots survive as the clause has literals
+        // (its rarest literals hold nearly everywhere: negated ones, mostly), the rows are walked instead,
+        // as k_tile_layer does (row l belongs to literal l; unused reads take the all-ones row).  (Measured on
+        // the colour workload, 2,000 graphs: the kernel takes 11.2 ms with one slot per literal as the limit,
+        // 10.1 ms with two, 10.5 with four, 11.7 never walking, 13.8 with half a slot.)
         bool walk = false;
         if ((header & 0x100u) && nz != 0) {
             int survivors = 0, literals = __popc(include0);
@@ -2226,7 +2230,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_wide(TileLayerAr
                 survivors += __shfl_xor(survivors, off);
                 literals += __shfl_xor(literals, off);
             }
-            walk = survivors > literals;
+            walk = survivors > literals * a.walk_factor;
         }
         if (walk) {
             const uint32_t row_bytes = (uint32_t)tw * 4u, ones = (uint32_t)(tg.rows - 1);
