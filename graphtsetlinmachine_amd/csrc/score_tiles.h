@@ -934,10 +934,12 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
 // and a clause's truth is its previous truth AND the rows of its included
 // message literals (kernels.py:505-527).
 //
-// A wave owns a clause at a time.  The clause's row list is wave-uniform: its
-// first 32 entries arrive by scalar loads issued while the previous clause is
-// being evaluated.  Lane L holds words [L*LW, (L+1)*LW) of the running AND; after
-// every 8 rows a clause that is false at every node slot of the tile is done.
+// A wave owns a clause at a time.  The clause's row list is wave-uniform: on layer 0
+// its first 32 entries arrive by scalar loads issued while the previous clause is
+// being evaluated; on message layers, whose rows are in LDS, the lists come by
+// vector loads through a few LDS words of the wave's own (see evaluate_listed).
+// Lane L holds words [L*LW, (L+1)*LW) of the running AND; after every 8 (16) rows a
+// clause that is false at every node slot of the tile is done.
 //
 // LAST: the clause's weights are added to the class sums of the graphs where it
 // is true at some node (kernels.py:297-315) and no bitmap is written; otherwise
@@ -1182,9 +1184,9 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_layer(TileLayerArgs a) {
     };
 
     if (SRC == ROWS_MESSAGES) {
-        // Message layers: most clauses are already false at every node slot of the tile.  A wave
-        // reads the truth rows of 8 of its clauses at once and fetches the list of, and evaluates,
-        // only those that are still true somewhere.
+        // Message layers: many clauses are already false at every node slot of the tile.  A wave reads
+        // the truth rows of 8 of its clauses at once, and with them the first entries of their lists,
+        // and evaluates only the clauses that are still true somewhere.
         constexpr int GROUP = 8;
         // (every lane loads, from an address that is always valid - a clause past the last one repeats the wave's
         // first, a lane past the row or the list reads its first word - and what must not count is dropped
