@@ -1209,11 +1209,11 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             profile_start("k_tile_node_messages + k_tile_edge_messages + k_tile_pack_messages", st);
             if (by_bit) {
                 const int pack = tg.tw <= 32 && !getenv("GTM_NO_TILE_PACK") ? 64 / tg.tw : 1;  // narrow tiles share a wave
-                hipLaunchKernelGGL(k_tile_node_messages_by_bit,
-                                   dim3((MW + NODE_MESSAGES_BY_BIT_WAVES - 1) / NODE_MESSAGES_BY_BIT_WAVES,
-                                        (n_tiles + pack - 1) / pack),
+                const int blocks_per_group = (MW + NODE_MESSAGES_BY_BIT_WAVES - 1) / NODE_MESSAGES_BY_BIT_WAVES;
+                const int n_groups = (n_tiles + pack - 1) / pack;
+                hipLaunchKernelGGL(k_tile_node_messages_by_bit, dim3((unsigned)((n_groups + 7) / 8 * 8 * blocks_per_group)),
                                    dim3(64 * NODE_MESSAGES_BY_BIT_WAVES), 0, st, w.tile_bitmap, d.C, tg.tw, w.bit_start,
-                                   w.bit_clauses, d.M, MW, n_tiles, pack, w.sent);
+                                   w.bit_clauses, d.M, MW, n_tiles, pack, blocks_per_group, n_groups, w.sent);
             }
             else
             hipLaunchKernelGGL(k_tile_node_messages, dim3((tg.tw + group - 1) / group, n_tiles),

@@ -541,24 +541,31 @@ __device__ __forceinline__ void message_bit_words(const uint32_t *__restrict__ r
 // rows: for each bit the rows of the bit's clauses are ORed (whole rows, coalesced; the clause
 // numbers come in by one load per bit and are handed round with readlane), the 32 resulting rows
 // are transposed inside each lane, 32 x 32 bits, and the lane stores word j of its 32 slots.
-// grid (ceil(MW / waves per block), ceil(tiles / pack)).  Every word of sent is written (no clearing
+// Every word of sent is written (no clearing
 // needed).  Tiles of at most 32 words are taken `pack` = 64 / tw at a time, lane l on word l % tw of tile
 // l / tw of the group (the clause numbers of a bit are the same for every tile).
 constexpr int NODE_MESSAGES_BY_BIT_WAVES = 4;
 
 __global__ __launch_bounds__(64 * NODE_MESSAGES_BY_BIT_WAVES) void k_tile_node_messages_by_bit(
     const uint32_t *__restrict__ bitmap, int C, int tw, const uint32_t *__restrict__ bit_start,
-    const uint32_t *__restrict__ bit_clauses, int M, int MW, int n_tiles, int pack, uint32_t *__restrict__ sent) {
+    const uint32_t *__restrict__ bit_clauses, int M, int MW, int n_tiles, int pack, int blocks_per_group, int n_groups,
+    uint32_t *__restrict__ sent) {
     __shared__ uint32_t stage_of_wave[NODE_MESSAGES_BY_BIT_WAVES][32][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int j = blockIdx.x * NODE_MESSAGES_BY_BIT_WAVES + wave;
+    // Workgroups go to the 8 XCDs in turn, and each XCD has its own L2: the workgroups of a group of tiles - they read
+    // the same truth rows, each for its own message bits - are given to one XCD, so that the rows come from memory
+    // once and not once per XCD.  1-D grid of ceil(groups / 8) * 8 * blocks_per_group workgroups.
+    const int xcd = blockIdx.x & 7, turn = blockIdx.x >> 3;
+    const int block_of_group = turn % blocks_per_group, group = (turn / blocks_per_group) * 8 + xcd;
+    if (group >= n_groups) return;
+    const int j = block_of_group * NODE_MESSAGES_BY_BIT_WAVES + wave;
     if (j >= MW) return;  // the block has no barrier
     uint32_t(*stage)[64] = stage_of_wave[wave];
     const int sub = pack > 1 ? lane / tw : 0, word_of_lane = pack > 1 ? lane - sub * tw : lane;
-    const int tile = (int)blockIdx.y * pack + sub;
+    const int tile = group * pack + sub;
     const bool tile_exists = sub < pack && tile < n_tiles;
-    const uint32_t *rows = bitmap + (int64_t)(tile_exists ? tile : (int)blockIdx.y * pack) * C * tw;
+    const uint32_t *rows = bitmap + (int64_t)(tile_exists ? tile : group * pack) * C * tw;
     // lane i <= 32 holds where the clauses of bit 32 j + i begin (bits past M: nothing)
     const int p_of_lane = 32 * j + lane < M ? 32 * j + lane : M;
     const uint32_t start_of_lane = lane <= 32 ? bit_start[p_of_lane] : 0u;
