@@ -1230,9 +1230,9 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                                    g->number_of_graph_node_edges, g->edge_index, g->edge, vector_words, w.got);
                 if (int rc = check_launch("tile_edge_messages")) return rc;
             }
-            hipLaunchKernelGGL(k_tile_pack_messages, dim3((tg.tw + 1) / 2, n_tiles), dim3(256),
+            hipLaunchKernelGGL(k_tile_pack_messages, dim3((unsigned)((n_tiles + 7) / 8 * 8 * ((tg.tw + 1) / 2))), dim3(256),
                                (size_t)64 * (MW + 1) * 4, st, w.got, tg, t0, g->number_of_graphs, d.M, MW,
-                               g->number_of_graph_nodes, w.message_rows);
+                               g->number_of_graph_nodes, w.message_rows, (tg.tw + 1) / 2, n_tiles);
             if (int rc = check_launch("tile_pack_messages")) return rc;
             profile_stop(st);
             a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;

@@ -711,10 +711,15 @@ __global__ void k_tile_edge_messages(const uint32_t *__restrict__ sent, TileGeom
 __global__ __launch_bounds__(256) void k_tile_pack_messages(const uint32_t *__restrict__ got, TileGeom tg, int tile0,
                                                              int G, int M, int MW,
                                                              const uint32_t *__restrict__ n_nodes,
-                                                             uint32_t *__restrict__ rows) {
+                                                             uint32_t *__restrict__ rows, int blocks_per_tile, int n_tiles) {
     extern __shared__ uint32_t block[];  // [64 slots][MW + 1]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int nb = blockIdx.x, tile_local = blockIdx.y;
+    // (the workgroups of a tile write neighbouring words of the same rows: they are given to one XCD - workgroups go to
+    // the 8 XCDs in turn - so that the words meet in one L2 before they go to memory.  1-D grid of
+    // ceil(tiles / 8) * 8 * blocks_per_tile workgroups.)
+    const int xcd = blockIdx.x & 7, turn = blockIdx.x >> 3;
+    const int nb = turn % blocks_per_tile, tile_local = (turn / blocks_per_tile) * 8 + xcd;
+    if (tile_local >= n_tiles) return;
     const int tw = tg.tw, slots = tw * 32;
     const int n_here = min(64, slots - nb * 64);
     const uint32_t *src = got + ((int64_t)tile_local * slots + nb * 64) * MW;
