@@ -107,12 +107,14 @@ def short_run(name, n_train, n_test, check_graphs):
     tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
     torch.cuda.synchronize()
     t_train = time.perf_counter() - t0
+    passes = 5  # (a pass over these test sets takes a millisecond or less: one call alone would time the call, not the GPU)
     tm.score_device(wl.graphs_test)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    sums = tm.score_device(wl.graphs_test)
+    for _ in range(passes):
+        sums = tm.score_device(wl.graphs_test)
     torch.cuda.synchronize()
-    t_test = time.perf_counter() - t0
+    t_test = (time.perf_counter() - t0) / passes
     sums = sums.cpu().numpy().reshape(n_test, -1)
     model = oracle_twin(tm, int(wl.graphs_test.max_number_of_graph_nodes))
     want = o.score(model, wl.graphs_test, range(check_graphs))
