@@ -93,6 +93,9 @@ PROTOTYPES = {
     "gtm_get_hyperliterals": (C.c_int, [_CFG, _P, _I, _I, _P, _P]),
     "gtm_transform_workspace_bytes": (_SZ, [_CFG, _GR, _I]),
     "gtm_transform": (C.c_int, [_CFG, _GR, _ST, _I, _I, _I, _P, _SZ, _P, _P, _I, _P, _P]),
+    "gtm_tuning_set": (C.c_int, [C.c_char_p, C.c_char_p]),
+    "gtm_tuning_get": (C.c_char_p, [C.c_char_p]),
+    "gtm_tuning_reload": (C.c_int, []),
     "gtm_profile_enable": (C.c_int, [C.c_int]),
     "gtm_profile_read": (C.c_int, [C.POINTER(C.c_char_p), C.POINTER(C.c_int32), C.POINTER(C.c_double)]),
     "gtm_profile_read_kernel": (C.c_int, [C.c_int32, C.POINTER(C.c_char_p), C.POINTER(C.c_int32), C.POINTER(C.c_double)]),
@@ -140,6 +143,12 @@ def call(name, *args):
     rc = getattr(lib, name)(*args)
     if rc != 0:
         raise GtmError("%s failed (%d): %s" % (name, rc, lib.gtm_last_error().decode("utf-8", "replace")))
+
+
+def tuning(name):
+    """Value of one of the library's GTM_* switches as the library holds it (None = not set)."""
+    v = lib.gtm_tuning_get(name.encode())
+    return None if v is None else v.decode()
 
 
 def make_config(

@@ -92,6 +92,7 @@ struct FitDeepParams {
     unsigned long long *class_sum;  // [3][K][FITP_SUM_PARTS] words FITP_SUM_STRIDE apart
     uint32_t *abort_flag;
     uint32_t spin_limit;
+    unsigned long long wait_ticks;
     int force_abort;
     int clauses_per_group;
     int NW;          // words of a row over the nodes of the largest graph
@@ -147,12 +148,14 @@ __device__ __forceinline__ uint32_t fitd_load(const uint32_t *p) {
 
 // Wave 0 of a workgroup waits until the counter (the sum of its parts) has reached `target`.
 __device__ __forceinline__ bool fitd_wait(const unsigned long long *parts, unsigned long long target,
-                                          uint32_t *abort_flag, uint32_t spin_limit, int force_abort, int lane) {
+                                          uint32_t *abort_flag, uint32_t spin_limit, unsigned long long wait_ticks,
+                                          int force_abort, int lane) {
     if (force_abort) {
         __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return false;
     }
     uint32_t polls = 0;
+    unsigned long long waiting_since = 0ull;
     for (;;) {
         unsigned long long v = lane < FITD_PARTS
                                    ? __hip_atomic_load(&parts[lane * FITD_STRIDE], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
@@ -161,7 +164,8 @@ __device__ __forceinline__ bool fitd_wait(const unsigned long long *parts, unsig
         for (int off = 1; off < FITD_PARTS; off <<= 1) v += __shfl_xor(v, off);
         v = __shfl(v, 0);
         if (v >= target) return true;
-        if (__hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 || ++polls > spin_limit) {
+        if (__hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
+            fit_wait_is_over(polls, spin_limit, waiting_since, wait_ticks)) {
             __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             return false;
         }
@@ -477,7 +481,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
             if (tid == 0)
                 __hip_atomic_fetch_add(&arrived[(g % FITD_PARTS) * FITD_STRIDE], 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (wave == 0) {
-                const bool ok = fitd_wait(arrived, everyone, p.abort_flag, p.spin_limit, p.force_abort, lane);
+                const bool ok = fitd_wait(arrived, everyone, p.abort_flag, p.spin_limit, p.wait_ticks, p.force_abort, lane);
                 if (lane == 0) go_on = ok ? 1 : 0;
             } else {
                 // (meanwhile) this group's share of the slot the next example will send into; the next
@@ -625,6 +629,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
             uint32_t *seen_slot = seen + (size_t)slot * 2 * K;
             const unsigned long long seen_own = ((unsigned long long)seen_slot[K + k] << 32) | seen_slot[k];
             uint32_t polls = 0;
+            unsigned long long waiting_since = 0ull;
             unsigned long long word = 0ull;
             bool ok = !p.force_abort;
             if (!ok) __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -636,7 +641,8 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                                              __HIP_MEMORY_SCOPE_AGENT);
                 word = all;
                 if ((((word - seen_own + FITP_HALF) >> 48) & 0xFFFFull) == everyone) break;
-                if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 || ++polls > p.spin_limit) {
+                if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
+                    fit_wait_is_over(polls, p.spin_limit, waiting_since, p.wait_ticks)) {
                     __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     ok = false;
                     break;

@@ -36,6 +36,22 @@
 
 constexpr int FITP_BLOCK = 1024;  // 16 waves: one clause per wave in flight, four waves per SIMD hide each other's latencies
 
+// A device-wide wait gives up after `spin_limit` polls or `wait_ticks` ticks of the wall clock (constant
+// rate, whatever the shader clock does), whichever comes first.  The clock is a memory instruction of its
+// own, so it is only looked at every 256th poll: an ordinary wait (a few polls) never reads it.
+__device__ __forceinline__ bool fit_wait_is_over(uint32_t &polls, uint32_t spin_limit, unsigned long long &since,
+                                                 unsigned long long wait_ticks) {
+    if (++polls > spin_limit) return true;
+    if ((polls & 255u) == 0u) {
+        const unsigned long long now = wall_clock64();
+        if (since == 0ull)
+            since = now;
+        else if (now - since > wait_ticks)
+            return true;
+    }
+    return false;
+}
+
 struct FitPersistParams {
     // data set
     const uint32_t *tiles;
@@ -55,7 +71,8 @@ struct FitPersistParams {
     // coordination
     unsigned long long *class_sum;  // [3][K][FITP_SUM_PARTS] words FITP_SUM_STRIDE apart, zero on entry (K <= FITP_BLOCK)
     uint32_t *abort_flag;           // [1], zero on entry
-    uint32_t spin_limit;
+    uint32_t spin_limit;  // polls after which a wait gives up (tests; 2^32 - 1 otherwise: the clock bounds the wait)
+    unsigned long long wait_ticks;  // ticks of the device's wall clock after which a wait gives up
     int force_abort;      // give up at the first wait without looking (exercises the drain path)
     int clauses_per_group;
     int rows_words;       // LDS words of one staged graph: (literals + n_types + 1) * max slot words
@@ -466,6 +483,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             uint32_t *seen_slot = seen + (size_t)(i % 3) * 2 * K;
             const unsigned long long seen_own = ((unsigned long long)seen_slot[K + k] << 32) | seen_slot[k];
             uint32_t polls = 0;
+            unsigned long long waiting_since = 0ull;
             unsigned long long word = 0ull;
             bool ok = !p.force_abort;
             if (!ok) __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -473,7 +491,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 word = read_sum(slot_now, k);
                 if (arrivals(word, seen_own) == everyone) break;
                 if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
-                    ++polls > p.spin_limit) {
+                    fit_wait_is_over(polls, p.spin_limit, waiting_since, p.wait_ticks)) {
                     __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     ok = false;
                     break;

@@ -47,6 +47,63 @@ int check_launch(const char *what) {
     return GTM_OK;
 }
 
+// ------------------------------------------------------------------ switches
+// Tuning and test aids.  The process environment is read ONCE, when the library is loaded; the
+// entry points then only look at this table.  gtm_tuning_set / gtm_tuning_reload (tests, tuning
+// runs) change it, and must not run while another call of the library is under way.
+#define GTM_SWITCHES(X) \
+    X(FIT_DEEP_CLAUSES_PER_GROUP) \
+    X(FIT_DEEP_IN_MEMORY) \
+    X(FIT_DEEP_NO_MASKS) \
+    X(FIT_DEEP_WINDOW_ROWS) \
+    X(FIT_FACTOR_MIN) \
+    X(FIT_PER_GROUP) \
+    X(FIT_SPIN_LIMIT) \
+    X(HALF_LANE_WORDS) \
+    X(NODE_MESSAGES_BY_ATOMICS) \
+    X(NO_DEEP_FIT) \
+    X(NO_DEEP_PERSISTENT_FIT) \
+    X(NO_DIRECT_FIT) \
+    X(NO_FUSED_MESSAGES) \
+    X(NO_HALF_TILES) \
+    X(NO_LISTS_IN_LDS) \
+    X(NO_NARROW_TWO_PHASE) \
+    X(NO_PERSISTENT_FIT) \
+    X(NO_SMALL_FIT) \
+    X(NO_TILE_PACK) \
+    X(NO_TILE_TRANSFORM) \
+    X(NO_TWO_PHASE) \
+    X(TILE_LANE_WORDS) \
+    X(WIDE_SPLITS) \
+    X(WIDE_WALK_FACTOR)
+
+enum Switch {
+#define X(name) T_##name,
+    GTM_SWITCHES(X)
+#undef X
+    T_COUNT
+};
+const char *const g_switch_name[T_COUNT] = {
+#define X(name) "GTM_" #name,
+    GTM_SWITCHES(X)
+#undef X
+};
+struct Switches {
+    bool set[T_COUNT];
+    char value[T_COUNT][24];
+    void put(int i, const char *v) {
+        set[i] = v != nullptr;
+        snprintf(value[i], sizeof value[i], "%s", v ? v : "");
+    }
+    Switches() {
+        for (int i = 0; i < T_COUNT; ++i) put(i, getenv(g_switch_name[i]));
+    }
+};
+Switches g_switches;  // filled from the environment when the library is loaded
+
+// The switch's value, or NULL when it is not set (what getenv gave when this was read per call).
+inline const char *tune(Switch which) { return g_switches.set[which] ? g_switches.value[which] : nullptr; }
+
 // --------------------------------------------------------------- profiling
 // When enabled (gtm_profile_enable), the launches of the kernels that do the work of a
 // driver loop are bracketed by HIP events on the caller's stream, each under its kernel's name.
@@ -61,8 +118,12 @@ struct Profile {
 };
 Profile g_prof;
 
+// Set for the duration of a call that must create no events (gtm_score_static): per thread, so that
+// other threads' calls and the global switch are left alone.
+thread_local bool g_prof_quiet = false;
+
 void profile_start(const char *name, hipStream_t st) {
-    if (!g_prof.on || g_prof.used >= Profile::MAX) return;
+    if (!g_prof.on || g_prof_quiet || g_prof.used >= Profile::MAX) return;
     if (g_prof.used >= g_prof.created) {
         if (hipEventCreate(&g_prof.start[g_prof.created]) != hipSuccess) return;
         if (hipEventCreate(&g_prof.stop[g_prof.created]) != hipSuccess) {
@@ -77,7 +138,7 @@ void profile_start(const char *name, hipStream_t st) {
 }
 
 void profile_stop(hipStream_t st) {
-    if (!g_prof.on || g_prof.used >= g_prof.created) return;
+    if (!g_prof.on || g_prof_quiet || g_prof.used >= g_prof.created) return;
     (void)hipEventRecord(g_prof.stop[g_prof.used], st);
     ++g_prof.used;
 }
@@ -802,7 +863,7 @@ size_t tiles_xpos_words(const TileGeom &tg, int literals) {
 
 // Inference on literal-major tiles (see score_tiles.h).
 int max_lane_words() {
-    const char *e = getenv("GTM_TILE_LANE_WORDS");  // 1, 2 or 4: upper bound on words per lane (tuning aid)
+    const char *e = tune(T_TILE_LANE_WORDS);  // 1, 2 or 4: upper bound on words per lane (tuning aid)
     int v = e ? atoi(e) : 4;
     return v == 1 || v == 2 ? v : 4;
 }
@@ -813,13 +874,13 @@ int max_lane_words() {
 bool half_tiles_allowed(const gtm_config *cfg, const gtm_graphs *g) {
     const int LA = (cfg->literals - 1) / 32 + 1;
     return cfg->depth == 1 && (g->flags & GTM_GRAPHS_COMPLEMENTARY) && cfg->literals % 64 == 0 && LA % 4 == 0 &&
-           LA <= 16 && !getenv("GTM_NO_HALF_TILES") && !getenv("GTM_NO_TWO_PHASE");
+           LA <= 16 && !tune(T_NO_HALF_TILES) && !tune(T_NO_TWO_PHASE);
 }
 
 TileGeom geometry_for(const gtm_config *cfg, const gtm_graphs *g, int classes) {
     return tile_geometry(cfg->literals, g->number_of_node_types, g->max_number_of_graph_nodes, g->number_of_graphs,
                          classes, max_lane_words(), cfg->depth > 1 ? tile_message_rows(cfg->message_size) : 0,
-                         half_tiles_allowed(cfg, g), getenv("GTM_HALF_LANE_WORDS") ? atoi(getenv("GTM_HALF_LANE_WORDS")) : 0);
+                         half_tiles_allowed(cfg, g), tune(T_HALF_LANE_WORDS) ? atoi(tune(T_HALF_LANE_WORDS)) : 0);
 }
 
 // The geometry every tile buffer of this process was built for, by address.  The driver loops
@@ -871,7 +932,7 @@ int launch_tile_layer_as(const TileLayerArgs &a_in, int n_tiles, const char *pro
     size_t lds = tile_layer_lds_bytes(a.tg, a.K, SRC, a.M);
     // message layers: room for every wave's clause list where LDS has it (GTM_NO_LISTS_IN_LDS: tuning and test aid)
     a.lists_in_lds = 0;
-    if (SRC == ROWS_MESSAGES && lds + (size_t)NW * TILE_LIST_LDS_WORDS * 4 <= 160 * 1024 && !getenv("GTM_NO_LISTS_IN_LDS")) {
+    if (SRC == ROWS_MESSAGES && lds + (size_t)NW * TILE_LIST_LDS_WORDS * 4 <= 160 * 1024 && !tune(T_NO_LISTS_IN_LDS)) {
         a.lists_in_lds = 1;
         lds += (size_t)NW * TILE_LIST_LDS_WORDS * 4;
     }
@@ -1013,7 +1074,7 @@ int launch_two_phase_wide_as(const TileLayerArgs &a, int n_tiles, int LA, hipStr
     // rows (if staged), padding, class sums, and the first node and node count of the tile's graphs
     // several narrow tiles per wave (rows read in place, truth rows only, one word per lane): see the kernel
     int pack = 1;
-    if (SRC == ROWS_GLOBAL && !LAST && LW == 1 && a.tg.tw <= 32 && !getenv("GTM_NO_TILE_PACK"))
+    if (SRC == ROWS_GLOBAL && !LAST && LW == 1 && a.tg.tw <= 32 && !tune(T_NO_TILE_PACK))
         pack = 64 / a.tg.tw;
     const int n_groups = (n_tiles + pack - 1) / pack;
     size_t lds = tile_layer_lds_bytes(a.tg, a.K, SRC, a.M) + (size_t)pack * a.tg.gpt * 8;
@@ -1029,7 +1090,7 @@ int launch_two_phase_wide_as(const TileLayerArgs &a, int n_tiles, int LA, hipStr
     if (SRC == ROWS_GLOBAL && !LAST) {
         splits = 2048 / (n_groups > 0 ? n_groups : 1);
         splits = splits < 1 ? 1 : (splits > 16 ? 16 : splits);
-        if (const char *e = getenv("GTM_WIDE_SPLITS")) splits = std::max(1, std::min(64, atoi(e)));
+        if (const char *e = tune(T_WIDE_SPLITS)) splits = std::max(1, std::min(64, atoi(e)));
     }
     profile_start(LAST ? "k_tile_two_phase_wide<score>" : "k_tile_two_phase_wide<layer0>", st);
     hipLaunchKernelGGL((k_tile_two_phase_wide<NW, LW, SRC, LAST>), dim3((unsigned)((n_groups + 7) / 8 * 8 * splits)),
@@ -1063,8 +1124,8 @@ bool two_phase_layer0(const Dims &d, const gtm_graphs *g, const TileGeom &tg) {
     if (tg.half) return true;  // such a geometry is only chosen for k_tile_two_phase_half (64-bit offsets into X)
     // k_tile_two_phase addresses X with 32-bit byte offsets: beyond 4 GiB of literal words (or with
     // GTM_NO_NARROW_TWO_PHASE, which lets tests take that way with small data) k_tile_two_phase_wide runs
-    const bool x_fits = (uint64_t)g->total_nodes * d.LA * 4 < (1ull << 32) && !getenv("GTM_NO_NARROW_TWO_PHASE");
-    return tg.slot_words > 0 && tg.stage0 && d.LA % 4 == 0 && d.LA <= 16 && x_fits && !getenv("GTM_NO_TWO_PHASE");
+    const bool x_fits = (uint64_t)g->total_nodes * d.LA * 4 < (1ull << 32) && !tune(T_NO_NARROW_TWO_PHASE);
+    return tg.slot_words > 0 && tg.stage0 && d.LA % 4 == 0 && d.LA <= 16 && x_fits && !tune(T_NO_TWO_PHASE);
 }
 
 // `_score`'s loop (tm.py:786-812) on tiles: per launch group of tiles, layer 0 and then one
@@ -1083,7 +1144,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     const int layers = cfg->depth;
     const bool narrow = two_phase_layer0(d, g, tg);
     // any other tile of whole-word slots whose row offsets fit the 16-bit entries: k_tile_two_phase_wide
-    const bool wide = !narrow && tg.slot_words > 0 && (int64_t)tg.rows * tg.tw / 4 < 65536 && !getenv("GTM_NO_TWO_PHASE");
+    const bool wide = !narrow && tg.slot_words > 0 && (int64_t)tg.rows * tg.tw / 4 < 65536 && !tune(T_NO_TWO_PHASE);
     const bool two_phase = narrow || wide;
     // compiled clause: 8 words of packed 16-bit row entries (16 words of byte offsets on half tiles) + the include words
     const int stride0 = tg.half ? 16 + d.LA : two_phase ? 8 + d.LA : w.list_stride;
@@ -1127,7 +1188,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     a.X = g->X;
     a.xpos = tg.half ? g->tiles + tiles_xpos_offset_words(tg, cfg->literals) : nullptr;
     a.walk_factor = 2;
-    if (const char *e = getenv("GTM_WIDE_WALK_FACTOR")) a.walk_factor = std::max(1, atoi(e));  // (tuning aid)
+    if (const char *e = tune(T_WIDE_WALK_FACTOR)) a.walk_factor = std::max(1, atoi(e));  // (tuning aid)
     auto layer0 = [&](int n_tiles, bool last) {
         a.lists = w.lists;
         a.stride = stride0;
@@ -1155,7 +1216,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     a.message_rows = w.message_rows;
     const size_t fused_lds = tg.slot_words > 0 ? tile_fused_messages_lds_bytes(tg, MW) : 0;
     bool fused_messages = layers > 1 && tg.slot_words > 0 && d.M % 32 == 0 && fused_lds <= 150 * 1024 &&
-                          !getenv("GTM_NO_FUSED_MESSAGES");
+                          !tune(T_NO_FUSED_MESSAGES);
     if (fused_messages) {
         static thread_local size_t fused_lds_set = 48 * 1024;
         if (fused_lds > fused_lds_set) {
@@ -1168,7 +1229,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             }
         }
     }
-    const bool by_bit = !getenv("GTM_NODE_MESSAGES_BY_ATOMICS");  // tuning aid: the earlier kernel
+    const bool by_bit = !tune(T_NODE_MESSAGES_BY_ATOMICS);  // tuning aid: the earlier kernel
     if (layers > 1 && (fused_messages || by_bit)) {
         // the clauses of every message bit, for the kernels that build what the nodes send
         hipLaunchKernelGGL(k_message_bit_index, dim3(1), dim3(BIT_INDEX_BLOCK), 0, st, s->hypervectors, d.C, d.MB, d.M,
@@ -1208,7 +1269,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             }
             profile_start("k_tile_node_messages + k_tile_edge_messages + k_tile_pack_messages", st);
             if (by_bit) {
-                const int pack = tg.tw <= 32 && !getenv("GTM_NO_TILE_PACK") ? 64 / tg.tw : 1;  // narrow tiles share a wave
+                const int pack = tg.tw <= 32 && !tune(T_NO_TILE_PACK) ? 64 / tg.tw : 1;  // narrow tiles share a wave
                 const int blocks_per_group = (MW + NODE_MESSAGES_BY_BIT_WAVES - 1) / NODE_MESSAGES_BY_BIT_WAVES;
                 const int n_groups = (n_tiles + pack - 1) / pack;
                 hipLaunchKernelGGL(k_tile_node_messages_by_bit, dim3((unsigned)((n_groups + 7) / 8 * 8 * blocks_per_group)),
@@ -1267,7 +1328,7 @@ bool tiles_usable(const gtm_config *cfg, const gtm_graphs *graphs, int classes, 
 }
 
 bool transform_uses_tiles(const gtm_config *cfg, const gtm_graphs *graphs, int classes, TileGeom *tg) {
-    return !getenv("GTM_NO_TILE_TRANSFORM") && tiles_usable(cfg, graphs, classes, tg);
+    return !tune(T_NO_TILE_TRANSFORM) && tiles_usable(cfg, graphs, classes, tg);
 }
 
 }  // namespace
@@ -1525,6 +1586,30 @@ int gtm_transform(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_sta
     return GTM_OK;
 }
 
+int gtm_tuning_set(const char *name, const char *value) {
+    if (!name) return fail(GTM_ERR_INVALID, "name is NULL");
+    for (int i = 0; i < T_COUNT; ++i)
+        if (strcmp(name, g_switch_name[i]) == 0) {
+            if (value && strlen(value) >= sizeof g_switches.value[i])
+                return fail(GTM_ERR_INVALID, "value of %s longer than %zu characters", name, sizeof g_switches.value[i] - 1);
+            g_switches.put(i, value);
+            return GTM_OK;
+        }
+    return fail(GTM_ERR_INVALID, "%s is not a switch of this library", name);
+}
+
+const char *gtm_tuning_get(const char *name) {
+    if (!name) return nullptr;
+    for (int i = 0; i < T_COUNT; ++i)
+        if (strcmp(name, g_switch_name[i]) == 0) return tune((Switch)i);
+    return nullptr;
+}
+
+int gtm_tuning_reload(void) {
+    g_switches = Switches();
+    return GTM_OK;
+}
+
 int gtm_profile_enable(int on) {
     g_prof.on = on != 0;
     g_prof.used = 0;
@@ -1730,17 +1815,40 @@ int gtm_score_static(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_
                     need, GTM_STATIC_SCRATCH_BYTES);
     void *ptr = nullptr;
     if (int rc = static_scratch(&ptr)) return rc;
-    // the launch timing of gtm_profile_enable creates events: not on this path
-    const bool profiling = g_prof.on;
-    g_prof.on = false;
+    // the launch timing of gtm_profile_enable creates events: not on this path (this thread's calls only;
+    // the switch itself, which other threads read, is not touched)
+    g_prof_quiet = true;
     const int rc = gtm_score(cfg, graphs, state, first_graph, n_graphs, batch, ptr, GTM_STATIC_SCRATCH_BYTES, class_sum, stream);
-    g_prof.on = profiling;
+    g_prof_quiet = false;
     return rc;
 }
 
 }  // extern "C"
 
 namespace {
+
+// How long a device-wide wait of the one-launch training kernels may last: a poll cap that only the
+// tests use (GTM_FIT_SPIN_LIMIT = a number of polls, or "abort" = give up at the first wait whatever
+// it shows) and 5 seconds of the device's wall clock otherwise.
+struct WaitBound {
+    uint32_t spin_limit;
+    unsigned long long wait_ticks;
+    int force_abort;
+};
+WaitBound wait_bound(int dev) {
+    WaitBound b{0xFFFFFFFFu, 0ull, 0};
+    int khz = 0;
+    if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || khz <= 0) {
+        (void)hipGetLastError();
+        khz = 100000;  // 100 MHz
+    }
+    b.wait_ticks = 5ull * 1000ull * (unsigned long long)khz;
+    if (const char *e = tune(T_FIT_SPIN_LIMIT)) {
+        b.force_abort = strcmp(e, "abort") == 0;
+        if (!b.force_abort) b.spin_limit = (uint32_t)strtoul(e, nullptr, 10);
+    }
+    return b;
+}
 
 // `_fit`'s inner loop as one cooperative launch (fit_persistent.h).  Returns
 // GTM_OK with *done = false when this device / shape cannot run it, so that the
@@ -1749,7 +1857,7 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                    const FitWs &w, const int32_t *encoded_Y, int first_example, int n_examples, uint64_t first_step,
                    hipStream_t st, bool *done) {
     *done = false;
-    if (getenv("GTM_NO_PERSISTENT_FIT") || d.K > FITP_BLOCK) return GTM_OK;
+    if (tune(T_NO_PERSISTENT_FIT) || d.K > FITP_BLOCK) return GTM_OK;
     int dev = 0, coop = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess) return GTM_OK;
     if (hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) != hipSuccess || !coop) return GTM_OK;
@@ -1758,7 +1866,7 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     FitPersistParams p{};
     p.max_words = tg.slot_words > 0 ? tg.slot_words : 1;
     // graphs of one or two nodes: the nodes are tested on their own literal words, no rows are staged
-    p.direct = g->max_number_of_graph_nodes <= FITP_DIRECT_NODES && !getenv("GTM_NO_DIRECT_FIT");
+    p.direct = g->max_number_of_graph_nodes <= FITP_DIRECT_NODES && !tune(T_NO_DIRECT_FIT);
     p.node_type = g->node_type;
     p.rows_words = p.direct ? 0 : (cfg->literals + g->number_of_node_types + 1) * p.max_words;
     p.x_words = (g->max_number_of_graph_nodes > 0 ? g->max_number_of_graph_nodes : 1) * d.LA;
@@ -1776,7 +1884,7 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     int per_group = (d.C + cus - 1) / cus;
     const int preferred = 8;
     if (per_group < preferred && lds_bytes(preferred) <= lds_limit) per_group = preferred;
-    if (const char *e = getenv("GTM_FIT_PER_GROUP")) {  // tuning: clauses per group, at least C / CUs
+    if (const char *e = tune(T_FIT_PER_GROUP)) {  // tuning: clauses per group, at least C / CUs
         const int asked = atoi(e);
         if (asked >= (d.C + cus - 1) / cus && asked <= FITP_BLOCK) per_group = asked;
     }
@@ -1835,12 +1943,8 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     p.q_thr = q_threshold(cfg->q, cfg->classes);
     p.class_sum = (unsigned long long *)w.class_sum;
     p.abort_flag = (uint32_t *)((unsigned long long *)w.class_sum + (size_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE);
-    p.spin_limit = 4000000u;  // a few seconds of polling at the very most
-    if (const char *e = getenv("GTM_FIT_SPIN_LIMIT")) {  // tests force the give-up path
-        // "abort": every workgroup gives up at its first wait, whatever it reads there
-        p.force_abort = strcmp(e, "abort") == 0;
-        if (!p.force_abort) p.spin_limit = (uint32_t)strtoul(e, nullptr, 10);
-    }
+    const WaitBound bound = wait_bound(dev);
+    p.spin_limit = bound.spin_limit, p.wait_ticks = bound.wait_ticks, p.force_abort = bound.force_abort;
     // A run that gives up leaves the workgroups at different examples.  The bank and the weights
     // are kept as they were, so that a failed call leaves the model as it found it.
     const size_t bank_bytes = (size_t)d.C * d.LA * d.B * 4, weights_bytes = (size_t)d.K * d.C * 4;
@@ -1867,6 +1971,10 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         if (e != hipSuccess)
             return fail(GTM_ERR_HIP, "training kernel gave up waiting at its device-wide barrier (%d workgroups) and "
                                      "the model state could not be restored: %s", groups, hipGetErrorString(e));
+        // The model is as it was.  A wait that really ran out (a GPU shared with other work, a very
+        // large graph) is no reason to fail the call: the caller goes on with the launches per example,
+        // which wait for nobody.  Only the forced give-up of the tests is reported.
+        if (!p.force_abort) return GTM_OK;  // *done stays false
         return fail(GTM_ERR_HIP, "training kernel gave up waiting at its device-wide barrier (%d workgroups); "
                                  "the model state is as it was before the call", groups);
     }
@@ -1881,7 +1989,7 @@ int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *
                         const FitWs &w, const int32_t *encoded_Y, int first_example, int n_examples, uint64_t first_step,
                         hipStream_t st, bool *done) {
     *done = false;
-    if (getenv("GTM_NO_DEEP_PERSISTENT_FIT") || getenv("GTM_NO_PERSISTENT_FIT") || cfg->depth < 2 || d.K > FITD_BLOCK) return GTM_OK;
+    if (tune(T_NO_DEEP_PERSISTENT_FIT) || tune(T_NO_PERSISTENT_FIT) || cfg->depth < 2 || d.K > FITD_BLOCK) return GTM_OK;
     if (d.M % 32 != 0 || d.NC > 64) return GTM_OK;  // whole words of message bits; one lane per word of a truth row
     int dev = 0, coop = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess) return GTM_OK;
@@ -1892,7 +2000,7 @@ int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *
 
     const int layers = cfg->depth - 1, MW = d.M / 32;
     int per_group = (d.C + cus - 1) / cus;
-    if (const char *e = getenv("GTM_FIT_DEEP_CLAUSES_PER_GROUP")) per_group = std::max(per_group, atoi(e));  // tuning aid
+    if (const char *e = tune(T_FIT_DEEP_CLAUSES_PER_GROUP)) per_group = std::max(per_group, atoi(e));  // tuning aid
     const int groups = (d.C + per_group - 1) / per_group;
     const int NW = d.NC;
     const int rows_words = (cfg->literals + g->number_of_node_types + 1) * NW;
@@ -1913,13 +2021,13 @@ int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *
     // automata, layer-0 rows and all received rows in LDS where they fit; else automata in memory, rows in
     // place and as wide a window of received rows as fits
     const size_t lds_cap = 158 * 1024;  // of 160 KiB; the kernel has a few words of its own
-    bool big = getenv("GTM_FIT_DEEP_IN_MEMORY") != nullptr;  // tuning aid: take the second layout anyway
+    bool big = tune(T_FIT_DEEP_IN_MEMORY) != nullptr;  // tuning aid: take the second layout anyway
     int window_rows = d.M;
     size_t lds = fit_deep_lds_words(false, cfg->depth, cfg->literals, per_group, d.LA, d.MC, d.MB, d.B, d.K, NW, rows_words, d.M, cfg->max_nodes,
                                     edge_cap, edge_types) * 4;
     if (lds > lds_cap) big = true;
     if (big) {
-        if (const char *e = getenv("GTM_FIT_DEEP_WINDOW_ROWS")) window_rows = std::max(32, std::min(d.M, atoi(e) / 32 * 32));
+        if (const char *e = tune(T_FIT_DEEP_WINDOW_ROWS)) window_rows = std::max(32, std::min(d.M, atoi(e) / 32 * 32));
         for (;; window_rows = (window_rows / 2 + 31) / 32 * 32) {
             lds = fit_deep_lds_words(true, cfg->depth, cfg->literals, per_group, d.LA, d.MC, d.MB, d.B, d.K, NW, 0, window_rows, cfg->max_nodes,
                                      edge_cap, edge_types) * 4;
@@ -1994,16 +2102,13 @@ int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *
     p.arrived = w.coop_arrived;
     p.class_sum = (unsigned long long *)w.class_sum;
     p.abort_flag = (uint32_t *)((unsigned long long *)w.class_sum + (size_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE);
-    p.spin_limit = 4000000u;
-    if (const char *e = getenv("GTM_FIT_SPIN_LIMIT")) {  // tests force the give-up path
-        p.force_abort = strcmp(e, "abort") == 0;
-        if (!p.force_abort) p.spin_limit = (uint32_t)strtoul(e, nullptr, 10);
-    }
+    const WaitBound bound = wait_bound(dev);
+    p.spin_limit = bound.spin_limit, p.wait_ticks = bound.wait_ticks, p.force_abort = bound.force_abort;
     p.clauses_per_group = per_group;
     p.NW = NW;
     p.rows_words = big ? 0 : rows_words;
     p.window_rows = window_rows;
-    p.by_masks = (size_t)window_rows * NW >= (size_t)(1 + edge_types) * cfg->max_nodes && !getenv("GTM_FIT_DEEP_NO_MASKS");
+    p.by_masks = (size_t)window_rows * NW >= (size_t)(1 + edge_types) * cfg->max_nodes && !tune(T_FIT_DEEP_NO_MASKS);
     p.order = g->tiles + tiles_words(tg) + (size_t)tg.rows * 2;
     p.max_nodes = cfg->max_nodes;
     p.edge_cap = edge_cap;
@@ -2059,6 +2164,7 @@ int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *
         if (e != hipSuccess)
             return fail(GTM_ERR_HIP, "training kernel gave up waiting at a device-wide barrier (%d workgroups) and the "
                                      "model state could not be restored: %s", groups, hipGetErrorString(e));
+        if (!p.force_abort) return GTM_OK;  // as in fit_persistent: the launches per example take over
         return fail(GTM_ERR_HIP, "training kernel gave up waiting at a device-wide barrier (%d workgroups); "
                                  "the model state is as it was before the call", groups);
     }
@@ -2131,7 +2237,7 @@ int fit_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, cons
 int fit_small(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const int32_t *encoded_Y,
               int first_example, int n_examples, uint64_t first_step, hipStream_t st, bool *done) {
     *done = false;
-    if (getenv("GTM_NO_SMALL_FIT")) return GTM_OK;
+    if (tune(T_NO_SMALL_FIT)) return GTM_OK;
     if (cfg->depth < 2 || d.M % 32 != 0 || g->max_number_of_graph_nodes > FITS_MAX_NODES ||
         g->number_of_node_types < 1)
         return GTM_OK;
@@ -2223,7 +2329,7 @@ int fit_deep_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g,
     // graph is big enough for the saved atomics to pay for the extra pass.
     const int MW = (d.M + 31) / 32;
     const bool factored = d.M % 32 == 0 && (size_t)32 * MW * 4 <= 48 * 1024;
-    const char *fm = getenv("GTM_FIT_FACTOR_MIN");  // clauses x nodes from which that path is taken (tuning aid)
+    const char *fm = tune(T_FIT_FACTOR_MIN);  // clauses x nodes from which that path is taken (tuning aid)
     const int64_t factor_min = fm ? atoll(fm) : 32768;
     if (factored) {
         const int64_t vector_words = (int64_t)cfg->max_nodes * MW;
@@ -2394,7 +2500,7 @@ int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *st
         if (int rc = fit_small(d, cfg, graphs, state, encoded_Y, first_example, n_examples, first_step, st, &done)) return rc;
         if (done) return GTM_OK;
     }
-    if (cfg->depth > 1 && graphs->tiles && graphs->number_of_node_types >= 1 && !getenv("GTM_NO_DEEP_FIT")) {
+    if (cfg->depth > 1 && graphs->tiles && graphs->number_of_node_types >= 1 && !tune(T_NO_DEEP_FIT)) {
         TileGeom tg = geometry_for(cfg, graphs, d.K);
         if (tg.ok && tg.slot_words <= 64 && cfg->max_nodes <= 2048) {  // one lane per word of the graph's nodes
             bool done = false;

@@ -17,6 +17,7 @@ accepted and ignored: launch shapes are chosen by the library.
 """
 
 import ctypes
+import io
 import os
 import pickle
 import sys
@@ -85,9 +86,8 @@ class _DeviceGraphs:
         layout keep tiles = NULL.  The geometry depends on the model's
         sizes, so a data set handed to a model of another shape is tiled
         again."""
-        key = (cfg.classes, cfg.literals, cfg.depth, cfg.message_size, os.environ.get("GTM_TILE_LANE_WORDS"),
-               os.environ.get("GTM_NO_HALF_TILES"), os.environ.get("GTM_NO_TWO_PHASE"),
-               os.environ.get("GTM_HALF_LANE_WORDS"))
+        key = (cfg.classes, cfg.literals, cfg.depth, cfg.message_size, _abi.tuning("GTM_TILE_LANE_WORDS"),
+               _abi.tuning("GTM_NO_HALF_TILES"), _abi.tuning("GTM_NO_TWO_PHASE"), _abi.tuning("GTM_HALF_LANE_WORDS"))
         if self._tiles_key == key:
             return
         self._tiles_key = key
@@ -123,6 +123,40 @@ _NPZ_SCALARS = (
     "boost_true_positive_feedback", "number_of_state_bits", "depth", "message_size", "message_bits",
     "double_hashing", "one_hot_encoding", "rng_seed", "rng_step",
 )
+
+
+class _StateUnpickler(pickle.Unpickler):
+    """Reads the dict that ``save`` pickles (tm.py:328-356: NumPy arrays, NumPy and Python scalars,
+    tuples, lists) and nothing else: a pickle may name any importable callable and have it run
+    while it loads, so every global it asks for is checked against the few that rebuild arrays
+    and scalars, and anything else ends the load before it runs."""
+
+    _ALLOWED = {
+        ("numpy", "ndarray"), ("numpy", "dtype"),
+        ("numpy.core.multiarray", "_reconstruct"), ("numpy._core.multiarray", "_reconstruct"),
+        ("numpy.core.multiarray", "scalar"), ("numpy._core.multiarray", "scalar"),
+        ("numpy.core.numeric", "_frombuffer"), ("numpy._core.numeric", "_frombuffer"),
+        ("builtins", "dict"), ("builtins", "tuple"), ("builtins", "list"), ("builtins", "int"),
+        ("builtins", "float"), ("builtins", "bool"), ("builtins", "complex"), ("builtins", "bytes"),
+        ("builtins", "str"), ("builtins", "bytearray"),
+    }
+
+    def find_class(self, module, name):
+        if (module, name) not in self._ALLOWED:
+            raise pickle.UnpicklingError(
+                "the state file asks for %s.%s: only NumPy arrays, scalars and plain containers are loaded"
+                % (module, name))
+        return super().find_class(module, name)
+
+
+def read_state_pickle(fname):
+    """The dict of a ``save(fname)`` pickle - this class's or the reference's (tm.py:356-357) - read
+    without running anything the file names."""
+    with open(fname, "rb") as f:
+        state_dict = _StateUnpickler(io.BytesIO(f.read())).load()
+    if not isinstance(state_dict, dict):
+        raise pickle.UnpicklingError("the state file holds a %s, not the dict that save() writes" % type(state_dict).__name__)
+    return state_dict
 
 
 def write_state_npz(state_dict, fname):
@@ -610,8 +644,14 @@ class CommonTsetlinMachine:
         self.ta_state = np.array([])
         self.clause_weights = np.array([])
 
-    def save(self, fname=""):
-        """tm.py:312-362: the reference's 24 keys plus the generator position."""
+    def save(self, fname="", format=None):
+        """tm.py:312-362: the reference's 24 keys plus the generator position.  The file is a NumPy
+        archive of plain arrays (nothing in it is pickled, so reading it back runs nothing) unless
+        ``format="pickle"`` asks for the reference's pickle of the same dict (tm.py:356-357), for
+        files that the reference itself is to load.  ``load`` tells the two apart by their first
+        bytes, whatever the file is called."""
+        if format not in (None, "npz", "pickle"):
+            raise _abi.GtmError("save: format=%r is neither 'npz' nor 'pickle'" % (format,))
         self._download()
         state_dict = {
             "ta_state": self.ta_state,
@@ -643,25 +683,25 @@ class CommonTsetlinMachine:
         }
         if len(fname) > 0:
             print(f"Saving model to {fname}.")
-            if fname.endswith(".npz"):
-                write_state_npz(state_dict, fname)
-            else:
+            if format == "pickle":
                 with open(fname, "wb") as f:
                     pickle.dump(state_dict, f)
+            else:
+                write_state_npz(state_dict, fname)
         return state_dict
 
     def load(self, state_dict={}, fname=""):
-        """tm.py:364-412."""
+        """tm.py:364-412.  A file is read as the NumPy archive that ``save`` writes or, when it is a
+        pickle (``save(format="pickle")``, or the reference's own ``save``), by an unpickler that only
+        rebuilds arrays, scalars and plain containers and refuses every other global a pickle names."""
         if len(fname) == 0 and len(state_dict) == 0:
             print("Error: No file or state_dict provided. Pass either a file name or a state_dict.")
             return
         if len(fname) > 0:
             print(f"Loading model from {fname}.")
-            if fname.endswith(".npz"):
-                state_dict = read_state_npz(fname)
-            else:
-                with open(fname, "rb") as f:
-                    state_dict = pickle.load(f)
+            with open(fname, "rb") as f:
+                is_archive = f.read(2) == b"PK"  # a NumPy archive is a zip file
+            state_dict = read_state_npz(fname) if is_archive else read_state_pickle(fname)
         # the constructor arguments travel with the state (tm.py:341-353 saves them; the reference's
         # load leaves them to the caller's constructor call): a model built with other arguments
         # must not run a loaded state with the wrong clause count, depth or automaton width

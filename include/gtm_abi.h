@@ -218,8 +218,10 @@ size_t gtm_fit_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs);
  * step first_step + i for its random draws.  With depth == 1 and
  * graphs->tiles set the whole run is one cooperative launch in which each
  * workgroup keeps its clauses' automata in LDS and the class sums are the
- * only exchange between workgroups; if that launch gives up waiting for a
- * workgroup (bounded wait) the call returns GTM_ERR_HIP. */
+ * only exchange between workgroups.  Its waits are bounded (5 s of the device's
+ * wall clock): if one runs out, the model is put back as it was before the
+ * launch and the examples are trained by launches per example instead, which
+ * wait for nobody - same results, the call still returns GTM_OK. */
 int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, const int32_t *encoded_Y,
             int32_t first_example, int32_t n_examples, uint64_t first_step, void *workspace,
             size_t workspace_bytes, void *stream);
@@ -248,11 +250,22 @@ int gtm_transform(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_sta
                   int32_t n_graphs, int32_t batch, void *workspace, size_t workspace_bytes, int32_t *transformed,
                   int32_t *nodewise, int32_t width, int32_t *class_sum, void *stream);
 
+/* No counterpart in the reference (its tuning knobs are the `grid` and `block` constructor
+ * arguments, tm.py:53-54).  The library's tuning and test switches - the GTM_* names listed in its
+ * documentation - are read from the process environment once, when the library is loaded, and
+ * never again by the entry points above.  gtm_tuning_set() sets one switch for the rest of the
+ * process (value NULL = not set), gtm_tuning_get() returns its value or NULL, gtm_tuning_reload()
+ * reads the environment again.  For tests and tuning runs: none of the three may run while another
+ * call of the library is under way. */
+int gtm_tuning_set(const char *name, const char *value);
+const char *gtm_tuning_get(const char *name);
+int gtm_tuning_reload(void);
+
 /* No counterpart in the reference.  While enabled, gtm_score / gtm_transform /
  * gtm_fit bracket the launches of the kernels that do their work (clause
  * evaluation per layer, message construction, the one-launch training kernels)
  * with HIP events on the caller's stream, each under its kernel's name (at most
- * 4096 launches are kept).  gtm_profile_read() waits for those events, returns
+ * 4096 launches are kept; gtm_score_static never records any).  gtm_profile_read() waits for those events, returns
  * the name of the kernel launched last, the number of launches seen and their
  * summed duration (all kernels together: a model without message layers has one),
  * and clears the record.  Not thread-safe; meant for the benchmark. */

@@ -27,3 +27,21 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def tune():
+    """tune(name, value): sets one of the library's GTM_* switches for the rest of the test (value
+    None = not set); every switch a test touched is unset again when the test ends.  The library reads
+    the environment only once, at load, so a test changes its switches through gtm_tuning_set."""
+    from graphtsetlinmachine_amd import _abi
+
+    touched = []
+
+    def set_switch(name, value="1"):
+        _abi.call("gtm_tuning_set", name.encode(), None if value is None else str(value).encode())
+        touched.append(name)
+
+    yield set_switch
+    for name in touched:
+        _abi.call("gtm_tuning_set", name.encode(), None)

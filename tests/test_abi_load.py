@@ -43,6 +43,34 @@ def test_invalid_config_is_rejected_without_touching_the_gpu():
     assert _abi.lib.gtm_score_workspace_bytes(ctypes.byref(cfg), None, 4) == 0
 
 
+def test_switches_are_read_at_load_and_changed_only_through_the_library(monkeypatch):
+    """The library looks at the environment once, when it is loaded: a variable set afterwards changes
+    nothing until gtm_tuning_reload; gtm_tuning_set sets and unsets one switch; unknown names and
+    over-long values are refused."""
+    from graphtsetlinmachine_amd import _abi
+
+    name = "GTM_WIDE_SPLITS"
+    before = _abi.tuning(name)
+    try:
+        monkeypatch.setenv(name, "7")
+        assert _abi.tuning(name) == before          # the environment is not read per call
+        _abi.call("gtm_tuning_reload")
+        assert _abi.tuning(name) == "7"
+        _abi.call("gtm_tuning_set", name.encode(), b"3")
+        assert _abi.tuning(name) == "3"
+        _abi.call("gtm_tuning_set", name.encode(), None)
+        assert _abi.tuning(name) is None
+        with pytest.raises(_abi.GtmError, match="not a switch"):
+            _abi.call("gtm_tuning_set", b"GTM_NO_SUCH_SWITCH", b"1")
+        with pytest.raises(_abi.GtmError, match="longer than"):
+            _abi.call("gtm_tuning_set", name.encode(), b"1" * 64)
+        assert _abi.tuning("GTM_NO_SUCH_SWITCH") is None
+    finally:
+        monkeypatch.delenv(name, raising=False)
+        _abi.call("gtm_tuning_reload")
+    assert _abi.tuning(name) is None or _abi.tuning(name) == os.environ.get(name)
+
+
 def test_ctypes_structs_match_the_header(tmp_path):
     from graphtsetlinmachine_amd import _abi
 

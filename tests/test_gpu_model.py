@@ -86,7 +86,7 @@ def test_save_load_roundtrip_and_resume(tmp_path):
     a = MultiClassGraphTsetlinMachine(**wl.params, seed=5)
     a.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
     path = str(tmp_path / "model.pkl")
-    state = a.save(path)
+    state = a.save(path, format="pickle")  # the reference's file format (tm.py:356-357)
     reference_keys = {
         "ta_state", "message_ta_state", "clause_weights", "hypervectors", "number_of_outputs", "number_of_literals",
         "number_of_message_literals", "min_y", "max_y", "negative_clauses", "max_number_of_graph_nodes",
@@ -99,6 +99,14 @@ def test_save_load_roundtrip_and_resume(tmp_path):
     b = MultiClassGraphTsetlinMachine(**wl.params, seed=777)
     b.load(fname=path)
     assert np.array_equal(b.score(wl.graphs_test), a.score(wl.graphs_test))
+    # by default the file is an archive of plain arrays whatever it is called; load tells by the content
+    plain = str(tmp_path / "model.tm")
+    a.save(plain)
+    with np.load(plain, allow_pickle=False) as z:
+        assert "ta_state" in z.files
+    c = MultiClassGraphTsetlinMachine(**wl.params, seed=778)
+    c.load(fname=plain)
+    assert np.array_equal(c.score(wl.graphs_test), a.score(wl.graphs_test))
     # resuming from the file continues exactly where the first model would have gone
     a.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
     b.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
@@ -214,7 +222,7 @@ def test_transform_and_read_outs_match_the_oracle():
     dict(g=dict(n_graphs=20, max_nodes=20, min_nodes=4, hv_size=20, edge_types=("x", "y", "z")),
          m=dict(depth=3, message_size=37, message_bits=3), clauses=50, classes=4),
 ], ids=["361-nodes", "tiny-graphs", "two-layers", "three-layers"])
-def test_transform_on_tiles(case, monkeypatch):
+def test_transform_on_tiles(case, tune):
     """gtm_transform from the truth rows of the tile kernels (k_tile_transform) == the dense path ==
     the oracle: per-clause outputs, per-node outputs and class sums, in one launch group and in groups
     of 7 graphs (which start and end inside tiles)."""
@@ -251,7 +259,7 @@ def test_transform_on_tiles(case, monkeypatch):
     assert np.array_equal(wide, want_wide) and np.array_equal(sums, want_sums)
     got, sums = tm._transform(graphs, False, batch=7)
     assert np.array_equal(got, want) and np.array_equal(sums, want_sums)
-    monkeypatch.setenv("GTM_NO_TILE_TRANSFORM", "1")
+    tune("GTM_NO_TILE_TRANSFORM", "1")
     dense, dense_sums = tm._transform(graphs, False)
     assert np.array_equal(dense, want) and np.array_equal(dense_sums, want_sums)
 

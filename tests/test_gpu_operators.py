@@ -321,7 +321,7 @@ DEEP_TILE_SHAPES = [
 @pytest.mark.parametrize("message_density", [0.0, 0.01, 0.1, 0.6])
 @pytest.mark.parametrize("messages", ["graph-per-workgroup", "graph-per-workgroup-lists-by-scalar-loads",
                                       "three-launches", "three-launches-atomics"])
-def test_tile_scoring_with_message_layers(shape, message_density, messages, monkeypatch):
+def test_tile_scoring_with_message_layers(shape, message_density, messages, tune):
     """gtm_score with message layers on literal-major tiles == oracle == the bitmap path, with the
     message rows built by one workgroup per graph (where the shape allows) and by the three
     launches that keep the vectors in global memory.  The clause lists of the message layers reach the
@@ -330,11 +330,11 @@ def test_tile_scoring_with_message_layers(shape, message_density, messages, monk
     from tests.gpu_harness import Device
 
     if not messages.startswith("graph-per-workgroup"):
-        monkeypatch.setenv("GTM_NO_FUSED_MESSAGES", "1")
+        tune("GTM_NO_FUSED_MESSAGES", "1")
     if messages == "graph-per-workgroup-lists-by-scalar-loads":
-        monkeypatch.setenv("GTM_NO_LISTS_IN_LDS", "1")
+        tune("GTM_NO_LISTS_IN_LDS", "1")
     if messages == "three-launches-atomics":
-        monkeypatch.setenv("GTM_NODE_MESSAGES_BY_ATOMICS", "1")
+        tune("GTM_NODE_MESSAGES_BY_ATOMICS", "1")
 
     graphs = helpers.random_graphs(shape["seed"], **shape["g"])
     m = dict(shape["m"])
@@ -360,16 +360,16 @@ def test_tile_scoring_with_message_layers(shape, message_density, messages, monk
 @pytest.mark.parametrize("shape", DEEP_TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
 @pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 9, 5)])
 @pytest.mark.parametrize("messages", ["by-node-vectors", "by-scatter"])
-def test_fused_fit_with_message_layers(shape, boost, max_included, state_bits, messages, monkeypatch):
+def test_fused_fit_with_message_layers(shape, boost, max_included, state_bits, messages, tune):
     """The fused training step of models with message layers == the oracle: automata of every
     bank and the weights after each of two epochs.  Both ways of building the messages (per-node
     bit vectors rotated along the edges, taken when MESSAGE_SIZE is a multiple of 32; one scatter
     per true clause, node and edge) are forced in turn."""
     from tests.gpu_harness import Device
 
-    monkeypatch.setenv("GTM_FIT_FACTOR_MIN", "0" if messages == "by-node-vectors" else str(1 << 60))
-    monkeypatch.setenv("GTM_NO_SMALL_FIT", "1")  # the one-workgroup kernel has its own test
-    monkeypatch.setenv("GTM_NO_DEEP_PERSISTENT_FIT", "1")  # and so has the one-launch kernel
+    tune("GTM_FIT_FACTOR_MIN", "0" if messages == "by-node-vectors" else str(1 << 60))
+    tune("GTM_NO_SMALL_FIT", "1")  # the one-workgroup kernel has its own test
+    tune("GTM_NO_DEEP_PERSISTENT_FIT", "1")  # and so has the one-launch kernel
 
     g = dict(shape["g"])
     if "sizes" not in g:
@@ -425,7 +425,7 @@ ONE_LAUNCH_DEEP_SHAPES = [
 @pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 9, 5), (1, None, 12)])
 @pytest.mark.parametrize("layout", ["in-lds", "in-lds-40-clauses-per-workgroup", "in-memory", "in-memory-32-row-windows",
                                     "in-memory-40-clauses-per-workgroup"])
-def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bits, layout, monkeypatch):
+def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bits, layout, tune):
     """A run of training examples of a model with message layers in one cooperative launch
     (k_fit_deep_persistent: clauses spread over workgroups, the nodes' messages and the class sums
     exchanged through device memory): automata of every bank and the weights after each of two
@@ -438,13 +438,13 @@ def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bi
     from tests.gpu_harness import Device
     from graphtsetlinmachine_amd import _abi
 
-    monkeypatch.setenv("GTM_NO_SMALL_FIT", "1")
+    tune("GTM_NO_SMALL_FIT", "1")
     if layout.startswith("in-memory"):
-        monkeypatch.setenv("GTM_FIT_DEEP_IN_MEMORY", "1")
+        tune("GTM_FIT_DEEP_IN_MEMORY", "1")
     if layout == "in-memory-32-row-windows":
-        monkeypatch.setenv("GTM_FIT_DEEP_WINDOW_ROWS", "32")
+        tune("GTM_FIT_DEEP_WINDOW_ROWS", "32")
     if layout.endswith("40-clauses-per-workgroup"):
-        monkeypatch.setenv("GTM_FIT_DEEP_CLAUSES_PER_GROUP", "40")
+        tune("GTM_FIT_DEEP_CLAUSES_PER_GROUP", "40")
     kernel = b"k_fit_deep_persistent<in memory>" if layout.startswith("in-memory") else b"k_fit_deep_persistent"
     graphs = helpers.random_graphs(shape["seed"], **shape["g"])
     m = dict(shape["m"])
@@ -476,16 +476,16 @@ def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bi
 
 
 @pytest.mark.parametrize("layout", ["in-lds", "in-memory"])
-def test_one_launch_fit_with_message_layers_gives_up_instead_of_hanging(layout, monkeypatch):
+def test_one_launch_fit_with_message_layers_gives_up_instead_of_hanging(layout, tune):
     """As for the depth-1 kernel: GTM_FIT_SPIN_LIMIT=abort makes every workgroup give up at its first
     device-wide wait; the kernel drains, the call reports it, every bank and the weights are as
     they were, and the same model trains normally afterwards."""
     from tests.gpu_harness import Device
     from graphtsetlinmachine_amd import _abi
 
-    monkeypatch.setenv("GTM_NO_SMALL_FIT", "1")
+    tune("GTM_NO_SMALL_FIT", "1")
     if layout == "in-memory":
-        monkeypatch.setenv("GTM_FIT_DEEP_IN_MEMORY", "1")
+        tune("GTM_FIT_DEEP_IN_MEMORY", "1")
     shape = ONE_LAUNCH_DEEP_SHAPES[1]
     graphs = helpers.random_graphs(shape["seed"], **shape["g"])
     m = dict(shape["m"])
@@ -503,10 +503,10 @@ def test_one_launch_fit_with_message_layers_gives_up_instead_of_hanging(layout, 
         return (np.array_equal(w, model.clause_weights) and np.array_equal(ta, model.ta_state) and
                 all(np.array_equal(banks[l], model.message_ta_state[l]) for l in range(depth - 1)))
 
-    monkeypatch.setenv("GTM_FIT_SPIN_LIMIT", "abort")
+    tune("GTM_FIT_SPIN_LIMIT", "abort")
     with pytest.raises(_abi.GtmError, match="gave up waiting.*as it was before the call"):
         dev.fit(Y, 0, G, 0)
-    monkeypatch.delenv("GTM_FIT_SPIN_LIMIT")
+    tune("GTM_FIT_SPIN_LIMIT", None)
     assert same_as_oracle()
     o.fit(model, graphs, Y)
     dev.fit(Y, 0, G, 0)
@@ -572,13 +572,13 @@ def test_one_workgroup_fit_with_message_layers(shape, boost, max_included, state
 @pytest.mark.parametrize("shape", TILE_SHAPES, ids=lambda s: "tiles%d" % s["seed"])
 @pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 6, 5)])
 @pytest.mark.parametrize("persistent", [True, False], ids=["one-launch", "two-per-graph"])
-def test_fused_fit_on_every_tile_geometry(shape, boost, max_included, state_bits, persistent, monkeypatch):
+def test_fused_fit_on_every_tile_geometry(shape, boost, max_included, state_bits, persistent, tune):
     """Both fused depth-1 training paths (one cooperative launch per run of
     examples; two launches per example) == the oracle."""
     from tests.gpu_harness import Device
 
     if not persistent:
-        monkeypatch.setenv("GTM_NO_PERSISTENT_FIT", "1")
+        tune("GTM_NO_PERSISTENT_FIT", "1")
 
     g = dict(shape["g"])
     g["n_graphs"] = min(g["n_graphs"], 24)
@@ -672,14 +672,14 @@ def test_more_classes_than_lanes(shape, classes):
 
 @pytest.mark.parametrize("shape", [TILE_SHAPES[3], TILE_SHAPES[5], TILE_SHAPES[6]], ids=lambda s: "tiles%d" % s["seed"])
 @pytest.mark.parametrize("per_group", [1, 3, 16, 20, 40])
-def test_one_launch_fit_with_any_number_of_clauses_per_workgroup(shape, per_group, monkeypatch):
+def test_one_launch_fit_with_any_number_of_clauses_per_workgroup(shape, per_group, tune):
     """The cooperative training kernel gives a workgroup 8 or more clauses; GTM_FIT_PER_GROUP sets
     the number.  Up to 16 (one clause per wave) a small clause's feedback runs inside its wave,
     above that a wave evaluates several clauses and the feedback is shared out over the group:
     every split == the oracle."""
     from tests.gpu_harness import Device
 
-    monkeypatch.setenv("GTM_FIT_PER_GROUP", str(per_group))
+    tune("GTM_FIT_PER_GROUP", str(per_group))
     g = dict(shape["g"])
     g["n_graphs"] = min(g["n_graphs"], 24)
     graphs = helpers.random_graphs(shape["seed"], **g)
@@ -709,13 +709,13 @@ def test_one_launch_fit_with_any_number_of_clauses_per_workgroup(shape, per_grou
 ], ids=lambda v: str(v) if isinstance(v, int) else "")
 @pytest.mark.parametrize("density", [0.3, 0.9])
 @pytest.mark.parametrize("persistent", [True, False], ids=["one-launch", "per-example"])
-def test_fused_fit_with_many_literals(seed, g, m, density, persistent, monkeypatch):
+def test_fused_fit_with_many_literals(seed, g, m, density, persistent, tune):
     """Clauses with many included literals (the training kernels AND a few of their rows and
     test the surviving nodes against the whole include mask) == the oracle."""
     from tests.gpu_harness import Device
 
     if not persistent:
-        monkeypatch.setenv("GTM_NO_PERSISTENT_FIT", "1")
+        tune("GTM_NO_PERSISTENT_FIT", "1")
     elif m["depth"] > 1:
         pytest.skip("models with message layers have one training path")
     graphs = helpers.random_graphs(seed, **g)
@@ -778,7 +778,7 @@ def test_empty_graphs_score_like_the_reference_arithmetic(hv_size, density):
     assert np.array_equal(dev.score(0, 6, 6), want)
 
 
-def test_training_kernel_gives_up_instead_of_hanging(monkeypatch):
+def test_training_kernel_gives_up_instead_of_hanging(tune):
     """The one-launch training kernel waits for the other workgroups with a
     bounded number of polls.  GTM_FIT_SPIN_LIMIT=abort makes every workgroup give up at
     its first wait whatever it reads there (no dependence on timing or on the number of
@@ -794,10 +794,10 @@ def test_training_kernel_gives_up_instead_of_hanging(monkeypatch):
     dev = Device(model, graphs)
     assert dev.build_tiles()
     Y = o.encode_labels(np.zeros(graphs.number_of_graphs, dtype=np.int64), cfg.classes, cfg.threshold)
-    monkeypatch.setenv("GTM_FIT_SPIN_LIMIT", "abort")
+    tune("GTM_FIT_SPIN_LIMIT", "abort")
     with pytest.raises(_abi.GtmError, match="gave up waiting.*as it was before the call"):
         dev.fit(Y, 0, graphs.number_of_graphs, 0)
-    monkeypatch.delenv("GTM_FIT_SPIN_LIMIT")
+    tune("GTM_FIT_SPIN_LIMIT", None)
     ta, _, w = dev.download()
     assert np.array_equal(w, model.clause_weights) and np.array_equal(ta, model.ta_state)
     # the same model trains normally afterwards
@@ -806,13 +806,13 @@ def test_training_kernel_gives_up_instead_of_hanging(monkeypatch):
     ta, _, w = dev.download()
     assert np.array_equal(w, model.clause_weights) and np.array_equal(ta, model.ta_state)
     # a limit of 0 polls: whoever does not see every arrival at its first look gives up
-    monkeypatch.setenv("GTM_FIT_SPIN_LIMIT", "0")
+    tune("GTM_FIT_SPIN_LIMIT", "0")
     try:
         dev.fit(Y, 0, graphs.number_of_graphs, graphs.number_of_graphs)
         o.fit(model, graphs, Y)  # nobody had to wait: the run went through
     except _abi.GtmError as e:
         assert "gave up waiting" in str(e)
-    monkeypatch.delenv("GTM_FIT_SPIN_LIMIT")
+    tune("GTM_FIT_SPIN_LIMIT", None)
     ta, _, w = dev.download()
     assert np.array_equal(w, model.clause_weights) and np.array_equal(ta, model.ta_state)
 
@@ -955,7 +955,7 @@ def test_data_that_is_not_complementary_is_detected_and_keeps_all_rows():
 
 
 @pytest.mark.parametrize("shape", [s for s in TILE_SHAPES if s["seed"] in (14, 15, 16, 17, 18)], ids=lambda s: "tiles%d" % s["seed"])
-def test_the_kernel_that_takes_over_beyond_4_gib_of_literal_words_follows_the_oracle(shape, monkeypatch):
+def test_the_kernel_that_takes_over_beyond_4_gib_of_literal_words_follows_the_oracle(shape, tune):
     """k_tile_two_phase addresses X with 32-bit byte offsets and hands data sets of 4 GiB and more to
     k_tile_two_phase_wide (64-bit offsets).  GTM_NO_NARROW_TWO_PHASE takes that way with small data."""
     from tests.gpu_harness import Device
@@ -966,7 +966,7 @@ def test_the_kernel_that_takes_over_beyond_4_gib_of_literal_words_follows_the_or
     dev = Device(model, graphs)
     G = graphs.number_of_graphs
     assert dev.build_tiles()
-    monkeypatch.setenv("GTM_NO_NARROW_TWO_PHASE", "1")
+    tune("GTM_NO_NARROW_TWO_PHASE", "1")
     _abi.call("gtm_profile_enable", 1)
     got = dev.score(0, G, G)
     name, launches, total = ctypes.c_char_p(), ctypes.c_int32(), ctypes.c_double()

@@ -60,6 +60,52 @@ def test_npz_state_file_round_trips_without_pickle(tmp_path):
     assert back["rng_seed"] == 2**64 - 3 and back["rng_step"] == 123456789012
 
 
+def test_a_pickled_state_is_read_without_running_what_it_names(tmp_path):
+    """A pickle can name any importable callable and have it called while it loads.  The reader of
+    state files rebuilds arrays, scalars and plain containers only: the reference's dict comes back
+    equal, and a file that names anything else is refused before that thing runs."""
+    import pickle
+
+    state = reference_shaped_state(np.random.default_rng(2))
+    state["q"] = np.float64(1.0)  # NumPy scalars travel too (numpy.core.multiarray.scalar)
+    path = str(tmp_path / "model.pkl")
+    with open(path, "wb") as f:
+        pickle.dump(state, f)
+    back = tm_module.read_state_pickle(path)
+    assert list(back) == REFERENCE_KEYS
+    for key in REFERENCE_KEYS:
+        if key == "message_ta_state":
+            assert all(np.array_equal(a, b) for a, b in zip(back[key], state[key]))
+        elif isinstance(state[key], np.ndarray):
+            assert back[key].dtype == state[key].dtype and np.array_equal(back[key], state[key])
+        else:
+            assert back[key] == state[key]
+
+    marker = tmp_path / "ran"
+
+    class Payload:
+        def __reduce__(self):
+            import os
+
+            return (os.system, ("touch %s" % marker,))
+
+    for poisoned in (Payload(), dict(state, T=Payload()), {"ta_state": [Payload()]}):
+        with open(path, "wb") as f:
+            pickle.dump(poisoned, f)
+        with pytest.raises(pickle.UnpicklingError, match="only NumPy arrays"):
+            tm_module.read_state_pickle(path)
+        assert not marker.exists()
+    # the model's load() goes through the same reader (no device is touched before the file is read)
+    with pytest.raises(pickle.UnpicklingError, match="only NumPy arrays"):
+        MultiClassGraphTsetlinMachine(10, 20, 1.0).load(fname=path)
+    assert not marker.exists()
+    # something that is not the dict of save()
+    with open(path, "wb") as f:
+        pickle.dump([1, 2, 3], f)
+    with pytest.raises(pickle.UnpicklingError, match="not the dict"):
+        tm_module.read_state_pickle(path)
+
+
 def test_more_outputs_than_allocated_is_refused_before_any_device_call(monkeypatch):
     """The weight buffer and the tile geometry are sized at the first fit; a later batch with a
     higher label must not reach the kernels (an out-of-bounds device write)."""

@@ -137,6 +137,28 @@ def test_classes_apply_in_order_to_the_same_bank():
     assert np.array_equal(decode(bank), states)  # Type II needs a fired clause
 
 
+def test_initial_weights_are_a_fair_coin():
+    """kernels.py:646-652: `1 - 2 * (curand % 2)` is +1 or -1 with equal probability, independently per
+    (class, clause).  Over 10 x 20,000 weights the mean stays within 5 standard errors of 0, so do the
+    means of every class row, neighbouring clauses are uncorrelated, and another seed gives another
+    draw; with NEGATIVE_CLAUSES == 0 every weight is 1."""
+    cfg = o.Config(classes=10, clauses=20000, literals=8, threshold=10)
+    _, w = o.prepare(cfg, seed=42)
+    assert w.shape == (10, 20000) and w.dtype == np.int32
+    assert set(np.unique(w)) == {-1, 1}
+    n = w.size
+    assert abs(w.mean()) < 5.0 / np.sqrt(n)
+    assert np.all(np.abs(w.mean(axis=1)) < 5.0 / np.sqrt(w.shape[1]))
+    assert abs((w[:, 1:] * w[:, :-1]).mean()) < 5.0 / np.sqrt(n)   # clause c against clause c + 1
+    assert abs((w[1:, :] * w[:-1, :]).mean()) < 5.0 / np.sqrt(n)   # class k against class k + 1
+    _, other = o.prepare(cfg, seed=43)
+    assert abs((w * other).mean()) < 5.0 / np.sqrt(n)
+    _, later = o.prepare(cfg, seed=42, step=7)  # (the draw is addressed by the training step as well)
+    assert abs((w * later).mean()) < 5.0 / np.sqrt(n)
+    _, ones = o.prepare(o.Config(classes=3, clauses=50, literals=8, threshold=10, negative_clauses=0), seed=42)
+    assert np.array_equal(ones, np.ones((3, 50), dtype=np.int32))
+
+
 def test_select_clause_updates_case_table():
     """Deterministic corners of kernels.py:371-402 (probabilities 0 and 1)."""
     T = 10

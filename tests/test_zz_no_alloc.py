@@ -56,6 +56,33 @@ def test_two_calls_in_a_row_the_second_smaller_equal_gtm_score(depth, tiles):
     assert np.array_equal(want_small, o.score(small_model, small_graphs, range(2, 9)))
     # and the first again, after the smaller one
     assert np.array_equal(score_static(big, 0, 60, 16), want_big)
+    # what the entry point is for: its calls leave the device's free memory as it was (the output
+    # tensors exist before the first reading; torch's allocator is not asked for anything in between),
+    # also while launch timing is switched on - this entry point records no events
+    out_big = torch.empty(60 * big.cfg.classes, dtype=torch.int32, device="cuda")
+    out_small = torch.empty(7 * small.cfg.classes, dtype=torch.int32, device="cuda")
+    st_big, st_small = big.state(), small.state()
+    torch.cuda.synchronize()
+    _abi.call("gtm_profile_enable", 1)
+    try:
+        free_before = torch.cuda.mem_get_info()[0]
+        for _ in range(3):
+            _abi.call("gtm_score_static", ctypes.byref(big.acfg), ctypes.byref(big.dg.desc), ctypes.byref(st_big), 0, 60,
+                      16, _ptr(out_big), _stream())
+            _abi.call("gtm_score_static", ctypes.byref(small.acfg), ctypes.byref(small.dg.desc), ctypes.byref(st_small),
+                      2, 7, 4, _ptr(out_small), _stream())
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        name, launches, total = ctypes.c_char_p(), ctypes.c_int32(), ctypes.c_double()
+        _abi.call("gtm_profile_read", ctypes.byref(name), ctypes.byref(launches), ctypes.byref(total))
+        assert launches.value == 0  # nothing was timed, and the switch is still on for other callers:
+        big.score(0, 60, 16)
+        _abi.call("gtm_profile_read", ctypes.byref(name), ctypes.byref(launches), ctypes.byref(total))
+        assert launches.value > 0
+    finally:
+        _abi.call("gtm_profile_enable", 0)
+    assert np.array_equal(out_big.cpu().numpy().reshape(60, -1), want_big)
+    assert np.array_equal(out_small.cpu().numpy().reshape(7, -1), want_small)
 
 
 def test_sizes_beyond_the_static_scratch_are_refused():
