@@ -16,6 +16,7 @@
 #include "../../include/gtm_abi.h"
 #include "philox.h"
 #include "score_tiles.h"
+#include "score_paired.h"
 
 namespace {
 
@@ -65,11 +66,15 @@ int check_launch(const char *what) {
     X(NO_DEEP_PERSISTENT_FIT) \
     X(NO_DIRECT_FIT) \
     X(NO_FUSED_MESSAGES) \
+    X(NO_HALF_ROWS) \
     X(NO_HALF_TILES) \
     X(NO_LISTS_IN_LDS) \
     X(NO_NARROW_TWO_PHASE) \
+    X(NO_PAIRED_LAYERS) \
     X(NO_PERSISTENT_FIT) \
     X(NO_SMALL_FIT) \
+    X(NO_TILE_LINE) \
+    X(TILE_LINE_GROUPS) \
     X(NO_TILE_PACK) \
     X(NO_TILE_TRANSFORM) \
     X(NO_TWO_PHASE) \
@@ -653,6 +658,9 @@ struct ScoreWs {
     uint32_t *sent, *got;     // [tiles per launch][tw * 32 node slots][ceil(M / 32)]  (tile path, depth > 1)
     uint32_t *message_rows;   // [tiles per launch][M + 2][tw]  (tile path, depth > 1)
     uint32_t *bit_start, *bit_cursor, *bit_clauses;  // [M + 1], [M], [C * MB]: the clauses of every message bit (tile path, depth > 1)
+    uint32_t *alive[2];       // [tiles per launch][PAIRED_STREAMS][alive_stride] clauses still true somewhere in a tile, layer to layer
+    int alive_stride;
+    TileSegment *segments;    // [tiles + 2 * TILE_SEGMENTS_MAX_SHARES] which clauses of which tile a workgroup takes (half tiles)
     size_t vector_words;      // words of sent (and of got)
     uint32_t *inc_t;          // [max(LA,MC)][C]
     uint32_t *bitmap_a;       // [batch][C][NC]
@@ -662,8 +670,8 @@ struct ScoreWs {
 };
 
 // Length of a compiled clause: header + type row + literals + what fills its two parts up to whole
-// 8-entry blocks, padded to 32 entries, + 32 entries that the kernel may fetch ahead unused.
-int clause_list_stride(int literals) { return ((literals + 2 + 14 + 31) & ~31) + 32; }
+// 8-entry blocks, padded to a whole number of 128-entry windows, + 32 entries that a kernel may fetch ahead unused.
+int clause_list_stride(int literals) { return ((literals + 2 + 14 + 127) & ~127) + 32; }
 
 // Tiles one launch group covers when the caller asks for `batch` graphs at a time.
 int tiles_per_batch(const TileGeom &tg, int batch) { return (batch + tg.gpt - 1) / tg.gpt; }
@@ -683,6 +691,8 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base,
     w.list_stride = clause_list_stride(cfg->literals);
     w.lists = (uint32_t *)take((size_t)d.C * w.list_stride * 4);
     w.wt = (int32_t *)take((size_t)d.C * d.K * 4);
+    if (tg && cfg->depth == 1 && tg->half)
+        w.segments = (TileSegment *)take(((size_t)tg->n_tiles + 2 * TILE_SEGMENTS_MAX_SHARES) * sizeof(TileSegment));
     if (tg && cfg->depth == 1 && !keep_rows) {
         w.bytes = off;
         return w;
@@ -705,6 +715,8 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base,
         w.bit_start = (uint32_t *)take(((size_t)d.M + 1) * 4);
         w.bit_cursor = (uint32_t *)take((size_t)d.M * 4);
         w.bit_clauses = (uint32_t *)take((size_t)d.C * d.MB * 4);
+        w.alive_stride = paired_alive_stride(d.C);
+        for (uint32_t *&list : w.alive) list = (uint32_t *)take(n_tiles * PAIRED_STREAMS * w.alive_stride * 4);
         w.bytes = off;
         return w;
     }
@@ -1023,8 +1035,46 @@ int launch_two_phase(const TileLayerArgs &a, int n_tiles, int la4, bool last, hi
     }
 }
 
+// Compute units of the current device (0 if it cannot be told).
+int compute_units() {
+    static thread_local int cus_of[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cus_of[dev] == 0) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0;
+        }
+        cus_of[dev] = cus;
+    }
+    return cus_of[dev];
+}
+
+// The tiles of a launch of k_tile_two_phase_half shared out among the compute units (tile_segments_block
+// in score_tiles.h) - when they do not fill a whole number of rounds of the chip, and a share is at least 64
+// clauses (a share stages its tile).  GTM_NO_TILE_LINE turns it off; GTM_TILE_LINE_GROUPS = n (tests) cuts the
+// tiles into n shares whatever the device has.  cus == 0 in the result: one workgroup per tile.
+SegmentPlan plan_segments(const TileLayerArgs &a, int n_tiles, TileSegment *segments) {
+    SegmentPlan sp{};
+    int cus = compute_units();
+    bool shared_out = cus > 0 && n_tiles % cus != 0 && (int64_t)(n_tiles % cus) * a.C / cus >= 64 && !tune(T_NO_TILE_LINE);
+    if (const char *e = tune(T_TILE_LINE_GROUPS)) {
+        cus = atoi(e);
+        shared_out = cus >= 1;
+    }
+    if (!shared_out || !segments || cus > TILE_SEGMENTS_MAX_SHARES) return sp;
+    sp.n_tiles = n_tiles, sp.C = a.C, sp.cus = cus, sp.gpt = a.tg.gpt, sp.K = a.K, sp.tile0 = a.tile0;
+    sp.first_graph = a.first_graph, sp.n_graphs = a.n_graphs, sp.segments = segments, sp.class_sum = a.class_sum;
+    return sp;
+}
+
 template <int NW, int LW, int LA4, bool LAST, bool FULL>
-int launch_two_phase_half_as(const TileLayerArgs &a, int n_tiles, hipStream_t st) {
+int launch_two_phase_half_as(const TileLayerArgs &a_in, int n_tiles, const SegmentPlan *sp, hipStream_t st) {
+    TileLayerArgs a = a_in;
+    const bool shared_out = LAST && sp && sp->cus > 0;
+    a.segments = shared_out ? sp->segments : nullptr;
+    const int groups = shared_out ? tile_segment_count(n_tiles, sp->cus) : n_tiles;
     const size_t lds = tile_lds_bytes(a.tg.rows - LA4 * 64, a.tg, a.K);  // the rows of the negated literals stay out
     static thread_local size_t lds_set = 48 * 1024;
     if (lds > lds_set) {
@@ -1034,38 +1084,38 @@ int launch_two_phase_half_as(const TileLayerArgs &a, int n_tiles, hipStream_t st
         lds_set = lds;
     }
     profile_start(LAST ? "k_tile_two_phase_half<score>" : "k_tile_two_phase_half<layer0>", st);
-    hipLaunchKernelGGL((k_tile_two_phase_half<NW, LW, LA4, LAST, FULL>), dim3(n_tiles), dim3(NW * 64), lds, st, a);
+    hipLaunchKernelGGL((k_tile_two_phase_half<NW, LW, LA4, LAST, FULL>), dim3(groups), dim3(NW * 64), lds, st, a);
     if (int rc = check_launch("tile_two_phase_half")) return rc;
     profile_stop(st);
     return GTM_OK;
 }
 
 template <int NW, int LW, int LA4>
-int launch_two_phase_half_la(const TileLayerArgs &a, int n_tiles, bool last, hipStream_t st) {
+int launch_two_phase_half_la(const TileLayerArgs &a, int n_tiles, bool last, const SegmentPlan *segments, hipStream_t st) {
     const bool full = a.tg.tw == 64 * LW;
     if (last)
-        return full ? launch_two_phase_half_as<NW, LW, LA4, true, true>(a, n_tiles, st)
-                    : launch_two_phase_half_as<NW, LW, LA4, true, false>(a, n_tiles, st);
-    return full ? launch_two_phase_half_as<NW, LW, LA4, false, true>(a, n_tiles, st)
-                : launch_two_phase_half_as<NW, LW, LA4, false, false>(a, n_tiles, st);
+        return full ? launch_two_phase_half_as<NW, LW, LA4, true, true>(a, n_tiles, segments, st)
+                    : launch_two_phase_half_as<NW, LW, LA4, true, false>(a, n_tiles, segments, st);
+    return full ? launch_two_phase_half_as<NW, LW, LA4, false, true>(a, n_tiles, segments, st)
+                : launch_two_phase_half_as<NW, LW, LA4, false, false>(a, n_tiles, segments, st);
 }
 
 template <int NW, int LW>
-int launch_two_phase_half_lw(const TileLayerArgs &a, int n_tiles, int la4, bool last, hipStream_t st) {
+int launch_two_phase_half_lw(const TileLayerArgs &a, int n_tiles, int la4, bool last, const SegmentPlan *segments, hipStream_t st) {
     switch (la4) {
-        case 1: return launch_two_phase_half_la<NW, LW, 1>(a, n_tiles, last, st);
-        case 2: return launch_two_phase_half_la<NW, LW, 2>(a, n_tiles, last, st);
-        case 3: return launch_two_phase_half_la<NW, LW, 3>(a, n_tiles, last, st);
-        default: return launch_two_phase_half_la<NW, LW, 4>(a, n_tiles, last, st);
+        case 1: return launch_two_phase_half_la<NW, LW, 1>(a, n_tiles, last, segments, st);
+        case 2: return launch_two_phase_half_la<NW, LW, 2>(a, n_tiles, last, segments, st);
+        case 3: return launch_two_phase_half_la<NW, LW, 3>(a, n_tiles, last, segments, st);
+        default: return launch_two_phase_half_la<NW, LW, 4>(a, n_tiles, last, segments, st);
     }
 }
 
-int launch_two_phase_half(const TileLayerArgs &a, int n_tiles, int la4, bool last, hipStream_t st) {
+int launch_two_phase_half(const TileLayerArgs &a, int n_tiles, int la4, bool last, const SegmentPlan *segments, hipStream_t st) {
     constexpr int NW = 16;
     switch (a.tg.lw) {
-        case 1: return launch_two_phase_half_lw<NW, 1>(a, n_tiles, la4, last, st);
-        case 2: return launch_two_phase_half_lw<NW, 2>(a, n_tiles, la4, last, st);
-        default: return launch_two_phase_half_lw<NW, 4>(a, n_tiles, la4, last, st);
+        case 1: return launch_two_phase_half_lw<NW, 1>(a, n_tiles, la4, last, segments, st);
+        case 2: return launch_two_phase_half_lw<NW, 2>(a, n_tiles, la4, last, segments, st);
+        default: return launch_two_phase_half_lw<NW, 4>(a, n_tiles, la4, last, segments, st);
     }
 }
 
@@ -1118,6 +1168,33 @@ int launch_two_phase_wide(const TileLayerArgs &a, int n_tiles, int LA, bool stag
     }
 }
 
+// Two clauses per wave on narrow tiles (score_paired.h).
+template <int SRC, bool LAST>
+int launch_paired_as(const TileLayerArgs &a, const PairedArgs &x, int n_tiles, hipStream_t st) {
+    const size_t lds = paired_lds_bytes(a.tg, a.K, paired_rows_lds(SRC, a.M, x.hv, x.n_types));
+    static thread_local size_t lds_set = 48 * 1024;
+    if (lds > lds_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)k_tile_layer_paired<SRC, LAST>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
+        lds_set = lds;
+    }
+    profile_start(SRC == ROWS_HALF ? (LAST ? "k_tile_layer_paired<score>" : "k_tile_layer_paired<layer0>")
+                                   : (LAST ? "k_tile_layer_paired<messages, score>" : "k_tile_layer_paired<messages>"),
+                  st);
+    hipLaunchKernelGGL((k_tile_layer_paired<SRC, LAST>), dim3(n_tiles), dim3(PAIRED_WAVES * 64), lds, st, a, x);
+    if (int rc = check_launch("tile_layer_paired")) return rc;
+    profile_stop(st);
+    return GTM_OK;
+}
+
+int launch_paired(const TileLayerArgs &a, const PairedArgs &x, int n_tiles, int src, bool last, hipStream_t st) {
+    if (src == ROWS_HALF)
+        return last ? launch_paired_as<ROWS_HALF, true>(a, x, n_tiles, st) : launch_paired_as<ROWS_HALF, false>(a, x, n_tiles, st);
+    return last ? launch_paired_as<ROWS_MESSAGES, true>(a, x, n_tiles, st)
+                : launch_paired_as<ROWS_MESSAGES, false>(a, x, n_tiles, st);
+}
+
 // Layer 0 can run in two phases (k_tile_two_phase) on tiles of whole-word graph slots staged in
 // LDS when a node has 4, 8, 12 or 16 literal words.  GTM_NO_TWO_PHASE (tuning aid) turns it off.
 bool two_phase_layer0(const Dims &d, const gtm_graphs *g, const TileGeom &tg) {
@@ -1146,12 +1223,35 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     // any other tile of whole-word slots whose row offsets fit the 16-bit entries: k_tile_two_phase_wide
     const bool wide = !narrow && tg.slot_words > 0 && (int64_t)tg.rows * tg.tw / 4 < 65536 && !tune(T_NO_TWO_PHASE);
     const bool two_phase = narrow || wide;
+    // Narrow tiles: two clauses per wave (score_paired.h) for the message layers, and for layer 0 when the data
+    // set's negated literals are the complements of its positive ones, so that the positive rows alone, which
+    // fit in LDS, will do.  GTM_NO_PAIRED_LAYERS / GTM_NO_HALF_ROWS (tuning and test aids) turn them off.
+    const size_t lds_limit = 160 * 1024;
+    const int hv = cfg->literals / 2;
+    const bool paired = paired_geometry(tg) && !tune(T_NO_PAIRED_LAYERS);
+    const bool paired_messages = paired && layers > 1 && paired_lds_bytes(tg, d.K, tile_message_rows(d.M)) <= lds_limit;
+    const bool half_rows0 = paired && !tg.half && (g->flags & GTM_GRAPHS_COMPLEMENTARY) && cfg->literals % 2 == 0 &&
+                            paired_lds_bytes(tg, d.K, hv + g->number_of_node_types + 1) <= lds_limit &&
+                            !tune(T_NO_HALF_ROWS);
     // compiled clause: 8 words of packed 16-bit row entries (16 words of byte offsets on half tiles) + the include words
-    const int stride0 = tg.half ? 16 + d.LA : two_phase ? 8 + d.LA : w.list_stride;
-    if (tg.half)
-        hipLaunchKernelGGL(k_compile_clauses_half, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C,
-                           d.LA, d.B, d.filter, cfg->literals, g->number_of_node_types, tg.tw, order, w.lists, stride0,
-                           d.K, layers == 1 ? s->clause_weights : nullptr, w.wt);
+    const int stride0 = half_rows0 ? w.list_stride : tg.half ? 16 + d.LA : two_phase ? 8 + d.LA : w.list_stride;
+    SegmentPlan plan{};
+    if (half_rows0)
+        // rows as k_tile_layer_paired<ROWS_HALF> stages them: positive literals, node types, all ones
+        hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C,
+                           d.LA, d.B, d.filter, cfg->literals, hv, g->number_of_node_types, hv, hv + g->number_of_node_types,
+                           tg.tw, w.list_stride, order, w.lists, d.K, layers == 1 ? s->clause_weights : nullptr, w.wt);
+    else if (tg.half) {
+        if (layers == 1 && !tr) {  // one launch over every tile of the range: its tiles may be shared out among the CUs
+            TileLayerArgs range{};
+            range.tg = tg, range.C = d.C, range.K = d.K, range.tile0 = first / tg.gpt, range.first_graph = first;
+            range.n_graphs = n_graphs, range.class_sum = class_sum;
+            plan = plan_segments(range, (first + n_graphs - 1) / tg.gpt - range.tile0 + 1, w.segments);
+        }
+        hipLaunchKernelGGL(k_compile_clauses_half, dim3(blocks_for(d.C, TPB / 64) + (plan.cus > 0 ? 1u : 0u)), dim3(TPB), 0, st,
+                           s->ta_state, d.C, d.LA, d.B, d.filter, cfg->literals, g->number_of_node_types, tg.tw, order, w.lists,
+                           stride0, d.K, layers == 1 ? s->clause_weights : nullptr, w.wt, plan);
+    }
     else if (two_phase)
         hipLaunchKernelGGL(k_compile_clauses_two_phase, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state,
                            d.C, d.LA, d.B, d.filter, cfg->literals, g->number_of_node_types, cfg->literals,
@@ -1189,10 +1289,22 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     a.xpos = tg.half ? g->tiles + tiles_xpos_offset_words(tg, cfg->literals) : nullptr;
     a.walk_factor = 2;
     if (const char *e = tune(T_WIDE_WALK_FACTOR)) a.walk_factor = std::max(1, atoi(e));  // (tuning aid)
+    PairedArgs px{};
+    px.alive_stride = w.alive_stride;
+    px.hv = hv;
+    px.n_types = g->number_of_node_types;
+    const uint32_t *alive_now = nullptr;  // what the last paired layer left for the next one
     auto layer0 = [&](int n_tiles, bool last) {
         a.lists = w.lists;
         a.stride = stride0;
-        if (tg.half) return launch_two_phase_half(a, n_tiles, d.LA / 4, last, st);
+        if (half_rows0) {
+            px.alive_in = nullptr;
+            px.alive_out = !last && paired_messages ? w.alive[0] : nullptr;
+            alive_now = px.alive_out;
+            return launch_paired(a, px, n_tiles, ROWS_HALF, last, st);
+        }
+        alive_now = nullptr;
+        if (tg.half) return launch_two_phase_half(a, n_tiles, d.LA / 4, last, &plan, st);
         if (narrow) return launch_two_phase(a, n_tiles, d.LA / 4, last, st);
         if (wide) return launch_two_phase_wide(a, n_tiles, d.LA, tg.stage0 != 0, last, st);
         return launch_tile_layer(a, n_tiles, tg.stage0 ? ROWS_STAGED : ROWS_GLOBAL, last, st);
@@ -1243,6 +1355,15 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit: %s", hipGetErrorString(e));
         node_messages_lds_raised = true;
     }
+    // the clause evaluation of message layer l on the rows just built (a.lists, a.stride, a.longest_list are set)
+    auto message_layer = [&](int n_tiles, int l) {
+        const bool last = l == layers - 1 && !tr;
+        if (!paired_messages) return launch_tile_layer(a, n_tiles, ROWS_MESSAGES, last, st);
+        px.alive_in = alive_now;
+        px.alive_out = last || l == layers - 1 ? nullptr : w.alive[alive_now == w.alive[0] ? 1 : 0];
+        alive_now = px.alive_out;
+        return launch_paired(a, px, n_tiles, ROWS_MESSAGES, last, st);
+    };
     for (int t0 = tile_first; t0 <= tile_last; t0 += tiles_per_launch) {
         const int n_tiles = tile_last - t0 + 1 < tiles_per_launch ? tile_last - t0 + 1 : tiles_per_launch;
         a.tile0 = t0;
@@ -1264,7 +1385,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                 a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
                 a.stride = w.message_list_stride;
                 a.longest_list = w.longest_list + (l - 1);
-                if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1 && !tr, st)) return rc;
+                if (int rc = message_layer(n_tiles, l)) return rc;
                 continue;
             }
             profile_start("k_tile_node_messages + k_tile_edge_messages + k_tile_pack_messages", st);
@@ -1299,7 +1420,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
             a.stride = w.message_list_stride;
             a.longest_list = w.longest_list + (l - 1);
-            if (int rc = launch_tile_layer(a, n_tiles, ROWS_MESSAGES, l == layers - 1 && !tr, st)) return rc;
+            if (int rc = message_layer(n_tiles, l)) return rc;
         }
         if (tr) {
             const int g_lo = std::max(first, t0 * tg.gpt), g_hi = std::min(first + n_graphs, (t0 + n_tiles) * tg.gpt);
@@ -1876,9 +1997,9 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     // group measured best on 2,000 and 2,500 clauses), but a group gets at least 8 where their
     // automata fit in LDS.
     auto lds_bytes = [&](int per_group) {
-        return (2 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group +
-                2 * (size_t)d.K + 5 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K + 2 * (size_t)p.x_words +
-                (size_t)cfg->literals + 8 * (size_t)d.K) * 4;
+        return (3 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group +
+                2 * (size_t)d.K + 5 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K + 3 * (size_t)p.x_words +
+                (size_t)cfg->literals + 9 * (size_t)d.K) * 4;
     };
     const size_t lds_limit = 150 * 1024;
     int per_group = (d.C + cus - 1) / cus;

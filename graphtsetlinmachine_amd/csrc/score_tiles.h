@@ -312,7 +312,8 @@ __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int 
     const int neg_padded = (n_neg + 7) & ~7;
     for (int i = n_neg + lane; i < neg_padded; i += 64) list[plain_padded + i] = ones + row_bytes;
     const int padded = plain_padded + neg_padded;
-    const int fill_to = padded < 32 ? 32 : (padded + 15) & ~15;
+    // (to a whole number of 128-entry windows: k_tile_layer_paired takes a list a window at a time)
+    const int fill_to = padded < 32 ? 128 : (padded + 127) & ~127;
     for (int i = padded + lane; i < fill_to; i += 64) list[i] = ones;
     // entry 0: blocks of rows to AND | blocks of rows whose complements to AND << 16
     if (lane == 0) list[0] = (uint32_t)(plain_padded >> 3) | ((uint32_t)(neg_padded >> 3) << 16);
@@ -387,6 +388,8 @@ struct TileLayerArgs {
     const uint32_t *xpos;   // [tiles][tw * 32 slots][LA / 2]: the positive literal words by node slot (half tiles)
     int walk_factor;        // k_tile_two_phase_wide: a clause's rows are all walked when more than this many slots per
                             // literal survive phase 1
+    const struct TileSegment *segments;  // k_tile_two_phase_half: which clauses of which tile each workgroup takes, or NULL:
+                            // workgroup b takes tile b whole
     int lists_in_lds;       // message layers: LDS holds TILE_LIST_LDS_WORDS more words per wave for the clause lists
     const uint32_t *longest_list;  // entries of the layer's longest list (message layers)
 };
@@ -1677,6 +1680,69 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
 
 
 // ---------------------------------------------------------------------------
+// Sharing the tiles of a launch out among the compute units when they do not fill a whole number of
+// rounds (477 tiles on 256 CUs: a second round that leaves 35 CUs idle).  The first R * cus tiles
+// (R = tiles / cus) are taken whole, one workgroup each.  The (tile, clause) pairs of the remaining
+// tiles, tile after tile, are cut into `cus` equal shares; a share lies in one tile or straddles two,
+// so it is at most two segments, each a workgroup of its own: 2 * cus more workgroups (some empty).
+// Workgroups are handed to the CUs in the order of their numbers as CUs fall free, so the first
+// segments come ordered by size, smallest first, and the second segments in the same order of their
+// shares - largest first, since the two add up to a share: whoever finishes a short first segment
+// finds a long second one next in line, and all finish together.  The table is made by one block,
+// which also clears the class sums of the graphs of the shared tiles, to which their workgroups add.
+struct TileSegment {
+    int tile_local, c_begin, c_end;
+};
+
+constexpr int TILE_SEGMENTS_MAX_SHARES = 1024;
+
+// What the table is made from; cus == 0: no table, one workgroup per tile.
+struct SegmentPlan {
+    int n_tiles, C, cus, gpt, K, tile0, first_graph, n_graphs;
+    TileSegment *segments;  // [tile_segment_count(n_tiles, cus)]
+    int32_t *class_sum;     // [n_graphs][K]
+};
+
+inline int tile_segment_count(int n_tiles, int cus) { return n_tiles / cus * cus + 2 * cus; }
+
+// The work of ONE block of `threads` threads (it runs as an extra block of the launch that compiles the
+// clauses, so that it costs the step no time of its own).
+__device__ __forceinline__ void tile_segments_block(const SegmentPlan &sp, int tid, int threads) {
+    __shared__ int first_len[TILE_SEGMENTS_MAX_SHARES];
+    const int C = sp.C, cus = sp.cus;
+    const int whole = sp.n_tiles / cus * cus, rest = sp.n_tiles - whole;
+    for (int b = tid; b < whole; b += threads) sp.segments[b] = TileSegment{b, 0, C};
+    const long long pairs = (long long)rest * C;
+    // share j = pairs [j * pairs / cus, (j + 1) * pairs / cus)
+    auto share = [&](int j, int *tile_a, int *at, int *len_a, int *len_b) {
+        const long long from = pairs * j / cus, to = pairs * (j + 1) / cus;
+        *tile_a = (int)(from / C);
+        *at = (int)(from - (long long)*tile_a * C);
+        *len_a = to - from < (long long)(C - *at) ? (int)(to - from) : C - *at;
+        *len_b = (int)(to - from) - *len_a;
+    };
+    for (int j = tid; j < cus; j += threads) {
+        int tile_a, at, len_a, len_b;
+        share(j, &tile_a, &at, &len_a, &len_b);
+        first_len[j] = len_a;
+    }
+    __syncthreads();
+    for (int j = tid; j < cus; j += threads) {
+        int tile_a, at, len_a, len_b;
+        share(j, &tile_a, &at, &len_a, &len_b);
+        int rank = 0;
+        for (int k = 0; k < cus; ++k) rank += first_len[k] < len_a || (first_len[k] == len_a && k < j);
+        sp.segments[whole + rank] = TileSegment{whole + tile_a, at, at + len_a};
+        sp.segments[whole + cus + rank] = TileSegment{whole + tile_a + 1, 0, len_b};  // (empty when the share lies in one tile)
+    }
+    // the class sums of the graphs of the shared tiles start at zero
+    const long long g_lo = (long long)(sp.tile0 + whole) * sp.gpt, g_hi = (long long)(sp.tile0 + sp.n_tiles) * sp.gpt;
+    const long long first = sp.first_graph, end = first + sp.n_graphs;
+    for (long long i = (g_lo > first ? g_lo : first) * sp.K + tid; i < (g_hi < end ? g_hi : end) * sp.K; i += threads)
+        sp.class_sum[i - first * sp.K] = 0;
+}
+
+// ---------------------------------------------------------------------------
 // The two-phase layer 0 on HALF tiles: LDS holds only the rows of the positive
 // literals (plus the node-type rows and the all-ones row), and a negated literal
 // l + hv is evaluated as the complement of row l.  That is exact where the data
@@ -1705,8 +1771,12 @@ struct alignas(16) Entries16 {
 __global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C, int chunks, int B, uint32_t filter,
                                        int literals, int n_types, int tw, const uint32_t *__restrict__ order,
                                        uint32_t *__restrict__ records, int record_words, int K,
-                                       const int32_t *__restrict__ weights, int32_t *__restrict__ wt) {
+                                       const int32_t *__restrict__ weights, int32_t *__restrict__ wt, SegmentPlan sp) {
     __shared__ uint32_t chosen_of_wave[4][16];
+    if (sp.cus > 0 && blockIdx.x == gridDim.x - 1) {  // the launch's extra block: which workgroup takes what (see above)
+        tile_segments_block(sp, threadIdx.x, blockDim.x);
+        return;
+    }
     const int lane = threadIdx.x & 63;
     const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (c >= C) return;  // whole waves leave; no barrier below
@@ -1797,11 +1867,20 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
     const int rows_lds = tg.rows - hv;           // + node types + all ones
     uint32_t *bt = lds;
     int32_t *sums = (int32_t *)(lds + (size_t)rows_lds * tw + TILE_LDS_PAD_WORDS);
-    const int tile = a.tile0 + blockIdx.x;
+    // This workgroup's share: a whole tile, or - with a table of segments (tile_segments_block above) - clauses
+    // [c_begin, c_end) of a tile whose other clauses other workgroups take.
+    int tile_local = blockIdx.x, c_begin = 0, c_end = C;
+    if (a.segments) {
+        const TileSegment seg = a.segments[blockIdx.x];
+        tile_local = seg.tile_local, c_begin = seg.c_begin, c_end = seg.c_end;
+        if (c_begin >= c_end) return;  // (an empty share: uniform over the workgroup)
+    }
+    const bool whole_tile = c_begin == 0 && c_end == C;
+    const int tile = a.tile0 + tile_local;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    uint32_t *bitmap = a.bitmap + (int64_t)blockIdx.x * C * tw;
+    uint32_t *bitmap = a.bitmap + (int64_t)tile_local * C * tw;
 
     {  // the tile's positive rows, then its node-type rows and the all-ones row -> LDS
         const uint4 *src = reinterpret_cast<const uint4 *>(a.tiles + (int64_t)tile * tg.rows * tw);
@@ -2066,7 +2145,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
     const int64_t rec_step = (int64_t)NWAVES * a.stride;
     const int wt_step = NWAVES * K;
     const int64_t truth_step = (int64_t)NWAVES * tw * 4;
-    const int first = wave < C ? wave : 0;
+    const int first = c_begin + wave < c_end ? c_begin + wave : c_begin;
     const uint32_t *rec_a = a.lists + (int64_t)first * a.stride;
     const int32_t *wt_a = LAST ? a.wt + (int64_t)first * K : nullptr;
     char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
@@ -2074,8 +2153,8 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
     Words<LA> ma, mb;
     Pending pa, pb;
     pa.live = pb.live = false;
-    for (int c = wave; c < C; c += 2 * NWAVES) {
-        const bool has_b = c + NWAVES < C;
+    for (int c = c_begin + wave; c < c_end; c += 2 * NWAVES) {
+        const bool has_b = c + NWAVES < c_end;
         const uint32_t *rec_b = has_b ? rec_a + rec_step : rec_a;
         const int32_t *wt_b = LAST ? (has_b ? wt_a + wt_step : wt_a) : nullptr;
         char *truth_b = has_b ? truth_a + truth_step : truth_a;
@@ -2083,7 +2162,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         const Entries16 eb = *reinterpret_cast<const Entries16 *>(rec_b);
         begin(pa, ea, wt_a, truth_a);
         finish(pb, mb);
-        const bool has_a = c + 2 * NWAVES < C;
+        const bool has_a = c + 2 * NWAVES < c_end;
         rec_a = has_a ? rec_b + rec_step : rec_b;
         if (LAST) wt_a = has_a ? wt_b + wt_step : wt_b;
         truth_a = has_a ? truth_b + truth_step : truth_b;
@@ -2101,8 +2180,13 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
     const int64_t g0 = (int64_t)tile * tg.gpt;
     for (int i = tid; i < tg.gpt * K; i += NT) {
         int64_t g = g0 + i / K;
-        if (g >= a.first_graph && g < (int64_t)a.first_graph + a.n_graphs)
-            a.class_sum[(g - a.first_graph) * K + (i % K)] = sums[i];
+        if (g >= a.first_graph && g < (int64_t)a.first_graph + a.n_graphs) {
+            int32_t *out = &a.class_sum[(g - a.first_graph) * K + (i % K)];
+            if (whole_tile)
+                *out = sums[i];
+            else if (sums[i] != 0)
+                atomicAdd(out, sums[i]);  // a tile shared with other workgroups (tile_segments_block cleared its sums)
+        }
     }
 }
 

@@ -181,3 +181,83 @@ def test_a_whole_epoch_of_the_convolutional_configuration_follows_the_c_oracle(c
     sums = tm.score(wl.graphs_test)
     assert np.array_equal(sums, oc.score(last, wl.graphs_test, threads=min(16, oc.threads_available())))
     assert (sums.argmax(axis=1) == wl.Y_test).mean() > 0.95
+
+
+TRAINED_COLOUR = {}
+
+
+def trained_colour_state():
+    """The colour configuration (8,000 clauses, three banks of 2,048 literals, 841 nodes, depth 3) after
+    4,096 training examples on the GPU: clauses of a few dozen literals that still hold at many nodes,
+    the regime the scoring and training kernels of this configuration spend their time in - a freshly
+    initialised model (every clause empty) or one after a handful of examples (a thousand literals per
+    clause) does not reach it.  Trained once per test session."""
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    if not TRAINED_COLOUR:
+        wl = workloads.colour_convolution(n_train=4096 + 48, n_test=64)
+        np.random.seed(42)
+        tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
+        tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True, examples=(0, 4096))
+        TRAINED_COLOUR.update(wl=wl, tm=tm, state=tm.save())
+    return TRAINED_COLOUR["wl"], TRAINED_COLOUR["tm"], TRAINED_COLOUR["state"]
+
+
+def oracle_at(tm, state, graphs):
+    model = oracle_twin(tm, graphs)
+    model.ta_state = state["ta_state"].reshape(model.ta_state.shape).copy()
+    model.message_ta_state = [b.reshape(model.message_ta_state[0].shape).copy() for b in state["message_ta_state"]]
+    model.clause_weights = state["clause_weights"].reshape(model.clause_weights.shape).copy()
+    model.step = int(state["rng_step"])
+    return model
+
+
+@pytest.mark.parametrize("scoring", ["default", "rows-in-place", "full-walk"])
+def test_scoring_the_colour_configuration_at_a_trained_state(scoring, tune):
+    """Every scoring path that this shape can take, on the trained state, against the C oracle."""
+    wl, tm, state = trained_colour_state()
+    included = np.unpackbits(state["ta_state"].reshape(8000, 64, 8)[:, :, 7].copy().view(np.uint8)).sum() / 8000
+    assert 8 < included < 400, "not the regime this test is for: %.1f literals per clause" % included
+    if scoring == "rows-in-place":
+        tune("GTM_NO_HALF_ROWS", "1")    # layer 0 on all 2,050 rows read in place, candidates tested on their own words
+    elif scoring == "full-walk":
+        tune("GTM_NO_HALF_ROWS", "1")
+        tune("GTM_NO_TWO_PHASE", "1")    # layer 0 as a walk of every literal's row
+    model = oracle_at(tm, state, wl.graphs_test)
+    want = oc.score(model, wl.graphs_test, threads=min(16, oc.threads_available()))
+    tm._test_graphs = None  # (the tiles are built per path)
+    assert np.array_equal(tm.score(wl.graphs_test), want)
+    assert len(np.unique(want.argmax(axis=1))) > 1  # the state tells classes apart
+
+
+@pytest.mark.parametrize("training", ["one-launch", "one-launch-small-windows", "launches-per-example"])
+def test_training_the_colour_configuration_from_a_trained_state(training, tune):
+    """48 more examples from the trained state, on every training path this shape can take, against the
+    C oracle: all three banks and the weights bit for bit, and the class sums afterwards."""
+    from graphtsetlinmachine_amd.tm import MultiClassGraphTsetlinMachine
+
+    wl, tm, state = trained_colour_state()
+    if "model_after" not in TRAINED_COLOUR:
+        model = oracle_at(tm, state, wl.graphs_train)
+        oc.fit(model, wl.graphs_train, o.encode_labels(wl.Y_train, tm.number_of_outputs, tm.T),
+               indices=range(4096, 4096 + 48), threads=min(16, oc.threads_available()))
+        TRAINED_COLOUR["model_after"] = model
+    model = TRAINED_COLOUR["model_after"]
+    if training == "one-launch-small-windows":
+        tune("GTM_FIT_DEEP_WINDOW_ROWS", "128")
+    elif training == "launches-per-example":
+        tune("GTM_NO_DEEP_PERSISTENT_FIT", "1")
+    np.random.seed(42)
+    again = MultiClassGraphTsetlinMachine(**wl.params, seed=1)
+    again.load(state)
+    assert again.step == 4096 and again.seed == 42
+    again.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True, examples=(4096, 48))
+    saved = again.save()
+    assert np.array_equal(saved["clause_weights"].reshape(model.clause_weights.shape), model.clause_weights)
+    assert np.array_equal(saved["ta_state"], model.ta_state.reshape(-1))
+    for got, want in zip(saved["message_ta_state"], model.message_ta_state):
+        assert np.array_equal(got, want.reshape(-1))
+    assert not np.array_equal(saved["ta_state"], state["ta_state"])  # the 48 examples did move the automata
+    few = list(range(8))
+    scorer = oracle_at(again, saved, wl.graphs_test)
+    assert np.array_equal(again.score(wl.graphs_test)[few], oc.score(scorer, wl.graphs_test, few, threads=8))

@@ -214,14 +214,17 @@ def test_transform_and_read_outs_match_the_oracle():
 
 @pytest.mark.parametrize("case", [
     # 361-node graphs, one layer (tiles of positive rows only); tiny graphs that share words of a tile row;
-    # two and three layers with edge types and graphs without nodes
+    # two and three layers with edge types and graphs without nodes; one graph of 21 words per tile (two
+    # clauses per wave)
     dict(g=dict(n_graphs=23, max_nodes=361, min_nodes=300, hv_size=128), m=dict(depth=1), clauses=70, classes=10),
     dict(g=dict(n_graphs=90, max_nodes=3, hv_size=16, node_types=("a", "b")), m=dict(depth=1), clauses=33, classes=2),
     dict(g=dict(n_graphs=30, hv_size=24, node_types=("a", "b"), edge_types=("l", "r"), sizes=[5, 0, 33, 1, 40, 64] * 5),
          m=dict(depth=2, message_size=64, message_bits=2), clauses=40, classes=3),
     dict(g=dict(n_graphs=20, max_nodes=20, min_nodes=4, hv_size=20, edge_types=("x", "y", "z")),
          m=dict(depth=3, message_size=37, message_bits=3), clauses=50, classes=4),
-], ids=["361-nodes", "tiny-graphs", "two-layers", "three-layers"])
+    dict(g=dict(n_graphs=6, max_nodes=650, min_nodes=400, hv_size=64, edge_types=("l", "r")),
+         m=dict(depth=3, message_size=1024, message_bits=2), clauses=60, classes=3),
+], ids=["361-nodes", "tiny-graphs", "two-layers", "three-layers", "narrow-tiles"])
 def test_transform_on_tiles(case, tune):
     """gtm_transform from the truth rows of the tile kernels (k_tile_transform) == the dense path ==
     the oracle: per-clause outputs, per-node outputs and class sums, in one launch group and in groups

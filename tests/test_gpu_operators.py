@@ -868,7 +868,7 @@ HALF_TILE_SHAPES = [
 
 @pytest.mark.parametrize("shape", HALF_TILE_SHAPES, ids=lambda s: "half%d" % s["seed"])
 @pytest.mark.parametrize("density", [0.0, 0.02, 0.2])
-def test_half_tile_scoring_equals_oracle(shape, density):
+def test_half_tile_scoring_equals_oracle(shape, density, tune):
     """Depth-1 gtm_score on tiles whose LDS copy holds the positive literals' rows only (negated
     literals as complements; data declared complementary after the library's own check) == oracle
     == the bitmap path == the tiles of all rows."""
@@ -915,6 +915,15 @@ def test_half_tile_scoring_equals_oracle(shape, density):
     sample = sorted(set([0, 1, G // 2, G - 1]))
     assert np.array_equal(half[sample], o.score(model, graphs, sample))
     assert np.array_equal(dev.score(3, G - 5, G), plain[3:G - 2])  # a range that starts and ends inside tiles
+    if shape.get("half", True):
+        # fewer workgroups than tiles, the tiles' clauses shared out evenly among them (what a launch does whose
+        # tiles do not fill a whole number of rounds of the chip): a workgroup takes the end of one tile's clauses,
+        # whole tiles and the start of another's, and workgroups that share a tile add their class sums
+        for groups in (1, 2, 3, 5):
+            tune("GTM_TILE_LINE_GROUPS", str(groups))
+            assert np.array_equal(dev.score(0, G, G), plain), groups
+            assert np.array_equal(dev.score(3, G - 5, G), plain[3:G - 2]), groups
+        tune("GTM_TILE_LINE_GROUPS", None)
     # one-launch training on the same tiles follows the oracle
     Y = o.encode_labels(rng.integers(0, cfg.classes, size=G), cfg.classes, cfg.threshold)
     o.fit(model, graphs, Y)
@@ -974,3 +983,66 @@ def test_the_kernel_that_takes_over_beyond_4_gib_of_literal_words_follows_the_or
     _abi.call("gtm_profile_enable", 0)
     assert name.value.decode() == "k_tile_two_phase_wide<score>"
     assert np.array_equal(got, o.score(model, graphs))
+
+
+NARROW_TILE_SHAPES = [
+    # one graph of 22 truth words per tile (the message rows leave room for no more); three graphs of 10 words
+    # per tile; the same with a graph without nodes (then the data set is not declared complementary: layer 0
+    # takes the kernels that keep every row, the message layers scan every clause); several node types
+    dict(seed=61, g=dict(n_graphs=5, sizes=[700, 520, 1, 33, 689], hv_size=64, edge_types=("l", "r")), classes=3),
+    dict(seed=62, g=dict(n_graphs=11, max_nodes=300, min_nodes=1, hv_size=64, edge_types=("l", "r", "u")), classes=2),
+    dict(seed=63, g=dict(n_graphs=7, sizes=[300, 0, 1, 290, 0, 17, 64], hv_size=64, edge_types=("l",)), classes=4),
+    dict(seed=64, g=dict(n_graphs=6, max_nodes=650, min_nodes=400, hv_size=352, n_symbols=9, node_types=("a", "b", "c"),
+                         edge_types=("l", "r")), classes=3),
+]
+
+
+@pytest.mark.parametrize("shape", NARROW_TILE_SHAPES, ids=lambda s: "narrow%d" % s["seed"])
+@pytest.mark.parametrize("depth", [1, 2, 3])
+@pytest.mark.parametrize("path", ["two-clauses-per-wave", "all-rows-layer-0", "one-clause-per-wave"])
+def test_scoring_on_narrow_tiles(shape, depth, path, tune):
+    """Tiles whose rows are at most 32 words wide: two clauses per wave (score_paired.h), for the message
+    layers and - on a data set whose negated literals are the complements of its positive ones - for
+    layer 0 on the positive rows alone; against the oracle and against the kernels that take one clause
+    per wave.  The clauses are of three kinds: random ones (most die within the first rows), ones made of
+    a few hundred literals that hold everywhere (negations of hypervector and message bits that nothing
+    sets: their lists take several windows of 128 entries and are walked to the end), and empty ones."""
+    from tests.gpu_harness import Device
+
+    if path == "all-rows-layer-0":
+        tune("GTM_NO_HALF_ROWS", "1")
+    elif path == "one-clause-per-wave":
+        tune("GTM_NO_PAIRED_LAYERS", "1")
+    graphs = helpers.random_graphs(shape["seed"], max_degree=3, **shape["g"])
+    hv = graphs.hypervector_size
+    M = 1024 if depth > 1 else 64
+    cfg = helpers.oracle_config(graphs, classes=shape["classes"], clauses=150, depth=depth, message_size=M)
+    # (random clauses of about three literals: some are true at some nodes of some graphs)
+    model = helpers.random_model(shape["seed"], cfg, depth, include_density=1.5 / hv, message_density=0.004)
+    rng = np.random.default_rng(shape["seed"])
+    top = cfg.state_bits - 1
+    unused = np.setdiff1d(np.arange(hv), np.unique(graphs.hypervectors))
+    sent = np.unique((model.hypervectors.reshape(-1, 1) + np.arange(4).reshape(1, -1)) % M)  # bits a message can hold
+    unsent = np.setdiff1d(np.arange(M), sent)
+    for c in range(0, cfg.clauses, 3):  # every third clause holds wherever its node type is
+        model.ta_state[c, :, top] = 0
+        for k in rng.permutation(unused)[: int(rng.integers(0, len(unused) + 1))]:
+            lit = hv + int(k)
+            model.ta_state[c, lit // 32, top] |= np.uint32(1 << (lit % 32))
+        for bank in model.message_ta_state:
+            bank[c, :, top] = 0
+            for p in rng.permutation(unsent)[: int(rng.integers(0, 500))]:
+                lit = M + int(p)
+                bank[c, lit // 32, top] |= np.uint32(1 << (lit % 32))
+    model.ta_state[6, :, top] = 0  # an empty clause
+    dev = Device(model, graphs)
+    G = graphs.number_of_graphs
+    want = o.score(model, graphs)
+    assert want.any()
+    complementary = dev.declare_complementary()
+    assert complementary == (0 not in list(shape["g"].get("sizes", [1])))
+    assert dev.build_tiles(), "this shape should have a tile layout"
+    assert np.array_equal(dev.score(0, G, G), want)
+    assert np.array_equal(dev.score(0, G, 2), want)       # several launch groups
+    if G > 5:
+        assert np.array_equal(dev.score(2, G - 3, 4), want[2:G - 1])  # a range that starts and ends inside tiles
