@@ -29,9 +29,11 @@
 // The workgroup's barriers order LDS traffic only, so none of them waits for the
 // adds or for the loads of the next graph.
 //
-// The wait is bounded: after `spin_limit` polls a workgroup raises the abort
-// flag and every workgroup leaves the loop at its next check, so the grid always
-// drains.  The host reports the flag as an error.
+// The wait is bounded (a few seconds of the device's wall clock; a number of polls
+// in tests): a workgroup whose wait runs out raises the abort flag and every
+// workgroup leaves the loop at its next check, so the grid always drains.  The
+// host then puts the model back as it was and trains the examples by launches per
+// example instead.
 #pragma once
 
 constexpr int FITP_BLOCK = 1024;  // 16 waves: one clause per wave in flight, four waves per SIMD hide each other's latencies
@@ -150,8 +152,8 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
     const int own_max = p.clauses_per_group;
 
     // LDS carve-up
-    uint32_t *rows_buf[3] = {lds, lds + p.rows_words, lds + 2 * p.rows_words};  // example i, i + 1, i + 2 in turn
-    uint32_t *ta = lds + 3 * p.rows_words;                     // [own][LA][B]
+    uint32_t *rows_buf[2] = {lds, lds + p.rows_words};
+    uint32_t *ta = lds + 2 * p.rows_words;                     // [own][LA][B]
     int32_t *wts = (int32_t *)(ta + (size_t)own_max * LA * B);  // [own][K]
     int32_t *upd = wts + (size_t)own_max * K;                  // [own][K]
     int32_t *node_of = upd + (size_t)own_max * K;              // [own]
@@ -161,16 +163,16 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
     uint32_t *gate = (uint32_t *)(votes + K);                  // [own][K][2] random words of the feedback gates
     uint32_t *fbits = gate + 2 * (size_t)own_max * K;          // [own][LA][K] Type I feedback bits
     int32_t *pair_list = (int32_t *)(fbits + (size_t)own_max * LA * K);  // [own * K] (clause, class) pairs with Type I feedback
-    uint32_t *x_buf[3] = {(uint32_t *)(pair_list + (size_t)own_max * K), (uint32_t *)(pair_list + (size_t)own_max * K) + p.x_words,
-                          (uint32_t *)(pair_list + (size_t)own_max * K) + 2 * p.x_words};  // [nodes][LA] of the graph
-    uint32_t *order_lds = x_buf[2] + p.x_words;                 // [literals]
+    uint32_t *x_buf[2] = {(uint32_t *)(pair_list + (size_t)own_max * K),
+                          (uint32_t *)(pair_list + (size_t)own_max * K) + p.x_words};  // [nodes][LA] of the graph
+    uint32_t *order_lds = x_buf[1] + p.x_words;                 // [literals]
     // thread k < K: its class-sum word as it stood when each of the three
     // slots was last complete (all zero before the first use): [slot][low, high][K]
     uint32_t *seen = order_lds + p.literals;
-    uint32_t *y_buf[3] = {seen + 6 * K, seen + 7 * K, seen + 8 * K};  // [K] labels of example i, i + 1, i + 2 in turn
+    uint32_t *y_buf[2] = {seen + 6 * K, seen + 7 * K};        // [K] labels of this and the next example
     __shared__ int go_on, n_pairs;
     __shared__ uint32_t after_lds[2];
-    __shared__ uint32_t types_lds[3][FITP_DIRECT_NODES];  // node types of the graphs in the three buffers (direct evaluation)
+    __shared__ uint32_t types_lds[2][FITP_DIRECT_NODES];  // node types of this and the next graph (direct evaluation)
 
     // own state -> LDS
     for (int k = tid; k < K; k += FITP_BLOCK) votes[k] = 0;
@@ -180,24 +182,19 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         wts[i] = p.weights[(int64_t)k * p.C + c0 + cl];
     }
     const int last = p.first_example + p.n_examples - 1;
-    // node counts and first nodes of examples i, i + 1 and i + 2
-    int n_now = 0, n_next = 0, n_after = 0;
-    uint32_t base_now = 0, base_next = 0, base_after = 0;
+    int n_now = 0, n_next = 0;          // node counts of example i and i + 1
+    uint32_t base_now = 0, base_next = 0;  // node_index of example i and i + 1
     if (p.n_examples > 0) {
-        const int e1 = min(p.first_example + 1, last), e2 = min(p.first_example + 2, last);
-        n_now = (int)p.n_nodes[p.first_example], base_now = p.node_index[p.first_example];
-        n_next = (int)p.n_nodes[e1], base_next = p.node_index[e1];
-        n_after = (int)p.n_nodes[e2], base_after = p.node_index[e2];
-        // the first two examples are staged here; from then on example i + 2 arrives while example i is worked on
-        for (int b = 0; b < 2 && b < p.n_examples; ++b) {
-            const int e = p.first_example + b, n = b ? n_next : n_now;
-            const uint32_t base = b ? base_next : base_now;
-            const FitGraph fg0 = fit_graph_slot(p.tg, e, n);
-            if (!p.direct) fitp_stage_rows(p, fg0, rows_buf[b], tid);
-            for (int at = tid; at < n * LA; at += FITP_BLOCK) x_buf[b][at] = p.X[(int64_t)base * LA + at];
-            if (p.direct && tid < n) types_lds[b][tid] = p.node_type[base + tid];
-            for (int k = tid; k < K; k += FITP_BLOCK) y_buf[b][k] = (uint32_t)p.encoded_Y[(int64_t)e * K + k];
-        }
+        n_now = (int)p.n_nodes[p.first_example];
+        base_now = p.node_index[p.first_example];
+        const int e1 = min(p.first_example + 1, last);
+        n_next = (int)p.n_nodes[e1];
+        base_next = p.node_index[e1];
+        FitGraph fg0 = fit_graph_slot(p.tg, p.first_example, n_now);
+        if (!p.direct) fitp_stage_rows(p, fg0, rows_buf[0], tid);
+        for (int at = tid; at < n_now * LA; at += FITP_BLOCK) x_buf[0][at] = p.X[(int64_t)base_now * LA + at];
+        if (p.direct && tid < n_now) types_lds[0][tid] = p.node_type[base_now + tid];
+        for (int k = tid; k < K; k += FITP_BLOCK) y_buf[0][k] = (uint32_t)p.encoded_Y[(int64_t)p.first_example * K + k];
     }
     for (int l = tid; l < p.literals; l += FITP_BLOCK) order_lds[l] = p.order[l];
     for (int j = tid; j < 6 * K; j += FITP_BLOCK) seen[j] = 0u;
@@ -206,232 +203,207 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
     const int ones_row = p.literals + p.n_types;
     // one small clause per wave: the feedback of a step runs inside the clause's wave
     const bool wave_local = own_max <= WAVES && K * LA <= 256;
-    // K1 + K7 for own clause `cl` on one staged graph (`rows`: its literal-major rows, `x_now`: its nodes' literal
-    // words, `types`: its node types when graphs are evaluated directly) with the automata as they stand in LDS
-    // now: the node picked for the feedback (-1: none), the number of included literals, and whether the clause
-    // votes.  Wave-uniform.
-    struct Evaluated {
-        int node, included;
-        bool fired;
-    };
-    auto evaluate = [&](int cl, const FitGraph &fg, const uint32_t *rows, const uint32_t *x_now, int n_now, uint32_t step,
-                        const uint32_t *types) {
-        const bool active = lane < fg.words;
-        const uint32_t *col = rows + (active ? lane : 0);
-        const int stride = fg.words;
-        const int c = c0 + cl;
-        const uint32_t *inc = ta + (size_t)cl * LA * B + (B - 1);
-        uint32_t acc = active && !p.direct ? col[(p.literals + c % p.n_types) * stride] : 0u;
-        int included = 0;
-        uint32_t first_words = 0;
-        for (int w0 = 0; w0 < LA; w0 += 64) {
-            uint32_t mine = w0 + lane < LA ? inc[(w0 + lane) * B] : 0u;
-            if (w0 + lane == LA - 1) mine &= p.filter;
-            if (w0 == 0) first_words = mine;
-            included += wave_sum_small(__popc(mine));
-        }
-        // A clause with many literals ANDs only the rows of its FITP_FILTER_ROWS rarest ones and then
-        // tests the few nodes that are left against its whole include mask on the nodes' own words.
-        const bool filter_only = included > FITP_WALK_ALL && n_now > 0 && !p.direct;
-        bool all_rows = false;  // every included literal's row has been applied: acc is the clause's truth
-        if (filter_only) {
-            int budget = FITP_FILTER_ROWS;
-            bool stop = false;
-            // The included literals in rarest-first order, 256 ranks at a time: the four LDS reads
-            // of the ranks and the four of the include words are each issued together (a clause
-            // whose rare literals are few would otherwise pay two LDS round trips per 64 ranks).
-            for (int g0 = 0; g0 < p.literals && !stop; g0 += 256) {
-                uint32_t lit4[4];
-                unsigned long long m4[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int r = g0 + 64 * u + lane;
-                    lit4[u] = r < p.literals ? order_lds[r] : 0u;
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int r = g0 + 64 * u + lane;
-                    uint32_t word = inc[(lit4[u] >> 5) * B];
-                    if ((int)(lit4[u] >> 5) == LA - 1) word &= p.filter;
-                    m4[u] = __ballot(r < p.literals && ((word >> (lit4[u] & 31u)) & 1u));
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    unsigned long long picked = m4[u];  // lanes whose literal is included and not applied yet
-                    const uint32_t lit = lit4[u];
-                    while (picked != 0ull && !stop) {
-                        if (budget <= 0) {
-                            // a few surviving nodes are cheapest tested one by one; more than that, and 8 more
-                            // rows (one LDS round trip) remove most of them at the price of testing one
-                            // (counted as lanes with a survivor, twice those with several: an estimate is enough)
-                            if (n_now <= FITP_FEW_NODES) {
-                                stop = true;
-                                break;
-                            }
-                            const int mine = active ? __popc((acc >> fg.shift) & fg.mask) : 0;
-                            const int left = __popcll(__ballot(mine > 0)) + __popcll(__ballot(mine > 1));
-                            if (left <= FITP_FEW_NODES) {
-                                stop = true;
-                                break;
-                            }
-                            budget = 8;
-                        }
-                        int row[8];
-#pragma unroll
-                        for (int v8 = 0; v8 < 8; ++v8) {
-                            row[v8] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
-                            picked &= picked - 1;
-                        }
-                        uint32_t r8[8];
-#pragma unroll
-                        for (int v8 = 0; v8 < 8; ++v8) r8[v8] = col[row[v8] * stride];
-#pragma unroll
-                        for (int v8 = 0; v8 < 8; ++v8) acc &= r8[v8];
-                        budget -= 8;
-                    }
-                }
-            }
-            all_rows = !stop;  // every included literal's row has been applied
-        } else if (!p.direct) {
-            for (int w0 = 0; w0 < LA; w0 += 64) {
-                uint32_t mine = w0 == 0 ? first_words : (w0 + lane < LA ? inc[(w0 + lane) * B] : 0u);
-                if (w0 != 0 && w0 + lane == LA - 1) mine &= p.filter;
-                unsigned long long nonzero = __ballot(mine != 0);
-                while (nonzero) {
-                    const int wl = __ffsll((long long)nonzero) - 1;
-                    nonzero &= nonzero - 1;
-                    uint32_t m = __builtin_amdgcn_readlane(mine, wl);
-                    const int base = (w0 + wl) << 5;
-                    while (m) {
-                        int row[8];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) {
-                            row[u] = m ? base + __builtin_ctz(m) : ones_row;
-                            m &= m - 1;
-                        }
-                        uint32_t r[8];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) r[u] = col[row[u] * stride];
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) acc &= r[u];
-                    }
-                }
-            }
-        }
-        uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
-        if (p.direct) {
-            // one or two nodes: the clause against each node's own literal words (kernels.py:443-466 as
-            // it stands), lane w on word w; no literal-major rows are read or staged
-            uint32_t bits = 0u;
-            for (int node = 0; node < n_now; ++node) {
-                bool violated = false;
-                for (int w0 = 0; w0 < LA; w0 += 64) {
-                    uint32_t mine = w0 == 0 ? first_words : (w0 + lane < LA ? inc[(w0 + lane) * B] : 0u);
-                    if (w0 != 0 && w0 + lane == LA - 1) mine &= p.filter;
-                    const uint32_t xs = w0 + lane < LA ? x_now[node * LA + w0 + lane] : 0xFFFFFFFFu;
-                    violated |= __ballot((mine & ~xs) != 0) != 0;
-                }
-                if (!violated && (int)types[node] == c % p.n_types) bits |= 1u << node;
-            }
-            v = lane == 0 ? bits : 0u;
-        }
-        if (filter_only && !all_rows) {
-            // lane L holds nodes 32 L .. 32 L + 31: the surviving ones are walked on the scalar unit; lane w
-            // compares include word w with the node's literal word w (LDS copy of the graph's X rows)
-            unsigned long long live = __ballot(v != 0);
-            while (live) {
-                const int L = __ffsll((long long)live) - 1;
-                live &= live - 1;
-                uint32_t word = __builtin_amdgcn_readlane(v, L);
-                uint32_t cleared = 0;
-                while (word) {
-                    const int b = __builtin_ctz(word);
-                    word &= word - 1;
-                    const uint32_t *x = x_now + (L * 32 + b) * LA;
-                    bool violated = false;
-                    for (int w0 = 0; w0 < LA; w0 += 64) {
-                        uint32_t mine = w0 == 0 ? first_words : (w0 + lane < LA ? inc[(w0 + lane) * B] : 0u);
-                        if (w0 != 0 && w0 + lane == LA - 1) mine &= p.filter;
-                        const uint32_t xs = w0 + lane < LA ? x[w0 + lane] : 0xFFFFFFFFu;
-                        violated |= __ballot((mine & ~xs) != 0) != 0;
-                    }
-                    if (violated) cleared |= 1u << b;
-                }
-                if (lane == L) v &= ~cleared;
-            }
-        }
-        const int pc = __popc(v);
-        int true_nodes, before;
-        wave_count_scan(pc, lane, &true_nodes, &before);
-        bool fired = true_nodes > 0;
-        int node = -1;
-        if (n_now == 0) {
-            fired = true;  // the reference's arithmetic for a graph without nodes (kernels.py:289-295)
-        } else if (fired) {
-            philox_out r = philox4x32_10((uint32_t)c, 0u, step, GTM_TAG_CLAUSE_NODE, p.k0, p.k1);
-            const int pick = (int)(((uint64_t)r.v[0] * (uint64_t)true_nodes) >> 32);
-            const bool mine_is = pick >= before && pick < before + pc;
-            int candidate = 0;
-            if (mine_is) {
-                uint32_t t = v;
-                for (int j = before; j < pick; ++j) t &= t - 1;
-                candidate = lane * 32 + __ffs(t) - 1;
-            }
-            const unsigned long long owner = __ballot(mine_is);
-            node = __builtin_amdgcn_readlane(candidate, __ffsll((long long)owner) - 1);
-        }
-        return Evaluated{node, included, fired};
-    };
-    // what the feedback and the exchange of the class sums need of an evaluation
-    auto publish = [&](int cl, const Evaluated &ev) {
-        if (lane == 0) {
-            node_of[cl] = ev.node;
-            incl_of[cl] = ev.included;
-        }
-        if (ev.fired)
-            for (int k = lane; k < K; k += 64) atomicAdd(&votes[k], wts[cl * K + k]);  // LDS
-    };
-
     int div_words = 0, div_dr = 0, div_r0 = 0;
-    // Evaluating ahead (one small clause per wave, at most 64 classes): while the class sums of example i are on their
-    // way - a device-wide exchange of a few microseconds - a wave evaluates its clause on example i + 1 with the
-    // automata as they are.  The feedback of example i comes after that; if it leaves the clause's include mask as
-    // it was (late in training it moves states without crossing the threshold, or does nothing at all), the
-    // evaluation stands, and otherwise it is done again, so the result is what it would be without looking ahead.
-    // The threads that poll for the class sums sit in the last wave, which has no clause in most configurations.
-    const bool look_ahead = wave_local && K <= 64;
-    const int poll0 = look_ahead ? (WAVES - 1) * 64 : 0;  // the first polling thread
-    bool ahead_valid = false;
-    Evaluated ahead{-1, 0, false};
+    // The threads that add the group's votes to the device-wide class sums and then poll for them are the first K
+    // of the LAST wave when K <= 64; that wave requests none of the next graph's words and draws no random
+    // numbers, so its polling starts at once and runs beside the other waves' work instead of after its own share.
+    const bool poll_apart = K <= 64;
+    const int poll0 = poll_apart ? (WAVES - 1) * 64 : 0;         // the first polling thread
+    const int loaders = poll_apart ? poll0 : FITP_BLOCK;        // threads 0 .. loaders - 1 request the next graph's words
     for (int i = 0; i < p.n_examples; ++i) {
         const int ex = p.first_example + i;
         const uint32_t step = p.first_step + (uint32_t)i;
         const FitGraph fg = fit_graph_slot(p.tg, ex, n_now);
-        const uint32_t *rows = rows_buf[i % 3];
+        const uint32_t *rows = rows_buf[i & 1];
         unsigned long long *slot_now = p.class_sum + (size_t)(i % 3) * K * FITP_SUM_PARTS * FITP_SUM_STRIDE;
 
-        // ---- 0. the slot of the graph after the next (example i + 2: its data are requested in this step, two
-        // examples ahead of their use, so that example i + 1 is complete in LDS while example i is worked on);
-        // the sizes of the graph after that are requested
-        const bool has_next = i + 1 < p.n_examples, has_after = i + 2 < p.n_examples;
-        const FitGraph fn = fit_graph_slot(p.tg, has_after ? ex + 2 : ex, has_after ? n_after : n_now);
-        const int next_total = has_after && !p.direct ? (p.literals + p.n_types + 1) * fn.words : 0;
-        const uint32_t *x_now = x_buf[i % 3];
-        // node count and first node of example i + 3, fetched by two threads with vector
+        // ---- 0. the next graph's slot; the sizes of the graph after it are requested
+        const bool has_next = i + 1 < p.n_examples;
+        const FitGraph fn = fit_graph_slot(p.tg, has_next ? ex + 1 : ex, has_next ? n_next : n_now);
+        const int next_total = has_next && !p.direct ? (p.literals + p.n_types + 1) * fn.words : 0;
+        const uint32_t *x_now = x_buf[i & 1];
+        // node count and first node of the graph after the next, fetched by two threads with vector
         // loads (scalar loads share their counter with LDS: the evaluation's first LDS read would wait
         // for them) and handed over through LDS at the end of the step
-        const int e3 = min(ex + 3, last);
+        const int e2 = min(ex + 2, last);
         uint32_t after = 0u;
-        if (tid < 2) after = (tid == 0 ? p.n_nodes : p.node_index)[e3];
+        if (tid < 2) after = (tid == 0 ? p.n_nodes : p.node_index)[e2];
         uint32_t type_ahead = 0u;
-        if (p.direct && has_after && tid < n_after) type_ahead = p.node_type[base_after + tid];
+        if (p.direct && has_next && tid < n_next) type_ahead = p.node_type[base_next + tid];
 
-        // ---- 1. evaluate own clauses (K1 + K7), votes (K6) - those that have not been evaluated ahead (see 2.)
+        // ---- 1. evaluate own clauses (K1 + K7), votes (K6)
+        const bool active = lane < fg.words;
+        const uint32_t *col = rows + (active ? lane : 0);
+        const int stride = fg.words;
         for (int cl = wave; cl < n_own; cl += WAVES) {
-            if (ahead_valid) break;  // (one clause per wave when evaluating ahead)
-            publish(cl, evaluate(cl, fg, rows, x_now, n_now, step, types_lds[i % 3]));
+            const int c = c0 + cl;
+            const uint32_t *inc = ta + (size_t)cl * LA * B + (B - 1);
+            uint32_t acc = active && !p.direct ? col[(p.literals + c % p.n_types) * stride] : 0u;
+            int included = 0;
+            uint32_t first_words = 0;
+            for (int w0 = 0; w0 < LA; w0 += 64) {
+                uint32_t mine = w0 + lane < LA ? inc[(w0 + lane) * B] : 0u;
+                if (w0 + lane == LA - 1) mine &= p.filter;
+                if (w0 == 0) first_words = mine;
+                included += wave_sum_small(__popc(mine));
+            }
+            // A clause with many literals ANDs only the rows of its FITP_FILTER_ROWS rarest ones and then
+            // tests the few nodes that are left against its whole include mask on the nodes' own words.
+            const bool filter_only = included > FITP_WALK_ALL && n_now > 0 && !p.direct;
+            bool all_rows = false;  // every included literal's row has been applied: acc is the clause's truth
+            if (filter_only) {
+                int budget = FITP_FILTER_ROWS;
+                bool stop = false;
+                // The included literals in rarest-first order, 256 ranks at a time: the four LDS reads
+                // of the ranks and the four of the include words are each issued together (a clause
+                // whose rare literals are few would otherwise pay two LDS round trips per 64 ranks).
+                for (int g0 = 0; g0 < p.literals && !stop; g0 += 256) {
+                    uint32_t lit4[4];
+                    unsigned long long m4[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int r = g0 + 64 * u + lane;
+                        lit4[u] = r < p.literals ? order_lds[r] : 0u;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int r = g0 + 64 * u + lane;
+                        uint32_t word = inc[(lit4[u] >> 5) * B];
+                        if ((int)(lit4[u] >> 5) == LA - 1) word &= p.filter;
+                        m4[u] = __ballot(r < p.literals && ((word >> (lit4[u] & 31u)) & 1u));
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        unsigned long long picked = m4[u];  // lanes whose literal is included and not applied yet
+                        const uint32_t lit = lit4[u];
+                        while (picked != 0ull && !stop) {
+                            if (budget <= 0) {
+                                // a few surviving nodes are cheapest tested one by one; more than that, and 8 more
+                                // rows (one LDS round trip) remove most of them at the price of testing one
+                                // (counted as lanes with a survivor, twice those with several: an estimate is enough)
+                                if (n_now <= FITP_FEW_NODES) {
+                                    stop = true;
+                                    break;
+                                }
+                                const int mine = active ? __popc((acc >> fg.shift) & fg.mask) : 0;
+                                const int left = __popcll(__ballot(mine > 0)) + __popcll(__ballot(mine > 1));
+                                if (left <= FITP_FEW_NODES) {
+                                    stop = true;
+                                    break;
+                                }
+                                budget = 8;
+                            }
+                            int row[8];
+#pragma unroll
+                            for (int v8 = 0; v8 < 8; ++v8) {
+                                row[v8] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
+                                picked &= picked - 1;
+                            }
+                            uint32_t r8[8];
+#pragma unroll
+                            for (int v8 = 0; v8 < 8; ++v8) r8[v8] = col[row[v8] * stride];
+#pragma unroll
+                            for (int v8 = 0; v8 < 8; ++v8) acc &= r8[v8];
+                            budget -= 8;
+                        }
+                    }
+                }
+                all_rows = !stop;  // every included literal's row has been applied
+            } else if (!p.direct) {
+                for (int w0 = 0; w0 < LA; w0 += 64) {
+                    uint32_t mine = w0 == 0 ? first_words : (w0 + lane < LA ? inc[(w0 + lane) * B] : 0u);
+                    if (w0 != 0 && w0 + lane == LA - 1) mine &= p.filter;
+                    unsigned long long nonzero = __ballot(mine != 0);
+                    while (nonzero) {
+                        const int wl = __ffsll((long long)nonzero) - 1;
+                        nonzero &= nonzero - 1;
+                        uint32_t m = __builtin_amdgcn_readlane(mine, wl);
+                        const int base = (w0 + wl) << 5;
+                        while (m) {
+                            int row[8];
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) {
+                                row[u] = m ? base + __builtin_ctz(m) : ones_row;
+                                m &= m - 1;
+                            }
+                            uint32_t r[8];
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) r[u] = col[row[u] * stride];
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) acc &= r[u];
+                        }
+                    }
+                }
+            }
+            uint32_t v = active ? (acc >> fg.shift) & fg.mask : 0u;
+            if (p.direct) {
+                // one or two nodes: the clause against each node's own literal words (kernels.py:443-466 as
+                // it stands), lane w on word w; no literal-major rows are read or staged
+                uint32_t bits = 0u;
+                for (int node = 0; node < n_now; ++node) {
+                    bool violated = false;
+                    for (int w0 = 0; w0 < LA; w0 += 64) {
+                        uint32_t mine = w0 == 0 ? first_words : (w0 + lane < LA ? inc[(w0 + lane) * B] : 0u);
+                        if (w0 != 0 && w0 + lane == LA - 1) mine &= p.filter;
+                        const uint32_t xs = w0 + lane < LA ? x_now[node * LA + w0 + lane] : 0xFFFFFFFFu;
+                        violated |= __ballot((mine & ~xs) != 0) != 0;
+                    }
+                    if (!violated && (int)types_lds[i & 1][node] == c % p.n_types) bits |= 1u << node;
+                }
+                v = lane == 0 ? bits : 0u;
+            }
+            if (filter_only && !all_rows) {
+                // lane L holds nodes 32 L .. 32 L + 31: the surviving ones are walked on the scalar unit; lane w
+                // compares include word w with the node's literal word w (LDS copy of the graph's X rows)
+                unsigned long long live = __ballot(v != 0);
+                while (live) {
+                    const int L = __ffsll((long long)live) - 1;
+                    live &= live - 1;
+                    uint32_t word = __builtin_amdgcn_readlane(v, L);
+                    uint32_t cleared = 0;
+                    while (word) {
+                        const int b = __builtin_ctz(word);
+                        word &= word - 1;
+                        const uint32_t *x = x_now + (L * 32 + b) * LA;
+                        bool violated = false;
+                        for (int w0 = 0; w0 < LA; w0 += 64) {
+                            uint32_t mine = w0 == 0 ? first_words : (w0 + lane < LA ? inc[(w0 + lane) * B] : 0u);
+                            if (w0 != 0 && w0 + lane == LA - 1) mine &= p.filter;
+                            const uint32_t xs = w0 + lane < LA ? x[w0 + lane] : 0xFFFFFFFFu;
+                            violated |= __ballot((mine & ~xs) != 0) != 0;
+                        }
+                        if (violated) cleared |= 1u << b;
+                    }
+                    if (lane == L) v &= ~cleared;
+                }
+            }
+            const int pc = __popc(v);
+            int true_nodes, before;
+            wave_count_scan(pc, lane, &true_nodes, &before);
+            bool fired = true_nodes > 0;
+            int node = -1;
+            if (n_now == 0) {
+                fired = true;  // the reference's arithmetic for a graph without nodes (kernels.py:289-295)
+            } else if (fired) {
+                philox_out r = philox4x32_10((uint32_t)c, 0u, step, GTM_TAG_CLAUSE_NODE, p.k0, p.k1);
+                const int pick = (int)(((uint64_t)r.v[0] * (uint64_t)true_nodes) >> 32);
+                const bool mine_is = pick >= before && pick < before + pc;
+                int candidate = 0;
+                if (mine_is) {
+                    uint32_t t = v;
+                    for (int j = before; j < pick; ++j) t &= t - 1;
+                    candidate = lane * 32 + __ffs(t) - 1;
+                }
+                const unsigned long long owner = __ballot(mine_is);
+                node = __builtin_amdgcn_readlane(candidate, __ffsll((long long)owner) - 1);
+            }
+            if (lane == 0) {
+                node_of[cl] = node;
+                incl_of[cl] = included;
+            }
+            if (fired)
+                for (int k = lane; k < K; k += 64) atomicAdd(&votes[k], wts[cl * K + k]);  // LDS
         }
-        ahead_valid = false;
 
         // ---- 2. class sums across the device (see the header comment)
         if (tid == 0) go_on = 1;
@@ -450,13 +422,13 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
             const uint32_t *tile = p.tiles + (int64_t)fn.tile * p.tg.rows * p.tg.tw + fn.word0;
             if (fn.words != div_words) {  // the divisions are redone only when the slot width changes
                 div_words = fn.words;
-                div_dr = FITP_BLOCK / fn.words;
+                div_dr = loaders / fn.words;
                 div_r0 = tid / fn.words;
             }
-            const int dr = div_dr, dw = FITP_BLOCK - dr * fn.words;
+            const int dr = div_dr, dw = loaders - dr * fn.words;
             int r = div_r0, w = tid - r * fn.words;
-            uint32_t *dst = rows_buf[(i + 2) % 3] + wave * 64;
-            for (int at0 = 0; at0 < next_total; at0 += FITP_BLOCK) {
+            uint32_t *dst = rows_buf[(i + 1) & 1] + wave * 64;
+            for (int at0 = 0; at0 < next_total && tid < loaders; at0 += loaders) {
                 if (at0 + tid < next_total) fitp_load_to_lds(tile + (int64_t)r * p.tg.tw + w, dst + at0);
                 r += dr;
                 w += dw;
@@ -466,29 +438,29 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 }
             }
         }
-        const int next_x_total = has_after ? n_after * LA : 0;
+        const int next_x_total = has_next ? n_next * LA : 0;
         {
-            const uint32_t *src = p.X + (int64_t)base_after * LA + tid;
-            uint32_t *dst = x_buf[(i + 2) % 3] + wave * 64;
-            for (int at0 = 0; at0 < next_x_total; at0 += FITP_BLOCK)
+            const uint32_t *src = p.X + (int64_t)base_next * LA + tid;
+            uint32_t *dst = x_buf[(i + 1) & 1] + wave * 64;
+            for (int at0 = 0; at0 < next_x_total && tid < loaders; at0 += loaders)
                 if (at0 + tid < next_x_total) fitp_load_to_lds(src + at0, dst + at0);
         }
-        if (has_after) {
-            const uint32_t *src = (const uint32_t *)p.encoded_Y + (int64_t)(ex + 2) * K + tid;
-            uint32_t *dst = y_buf[(i + 2) % 3] + wave * 64;
-            for (int at0 = 0; at0 < K; at0 += FITP_BLOCK)
+        if (has_next) {
+            const uint32_t *src = (const uint32_t *)p.encoded_Y + (int64_t)(ex + 1) * K + tid;
+            uint32_t *dst = y_buf[(i + 1) & 1] + wave * 64;
+            for (int at0 = 0; at0 < K && tid < loaders; at0 += loaders)
                 if (at0 + tid < K) fitp_load_to_lds(src + at0, dst + at0);
         }
-        if (p.direct && has_after && tid < n_after) types_lds[(i + 2) % 3][tid] = type_ahead;
+        if (p.direct && has_next && tid < n_next) types_lds[(i + 1) & 1][tid] = type_ahead;
         // The random words of the feedback gates are drawn by the waves that do not poll, while the
         // class sums are on their way. (Drawing the Type I feedback bits of every (clause, class,
         // word) here as well costs more generator work than the exchange hides: they are drawn
         // afterwards, for the pairs that turn out to need them.)
         const int pollers = (K + 63) & ~63, helpers = FITP_BLOCK - pollers;
         if (helpers >= FITP_BLOCK / 2) {
-            // (the polling threads are the first `pollers`, or - when evaluating ahead - the last 64)
-            if (look_ahead ? tid < poll0 : tid >= pollers)
-                for (int j = look_ahead ? tid : tid - pollers; j < n_own * K; j += helpers) {
+            // (the polling threads are the first `pollers`, or - set apart - within the last 64)
+            if (poll_apart ? tid < poll0 : tid >= pollers)
+                for (int j = poll_apart ? tid : tid - pollers; j < n_own * K; j += helpers) {
                     const int cl = j / K, k = j - cl * K;
                     philox_out r = philox4x32_10((uint32_t)(c0 + cl), (uint32_t)k, step, GTM_TAG_CLAUSE_UPDATES, p.k0, p.k1);
                     gate[2 * j] = r.v[0];
@@ -502,13 +474,6 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                 gate[2 * j + 1] = r.v[1];
             }
             lds_barrier();
-        }
-        // Evaluating ahead: this wave's clause on example i + 1 (complete in LDS since the end of the step before),
-        // with the automata as they are before the feedback of example i
-        if (look_ahead && has_next && wave < n_own && wave != WAVES - 1) {
-            const FitGraph f1 = fit_graph_slot(p.tg, ex + 1, n_next);
-            ahead = evaluate(wave, f1, rows_buf[(i + 1) % 3], x_buf[(i + 1) % 3], n_next, step + 1u, types_lds[(i + 1) % 3]);
-            ahead_valid = true;
         }
         if (tid >= poll0 && tid - poll0 < K) {
             const int k = tid - poll0;
@@ -554,7 +519,7 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         if (!go_on) break;  // uniform over the group; every group leaves at its next check
 
         // ---- 3. feedback (K8) and automaton updates (K9) on the LDS copies
-        const int32_t *y = (const int32_t *)y_buf[i % 3];
+        const int32_t *y = (const int32_t *)y_buf[i & 1];
         const uint32_t *X_rows = x_now;  // the graph's literal words, node-major, in LDS
         auto decide = [&](int j, int k) {  // K8 for (clause, class) pair j = cl * K + k
             const int cl = j / K;
@@ -603,28 +568,16 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
                     }
                 }
                 fitp_wave_lds_sync();
-                bool include_mask_moved = false;
                 if (any) {
                     const int node = node_of[cl];
                     const bool fired = node != -1;
                     const bool within = incl_of[cl] <= p.max_included;
                     for (int w = lane; w < LA; w += 64) {
                         const uint32_t x = fired ? X_rows[node * LA + w] : 0u;
-                        uint32_t *planes = ta + ((size_t)cl * LA + w) * B;
-                        const uint32_t include_before = planes[B - 1];
-                        feedback_word<MAXB>(planes, B, K, upd + cl * K, 1, fired, within, p.boost, x, p.k0,
+                        feedback_word<MAXB>(ta + ((size_t)cl * LA + w) * B, B, K, upd + cl * K, 1, fired, within, p.boost, x, p.k0,
                                             p.k1, (uint32_t)(c0 + cl), (uint32_t)w, step, 0u, p.thr16,
                                             fbits + ((size_t)cl * LA + w) * K);
-                        include_mask_moved |= planes[B - 1] != include_before;
                     }
-                    include_mask_moved = __ballot(include_mask_moved) != 0ull;
-                }
-                // what was evaluated ahead stands if the clause includes the same literals as before
-                if (ahead_valid) {
-                    if (include_mask_moved)
-                        ahead_valid = false;
-                    else
-                        publish(cl, ahead);
                 }
             }
         } else {
@@ -669,9 +622,10 @@ __global__ __launch_bounds__(FITP_BLOCK) void k_fit_persistent(FitPersistParams 
         // With the feedback inside the clause's wave, the wave goes on to evaluate its clause on the
         // next graph (everything that evaluation reads was complete at the barrier above).
         if (!wave_local) lds_barrier();
-        n_now = n_next, base_now = base_next;
-        n_next = n_after, base_next = base_after;
-        n_after = (int)after_lds[0], base_after = after_lds[1];
+        n_now = n_next;
+        base_now = base_next;
+        n_next = (int)after_lds[0];
+        base_next = after_lds[1];
     }
     __builtin_amdgcn_s_waitcnt(FITP_WAIT_VMEM);  // no load into LDS is left in flight when the group ends
     lds_barrier();

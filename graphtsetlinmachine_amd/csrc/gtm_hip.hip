@@ -16,7 +16,7 @@
 #include "../../include/gtm_abi.h"
 #include "philox.h"
 #include "score_tiles.h"
-#include "score_paired.h"
+#include "score_narrow.h"
 
 namespace {
 
@@ -70,7 +70,7 @@ int check_launch(const char *what) {
     X(NO_HALF_TILES) \
     X(NO_LISTS_IN_LDS) \
     X(NO_NARROW_TWO_PHASE) \
-    X(NO_PAIRED_LAYERS) \
+    X(NO_NARROW_LAYERS) \
     X(NO_PERSISTENT_FIT) \
     X(NO_SMALL_FIT) \
     X(NO_TILE_LINE) \
@@ -658,7 +658,7 @@ struct ScoreWs {
     uint32_t *sent, *got;     // [tiles per launch][tw * 32 node slots][ceil(M / 32)]  (tile path, depth > 1)
     uint32_t *message_rows;   // [tiles per launch][M + 2][tw]  (tile path, depth > 1)
     uint32_t *bit_start, *bit_cursor, *bit_clauses;  // [M + 1], [M], [C * MB]: the clauses of every message bit (tile path, depth > 1)
-    uint32_t *alive[2];       // [tiles per launch][PAIRED_STREAMS][alive_stride] clauses still true somewhere in a tile, layer to layer
+    uint32_t *alive[2];       // [tiles per launch][NARROW_STREAMS][alive_stride] clauses still true somewhere in a tile, layer to layer
     int alive_stride;
     TileSegment *segments;    // [tiles + 2 * TILE_SEGMENTS_MAX_SHARES] which clauses of which tile a workgroup takes (half tiles)
     size_t vector_words;      // words of sent (and of got)
@@ -715,8 +715,8 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base,
         w.bit_start = (uint32_t *)take(((size_t)d.M + 1) * 4);
         w.bit_cursor = (uint32_t *)take((size_t)d.M * 4);
         w.bit_clauses = (uint32_t *)take((size_t)d.C * d.MB * 4);
-        w.alive_stride = paired_alive_stride(d.C);
-        for (uint32_t *&list : w.alive) list = (uint32_t *)take(n_tiles * PAIRED_STREAMS * w.alive_stride * 4);
+        w.alive_stride = narrow_alive_stride(d.C);
+        for (uint32_t *&list : w.alive) list = (uint32_t *)take(n_tiles * NARROW_STREAMS * w.alive_stride * 4);
         w.bytes = off;
         return w;
     }
@@ -1168,31 +1168,31 @@ int launch_two_phase_wide(const TileLayerArgs &a, int n_tiles, int LA, bool stag
     }
 }
 
-// Two clauses per wave on narrow tiles (score_paired.h).
+// Four clauses per wave on narrow tiles (score_narrow.h).
 template <int SRC, bool LAST>
-int launch_paired_as(const TileLayerArgs &a, const PairedArgs &x, int n_tiles, hipStream_t st) {
-    const size_t lds = paired_lds_bytes(a.tg, a.K, paired_rows_lds(SRC, a.M, x.hv, x.n_types));
+int launch_narrow_as(const TileLayerArgs &a, const NarrowArgs &x, int n_tiles, hipStream_t st) {
+    const size_t lds = narrow_lds_bytes(a.tg, a.K, narrow_rows_lds(SRC, a.M, x.hv, x.n_types));
     static thread_local size_t lds_set = 48 * 1024;
     if (lds > lds_set) {
-        hipError_t e = hipFuncSetAttribute((const void *)k_tile_layer_paired<SRC, LAST>,
+        hipError_t e = hipFuncSetAttribute((const void *)k_tile_layer_narrow<SRC, LAST>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
         lds_set = lds;
     }
-    profile_start(SRC == ROWS_HALF ? (LAST ? "k_tile_layer_paired<score>" : "k_tile_layer_paired<layer0>")
-                                   : (LAST ? "k_tile_layer_paired<messages, score>" : "k_tile_layer_paired<messages>"),
+    profile_start(SRC == ROWS_HALF ? (LAST ? "k_tile_layer_narrow<score>" : "k_tile_layer_narrow<layer0>")
+                                   : (LAST ? "k_tile_layer_narrow<messages, score>" : "k_tile_layer_narrow<messages>"),
                   st);
-    hipLaunchKernelGGL((k_tile_layer_paired<SRC, LAST>), dim3(n_tiles), dim3(PAIRED_WAVES * 64), lds, st, a, x);
-    if (int rc = check_launch("tile_layer_paired")) return rc;
+    hipLaunchKernelGGL((k_tile_layer_narrow<SRC, LAST>), dim3(n_tiles), dim3(NARROW_WAVES * 64), lds, st, a, x);
+    if (int rc = check_launch("tile_layer_narrow")) return rc;
     profile_stop(st);
     return GTM_OK;
 }
 
-int launch_paired(const TileLayerArgs &a, const PairedArgs &x, int n_tiles, int src, bool last, hipStream_t st) {
+int launch_narrow(const TileLayerArgs &a, const NarrowArgs &x, int n_tiles, int src, bool last, hipStream_t st) {
     if (src == ROWS_HALF)
-        return last ? launch_paired_as<ROWS_HALF, true>(a, x, n_tiles, st) : launch_paired_as<ROWS_HALF, false>(a, x, n_tiles, st);
-    return last ? launch_paired_as<ROWS_MESSAGES, true>(a, x, n_tiles, st)
-                : launch_paired_as<ROWS_MESSAGES, false>(a, x, n_tiles, st);
+        return last ? launch_narrow_as<ROWS_HALF, true>(a, x, n_tiles, st) : launch_narrow_as<ROWS_HALF, false>(a, x, n_tiles, st);
+    return last ? launch_narrow_as<ROWS_MESSAGES, true>(a, x, n_tiles, st)
+                : launch_narrow_as<ROWS_MESSAGES, false>(a, x, n_tiles, st);
 }
 
 // Layer 0 can run in two phases (k_tile_two_phase) on tiles of whole-word graph slots staged in
@@ -1223,21 +1223,21 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     // any other tile of whole-word slots whose row offsets fit the 16-bit entries: k_tile_two_phase_wide
     const bool wide = !narrow && tg.slot_words > 0 && (int64_t)tg.rows * tg.tw / 4 < 65536 && !tune(T_NO_TWO_PHASE);
     const bool two_phase = narrow || wide;
-    // Narrow tiles: two clauses per wave (score_paired.h) for the message layers, and for layer 0 when the data
+    // Narrow tiles: four clauses per wave (score_narrow.h) for the message layers, and for layer 0 when the data
     // set's negated literals are the complements of its positive ones, so that the positive rows alone, which
-    // fit in LDS, will do.  GTM_NO_PAIRED_LAYERS / GTM_NO_HALF_ROWS (tuning and test aids) turn them off.
+    // fit in LDS, will do.  GTM_NO_NARROW_LAYERS / GTM_NO_HALF_ROWS (tuning and test aids) turn them off.
     const size_t lds_limit = 160 * 1024;
     const int hv = cfg->literals / 2;
-    const bool paired = paired_geometry(tg) && !tune(T_NO_PAIRED_LAYERS);
-    const bool paired_messages = paired && layers > 1 && paired_lds_bytes(tg, d.K, tile_message_rows(d.M)) <= lds_limit;
-    const bool half_rows0 = paired && !tg.half && (g->flags & GTM_GRAPHS_COMPLEMENTARY) && cfg->literals % 2 == 0 &&
-                            paired_lds_bytes(tg, d.K, hv + g->number_of_node_types + 1) <= lds_limit &&
+    const bool narrow_tiles = narrow_geometry(tg) && !tune(T_NO_NARROW_LAYERS);
+    const bool narrow_messages = narrow_tiles && layers > 1 && narrow_lds_bytes(tg, d.K, tile_message_rows(d.M)) <= lds_limit;
+    const bool half_rows0 = narrow_tiles && !tg.half && (g->flags & GTM_GRAPHS_COMPLEMENTARY) && cfg->literals % 2 == 0 &&
+                            narrow_lds_bytes(tg, d.K, hv + g->number_of_node_types + 1) <= lds_limit &&
                             !tune(T_NO_HALF_ROWS);
     // compiled clause: 8 words of packed 16-bit row entries (16 words of byte offsets on half tiles) + the include words
     const int stride0 = half_rows0 ? w.list_stride : tg.half ? 16 + d.LA : two_phase ? 8 + d.LA : w.list_stride;
     SegmentPlan plan{};
     if (half_rows0)
-        // rows as k_tile_layer_paired<ROWS_HALF> stages them: positive literals, node types, all ones
+        // rows as k_tile_layer_narrow<ROWS_HALF> stages them: positive literals, node types, all ones
         hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C,
                            d.LA, d.B, d.filter, cfg->literals, hv, g->number_of_node_types, hv, hv + g->number_of_node_types,
                            tg.tw, w.list_stride, order, w.lists, d.K, layers == 1 ? s->clause_weights : nullptr, w.wt);
@@ -1289,19 +1289,19 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     a.xpos = tg.half ? g->tiles + tiles_xpos_offset_words(tg, cfg->literals) : nullptr;
     a.walk_factor = 2;
     if (const char *e = tune(T_WIDE_WALK_FACTOR)) a.walk_factor = std::max(1, atoi(e));  // (tuning aid)
-    PairedArgs px{};
+    NarrowArgs px{};
     px.alive_stride = w.alive_stride;
     px.hv = hv;
     px.n_types = g->number_of_node_types;
-    const uint32_t *alive_now = nullptr;  // what the last paired layer left for the next one
+    const uint32_t *alive_now = nullptr;  // what the last layer on narrow tiles left for the next one
     auto layer0 = [&](int n_tiles, bool last) {
         a.lists = w.lists;
         a.stride = stride0;
         if (half_rows0) {
             px.alive_in = nullptr;
-            px.alive_out = !last && paired_messages ? w.alive[0] : nullptr;
+            px.alive_out = !last && narrow_messages ? w.alive[0] : nullptr;
             alive_now = px.alive_out;
-            return launch_paired(a, px, n_tiles, ROWS_HALF, last, st);
+            return launch_narrow(a, px, n_tiles, ROWS_HALF, last, st);
         }
         alive_now = nullptr;
         if (tg.half) return launch_two_phase_half(a, n_tiles, d.LA / 4, last, &plan, st);
@@ -1358,11 +1358,11 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     // the clause evaluation of message layer l on the rows just built (a.lists, a.stride, a.longest_list are set)
     auto message_layer = [&](int n_tiles, int l) {
         const bool last = l == layers - 1 && !tr;
-        if (!paired_messages) return launch_tile_layer(a, n_tiles, ROWS_MESSAGES, last, st);
+        if (!narrow_messages) return launch_tile_layer(a, n_tiles, ROWS_MESSAGES, last, st);
         px.alive_in = alive_now;
         px.alive_out = last || l == layers - 1 ? nullptr : w.alive[alive_now == w.alive[0] ? 1 : 0];
         alive_now = px.alive_out;
-        return launch_paired(a, px, n_tiles, ROWS_MESSAGES, last, st);
+        return launch_narrow(a, px, n_tiles, ROWS_MESSAGES, last, st);
     };
     for (int t0 = tile_first; t0 <= tile_last; t0 += tiles_per_launch) {
         const int n_tiles = tile_last - t0 + 1 < tiles_per_launch ? tile_last - t0 + 1 : tiles_per_launch;
@@ -1997,9 +1997,9 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     // group measured best on 2,000 and 2,500 clauses), but a group gets at least 8 where their
     // automata fit in LDS.
     auto lds_bytes = [&](int per_group) {
-        return (3 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group +
-                2 * (size_t)d.K + 5 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K + 3 * (size_t)p.x_words +
-                (size_t)cfg->literals + 9 * (size_t)d.K) * 4;
+        return (2 * (size_t)p.rows_words + (size_t)per_group * d.LA * d.B + 2 * (size_t)per_group +
+                2 * (size_t)d.K + 5 * (size_t)per_group * d.K + (size_t)per_group * d.LA * d.K + 2 * (size_t)p.x_words +
+                (size_t)cfg->literals + 8 * (size_t)d.K) * 4;
     };
     const size_t lds_limit = 150 * 1024;
     int per_group = (d.C + cus - 1) / cus;

@@ -214,7 +214,7 @@ def test_transform_and_read_outs_match_the_oracle():
 
 @pytest.mark.parametrize("case", [
     # 361-node graphs, one layer (tiles of positive rows only); tiny graphs that share words of a tile row;
-    # two and three layers with edge types and graphs without nodes; one graph of 21 words per tile (two
+    # two and three layers with edge types and graphs without nodes; one graph of 21 words per tile (four
     # clauses per wave)
     dict(g=dict(n_graphs=23, max_nodes=361, min_nodes=300, hv_size=128), m=dict(depth=1), clauses=70, classes=10),
     dict(g=dict(n_graphs=90, max_nodes=3, hv_size=16, node_types=("a", "b")), m=dict(depth=1), clauses=33, classes=2),

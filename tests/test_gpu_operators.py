@@ -999,9 +999,9 @@ NARROW_TILE_SHAPES = [
 
 @pytest.mark.parametrize("shape", NARROW_TILE_SHAPES, ids=lambda s: "narrow%d" % s["seed"])
 @pytest.mark.parametrize("depth", [1, 2, 3])
-@pytest.mark.parametrize("path", ["two-clauses-per-wave", "all-rows-layer-0", "one-clause-per-wave"])
+@pytest.mark.parametrize("path", ["four-clauses-per-wave", "all-rows-layer-0", "one-clause-per-wave"])
 def test_scoring_on_narrow_tiles(shape, depth, path, tune):
-    """Tiles whose rows are at most 32 words wide: two clauses per wave (score_paired.h), for the message
+    """Tiles whose rows are at most 32 words wide: four clauses per wave (score_narrow.h), for the message
     layers and - on a data set whose negated literals are the complements of its positive ones - for
     layer 0 on the positive rows alone; against the oracle and against the kernels that take one clause
     per wave.  The clauses are of three kinds: random ones (most die within the first rows), ones made of
@@ -1012,7 +1012,7 @@ def test_scoring_on_narrow_tiles(shape, depth, path, tune):
     if path == "all-rows-layer-0":
         tune("GTM_NO_HALF_ROWS", "1")
     elif path == "one-clause-per-wave":
-        tune("GTM_NO_PAIRED_LAYERS", "1")
+        tune("GTM_NO_NARROW_LAYERS", "1")
     graphs = helpers.random_graphs(shape["seed"], max_degree=3, **shape["g"])
     hv = graphs.hypervector_size
     M = 1024 if depth > 1 else 64
