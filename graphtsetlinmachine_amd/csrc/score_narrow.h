@@ -22,7 +22,7 @@
 // A clause's compiled list (k_compile_clauses with `half` set: header, rows to AND, rows whose
 // complements to AND, each part a whole number of 8-entry blocks, filled up with the all-ones row
 // to a whole number of windows) is brought in by the quarter-wave that evaluates it, a window of
-// 64 entries at a time - one 16-byte load per lane, requested four clauses ahead - and passes
+// 64 entries at a time - one 16-byte load per lane, the first two windows requested two clauses ahead - and passes
 // through 96 words of LDS of the quarter-wave's own, from which the walk reads it back a block
 // ahead of the rows (the four lanes of a quad read entries 0..3 and 4..7 of a block, and an entry
 // reaches all lanes inside the add that forms the row's address).  Two blocks per trip, 16 row
@@ -48,7 +48,7 @@ constexpr int NARROW_PER_WAVE = 64 / NARROW_GROUP;     // clauses under way in a
 constexpr int NARROW_STREAMS = NARROW_PER_WAVE * NARROW_WAVES;
 constexpr int NARROW_WINDOW = 4 * NARROW_GROUP;        // list entries of a clause in LDS at a time: 4 per lane of its group
 constexpr int NARROW_LIST_WORDS = NARROW_WINDOW + 32;  // + what the walk reads ahead of the rows it is at
-constexpr int NARROW_AHEAD = 4;                        // clauses of a stream whose list and truth words are on their way
+constexpr int NARROW_AHEAD = 2;                        // clauses of a stream whose list and truth words are on their way
 constexpr int NARROW_MAX_WORDS = 2 * NARROW_GROUP;     // widest row
 
 struct NarrowArgs {
@@ -99,6 +99,10 @@ __device__ __forceinline__ void narrow_block_addresses(uint32_t lo, uint32_t hi,
 __device__ __forceinline__ uint32_t narrow_pair(uint32_t r0, uint32_t r1, uint32_t flip) {
     // truth table over (r0, r1, flip): 1 for (1, 1, 0) and for (0, 0, 1)
     return (uint32_t)__builtin_amdgcn_bitop3_b32((int)r0, (int)r1, (int)flip, 0x42);
+}
+
+__device__ __forceinline__ uint32_t narrow_and3(uint32_t a, uint32_t b, uint32_t c) {
+    return (uint32_t)__builtin_amdgcn_bitop3_b32((int)a, (int)b, (int)c, 0x80);
 }
 
 template <int SRC, bool LAST>
@@ -189,7 +193,7 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
     };
     struct Item {
         int c;        // the clause, -1: none
-        uint4 e;      // entries 4 gl .. 4 gl + 3 of its list
+        uint4 e, e2;  // entries 4 gl .. 4 gl + 3 of the first and of the second window of its list
         uint2 truth;  // words 2 gl, 2 gl + 1 of its truth row (message layers)
     };
     auto fetch = [&](int i, Item &it) {  // item i's loads; i runs up by one from call to call
@@ -199,7 +203,9 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
         }
         it.c = clause_of(i);
         const int c = it.c < 0 ? 0 : it.c;
-        it.e = *reinterpret_cast<const uint4 *>(a.lists + (int64_t)c * a.stride + 4 * gl);
+        const uint4 *list = reinterpret_cast<const uint4 *>(a.lists + (int64_t)c * a.stride + 4 * gl);
+        it.e = list[0];
+        it.e2 = list[NARROW_WINDOW / 4];  // (a list is at least two windows long, filled up with the all-ones row)
         it.truth = make_uint2(0u, 0u);
         if (SRC == ROWS_MESSAGES) it.truth = *reinterpret_cast<const uint2 *>(bitmap + (int64_t)c * tw + (active ? 2 * gl : 0));
     };
@@ -250,7 +256,10 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
             uint4 e = now.e;
             for (int b0 = 0; b0 < nb_most; b0 += NARROW_WINDOW / 8) {  // one window of the lists after the other
                 if (!work_left(b0)) break;
-                if (b0 > 0) e = *reinterpret_cast<const uint4 *>(a.lists + (int64_t)c * a.stride + b0 * 8 + 4 * gl);
+                if (b0 == NARROW_WINDOW / 8)
+                    e = now.e2;
+                else if (b0 > 0)  // (a clause of more than 126 literals: its further windows are fetched when it gets there)
+                    e = *reinterpret_cast<const uint4 *>(a.lists + (int64_t)c * a.stride + b0 * 8 + 4 * gl);
                 // The compiled list is filled up with the all-ones row to the end of its last window.  A group whose
                 // list has no such window (it ended in an earlier one; no clause; a clause false everywhere on arrival:
                 // nb = 0) walks the all-ones row while the others go on.
@@ -260,7 +269,11 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
                 *reinterpret_cast<uint4 *>(my_list + 4 * gl) = e;
                 // (a wave's LDS accesses are carried out in order: the reads below see the entries just written)
                 const int lim_most = nb_most - b0 < NARROW_WINDOW / 8 ? nb_most - b0 : NARROW_WINDOW / 8;
+                // bit b: block b0 + b of this group's list is one of complements (blocks plain .. nb - 1): its rows come in inverted
+                const int from = plain - b0 < 0 ? 0 : plain - b0 > 8 ? 8 : plain - b0, to = nb - b0 < 0 ? 0 : nb - b0 > 8 ? 8 : nb - b0;
+                const int flip_bits = to > from ? ((1 << to) - 1) & ~((1 << from) - 1) : 0;
                 uint32_t lo0 = quad_entry[0], hi0 = quad_entry[4], lo1 = quad_entry[8], hi1 = quad_entry[12];
+#pragma unroll 2
                 for (int b = 0; b < lim_most && work_left(b0 + b); b += 2) {
                     const uint32_t n_lo0 = quad_entry[8 * b + 16], n_hi0 = quad_entry[8 * b + 20];
                     const uint32_t n_lo1 = quad_entry[8 * b + 24], n_hi1 = quad_entry[8 * b + 28];
@@ -272,21 +285,22 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
                     for (int u = 0; u < 8; ++u) r[u] = *(NarrowLdsWords)(uintptr_t)adr0[u];
 #pragma unroll
                     for (int u = 0; u < 8; ++u) r[8 + u] = *(NarrowLdsWords)(uintptr_t)adr1[u];
-                    // a block of complements for this group (blocks plain .. nb - 1 of its list): the rows come in inverted
-                    const int gb = b0 + b;
-                    uint32_t flip0 = gb >= plain && gb < nb ? 0xFFFFFFFFu : 0u;
-                    uint32_t flip1 = gb + 1 >= plain && gb + 1 < nb ? 0xFFFFFFFFu : 0u;
-                    asm("" : "+v"(flip0), "+v"(flip1));  // (plain words from here on: one three-input operation per pair of rows)
-                    uint2 t[8];
+                    // all ones for a block of complements, else zero (a signed one-bit field of flip_bits)
+                    const uint32_t flip0 = (uint32_t)__builtin_amdgcn_sbfe(flip_bits, b, 1);
+                    const uint32_t flip1 = (uint32_t)__builtin_amdgcn_sbfe(flip_bits, b + 1, 1);
+                    uint32_t tx[8], ty[8];
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
-                        t[u].x = narrow_pair(r[2 * u].x, r[2 * u + 1].x, flip0);
-                        t[u].y = narrow_pair(r[2 * u].y, r[2 * u + 1].y, flip0);
-                        t[4 + u].x = narrow_pair(r[8 + 2 * u].x, r[9 + 2 * u].x, flip1);
-                        t[4 + u].y = narrow_pair(r[8 + 2 * u].y, r[9 + 2 * u].y, flip1);
+                        tx[u] = narrow_pair(r[2 * u].x, r[2 * u + 1].x, flip0);
+                        ty[u] = narrow_pair(r[2 * u].y, r[2 * u + 1].y, flip0);
+                        tx[4 + u] = narrow_pair(r[8 + 2 * u].x, r[9 + 2 * u].x, flip1);
+                        ty[4 + u] = narrow_pair(r[8 + 2 * u].y, r[9 + 2 * u].y, flip1);
                     }
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) acc.x &= t[u].x, acc.y &= t[u].y;
+                    for (int u = 0; u < 8; u += 2) {
+                        acc.x = narrow_and3(acc.x, tx[u], tx[u + 1]);
+                        acc.y = narrow_and3(acc.y, ty[u], ty[u + 1]);
+                    }
                     nzw = __ballot((acc.x | acc.y) != 0u);
                     lo0 = n_lo0, hi0 = n_hi0, lo1 = n_lo1, hi1 = n_hi1;
                 }
