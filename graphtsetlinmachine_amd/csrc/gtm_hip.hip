@@ -17,6 +17,7 @@
 #include "philox.h"
 #include "score_tiles.h"
 #include "score_narrow.h"
+#include "score_messages.h"
 
 namespace {
 
@@ -61,6 +62,7 @@ int check_launch(const char *what) {
     X(FIT_PER_GROUP) \
     X(FIT_SPIN_LIMIT) \
     X(HALF_LANE_WORDS) \
+    X(MESSAGES_IN_LDS) \
     X(NODE_MESSAGES_BY_ATOMICS) \
     X(NO_DEEP_FIT) \
     X(NO_DEEP_PERSISTENT_FIT) \
@@ -1341,8 +1343,30 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             }
         }
     }
+    // One tile per workgroup with the vectors in LDS (score_messages.h) where a graph's two sets of vectors are too
+    // big for the kernel above.  GTM_MESSAGES_IN_LDS (tuning and test aid): 0 keeps the three launches, 1 prefers
+    // this kernel wherever the shape allows it.
+    TileMessagesPlan in_lds{};
+    {
+        const char *e = tune(T_MESSAGES_IN_LDS);
+        const bool off = e && atoi(e) == 0, preferred = e && atoi(e) != 0;
+        if (layers > 1 && !off && (preferred || !fused_messages)) in_lds = tile_messages_lds_plan(tg, d.M, lds_limit);
+    }
+    if (in_lds.ok) {
+        static thread_local size_t in_lds_set = 48 * 1024;
+        if (in_lds.lds_bytes > in_lds_set) {
+            if (hipFuncSetAttribute((const void *)k_tile_messages_in_lds, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)in_lds.lds_bytes) != hipSuccess) {
+                (void)hipGetLastError();
+                in_lds.ok = 0;
+            } else {
+                in_lds_set = in_lds.lds_bytes;
+            }
+        }
+    }
+    if (in_lds.ok) fused_messages = false;
     const bool by_bit = !tune(T_NODE_MESSAGES_BY_ATOMICS);  // tuning aid: the earlier kernel
-    if (layers > 1 && (fused_messages || by_bit)) {
+    if (layers > 1 && !in_lds.ok && (fused_messages || by_bit)) {
         // the clauses of every message bit, for the kernels that build what the nodes send
         hipLaunchKernelGGL(k_message_bit_index, dim3(1), dim3(BIT_INDEX_BLOCK), 0, st, s->hypervectors, d.C, d.MB, d.M,
                            w.bit_start, w.bit_cursor, w.bit_clauses);
@@ -1374,6 +1398,21 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         for (int l = 1; l < layers; ++l) {
             // the layer's message rows for these tiles (score_tiles.h): one graph per workgroup with its
             // vectors in LDS when they fit, else three launches with the vectors in global memory
+            if (in_lds.ok) {
+                profile_start("k_tile_messages_in_lds", st);
+                hipLaunchKernelGGL(k_tile_messages_in_lds, dim3(n_tiles), dim3(TILE_MESSAGES_LDS_BLOCK), in_lds.lds_bytes, st,
+                                   w.tile_bitmap, d.C, tg, t0, g->number_of_graphs, d.M, s->hypervectors, d.MB, alive_now,
+                                   w.alive_stride, g->node_index, g->number_of_graph_nodes, g->number_of_graph_node_edges,
+                                   g->edge_index, g->edge, g->total_edges > 0 ? 1 : 0, in_lds.main_words, in_lds.range_words,
+                                   w.message_rows);
+                if (int rc = check_launch("tile_messages_in_lds")) return rc;
+                profile_stop(st);
+                a.lists = w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride;
+                a.stride = w.message_list_stride;
+                a.longest_list = w.longest_list + (l - 1);
+                if (int rc = message_layer(n_tiles, l)) return rc;
+                continue;
+            }
             if (fused_messages) {
                 profile_start("k_tile_messages_fused", st);
                 hipLaunchKernelGGL(k_tile_messages_fused, dim3(tg.gpt, n_tiles), dim3(TILE_FUSED_MESSAGES_BLOCK),

@@ -1,0 +1,255 @@
+// The message rows of a layer, one TILE per workgroup, with everything between the truth rows
+// and the literal-major rows kept in LDS (graphs too big for k_tile_messages_fused, whose two sets
+// of vectors per graph must both fit: a graph of 841 nodes with messages of 1,024 bits).
+//
+// A message factors (kernels.py:565-588): what a node sends is the OR of the hypervector bits of
+// the clauses true at it, and what a neighbour receives along an edge of type t is that vector
+// rotated by t.  Four steps on one region of LDS:
+//   1. rows[p] |= truth row of every clause whose hypervector holds bit p: M rows of tw words,
+//      LDS atomics.  Each truth row is read ONCE (a quarter-wave per clause, 8 bytes per lane,
+//      the way k_tile_layer_narrow wrote it), and only the rows of the clauses that the
+//      evaluation listed as true somewhere in the tile when such lists are handed in;
+//   2. the M x (32 tw) bit matrix is turned node-major in place - every half-wave takes 32 x 32
+//      bit blocks through registers (a transposition across its lanes), all blocks are read
+//      before any is written back: slot n's vector of MW words now starts at n (MW + 1);
+//   3. along the edges, a range of destination slots at a time (as many as the LDS left over
+//      holds): every thread owns a source slot and ORs its vector, rotated by the edge's type,
+//      into the vectors of its destinations inside the range (LDS atomics; the edges of a node
+//      come from global memory once, the first four stay in registers);
+//   4. the range's received vectors are turned literal-major, 32 x 32 bits per half-wave again,
+//      and stored, 16 bytes per lane, as words of the rows [M + 2][tw] that the next layer's
+//      evaluation stages.
+// No vector ever goes to global memory and nothing is cleared there.
+#pragma once
+
+#include <type_traits>
+
+constexpr int TILE_MESSAGES_LDS_BLOCK = 1024;
+static_assert(TILE_MESSAGES_LDS_BLOCK / 16 == NARROW_STREAMS, "a quarter-wave per stream of k_tile_layer_narrow");
+
+// The word of lane `from` (0 .. 15) of this lane's row of 16 lanes: a lane move on the vector unit.  (`from` is
+// a constant wherever this is called - an unrolled loop's counter - and the switch folds away.)
+__device__ __forceinline__ uint32_t tile_row_share(uint32_t v, int from) {
+    switch (from & 15) {
+#define GTM_ROW_SHARE(n) \
+    case n: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x150 + n, 0xF, 0xF, true);
+        GTM_ROW_SHARE(0) GTM_ROW_SHARE(1) GTM_ROW_SHARE(2) GTM_ROW_SHARE(3) GTM_ROW_SHARE(4) GTM_ROW_SHARE(5)
+        GTM_ROW_SHARE(6) GTM_ROW_SHARE(7) GTM_ROW_SHARE(8) GTM_ROW_SHARE(9) GTM_ROW_SHARE(10) GTM_ROW_SHARE(11)
+        GTM_ROW_SHARE(12) GTM_ROW_SHARE(13) GTM_ROW_SHARE(14)
+#undef GTM_ROW_SHARE
+    default: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x15F, 0xF, 0xF, true);
+    }
+}
+
+struct TileMessagesPlan {
+    int ok;
+    int main_words;   // LDS words of the region that holds the rows, then the vectors
+    int range_words;  // words of destination slots (32 each) whose received vectors fit beside it
+    size_t lds_bytes;
+};
+
+// Shapes the kernel takes: M a multiple of 32 and at most 1,024, tiles of at most 32 words (one
+// thread per node slot), and room in LDS for the vectors plus at least 128 received ones.
+inline TileMessagesPlan tile_messages_lds_plan(const TileGeom &g, int M, size_t lds_limit) {
+    TileMessagesPlan p{};
+    if (!g.ok || M < 32 || M % 32 != 0 || M > 1024 || g.tw > 32 || g.tw % 4 != 0) return p;
+    const int MW = M / 32;
+    const size_t rows = (size_t)M * g.tw, vectors = (size_t)g.tw * 32 * (MW + 1);
+    const size_t main_words = rows > vectors ? rows : vectors;
+    const size_t per_word = (size_t)32 * (MW + 1);
+    if ((main_words + 4 * per_word) * 4 > lds_limit) return p;
+    size_t range = (lds_limit / 4 - main_words) / per_word & ~(size_t)3;  // (rows are stored four words at a time)
+    if (range > (size_t)g.tw) range = (size_t)g.tw;
+    p.ok = 1;
+    p.main_words = (int)main_words;
+    p.range_words = (int)range;
+    p.lds_bytes = (main_words + range * per_word) * 4;
+    return p;
+}
+
+__global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_lds(
+    const uint32_t *__restrict__ bitmap, int C, TileGeom tg, int tile0, int G, int M, const uint32_t *__restrict__ hv, int MB,
+    const uint32_t *__restrict__ alive, int alive_stride, const uint32_t *__restrict__ node_index,
+    const uint32_t *__restrict__ n_nodes, const uint32_t *__restrict__ n_edges, const uint32_t *__restrict__ edge_index,
+    const uint32_t *__restrict__ edge, int has_edges, int main_words, int range_words, uint32_t *__restrict__ rows) {
+    extern __shared__ uint32_t lds[];
+    constexpr int NT = TILE_MESSAGES_LDS_BLOCK;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tile_local = blockIdx.x;
+    const int tw = tg.tw, MW = M >> 5, VS = MW + 1, S = tw * 32;
+    uint32_t *main_region = lds;
+    uint32_t *got = lds + main_words;
+    uint32_t *out = rows + (int64_t)tile_local * (M + 2) * tw;
+
+    for (int i = tid; i < M * tw; i += NT) main_region[i] = 0u;
+    __syncthreads();
+
+    // 1. the rows of what is sent, literal-major.  Lane l of a quarter-wave fetches the number and the first two
+    // hypervector bits of the stream's clause 16 k + l, a group of 16 clauses ahead of the truth rows; a clause's
+    // number and bits then reach the 16 lanes by a lane move (row_share), and eight truth rows are on their way
+    // per quarter-wave.
+    {
+        const int group = lane >> 4, gl = lane & 15, q = wave * 4 + group;
+        const uint32_t *truth = bitmap + (int64_t)tile_local * C * tw;
+        const uint32_t *list = alive ? alive + ((int64_t)tile_local * NARROW_STREAMS + q) * alive_stride : nullptr;
+        const int n_mine = list ? (int)list[0] : (q < C ? (C - q + NARROW_STREAMS - 1) / NARROW_STREAMS : 0);
+        const bool has_words = 2 * gl < tw;
+        uint32_t id_next = 0u, bit0_next = 0u, bit1_next = 0u;
+        // (every load below is unconditional, from an address that exists, and what it brought is dropped
+        // afterwards where it was not wanted: loads under a condition would wait for one another)
+        auto fetch = [&](int i) {
+            const int at = i < n_mine ? i : n_mine - 1;
+            id_next = list ? list[1 + at] : (uint32_t)(q + NARROW_STREAMS * at);
+            bit0_next = hv[(int64_t)id_next * MB];
+            bit1_next = hv[(int64_t)id_next * MB + (MB > 1 ? 1 : 0)];
+        };
+        if (n_mine > 0) fetch(gl);
+        for (int i0 = 0; i0 < n_mine; i0 += 16) {  // (the lanes of a quarter-wave leave the loop together)
+            const uint32_t id = id_next, bit0 = bit0_next, bit1 = bit1_next;
+            fetch(i0 + 16 + gl);
+            const int n_here = n_mine - i0 < 16 ? n_mine - i0 : 16;
+            auto eight = [&](auto first_of_eight) {  // clauses u0 .. u0 + 7 of the 16
+                constexpr int u0 = decltype(first_of_eight)::value;
+                uint32_t c[8];
+                uint2 t[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    c[u] = tile_row_share(id, u0 + u);  // (past the stream's end: its last clause once more)
+                    t[u] = *reinterpret_cast<const uint2 *>(truth + (int64_t)c[u] * tw + (has_words ? 2 * gl : 0));
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const uint32_t h0 = tile_row_share(bit0, u0 + u), h1 = tile_row_share(bit1, u0 + u);
+                    if (u0 + u >= n_here || !has_words || (t[u].x | t[u].y) == 0u) continue;
+                    const unsigned long long both = (unsigned long long)t[u].x | ((unsigned long long)t[u].y << 32);
+                    for (int j = 0; j < MB; ++j) {
+                        const uint32_t h = j == 0 ? h0 : j == 1 ? h1 : hv[(int64_t)c[u] * MB + j];
+                        if (h >= (uint32_t)M) continue;
+                        // (tw is even: the two words are one aligned 64-bit word of LDS)
+                        atomicOr(reinterpret_cast<unsigned long long *>(main_region + h * tw + 2 * gl), both);
+                    }
+                }
+            };
+            eight(std::integral_constant<int, 0>{});
+            if (n_here > 8) eight(std::integral_constant<int, 8>{});
+        }
+    }
+    __syncthreads();
+
+    // 2. node-major in place: block (j, w) - rows 32 j .. 32 j + 31, word w - becomes word j of slots 32 w .. 32 w + 31
+    const int hw = tid >> 5, hl = lane & 31;
+    {
+        const int n_blocks = MW * tw;
+        uint32_t held[32];
+#pragma unroll
+        for (int k = 0; k < 32; ++k) {
+            held[k] = 0u;
+            if (k * 32 >= n_blocks) continue;  // (the same for every thread)
+            const int id = k * 32 + hw;
+            uint32_t v = 0u;
+            if (id < n_blocks) {
+                const int j = id / tw, w = id - j * tw;
+                v = main_region[(32 * j + hl) * tw + w];
+            }
+            held[k] = tile_transpose32(v, lane);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 32; ++k) {
+            const int id = k * 32 + hw;
+            if (id < n_blocks) {
+                const int j = id / tw, w = id - j * tw;
+                main_region[(32 * w + hl) * VS + j] = held[k];
+            }
+        }
+    }
+
+    // the all-ones row and the row of graphs without nodes (slot bit 0 of each: kernels.py:443-466,505-527 leave every
+    // clause true for such a graph at every layer, which the message literals must not undo)
+    for (int w = tid; w < tw; w += NT) {
+        const int used = tg.slot_words == 0 ? tw : tg.gpt * tg.slot_words;
+        uint32_t empties = 0u;
+        for (int b = 0; b < 32; ++b) {
+            const int pos = w * 32 + b, gj = pos / tg.slot_bits;
+            const int64_t g = (int64_t)(tile0 + tile_local) * tg.gpt + gj;
+            if (pos == gj * tg.slot_bits && gj < tg.gpt && g < G && n_nodes[g] == 0u) empties |= 1u << b;
+        }
+        out[(int64_t)M * tw + w] = w < used ? 0xFFFFFFFFu : 0u;
+        out[(int64_t)(M + 1) * tw + w] = empties;
+    }
+
+    // this thread's source slot and its edges
+    uint32_t ne = 0u, nodes_of_graph = 0u;
+    int slot0 = 0;
+    const uint2 *out_edges = nullptr;
+    if (tid < S && has_edges) {
+        const int gj = tid / tg.slot_bits, n = tid - gj * tg.slot_bits;
+        const int64_t g = (int64_t)(tile0 + tile_local) * tg.gpt + gj;
+        if (gj < tg.gpt && g < G && (uint32_t)n < n_nodes[g]) {
+            const int64_t row = (int64_t)node_index[g] + n;
+            ne = n_edges[row];
+            out_edges = reinterpret_cast<const uint2 *>(edge) + edge_index[row];
+            nodes_of_graph = n_nodes[g];
+            slot0 = gj * tg.slot_bits;
+        }
+    }
+    uint2 first[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) first[u] = (uint32_t)u < ne ? out_edges[u] : make_uint2(0u, 0u);
+    const uint32_t *mine = main_region + (tid < S ? tid : 0) * VS;
+
+    for (int w_lo = 0; w_lo < tw; w_lo += range_words) {
+        const int w_hi = w_lo + range_words < tw ? w_lo + range_words : tw, nw = w_hi - w_lo;
+        for (int i = tid; i < nw * 32 * VS; i += NT) got[i] = 0u;
+        __syncthreads();  // (also: every vector of step 2 is in place)
+
+        // 3. along the edges into the range
+        for (uint32_t e0 = 0; e0 < ne; e0 += 4) {
+            uint2 pair[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                pair[u] = e0 == 0 ? first[u] : (e0 + u < ne ? out_edges[e0 + u] : make_uint2(0u, 0u));
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (e0 + u >= ne) break;
+                const uint32_t dst = pair[u].x;
+                if (dst >= nodes_of_graph) continue;
+                const int to_slot = slot0 + (int)dst, to_word = to_slot >> 5;
+                if (to_word < w_lo || to_word >= w_hi) continue;
+                const uint32_t shift = pair[u].y % (uint32_t)M;
+                const int r = (int)(shift & 31u);
+                uint32_t *to = got + (to_slot - 32 * w_lo) * VS;
+                // bit p of what arrives is bit (p - shift) mod M of what was sent: word j, moved up by r bits with
+                // the top of word j - 1 below it, lands in word (j + shift / 32) mod MW
+                int at = (int)(shift >> 5);
+                uint32_t below = mine[MW - 1];
+                for (int j = 0; j < MW; ++j) {
+                    const uint32_t cur = mine[j];
+                    const uint32_t word = r ? (cur << r) | (below >> (32 - r)) : cur;
+                    if (word) atomicOr(&to[at], word);
+                    at = at + 1 == MW ? 0 : at + 1;
+                    below = cur;
+                }
+            }
+        }
+        __syncthreads();
+
+        // 4. literal-major: block (j, w) of the range - word j of slots 32 w .. 32 w + 31 - becomes word w of rows
+        // 32 j .. 32 j + 31; a half-wave turns four neighbouring blocks and each lane stores its row's four words at once
+        const int nq = nw >> 2, n_units = MW * nq;
+        for (int k = 0; k * 32 < n_units; ++k) {
+            const int id = k * 32 + hw;
+            const int j = id / nq, wq = id - j * nq;
+            uint32_t column[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t v = id < n_units ? got[(32 * (4 * wq + u) + hl) * VS + j] : 0u;
+                column[u] = tile_transpose32(v, lane);
+            }
+            if (id < n_units)
+                *reinterpret_cast<uint4 *>(out + (int64_t)(32 * j + hl) * tw + w_lo + 4 * wq) =
+                    make_uint4(column[0], column[1], column[2], column[3]);
+        }
+        __syncthreads();
+    }
+}

@@ -212,7 +212,7 @@ def oracle_at(tm, state, graphs):
     return model
 
 
-@pytest.mark.parametrize("scoring", ["default", "rows-in-place", "full-walk"])
+@pytest.mark.parametrize("scoring", ["default", "rows-in-place", "full-walk", "messages-in-three-launches"])
 def test_scoring_the_colour_configuration_at_a_trained_state(scoring, tune):
     """Every scoring path that this shape can take, on the trained state, against the C oracle."""
     wl, tm, state = trained_colour_state()
@@ -223,6 +223,8 @@ def test_scoring_the_colour_configuration_at_a_trained_state(scoring, tune):
     elif scoring == "full-walk":
         tune("GTM_NO_HALF_ROWS", "1")
         tune("GTM_NO_TWO_PHASE", "1")    # layer 0 as a walk of every literal's row
+    elif scoring == "messages-in-three-launches":
+        tune("GTM_MESSAGES_IN_LDS", "0")  # the vectors of what the nodes send and receive in global memory
     model = oracle_at(tm, state, wl.graphs_test)
     want = oc.score(model, wl.graphs_test, threads=min(16, oc.threads_available()))
     tm._test_graphs = None  # (the tiles are built per path)

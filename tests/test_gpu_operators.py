@@ -999,7 +999,8 @@ NARROW_TILE_SHAPES = [
 
 @pytest.mark.parametrize("shape", NARROW_TILE_SHAPES, ids=lambda s: "narrow%d" % s["seed"])
 @pytest.mark.parametrize("depth", [1, 2, 3])
-@pytest.mark.parametrize("path", ["four-clauses-per-wave", "all-rows-layer-0", "one-clause-per-wave"])
+@pytest.mark.parametrize("path", ["four-clauses-per-wave", "all-rows-layer-0", "one-clause-per-wave",
+                                  "messages-of-a-tile-in-lds", "messages-in-three-launches"])
 def test_scoring_on_narrow_tiles(shape, depth, path, tune):
     """Tiles whose rows are at most 32 words wide: four clauses per wave (score_narrow.h), for the message
     layers and - on a data set whose negated literals are the complements of its positive ones - for
@@ -1013,6 +1014,13 @@ def test_scoring_on_narrow_tiles(shape, depth, path, tune):
         tune("GTM_NO_HALF_ROWS", "1")
     elif path == "one-clause-per-wave":
         tune("GTM_NO_NARROW_LAYERS", "1")
+    elif depth == 1:
+        pytest.skip("no messages at depth 1")
+    elif path == "messages-of-a-tile-in-lds":  # (score_messages.h; by itself only where a graph's vectors are too big
+        tune("GTM_MESSAGES_IN_LDS", "1")       # for one workgroup per graph: the graphs of 650 and 700 nodes here)
+    elif path == "messages-in-three-launches":
+        tune("GTM_MESSAGES_IN_LDS", "0")
+        tune("GTM_NO_FUSED_MESSAGES", "1")
     graphs = helpers.random_graphs(shape["seed"], max_degree=3, **shape["g"])
     hv = graphs.hypervector_size
     M = 1024 if depth > 1 else 64
