@@ -150,10 +150,7 @@ def other_run(name, n_train, n_test, check_graphs, check_seconds=12.0):
     tm = MultiClassGraphTsetlinMachine(**wl.params, seed=42)
     tm.fit(wl.graphs_train, wl.Y_train, epochs=0, incremental=True)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
-    torch.cuda.synchronize()
-    t_train = time.perf_counter() - t0
+    t_train, train_kernels = timed_fit(tm, wl.graphs_train, wl.Y_train, epochs=1, incremental=True)
     tm.score_device(wl.graphs_test)  # uploads the test graphs
     torch.cuda.synchronize()
     # (a pass over the small test sets takes a millisecond or less: one call alone would time the call, not the GPU)
@@ -188,6 +185,7 @@ def other_run(name, n_train, n_test, check_graphs, check_seconds=12.0):
     n_checked = sum(v if isinstance(v, int) else len(v) for v in checked.values())
     return {
         "train_graphs": n_train, "test_graphs": n_test, "train_graphs_per_s": round(n_train / t_train, 1),
+        "train_kernels": train_kernels,
         "inference_graphs_per_s": round(n_test * 5 / run["wall"], 1),
         "test_accuracy": round(float((sums.argmax(axis=1) == wl.Y_test).mean()), 4),
         "mean_included_literals": round(mean_included_literals(tm), 2),
@@ -382,6 +380,24 @@ def mean_included_literals(tm):
     return float(np.unpackbits(plane.view(np.uint8)).sum()) / tm.number_of_clauses
 
 
+def timed_fit(tm, *fit_args, **fit_kwargs):
+    """(seconds, [{kernel, launches, ms}]) of a call of tm.fit: wall clock around the call, and the library's own
+    events around the training kernels it launched (one launch per call for the one-launch kernels)."""
+    import torch
+
+    from graphtsetlinmachine_amd import _abi
+
+    _abi.call("gtm_profile_enable", 1)
+    t0 = time.perf_counter()
+    tm.fit(*fit_args, **fit_kwargs)
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    kernels = [{"kernel": k, "launches": n, "ms": round(ms, 3)} for k, n, ms in read_kernel_breakdown()]
+    read_kernel_profile()  # (clears the record)
+    _abi.call("gtm_profile_enable", 0)
+    return seconds, kernels
+
+
 def time_scoring(tm, test, steps, warmup, graphs):
     """`steps` timed passes of gtm_score over the resident test graphs after `warmup` untimed ones."""
     import torch
@@ -490,7 +506,7 @@ def main():
     # (the headline, `value`), and after two epochs more.
     states = []
     early = min(5000, args.train_graphs // 2)
-    t_train = 0.0
+    t_train, train_kernels = 0.0, []
     if early > 0 and args.train_epochs >= 1 and not args.one_state:
         t0 = time.time()
         tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True, examples=(0, early))
@@ -498,17 +514,13 @@ def main():
         t_train += time.time() - t0
         run = time_scoring(tm, test, args.steps, args.warmup, args.graphs)
         states.append(state_entry("after %d training graphs" % early, run, None if args.no_cpu else c_oracle_agrees(run)))
-        t0 = time.time()
-        tm.fit(wl.graphs_train, wl.Y_train, epochs=1, incremental=True, examples=(early, args.train_graphs - early))
+        seconds, train_kernels = timed_fit(tm, wl.graphs_train, wl.Y_train, epochs=1, incremental=True,
+                                           examples=(early, args.train_graphs - early))
+        t_train += seconds
         if args.train_epochs > 1:
-            tm.fit(wl.graphs_train, wl.Y_train, epochs=args.train_epochs - 1, incremental=True)
+            t_train += timed_fit(tm, wl.graphs_train, wl.Y_train, epochs=args.train_epochs - 1, incremental=True)[0]
     elif not args.load_state:
-        t0 = time.time()
-        tm.fit(wl.graphs_train, wl.Y_train, epochs=args.train_epochs, incremental=True)
-    else:
-        t0 = time.time()
-    torch.cuda.synchronize()
-    t_train += time.time() - t0
+        t_train, train_kernels = timed_fit(tm, wl.graphs_train, wl.Y_train, epochs=args.train_epochs, incremental=True)
     train_gps = args.train_graphs * args.train_epochs / max(t_train, 1e-9)
     if args.save_state:
         import contextlib
@@ -660,7 +672,7 @@ def main():
                    "mean_included_literals": round(included_main, 2),
                    "untimed_passes_before_warmup": SETTLE},
         "roofline": roofline, "cpu_baseline": cpu,
-        "train_graphs_per_s": round(train_gps, 1), "test_accuracy": round(accuracy, 4),
+        "train_graphs_per_s": round(train_gps, 1), "train_kernels": train_kernels, "test_accuracy": round(accuracy, 4),
         "event_ms_per_step": round(event_ms, 4), "data_build_s": round(t_data, 1),
         "other_workloads": others,
     }
