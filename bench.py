@@ -29,16 +29,16 @@ VALU_PEAK_LANE_OPS = 256 * 64 * 2.4e9  # 32-bit integer lane operations per seco
 # Hardware counters of the scoring kernel on the convolutional workload (10,000 graphs per launch, state after
 # one epoch), from rocprofv3 --pmc runs of this file; the summaries and the commands are under profiles/.
 # FETCH_SIZE counts 2 KiB per unit and WRITE_SIZE 1 KiB per unit on this part (a 256 MiB copy kernel reads
-# 131,085 and writes 262,144).  valu_busy = SQ_INSTS_VALU x 4 clocks / (1,024 SIMDs x the launch's clocks at
-# 2.4 GHz).  The figures belong to the kernel's source text as it was when they were taken: `source_sha256` is
+# 131,087 and writes 262,144).  valu_busy = SQ_INSTS_VALU x 4 clocks / (4 SIMDs x SQ_BUSY_CU_CYCLES): the share of
+# the clocks in which a CU has work in which its vector ALUs issue.  The figures belong to the kernel's source text as it was when they were taken: `source_sha256` is
 # the hash of the text of the functions named in `functions` (kernel_source_hash below), and a run whose
 # library was built from another text reports no counters rather than stale ones.
 MEASURED_COUNTERS = {
     "convolutional_images": {
-        "kernel": "k_tile_two_phase_half<score>", "commit": "9ca7f4a",
-        "functions": ("k_compile_clauses_half", "half_combine", "k_tile_two_phase_half"),
-        "source_sha256": "4674b2f768f2680cb3bb17b2d6e4a5e943a501f092c1e4fc1531b1ee59ce3ed8",
-        "fetch_units": 81892.2, "write_units": 401.8, "valu_busy": 0.65, "graphs": 10000,
+        "kernel": "k_tile_two_phase_half<score>", "commit": "40c229b",
+        "functions": ("tile_segments_block", "k_compile_clauses_half", "half_combine", "k_tile_two_phase_half"),
+        "source_sha256": "dea60f50bdf82c2f6d25df88e1b65e4a6c028fc8a532703f6dbe672ad5b6be9b",
+        "fetch_units": 120409.8, "write_units": 648.6, "valu_busy": 0.72, "graphs": 10000,
     },
 }
 
