@@ -63,6 +63,7 @@ int check_launch(const char *what) {
     X(FIT_SPIN_LIMIT) \
     X(HALF_LANE_WORDS) \
     X(MESSAGES_IN_LDS) \
+    X(NARROW_READS) \
     X(NODE_MESSAGES_BY_ATOMICS) \
     X(NO_DEEP_FIT) \
     X(NO_DEEP_PERSISTENT_FIT) \
@@ -660,8 +661,8 @@ struct ScoreWs {
     uint32_t *sent, *got;     // [tiles per launch][tw * 32 node slots][ceil(M / 32)]  (tile path, depth > 1)
     uint32_t *message_rows;   // [tiles per launch][M + 2][tw]  (tile path, depth > 1)
     uint32_t *bit_start, *bit_cursor, *bit_clauses;  // [M + 1], [M], [C * MB]: the clauses of every message bit (tile path, depth > 1)
-    uint32_t *alive[2];       // [tiles per launch][NARROW_STREAMS][alive_stride] clauses still true somewhere in a tile, layer to layer
-    int alive_stride;
+    uint32_t *alive[2];       // [tiles per launch][streams][alive_stride] clauses still true somewhere in a tile, layer to layer
+    size_t alive_words;       // room per tile
     TileSegment *segments;    // [tiles + 2 * TILE_SEGMENTS_MAX_SHARES] which clauses of which tile a workgroup takes (half tiles)
     size_t vector_words;      // words of sent (and of got)
     uint32_t *inc_t;          // [max(LA,MC)][C]
@@ -717,8 +718,9 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base,
         w.bit_start = (uint32_t *)take(((size_t)d.M + 1) * 4);
         w.bit_cursor = (uint32_t *)take((size_t)d.M * 4);
         w.bit_clauses = (uint32_t *)take((size_t)d.C * d.MB * 4);
-        w.alive_stride = narrow_alive_stride(d.C);
-        for (uint32_t *&list : w.alive) list = (uint32_t *)take(n_tiles * NARROW_STREAMS * w.alive_stride * 4);
+        // (per tile: `streams` lists of 1 + ceil(C / streams) words, whichever shape k_tile_layer_narrow takes)
+        w.alive_words = (size_t)d.C + 2 * NARROW_MAX_STREAMS;
+        for (uint32_t *&list : w.alive) list = (uint32_t *)take(n_tiles * w.alive_words * 4);
         w.bytes = off;
         return w;
     }
@@ -1170,13 +1172,13 @@ int launch_two_phase_wide(const TileLayerArgs &a, int n_tiles, int LA, bool stag
     }
 }
 
-// Four clauses per wave on narrow tiles (score_narrow.h).
-template <int SRC, bool LAST>
+// Several clauses per wave on narrow tiles (score_narrow.h).
+template <int SRC, bool LAST, int GROUP, int WPL>
 int launch_narrow_as(const TileLayerArgs &a, const NarrowArgs &x, int n_tiles, hipStream_t st) {
-    const size_t lds = narrow_lds_bytes(a.tg, a.K, narrow_rows_lds(SRC, a.M, x.hv, x.n_types));
+    const size_t lds = narrow_lds_bytes(a.tg, NarrowChoice{GROUP, WPL}, a.K, narrow_rows_lds(SRC, a.M, x.hv, x.n_types));
     static thread_local size_t lds_set = 48 * 1024;
     if (lds > lds_set) {
-        hipError_t e = hipFuncSetAttribute((const void *)k_tile_layer_narrow<SRC, LAST>,
+        hipError_t e = hipFuncSetAttribute((const void *)k_tile_layer_narrow<SRC, LAST, GROUP, WPL>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(GTM_ERR_HIP, "raising the LDS limit to %zu: %s", lds, hipGetErrorString(e));
         lds_set = lds;
@@ -1184,17 +1186,27 @@ int launch_narrow_as(const TileLayerArgs &a, const NarrowArgs &x, int n_tiles, h
     profile_start(SRC == ROWS_HALF ? (LAST ? "k_tile_layer_narrow<score>" : "k_tile_layer_narrow<layer0>")
                                    : (LAST ? "k_tile_layer_narrow<messages, score>" : "k_tile_layer_narrow<messages>"),
                   st);
-    hipLaunchKernelGGL((k_tile_layer_narrow<SRC, LAST>), dim3(n_tiles), dim3(NARROW_WAVES * 64), lds, st, a, x);
+    hipLaunchKernelGGL((k_tile_layer_narrow<SRC, LAST, GROUP, WPL>), dim3(n_tiles), dim3(NARROW_WAVES * 64), lds, st, a, x);
     if (int rc = check_launch("tile_layer_narrow")) return rc;
     profile_stop(st);
     return GTM_OK;
 }
 
-int launch_narrow(const TileLayerArgs &a, const NarrowArgs &x, int n_tiles, int src, bool last, hipStream_t st) {
+template <int GROUP, int WPL>
+int launch_narrow_shape(const TileLayerArgs &a, const NarrowArgs &x, int n_tiles, int src, bool last, hipStream_t st) {
     if (src == ROWS_HALF)
-        return last ? launch_narrow_as<ROWS_HALF, true>(a, x, n_tiles, st) : launch_narrow_as<ROWS_HALF, false>(a, x, n_tiles, st);
-    return last ? launch_narrow_as<ROWS_MESSAGES, true>(a, x, n_tiles, st)
-                : launch_narrow_as<ROWS_MESSAGES, false>(a, x, n_tiles, st);
+        return last ? launch_narrow_as<ROWS_HALF, true, GROUP, WPL>(a, x, n_tiles, st)
+                    : launch_narrow_as<ROWS_HALF, false, GROUP, WPL>(a, x, n_tiles, st);
+    return last ? launch_narrow_as<ROWS_MESSAGES, true, GROUP, WPL>(a, x, n_tiles, st)
+                : launch_narrow_as<ROWS_MESSAGES, false, GROUP, WPL>(a, x, n_tiles, st);
+}
+
+int launch_narrow(const TileLayerArgs &a, const NarrowArgs &x, const NarrowChoice &shape, int n_tiles, int src, bool last,
+                  hipStream_t st) {
+    if (shape.group == 8 && shape.wpl == 4) return launch_narrow_shape<8, 4>(a, x, n_tiles, src, last, st);
+    if (shape.group == 16 && shape.wpl == 4) return launch_narrow_shape<16, 4>(a, x, n_tiles, src, last, st);
+    if (shape.group == 16 && shape.wpl == 2) return launch_narrow_shape<16, 2>(a, x, n_tiles, src, last, st);
+    return fail(GTM_ERR_INVALID, "no narrow-tile kernel for %d lanes per clause and %d words per lane", shape.group, shape.wpl);
 }
 
 // Layer 0 can run in two phases (k_tile_two_phase) on tiles of whole-word graph slots staged in
@@ -1230,10 +1242,16 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     // fit in LDS, will do.  GTM_NO_NARROW_LAYERS / GTM_NO_HALF_ROWS (tuning and test aids) turn them off.
     const size_t lds_limit = 160 * 1024;
     const int hv = cfg->literals / 2;
-    const bool narrow_tiles = narrow_geometry(tg) && !tune(T_NO_NARROW_LAYERS);
-    const bool narrow_messages = narrow_tiles && layers > 1 && narrow_lds_bytes(tg, d.K, tile_message_rows(d.M)) <= lds_limit;
-    const bool half_rows0 = narrow_tiles && !tg.half && (g->flags & GTM_GRAPHS_COMPLEMENTARY) && cfg->literals % 2 == 0 &&
-                            narrow_lds_bytes(tg, d.K, hv + g->number_of_node_types + 1) <= lds_limit &&
+    // (GTM_NARROW_READS=128, tuning and test aid: rows of at most 32 words on 128-bit reads, eight clauses per wave)
+    const char *narrow_reads = tune(T_NARROW_READS);
+    const NarrowChoice shape = narrow_choice(tg, narrow_reads && atoi(narrow_reads) == 128);
+    const bool narrow_tiles = shape.group != 0 && !tune(T_NO_NARROW_LAYERS);
+    const bool narrow_messages =
+        narrow_tiles && layers > 1 && narrow_lds_bytes(tg, shape, d.K, tile_message_rows(d.M)) <= lds_limit;
+    // (layer 0 of a model without message layers keeps the two-phase kernels on rows of more than 32 words)
+    const bool half_rows0 = narrow_tiles && !tg.half && (layers > 1 || tg.tw <= 32) &&
+                            (g->flags & GTM_GRAPHS_COMPLEMENTARY) && cfg->literals % 2 == 0 &&
+                            narrow_lds_bytes(tg, shape, d.K, hv + g->number_of_node_types + 1) <= lds_limit &&
                             !tune(T_NO_HALF_ROWS);
     // compiled clause: 8 words of packed 16-bit row entries (16 words of byte offsets on half tiles) + the include words
     const int stride0 = half_rows0 ? w.list_stride : tg.half ? 16 + d.LA : two_phase ? 8 + d.LA : w.list_stride;
@@ -1292,7 +1310,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     a.walk_factor = 2;
     if (const char *e = tune(T_WIDE_WALK_FACTOR)) a.walk_factor = std::max(1, atoi(e));  // (tuning aid)
     NarrowArgs px{};
-    px.alive_stride = w.alive_stride;
+    px.alive_stride = narrow_tiles ? narrow_alive_stride(d.C, shape.streams()) : 0;
     px.hv = hv;
     px.n_types = g->number_of_node_types;
     const uint32_t *alive_now = nullptr;  // what the last layer on narrow tiles left for the next one
@@ -1303,7 +1321,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             px.alive_in = nullptr;
             px.alive_out = !last && narrow_messages ? w.alive[0] : nullptr;
             alive_now = px.alive_out;
-            return launch_narrow(a, px, n_tiles, ROWS_HALF, last, st);
+            return launch_narrow(a, px, shape, n_tiles, ROWS_HALF, last, st);
         }
         alive_now = nullptr;
         if (tg.half) return launch_two_phase_half(a, n_tiles, d.LA / 4, last, &plan, st);
@@ -1386,7 +1404,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         px.alive_in = alive_now;
         px.alive_out = last || l == layers - 1 ? nullptr : w.alive[alive_now == w.alive[0] ? 1 : 0];
         alive_now = px.alive_out;
-        return launch_narrow(a, px, n_tiles, ROWS_MESSAGES, last, st);
+        return launch_narrow(a, px, shape, n_tiles, ROWS_MESSAGES, last, st);
     };
     for (int t0 = tile_first; t0 <= tile_last; t0 += tiles_per_launch) {
         const int n_tiles = tile_last - t0 + 1 < tiles_per_launch ? tile_last - t0 + 1 : tiles_per_launch;
@@ -1402,7 +1420,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                 profile_start("k_tile_messages_in_lds", st);
                 hipLaunchKernelGGL(k_tile_messages_in_lds, dim3(n_tiles), dim3(TILE_MESSAGES_LDS_BLOCK), in_lds.lds_bytes, st,
                                    w.tile_bitmap, d.C, tg, t0, g->number_of_graphs, d.M, s->hypervectors, d.MB, alive_now,
-                                   w.alive_stride, g->node_index, g->number_of_graph_nodes, g->number_of_graph_node_edges,
+                                   narrow_tiles ? shape.streams() : TILE_MESSAGES_LDS_BLOCK / 16, px.alive_stride, g->node_index, g->number_of_graph_nodes, g->number_of_graph_node_edges,
                                    g->edge_index, g->edge, g->total_edges > 0 ? 1 : 0, in_lds.main_words, in_lds.range_words,
                                    w.message_rows);
                 if (int rc = check_launch("tile_messages_in_lds")) return rc;

@@ -6,8 +6,7 @@
 // the clauses true at it, and what a neighbour receives along an edge of type t is that vector
 // rotated by t.  Four steps on one region of LDS:
 //   1. rows[p] |= truth row of every clause whose hypervector holds bit p: M rows of tw words,
-//      LDS atomics.  Each truth row is read ONCE (a quarter-wave per clause, 8 bytes per lane,
-//      the way k_tile_layer_narrow wrote it), and only the rows of the clauses that the
+//      LDS atomics.  Each truth row is read ONCE (a quarter-wave per clause, 8 bytes per lane), and only the rows of the clauses that the
 //      evaluation listed as true somewhere in the tile when such lists are handed in;
 //   2. the M x (32 tw) bit matrix is turned node-major in place - every half-wave takes 32 x 32
 //      bit blocks through registers (a transposition across its lanes), all blocks are read
@@ -25,7 +24,6 @@
 #include <type_traits>
 
 constexpr int TILE_MESSAGES_LDS_BLOCK = 1024;
-static_assert(TILE_MESSAGES_LDS_BLOCK / 16 == NARROW_STREAMS, "a quarter-wave per stream of k_tile_layer_narrow");
 
 // The word of lane `from` (0 .. 15) of this lane's row of 16 lanes: a lane move on the vector unit.  (`from` is
 // a constant wherever this is called - an unrolled loop's counter - and the switch folds away.)
@@ -69,7 +67,7 @@ inline TileMessagesPlan tile_messages_lds_plan(const TileGeom &g, int M, size_t 
 
 __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_lds(
     const uint32_t *__restrict__ bitmap, int C, TileGeom tg, int tile0, int G, int M, const uint32_t *__restrict__ hv, int MB,
-    const uint32_t *__restrict__ alive, int alive_stride, const uint32_t *__restrict__ node_index,
+    const uint32_t *__restrict__ alive, int streams, int alive_stride, const uint32_t *__restrict__ node_index,
     const uint32_t *__restrict__ n_nodes, const uint32_t *__restrict__ n_edges, const uint32_t *__restrict__ edge_index,
     const uint32_t *__restrict__ edge, int has_edges, int main_words, int range_words, uint32_t *__restrict__ rows) {
     extern __shared__ uint32_t lds[];
@@ -89,17 +87,19 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
     // number and bits then reach the 16 lanes by a lane move (row_share), and eight truth rows are on their way
     // per quarter-wave.
     {
-        const int group = lane >> 4, gl = lane & 15, q = wave * 4 + group;
+        const int group = lane >> 4, gl = lane & 15;
         const uint32_t *truth = bitmap + (int64_t)tile_local * C * tw;
-        const uint32_t *list = alive ? alive + ((int64_t)tile_local * NARROW_STREAMS + q) * alive_stride : nullptr;
-        const int n_mine = list ? (int)list[0] : (q < C ? (C - q + NARROW_STREAMS - 1) / NARROW_STREAMS : 0);
         const bool has_words = 2 * gl < tw;
+        // a quarter-wave takes the streams q, q + 64, ... of the evaluation that wrote the truth rows
+        for (int q = wave * 4 + group; q < streams; q += TILE_MESSAGES_LDS_BLOCK / 16) {
+        const uint32_t *list = alive ? alive + ((int64_t)tile_local * streams + q) * alive_stride : nullptr;
+        const int n_mine = list ? (int)list[0] : (q < C ? (C - q + streams - 1) / streams : 0);
         uint32_t id_next = 0u, bit0_next = 0u, bit1_next = 0u;
         // (every load below is unconditional, from an address that exists, and what it brought is dropped
         // afterwards where it was not wanted: loads under a condition would wait for one another)
         auto fetch = [&](int i) {
             const int at = i < n_mine ? i : n_mine - 1;
-            id_next = list ? list[1 + at] : (uint32_t)(q + NARROW_STREAMS * at);
+            id_next = list ? list[1 + at] : (uint32_t)(q + streams * at);
             bit0_next = hv[(int64_t)id_next * MB];
             bit1_next = hv[(int64_t)id_next * MB + (MB > 1 ? 1 : 0)];
         };
@@ -132,6 +132,7 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
             };
             eight(std::integral_constant<int, 0>{});
             if (n_here > 8) eight(std::integral_constant<int, 8>{});
+        }
         }
     }
     __syncthreads();

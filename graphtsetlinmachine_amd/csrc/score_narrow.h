@@ -1,12 +1,14 @@
-// Clause evaluation on NARROW tiles, four clauses per wave.
+// Clause evaluation on NARROW tiles, several clauses per wave.
 //
-// When a tile's rows are at most 32 words wide (graphs of 500 to 1,000 nodes whose thousand message
-// rows have to share a workgroup's LDS: one graph per tile), a wave that walks one clause's rows at
-// a word per lane has half its lanes idle - and reads LDS at half its rate, which 32-bit reads
-// cannot exceed.  Here each QUARTER of a wave walks a clause of its own, two words per lane: lanes
-// 16 g .. 16 g + 15 hold words 2 l, 2 l + 1 of the truth row of the clause of group g.  Every row
-// read (64 bits per lane: the LDS at full rate), address add and AND serves four clauses, and the
-// waves of a workgroup are 64 independent clause streams.
+// When a tile's rows are at most 64 words wide (graphs of 500 to 1,000 nodes whose thousand message
+// rows have to share a workgroup's LDS: one or two graphs per tile), a wave that walks one clause's
+// rows at a word per lane leaves lanes idle and reads LDS 256 bytes at a time, and a CU takes an
+// LDS instruction only every four clocks or so whatever its width.  Here a GROUP of 8 or 16 lanes
+// walks a clause of its own, WPL = 2 or 4 words per lane: lane l of a group holds words WPL l ..
+// WPL l + WPL - 1 of the truth row of the group's clause.  Every row read (64 or 128 bits per
+// lane), address add and AND serves 64 / GROUP clauses, and the waves of a workgroup are 64 or 128
+// independent clause streams.  Shapes: (GROUP 16, WPL 2) for rows of at most 32 words, (16, 4) for
+// rows of at most 64; (8, 4) - rows of at most 32 words on 128-bit reads - is kept for comparison.
 //
 // The same kernel evaluates
 //   * a message layer (ROWS_MESSAGES; kernels.py:505-527): previous truth AND the rows of the
@@ -21,58 +23,79 @@
 //
 // A clause's compiled list (k_compile_clauses with `half` set: header, rows to AND, rows whose
 // complements to AND, each part a whole number of 8-entry blocks, filled up with the all-ones row
-// to a whole number of windows) is brought in by the quarter-wave that evaluates it, a window of
-// 64 entries at a time - one 16-byte load per lane, the first two windows requested two clauses ahead - and passes
-// through 96 words of LDS of the quarter-wave's own, from which the walk reads it back a block
-// ahead of the rows (the four lanes of a quad read entries 0..3 and 4..7 of a block, and an entry
-// reaches all lanes inside the add that forms the row's address).  Two blocks per trip, 16 row
-// reads in flight per lane, one test per trip for "false at every node slot of the tile" - per
-// group: a wave goes on while any of its clauses is alive and has rows left.  What differs between
-// the groups in a trip - a block of rows to AND against a block of complements, a list that has
-// ended - is a per-lane XOR mask folded into the AND (one three-input operation per pair of rows)
-// and windows past a list's end replaced by the all-ones row.
+// to a whole number of 128 entries) is brought in by the group that evaluates it, a window of
+// 4 GROUP entries at a time - one 16-byte load per lane, the first 96 or 128 entries requested two
+// clauses ahead - and passes through a few words of LDS of the group's own, from which the walk
+// reads it back a block ahead of the rows (the four lanes of a quad read entries 0..3 and 4..7 of
+// a block, and an entry reaches all lanes inside the add that forms the row's address).  16 row
+// words in flight per lane and trip (two blocks at 2 words per lane, one at 4), one test per trip
+// for "false at every node slot of the tile" - per group: a wave goes on while any of its clauses
+// is alive and has rows left.  What differs between the groups in a trip - a block of rows to AND
+// against a block of complements, a list that has ended - is a per-lane XOR mask folded into the
+// AND (one three-input operation per pair of rows) and windows past a list's end replaced by the
+// all-ones row.
 //
 // Between layers a stream also hands on WHICH of its clauses are still true somewhere in the tile
 // (`alive`: per tile and stream a count and the clause numbers, written without atomics because a
 // stream owns its clauses in every layer).  The next layer walks that list instead of testing the
 // truth rows of all clauses - after the first message layer most are false everywhere.  The truth
-// rows themselves stay complete: a clause that dies gets its row of zeros, because the kernels
-// that build the messages read every clause's row.
+// rows themselves stay complete: a clause that dies gets its row of zeros.
 #pragma once
 
 constexpr int ROWS_HALF = 3;  // layer 0 on the positive literals' rows (+ node types, all ones), staged in LDS
 
 constexpr int NARROW_WAVES = 16;
-constexpr int NARROW_GROUP = 16;                       // lanes that share a clause
-constexpr int NARROW_PER_WAVE = 64 / NARROW_GROUP;     // clauses under way in a wave
-constexpr int NARROW_STREAMS = NARROW_PER_WAVE * NARROW_WAVES;
-constexpr int NARROW_WINDOW = 4 * NARROW_GROUP;        // list entries of a clause in LDS at a time: 4 per lane of its group
-constexpr int NARROW_LIST_WORDS = NARROW_WINDOW + 32;  // + what the walk reads ahead of the rows it is at
-constexpr int NARROW_AHEAD = 2;                        // clauses of a stream whose list and truth words are on their way
-constexpr int NARROW_MAX_WORDS = 2 * NARROW_GROUP;     // widest row
+constexpr int NARROW_AHEAD = 2;         // clauses of a stream whose list and truth words are on their way
+constexpr int NARROW_LIST_AHEAD = 128;  // entries of a clause's list requested with it (a list is at least as long)
+constexpr int NARROW_MAX_STREAMS = 128;
+
+// What depends on the lanes that share a clause.
+template <int GROUP>
+struct NarrowShape {
+    static_assert(GROUP == 8 || GROUP == 16, "a half or a whole row of 16 lanes");
+    static constexpr int PER_WAVE = 64 / GROUP;               // clauses under way in a wave
+    static constexpr int STREAMS = PER_WAVE * NARROW_WAVES;   // clause streams of a workgroup
+    static constexpr int WINDOW = 4 * GROUP;                  // list entries of a clause in LDS at a time: 4 per lane
+    static constexpr int LIST_WORDS = WINDOW + 32;            // + what the walk reads ahead of the rows it is at
+    // windows requested with the clause (of the 128 entries that every list has at least): 96 or 128 entries
+    static constexpr int WINDOWS_AHEAD = NARROW_LIST_AHEAD / WINDOW > 3 ? 3 : NARROW_LIST_AHEAD / WINDOW;
+};
 
 struct NarrowArgs {
-    const uint32_t *alive_in;  // [tiles of the launch][NARROW_STREAMS][alive_stride]: word 0 = n, then the stream's clauses
-                               // that are true somewhere in the tile; NULL: every clause (q, q + 64, ...) is looked at
+    const uint32_t *alive_in;  // [tiles of the launch][streams][alive_stride]: word 0 = n, then the stream's clauses
+                               // that are true somewhere in the tile; NULL: every clause (q, q + streams, ...) is looked at
     uint32_t *alive_out;       // the same for the next layer, or NULL
-    int alive_stride;          // >= 1 + ceil(C / NARROW_STREAMS)
+    int alive_stride;          // >= 1 + ceil(C / streams)
     int hv, n_types;           // ROWS_HALF: positive literals (= LDS rows before the node-type rows), node types
 };
 
-inline int narrow_alive_stride(int C) { return 1 + (C + NARROW_STREAMS - 1) / NARROW_STREAMS; }
+// The shape for a tile geometry: lanes per clause and words per lane (0, 0: none).  Rows of at most 32 words take
+// 64-bit reads, four clauses per wave: with 128-bit reads a wave instruction covers eight rows at unrelated
+// offsets, their bank conflicts cost more than the wider reads save (measured on 28-word rows: 5.7 against 4.7 ms),
+// and 128 streams double the per-clause work around the walk.  `wide_reads` asks for that shape all the same
+// (GTM_NARROW_READS=128, tuning and test aid).
+struct NarrowChoice {
+    int group, wpl;
+    int streams() const { return group ? 64 / group * NARROW_WAVES : 0; }
+    int list_words() const { return 4 * group + 32; }
+};
+
+inline NarrowChoice narrow_choice(const TileGeom &g, bool wide_reads = false) {
+    // whole-word slots, rows a multiple of 4 words, built at one word per lane
+    if (!g.ok || g.slot_words <= 0 || g.lw != 1 || g.tw % 4 != 0) return NarrowChoice{0, 0};
+    if (g.tw <= 32) return wide_reads ? NarrowChoice{8, 4} : NarrowChoice{16, 2};
+    if (g.tw <= 64) return NarrowChoice{16, 4};
+    return NarrowChoice{0, 0};
+}
+
+inline int narrow_alive_stride(int C, int streams) { return 1 + (C + streams - 1) / streams; }
 
 inline int narrow_rows_lds(int src, int M, int hv, int n_types) { return src == ROWS_HALF ? hv + n_types + 1 : M + 2; }
 
-inline size_t narrow_lds_bytes(const TileGeom &g, int classes, int rows_lds) {
+inline size_t narrow_lds_bytes(const TileGeom &g, const NarrowChoice &shape, int classes, int rows_lds) {
     const size_t sums = ((size_t)g.gpt * classes + 3) & ~(size_t)3;  // the lists after them stay 16-byte aligned
-    return ((size_t)rows_lds * g.tw + TILE_LDS_PAD_WORDS + sums + (size_t)NARROW_STREAMS * NARROW_LIST_WORDS) * 4;
+    return ((size_t)rows_lds * g.tw + TILE_LDS_PAD_WORDS + sums + (size_t)shape.streams() * shape.list_words()) * 4;
 }
-
-// Geometry the kernel takes: whole-word slots, rows of at most 32 words (a multiple of 4), built at one word per lane.
-inline bool narrow_geometry(const TileGeom &g) { return g.ok && g.slot_words > 0 && g.lw == 1 && g.tw <= NARROW_MAX_WORDS; }
-
-typedef uint32_t NarrowWords __attribute__((ext_vector_type(2)));  // the two words of a row that a lane holds
-typedef __attribute__((address_space(3))) const NarrowWords *NarrowLdsWords;
 
 // The LDS addresses of a block's 8 rows for this lane: adr[i] = base + entry i of the block, where the
 // four lanes of every quad hold entries 0..3 in `lo` and 4..7 in `hi`.  The entry comes across the quad
@@ -105,9 +128,36 @@ __device__ __forceinline__ uint32_t narrow_and3(uint32_t a, uint32_t b, uint32_t
     return (uint32_t)__builtin_amdgcn_bitop3_b32((int)a, (int)b, (int)c, 0x80);
 }
 
-template <int SRC, bool LAST>
+// The WPL words of a row that a lane holds (a native vector: the values stay in registers through copies and selects).
+template <int WPL>
+struct NarrowRow {
+    typedef uint32_t Vec __attribute__((ext_vector_type(WPL)));
+    Vec w;
+    __device__ __forceinline__ bool any() const {
+        uint32_t m = w[0];
+#pragma unroll
+        for (int u = 1; u < WPL; ++u) m |= w[u];
+        return m != 0u;
+    }
+    __device__ __forceinline__ void fill(uint32_t v) { w = Vec(v); }
+    __device__ __forceinline__ void load_lds(uint32_t address) {
+        w = *(__attribute__((address_space(3))) const Vec *)(uintptr_t)address;
+    }
+    __device__ __forceinline__ void load(const uint32_t *p) { w = *reinterpret_cast<const Vec *>(p); }
+    __device__ __forceinline__ void store(uint32_t *p) const { *reinterpret_cast<Vec *>(p) = w; }
+};
+
+typedef uint32_t NarrowEntries __attribute__((ext_vector_type(4)));  // four entries of a compiled list
+
+template <int SRC, bool LAST, int GROUP, int WPL>
 __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLayerArgs a, NarrowArgs x) {
     static_assert(SRC == ROWS_HALF || SRC == ROWS_MESSAGES, "layer 0 on half rows, or a message layer");
+    static_assert(WPL == 2 || WPL == 4, "64- or 128-bit row reads");
+    using Shape = NarrowShape<GROUP>;
+    using Row = NarrowRow<WPL>;
+    constexpr int PER = Shape::PER_WAVE, STREAMS = Shape::STREAMS, WINDOW = Shape::WINDOW, AHEAD_W = Shape::WINDOWS_AHEAD;
+    constexpr int TRIP = 4 / WPL;  // blocks of 8 rows per trip: 16 row words in flight per lane
+    constexpr uint32_t GROUP_MASK = (1u << GROUP) - 1u;
     extern __shared__ uint32_t lds[];
     const TileGeom &tg = a.tg;
     const int tw = tg.tw, C = a.C, K = a.K;
@@ -117,9 +167,9 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
     int32_t *sums = (int32_t *)(lds + (size_t)rows_lds * tw + TILE_LDS_PAD_WORDS);
     uint32_t *lists = (uint32_t *)sums + ((tg.gpt * K + 3) & ~3);
     const int tile_local = blockIdx.x, tile = a.tile0 + tile_local;
-    const int tid = threadIdx.x, lane = tid & 63, gl = lane & (NARROW_GROUP - 1), group = lane / NARROW_GROUP;
+    const int tid = threadIdx.x, lane = tid & 63, gl = lane & (GROUP - 1), group = lane / GROUP;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int q = NARROW_PER_WAVE * wave + group;  // this group's stream
+    const int q = PER * wave + group;  // this group's stream
     uint32_t *bitmap = a.bitmap + (int64_t)tile_local * C * tw;
 
     {  // rows -> LDS, 16 bytes per thread and trip, four loads in flight
@@ -153,61 +203,68 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
     __syncthreads();
 
     // Lanes past the row width keep a running AND of zero; they read the words after the row.
-    const bool active = 2 * gl < tw;
-    const uint32_t col_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t *)(bt + 2 * gl);
-    uint32_t *my_list = lists + q * NARROW_LIST_WORDS;
+    const bool active = WPL * gl < tw;
+    const uint32_t col_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t *)(bt + WPL * gl);
+    uint32_t *my_list = lists + q * Shape::LIST_WORDS;
     const uint32_t *quad_entry = my_list + (lane & 3);
     const uint32_t ones_entry = (uint32_t)(rows_lds - 1 - (SRC == ROWS_MESSAGES ? 1 : 0)) * (uint32_t)tw * 4u;
-    const int shift16 = group * NARROW_GROUP;  // this group's lanes in a 64-bit vote
+    // this group's lanes in a 64-bit vote: bits shift .. shift + GROUP - 1 of its low or high half
+    const bool upper_half = lane >= 32;
+    const uint32_t shift = (uint32_t)(group * GROUP) & 31u;
+    auto votes_of_group = [&](unsigned long long vote) {
+        const uint32_t half = upper_half ? (uint32_t)(vote >> 32) : (uint32_t)vote;
+        return (half >> shift) & GROUP_MASK;
+    };
 
     // slot bit 0 of the graphs without nodes (message layers): such a graph keeps every clause true
-    uint2 empties = make_uint2(0u, 0u);
+    Row empties;
+    empties.fill(0u);
     bool any_empty = false;
     if (SRC == ROWS_MESSAGES) {
-        if (active) empties = *reinterpret_cast<const uint2 *>(bt + (size_t)(a.M + 1) * tw + 2 * gl);
-        any_empty = __ballot((empties.x | empties.y) != 0u) != 0ull;
+        if (active) empties.load(bt + (size_t)(a.M + 1) * tw + WPL * gl);
+        any_empty = __ballot(empties.any()) != 0ull;
     }
 
     // this stream's clauses
-    const uint32_t *seg_in = x.alive_in ? x.alive_in + ((int64_t)tile_local * NARROW_STREAMS + q) * x.alive_stride : nullptr;
-    const int n_mine = seg_in ? (int)seg_in[0] : (q < C ? (C - q + NARROW_STREAMS - 1) / NARROW_STREAMS : 0);
+    const uint32_t *seg_in = x.alive_in ? x.alive_in + ((int64_t)tile_local * STREAMS + q) * x.alive_stride : nullptr;
+    const int n_mine = seg_in ? (int)seg_in[0] : (q < C ? (C - q + STREAMS - 1) / STREAMS : 0);
     int n_most = 0;
 #pragma unroll
-    for (int g = 0; g < NARROW_PER_WAVE; ++g) n_most = max(n_most, __builtin_amdgcn_readlane(n_mine, g * NARROW_GROUP));
-    uint32_t *seg_out = x.alive_out ? x.alive_out + ((int64_t)tile_local * NARROW_STREAMS + q) * x.alive_stride : nullptr;
+    for (int g = 0; g < PER; ++g) n_most = max(n_most, __builtin_amdgcn_readlane(n_mine, g * GROUP));
+    uint32_t *seg_out = x.alive_out ? x.alive_out + ((int64_t)tile_local * STREAMS + q) * x.alive_stride : nullptr;
     int n_out = 0;
 
     const int pairs = tg.gpt * K, sw = tg.slot_words;
 
-    // The clause of item i of this stream (-1 past its end).  With a list of the clauses still alive, 16 items
+    // The clause of item i of this stream (-1 past its end).  With a list of the clauses still alive, GROUP items
     // are held one per lane of the group and handed out with a lane read.
     uint32_t seg_now = 0u, seg_next = 0u;
     if (seg_in) {
         seg_now = gl < n_mine ? seg_in[1 + gl] : 0u;
-        seg_next = NARROW_GROUP + gl < n_mine ? seg_in[1 + NARROW_GROUP + gl] : 0u;
+        seg_next = GROUP + gl < n_mine ? seg_in[1 + GROUP + gl] : 0u;
     }
     auto clause_of = [&](int i) {
         if (i >= n_mine) return -1;
-        if (!seg_in) return q + NARROW_STREAMS * i;
-        return (int)__shfl(seg_now, shift16 | (i & (NARROW_GROUP - 1)));
+        if (!seg_in) return q + STREAMS * i;
+        return (int)__shfl(seg_now, (lane & ~(GROUP - 1)) | (i & (GROUP - 1)));
     };
     struct Item {
-        int c;        // the clause, -1: none
-        uint4 e, e2;  // entries 4 gl .. 4 gl + 3 of the first and of the second window of its list
-        uint2 truth;  // words 2 gl, 2 gl + 1 of its truth row (message layers)
+        int c;              // the clause, -1: none
+        NarrowEntries e[AHEAD_W];  // entries 4 gl .. 4 gl + 3 of the first windows of its list
+        Row truth;          // its words of the clause's truth row (message layers)
     };
     auto fetch = [&](int i, Item &it) {  // item i's loads; i runs up by one from call to call
-        if (seg_in && i > 0 && (i & (NARROW_GROUP - 1)) == 0) {  // the next 16 clauses of the stream's list move up
+        if (seg_in && i > 0 && (i & (GROUP - 1)) == 0) {  // the next GROUP clauses of the stream's list move up
             seg_now = seg_next;
-            seg_next = i + NARROW_GROUP + gl < n_mine ? seg_in[1 + i + NARROW_GROUP + gl] : 0u;
+            seg_next = i + GROUP + gl < n_mine ? seg_in[1 + i + GROUP + gl] : 0u;
         }
         it.c = clause_of(i);
         const int c = it.c < 0 ? 0 : it.c;
-        const uint4 *list = reinterpret_cast<const uint4 *>(a.lists + (int64_t)c * a.stride + 4 * gl);
-        it.e = list[0];
-        it.e2 = list[NARROW_WINDOW / 4];  // (a list is at least two windows long, filled up with the all-ones row)
-        it.truth = make_uint2(0u, 0u);
-        if (SRC == ROWS_MESSAGES) it.truth = *reinterpret_cast<const uint2 *>(bitmap + (int64_t)c * tw + (active ? 2 * gl : 0));
+        const NarrowEntries *list = reinterpret_cast<const NarrowEntries *>(a.lists + (int64_t)c * a.stride + 4 * gl);
+#pragma unroll
+        for (int v = 0; v < AHEAD_W; ++v) it.e[v] = list[v * (WINDOW / 4)];  // (a list is at least 128 entries long)
+        it.truth.fill(0u);
+        if (SRC == ROWS_MESSAGES) it.truth.load(bitmap + (int64_t)c * tw + (active ? WPL * gl : 0));
     };
 
     // NARROW_AHEAD items are under way per stream: a clause's list and truth words come from L2 or further, a few
@@ -225,113 +282,121 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
 
             const bool has = now.c >= 0;
             const int c = has ? now.c : 0;
-            uint2 truth_in = make_uint2(0u, 0u);
+            Row truth_in, acc;
+            truth_in.fill(0u);
             if (SRC == ROWS_MESSAGES && active && has) truth_in = now.truth;
-            uint2 acc = SRC == ROWS_MESSAGES ? truth_in : (active && has ? make_uint2(0xFFFFFFFFu, 0xFFFFFFFFu) : make_uint2(0u, 0u));
+            if (SRC == ROWS_MESSAGES)
+                acc = truth_in;
+            else
+                acc.fill(active && has ? 0xFFFFFFFFu : 0u);
             // header (entry 0, in lane 0 of each group): blocks of rows to AND | blocks of rows whose complements to AND << 16
             uint32_t header = 0u;
 #pragma unroll
-            for (int g = 0; g < NARROW_PER_WAVE; ++g) {
-                const uint32_t h = __builtin_amdgcn_readlane(now.e.x, g * NARROW_GROUP);
+            for (int g = 0; g < PER; ++g) {
+                const uint32_t h = __builtin_amdgcn_readlane(now.e[0].x, g * GROUP);
                 header = group == g ? h : header;
             }
             int plain = (int)(header & 0xFFFFu), nb = plain + (int)(header >> 16);
-            unsigned long long nzw = __ballot((acc.x | acc.y) != 0u);
-            const bool arrived_alive = ((nzw >> shift16) & 0xFFFFull) != 0ull;
+            unsigned long long nzw = __ballot(acc.any());
+            const bool arrived_alive = votes_of_group(nzw) != 0u;
             if (!has || !arrived_alive) nb = 0, plain = 0;
-            int nb_of[NARROW_PER_WAVE], nb_most = 0;
+            int nb_most = 0;
 #pragma unroll
-            for (int g = 0; g < NARROW_PER_WAVE; ++g) {
-                nb_of[g] = __builtin_amdgcn_readlane(nb, g * NARROW_GROUP);
-                nb_most = max(nb_most, nb_of[g]);
-            }
+            for (int g = 0; g < PER; ++g) nb_most = max(nb_most, __builtin_amdgcn_readlane(nb, g * GROUP));
             // does some group have a live clause with blocks left from block b on?
-            auto work_left = [&](int b) {
-                bool left = false;
-#pragma unroll
-                for (int g = 0; g < NARROW_PER_WAVE; ++g) left |= b < nb_of[g] && ((nzw >> (g * NARROW_GROUP)) & 0xFFFFull) != 0ull;
-                return left;
-            };
+            auto work_left = [&](int b) { return __ballot(b < nb && votes_of_group(nzw) != 0u) != 0ull; };
 
-            uint4 e = now.e;
-            for (int b0 = 0; b0 < nb_most; b0 += NARROW_WINDOW / 8) {  // one window of the lists after the other
+            for (int b0 = 0; b0 < nb_most; b0 += WINDOW / 8) {  // one window of the lists after the other
                 if (!work_left(b0)) break;
-                if (b0 == NARROW_WINDOW / 8)
-                    e = now.e2;
-                else if (b0 > 0)  // (a clause of more than 126 literals: its further windows are fetched when it gets there)
-                    e = *reinterpret_cast<const uint4 *>(a.lists + (int64_t)c * a.stride + b0 * 8 + 4 * gl);
-                // The compiled list is filled up with the all-ones row to the end of its last window.  A group whose
-                // list has no such window (it ended in an earlier one; no clause; a clause false everywhere on arrival:
-                // nb = 0) walks the all-ones row while the others go on.
-                const bool past = b0 * 8 >= ((nb * 8 + NARROW_WINDOW - 1) & ~(NARROW_WINDOW - 1));
-                if (past) e = make_uint4(ones_entry, ones_entry, ones_entry, ones_entry);
+                NarrowEntries e;
+                const int window = b0 / (WINDOW / 8);
+                if (window < AHEAD_W) {
+                    e = now.e[0];
+#pragma unroll
+                    for (int v = 1; v < AHEAD_W; ++v) e = window == v ? now.e[v] : e;
+                } else {  // (a clause of more literals than that: its further windows are fetched when it gets there)
+                    e = *reinterpret_cast<const NarrowEntries *>(a.lists + (int64_t)c * a.stride + b0 * 8 + 4 * gl);
+                }
+                // The compiled list is filled up with the all-ones row to a whole number of 128 entries.  A group
+                // whose list has no such window (it ended in an earlier one; no clause; a clause false everywhere on
+                // arrival: nb = 0) walks the all-ones row while the others go on.
+                const bool past = b0 * 8 >= ((nb * 8 + NARROW_LIST_AHEAD - 1) & ~(NARROW_LIST_AHEAD - 1));
+                if (past) e = NarrowEntries(ones_entry);
                 if (b0 == 0 && gl == 0) e.x = ones_entry;  // in the place of the header
-                *reinterpret_cast<uint4 *>(my_list + 4 * gl) = e;
+                *reinterpret_cast<NarrowEntries *>(my_list + 4 * gl) = e;
                 // (a wave's LDS accesses are carried out in order: the reads below see the entries just written)
-                const int lim_most = nb_most - b0 < NARROW_WINDOW / 8 ? nb_most - b0 : NARROW_WINDOW / 8;
+                const int lim_most = nb_most - b0 < WINDOW / 8 ? nb_most - b0 : WINDOW / 8;
                 // bit b: block b0 + b of this group's list is one of complements (blocks plain .. nb - 1): its rows come in inverted
-                const int from = plain - b0 < 0 ? 0 : plain - b0 > 8 ? 8 : plain - b0, to = nb - b0 < 0 ? 0 : nb - b0 > 8 ? 8 : nb - b0;
+                const int from = plain - b0 < 0 ? 0 : plain - b0 > WINDOW / 8 ? WINDOW / 8 : plain - b0;
+                const int to = nb - b0 < 0 ? 0 : nb - b0 > WINDOW / 8 ? WINDOW / 8 : nb - b0;
                 const int flip_bits = to > from ? ((1 << to) - 1) & ~((1 << from) - 1) : 0;
-                uint32_t lo0 = quad_entry[0], hi0 = quad_entry[4], lo1 = quad_entry[8], hi1 = quad_entry[12];
+                uint32_t lo[TRIP], hi[TRIP];
+#pragma unroll
+                for (int t = 0; t < TRIP; ++t) lo[t] = quad_entry[8 * t], hi[t] = quad_entry[8 * t + 4];
 #pragma unroll 2
-                for (int b = 0; b < lim_most && work_left(b0 + b); b += 2) {
-                    const uint32_t n_lo0 = quad_entry[8 * b + 16], n_hi0 = quad_entry[8 * b + 20];
-                    const uint32_t n_lo1 = quad_entry[8 * b + 24], n_hi1 = quad_entry[8 * b + 28];
-                    uint32_t adr0[8], adr1[8];
-                    narrow_block_addresses(lo0, hi0, col_lds, adr0);
-                    narrow_block_addresses(lo1, hi1, col_lds, adr1);
-                    NarrowWords r[16];
+                for (int b = 0; b < lim_most && work_left(b0 + b); b += TRIP) {
+                    uint32_t n_lo[TRIP], n_hi[TRIP];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) r[u] = *(NarrowLdsWords)(uintptr_t)adr0[u];
+                    for (int t = 0; t < TRIP; ++t)
+                        n_lo[t] = quad_entry[8 * (b + TRIP + t)], n_hi[t] = quad_entry[8 * (b + TRIP + t) + 4];
+                    uint32_t adr[TRIP][8];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) r[8 + u] = *(NarrowLdsWords)(uintptr_t)adr1[u];
-                    // all ones for a block of complements, else zero (a signed one-bit field of flip_bits)
-                    const uint32_t flip0 = (uint32_t)__builtin_amdgcn_sbfe(flip_bits, b, 1);
-                    const uint32_t flip1 = (uint32_t)__builtin_amdgcn_sbfe(flip_bits, b + 1, 1);
-                    uint32_t tx[8], ty[8];
+                    for (int t = 0; t < TRIP; ++t) narrow_block_addresses(lo[t], hi[t], col_lds, adr[t]);
+                    Row r[TRIP][8];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        tx[u] = narrow_pair(r[2 * u].x, r[2 * u + 1].x, flip0);
-                        ty[u] = narrow_pair(r[2 * u].y, r[2 * u + 1].y, flip0);
-                        tx[4 + u] = narrow_pair(r[8 + 2 * u].x, r[9 + 2 * u].x, flip1);
-                        ty[4 + u] = narrow_pair(r[8 + 2 * u].y, r[9 + 2 * u].y, flip1);
+                    for (int t = 0; t < TRIP; ++t)
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) r[t][u].load_lds(adr[t][u]);
+#pragma unroll
+                    for (int t = 0; t < TRIP; ++t) {
+                        // all ones for a block of complements, else zero (a signed one-bit field of flip_bits)
+                        const uint32_t flip = (uint32_t)__builtin_amdgcn_sbfe(flip_bits, b + t, 1);
+#pragma unroll
+                        for (int v = 0; v < WPL; ++v) {
+                            const uint32_t p0 = narrow_pair(r[t][0].w[v], r[t][1].w[v], flip);
+                            const uint32_t p1 = narrow_pair(r[t][2].w[v], r[t][3].w[v], flip);
+                            const uint32_t p2 = narrow_pair(r[t][4].w[v], r[t][5].w[v], flip);
+                            const uint32_t p3 = narrow_pair(r[t][6].w[v], r[t][7].w[v], flip);
+                            acc.w[v] = narrow_and3(narrow_and3(acc.w[v], p0, p1), p2, p3);
+                        }
                     }
+                    nzw = __ballot(acc.any());
 #pragma unroll
-                    for (int u = 0; u < 8; u += 2) {
-                        acc.x = narrow_and3(acc.x, tx[u], tx[u + 1]);
-                        acc.y = narrow_and3(acc.y, ty[u], ty[u + 1]);
-                    }
-                    nzw = __ballot((acc.x | acc.y) != 0u);
-                    lo0 = n_lo0, hi0 = n_hi0, lo1 = n_lo1, hi1 = n_hi1;
+                    for (int t = 0; t < TRIP; ++t) lo[t] = n_lo[t], hi[t] = n_hi[t];
                 }
             }
             if (SRC == ROWS_MESSAGES && any_empty) {
-                acc.x |= truth_in.x & empties.x, acc.y |= truth_in.y & empties.y;
-                nzw = __ballot((acc.x | acc.y) != 0u);
+#pragma unroll
+                for (int v = 0; v < WPL; ++v) acc.w[v] = acc.w[v] | (truth_in.w[v] & empties.w[v]);
+                nzw = __ballot(acc.any());
             }
-            const uint32_t nzg = (uint32_t)(nzw >> shift16) & 0xFFFFu;  // this group's lanes with a true node slot
+            const uint32_t nzg = votes_of_group(nzw);  // this group's lanes with a true node slot
             if (has) {
                 if (!LAST) {
                     // (a clause that was false everywhere on arrival has its row of zeros in place already)
-                    if (active && (SRC == ROWS_HALF || arrived_alive))
-                        *reinterpret_cast<uint2 *>(bitmap + (int64_t)c * tw + 2 * gl) = acc;
+                    if (active && (SRC == ROWS_HALF || arrived_alive)) acc.store(bitmap + (int64_t)c * tw + WPL * gl);
                     if (seg_out && nzg != 0u) {
                         if (gl == 0) seg_out[1 + n_out] = (uint32_t)c;
                         ++n_out;
                     }
                 } else if (nzg != 0u) {
                     // graph j of the tile owns words [j * sw, (j + 1) * sw) of the row; lane p of the group adds weight
-                    // k = p % K to graph j = p / K, for p = gl, gl + 16, ...: which words of the group are non-zero
-                    const uint32_t even = (uint32_t)(__ballot(acc.x != 0u) >> shift16) & 0xFFFFu;  // bit l: word 2 l
-                    const uint32_t odd = (uint32_t)(__ballot(acc.y != 0u) >> shift16) & 0xFFFFu;   // bit l: word 2 l + 1
+                    // k = p % K to graph j = p / K, for p = gl, gl + GROUP, ...: which words of the group are non-zero
+                    uint32_t nonzero[WPL];  // bit l: word WPL l + v
+#pragma unroll
+                    for (int v = 0; v < WPL; ++v) nonzero[v] = votes_of_group(__ballot(acc.w[v] != 0u));
                     const int32_t *weights_of_clause = a.wt + (int64_t)c * K;
-                    for (int p = gl; p < pairs; p += NARROW_GROUP) {
+                    for (int p = gl; p < pairs; p += GROUP) {
                         const int j = p / K, k = p - j * K;
                         const int w_lo = j * sw, w_hi = w_lo + sw;  // the graph's words
-                        // lanes whose even word lies in [w_lo, w_hi): ceil(w_lo / 2) .. ceil(w_hi / 2) - 1; odd word: w_lo / 2 .. w_hi / 2 - 1
-                        const uint32_t even_lanes = ((1u << ((w_hi + 1) >> 1)) - 1u) & ~((1u << ((w_lo + 1) >> 1)) - 1u);
-                        const uint32_t odd_lanes = ((1u << (w_hi >> 1)) - 1u) & ~((1u << (w_lo >> 1)) - 1u);
-                        if ((even & even_lanes) | (odd & odd_lanes)) atomicAdd(&sums[p], weights_of_clause[k]);
+                        uint32_t hit = 0u;
+#pragma unroll
+                        for (int v = 0; v < WPL; ++v) {
+                            // lanes whose word WPL l + v lies in [w_lo, w_hi): ceil((w_lo - v) / WPL) <= l < ceil((w_hi - v) / WPL)
+                            const int l_lo = (w_lo + WPL - 1 - v) / WPL, l_hi = (w_hi + WPL - 1 - v) / WPL;
+                            hit |= nonzero[v] & ((1u << l_hi) - 1u) & ~((1u << l_lo) - 1u);
+                        }
+                        if (hit) atomicAdd(&sums[p], weights_of_clause[k]);
                     }
                 }
             }

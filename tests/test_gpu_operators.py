@@ -994,15 +994,20 @@ NARROW_TILE_SHAPES = [
     dict(seed=63, g=dict(n_graphs=7, sizes=[300, 0, 1, 290, 0, 17, 64], hv_size=64, edge_types=("l",)), classes=4),
     dict(seed=64, g=dict(n_graphs=6, max_nodes=650, min_nodes=400, hv_size=352, n_symbols=9, node_types=("a", "b", "c"),
                          edge_types=("l", "r")), classes=3),
+    # rows of 33 to 64 words (messages of 512 bits, so that their rows fit beside them): one graph of up to 2,000
+    # nodes per tile; two graphs of 32 words per tile, one of them without nodes in one tile
+    dict(seed=65, g=dict(n_graphs=4, sizes=[1500, 1025, 2000, 33], hv_size=64, edge_types=("l", "r")), classes=3, M=512),
+    dict(seed=66, g=dict(n_graphs=6, sizes=[1000, 900, 0, 1000, 512, 1], hv_size=64, edge_types=("l", "r", "u")), classes=2,
+         M=512),
 ]
 
 
 @pytest.mark.parametrize("shape", NARROW_TILE_SHAPES, ids=lambda s: "narrow%d" % s["seed"])
 @pytest.mark.parametrize("depth", [1, 2, 3])
-@pytest.mark.parametrize("path", ["four-clauses-per-wave", "all-rows-layer-0", "one-clause-per-wave",
+@pytest.mark.parametrize("path", ["several-clauses-per-wave", "128-bit-reads", "all-rows-layer-0", "one-clause-per-wave",
                                   "messages-of-a-tile-in-lds", "messages-in-three-launches"])
 def test_scoring_on_narrow_tiles(shape, depth, path, tune):
-    """Tiles whose rows are at most 32 words wide: four clauses per wave (score_narrow.h), for the message
+    """Tiles whose rows are at most 64 words wide: eight or four clauses per wave (score_narrow.h), for the message
     layers and - on a data set whose negated literals are the complements of its positive ones - for
     layer 0 on the positive rows alone; against the oracle and against the kernels that take one clause
     per wave.  The clauses are of three kinds: random ones (most die within the first rows), ones made of
@@ -1010,7 +1015,9 @@ def test_scoring_on_narrow_tiles(shape, depth, path, tune):
     sets: their lists take several windows of 128 entries and are walked to the end), and empty ones."""
     from tests.gpu_harness import Device
 
-    if path == "all-rows-layer-0":
+    if path == "128-bit-reads":  # (rows of at most 32 words: eight clauses per wave, four words per lane)
+        tune("GTM_NARROW_READS", "128")
+    elif path == "all-rows-layer-0":
         tune("GTM_NO_HALF_ROWS", "1")
     elif path == "one-clause-per-wave":
         tune("GTM_NO_NARROW_LAYERS", "1")
@@ -1023,7 +1030,7 @@ def test_scoring_on_narrow_tiles(shape, depth, path, tune):
         tune("GTM_NO_FUSED_MESSAGES", "1")
     graphs = helpers.random_graphs(shape["seed"], max_degree=3, **shape["g"])
     hv = graphs.hypervector_size
-    M = 1024 if depth > 1 else 64
+    M = shape.get("M", 1024) if depth > 1 else 64
     cfg = helpers.oracle_config(graphs, classes=shape["classes"], clauses=150, depth=depth, message_size=M)
     # (random clauses of about three literals: some are true at some nodes of some graphs)
     model = helpers.random_model(shape["seed"], cfg, depth, include_density=1.5 / hv, message_density=0.004)
