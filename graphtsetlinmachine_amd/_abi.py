@@ -8,7 +8,7 @@ import ctypes as C
 import os
 
 GTM_MAX_DEPTH = 8
-GTM_ABI_VERSION = 2
+GTM_ABI_VERSION = 3
 GTM_GRAPHS_COMPLEMENTARY = 1
 
 _HERE = os.path.dirname(os.path.abspath(__file__))

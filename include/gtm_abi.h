@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define GTM_ABI_VERSION 2
+#define GTM_ABI_VERSION 3
 #define GTM_MAX_DEPTH 8
 
 #define GTM_OK 0
