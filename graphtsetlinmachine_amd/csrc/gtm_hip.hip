@@ -1055,7 +1055,7 @@ int compute_units() {
     return cus_of[dev];
 }
 
-// The tiles of a launch of k_tile_two_phase_half shared out among the compute units (tile_segments_block
+// The tiles of a launch of k_tile_two_phase_half shared out among the compute units (tile_segments_part
 // in score_tiles.h) - when they do not fill a whole number of rounds of the chip, and a share is at least 64
 // clauses (a share stages its tile).  GTM_NO_TILE_LINE turns it off; GTM_TILE_LINE_GROUPS = n (tests) cuts the
 // tiles into n shares whatever the device has.  cus == 0 in the result: one workgroup per tile.
@@ -1067,7 +1067,8 @@ SegmentPlan plan_segments(const TileLayerArgs &a, int n_tiles, TileSegment *segm
         cus = atoi(e);
         shared_out = cus >= 1;
     }
-    if (!shared_out || !segments || cus > TILE_SEGMENTS_MAX_SHARES) return sp;
+    // (the table's arithmetic is 32-bit; a block of the compile launch holds at most 16 waves)
+    if (!shared_out || !segments || cus > TILE_SEGMENTS_MAX_SHARES || (int64_t)(n_tiles % cus) * a.C >= (1ll << 31)) return sp;
     sp.n_tiles = n_tiles, sp.C = a.C, sp.cus = cus, sp.gpt = a.tg.gpt, sp.K = a.K, sp.tile0 = a.tile0;
     sp.first_graph = a.first_graph, sp.n_graphs = a.n_graphs, sp.segments = segments, sp.class_sum = a.class_sum;
     return sp;
@@ -1268,7 +1269,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             range.n_graphs = n_graphs, range.class_sum = class_sum;
             plan = plan_segments(range, (first + n_graphs - 1) / tg.gpt - range.tile0 + 1, w.segments);
         }
-        hipLaunchKernelGGL(k_compile_clauses_half, dim3(blocks_for(d.C, TPB / 64) + (plan.cus > 0 ? 1u : 0u)), dim3(TPB), 0, st,
+        hipLaunchKernelGGL(k_compile_clauses_half, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st,
                            s->ta_state, d.C, d.LA, d.B, d.filter, cfg->literals, g->number_of_node_types, tg.tw, order, w.lists,
                            stride0, d.K, layers == 1 ? s->clause_weights : nullptr, w.wt, plan);
     }
@@ -1373,7 +1374,10 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     if (in_lds.ok) {
         static thread_local size_t in_lds_set = 48 * 1024;
         if (in_lds.lds_bytes > in_lds_set) {
-            if (hipFuncSetAttribute((const void *)k_tile_messages_in_lds, hipFuncAttributeMaxDynamicSharedMemorySize,
+            // (both forms of the kernel, so that the limit that is remembered holds for either)
+            if (hipFuncSetAttribute((const void *)k_tile_messages_in_lds<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)in_lds.lds_bytes) != hipSuccess ||
+                hipFuncSetAttribute((const void *)k_tile_messages_in_lds<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)in_lds.lds_bytes) != hipSuccess) {
                 (void)hipGetLastError();
                 in_lds.ok = 0;
@@ -1418,7 +1422,8 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
             // vectors in LDS when they fit, else three launches with the vectors in global memory
             if (in_lds.ok) {
                 profile_start("k_tile_messages_in_lds", st);
-                hipLaunchKernelGGL(k_tile_messages_in_lds, dim3(n_tiles), dim3(TILE_MESSAGES_LDS_BLOCK), in_lds.lds_bytes, st,
+                hipLaunchKernelGGL(tg.tw > 32 ? k_tile_messages_in_lds<true> : k_tile_messages_in_lds<false>, dim3(n_tiles),
+                                   dim3(TILE_MESSAGES_LDS_BLOCK), in_lds.lds_bytes, st,
                                    w.tile_bitmap, d.C, tg, t0, g->number_of_graphs, d.M, s->hypervectors, d.MB, alive_now,
                                    narrow_tiles ? shape.streams() : TILE_MESSAGES_LDS_BLOCK / 16, px.alive_stride, g->node_index, g->number_of_graph_nodes, g->number_of_graph_node_edges,
                                    g->edge_index, g->edge, g->total_edges > 0 ? 1 : 0, in_lds.main_words, in_lds.range_words,

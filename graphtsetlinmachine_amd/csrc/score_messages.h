@@ -46,12 +46,14 @@ struct TileMessagesPlan {
     size_t lds_bytes;
 };
 
-// Shapes the kernel takes: M a multiple of 32 and at most 1,024, tiles of at most 32 words (one
-// thread per node slot), and room in LDS for the vectors plus at least 128 received ones.
+// Shapes the kernel takes: M a multiple of 32 and at most 1,024, tiles of at most 64 words (one or two node slots
+// per thread), at most 1,024 blocks of 32 x 32 bits in the rows, and room in LDS for the vectors plus at least
+// 128 received ones.
 inline TileMessagesPlan tile_messages_lds_plan(const TileGeom &g, int M, size_t lds_limit) {
     TileMessagesPlan p{};
-    if (!g.ok || M < 32 || M % 32 != 0 || M > 1024 || g.tw > 32 || g.tw % 4 != 0) return p;
+    if (!g.ok || M < 32 || M % 32 != 0 || M > 1024 || g.tw > 64 || g.tw % 4 != 0) return p;
     const int MW = M / 32;
+    if (MW * g.tw > 1024) return p;
     const size_t rows = (size_t)M * g.tw, vectors = (size_t)g.tw * 32 * (MW + 1);
     const size_t main_words = rows > vectors ? rows : vectors;
     const size_t per_word = (size_t)32 * (MW + 1);
@@ -65,6 +67,9 @@ inline TileMessagesPlan tile_messages_lds_plan(const TileGeom &g, int M, size_t 
     return p;
 }
 
+// WIDE: rows of 33 to 64 words - a quarter-wave reads a truth row at four words per lane, and a thread owns two
+// node slots.
+template <bool WIDE>
 __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_lds(
     const uint32_t *__restrict__ bitmap, int C, TileGeom tg, int tile0, int G, int M, const uint32_t *__restrict__ hv, int MB,
     const uint32_t *__restrict__ alive, int streams, int alive_stride, const uint32_t *__restrict__ node_index,
@@ -87,9 +92,11 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
     // number and bits then reach the 16 lanes by a lane move (row_share), and eight truth rows are on their way
     // per quarter-wave.
     {
+        constexpr int WPL = WIDE ? 4 : 2;  // words of a truth row per lane
+        typedef uint32_t Words __attribute__((ext_vector_type(WPL)));
         const int group = lane >> 4, gl = lane & 15;
         const uint32_t *truth = bitmap + (int64_t)tile_local * C * tw;
-        const bool has_words = 2 * gl < tw;
+        const bool has_words = WPL * gl < tw;
         // a quarter-wave takes the streams q, q + 64, ... of the evaluation that wrote the truth rows
         for (int q = wave * 4 + group; q < streams; q += TILE_MESSAGES_LDS_BLOCK / 16) {
         const uint32_t *list = alive ? alive + ((int64_t)tile_local * streams + q) * alive_stride : nullptr;
@@ -111,22 +118,29 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
             auto eight = [&](auto first_of_eight) {  // clauses u0 .. u0 + 7 of the 16
                 constexpr int u0 = decltype(first_of_eight)::value;
                 uint32_t c[8];
-                uint2 t[8];
+                Words t[8];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     c[u] = tile_row_share(id, u0 + u);  // (past the stream's end: its last clause once more)
-                    t[u] = *reinterpret_cast<const uint2 *>(truth + (int64_t)c[u] * tw + (has_words ? 2 * gl : 0));
+                    t[u] = *reinterpret_cast<const Words *>(truth + (int64_t)c[u] * tw + (has_words ? WPL * gl : 0));
                 }
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     const uint32_t h0 = tile_row_share(bit0, u0 + u), h1 = tile_row_share(bit1, u0 + u);
-                    if (u0 + u >= n_here || !has_words || (t[u].x | t[u].y) == 0u) continue;
-                    const unsigned long long both = (unsigned long long)t[u].x | ((unsigned long long)t[u].y << 32);
+                    uint32_t any = t[u][0] | t[u][1];
+                    if (WIDE) any |= t[u][2] | t[u][3];
+                    if (u0 + u >= n_here || !has_words || any == 0u) continue;
                     for (int j = 0; j < MB; ++j) {
                         const uint32_t h = j == 0 ? h0 : j == 1 ? h1 : hv[(int64_t)c[u] * MB + j];
                         if (h >= (uint32_t)M) continue;
-                        // (tw is even: the two words are one aligned 64-bit word of LDS)
-                        atomicOr(reinterpret_cast<unsigned long long *>(main_region + h * tw + 2 * gl), both);
+                        // (tw is a multiple of 4: each pair of words is one aligned 64-bit word of LDS)
+                        unsigned long long *row = reinterpret_cast<unsigned long long *>(main_region + h * tw + WPL * gl);
+#pragma unroll
+                        for (int v = 0; v < WPL / 2; ++v) {
+                            const unsigned long long both =
+                                (unsigned long long)t[u][2 * v] | ((unsigned long long)t[u][2 * v + 1] << 32);
+                            if (both) atomicOr(&row[v], both);
+                        }
                     }
                 }
             };
@@ -179,25 +193,32 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
         out[(int64_t)(M + 1) * tw + w] = empties;
     }
 
-    // this thread's source slot and its edges
-    uint32_t ne = 0u, nodes_of_graph = 0u;
-    int slot0 = 0;
-    const uint2 *out_edges = nullptr;
-    if (tid < S && has_edges) {
-        const int gj = tid / tg.slot_bits, n = tid - gj * tg.slot_bits;
-        const int64_t g = (int64_t)(tile0 + tile_local) * tg.gpt + gj;
-        if (gj < tg.gpt && g < G && (uint32_t)n < n_nodes[g]) {
-            const int64_t row = (int64_t)node_index[g] + n;
-            ne = n_edges[row];
-            out_edges = reinterpret_cast<const uint2 *>(edge) + edge_index[row];
-            nodes_of_graph = n_nodes[g];
-            slot0 = gj * tg.slot_bits;
-        }
-    }
-    uint2 first[4];
+    // this thread's source slots (tid, and tid + 1,024 on rows of more than 32 words) and their edges
+    constexpr int SPT = WIDE ? 2 : 1;
+    uint32_t ne[SPT], nodes_of_graph[SPT];
+    int slot0[SPT];
+    const uint2 *out_edges[SPT];
+    uint2 first[SPT][4];
+    const uint32_t *mine[SPT];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) first[u] = (uint32_t)u < ne ? out_edges[u] : make_uint2(0u, 0u);
-    const uint32_t *mine = main_region + (tid < S ? tid : 0) * VS;
+    for (int h = 0; h < SPT; ++h) {
+        const int slot = tid + h * NT;
+        ne[h] = 0u, nodes_of_graph[h] = 0u, slot0[h] = 0, out_edges[h] = nullptr;
+        if (slot < S && has_edges) {
+            const int gj = slot / tg.slot_bits, n = slot - gj * tg.slot_bits;
+            const int64_t g = (int64_t)(tile0 + tile_local) * tg.gpt + gj;
+            if (gj < tg.gpt && g < G && (uint32_t)n < n_nodes[g]) {
+                const int64_t row = (int64_t)node_index[g] + n;
+                ne[h] = n_edges[row];
+                out_edges[h] = reinterpret_cast<const uint2 *>(edge) + edge_index[row];
+                nodes_of_graph[h] = n_nodes[g];
+                slot0[h] = gj * tg.slot_bits;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) first[h][u] = (uint32_t)u < ne[h] ? out_edges[h][u] : make_uint2(0u, 0u);
+        mine[h] = main_region + (slot < S ? slot : 0) * VS;
+    }
 
     for (int w_lo = 0; w_lo < tw; w_lo += range_words) {
         const int w_hi = w_lo + range_words < tw ? w_lo + range_words : tw, nw = w_hi - w_lo;
@@ -205,34 +226,36 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
         __syncthreads();  // (also: every vector of step 2 is in place)
 
         // 3. along the edges into the range
-        for (uint32_t e0 = 0; e0 < ne; e0 += 4) {
-            uint2 pair[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
-                pair[u] = e0 == 0 ? first[u] : (e0 + u < ne ? out_edges[e0 + u] : make_uint2(0u, 0u));
+        for (int h = 0; h < SPT; ++h)
+            for (uint32_t e0 = 0; e0 < ne[h]; e0 += 4) {
+                uint2 pair[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if (e0 + u >= ne) break;
-                const uint32_t dst = pair[u].x;
-                if (dst >= nodes_of_graph) continue;
-                const int to_slot = slot0 + (int)dst, to_word = to_slot >> 5;
-                if (to_word < w_lo || to_word >= w_hi) continue;
-                const uint32_t shift = pair[u].y % (uint32_t)M;
-                const int r = (int)(shift & 31u);
-                uint32_t *to = got + (to_slot - 32 * w_lo) * VS;
-                // bit p of what arrives is bit (p - shift) mod M of what was sent: word j, moved up by r bits with
-                // the top of word j - 1 below it, lands in word (j + shift / 32) mod MW
-                int at = (int)(shift >> 5);
-                uint32_t below = mine[MW - 1];
-                for (int j = 0; j < MW; ++j) {
-                    const uint32_t cur = mine[j];
-                    const uint32_t word = r ? (cur << r) | (below >> (32 - r)) : cur;
-                    if (word) atomicOr(&to[at], word);
-                    at = at + 1 == MW ? 0 : at + 1;
-                    below = cur;
+                for (int u = 0; u < 4; ++u)
+                    pair[u] = e0 == 0 ? first[h][u] : (e0 + u < ne[h] ? out_edges[h][e0 + u] : make_uint2(0u, 0u));
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (e0 + u >= ne[h]) break;
+                    const uint32_t dst = pair[u].x;
+                    if (dst >= nodes_of_graph[h]) continue;
+                    const int to_slot = slot0[h] + (int)dst, to_word = to_slot >> 5;
+                    if (to_word < w_lo || to_word >= w_hi) continue;
+                    const uint32_t shift = pair[u].y % (uint32_t)M;
+                    const int r = (int)(shift & 31u);
+                    uint32_t *to = got + (to_slot - 32 * w_lo) * VS;
+                    // bit p of what arrives is bit (p - shift) mod M of what was sent: word j, moved up by r bits with
+                    // the top of word j - 1 below it, lands in word (j + shift / 32) mod MW
+                    int at = (int)(shift >> 5);
+                    uint32_t below = mine[h][MW - 1];
+                    for (int j = 0; j < MW; ++j) {
+                        const uint32_t cur = mine[h][j];
+                        const uint32_t word = r ? (cur << r) | (below >> (32 - r)) : cur;
+                        if (word) atomicOr(&to[at], word);
+                        at = at + 1 == MW ? 0 : at + 1;
+                        below = cur;
+                    }
                 }
             }
-        }
         __syncthreads();
 
         // 4. literal-major: block (j, w) of the range - word j of slots 32 w .. 32 w + 31 - becomes word w of rows

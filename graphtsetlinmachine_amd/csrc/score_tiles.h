@@ -1688,8 +1688,9 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase(TileLayerArgs a)
 // Workgroups are handed to the CUs in the order of their numbers as CUs fall free, so the first
 // segments come ordered by size, smallest first, and the second segments in the same order of their
 // shares - largest first, since the two add up to a share: whoever finishes a short first segment
-// finds a long second one next in line, and all finish together.  The table is made by one block,
-// which also clears the class sums of the graphs of the shared tiles, to which their workgroups add.
+// finds a long second one next in line, and all finish together.  The table is made, a few entries per
+// block, by the launch that compiles the clauses, which also clears the class sums of the graphs of the
+// shared tiles, to which their workgroups add.
 struct TileSegment {
     int tile_local, c_begin, c_end;
 };
@@ -1705,41 +1706,53 @@ struct SegmentPlan {
 
 inline int tile_segment_count(int n_tiles, int cus) { return n_tiles / cus * cus + 2 * cus; }
 
-// The work of ONE block of `threads` threads (it runs as an extra block of the launch that compiles the
-// clauses, so that it costs the step no time of its own).
-__device__ __forceinline__ void tile_segments_block(const SegmentPlan &sp, int tid, int threads) {
-    __shared__ int first_len[TILE_SEGMENTS_MAX_SHARES];
-    const int C = sp.C, cus = sp.cus;
-    const int whole = sp.n_tiles / cus * cus, rest = sp.n_tiles - whole;
-    for (int b = tid; b < whole; b += threads) sp.segments[b] = TileSegment{b, 0, C};
-    const long long pairs = (long long)rest * C;
-    // share j = pairs [j * pairs / cus, (j + 1) * pairs / cus)
-    auto share = [&](int j, int *tile_a, int *at, int *len_a, int *len_b) {
-        const long long from = pairs * j / cus, to = pairs * (j + 1) / cus;
-        *tile_a = (int)(from / C);
-        *at = (int)(from - (long long)*tile_a * C);
-        *len_a = to - from < (long long)(C - *at) ? (int)(to - from) : C - *at;
-        *len_b = (int)(to - from) - *len_a;
-    };
-    for (int j = tid; j < cus; j += threads) {
-        int tile_a, at, len_a, len_b;
-        share(j, &tile_a, &at, &len_a, &len_b);
-        first_len[j] = len_a;
-    }
-    __syncthreads();
-    for (int j = tid; j < cus; j += threads) {
-        int tile_a, at, len_a, len_b;
-        share(j, &tile_a, &at, &len_a, &len_b);
-        int rank = 0;
-        for (int k = 0; k < cus; ++k) rank += first_len[k] < len_a || (first_len[k] == len_a && k < j);
-        sp.segments[whole + rank] = TileSegment{whole + tile_a, at, at + len_a};
-        sp.segments[whole + cus + rank] = TileSegment{whole + tile_a + 1, 0, len_b};  // (empty when the share lies in one tile)
-    }
+// Block `block` of `n_blocks` (the blocks of the launch that compiles the clauses: every block does a little of
+// this before its clauses, so that the table costs the step no time of its own): its slice of the whole-tile
+// entries and of the class sums to clear, and the two segments of the shares block, block + n_blocks, ...
+// Share j is pairs [from(j), from(j + 1)) of the remaining tiles' (tile, clause) pairs, from(j) = j * (pairs /
+// cus) + min(j, pairs % cus); its place in the table is the rank of its first segment's length among all shares
+// (ties by share number), which every block works out for its own shares by counting.  All threads of the block
+// must call this (it has barriers); pairs < 2^31 (plan_segments).
+__device__ __forceinline__ void tile_segments_part(const SegmentPlan &sp, int block, int n_blocks, int tid, int threads) {
+    __shared__ int counted[16];
+    const uint32_t C = (uint32_t)sp.C, cus = (uint32_t)sp.cus;
+    const int whole = sp.n_tiles / sp.cus * sp.cus, rest = sp.n_tiles - whole;
+    for (int b = block * threads + tid; b < whole; b += n_blocks * threads) sp.segments[b] = TileSegment{b, 0, sp.C};
     // the class sums of the graphs of the shared tiles start at zero
     const long long g_lo = (long long)(sp.tile0 + whole) * sp.gpt, g_hi = (long long)(sp.tile0 + sp.n_tiles) * sp.gpt;
     const long long first = sp.first_graph, end = first + sp.n_graphs;
-    for (long long i = (g_lo > first ? g_lo : first) * sp.K + tid; i < (g_hi < end ? g_hi : end) * sp.K; i += threads)
+    for (long long i = (g_lo > first ? g_lo : first) * sp.K + block * threads + tid; i < (g_hi < end ? g_hi : end) * sp.K;
+         i += (long long)n_blocks * threads)
         sp.class_sum[i - first * sp.K] = 0;
+    const uint32_t pairs = (uint32_t)rest * C, base = pairs / cus, extra = pairs % cus;
+    auto from_of = [&](uint32_t j) { return j * base + (j < extra ? j : extra); };
+    auto first_length = [&](uint32_t j, uint32_t *tile_a, uint32_t *at, uint32_t *length) {
+        const uint32_t from = from_of(j);
+        *length = from_of(j + 1) - from;
+        *tile_a = from / C;
+        *at = from - *tile_a * C;
+        return *length < C - *at ? *length : C - *at;
+    };
+    for (uint32_t j = (uint32_t)block; j < cus; j += (uint32_t)n_blocks) {
+        uint32_t tile_a, at, length, t, a2, l2;
+        const uint32_t len_a = first_length(j, &tile_a, &at, &length);
+        int before = 0;
+        for (uint32_t k = (uint32_t)tid; k < cus; k += (uint32_t)threads) {
+            const uint32_t len_k = first_length(k, &t, &a2, &l2);
+            before += len_k < len_a || (len_k == len_a && k < j);
+        }
+        for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off);
+        __syncthreads();  // (the block's last round has been read)
+        if ((tid & 63) == 0) counted[(tid >> 6) & 15] = before;
+        __syncthreads();
+        if (tid == 0) {
+            int rank = 0;
+            for (int w = 0; w < (threads + 63) / 64 && w < 16; ++w) rank += counted[w];
+            sp.segments[whole + rank] = TileSegment{whole + (int)tile_a, (int)at, (int)(at + len_a)};
+            // (empty when the share lies in one tile)
+            sp.segments[whole + (int)cus + rank] = TileSegment{whole + (int)tile_a + 1, 0, (int)(length - len_a)};
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -1773,10 +1786,7 @@ __global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C,
                                        uint32_t *__restrict__ records, int record_words, int K,
                                        const int32_t *__restrict__ weights, int32_t *__restrict__ wt, SegmentPlan sp) {
     __shared__ uint32_t chosen_of_wave[4][16];
-    if (sp.cus > 0 && blockIdx.x == gridDim.x - 1) {  // the launch's extra block: which workgroup takes what (see above)
-        tile_segments_block(sp, threadIdx.x, blockDim.x);
-        return;
-    }
+    if (sp.cus > 0) tile_segments_part(sp, blockIdx.x, gridDim.x, threadIdx.x, blockDim.x);  // which workgroup takes what (see above)
     const int lane = threadIdx.x & 63;
     const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (c >= C) return;  // whole waves leave; no barrier below
@@ -1867,7 +1877,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
     const int rows_lds = tg.rows - hv;           // + node types + all ones
     uint32_t *bt = lds;
     int32_t *sums = (int32_t *)(lds + (size_t)rows_lds * tw + TILE_LDS_PAD_WORDS);
-    // This workgroup's share: a whole tile, or - with a table of segments (tile_segments_block above) - clauses
+    // This workgroup's share: a whole tile, or - with a table of segments (tile_segments_part above) - clauses
     // [c_begin, c_end) of a tile whose other clauses other workgroups take.
     int tile_local = blockIdx.x, c_begin = 0, c_end = C;
     if (a.segments) {
@@ -2185,7 +2195,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
             if (whole_tile)
                 *out = sums[i];
             else if (sums[i] != 0)
-                atomicAdd(out, sums[i]);  // a tile shared with other workgroups (tile_segments_block cleared its sums)
+                atomicAdd(out, sums[i]);  // a tile shared with other workgroups (tile_segments_part cleared its sums)
         }
     }
 }
