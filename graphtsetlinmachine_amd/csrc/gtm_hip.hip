@@ -64,6 +64,7 @@ int check_launch(const char *what) {
     X(HALF_LANE_WORDS) \
     X(MESSAGES_IN_LDS) \
     X(NARROW_READS) \
+    X(NARROW_ROWS_AS_STORED) \
     X(NODE_MESSAGES_BY_ATOMICS) \
     X(NO_DEEP_FIT) \
     X(NO_DEEP_PERSISTENT_FIT) \
@@ -1176,7 +1177,7 @@ int launch_two_phase_wide(const TileLayerArgs &a, int n_tiles, int LA, bool stag
 // Several clauses per wave on narrow tiles (score_narrow.h).
 template <int SRC, bool LAST, int GROUP, int WPL>
 int launch_narrow_as(const TileLayerArgs &a, const NarrowArgs &x, int n_tiles, hipStream_t st) {
-    const size_t lds = narrow_lds_bytes(a.tg, NarrowChoice{GROUP, WPL}, a.K, narrow_rows_lds(SRC, a.M, x.hv, x.n_types));
+    const size_t lds = narrow_lds_bytes(a.tg, NarrowChoice{GROUP, WPL}, a.K, narrow_rows_lds(SRC, a.M, x.hv, x.n_types), x.row_words);
     static thread_local size_t lds_set = 48 * 1024;
     if (lds > lds_set) {
         hipError_t e = hipFuncSetAttribute((const void *)k_tile_layer_narrow<SRC, LAST, GROUP, WPL>,
@@ -1248,12 +1249,18 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     const NarrowChoice shape = narrow_choice(tg, narrow_reads && atoi(narrow_reads) == 128);
     const bool narrow_tiles = shape.group != 0 && !tune(T_NO_NARROW_LAYERS);
     const bool narrow_messages =
-        narrow_tiles && layers > 1 && narrow_lds_bytes(tg, shape, d.K, tile_message_rows(d.M)) <= lds_limit;
+        narrow_tiles && layers > 1 && narrow_lds_bytes(tg, shape, d.K, tile_message_rows(d.M), tg.tw) <= lds_limit;
     // (layer 0 of a model without message layers keeps the two-phase kernels on rows of more than 32 words)
     const bool half_rows0 = narrow_tiles && !tg.half && (layers > 1 || tg.tw <= 32) &&
                             (g->flags & GTM_GRAPHS_COMPLEMENTARY) && cfg->literals % 2 == 0 &&
-                            narrow_lds_bytes(tg, shape, d.K, hv + g->number_of_node_types + 1) <= lds_limit &&
+                            narrow_lds_bytes(tg, shape, d.K, hv + g->number_of_node_types + 1, tg.tw) <= lds_limit &&
                             !tune(T_NO_HALF_ROWS);
+    // words from row to row in LDS (128 bytes apart where that fits; GTM_NARROW_ROWS_AS_STORED, tuning aid: as in memory)
+    const bool as_stored = tune(T_NARROW_ROWS_AS_STORED) != nullptr;
+    const int row_words0 = half_rows0 && !as_stored
+                               ? narrow_row_words(tg, shape, d.K, hv + g->number_of_node_types + 1, lds_limit) : tg.tw;
+    const int row_words_m = narrow_messages && !as_stored
+                                ? narrow_row_words(tg, shape, d.K, tile_message_rows(d.M), lds_limit) : tg.tw;
     // compiled clause: 8 words of packed 16-bit row entries (16 words of byte offsets on half tiles) + the include words
     const int stride0 = half_rows0 ? w.list_stride : tg.half ? 16 + d.LA : two_phase ? 8 + d.LA : w.list_stride;
     SegmentPlan plan{};
@@ -1261,7 +1268,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         // rows as k_tile_layer_narrow<ROWS_HALF> stages them: positive literals, node types, all ones
         hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, s->ta_state, d.C,
                            d.LA, d.B, d.filter, cfg->literals, hv, g->number_of_node_types, hv, hv + g->number_of_node_types,
-                           tg.tw, w.list_stride, order, w.lists, d.K, layers == 1 ? s->clause_weights : nullptr, w.wt);
+                           row_words0, w.list_stride, order, w.lists, d.K, layers == 1 ? s->clause_weights : nullptr, w.wt);
     else if (tg.half) {
         if (layers == 1 && !tr) {  // one launch over every tile of the range: its tiles may be shared out among the CUs
             TileLayerArgs range{};
@@ -1289,7 +1296,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     }
     for (int l = 1; l < layers; ++l) {
         hipLaunchKernelGGL(k_compile_clauses, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st,
-                           s->message_ta_state[l - 1], d.C, d.MC, d.B, d.mfilter, 2 * d.M, d.M, 0, 0, d.M, tg.tw,
+                           s->message_ta_state[l - 1], d.C, d.MC, d.B, d.mfilter, 2 * d.M, d.M, 0, 0, d.M, row_words_m,
                            w.message_list_stride, (const uint32_t *)nullptr,
                            w.message_lists + (size_t)(l - 1) * d.C * w.message_list_stride, d.K,
                            l == layers - 1 ? s->clause_weights : nullptr, w.wt, w.longest_list + (l - 1));
@@ -1321,6 +1328,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         if (half_rows0) {
             px.alive_in = nullptr;
             px.alive_out = !last && narrow_messages ? w.alive[0] : nullptr;
+            px.row_words = row_words0;
             alive_now = px.alive_out;
             return launch_narrow(a, px, shape, n_tiles, ROWS_HALF, last, st);
         }
@@ -1406,6 +1414,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         const bool last = l == layers - 1 && !tr;
         if (!narrow_messages) return launch_tile_layer(a, n_tiles, ROWS_MESSAGES, last, st);
         px.alive_in = alive_now;
+        px.row_words = row_words_m;
         px.alive_out = last || l == layers - 1 ? nullptr : w.alive[alive_now == w.alive[0] ? 1 : 0];
         alive_now = px.alive_out;
         return launch_narrow(a, px, shape, n_tiles, ROWS_MESSAGES, last, st);

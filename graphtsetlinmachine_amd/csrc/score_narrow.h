@@ -67,6 +67,7 @@ struct NarrowArgs {
     uint32_t *alive_out;       // the same for the next layer, or NULL
     int alive_stride;          // >= 1 + ceil(C / streams)
     int hv, n_types;           // ROWS_HALF: positive literals (= LDS rows before the node-type rows), node types
+    int row_words;             // words from one row to the next in LDS (>= tw, a multiple of 4): what the lists' entries count in
 };
 
 // The shape for a tile geometry: lanes per clause and words per lane (0, 0: none).  Rows of at most 32 words take
@@ -92,9 +93,19 @@ inline int narrow_alive_stride(int C, int streams) { return 1 + (C + streams - 1
 
 inline int narrow_rows_lds(int src, int M, int hv, int n_types) { return src == ROWS_HALF ? hv + n_types + 1 : M + 2; }
 
-inline size_t narrow_lds_bytes(const TileGeom &g, const NarrowChoice &shape, int classes, int rows_lds) {
+inline size_t narrow_lds_bytes(const TileGeom &g, const NarrowChoice &shape, int classes, int rows_lds, int row_words) {
     const size_t sums = ((size_t)g.gpt * classes + 3) & ~(size_t)3;  // the lists after them stay 16-byte aligned
-    return ((size_t)rows_lds * g.tw + TILE_LDS_PAD_WORDS + sums + (size_t)shape.streams() * shape.list_words()) * 4;
+    return ((size_t)rows_lds * row_words + TILE_LDS_PAD_WORDS + sums + (size_t)shape.streams() * shape.list_words()) * 4;
+}
+
+// Rows in LDS start 128 bytes apart where that fits: a group's read of a row then covers one aligned half of
+// the 64 banks, and two groups of a wave collide only when their rows lie in the same half.  With rows 112 bytes
+// apart (28-word rows as they lie in memory) nearly every pair of reads overlaps in some banks: a micro-benchmark
+// of 16 waves reading four unrelated rows per 64-bit instruction takes 2.1 ns per instruction and CU at 112 bytes
+// and 1.2 ns at 128.
+inline int narrow_row_words(const TileGeom &g, const NarrowChoice &shape, int classes, int rows_lds, size_t lds_limit) {
+    const int padded = (g.tw + 31) & ~31;
+    return narrow_lds_bytes(g, shape, classes, rows_lds, padded) <= lds_limit ? padded : g.tw;
 }
 
 // The LDS addresses of a block's 8 rows for this lane: adr[i] = base + entry i of the block, where the
@@ -160,11 +171,11 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
     constexpr uint32_t GROUP_MASK = (1u << GROUP) - 1u;
     extern __shared__ uint32_t lds[];
     const TileGeom &tg = a.tg;
-    const int tw = tg.tw, C = a.C, K = a.K;
+    const int tw = tg.tw, rw = x.row_words, C = a.C, K = a.K;
     constexpr int NT = NARROW_WAVES * 64;
     const int rows_lds = SRC == ROWS_HALF ? x.hv + x.n_types + 1 : a.M + 2;
     uint32_t *bt = lds;
-    int32_t *sums = (int32_t *)(lds + (size_t)rows_lds * tw + TILE_LDS_PAD_WORDS);
+    int32_t *sums = (int32_t *)(lds + (size_t)rows_lds * rw + TILE_LDS_PAD_WORDS);
     uint32_t *lists = (uint32_t *)sums + ((tg.gpt * K + 3) & ~3);
     const int tile_local = blockIdx.x, tile = a.tile0 + tile_local;
     const int tid = threadIdx.x, lane = tid & 63, gl = lane & (GROUP - 1), group = lane / GROUP;
@@ -184,6 +195,7 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
         }
         uint4 *dst = reinterpret_cast<uint4 *>(bt);
         const int n4 = (rows_lds * tw) >> 2;  // tw is a multiple of 4
+        const int pieces = tw >> 2, apart = rw >> 2;  // 16-byte pieces of a row; from row to row in LDS
         for (int i = tid; i < n4; i += NT * 4) {
             uint4 v[4];
 #pragma unroll
@@ -194,11 +206,11 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int at = i + u * NT;
-                if (at < n4) dst[at] = v[u];
+                if (at < n4) dst[rw == tw ? at : at / pieces * apart + at % pieces] = v[u];
             }
         }
         // the words after the rows read as zero (the complement of "no row": all ones), the class sums start at zero
-        for (int i = tid; i < TILE_LDS_PAD_WORDS + ((tg.gpt * K + 3) & ~3); i += NT) bt[(size_t)rows_lds * tw + i] = 0;
+        for (int i = tid; i < TILE_LDS_PAD_WORDS + ((tg.gpt * K + 3) & ~3); i += NT) bt[(size_t)rows_lds * rw + i] = 0;
     }
     __syncthreads();
 
@@ -207,7 +219,7 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
     const uint32_t col_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint32_t *)(bt + WPL * gl);
     uint32_t *my_list = lists + q * Shape::LIST_WORDS;
     const uint32_t *quad_entry = my_list + (lane & 3);
-    const uint32_t ones_entry = (uint32_t)(rows_lds - 1 - (SRC == ROWS_MESSAGES ? 1 : 0)) * (uint32_t)tw * 4u;
+    const uint32_t ones_entry = (uint32_t)(rows_lds - 1 - (SRC == ROWS_MESSAGES ? 1 : 0)) * (uint32_t)rw * 4u;
     // this group's lanes in a 64-bit vote: bits shift .. shift + GROUP - 1 of its low or high half
     const bool upper_half = lane >= 32;
     const uint32_t shift = (uint32_t)(group * GROUP) & 31u;
@@ -221,7 +233,7 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
     empties.fill(0u);
     bool any_empty = false;
     if (SRC == ROWS_MESSAGES) {
-        if (active) empties.load(bt + (size_t)(a.M + 1) * tw + WPL * gl);
+        if (active) empties.load(bt + (size_t)(a.M + 1) * rw + WPL * gl);
         any_empty = __ballot(empties.any()) != 0ull;
     }
 

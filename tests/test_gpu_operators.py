@@ -1004,7 +1004,7 @@ NARROW_TILE_SHAPES = [
 
 @pytest.mark.parametrize("shape", NARROW_TILE_SHAPES, ids=lambda s: "narrow%d" % s["seed"])
 @pytest.mark.parametrize("depth", [1, 2, 3])
-@pytest.mark.parametrize("path", ["several-clauses-per-wave", "128-bit-reads", "all-rows-layer-0", "one-clause-per-wave",
+@pytest.mark.parametrize("path", ["several-clauses-per-wave", "128-bit-reads", "rows-as-stored", "all-rows-layer-0", "one-clause-per-wave",
                                   "messages-of-a-tile-in-lds", "messages-in-three-launches"])
 def test_scoring_on_narrow_tiles(shape, depth, path, tune):
     """Tiles whose rows are at most 64 words wide: eight or four clauses per wave (score_narrow.h), for the message
@@ -1017,6 +1017,8 @@ def test_scoring_on_narrow_tiles(shape, depth, path, tune):
 
     if path == "128-bit-reads":  # (rows of at most 32 words: eight clauses per wave, four words per lane)
         tune("GTM_NARROW_READS", "128")
+    elif path == "rows-as-stored":  # (rows in LDS as far apart as in memory, not 128 bytes)
+        tune("GTM_NARROW_ROWS_AS_STORED", "1")
     elif path == "all-rows-layer-0":
         tune("GTM_NO_HALF_ROWS", "1")
     elif path == "one-clause-per-wave":
