@@ -28,7 +28,7 @@
 // clauses ahead - and passes through a few words of LDS of the group's own, from which the walk
 // reads it back a block ahead of the rows (the four lanes of a quad read entries 0..3 and 4..7 of
 // a block, and an entry reaches all lanes inside the add that forms the row's address).  16 row
-// words in flight per lane and trip (two blocks at 2 words per lane, one at 4), one test per trip
+// words in flight per lane and trip (two blocks at 2 words per lane, one at 4), one test per two trips
 // for "false at every node slot of the tile" - per group: a wave goes on while any of its clauses
 // is alive and has rows left.  What differs between the groups in a trip - a block of rows to AND
 // against a block of complements, a list that has ended - is a per-lane XOR mask folded into the
@@ -345,36 +345,42 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
                 uint32_t lo[TRIP], hi[TRIP];
 #pragma unroll
                 for (int t = 0; t < TRIP; ++t) lo[t] = quad_entry[8 * t], hi[t] = quad_entry[8 * t + 4];
-#pragma unroll 2
-                for (int b = 0; b < lim_most && work_left(b0 + b); b += TRIP) {
-                    uint32_t n_lo[TRIP], n_hi[TRIP];
+                // Two trips between tests for "some group still has a live clause with blocks left": in the regime
+                // that costs the time every clause walks its whole list, and the test is a sixth of a trip's vector
+                // work.  (The blocks past a group's last one are the all-ones row: reading them changes nothing.)
+                for (int b = 0; b < lim_most && work_left(b0 + b); b += 2 * TRIP) {
 #pragma unroll
-                    for (int t = 0; t < TRIP; ++t)
-                        n_lo[t] = quad_entry[8 * (b + TRIP + t)], n_hi[t] = quad_entry[8 * (b + TRIP + t) + 4];
-                    uint32_t adr[TRIP][8];
+                    for (int half = 0; half < 2; ++half) {
+                        const int at = b + half * TRIP;
+                        uint32_t n_lo[TRIP], n_hi[TRIP];
 #pragma unroll
-                    for (int t = 0; t < TRIP; ++t) narrow_block_addresses(lo[t], hi[t], col_lds, adr[t]);
-                    Row r[TRIP][8];
+                        for (int t = 0; t < TRIP; ++t)
+                            n_lo[t] = quad_entry[8 * (at + TRIP + t)], n_hi[t] = quad_entry[8 * (at + TRIP + t) + 4];
+                        uint32_t adr[TRIP][8];
 #pragma unroll
-                    for (int t = 0; t < TRIP; ++t)
+                        for (int t = 0; t < TRIP; ++t) narrow_block_addresses(lo[t], hi[t], col_lds, adr[t]);
+                        Row r[TRIP][8];
 #pragma unroll
-                        for (int u = 0; u < 8; ++u) r[t][u].load_lds(adr[t][u]);
+                        for (int t = 0; t < TRIP; ++t)
 #pragma unroll
-                    for (int t = 0; t < TRIP; ++t) {
-                        // all ones for a block of complements, else zero (a signed one-bit field of flip_bits)
-                        const uint32_t flip = (uint32_t)__builtin_amdgcn_sbfe(flip_bits, b + t, 1);
+                            for (int u = 0; u < 8; ++u) r[t][u].load_lds(adr[t][u]);
 #pragma unroll
-                        for (int v = 0; v < WPL; ++v) {
-                            const uint32_t p0 = narrow_pair(r[t][0].w[v], r[t][1].w[v], flip);
-                            const uint32_t p1 = narrow_pair(r[t][2].w[v], r[t][3].w[v], flip);
-                            const uint32_t p2 = narrow_pair(r[t][4].w[v], r[t][5].w[v], flip);
-                            const uint32_t p3 = narrow_pair(r[t][6].w[v], r[t][7].w[v], flip);
-                            acc.w[v] = narrow_and3(narrow_and3(acc.w[v], p0, p1), p2, p3);
+                        for (int t = 0; t < TRIP; ++t) {
+                            // all ones for a block of complements, else zero (a signed one-bit field of flip_bits)
+                            const uint32_t flip = (uint32_t)__builtin_amdgcn_sbfe(flip_bits, at + t, 1);
+#pragma unroll
+                            for (int v = 0; v < WPL; ++v) {
+                                const uint32_t p0 = narrow_pair(r[t][0].w[v], r[t][1].w[v], flip);
+                                const uint32_t p1 = narrow_pair(r[t][2].w[v], r[t][3].w[v], flip);
+                                const uint32_t p2 = narrow_pair(r[t][4].w[v], r[t][5].w[v], flip);
+                                const uint32_t p3 = narrow_pair(r[t][6].w[v], r[t][7].w[v], flip);
+                                acc.w[v] = narrow_and3(narrow_and3(acc.w[v], p0, p1), p2, p3);
+                            }
                         }
+#pragma unroll
+                        for (int t = 0; t < TRIP; ++t) lo[t] = n_lo[t], hi[t] = n_hi[t];
                     }
                     nzw = __ballot(acc.any());
-#pragma unroll
-                    for (int t = 0; t < TRIP; ++t) lo[t] = n_lo[t], hi[t] = n_hi[t];
                 }
             }
             if (SRC == ROWS_MESSAGES && any_empty) {
