@@ -95,6 +95,7 @@ struct FitDeepParams {
     unsigned long long wait_ticks;
     int force_abort;
     int clauses_per_group;
+    const int *perm;  // [groups][clauses_per_group] the clause in each workgroup's slots, -1 after its last; NULL: clauses in order
     int NW;          // words of a row over the nodes of the largest graph
     int rows_words;  // LDS words of the staged layer-0 rows: (literals + n_types + 1) * NW; 0 when they are read in place (BIG)
     int window_rows; // received rows that pass through LDS at a time: a multiple of 32, M unless BIG
@@ -233,6 +234,64 @@ __device__ __forceinline__ void fitd_and_rows(const uint32_t *inc, int inc_strid
     }
 }
 
+// Clauses dealt out to the workgroups by what they cost.  A workgroup owns its clauses for a whole launch, and
+// an example takes as long as the slowest workgroup: with clauses in order, 32 to a workgroup, the sum of 32
+// costs that differ by an order of magnitude (a clause of a hundred literals that holds at many nodes walks all
+// its rows; an empty one costs next to nothing) varies by a third between workgroups.  Between launches of a
+// run of examples the clauses are therefore sorted by the number of literals they include in all banks - what
+// a clause's evaluation and feedback walk - and dealt out in rounds, back and forth over the workgroups, so
+// that every workgroup gets the same mix.  Nothing moves: the table says which clause sits in which slot.
+constexpr int FITD_MAX_DEALT = 64;     // clauses per workgroup that the table can hold
+constexpr int FITD_DEAL_MAX = 8192;    // clauses that one workgroup sorts in LDS
+
+struct FitDeepBanks {
+    const uint32_t *bank[GTM_MAX_DEPTH];
+};
+
+// cost[c] = included literals of clause c over all banks (one wave per clause)
+__global__ void k_fit_deep_cost(FitDeepBanks banks, int depth, int C, int LA, int MC, int B, uint32_t *__restrict__ cost) {
+    const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (c >= C) return;
+    uint32_t n = 0u;
+    for (int l = 0; l < depth; ++l) {
+        const int chunks = l == 0 ? LA : MC;
+        for (int w = lane; w < chunks; w += 64) n += (uint32_t)__popc(banks.bank[l][((int64_t)c * chunks + w) * B + (B - 1)]);
+    }
+    for (int off = 32; off > 0; off >>= 1) n += __shfl_xor(n, off);
+    if (lane == 0) cost[c] = n;
+}
+
+// One workgroup of 1,024 threads: the clauses sorted by cost, dearest first (ties by clause number), and dealt
+// out: the clause at place r * G + j goes to slot r of workgroup j (r even) or G - 1 - j (r odd).  Dynamic LDS:
+// 8 bytes per clause, rounded up to a power of two.
+__global__ __launch_bounds__(1024) void k_fit_deep_deal(const uint32_t *__restrict__ cost, int C, int G, int own_max,
+                                                         int *__restrict__ perm) {
+    extern __shared__ unsigned long long deal_keys[];
+    int N = 1;
+    while (N < C) N <<= 1;
+    for (int i = threadIdx.x; i < N; i += 1024)  // descending by cost, then ascending by clause: ~clause in the low word
+        deal_keys[i] = i < C ? ((unsigned long long)cost[i] << 32) | (uint32_t)(0x7FFFFFFF - i) : 0ull;
+    for (int i = threadIdx.x; i < G * own_max; i += 1024) perm[i] = -1;
+    __syncthreads();
+    for (int k = 2; k <= N; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = threadIdx.x; i < N; i += 1024) {
+                const int partner = i ^ j;
+                if (partner > i) {
+                    const unsigned long long a = deal_keys[i], b = deal_keys[partner];
+                    const bool descending = (i & k) == 0;
+                    if (descending ? a < b : a > b) deal_keys[i] = b, deal_keys[partner] = a;
+                }
+            }
+            __syncthreads();
+        }
+    for (int at = threadIdx.x; at < C; at += 1024) {
+        const int c = 0x7FFFFFFF - (int)(uint32_t)deal_keys[at];
+        const int r = at / G, j = at - r * G;
+        perm[((r & 1) ? G - 1 - j : j) * own_max + r] = c;
+    }
+}
+
 // MAXB: bit planes of an automaton kept in registers while a word is updated (>= B).
 // BIG: automata in global memory, layer-0 rows read in place, received rows in windows (see the top).
 template <int MAXB, bool BIG>
@@ -244,8 +303,21 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
     constexpr int WAVES = FITD_BLOCK / 64;
     const int G = (int)gridDim.x, g = (int)blockIdx.x;
     const int own_max = p.clauses_per_group;
-    const int c0 = g * own_max;
-    const int n_own = min(own_max, p.C - c0);
+    // The workgroup's clauses: `own_max` slots, the first n_own of them taken - clauses g * own_max .. in order, or
+    // what the table says (clauses dealt out by what they cost, k_fit_deep_deal below).  Everything that is
+    // indexed by clause - automata, weights, hypervector bits, node types, random numbers - goes by own_id.
+    __shared__ int own_id[FITD_MAX_DEALT];
+    __shared__ int n_own_shared;
+    if (tid == 0) {
+        int n = 0;
+        for (int cl = 0; cl < own_max; ++cl) {
+            const int c = p.perm ? p.perm[g * own_max + cl] : (g * own_max + cl < p.C ? g * own_max + cl : -1);
+            if (c >= 0 && cl < FITD_MAX_DEALT) own_id[n++] = c;
+        }
+        n_own_shared = n;
+    }
+    __syncthreads();
+    const int n_own = n_own_shared;
     const int LA = p.LA, MC = p.MC, MW = p.MW, M = p.M, B = p.B, K = p.K, NW = p.NW, L = p.depth - 1, TE = p.edge_types;
     const int WR = p.window_rows;
     const int per_clause = LA + L * MC;  // automaton words of a clause over all banks
@@ -278,7 +350,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
     auto word_in_memory = [&](int cl, int w) -> uint32_t * {
         const int bank = w < LA ? 0 : 1 + (w - LA) / MC;
         const int wl = w < LA ? w : (w - LA) % MC, chunks = bank == 0 ? LA : MC;
-        return p.bank[bank] + ((int64_t)(c0 + cl) * chunks + wl) * B;
+        return p.bank[bank] + ((int64_t)own_id[cl] * chunks + wl) * B;
     };
 
     // own state -> LDS
@@ -291,9 +363,9 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
     }
     for (int i = tid; i < n_own * K; i += FITD_BLOCK) {
         const int cl = i / K, k = i - cl * K;
-        wts[i] = p.weights[(int64_t)k * p.C + c0 + cl];
+        wts[i] = p.weights[(int64_t)k * p.C + own_id[cl]];
     }
-    for (int i = tid; i < n_own * p.MB; i += FITD_BLOCK) hv_own[i] = p.hv[(int64_t)c0 * p.MB + i];
+    for (int i = tid; i < n_own * p.MB; i += FITD_BLOCK) hv_own[i] = p.hv[(int64_t)own_id[i / p.MB] * p.MB + i % p.MB];
     if constexpr (BIG)
         for (int i = tid; i < p.literals; i += FITD_BLOCK) order[i] = p.order[i];
     if (tid == 0) go_on = 1, next_unit[0] = 0;
@@ -377,7 +449,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
             for (int cl = take_unit(0); cl < n_own; cl = take_unit(0)) {
                 int included;
                 const uint32_t v = fit_clause_truth(ta + (size_t)cl * per_clause, 1, LA, p.filter, tile + (active ? lane : 0), row_stride,
-                                                    p.literals, p.literals + (c0 + cl) % p.n_types, ones_row, fg, n, FIT_WALK_ALL,
+                                                    p.literals, p.literals + own_id[cl] % p.n_types, ones_row, fg, n, FIT_WALK_ALL,
                                                     p.X + base * LA, order, active, lane, &included);
                 if (lane < NW) truth[cl * NW + lane] = v;
                 if (lane == 0) incl_of[cl] = included;
@@ -387,7 +459,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
         } else {
             for (int at = tid; at < n_own * NW; at += FITD_BLOCK) {
                 const int cl = at / NW, w = at - cl * NW;
-                truth[at] = w < words ? rows0[(int64_t)(p.literals + (c0 + cl) % p.n_types) * row_stride + w] : 0u;
+                truth[at] = w < words ? rows0[(int64_t)(p.literals + own_id[cl] % p.n_types) * row_stride + w] : 0u;
             }
             lds_barrier();
             FITD_TICK(0)
@@ -557,7 +629,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
 
         // ---- 3. node pick (K7) and votes (K6)
         for (int cl = wave; cl < n_own; cl += WAVES) {
-            const int c = c0 + cl;
+            const int c = own_id[cl];
             const uint32_t v = lane < NW ? truth[cl * NW + lane] : 0u;
             const int pc = __popc(v);
             int true_nodes, before;
@@ -668,7 +740,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
             const int sign = (w >= 0) - (w < 0);
             int err = yk - cs;
             err = err < 0 ? -err : err;
-            philox_out r = philox4x32_10((uint32_t)(c0 + cl), (uint32_t)k, step, GTM_TAG_CLAUSE_UPDATES, p.k0, p.k1);
+            philox_out r = philox4x32_10((uint32_t)own_id[cl], (uint32_t)k, step, GTM_TAG_CLAUSE_UPDATES, p.k0, p.k1);
             const bool skip = (target == -1 && (uint64_t)r.v[0] >= p.q_thr) ||
                               ((uint64_t)r.v[1] * (uint64_t)(2 * (int64_t)p.T) >= ((uint64_t)err << 32));
             const int u = skip ? 0 : target * sign;
@@ -700,7 +772,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                 const int wl = w < LA ? w : (w - LA) % MC;
                 uint32_t x = 0u;
                 if (fired) x = bank != 0 ? mlit[((size_t)cl * L + (bank - 1)) * MC + wl] : at == tid ? x_first : p.X[(base + node) * LA + wl];
-                feedback_word<MAXB>(ta + (size_t)at * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1, (uint32_t)(c0 + cl),
+                feedback_word<MAXB>(ta + (size_t)at * B, B, K, u_of, 1, fired, within, p.boost, x, p.k0, p.k1, (uint32_t)own_id[cl],
                                     (uint32_t)wl, step, (uint32_t)bank, p.thr16[bank]);
             }
         } else {
@@ -736,7 +808,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                     const int wl = w < LA ? w : (w - LA) % MC;
                     // (the include plane's copy in LDS follows)
                     ta[at] = feedback_word<MAXB>(word_in_memory(cl, w), B, K, upd + cl * K, 1, node_of[cl] != -1,
-                                                 incl_of[cl] <= p.max_included, p.boost, x[u], p.k0, p.k1, (uint32_t)(c0 + cl),
+                                                 incl_of[cl] <= p.max_included, p.boost, x[u], p.k0, p.k1, (uint32_t)own_id[cl],
                                                  (uint32_t)wl, step, (uint32_t)bank, p.thr16[bank]);
                 }
             }
@@ -759,6 +831,6 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
         }
     for (int i = tid; i < n_own * K; i += FITD_BLOCK) {
         const int cl = i / K, k = i - cl * K;
-        p.weights[(int64_t)k * p.C + c0 + cl] = wts[i];
+        p.weights[(int64_t)k * p.C + own_id[cl]] = wts[i];
     }
 }

@@ -54,8 +54,10 @@ int check_launch(const char *what) {
 // entry points then only look at this table.  gtm_tuning_set / gtm_tuning_reload (tests, tuning
 // runs) change it, and must not run while another call of the library is under way.
 #define GTM_SWITCHES(X) \
+    X(FIT_DEEP_CHUNK) \
     X(FIT_DEEP_CLAUSES_PER_GROUP) \
     X(FIT_DEEP_IN_MEMORY) \
+    X(FIT_DEEP_NO_DEAL) \
     X(FIT_DEEP_NO_MASKS) \
     X(FIT_DEEP_WINDOW_ROWS) \
     X(FIT_FACTOR_MIN) \
@@ -752,6 +754,8 @@ struct FitWs {
     uint32_t *coop_vec;                     // [depth - 1][max_nodes][M / 32] the same, node-major
     unsigned long long *coop_arrived;       // [depth - 1][FITD_PARTS * FITD_STRIDE]
     size_t coop_words;                      // words of coop_got
+    int *coop_perm;                         // [C + 2,048] which clause sits in which workgroup's slots (k_fit_deep_deal)
+    uint32_t *coop_cost;                    // [C]
     size_t bytes;
 };
 
@@ -785,6 +789,8 @@ FitWs carve_fit(const Dims &d, const gtm_config *cfg, char *base) {
     w.coop_got = cfg->depth > 1 ? (uint32_t *)take(w.coop_words * 4) : nullptr;
     w.coop_vec = cfg->depth > 1 ? (uint32_t *)take((size_t)(cfg->depth - 1) * cfg->max_nodes * d.MC * 2) : nullptr;
     w.coop_arrived = cfg->depth > 1 ? (unsigned long long *)take((size_t)(cfg->depth - 1) * FITD_PARTS * FITD_STRIDE * 8) : nullptr;
+    w.coop_perm = cfg->depth > 1 ? (int *)take(((size_t)d.C + 2048) * 4) : nullptr;
+    w.coop_cost = cfg->depth > 1 ? (uint32_t *)take((size_t)d.C * 4) : nullptr;
     w.bytes = off;
     return w;
 }
@@ -2177,10 +2183,14 @@ int fit_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
 // `_fit`'s inner loop of a model with message layers as one cooperative launch (fit_deep_persistent.h).
 // Returns GTM_OK with *done = false when this device or shape cannot run it, so that the caller
 // falls back to the launches per example.  GTM_NO_DEEP_PERSISTENT_FIT (tuning aid) turns it off.
+// With several clauses per workgroup the run is cut into launches of a few hundred to a few thousand examples
+// and the clauses are dealt out anew before each (k_fit_deep_deal); *examples_done says how far the run got
+// when a launch gave up (the model is then as it was before that launch).
 int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, const gtm_state *s, const TileGeom &tg,
                         const FitWs &w, const int32_t *encoded_Y, int first_example, int n_examples, uint64_t first_step,
-                        hipStream_t st, bool *done) {
+                        hipStream_t st, bool *done, int *examples_done) {
     *done = false;
+    *examples_done = 0;
     if (tune(T_NO_DEEP_PERSISTENT_FIT) || tune(T_NO_PERSISTENT_FIT) || cfg->depth < 2 || d.K > FITD_BLOCK) return GTM_OK;
     if (d.M % 32 != 0 || d.NC > 64) return GTM_OK;  // whole words of message bits; one lane per word of a truth row
     int dev = 0, coop = 0, cus = 0;
@@ -2306,59 +2316,97 @@ int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *
     p.edge_cap = edge_cap;
     p.edge_types = edge_types;
 
-    // the exchange buffers start at zero; the model is kept as it was in case the run gives up
-    hipLaunchKernelGGL(k_fill_u64, dim3(blocks_for((int64_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE + 1, TPB)), dim3(TPB), 0, st,
-                       (unsigned long long *)w.class_sum, (int64_t)0, 0ull, (int64_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE + 1);
-    if (int rc = check_launch("fill")) return rc;
-    hipLaunchKernelGGL(k_fill_u64, dim3(blocks_for((int64_t)layers * FITD_PARTS * FITD_STRIDE, TPB)), dim3(TPB), 0, st,
-                       w.coop_arrived, (int64_t)0, 0ull, (int64_t)layers * FITD_PARTS * FITD_STRIDE);
-    if (int rc = check_launch("fill")) return rc;
-    hipLaunchKernelGGL(k_fill_i32, dim3(blocks_for((int64_t)w.coop_words, TPB)), dim3(TPB), 0, st, (int32_t *)w.coop_got,
-                       (int64_t)w.coop_words, 0);
-    if (int rc = check_launch("fill")) return rc;
-    const size_t bank0_bytes = (size_t)d.C * d.LA * d.B * 4, bankm_bytes = (size_t)d.C * d.MC * d.B * 4;
-    const size_t weights_bytes = (size_t)d.K * d.C * 4;
-    hipError_t e = hipMemcpyAsync(w.bank_backup, s->ta_state, bank0_bytes, hipMemcpyDeviceToDevice, st);
-    for (int l = 0; l < layers && e == hipSuccess; ++l)
-        e = hipMemcpyAsync((char *)w.bank_backup + bank0_bytes + (size_t)l * bankm_bytes, s->message_ta_state[l], bankm_bytes,
-                           hipMemcpyDeviceToDevice, st);
-    if (e == hipSuccess) e = hipMemcpyAsync(w.weights_backup, s->clause_weights, weights_bytes, hipMemcpyDeviceToDevice, st);
-    if (e != hipSuccess) return fail(GTM_ERR_HIP, "keeping a copy of the model state: %s", hipGetErrorString(e));
+    // Several clauses per workgroup: the run in launches of 256, 512, ... 2,048 examples (early in training the
+    // clauses change fastest), the clauses dealt out by their cost before each.  GTM_FIT_DEEP_CHUNK = n (tests):
+    // launches of n examples; GTM_FIT_DEEP_NO_DEAL: one launch, clauses in order.
+    const bool deal = per_group >= 2 && per_group <= FITD_MAX_DEALT && d.C <= FITD_DEAL_MAX && w.coop_perm && w.coop_cost &&
+                      (size_t)groups * per_group <= (size_t)d.C + 2048 && !tune(T_FIT_DEEP_NO_DEAL);
+    int chunk = deal ? 256 : n_examples;
+    if (const char *e = tune(T_FIT_DEEP_CHUNK)) chunk = deal ? std::max(1, atoi(e)) : n_examples;
+    const bool chunk_grows = deal && !tune(T_FIT_DEEP_CHUNK);
+    static thread_local bool deal_lds_raised = false;
+    if (deal && !deal_lds_raised) {
+        if (hipFuncSetAttribute((const void *)k_fit_deep_deal, hipFuncAttributeMaxDynamicSharedMemorySize, FITD_DEAL_MAX * 8) !=
+            hipSuccess)
+            return fail(GTM_ERR_HIP, "raising the LDS limit of the dealing kernel");
+        deal_lds_raised = true;
+    }
+    for (int at = 0; at < n_examples;) {
+        const int n_now = std::min(chunk, n_examples - at);
+        p.first_example = first_example + at;
+        p.n_examples = n_now;
+        p.first_step = (uint32_t)(first_step + (uint64_t)at);
+        p.perm = nullptr;
+        if (deal) {
+            FitDeepBanks banks{};
+            for (int l = 0; l < cfg->depth; ++l) banks.bank[l] = p.bank[l];
+            hipLaunchKernelGGL(k_fit_deep_cost, dim3(blocks_for(d.C, TPB / 64)), dim3(TPB), 0, st, banks, cfg->depth, d.C, d.LA, d.MC,
+                               d.B, w.coop_cost);
+            if (int rc = check_launch("fit_deep_cost")) return rc;
+            int pow2 = 1;
+            while (pow2 < d.C) pow2 <<= 1;
+            hipLaunchKernelGGL(k_fit_deep_deal, dim3(1), dim3(1024), (size_t)pow2 * 8, st, w.coop_cost, d.C, groups, per_group,
+                               w.coop_perm);
+            if (int rc = check_launch("fit_deep_deal")) return rc;
+            p.perm = w.coop_perm;
+        }
+        // the exchange buffers start at zero; the model is kept as it was in case the run gives up
+        hipLaunchKernelGGL(k_fill_u64, dim3(blocks_for((int64_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE + 1, TPB)), dim3(TPB), 0, st,
+                           (unsigned long long *)w.class_sum, (int64_t)0, 0ull, (int64_t)d.K * 3 * FITP_SUM_PARTS * FITP_SUM_STRIDE + 1);
+        if (int rc = check_launch("fill")) return rc;
+        hipLaunchKernelGGL(k_fill_u64, dim3(blocks_for((int64_t)layers * FITD_PARTS * FITD_STRIDE, TPB)), dim3(TPB), 0, st,
+                           w.coop_arrived, (int64_t)0, 0ull, (int64_t)layers * FITD_PARTS * FITD_STRIDE);
+        if (int rc = check_launch("fill")) return rc;
+        hipLaunchKernelGGL(k_fill_i32, dim3(blocks_for((int64_t)w.coop_words, TPB)), dim3(TPB), 0, st, (int32_t *)w.coop_got,
+                           (int64_t)w.coop_words, 0);
+        if (int rc = check_launch("fill")) return rc;
+        const size_t bank0_bytes = (size_t)d.C * d.LA * d.B * 4, bankm_bytes = (size_t)d.C * d.MC * d.B * 4;
+        const size_t weights_bytes = (size_t)d.K * d.C * 4;
+        hipError_t e = hipMemcpyAsync(w.bank_backup, s->ta_state, bank0_bytes, hipMemcpyDeviceToDevice, st);
+        for (int l = 0; l < layers && e == hipSuccess; ++l)
+            e = hipMemcpyAsync((char *)w.bank_backup + bank0_bytes + (size_t)l * bankm_bytes, s->message_ta_state[l], bankm_bytes,
+                               hipMemcpyDeviceToDevice, st);
+        if (e == hipSuccess) e = hipMemcpyAsync(w.weights_backup, s->clause_weights, weights_bytes, hipMemcpyDeviceToDevice, st);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "keeping a copy of the model state: %s", hipGetErrorString(e));
 
 #ifdef FITD_CLOCKS
-    p.clocks = (unsigned long long *)w.bank_backup;  // (development builds only: an aborted run is not restored correctly)
+        p.clocks = (unsigned long long *)w.bank_backup;  // (development builds only: an aborted run is not restored correctly)
 #endif
-    void *args[] = {&p};
-    profile_start(big ? "k_fit_deep_persistent<in memory>" : "k_fit_deep_persistent", st);
-    e = hipLaunchCooperativeKernel(kernel, dim3(groups), dim3(FITD_BLOCK), args, (unsigned)lds, st);
-    if (e != hipSuccess) return fail(GTM_ERR_HIP, "cooperative launch of the training kernel: %s", hipGetErrorString(e));
-    profile_stop(st);
-    uint32_t flag = 0;
-    e = hipMemcpyAsync(&flag, p.abort_flag, 4, hipMemcpyDeviceToHost, st);
-    if (e == hipSuccess) e = hipStreamSynchronize(st);
-    if (e != hipSuccess) return fail(GTM_ERR_HIP, "training kernel: %s", hipGetErrorString(e));
-#ifdef FITD_CLOCKS
-    {
-        unsigned long long clk[16];
-        (void)hipMemcpy(clk, w.bank_backup, sizeof(clk), hipMemcpyDeviceToHost);
-        fprintf(stderr, "fitd clocks (us per example, %d groups):", groups);
-        for (int k = 0; k < 13; ++k) fprintf(stderr, " %d:%.2f", k, clk[k] * 0.01 / n_examples);
-        fprintf(stderr, "\n");
-    }
-#endif
-    if (flag != 0) {
-        e = hipMemcpyAsync(s->ta_state, w.bank_backup, bank0_bytes, hipMemcpyDeviceToDevice, st);
-        for (int l = 0; l < layers && e == hipSuccess; ++l)
-            e = hipMemcpyAsync(s->message_ta_state[l], (char *)w.bank_backup + bank0_bytes + (size_t)l * bankm_bytes, bankm_bytes,
-                               hipMemcpyDeviceToDevice, st);
-        if (e == hipSuccess) e = hipMemcpyAsync(s->clause_weights, w.weights_backup, weights_bytes, hipMemcpyDeviceToDevice, st);
+        void *args[] = {&p};
+        profile_start(big ? "k_fit_deep_persistent<in memory>" : "k_fit_deep_persistent", st);
+        e = hipLaunchCooperativeKernel(kernel, dim3(groups), dim3(FITD_BLOCK), args, (unsigned)lds, st);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "cooperative launch of the training kernel: %s", hipGetErrorString(e));
+        profile_stop(st);
+        uint32_t flag = 0;
+        e = hipMemcpyAsync(&flag, p.abort_flag, 4, hipMemcpyDeviceToHost, st);
         if (e == hipSuccess) e = hipStreamSynchronize(st);
-        if (e != hipSuccess)
-            return fail(GTM_ERR_HIP, "training kernel gave up waiting at a device-wide barrier (%d workgroups) and the "
-                                     "model state could not be restored: %s", groups, hipGetErrorString(e));
-        if (!p.force_abort) return GTM_OK;  // as in fit_persistent: the launches per example take over
-        return fail(GTM_ERR_HIP, "training kernel gave up waiting at a device-wide barrier (%d workgroups); "
-                                 "the model state is as it was before the call", groups);
+        if (e != hipSuccess) return fail(GTM_ERR_HIP, "training kernel: %s", hipGetErrorString(e));
+#ifdef FITD_CLOCKS
+        {
+            unsigned long long clk[16];
+            (void)hipMemcpy(clk, w.bank_backup, sizeof(clk), hipMemcpyDeviceToHost);
+            fprintf(stderr, "fitd clocks (us per example, %d groups):", groups);
+            for (int k = 0; k < 13; ++k) fprintf(stderr, " %d:%.2f", k, clk[k] * 0.01 / n_examples);
+            fprintf(stderr, "\n");
+        }
+#endif
+        if (flag != 0) {
+            e = hipMemcpyAsync(s->ta_state, w.bank_backup, bank0_bytes, hipMemcpyDeviceToDevice, st);
+            for (int l = 0; l < layers && e == hipSuccess; ++l)
+                e = hipMemcpyAsync(s->message_ta_state[l], (char *)w.bank_backup + bank0_bytes + (size_t)l * bankm_bytes, bankm_bytes,
+                                   hipMemcpyDeviceToDevice, st);
+            if (e == hipSuccess) e = hipMemcpyAsync(s->clause_weights, w.weights_backup, weights_bytes, hipMemcpyDeviceToDevice, st);
+            if (e == hipSuccess) e = hipStreamSynchronize(st);
+            if (e != hipSuccess)
+                return fail(GTM_ERR_HIP, "training kernel gave up waiting at a device-wide barrier (%d workgroups) and the "
+                                         "model state could not be restored: %s", groups, hipGetErrorString(e));
+            if (!p.force_abort) return GTM_OK;  // as in fit_persistent: the launches per example take over
+            return fail(GTM_ERR_HIP, "training kernel gave up waiting at a device-wide barrier (%d workgroups); "
+                                     "the model state is as it was before the call", groups);
+        }
+        at += n_now;
+        *examples_done = at;
+        if (chunk_grows && chunk < 2048) chunk *= 2;
     }
     *done = true;
     return GTM_OK;
@@ -2696,10 +2744,12 @@ int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *st
         TileGeom tg = geometry_for(cfg, graphs, d.K);
         if (tg.ok && tg.slot_words <= 64 && cfg->max_nodes <= 2048) {  // one lane per word of the graph's nodes
             bool done = false;
+            int so_far = 0;  // examples that launches which did not give up have trained on
             if (int rc = fit_deep_persistent(d, cfg, graphs, state, tg, w, encoded_Y, first_example, n_examples, first_step, st,
-                                             &done))
+                                             &done, &so_far))
                 return rc;
             if (done) return GTM_OK;
+            first_example += so_far, n_examples -= so_far, first_step += (uint64_t)so_far, h_n += so_far, h_base += so_far;
         }
         if (tg.ok && tg.slot_words <= 64 && cfg->max_nodes <= 2048)
             return fit_deep_on_tiles(d, cfg, graphs, state, tg, w, encoded_Y, first_example, n_examples, first_step, h_n,

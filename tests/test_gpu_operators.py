@@ -424,7 +424,8 @@ ONE_LAUNCH_DEEP_SHAPES = [
 @pytest.mark.parametrize("shape", ONE_LAUNCH_DEEP_SHAPES, ids=lambda s: "deep%d" % s["seed"])
 @pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 9, 5), (1, None, 12)])
 @pytest.mark.parametrize("layout", ["in-lds", "in-lds-40-clauses-per-workgroup", "in-memory", "in-memory-32-row-windows",
-                                    "in-memory-40-clauses-per-workgroup"])
+                                    "in-memory-40-clauses-per-workgroup", "in-memory-dealt-anew-every-3-examples",
+                                    "in-lds-dealt-anew-every-5-examples", "in-memory-clauses-in-order"])
 def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bits, layout, tune):
     """A run of training examples of a model with message layers in one cooperative launch
     (k_fit_deep_persistent: clauses spread over workgroups, the nodes' messages and the class sums
@@ -433,7 +434,9 @@ def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bi
     through memory and the restart of the exchange buffers are covered.  Both layouts: automata
     and all rows in LDS; automata in memory with the received rows passing through LDS in windows
     (as wide as fits, and 32 rows wide, so that every layer takes several).  With 40 clauses per
-    workgroup what the clauses send is worked out 32 clauses at a time, in two passes."""
+    workgroup what the clauses send is worked out 32 clauses at a time, in two passes.  With several clauses per
+    workgroup the clauses are dealt out to the workgroups by their number of literals before every launch; a run is
+    then cut into several launches (here: of 3 or 5 examples), or the clauses stay in order."""
     import ctypes
     from tests.gpu_harness import Device
     from graphtsetlinmachine_amd import _abi
@@ -445,6 +448,12 @@ def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bi
         tune("GTM_FIT_DEEP_WINDOW_ROWS", "32")
     if layout.endswith("40-clauses-per-workgroup"):
         tune("GTM_FIT_DEEP_CLAUSES_PER_GROUP", "40")
+    if "dealt-anew" in layout:
+        tune("GTM_FIT_DEEP_CLAUSES_PER_GROUP", "7")
+        tune("GTM_FIT_DEEP_CHUNK", "3" if "every-3" in layout else "5")
+    if layout.endswith("clauses-in-order"):
+        tune("GTM_FIT_DEEP_CLAUSES_PER_GROUP", "7")
+        tune("GTM_FIT_DEEP_NO_DEAL", "1")
     kernel = b"k_fit_deep_persistent<in memory>" if layout.startswith("in-memory") else b"k_fit_deep_persistent"
     graphs = helpers.random_graphs(shape["seed"], **shape["g"])
     m = dict(shape["m"])
@@ -466,7 +475,9 @@ def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bi
         dev.fit(Y, G // 3, G - G // 3, epoch * G + G // 3)
         _abi.call("gtm_profile_read", ctypes.byref(name), ctypes.byref(launches), ctypes.byref(total))
         _abi.call("gtm_profile_enable", 0)
-        assert (name.value, launches.value) == (kernel, 2), "the one-launch kernel should have run"
+        chunk = 3 if "every-3" in layout else 5 if "every-5" in layout else G
+        expected = -(-(G // 3) // chunk) + -(-(G - G // 3) // chunk)  # launches of the two calls
+        assert (name.value, launches.value) == (kernel, expected), "the one-launch kernel should have run"
         ta, banks, w = dev.download()
         assert np.array_equal(w, model.clause_weights), "weights after epoch %d" % epoch
         assert np.array_equal(ta, model.ta_state), "layer-0 automata after epoch %d" % epoch
