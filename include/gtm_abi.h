@@ -218,10 +218,15 @@ size_t gtm_fit_workspace_bytes(const gtm_config *cfg, const gtm_graphs *graphs);
  * step first_step + i for its random draws.  With depth == 1 and
  * graphs->tiles set the whole run is one cooperative launch in which each
  * workgroup keeps its clauses' automata in LDS and the class sums are the
- * only exchange between workgroups.  Its waits are bounded (5 s of the device's
- * wall clock): if one runs out, the model is put back as it was before the
- * launch and the examples are trained by launches per example instead, which
- * wait for nobody - same results, the call still returns GTM_OK. */
+ * only exchange between workgroups.  Models with message layers whose
+ * MESSAGE_SIZE is a multiple of 32 run the same way, with one more exchange
+ * per layer; when a workgroup owns several clauses the run is a few such
+ * launches, of 256 to 2,048 examples, and the clauses are shared out among the
+ * workgroups anew before each.  The waits are bounded (5 s of the device's
+ * wall clock): if one runs out, the model is put back as it was before that
+ * launch and the remaining examples are trained by launches per example
+ * instead, which wait for nobody - same results, the call still returns
+ * GTM_OK. */
 int gtm_fit(const gtm_config *cfg, const gtm_graphs *graphs, const gtm_state *state, const int32_t *encoded_Y,
             int32_t first_example, int32_t n_examples, uint64_t first_step, void *workspace,
             size_t workspace_bytes, void *stream);
