@@ -115,7 +115,7 @@ inline size_t fit_deep_lds_words(bool big, int depth, int literals, int per_grou
     return 2 * ((size_t)rows_words + 2 * (size_t)max_nodes + (size_t)edge_cap + (size_t)K) + (size_t)window_rows * NW +
            (size_t)per_group * edge_types * NW + (size_t)per_group * per_clause * (big ? 1 : B) + 2 * (size_t)per_group * K +
            2 * (size_t)per_group + (size_t)per_group * NW + 2 * (size_t)K + 6 * (size_t)K +
-           (big ? (size_t)literals : (size_t)per_group * (depth - 1) * MC) + (size_t)per_group * MB + 64;
+           (big ? (size_t)literals : (size_t)per_group * (depth - 1) * MC) + (size_t)per_group * MB + (size_t)per_group + 64;
 }
 
 // What the cooperative kernel has to know about the edges of a run of examples: [0] most edges of
@@ -241,7 +241,6 @@ __device__ __forceinline__ void fitd_and_rows(const uint32_t *inc, int inc_strid
 // run of examples the clauses are therefore sorted by the number of literals they include in all banks - what
 // a clause's evaluation and feedback walk - and dealt out in rounds, back and forth over the workgroups, so
 // that every workgroup gets the same mix.  Nothing moves: the table says which clause sits in which slot.
-constexpr int FITD_MAX_DEALT = 64;     // clauses per workgroup that the table can hold
 constexpr int FITD_DEAL_MAX = 8192;    // clauses that one workgroup sorts in LDS
 
 struct FitDeepBanks {
@@ -303,21 +302,6 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
     constexpr int WAVES = FITD_BLOCK / 64;
     const int G = (int)gridDim.x, g = (int)blockIdx.x;
     const int own_max = p.clauses_per_group;
-    // The workgroup's clauses: `own_max` slots, the first n_own of them taken - clauses g * own_max .. in order, or
-    // what the table says (clauses dealt out by what they cost, k_fit_deep_deal below).  Everything that is
-    // indexed by clause - automata, weights, hypervector bits, node types, random numbers - goes by own_id.
-    __shared__ int own_id[FITD_MAX_DEALT];
-    __shared__ int n_own_shared;
-    if (tid == 0) {
-        int n = 0;
-        for (int cl = 0; cl < own_max; ++cl) {
-            const int c = p.perm ? p.perm[g * own_max + cl] : (g * own_max + cl < p.C ? g * own_max + cl : -1);
-            if (c >= 0 && cl < FITD_MAX_DEALT) own_id[n++] = c;
-        }
-        n_own_shared = n;
-    }
-    __syncthreads();
-    const int n_own = n_own_shared;
     const int LA = p.LA, MC = p.MC, MW = p.MW, M = p.M, B = p.B, K = p.K, NW = p.NW, L = p.depth - 1, TE = p.edge_types;
     const int WR = p.window_rows;
     const int per_clause = LA + L * MC;  // automaton words of a clause over all banks
@@ -343,6 +327,21 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
     uint32_t *hv_own = seen + 6 * K;                              // [own][MB] hypervector bits of the own clauses
     uint32_t *mlit = hv_own + (size_t)own_max * p.MB;             // [own][L][MC] message literal words of the picked node (not BIG)
     uint32_t *order = mlit;                                       // [literals] the literals, the ones that seldom hold first (BIG)
+    // The workgroup's clauses: `own_max` slots, the first n_own of them taken - clauses g * own_max .. in order, or
+    // what the table says (clauses dealt out by what they cost, k_fit_deep_deal below).  Everything that is
+    // indexed by clause - automata, weights, hypervector bits, node types, random numbers - goes by own_id.
+    int *own_id = (int *)(mlit + (BIG ? (size_t)p.literals : (size_t)own_max * L * MC));  // [own]
+    __shared__ int n_own_shared;
+    if (tid == 0) {
+        int n = 0;
+        for (int cl = 0; cl < own_max; ++cl) {
+            const int c = p.perm ? p.perm[g * own_max + cl] : (g * own_max + cl < p.C ? g * own_max + cl : -1);
+            if (c >= 0) own_id[n++] = c;
+        }
+        n_own_shared = n;
+    }
+    __syncthreads();
+    const int n_own = n_own_shared;
     __shared__ int go_on;
     __shared__ int next_unit[2];  // waves take their units of work (a clause, or some words of one) from here: [0] layer 0, [1] a message layer
 

@@ -2319,7 +2319,7 @@ int fit_deep_persistent(const Dims &d, const gtm_config *cfg, const gtm_graphs *
     // Several clauses per workgroup: the run in launches of 256, 512, ... 2,048 examples (early in training the
     // clauses change fastest), the clauses dealt out by their cost before each.  GTM_FIT_DEEP_CHUNK = n (tests):
     // launches of n examples; GTM_FIT_DEEP_NO_DEAL: one launch, clauses in order.
-    const bool deal = per_group >= 2 && per_group <= FITD_MAX_DEALT && d.C <= FITD_DEAL_MAX && w.coop_perm && w.coop_cost &&
+    const bool deal = per_group >= 2 && d.C <= FITD_DEAL_MAX && w.coop_perm && w.coop_cost &&
                       (size_t)groups * per_group <= (size_t)d.C + 2048 && !tune(T_FIT_DEEP_NO_DEAL);
     int chunk = deal ? 256 : n_examples;
     if (const char *e = tune(T_FIT_DEEP_CHUNK)) chunk = deal ? std::max(1, atoi(e)) : n_examples;

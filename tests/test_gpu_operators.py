@@ -425,7 +425,8 @@ ONE_LAUNCH_DEEP_SHAPES = [
 @pytest.mark.parametrize("boost,max_included,state_bits", [(1, None, 8), (0, 9, 5), (1, None, 12)])
 @pytest.mark.parametrize("layout", ["in-lds", "in-lds-40-clauses-per-workgroup", "in-memory", "in-memory-32-row-windows",
                                     "in-memory-40-clauses-per-workgroup", "in-memory-dealt-anew-every-3-examples",
-                                    "in-lds-dealt-anew-every-5-examples", "in-memory-clauses-in-order"])
+                                    "in-lds-dealt-anew-every-5-examples", "in-memory-clauses-in-order",
+                                    "in-memory-70-clauses-per-workgroup"])
 def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bits, layout, tune):
     """A run of training examples of a model with message layers in one cooperative launch
     (k_fit_deep_persistent: clauses spread over workgroups, the nodes' messages and the class sums
@@ -448,6 +449,8 @@ def test_one_launch_fit_with_message_layers(shape, boost, max_included, state_bi
         tune("GTM_FIT_DEEP_WINDOW_ROWS", "32")
     if layout.endswith("40-clauses-per-workgroup"):
         tune("GTM_FIT_DEEP_CLAUSES_PER_GROUP", "40")
+    if layout.endswith("70-clauses-per-workgroup"):
+        tune("GTM_FIT_DEEP_CLAUSES_PER_GROUP", "70")
     if "dealt-anew" in layout:
         tune("GTM_FIT_DEEP_CLAUSES_PER_GROUP", "7")
         tune("GTM_FIT_DEEP_CHUNK", "3" if "every-3" in layout else "5")
