@@ -877,6 +877,8 @@ HALF_TILE_SHAPES = [
     # more (graph, class) pairs per tile than four per lane
     dict(seed=56, g=dict(n_graphs=30, max_nodes=361, min_nodes=200, hv_size=128, n_symbols=20, max_degree=0), classes=70,
          clauses=50),
+    # so few clauses that the launch which compiles them has fewer workgroups than the tiles have shares
+    dict(seed=57, g=dict(n_graphs=50, max_nodes=361, min_nodes=250, hv_size=128, max_degree=0), classes=5, clauses=12),
 ]
 
 
