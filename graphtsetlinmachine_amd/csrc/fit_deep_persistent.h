@@ -115,7 +115,8 @@ inline size_t fit_deep_lds_words(bool big, int depth, int literals, int per_grou
     return 2 * ((size_t)rows_words + 2 * (size_t)max_nodes + (size_t)edge_cap + (size_t)K) + (size_t)window_rows * NW +
            (size_t)per_group * edge_types * NW + (size_t)per_group * per_clause * (big ? 1 : B) + 2 * (size_t)per_group * K +
            2 * (size_t)per_group + (size_t)per_group * NW + 2 * (size_t)K + 6 * (size_t)K +
-           (big ? (size_t)literals : (size_t)per_group * (depth - 1) * MC) + (size_t)per_group * MB + (size_t)per_group + 64;
+           (big ? (size_t)literals : (size_t)per_group * (depth - 1) * MC) + (size_t)per_group * MB + (size_t)per_group +
+           (big ? (size_t)(FITD_BLOCK / 64) * FIT_QUEUE : 0) + 64;
 }
 
 // What the cooperative kernel has to know about the edges of a run of examples: [0] most edges of
@@ -196,8 +197,9 @@ __device__ __forceinline__ uint32_t fitd_transpose32(uint32_t a, int lane) {
 // most 32 words then) - and adds how many they hold to *included (an LDS counter).  `inc` points at the include
 // plane's word 0 (words inc_stride apart); row r of the literal rows is at col[(r - row_base) * stride] for this
 // lane; literals >= `half` are negated: the complement of row (literal - half) when `complement`, else a row of
-// their own.  One wave.
-template <typename Rows>
+// their own.  One wave.  PACKED: a batch of row reads takes literals from as many include words as it needs (for
+// clauses whose include words hold one or two literals each); else a word's literals, eight at a time.
+template <bool PACKED, typename Rows>
 __device__ __forceinline__ void fitd_and_rows(const uint32_t *inc, int inc_stride, int w_lo, int w_hi, int twin, int last_word,
                                               uint32_t filter, Rows col, int stride, int row_base, int half, bool complement,
                                               int ones_row, uint32_t &acc, int *included, int lane) {
@@ -209,26 +211,62 @@ __device__ __forceinline__ void fitd_and_rows(const uint32_t *inc, int inc_strid
         if (mine_is == last_word) mine &= filter;
         if (mine != 0u) atomicAdd(included, __popc(mine));
         unsigned long long nonzero = __ballot(mine != 0);
-        while (nonzero) {
-            if (__ballot(acc != 0u) == 0ull) break;  // false everywhere stays false: only the count matters
-            const int wl = __ffsll((long long)nonzero) - 1;
-            nonzero &= nonzero - 1;
-            uint32_t m = __builtin_amdgcn_readlane(mine, wl);
-            const int first = (wl < span ? w0 + wl : twin + w0 + wl - span) << 5;
-            const bool negated = complement && first >= half;  // (a word holds positive or negated literals, never both)
-            const int row0 = (negated ? first - half : first) - row_base;
-            const uint32_t flip = negated ? 0xFFFFFFFFu : 0u;
-            while (m) {
+        if constexpr (PACKED) {
+            // The set bits of the held words, word after word, eight rows per batch of reads whatever words they
+            // come from: with a batch per word, a clause of a hundred literals in 64 words read eight rows for every
+            // one or two that it wanted.  (All of this is the same for every lane: scalar state.)
+            uint32_t m = 0u, flip = 0u;
+            int row0 = 0;
+            auto next_word = [&]() {  // on to the next word that holds literals; false: none is left
+                if (!nonzero) return false;
+                const int wl = __ffsll((long long)nonzero) - 1;
+                nonzero &= nonzero - 1;
+                m = __builtin_amdgcn_readlane(mine, wl);
+                const int first = (wl < span ? w0 + wl : twin + w0 + wl - span) << 5;
+                const bool negated = complement && first >= half;  // (a word holds positive or negated literals, never both)
+                row0 = (negated ? first - half : first) - row_base;
+                flip = negated ? 0xFFFFFFFFu : 0u;
+                return true;
+            };
+            bool more = next_word();
+            while (more) {
+                if (__ballot(acc != 0u) == 0ull) break;  // false everywhere stays false: only the count matters
                 uint32_t r[8];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
-                    const bool used = m != 0;
+                    const bool used = more;
                     const int row = used ? row0 + __builtin_ctz(m) : ones_row - row_base;
-                    m &= m - 1;
-                    r[u] = (col[(int64_t)row * stride] ^ flip) | (used ? 0u : 0xFFFFFFFFu);
+                    r[u] = (col[(int64_t)row * stride] ^ (used ? flip : 0u)) | (used ? 0u : 0xFFFFFFFFu);
+                    if (used) {
+                        m &= m - 1;
+                        if (m == 0u) more = next_word();
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < 8; ++u) acc &= r[u];
+            }
+        } else {
+            while (nonzero) {
+                if (__ballot(acc != 0u) == 0ull) break;  // false everywhere stays false: only the count matters
+                const int wl = __ffsll((long long)nonzero) - 1;
+                nonzero &= nonzero - 1;
+                uint32_t m = __builtin_amdgcn_readlane(mine, wl);
+                const int first = (wl < span ? w0 + wl : twin + w0 + wl - span) << 5;
+                const bool negated = complement && first >= half;  // (a word holds positive or negated literals, never both)
+                const int row0 = (negated ? first - half : first) - row_base;
+                const uint32_t flip = negated ? 0xFFFFFFFFu : 0u;
+                while (m) {
+                    uint32_t r[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const bool used = m != 0;
+                        const int row = used ? row0 + __builtin_ctz(m) : ones_row - row_base;
+                        m &= m - 1;
+                        r[u] = (col[(int64_t)row * stride] ^ flip) | (used ? 0u : 0xFFFFFFFFu);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc &= r[u];
+                }
             }
         }
     }
@@ -331,6 +369,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
     // what the table says (clauses dealt out by what they cost, k_fit_deep_deal below).  Everything that is
     // indexed by clause - automata, weights, hypervector bits, node types, random numbers - goes by own_id.
     int *own_id = (int *)(mlit + (BIG ? (size_t)p.literals : (size_t)own_max * L * MC));  // [own]
+    uint32_t *queue_of_wave = (uint32_t *)(own_id + own_max);  // [waves][FIT_QUEUE] included literals waiting for their rows (BIG)
     __shared__ int n_own_shared;
     if (tid == 0) {
         int n = 0;
@@ -449,7 +488,8 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                 int included;
                 const uint32_t v = fit_clause_truth(ta + (size_t)cl * per_clause, 1, LA, p.filter, tile + (active ? lane : 0), row_stride,
                                                     p.literals, p.literals + own_id[cl] % p.n_types, ones_row, fg, n, FIT_WALK_ALL,
-                                                    p.X + base * LA, order, active, lane, &included);
+                                                    p.X + base * LA, order, active, lane, &included,
+                                                    queue_of_wave + wave * FIT_QUEUE);
                 if (lane < NW) truth[cl * NW + lane] = v;
                 if (lane == 0) incl_of[cl] = included;
             }
@@ -467,7 +507,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                 const int cl = u / parts0, part = u - cl * parts0;
                 uint32_t acc = active ? truth[cl * NW + lane] : 0u;
                 const uint32_t before = acc;
-                fitd_and_rows(ta + (size_t)cl * per_clause * SB + (SB - 1), SB, part * chunk0, min(LA, (part + 1) * chunk0), -1,
+                fitd_and_rows<false>(ta + (size_t)cl * per_clause * SB + (SB - 1), SB, part * chunk0, min(LA, (part + 1) * chunk0), -1,
                               LA - 1, p.filter, (const uint32_t *)rows0 + (active ? lane : 0), row_stride, 0, 0, false, ones_row, acc,
                               &incl_of[cl], lane);
                 if (active && acc != before) atomicAnd(&truth[cl * NW + lane], acc);
@@ -605,7 +645,7 @@ __global__ __launch_bounds__(FITD_BLOCK) void k_fit_deep_persistent(FitDeepParam
                         const int lo = w_first + part * chunk1, hi = min(w_first + window_words, lo + chunk1);
                         // (2 M is a multiple of 32: the last word has no tail to mask) the words of the positive literals and,
                         // in the same pass, those of the negated ones (MW words further on)
-                        fitd_and_rows(inc, SB, lo, hi, MW, -1, 0u, col, NW, r0, M, true, r0, acc, &incl_of[cl], lane);
+                        fitd_and_rows<BIG>(inc, SB, lo, hi, MW, -1, 0u, col, NW, r0, M, true, r0, acc, &incl_of[cl], lane);
                         if (active && acc != before) atomicAnd(&truth[cl * NW + lane], acc);
                     }
                 }

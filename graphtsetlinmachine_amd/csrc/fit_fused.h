@@ -31,6 +31,7 @@ constexpr int FIT_WALK_ALL = 40;      // clauses with at most this many literals
 constexpr int FIT_WALK_ALL_LDS = 512; // the same with the rows staged in LDS
 constexpr int FIT_FILTER_ROWS = 16;  // rows the others AND before testing nodes
 constexpr int FIT_FEW_NODES = 2;    // up to this many surviving nodes (estimate) are tested one by one, more are filtered further
+constexpr int FIT_QUEUE = 128;     // words of LDS per wave: included literals found in `order`, waiting for a batch of row reads
 
 struct FitGraph {
     int tile;        // tile holding the graph
@@ -123,7 +124,7 @@ __device__ __forceinline__ uint32_t fit_clause_truth(const uint32_t *inc, int in
                                                      const uint32_t *col, int stride, int literals, int type_row, int ones_row,
                                                      const FitGraph &fg, int n_nodes, int walk_all,
                                                      const uint32_t *__restrict__ X_rows, const uint32_t *__restrict__ order,
-                                                     bool active, int lane, int *included_out) {
+                                                     bool active, int lane, int *included_out, uint32_t *queue = nullptr) {
     // lane w fetches include word w0 + w: one memory latency for up to 64 words
     auto include_words = [&](int w0) {
         uint32_t mine = w0 + lane < LA ? inc[(int64_t)(w0 + lane) * inc_stride] : 0u;
@@ -148,10 +149,14 @@ __device__ __forceinline__ uint32_t fit_clause_truth(const uint32_t *inc, int in
         // trip of row reads removes most of them, testing them costs a round trip per word of nodes.
         // A clause that still holds at many nodes after 32 rows is not one that a few rows decide:
         // it takes all its rows, and stops early only when no node is left.
+        // With `queue` (FIT_QUEUE words of LDS of this wave's own) the included literals found in `order` wait
+        // there until 16 are together: a clause of 70 of 2,048 literals finds two per 64 places of `order`, and a
+        // batch of row reads per 64 places would be 32 memory round trips of 2 rows instead of 5 of 16.
         int budget = FIT_FILTER_ROWS, applied = 0;
         int r0 = 0;
         unsigned long long picked = 0ull;  // lanes whose literal (in `order`) is included and not applied yet
         uint32_t lit = 0u;
+        int head = 0, tail = 0;  // with `queue`: its entries [head, tail), places counted modulo FIT_QUEUE
         for (;;) {
             if (budget <= 0) {
                 const int mine = active ? __popc((acc >> fg.shift) & fg.mask) : 0;
@@ -159,24 +164,51 @@ __device__ __forceinline__ uint32_t fit_clause_truth(const uint32_t *inc, int in
                 if (left <= FIT_FEW_NODES) break;
                 budget = applied >= 32 ? 0x7FFFFFFF : 16;
             }
-            if (picked == 0ull) {
-                if (r0 >= literals) {
+            int row[16];
+            if (queue) {
+                while (tail - head < 16 && r0 < literals) {
+                    const int r = r0 + lane;
+                    lit = r < literals ? order[r] : 0u;
+                    uint32_t word = inc[(int64_t)(lit >> 5) * inc_stride];
+                    if ((int)(lit >> 5) == LA - 1) word &= filter;
+                    const bool mine = r < literals && ((word >> (lit & 31u)) & 1u);
+                    picked = __ballot(mine);
+                    if (mine) queue[(tail + __popcll(picked & ((1ull << lane) - 1ull))) & (FIT_QUEUE - 1)] = lit;
+                    tail += __popcll(picked);
+                    r0 += 64;
+                }
+                if (tail == head) {
                     all_rows = true;
                     break;
                 }
-                const int r = r0 + lane;
-                lit = r < literals ? order[r] : 0u;
-                uint32_t word = inc[(int64_t)(lit >> 5) * inc_stride];
-                if ((int)(lit >> 5) == LA - 1) word &= filter;
-                picked = __ballot(r < literals && ((word >> (lit & 31u)) & 1u));
-                r0 += 64;
-                continue;
-            }
-            int row[16];
+                // (a wave's LDS accesses are carried out in order: the reads below see what was just written)
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+                const int n = tail - head < 16 ? tail - head : 16;
 #pragma unroll
-            for (int u = 0; u < 16; ++u) {
-                row[u] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
-                picked &= picked - 1;
+                for (int u = 0; u < 16; ++u)
+                    row[u] = u < n ? __builtin_amdgcn_readfirstlane((int)queue[(head + u) & (FIT_QUEUE - 1)]) : ones_row;
+                head += n;
+            } else {
+                if (picked == 0ull) {
+                    if (r0 >= literals) {
+                        all_rows = true;
+                        break;
+                    }
+                    const int r = r0 + lane;
+                    lit = r < literals ? order[r] : 0u;
+                    uint32_t word = inc[(int64_t)(lit >> 5) * inc_stride];
+                    if ((int)(lit >> 5) == LA - 1) word &= filter;
+                    picked = __ballot(r < literals && ((word >> (lit & 31u)) & 1u));
+                    r0 += 64;
+                    continue;
+                }
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    row[u] = picked ? (int)__builtin_amdgcn_readlane(lit, __ffsll((long long)picked) - 1) : ones_row;
+                    picked &= picked - 1;
+                }
             }
             uint32_t r16[16];
 #pragma unroll
@@ -190,29 +222,41 @@ __device__ __forceinline__ uint32_t fit_clause_truth(const uint32_t *inc, int in
             }
         }
     } else {
+        // The literals in the order of the include words, 16 rows per batch of reads whatever words they come from (a
+        // clause of 30 literals has them in 25 of its 64 words: a batch per word would be 25 memory round trips of
+        // one or two rows).  Scalar state: the word at hand, what is left of it, the words still to come.
         int budget = filter_only ? FIT_FILTER_ROWS : 0x7FFFFFFF;
         for (int w0 = 0; w0 < LA && budget > 0; w0 += 64) {
             const uint32_t mine = w0 == 0 ? first_words : include_words(w0);
             unsigned long long nonzero = __ballot(mine != 0);
-            while (nonzero && budget > 0) {
+            uint32_t m = 0u;
+            int base = 0;
+            auto next_word = [&]() {  // on to the next word that holds literals; false: none is left
+                if (!nonzero) return false;
                 const int wl = __ffsll((long long)nonzero) - 1;
                 nonzero &= nonzero - 1;
-                uint32_t m = __builtin_amdgcn_readlane(mine, wl);
-                const int base = (w0 + wl) << 5;
-                while (m && budget > 0) {
-                    int row[8];
+                m = __builtin_amdgcn_readlane(mine, wl);
+                base = (w0 + wl) << 5;
+                return true;
+            };
+            bool more = next_word();
+            while (more && budget > 0) {
+                int row[16];
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) {
-                        row[u] = m ? base + __builtin_ctz(m) : ones_row;
+                for (int u = 0; u < 16; ++u) {
+                    const bool used = more;
+                    row[u] = used ? base + __builtin_ctz(m) : ones_row;
+                    if (used) {
                         m &= m - 1;
+                        if (m == 0u) more = next_word();
                     }
-                    uint32_t r[8];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) r[u] = col[(int64_t)row[u] * stride];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) acc &= r[u];
-                    budget -= 8;
                 }
+                uint32_t r[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) r[u] = col[(int64_t)row[u] * stride];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) acc &= r[u];
+                budget -= 16;
             }
         }
     }
@@ -304,12 +348,14 @@ __global__ __launch_bounds__(FIT_EVAL_BLOCK) void k_fit_eval(
 
     const bool active = lane < fg.words;
     const uint32_t *col = rows + (active ? lane : 0);
+    __shared__ uint32_t queue_of_wave[WAVES][FIT_QUEUE];
     int partial = 0;  // lane k < K: this wave's contribution to class k
     for (int c = blockIdx.x * WAVES + wave; c < C; c += gridDim.x * WAVES) {
         int included;
         const uint32_t v = fit_clause_truth(bank + (int64_t)c * LA * B + (B - 1), B, LA, filter, col, stride, literals,
                                             literals + c % n_types, ones_row, fg, n_nodes,
-                                            STAGE ? FIT_WALK_ALL_LDS : FIT_WALK_ALL, X_rows, order, active, lane, &included);
+                                            STAGE ? FIT_WALK_ALL_LDS : FIT_WALK_ALL, X_rows, order, active, lane, &included,
+                                            queue_of_wave[wave]);
         if (lane == 0) n_incl[c] = included;
         fit_clause_tail(v, lane, fg.words, NC, n_nodes, c, C, K, weights, k0, k1, step, finish != 0,
                         bitmap + (int64_t)c * NC, clause_node, class_sum, &partial);
