@@ -893,11 +893,11 @@ int max_lane_words() {
 
 // Half tiles (positive rows only in LDS, k_tile_two_phase_half): a depth-1 model on a data set that
 // the caller has declared complementary, with word-aligned halves of 4 to 16 literal words per node.
-// GTM_NO_HALF_TILES (tuning aid) turns them off.
+// GTM_NO_HALF_TILES (tuning aid) turns them off.  (The kernel reads the weights at 32-bit byte offsets.)
 bool half_tiles_allowed(const gtm_config *cfg, const gtm_graphs *g) {
     const int LA = (cfg->literals - 1) / 32 + 1;
     return cfg->depth == 1 && (g->flags & GTM_GRAPHS_COMPLEMENTARY) && cfg->literals % 64 == 0 && LA % 4 == 0 &&
-           LA <= 16 && !tune(T_NO_HALF_TILES) && !tune(T_NO_TWO_PHASE);
+           LA <= 16 && (int64_t)cfg->clauses * cfg->classes < (1 << 28) && !tune(T_NO_HALF_TILES) && !tune(T_NO_TWO_PHASE);
 }
 
 TileGeom geometry_for(const gtm_config *cfg, const gtm_graphs *g, int classes) {

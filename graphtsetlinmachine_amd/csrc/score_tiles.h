@@ -1781,6 +1781,20 @@ struct alignas(16) Entries16 {
     uint32_t v[16];
 };
 
+// Index of the lowest set bit, ~0 for 0: what the instruction gives by itself (the compiler's count of trailing
+// zeros is either undefined for 0 or comes with a comparison and a select for it).
+__device__ __forceinline__ uint32_t lowest_bit_or_ones(uint32_t x) {
+    uint32_t r;
+    asm("v_ffbl_b32 %0, %1" : "=v"(r) : "v"(x));
+    return r;
+}
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// Last word of a buffer descriptor for plain 32-bit data on this GPU family (raw buffer: byte offsets, range
+// checked against the size in bytes).
+constexpr int BUFFER_RSRC_FLAGS = 0x00020000;
+
 __global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C, int chunks, int B, uint32_t filter,
                                        int literals, int n_types, int tw, const uint32_t *__restrict__ order,
                                        uint32_t *__restrict__ records, int record_words, int K,
@@ -1921,24 +1935,55 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
     const int lane_j = lane / lpg;
     const int64_t lane_g = (int64_t)tile * tg.gpt + lane_j;
     const bool has_graph = active && lane_j < tg.gpt && lane_g < a.G;
-    // the positive literal words of the node slots of this lane's words (LA / 2 words per slot)
+    // the positive literal words of the node slots of this lane's words (LA / 2 words per slot): the tile's
+    // part of `xpos` through a buffer descriptor, so that a load is the descriptor (scalar registers), a
+    // 32-bit byte offset per lane and nothing else
     const char *x_base = reinterpret_cast<const char *>(a.xpos) + (int64_t)tile * tw * 32 * (LA * 2);
-    const char *x_lane = x_base + (active ? lane * LW * 32 : 0) * (LA * 2);
+    const __amdgpu_buffer_rsrc_t x_of_tile =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(x_base), 0, tw * 32 * (LA * 2), BUFFER_RSRC_FLAGS);
+    const uint32_t x_lane = (uint32_t)(active ? lane * LW * 32 : 0) * (LA * 2u);
+    auto load_x = [&](uint32_t at, uint2 *x) {
+        if (LA4 % 2 == 0) {
+#pragma unroll
+            for (int q = 0; q < LA4; q += 2) {
+                const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(x_of_tile, (int)at + q * 8, 0, 0);
+                x[q] = make_uint2(v.x, v.y);
+                x[q + 1] = make_uint2(v.z, v.w);
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < LA4; ++q) {
+                const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(x_of_tile, (int)at + q * 8, 0, 0);
+                x[q] = make_uint2(v.x, v.y);
+            }
+        }
+    };
+    // the clause-major weights, read at a byte offset per lane and a scalar one per clause
+    const __amdgpu_buffer_rsrc_t weights_of_clauses =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t *>(LAST ? a.wt : nullptr), 0, LAST ? C * K * 4 : 0, BUFFER_RSRC_FLAGS);
 
-    // lane p adds weight k = p % K to graph j = p / K of the tile, for p = lane, lane + 64, lane + 128, lane + 192
+    // Votes: lane l belongs to graph j = l / lanes_per_graph of the tile and adds, when a clause holds somewhere in
+    // that graph, the clause's weights of the classes i, i + lanes_per_graph, ... (i = l % lanes_per_graph): whether
+    // the graph fires is worked out once per lane and clause, and every vote after that is an LDS atomic.  A vote
+    // that a lane does not have reads its weight out of the buffer's range, which gives 0 without a memory access,
+    // and adds that to a sum of the lane's own: no execution masks to keep.
     const int pairs = tg.gpt * K;
     constexpr int VOTES = 4;
-    uint32_t vote_k_bytes[VOTES], vote_shift[VOTES];
-    bool vote_on[VOTES];
+    const int n_votes = (K + lpg - 1) / lpg;
+    const bool votes_by_owner = lpg <= 32 && n_votes <= VOTES;
+    const bool owner = LAST && votes_by_owner && lane_j < tg.gpt;
+    const unsigned long long slot_lanes = lpg >= 64 ? ~0ull : (1ull << lpg) - 1ull;
+    const uint32_t graph_lanes = owner ? (uint32_t)slot_lanes : 0u;
+    const uint32_t graph_shift = (uint32_t)(owner ? lane_j * lpg : 0);  // first lane of this lane's graph
+    uint32_t vote_k_bytes[VOTES], vote_at[VOTES];
 #pragma unroll
     for (int v = 0; v < VOTES; ++v) {
-        const int q = lane + 64 * v, j = q / K;
-        vote_on[v] = LAST && q < pairs;
-        vote_k_bytes[v] = vote_on[v] ? (uint32_t)(q - j * K) * 4u : 0u;
-        vote_shift[v] = vote_on[v] ? (uint32_t)(j * lpg) : 0u;  // first lane of the pair's graph
+        const int i = lane - lane_j * lpg, k = i + lpg * v;
+        const bool on = owner && k < K;
+        vote_k_bytes[v] = on ? (uint32_t)k * 4u : 0x7FFFFFF0u;
+        vote_at[v] = on ? (uint32_t)(lane_j * K + k) : owner && i < K ? (uint32_t)(lane_j * K + i) : 0u;
     }
     const int my_shift = (lane < tg.gpt ? lane : 0) * lpg;
-    const unsigned long long slot_lanes = lpg >= 64 ? ~0ull : (1ull << lpg) - 1ull;
 
     auto any_bit = [](const LaneWords<LW> &x) {
         uint32_t m = x.w[0];
@@ -1974,20 +2019,20 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         bool live, test;         // wave-uniform: a clause is pending / its phase 2 runs
         unsigned long long nz;   // lanes with a surviving slot after phase 1
         int weight[VOTES];
-        const int32_t *weights;
+        uint32_t weights_at;     // byte offset of the clause's weights
         char *truth_out;
     };
 
     // Phase 1 and the loads of phase 2.  Every load is issued by all lanes whatever the clause
     // does, so that the number of loads in flight is known when the pending clause is finished.
-    auto begin = [&](Pending &p, const Entries16 &rec, const int32_t *weights_of_clause, char *truth_out) {
+    auto begin = [&](Pending &p, const Entries16 &rec, uint32_t weights_at, char *truth_out) {
         p.live = true;
-        p.weights = weights_of_clause;
+        p.weights_at = weights_at;
         p.truth_out = truth_out;
         if (LAST) {  // needed only if the clause fires
-            const char *wb = reinterpret_cast<const char *>(weights_of_clause);
 #pragma unroll
-            for (int v = 0; v < VOTES; ++v) p.weight[v] = *reinterpret_cast<const int32_t *>(wb + vote_k_bytes[v]);
+            for (int v = 0; v < VOTES; ++v)
+                p.weight[v] = (int)__builtin_amdgcn_raw_buffer_load_b32(weights_of_clauses, (int)vote_k_bytes[v], (int)weights_at, 0);
         }
         const uint32_t header = rec.v[0] & 0xFFFFu;
         const uint32_t positive_pairs = header >> 12;
@@ -2019,23 +2064,19 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
                 default: half_combine<LW, 3, 3>(acc, r); break;
             }
         }
-        p.nz = __ballot(any_bit(acc));
-        p.test = (header & 0x100u) && p.nz != 0;
-        // lowest surviving slot of the lane: the lowest set bit of its first word that has one
-        // (__ffs(0) - 1 is ~0, which survives the OR: no slot)
-        uint32_t first_word = acc.w[LW - 1], first_base = (uint32_t)(LW - 1) * 32u;
+        // lowest surviving slot of the lane: the smallest of its words' lowest set bits (~0 for a word without
+        // one, which survives the OR with the word's base and loses every comparison: no slot)
+        uint32_t bit = lowest_bit_or_ones(acc.w[0]);
 #pragma unroll
-        for (int u = LW - 2; u >= 0; --u) {
-            const bool here = acc.w[u] != 0u;
-            first_word = here ? acc.w[u] : first_word;
-            first_base = here ? (uint32_t)u * 32u : first_base;
+        for (int u = 1; u < LW; ++u) {
+            const uint32_t here = lowest_bit_or_ones(acc.w[u]) | (uint32_t)u * 32u;
+            bit = here < bit ? here : bit;
         }
-        const uint32_t bit = (uint32_t)(__ffs(first_word) - 1) | first_base;
+        p.nz = __ballot(bit != ~0u);
+        p.test = (header & 0x100u) && p.nz != 0;
         p.bit = has_graph ? bit : ~0u;
         // lanes with nothing to test all read the tile's first slot (one cache line for the wave)
-        const uint2 *x = reinterpret_cast<const uint2 *>(p.bit != ~0u ? x_lane + p.bit * (LA * 2u) : x_base);
-#pragma unroll
-        for (int q = 0; q < LA4; ++q) p.x[q] = x[q];
+        load_x(p.bit != ~0u ? x_lane + p.bit * (LA * 2u) : 0u, p.x);
         p.acc = acc;
     };
 
@@ -2120,7 +2161,8 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
                         while (todo) {
                             const int b = __ffs(todo) - 1;
                             todo &= todo - 1;
-                            const uint2 *x = reinterpret_cast<const uint2 *>(x_lane + (u * 32 + b) * (LA * 2u));
+                            uint2 x[LA4];
+                            load_x(x_lane + (uint32_t)(u * 32 + b) * (LA * 2u), x);
                             if (violates(include, x)) acc.w[u] &= ~(1u << b);
                         }
                     }
@@ -2134,16 +2176,18 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         }
         if (nz == 0) return;
         // graph j owns lanes [j * lanes_per_graph, (j + 1) * lanes_per_graph)
-        if (lpg <= 32 && pairs <= 64 * VOTES) {
-            const uint32_t m = (uint32_t)slot_lanes;
+        if (votes_by_owner) {
+            if (((uint32_t)(nz >> graph_shift) & graph_lanes) != 0) {
 #pragma unroll
-            for (int v = 0; v < VOTES; ++v)
-                if (vote_on[v] && ((uint32_t)(nz >> vote_shift[v]) & m) != 0) atomicAdd(&sums[lane + 64 * v], p.weight[v]);
+                for (int v = 0; v < VOTES; ++v)
+                    if (v < n_votes) atomicAdd(&sums[vote_at[v]], p.weight[v]);
+            }
         } else {
             const unsigned long long gm = __ballot(lane < tg.gpt && ((nz >> my_shift) & slot_lanes) != 0);
+            const int32_t *weights = a.wt + (p.weights_at >> 2);
             for (int q = lane; q < pairs; q += 64) {
                 const int j = q / K, k = q - j * K;
-                if ((gm >> j) & 1ull) atomicAdd(&sums[q], p.weights[k]);
+                if ((gm >> j) & 1ull) atomicAdd(&sums[q], weights[k]);
             }
         }
     };
@@ -2153,11 +2197,11 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
     // finished, one phase 1 later).  Pointers step by NWAVES clauses; past the end they stay on
     // the wave's last clause (a valid address whose data is not used).
     const int64_t rec_step = (int64_t)NWAVES * a.stride;
-    const int wt_step = NWAVES * K;
+    const uint32_t wt_step = (uint32_t)(NWAVES * K) * 4u;
     const int64_t truth_step = (int64_t)NWAVES * tw * 4;
     const int first = c_begin + wave < c_end ? c_begin + wave : c_begin;
     const uint32_t *rec_a = a.lists + (int64_t)first * a.stride;
-    const int32_t *wt_a = LAST ? a.wt + (int64_t)first * K : nullptr;
+    uint32_t wt_a = LAST ? (uint32_t)(first * K) * 4u : 0u;
     char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
     Entries16 ea = *reinterpret_cast<const Entries16 *>(rec_a);
     Words<LA> ma, mb;
@@ -2166,7 +2210,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
     for (int c = c_begin + wave; c < c_end; c += 2 * NWAVES) {
         const bool has_b = c + NWAVES < c_end;
         const uint32_t *rec_b = has_b ? rec_a + rec_step : rec_a;
-        const int32_t *wt_b = LAST ? (has_b ? wt_a + wt_step : wt_a) : nullptr;
+        const uint32_t wt_b = LAST && has_b ? wt_a + wt_step : wt_a;
         char *truth_b = has_b ? truth_a + truth_step : truth_a;
         ma = *reinterpret_cast<const Words<LA> *>(rec_a + 16);
         const Entries16 eb = *reinterpret_cast<const Entries16 *>(rec_b);
@@ -2174,7 +2218,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         finish(pb, mb);
         const bool has_a = c + 2 * NWAVES < c_end;
         rec_a = has_a ? rec_b + rec_step : rec_b;
-        if (LAST) wt_a = has_a ? wt_b + wt_step : wt_b;
+        wt_a = LAST && has_a ? wt_b + wt_step : wt_b;
         truth_a = has_a ? truth_b + truth_step : truth_b;
         // without a second clause this repeats the first one and drops the result: keeping the
         // sequence of loads the same on every trip lets the waits stay partial
