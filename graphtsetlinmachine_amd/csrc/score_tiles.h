@@ -1959,6 +1959,18 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         }
     };
     // the clause-major weights, read at a byte offset per lane and a scalar one per clause
+    // the include words of a clause (after the 16 entries of its record), the same for every lane, into VECTOR registers
+    const __amdgpu_buffer_rsrc_t records =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(a.lists), 0, C * a.stride * 4, BUFFER_RSRC_FLAGS);
+    auto load_include = [&](uint32_t record_at) {
+        Words<LA> m;
+#pragma unroll
+        for (int q = 0; q < LA4; ++q) {
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(records, 64 + 16 * q, (int)record_at, 0);
+            m.v[4 * q] = v.x, m.v[4 * q + 1] = v.y, m.v[4 * q + 2] = v.z, m.v[4 * q + 3] = v.w;
+        }
+        return m;
+    };
     const __amdgpu_buffer_rsrc_t weights_of_clauses =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t *>(LAST ? a.wt : nullptr), 0, LAST ? C * K * 4 : 0, BUFFER_RSRC_FLAGS);
 
@@ -1993,15 +2005,19 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
     };
     auto entry_of = [](const Entries16 &rec, int i) { return rec.v[i]; };
     // a positive literal is violated where the node lacks it, a negated one (include words LA / 2 ..)
-    // where the node has it: (include_pos & ~x) | (include_neg & x), one 3-input operation per word
+    // where the node has it: x ? include_neg : include_pos, one 3-input operation per word (the include
+    // words are in vector registers, see the loads in the loop below: with two of three operands in
+    // scalar registers it is two operations and a move)
     auto violates = [](const Words<LA> &include, const uint2 *x) {
-        uint32_t violated = 0;
+        uint32_t t[2 * LA4];
 #pragma unroll
         for (int q = 0; q < LA4; ++q) {
-            const uint2 v = x[q];
-            violated |= (include.v[2 * q] & ~v.x) | (include.v[2 * q + LA / 2] & v.x) | (include.v[2 * q + 1] & ~v.y) |
-                        (include.v[2 * q + 1 + LA / 2] & v.y);
+            t[2 * q] = __builtin_amdgcn_bitop3_b32(x[q].x, include.v[2 * q + 2 * LA4], include.v[2 * q], 0xCA);
+            t[2 * q + 1] = __builtin_amdgcn_bitop3_b32(x[q].y, include.v[2 * q + 1 + 2 * LA4], include.v[2 * q + 1], 0xCA);
         }
+        uint32_t violated = t[0];
+#pragma unroll
+        for (int w = 1; w < 2 * LA4; ++w) violated |= t[w];
         return violated != 0;
     };
     // the word set with only `bit` set (bit < 32 * LW)
@@ -2072,11 +2088,12 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
             const uint32_t here = lowest_bit_or_ones(acc.w[u]) | (uint32_t)u * 32u;
             bit = here < bit ? here : bit;
         }
+        // (no slot survives in lanes without a graph: the node-type row is zero there)
         p.nz = __ballot(bit != ~0u);
         p.test = (header & 0x100u) && p.nz != 0;
-        p.bit = has_graph ? bit : ~0u;
+        p.bit = bit;
         // lanes with nothing to test all read the tile's first slot (one cache line for the wave)
-        load_x(p.bit != ~0u ? x_lane + p.bit * (LA * 2u) : 0u, p.x);
+        load_x(bit != ~0u ? x_lane + bit * (LA * 2u) : 0u, p.x);
         p.acc = acc;
     };
 
@@ -2192,43 +2209,51 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         }
     };
 
-    // Clause records: the 8 words of row entries are fetched one clause ahead of phase 1, the
-    // include mask at the start of the clause's phase 1 (it is first needed when the clause is
-    // finished, one phase 1 later).  Pointers step by NWAVES clauses; past the end they stay on
-    // the wave's last clause (a valid address whose data is not used).
+    // Clause records: the 16 words of row entries are fetched one clause ahead of phase 1 (scalar
+    // loads), the include words when the clause's phase 1 is over, just before the other clause's
+    // (vector loads: they are first needed when the clause is finished, one phase 1 later).  Pointers
+    // and offsets step by NWAVES clauses; past the end they stay on the wave's last clause (a valid
+    // address whose data is not used).
     const int64_t rec_step = (int64_t)NWAVES * a.stride;
     const uint32_t wt_step = (uint32_t)(NWAVES * K) * 4u;
     const int64_t truth_step = (int64_t)NWAVES * tw * 4;
     const int first = c_begin + wave < c_end ? c_begin + wave : c_begin;
     const uint32_t *rec_a = a.lists + (int64_t)first * a.stride;
+    const uint32_t at_step = (uint32_t)(NWAVES * a.stride) * 4u;
+    uint32_t at_a = (uint32_t)(first * a.stride) * 4u;  // rec_a as a byte offset
     uint32_t wt_a = LAST ? (uint32_t)(first * K) * 4u : 0u;
     char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
     Entries16 ea = *reinterpret_cast<const Entries16 *>(rec_a);
-    Words<LA> ma, mb;
     Pending pa, pb;
     pa.live = pb.live = false;
+    uint32_t at_pending = at_a;  // the record of the clause in pb (a valid record while there is none)
     for (int c = c_begin + wave; c < c_end; c += 2 * NWAVES) {
         const bool has_b = c + NWAVES < c_end;
         const uint32_t *rec_b = has_b ? rec_a + rec_step : rec_a;
         const uint32_t wt_b = LAST && has_b ? wt_a + wt_step : wt_a;
+        const uint32_t at_b = has_b ? at_a + at_step : at_a;
         char *truth_b = has_b ? truth_a + truth_step : truth_a;
-        ma = *reinterpret_cast<const Words<LA> *>(rec_a + 16);
+        // The include words of the pending clause are requested before the phase 1 that runs ahead of its end,
+        // so only one clause's are in registers at a time.
+        Words<LA> include = load_include(at_pending);
         const Entries16 eb = *reinterpret_cast<const Entries16 *>(rec_b);
         begin(pa, ea, wt_a, truth_a);
-        finish(pb, mb);
+        finish(pb, include);
+        include = load_include(at_a);
         const bool has_a = c + 2 * NWAVES < c_end;
         rec_a = has_a ? rec_b + rec_step : rec_b;
         wt_a = LAST && has_a ? wt_b + wt_step : wt_b;
+        at_a = has_a ? at_b + at_step : at_b;
         truth_a = has_a ? truth_b + truth_step : truth_b;
         // without a second clause this repeats the first one and drops the result: keeping the
         // sequence of loads the same on every trip lets the waits stay partial
-        mb = *reinterpret_cast<const Words<LA> *>(rec_b + 16);
         ea = *reinterpret_cast<const Entries16 *>(rec_a);
         begin(pb, eb, wt_b, truth_b);
         pb.live = has_b;
-        finish(pa, ma);
+        finish(pa, include);
+        at_pending = at_b;
     }
-    finish(pb, mb);
+    if (pb.live) finish(pb, load_include(at_pending));
     if (!LAST) return;
     __syncthreads();
     const int64_t g0 = (int64_t)tile * tg.gpt;
