@@ -2041,7 +2041,8 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
 
     // Phase 1 and the loads of phase 2.  Every load is issued by all lanes whatever the clause
     // does, so that the number of loads in flight is known when the pending clause is finished.
-    auto begin = [&](Pending &p, const Entries16 &rec, uint32_t weights_at, char *truth_out) {
+    auto begin = [&](Pending &p, const Entries16 &rec, uint32_t weights_at, char *truth_out, const uint32_t *record_next,
+                     Entries16 &next) {
         p.live = true;
         p.weights_at = weights_at;
         p.truth_out = truth_out;
@@ -2080,6 +2081,9 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
                 default: half_combine<LW, 3, 3>(acc, r); break;
             }
         }
+        // (the next record is requested only now: scalar loads and LDS reads are waited for with one counter, so a
+        // request before the rows would have been waited for along with them)
+        next = *reinterpret_cast<const Entries16 *>(record_next);
         // lowest surviving slot of the lane: the smallest of its words' lowest set bits (~0 for a word without
         // one, which survives the OR with the word's base and loses every comparison: no slot)
         uint32_t bit = lowest_bit_or_ones(acc.w[0]);
@@ -2236,21 +2240,22 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         // The include words of the pending clause are requested before the phase 1 that runs ahead of its end,
         // so only one clause's are in registers at a time.
         Words<LA> include = load_include(at_pending);
-        const Entries16 eb = *reinterpret_cast<const Entries16 *>(rec_b);
-        begin(pa, ea, wt_a, truth_a);
+        Entries16 eb;
+        begin(pa, ea, wt_a, truth_a, rec_b, eb);
         finish(pb, include);
         include = load_include(at_a);
         const bool has_a = c + 2 * NWAVES < c_end;
         rec_a = has_a ? rec_b + rec_step : rec_b;
-        wt_a = LAST && has_a ? wt_b + wt_step : wt_b;
+        const uint32_t wt_next = LAST && has_a ? wt_b + wt_step : wt_b;
         at_a = has_a ? at_b + at_step : at_b;
-        truth_a = has_a ? truth_b + truth_step : truth_b;
+        char *truth_next = has_a ? truth_b + truth_step : truth_b;
         // without a second clause this repeats the first one and drops the result: keeping the
         // sequence of loads the same on every trip lets the waits stay partial
-        ea = *reinterpret_cast<const Entries16 *>(rec_a);
-        begin(pb, eb, wt_b, truth_b);
+        begin(pb, eb, wt_b, truth_b, rec_a, ea);
         pb.live = has_b;
         finish(pa, include);
+        wt_a = wt_next;
+        truth_a = truth_next;
         at_pending = at_b;
     }
     if (pb.live) finish(pb, load_include(at_pending));
