@@ -2121,6 +2121,40 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
             if (__ballot(failed && slots_left > 1) == 0ull) {
                 nz = __ballot(tested && !failed);
                 settled = true;
+            } else {
+                // Some lane's first candidate failed and it has others.  All such lanes test their next candidate
+                // at the same time, one memory round trip per turn, and a lane stops at its first candidate that
+                // holds: as many turns as the unluckiest lane needs.  (With many candidates left somewhere the
+                // rows of all the clause's literals are ANDed instead, below.)
+                const LaneWords<LW> hot = one_hot(p.bit);
+                LaneWords<LW> rest;
+                int others = 0;
+#pragma unroll
+                for (int u = 0; u < LW; ++u) {
+                    rest.w[u] = failed ? acc.w[u] & ~hot.w[u] : 0u;
+                    others += __popc(rest.w[u]);
+                }
+                if (__ballot(others >= TWO_PHASE_WALK_FROM) == 0ull) {
+                    bool holds = tested && !failed;
+                    while (__ballot(any_bit(rest)) != 0ull) {
+                        uint32_t bit = lowest_bit_or_ones(rest.w[0]);
+#pragma unroll
+                        for (int u = 1; u < LW; ++u) {
+                            const uint32_t here = lowest_bit_or_ones(rest.w[u]) | (uint32_t)u * 32u;
+                            bit = here < bit ? here : bit;
+                        }
+                        const bool searching = bit != ~0u;
+                        uint2 x[LA4];
+                        load_x(searching ? x_lane + bit * (LA * 2u) : 0u, x);
+                        const bool ok = searching && !violates(include, x);
+                        holds = holds || ok;
+                        const LaneWords<LW> tried = one_hot(bit);  // (no word for ~0)
+#pragma unroll
+                        for (int u = 0; u < LW; ++u) rest.w[u] = ok ? 0u : rest.w[u] & ~tried.w[u];
+                    }
+                    nz = __ballot(holds);
+                    settled = true;
+                }
             }
         }
         if (p.test && !settled) {
