@@ -2027,6 +2027,19 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         for (int u = 0; u < LW; ++u) m.w[u] = (int)(bit >> 5) == u ? 1u << (bit & 31u) : 0u;
         return m;
     };
+    // the word set W without its lowest set bit: W & (W - 1), the decrement carried through the words
+    auto without_lowest_bit = [](const LaneWords<LW> &x) {
+        LaneWords<LW> r;
+        uint32_t borrow = 1u;
+#pragma unroll
+        for (int u = 0; u < LW; ++u) {
+            uint32_t out;
+            const uint32_t less = __builtin_subc(x.w[u], 0u, borrow, &out);
+            borrow = out;
+            r.w[u] = x.w[u] & less;
+        }
+        return r;
+    };
 
     struct Pending {
         LaneWords<LW> acc;
@@ -2126,12 +2139,13 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
                 // at the same time, one memory round trip per turn, and a lane stops at its first candidate that
                 // holds: as many turns as the unluckiest lane needs.  (With many candidates left somewhere the
                 // rows of all the clause's literals are ANDed instead, below.)
-                const LaneWords<LW> hot = one_hot(p.bit);
-                LaneWords<LW> rest;
+                // (the candidate under test is always the lowest set bit of the lane's words taken as one number W:
+                // W & (W - 1) takes it out)
+                LaneWords<LW> rest = without_lowest_bit(acc);
                 int others = 0;
 #pragma unroll
                 for (int u = 0; u < LW; ++u) {
-                    rest.w[u] = failed ? acc.w[u] & ~hot.w[u] : 0u;
+                    rest.w[u] = failed ? rest.w[u] : 0u;
                     others += __popc(rest.w[u]);
                 }
                 if (__ballot(others >= TWO_PHASE_WALK_FROM) == 0ull) {
@@ -2146,11 +2160,11 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
                         const bool searching = bit != ~0u;
                         uint2 x[LA4];
                         load_x(searching ? x_lane + bit * (LA * 2u) : 0u, x);
+                        const LaneWords<LW> next = without_lowest_bit(rest);
                         const bool ok = searching && !violates(include, x);
                         holds = holds || ok;
-                        const LaneWords<LW> tried = one_hot(bit);  // (no word for ~0)
 #pragma unroll
-                        for (int u = 0; u < LW; ++u) rest.w[u] = ok ? 0u : rest.w[u] & ~tried.w[u];
+                        for (int u = 0; u < LW; ++u) rest.w[u] = ok ? 0u : next.w[u];
                     }
                     nz = __ballot(holds);
                     settled = true;
