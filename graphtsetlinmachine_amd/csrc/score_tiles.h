@@ -2043,7 +2043,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
 
     struct Pending {
         LaneWords<LW> acc;
-        uint2 x[LA4];
+        uint2 x[LA4], x2[LA4];   // the words of the lane's first and (for the class sums) second surviving slot
         uint32_t bit;            // the node slot this lane has under test (index into its LW words), ~0 if none
         bool live, test;         // wave-uniform: a clause is pending / its phase 2 runs
         unsigned long long nz;   // lanes with a surviving slot after phase 1
@@ -2111,6 +2111,18 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         p.bit = bit;
         // lanes with nothing to test all read the tile's first slot (one cache line for the wave)
         load_x(bit != ~0u ? x_lane + bit * (LA * 2u) : 0u, p.x);
+        if (LAST) {
+            // The second surviving slot's words come along: a first candidate fails often enough, and a test that
+            // starts only then has its memory round trip in the open.
+            const LaneWords<LW> after = without_lowest_bit(acc);
+            uint32_t bit2 = lowest_bit_or_ones(after.w[0]);
+#pragma unroll
+            for (int u = 1; u < LW; ++u) {
+                const uint32_t here = lowest_bit_or_ones(after.w[u]) | (uint32_t)u * 32u;
+                bit2 = here < bit2 ? here : bit2;
+            }
+            load_x(bit2 != ~0u ? x_lane + bit2 * (LA * 2u) : 0u, p.x2);
+        }
         p.acc = acc;
     };
 
@@ -2127,29 +2139,29 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
             // Only a lane whose first candidate failed and that has others needs more tests (rare: then
             // the exact path below runs).
             const bool tested = p.bit != ~0u;
-            const bool failed = violates(include, p.x) && tested;
             int slots_left = 0;
 #pragma unroll
             for (int u = 0; u < LW; ++u) slots_left += __popc(acc.w[u]);
-            if (__ballot(failed && slots_left > 1) == 0ull) {
-                nz = __ballot(tested && !failed);
+            bool holds = tested && (!violates(include, p.x) || (slots_left > 1 && !violates(include, p.x2)));
+            const bool more = tested && !holds && slots_left > 2;
+            if (__ballot(more) == 0ull) {
+                nz = __ballot(holds);
                 settled = true;
             } else {
-                // Some lane's first candidate failed and it has others.  All such lanes test their next candidate
+                // Both candidates of some lane failed and it has others.  All such lanes test their next candidate
                 // at the same time, one memory round trip per turn, and a lane stops at its first candidate that
                 // holds: as many turns as the unluckiest lane needs.  (With many candidates left somewhere the
                 // rows of all the clause's literals are ANDed instead, below.)
                 // (the candidate under test is always the lowest set bit of the lane's words taken as one number W:
                 // W & (W - 1) takes it out)
-                LaneWords<LW> rest = without_lowest_bit(acc);
+                LaneWords<LW> rest = without_lowest_bit(without_lowest_bit(acc));
                 int others = 0;
 #pragma unroll
                 for (int u = 0; u < LW; ++u) {
-                    rest.w[u] = failed ? rest.w[u] : 0u;
+                    rest.w[u] = more ? rest.w[u] : 0u;
                     others += __popc(rest.w[u]);
                 }
-                if (__ballot(others >= TWO_PHASE_WALK_FROM) == 0ull) {
-                    bool holds = tested && !failed;
+                if (__ballot(others + 1 >= TWO_PHASE_WALK_FROM) == 0ull) {
                     while (__ballot(any_bit(rest)) != 0ull) {
                         uint32_t bit = lowest_bit_or_ones(rest.w[0]);
 #pragma unroll
