@@ -65,6 +65,7 @@ int check_launch(const char *what) {
     X(FIT_SPIN_LIMIT) \
     X(HALF_LANE_WORDS) \
     X(MESSAGES_IN_LDS) \
+    X(NARROW_IN_ORDER) \
     X(NARROW_READS) \
     X(NARROW_ROWS_AS_STORED) \
     X(NODE_MESSAGES_BY_ATOMICS) \
@@ -665,6 +666,7 @@ struct ScoreWs {
     uint32_t *message_rows;   // [tiles per launch][M + 2][tw]  (tile path, depth > 1)
     uint32_t *bit_start, *bit_cursor, *bit_clauses;  // [M + 1], [M], [C * MB]: the clauses of every message bit (tile path, depth > 1)
     uint32_t *alive[2];       // [tiles per launch][streams][alive_stride] clauses still true somewhere in a tile, layer to layer
+    uint32_t *stream_order;   // [streams][alive_stride] every clause, by length of its layer-0 list (k_narrow_stream_order)
     size_t alive_words;       // room per tile
     TileSegment *segments;    // [tiles + 2 * TILE_SEGMENTS_MAX_SHARES] which clauses of which tile a workgroup takes (half tiles)
     size_t vector_words;      // words of sent (and of got)
@@ -697,6 +699,7 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base,
     w.list_stride = clause_list_stride(cfg->literals);
     w.lists = (uint32_t *)take((size_t)d.C * w.list_stride * 4);
     w.wt = (int32_t *)take((size_t)d.C * d.K * 4);
+    if (tg) w.stream_order = (uint32_t *)take(((size_t)d.C + 2 * NARROW_MAX_STREAMS) * 4);
     if (tg && cfg->depth == 1 && tg->half)
         w.segments = (TileSegment *)take(((size_t)tg->n_tiles + 2 * TILE_SEGMENTS_MAX_SHARES) * sizeof(TileSegment));
     if (tg && cfg->depth == 1 && !keep_rows) {
@@ -1308,6 +1311,15 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
                            l == layers - 1 ? s->clause_weights : nullptr, w.wt, w.longest_list + (l - 1));
         if (int rc = check_launch("compile_clauses")) return rc;
     }
+    // layer 0 on narrow tiles takes its clauses by length (GTM_NARROW_IN_ORDER, tuning and test aid: by number)
+    const bool by_length = half_rows0 && d.C <= NARROW_ORDER_MAX_CLAUSES && !tune(T_NARROW_IN_ORDER);
+    if (by_length) {
+        hipLaunchKernelGGL(k_narrow_stream_order, dim3(blocks_for(d.C, NARROW_ORDER_BLOCK)), dim3(NARROW_ORDER_BLOCK),
+                           (size_t)((d.C + 3) & ~3) * 4, st, w.lists, w.list_stride, w.message_lists, w.message_list_stride,
+                           narrow_messages ? layers - 1 : 0, d.C, shape.streams(), narrow_alive_stride(d.C, shape.streams()),
+                           w.stream_order);
+        if (int rc = check_launch("narrow_stream_order")) return rc;
+    }
     TileLayerArgs a{};
     a.tiles = g->tiles;
     a.tg = tg;
@@ -1332,7 +1344,8 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         a.lists = w.lists;
         a.stride = stride0;
         if (half_rows0) {
-            px.alive_in = nullptr;
+            px.alive_in = by_length ? w.stream_order : nullptr;
+            px.alive_in_shared = 1;
             px.alive_out = !last && narrow_messages ? w.alive[0] : nullptr;
             px.row_words = row_words0;
             alive_now = px.alive_out;
@@ -1420,6 +1433,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
         const bool last = l == layers - 1 && !tr;
         if (!narrow_messages) return launch_tile_layer(a, n_tiles, ROWS_MESSAGES, last, st);
         px.alive_in = alive_now;
+        px.alive_in_shared = 0;
         px.row_words = row_words_m;
         px.alive_out = last || l == layers - 1 ? nullptr : w.alive[alive_now == w.alive[0] ? 1 : 0];
         alive_now = px.alive_out;

@@ -66,6 +66,7 @@ struct NarrowArgs {
                                // that are true somewhere in the tile; NULL: every clause (q, q + streams, ...) is looked at
     uint32_t *alive_out;       // the same for the next layer, or NULL
     int alive_stride;          // >= 1 + ceil(C / streams)
+    int alive_in_shared;       // alive_in is ONE set of lists for every tile (k_narrow_stream_order: all clauses, by length)
     int hv, n_types;           // ROWS_HALF: positive literals (= LDS rows before the node-type rows), node types
     int row_words;             // words from one row to the next in LDS (>= tw, a multiple of 4): what the lists' entries count in
 };
@@ -160,6 +161,59 @@ struct NarrowRow {
 
 typedef uint32_t NarrowEntries __attribute__((ext_vector_type(4)));  // four entries of a compiled list
 
+// Which clauses a stream takes when every clause is looked at (layer 0), in the format of the lists of clauses
+// still alive: the clauses by falling length of their compiled lists, dealt out to the streams in turn - stream q
+// takes ranks q, q + streams, ... - so that the groups of a wave, which stay together until the longest of their
+// lists has been walked, hold lists of nearly the same length at every step, and a workgroup's long clauses come
+// first.  The message layers take their clauses in the same order, as far as they are still alive, so among the
+// clauses of one length in layer 0 (there are few different lengths) the order is by the length in the first
+// message layer, then the second.  Ties by clause number: the table is the same from call to call.  One thread per
+// clause; every block first copies the keys (from entry 0 of each list: blocks of rows | blocks of complements << 16)
+// into LDS.
+constexpr int NARROW_ORDER_BLOCK = 256;
+static_assert(NARROW_ORDER_BLOCK >= NARROW_MAX_STREAMS, "one thread per stream writes its count");
+constexpr int NARROW_ORDER_MAX_CLAUSES = 16384;  // 64 KB of LDS
+__global__ __launch_bounds__(NARROW_ORDER_BLOCK) void k_narrow_stream_order(const uint32_t *__restrict__ lists, int list_stride,
+                                                                           const uint32_t *__restrict__ message_lists,
+                                                                           int message_list_stride, int message_layers,
+                                                                           int C, int streams, int alive_stride,
+                                                                           uint32_t *__restrict__ table) {
+    extern __shared__ uint32_t keys[];  // [C rounded up to 4]
+    const int padded = (C + 3) & ~3;
+    auto blocks_of = [](uint32_t header) {
+        const uint32_t n = (header & 0xFFFFu) + (header >> 16);
+        return n < 1023u ? n : 1023u;
+    };
+    for (int i = threadIdx.x; i < padded; i += NARROW_ORDER_BLOCK) {
+        uint32_t key = 0u;
+        if (i < C) {
+            key = blocks_of(lists[(int64_t)i * list_stride]) << 20;
+            for (int l = 0; l < message_layers && l < 2; ++l)
+                key |= blocks_of(message_lists[((int64_t)l * C + i) * message_list_stride]) << (10 - 10 * l);
+        }
+        keys[i] = key;
+    }
+    __syncthreads();
+    const int c = blockIdx.x * NARROW_ORDER_BLOCK + threadIdx.x;
+    // (a stream beyond the last clause has none: the launch has at least NARROW_ORDER_BLOCK >= streams threads)
+    if (c < streams) table[(int64_t)c * alive_stride] = c < C ? (uint32_t)((C - c + streams - 1) / streams) : 0u;
+    if (c >= C) return;
+    const uint32_t mine = keys[c];
+    // rank = clauses with a greater key, or the same key and a smaller number; four keys per LDS read
+    int rank = 0;
+    const uint4 *four = reinterpret_cast<const uint4 *>(keys);
+    for (int i = 0; i < padded / 4; ++i) {
+        const uint4 v = four[i];
+        const uint32_t k[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int at = 4 * i + u;
+            rank += (k[u] > mine || (k[u] == mine && at < c)) && at < C;
+        }
+    }
+    table[(int64_t)(rank % streams) * alive_stride + 1 + rank / streams] = (uint32_t)c;
+}
+
 template <int SRC, bool LAST, int GROUP, int WPL>
 __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLayerArgs a, NarrowArgs x) {
     static_assert(SRC == ROWS_HALF || SRC == ROWS_MESSAGES, "layer 0 on half rows, or a message layer");
@@ -238,7 +292,8 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
     }
 
     // this stream's clauses
-    const uint32_t *seg_in = x.alive_in ? x.alive_in + ((int64_t)tile_local * STREAMS + q) * x.alive_stride : nullptr;
+    const uint32_t *seg_in =
+        x.alive_in ? x.alive_in + ((int64_t)(x.alive_in_shared ? 0 : tile_local) * STREAMS + q) * x.alive_stride : nullptr;
     const int n_mine = seg_in ? (int)seg_in[0] : (q < C ? (C - q + STREAMS - 1) / STREAMS : 0);
     int n_most = 0;
 #pragma unroll
@@ -352,6 +407,7 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
 #pragma unroll
                     for (int half = 0; half < 2; ++half) {
                         const int at = b + half * TRIP;
+                        if (half == 1 && at >= lim_most) break;  // (no group has a block there; uniform over the wave)
                         uint32_t n_lo[TRIP], n_hi[TRIP];
 #pragma unroll
                         for (int t = 0; t < TRIP; ++t)

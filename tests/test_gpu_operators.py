@@ -1020,8 +1020,8 @@ NARROW_TILE_SHAPES = [
 
 @pytest.mark.parametrize("shape", NARROW_TILE_SHAPES, ids=lambda s: "narrow%d" % s["seed"])
 @pytest.mark.parametrize("depth", [1, 2, 3])
-@pytest.mark.parametrize("path", ["several-clauses-per-wave", "128-bit-reads", "rows-as-stored", "all-rows-layer-0", "one-clause-per-wave",
-                                  "messages-of-a-tile-in-lds", "messages-in-three-launches"])
+@pytest.mark.parametrize("path", ["several-clauses-per-wave", "128-bit-reads", "rows-as-stored", "clauses-by-number", "all-rows-layer-0",
+                                  "one-clause-per-wave", "messages-of-a-tile-in-lds", "messages-in-three-launches"])
 def test_scoring_on_narrow_tiles(shape, depth, path, tune):
     """Tiles whose rows are at most 64 words wide: eight or four clauses per wave (score_narrow.h), for the message
     layers and - on a data set whose negated literals are the complements of its positive ones - for
@@ -1035,6 +1035,8 @@ def test_scoring_on_narrow_tiles(shape, depth, path, tune):
         tune("GTM_NARROW_READS", "128")
     elif path == "rows-as-stored":  # (rows in LDS as far apart as in memory, not 128 bytes)
         tune("GTM_NARROW_ROWS_AS_STORED", "1")
+    elif path == "clauses-by-number":  # (layer 0 takes clauses q, q + streams, ... instead of by length of their lists)
+        tune("GTM_NARROW_IN_ORDER", "1")
     elif path == "all-rows-layer-0":
         tune("GTM_NO_HALF_ROWS", "1")
     elif path == "one-clause-per-wave":

@@ -18,7 +18,7 @@ CASES_PER_TEST = 25
 SWITCHES = [(), (("GTM_MESSAGES_IN_LDS", "1"),), (("GTM_MESSAGES_IN_LDS", "0"),), (("GTM_NARROW_READS", "128"),),
             (("GTM_NO_HALF_ROWS", "1"),), (("GTM_MESSAGES_IN_LDS", "1"), ("GTM_NARROW_READS", "128")),
             (("GTM_NO_FUSED_MESSAGES", "1"),), (("GTM_MESSAGES_IN_LDS", "0"), ("GTM_NO_FUSED_MESSAGES", "1")),
-            (("GTM_NARROW_ROWS_AS_STORED", "1"),)]
+            (("GTM_NARROW_ROWS_AS_STORED", "1"),), (("GTM_NARROW_IN_ORDER", "1"),)]
 
 
 def pick(rng, xs):
