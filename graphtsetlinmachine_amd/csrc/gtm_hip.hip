@@ -1314,10 +1314,11 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     // layer 0 on narrow tiles takes its clauses by length (GTM_NARROW_IN_ORDER, tuning and test aid: by number)
     const bool by_length = half_rows0 && d.C <= NARROW_ORDER_MAX_CLAUSES && !tune(T_NARROW_IN_ORDER);
     if (by_length) {
-        hipLaunchKernelGGL(k_narrow_stream_order, dim3(blocks_for(d.C, NARROW_ORDER_BLOCK)), dim3(NARROW_ORDER_BLOCK),
-                           (size_t)((d.C + 3) & ~3) * 4, st, w.lists, w.list_stride, w.message_lists, w.message_list_stride,
-                           narrow_messages ? layers - 1 : 0, d.C, shape.streams(), narrow_alive_stride(d.C, shape.streams()),
-                           w.stream_order);
+        size_t pairs = 1;
+        while (pairs < (size_t)d.C) pairs <<= 1;
+        hipLaunchKernelGGL(k_narrow_stream_order, dim3(1), dim3(NARROW_ORDER_BLOCK), pairs * 8, st, w.lists, w.list_stride,
+                           w.message_lists, w.message_list_stride, narrow_messages ? layers - 1 : 0, d.C, shape.streams(),
+                           narrow_alive_stride(d.C, shape.streams()), w.stream_order);
         if (int rc = check_launch("narrow_stream_order")) return rc;
     }
     TileLayerArgs a{};

@@ -167,51 +167,52 @@ typedef uint32_t NarrowEntries __attribute__((ext_vector_type(4)));  // four ent
 // lists has been walked, hold lists of nearly the same length at every step, and a workgroup's long clauses come
 // first.  The message layers take their clauses in the same order, as far as they are still alive, so among the
 // clauses of one length in layer 0 (there are few different lengths) the order is by the length in the first
-// message layer, then the second.  Ties by clause number: the table is the same from call to call.  One thread per
-// clause; every block first copies the keys (from entry 0 of each list: blocks of rows | blocks of complements << 16)
-// into LDS.
-constexpr int NARROW_ORDER_BLOCK = 256;
-static_assert(NARROW_ORDER_BLOCK >= NARROW_MAX_STREAMS, "one thread per stream writes its count");
-constexpr int NARROW_ORDER_MAX_CLAUSES = 16384;  // 64 KB of LDS
+// message layer, then the second.  Ties by clause number: the table is the same from call to call.  One workgroup
+// sorts (key, clause) pairs in LDS (bitonic, 8 bytes per clause rounded up to a power of two); the lengths come
+// from entry 0 of each list: blocks of rows | blocks of complements << 16.
+constexpr int NARROW_ORDER_BLOCK = 1024;
+constexpr int NARROW_ORDER_MAX_CLAUSES = 8192;  // 64 KB of LDS
 __global__ __launch_bounds__(NARROW_ORDER_BLOCK) void k_narrow_stream_order(const uint32_t *__restrict__ lists, int list_stride,
                                                                            const uint32_t *__restrict__ message_lists,
                                                                            int message_list_stride, int message_layers,
                                                                            int C, int streams, int alive_stride,
                                                                            uint32_t *__restrict__ table) {
-    extern __shared__ uint32_t keys[];  // [C rounded up to 4]
-    const int padded = (C + 3) & ~3;
+    extern __shared__ unsigned long long order_keys[];
+    constexpr int NT = NARROW_ORDER_BLOCK;
+    int N = 1;
+    while (N < C) N <<= 1;
     auto blocks_of = [](uint32_t header) {
         const uint32_t n = (header & 0xFFFFu) + (header >> 16);
         return n < 1023u ? n : 1023u;
     };
-    for (int i = threadIdx.x; i < padded; i += NARROW_ORDER_BLOCK) {
-        uint32_t key = 0u;
+    for (int i = threadIdx.x; i < N; i += NT) {
+        unsigned long long pair = 0ull;  // (sorts last)
         if (i < C) {
-            key = blocks_of(lists[(int64_t)i * list_stride]) << 20;
+            uint32_t key = blocks_of(lists[(int64_t)i * list_stride]) << 20;
             for (int l = 0; l < message_layers && l < 2; ++l)
                 key |= blocks_of(message_lists[((int64_t)l * C + i) * message_list_stride]) << (10 - 10 * l);
+            // descending by key, then ascending by clause: ~clause in the low word
+            pair = ((unsigned long long)key << 32) | (uint32_t)(0x7FFFFFFF - i);
         }
-        keys[i] = key;
+        order_keys[i] = pair;
     }
+    for (int q = threadIdx.x; q < streams; q += NT)
+        table[(int64_t)q * alive_stride] = q < C ? (uint32_t)((C - q + streams - 1) / streams) : 0u;
     __syncthreads();
-    const int c = blockIdx.x * NARROW_ORDER_BLOCK + threadIdx.x;
-    // (a stream beyond the last clause has none: the launch has at least NARROW_ORDER_BLOCK >= streams threads)
-    if (c < streams) table[(int64_t)c * alive_stride] = c < C ? (uint32_t)((C - c + streams - 1) / streams) : 0u;
-    if (c >= C) return;
-    const uint32_t mine = keys[c];
-    // rank = clauses with a greater key, or the same key and a smaller number; four keys per LDS read
-    int rank = 0;
-    const uint4 *four = reinterpret_cast<const uint4 *>(keys);
-    for (int i = 0; i < padded / 4; ++i) {
-        const uint4 v = four[i];
-        const uint32_t k[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int at = 4 * i + u;
-            rank += (k[u] > mine || (k[u] == mine && at < c)) && at < C;
+    for (int k = 2; k <= N; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = threadIdx.x; i < N; i += NT) {
+                const int partner = i ^ j;
+                if (partner > i) {
+                    const unsigned long long a = order_keys[i], b = order_keys[partner];
+                    const bool descending = (i & k) == 0;
+                    if (descending ? a < b : a > b) order_keys[i] = b, order_keys[partner] = a;
+                }
+            }
+            __syncthreads();
         }
-    }
-    table[(int64_t)(rank % streams) * alive_stride + 1 + rank / streams] = (uint32_t)c;
+    for (int rank = threadIdx.x; rank < C; rank += NT)
+        table[(int64_t)(rank % streams) * alive_stride + 1 + rank / streams] = 0x7FFFFFFFu - (uint32_t)order_keys[rank];
 }
 
 template <int SRC, bool LAST, int GROUP, int WPL>
