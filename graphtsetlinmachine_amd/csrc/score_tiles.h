@@ -280,22 +280,38 @@ __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int 
     // With negated literals as complements of rows (half > 0: message layers) the list comes in two parts, each a
     // whole number of 8-entry blocks: the rows to AND, then the rows whose complements to AND - a block is all of
     // one kind, so the evaluation needs no per-entry flag.  `plain`: entries of the first part.
-    int plain = n;
-    for (int r0 = 0; r0 < literals; r0 += 64) {
-        const int r = r0 + lane;
-        const uint32_t lit = r < literals ? (order ? order[r] : (uint32_t)r) : 0u;
-        uint32_t word = inc[(int64_t)(lit >> 5) * B];
-        if ((int)(lit >> 5) == chunks - 1) word &= filter;
-        plain += __popcll(__ballot(r < literals && (half == 0 || (int)lit < half) && ((word >> (lit & 31)) & 1u)));
+    // (the number of entries of the first part is a count of include bits: no walk needed for it)
+    int plain = 0;
+    for (int w = lane; w < chunks; w += 64) {
+        uint32_t word = inc[(int64_t)w * B];
+        if (w == chunks - 1) word &= filter;
+        if (half > 0) word = w < (half >> 5) ? word : w == (half >> 5) ? word & ((1u << (half & 31)) - 1u) : 0u;
+        plain += __popc(word);
     }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) plain += __shfl_xor(plain, off);
+    plain += n;
     const int plain_padded = (plain + 7) & ~7;
+    // With at most 64 include words lane w keeps word w, and a literal's bit comes by a lane read instead of a
+    // load that depends on the load of `order`.
+    const bool in_lanes = chunks <= 64;
+    uint32_t word_of_lane = 0u;
+    if (in_lanes && lane < chunks) {
+        word_of_lane = inc[(int64_t)lane * B];
+        if (lane == chunks - 1) word_of_lane &= filter;
+    }
     int n_neg = 0;
     for (int r0 = 0; r0 < literals; r0 += 64) {
         int r = r0 + lane;
         uint32_t lit = r < literals ? (order ? order[r] : (uint32_t)r) : 0u;
         uint32_t w = lit >> 5;
-        uint32_t word = inc[(int64_t)w * B];
-        if ((int)w == chunks - 1) word &= filter;
+        uint32_t word;
+        if (in_lanes) {
+            word = (uint32_t)__shfl((int)word_of_lane, (int)w);
+        } else {
+            word = inc[(int64_t)w * B];
+            if ((int)w == chunks - 1) word &= filter;
+        }
         const bool included = r < literals && ((word >> (lit & 31)) & 1u);
         const bool negated = included && half > 0 && (int)lit >= half;
         const unsigned long long below = (1ull << lane) - 1ull;
