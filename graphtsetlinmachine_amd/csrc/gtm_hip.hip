@@ -1314,7 +1314,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     // layer 0 on narrow tiles takes its clauses by length (GTM_NARROW_IN_ORDER, tuning and test aid: by number)
     const bool by_length = half_rows0 && d.C <= NARROW_ORDER_MAX_CLAUSES && !tune(T_NARROW_IN_ORDER);
     if (by_length) {
-        size_t pairs = 1;
+        size_t pairs = 2;
         while (pairs < (size_t)d.C) pairs <<= 1;
         hipLaunchKernelGGL(k_narrow_stream_order, dim3(1), dim3(NARROW_ORDER_BLOCK), pairs * 8, st, w.lists, w.list_stride,
                            w.message_lists, w.message_list_stride, narrow_messages ? layers - 1 : 0, d.C, shape.streams(),

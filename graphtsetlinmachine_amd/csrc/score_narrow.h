@@ -179,34 +179,52 @@ __global__ __launch_bounds__(NARROW_ORDER_BLOCK) void k_narrow_stream_order(cons
                                                                            uint32_t *__restrict__ table) {
     extern __shared__ unsigned long long order_keys[];
     constexpr int NT = NARROW_ORDER_BLOCK;
-    int N = 1;
+    constexpr int AT_ONCE = 4;  // independent loads (keys) or exchanges (sort) a thread has under way
+    int N = 2;
     while (N < C) N <<= 1;
     auto blocks_of = [](uint32_t header) {
         const uint32_t n = (header & 0xFFFFu) + (header >> 16);
         return n < 1023u ? n : 1023u;
     };
-    for (int i = threadIdx.x; i < N; i += NT) {
-        unsigned long long pair = 0ull;  // (sorts last)
-        if (i < C) {
-            uint32_t key = blocks_of(lists[(int64_t)i * list_stride]) << 20;
-            for (int l = 0; l < message_layers && l < 2; ++l)
-                key |= blocks_of(message_lists[((int64_t)l * C + i) * message_list_stride]) << (10 - 10 * l);
-            // descending by key, then ascending by clause: ~clause in the low word
-            pair = ((unsigned long long)key << 32) | (uint32_t)(0x7FFFFFFF - i);
+    for (int i0 = threadIdx.x; i0 < N; i0 += NT * AT_ONCE) {
+        uint32_t h[AT_ONCE][3];
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; ++u) {
+            const int i = i0 + u * NT;
+            h[u][0] = i < C ? lists[(int64_t)i * list_stride] : 0u;
+#pragma unroll
+            for (int l = 0; l < 2; ++l)
+                h[u][1 + l] = i < C && l < message_layers ? message_lists[((int64_t)l * C + i) * message_list_stride] : 0u;
         }
-        order_keys[i] = pair;
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; ++u) {
+            const int i = i0 + u * NT;
+            const uint32_t key = blocks_of(h[u][0]) << 20 | blocks_of(h[u][1]) << 10 | blocks_of(h[u][2]);
+            // descending by key, then ascending by clause: ~clause in the low word; what fills the table up sorts last
+            if (i < N) order_keys[i] = i < C ? ((unsigned long long)key << 32) | (uint32_t)(0x7FFFFFFF - i) : 0ull;
+        }
     }
     for (int q = threadIdx.x; q < streams; q += NT)
         table[(int64_t)q * alive_stride] = q < C ? (uint32_t)((C - q + streams - 1) / streams) : 0u;
     __syncthreads();
+    // thread t takes the exchanges t, t + NT, ... of a stage: exchange e is between places i = e with a zero bit
+    // inserted at bit log2(j), and i + j
     for (int k = 2; k <= N; k <<= 1)
         for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int i = threadIdx.x; i < N; i += NT) {
-                const int partner = i ^ j;
-                if (partner > i) {
-                    const unsigned long long a = order_keys[i], b = order_keys[partner];
-                    const bool descending = (i & k) == 0;
-                    if (descending ? a < b : a > b) order_keys[i] = b, order_keys[partner] = a;
+            for (int e0 = threadIdx.x; e0 < N / 2; e0 += NT * AT_ONCE) {
+                unsigned long long a[AT_ONCE], b[AT_ONCE];
+                int at[AT_ONCE];
+#pragma unroll
+                for (int u = 0; u < AT_ONCE; ++u) {
+                    const int e = e0 + u * NT;
+                    at[u] = e < N / 2 ? ((e & ~(j - 1)) << 1) | (e & (j - 1)) : -1;
+                    a[u] = at[u] >= 0 ? order_keys[at[u]] : 0ull;
+                    b[u] = at[u] >= 0 ? order_keys[at[u] + j] : 0ull;
+                }
+#pragma unroll
+                for (int u = 0; u < AT_ONCE; ++u) {
+                    const bool descending = (at[u] & k) == 0;
+                    if (at[u] >= 0 && (descending ? a[u] < b[u] : a[u] > b[u])) order_keys[at[u]] = b[u], order_keys[at[u] + j] = a[u];
                 }
             }
             __syncthreads();
