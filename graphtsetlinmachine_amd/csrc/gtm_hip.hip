@@ -666,7 +666,7 @@ struct ScoreWs {
     uint32_t *message_rows;   // [tiles per launch][M + 2][tw]  (tile path, depth > 1)
     uint32_t *bit_start, *bit_cursor, *bit_clauses;  // [M + 1], [M], [C * MB]: the clauses of every message bit (tile path, depth > 1)
     uint32_t *alive[2];       // [tiles per launch][streams][alive_stride] clauses still true somewhere in a tile, layer to layer
-    uint32_t *stream_order;   // [streams][alive_stride] every clause, by length of its layer-0 list (k_narrow_stream_order)
+    uint32_t *stream_order;   // [streams][alive_stride] every clause, by length of its lists (k_narrow_order_keys, _ranks), then [C] keys
     size_t alive_words;       // room per tile
     TileSegment *segments;    // [tiles + 2 * TILE_SEGMENTS_MAX_SHARES] which clauses of which tile a workgroup takes (half tiles)
     size_t vector_words;      // words of sent (and of got)
@@ -699,7 +699,8 @@ ScoreWs carve_score(const Dims &d, const gtm_config *cfg, int batch, char *base,
     w.list_stride = clause_list_stride(cfg->literals);
     w.lists = (uint32_t *)take((size_t)d.C * w.list_stride * 4);
     w.wt = (int32_t *)take((size_t)d.C * d.K * 4);
-    if (tg) w.stream_order = (uint32_t *)take(((size_t)d.C + 2 * NARROW_MAX_STREAMS) * 4);
+    // (+ a key per clause after the table)
+    if (tg) w.stream_order = (uint32_t *)take((2 * (size_t)d.C + 2 * NARROW_MAX_STREAMS) * 4);
     if (tg && cfg->depth == 1 && tg->half)
         w.segments = (TileSegment *)take(((size_t)tg->n_tiles + 2 * TILE_SEGMENTS_MAX_SHARES) * sizeof(TileSegment));
     if (tg && cfg->depth == 1 && !keep_rows) {
@@ -1314,12 +1315,14 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     // layer 0 on narrow tiles takes its clauses by length (GTM_NARROW_IN_ORDER, tuning and test aid: by number)
     const bool by_length = half_rows0 && d.C <= NARROW_ORDER_MAX_CLAUSES && !tune(T_NARROW_IN_ORDER);
     if (by_length) {
-        size_t pairs = 2;
-        while (pairs < (size_t)d.C) pairs <<= 1;
-        hipLaunchKernelGGL(k_narrow_stream_order, dim3(1), dim3(NARROW_ORDER_BLOCK), pairs * 8, st, w.lists, w.list_stride,
-                           w.message_lists, w.message_list_stride, narrow_messages ? layers - 1 : 0, d.C, shape.streams(),
-                           narrow_alive_stride(d.C, shape.streams()), w.stream_order);
-        if (int rc = check_launch("narrow_stream_order")) return rc;
+        uint32_t *keys = w.stream_order + (size_t)d.C + 2 * NARROW_MAX_STREAMS;
+        hipLaunchKernelGGL(k_narrow_order_keys, dim3(blocks_for(d.C, NARROW_ORDER_BLOCK)), dim3(NARROW_ORDER_BLOCK), 0, st,
+                           w.lists, w.list_stride, w.message_lists, w.message_list_stride, narrow_messages ? layers - 1 : 0,
+                           d.C, shape.streams(), narrow_alive_stride(d.C, shape.streams()), keys, w.stream_order);
+        if (int rc = check_launch("narrow_order_keys")) return rc;
+        hipLaunchKernelGGL(k_narrow_order_ranks, dim3(blocks_for(d.C, NARROW_ORDER_BLOCK / 64)), dim3(NARROW_ORDER_BLOCK), 0,
+                           st, keys, d.C, shape.streams(), narrow_alive_stride(d.C, shape.streams()), w.stream_order);
+        if (int rc = check_launch("narrow_order_ranks")) return rc;
     }
     TileLayerArgs a{};
     a.tiles = g->tiles;

@@ -66,7 +66,7 @@ struct NarrowArgs {
                                // that are true somewhere in the tile; NULL: every clause (q, q + streams, ...) is looked at
     uint32_t *alive_out;       // the same for the next layer, or NULL
     int alive_stride;          // >= 1 + ceil(C / streams)
-    int alive_in_shared;       // alive_in is ONE set of lists for every tile (k_narrow_stream_order: all clauses, by length)
+    int alive_in_shared;       // alive_in is ONE set of lists for every tile (k_narrow_order_ranks: all clauses, by length)
     int hv, n_types;           // ROWS_HALF: positive literals (= LDS rows before the node-type rows), node types
     int row_words;             // words from one row to the next in LDS (>= tw, a multiple of 4): what the lists' entries count in
 };
@@ -167,70 +167,55 @@ typedef uint32_t NarrowEntries __attribute__((ext_vector_type(4)));  // four ent
 // lists has been walked, hold lists of nearly the same length at every step, and a workgroup's long clauses come
 // first.  The message layers take their clauses in the same order, as far as they are still alive, so among the
 // clauses of one length in layer 0 (there are few different lengths) the order is by the length in the first
-// message layer, then the second.  Ties by clause number: the table is the same from call to call.  One workgroup
-// sorts (key, clause) pairs in LDS (bitonic, 8 bytes per clause rounded up to a power of two); the lengths come
-// from entry 0 of each list: blocks of rows | blocks of complements << 16.
-constexpr int NARROW_ORDER_BLOCK = 1024;
-constexpr int NARROW_ORDER_MAX_CLAUSES = 8192;  // 64 KB of LDS
-__global__ __launch_bounds__(NARROW_ORDER_BLOCK) void k_narrow_stream_order(const uint32_t *__restrict__ lists, int list_stride,
-                                                                           const uint32_t *__restrict__ message_lists,
-                                                                           int message_list_stride, int message_layers,
-                                                                           int C, int streams, int alive_stride,
-                                                                           uint32_t *__restrict__ table) {
-    extern __shared__ unsigned long long order_keys[];
-    constexpr int NT = NARROW_ORDER_BLOCK;
-    constexpr int AT_ONCE = 4;  // independent loads (keys) or exchanges (sort) a thread has under way
-    int N = 2;
-    while (N < C) N <<= 1;
+// message layer, then the second.  Ties by clause number: the table is the same from call to call.  Two launches:
+// a key per clause (from entry 0 of each of its lists: blocks of rows | blocks of complements << 16), then a wave
+// per clause that finds the clause's rank by counting the keys before its own, 64 at a time - work for the whole
+// chip (a sort in one workgroup's LDS took 130 us for 8,000 clauses, this takes a fifth).
+constexpr int NARROW_ORDER_BLOCK = 256;
+constexpr int NARROW_ORDER_MAX_CLAUSES = 32768;
+__global__ __launch_bounds__(NARROW_ORDER_BLOCK) void k_narrow_order_keys(const uint32_t *__restrict__ lists, int list_stride,
+                                                                         const uint32_t *__restrict__ message_lists,
+                                                                         int message_list_stride, int message_layers,
+                                                                         int C, int streams, int alive_stride,
+                                                                         uint32_t *__restrict__ keys, uint32_t *__restrict__ table) {
+    const int c = blockIdx.x * NARROW_ORDER_BLOCK + threadIdx.x;
+    // (a stream beyond the last clause has none; the launch has at least NARROW_ORDER_BLOCK >= streams threads)
+    if (c < streams) table[(int64_t)c * alive_stride] = c < C ? (uint32_t)((C - c + streams - 1) / streams) : 0u;
+    if (c >= C) return;
     auto blocks_of = [](uint32_t header) {
         const uint32_t n = (header & 0xFFFFu) + (header >> 16);
         return n < 1023u ? n : 1023u;
     };
-    for (int i0 = threadIdx.x; i0 < N; i0 += NT * AT_ONCE) {
-        uint32_t h[AT_ONCE][3];
+    uint32_t h[3];
+    h[0] = lists[(int64_t)c * list_stride];
 #pragma unroll
-        for (int u = 0; u < AT_ONCE; ++u) {
-            const int i = i0 + u * NT;
-            h[u][0] = i < C ? lists[(int64_t)i * list_stride] : 0u;
+    for (int l = 0; l < 2; ++l) h[1 + l] = l < message_layers ? message_lists[((int64_t)l * C + c) * message_list_stride] : 0u;
+    keys[c] = blocks_of(h[0]) << 20 | blocks_of(h[1]) << 10 | blocks_of(h[2]);
+}
+static_assert(NARROW_ORDER_BLOCK >= NARROW_MAX_STREAMS, "one thread per stream writes its count");
+
+__global__ __launch_bounds__(NARROW_ORDER_BLOCK) void k_narrow_order_ranks(const uint32_t *__restrict__ keys, int C, int streams,
+                                                                          int alive_stride, uint32_t *__restrict__ table) {
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.x * (NARROW_ORDER_BLOCK / 64) + (threadIdx.x >> 6);
+    if (c >= C) return;  // (whole waves)
+    const uint32_t mine = keys[c];
+    // clauses that come before this one: a greater key, or the same key and a smaller number
+    int before = 0;
+    for (int i0 = 0; i0 < C; i0 += 256) {
+        uint32_t k[4];
 #pragma unroll
-            for (int l = 0; l < 2; ++l)
-                h[u][1 + l] = i < C && l < message_layers ? message_lists[((int64_t)l * C + i) * message_list_stride] : 0u;
+        for (int u = 0; u < 4; ++u) {
+            const int i = i0 + 64 * u + lane;
+            k[u] = i < C ? keys[i] : 0u;
         }
 #pragma unroll
-        for (int u = 0; u < AT_ONCE; ++u) {
-            const int i = i0 + u * NT;
-            const uint32_t key = blocks_of(h[u][0]) << 20 | blocks_of(h[u][1]) << 10 | blocks_of(h[u][2]);
-            // descending by key, then ascending by clause: ~clause in the low word; what fills the table up sorts last
-            if (i < N) order_keys[i] = i < C ? ((unsigned long long)key << 32) | (uint32_t)(0x7FFFFFFF - i) : 0ull;
+        for (int u = 0; u < 4; ++u) {
+            const int i = i0 + 64 * u + lane;
+            before += __popcll(__ballot(i < C && (k[u] > mine || (k[u] == mine && i < c))));
         }
     }
-    for (int q = threadIdx.x; q < streams; q += NT)
-        table[(int64_t)q * alive_stride] = q < C ? (uint32_t)((C - q + streams - 1) / streams) : 0u;
-    __syncthreads();
-    // thread t takes the exchanges t, t + NT, ... of a stage: exchange e is between places i = e with a zero bit
-    // inserted at bit log2(j), and i + j
-    for (int k = 2; k <= N; k <<= 1)
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int e0 = threadIdx.x; e0 < N / 2; e0 += NT * AT_ONCE) {
-                unsigned long long a[AT_ONCE], b[AT_ONCE];
-                int at[AT_ONCE];
-#pragma unroll
-                for (int u = 0; u < AT_ONCE; ++u) {
-                    const int e = e0 + u * NT;
-                    at[u] = e < N / 2 ? ((e & ~(j - 1)) << 1) | (e & (j - 1)) : -1;
-                    a[u] = at[u] >= 0 ? order_keys[at[u]] : 0ull;
-                    b[u] = at[u] >= 0 ? order_keys[at[u] + j] : 0ull;
-                }
-#pragma unroll
-                for (int u = 0; u < AT_ONCE; ++u) {
-                    const bool descending = (at[u] & k) == 0;
-                    if (at[u] >= 0 && (descending ? a[u] < b[u] : a[u] > b[u])) order_keys[at[u]] = b[u], order_keys[at[u] + j] = a[u];
-                }
-            }
-            __syncthreads();
-        }
-    for (int rank = threadIdx.x; rank < C; rank += NT)
-        table[(int64_t)(rank % streams) * alive_stride + 1 + rank / streams] = 0x7FFFFFFFu - (uint32_t)order_keys[rank];
+    if (lane == 0) table[(int64_t)(before % streams) * alive_stride + 1 + before / streams] = (uint32_t)c;
 }
 
 template <int SRC, bool LAST, int GROUP, int WPL>
