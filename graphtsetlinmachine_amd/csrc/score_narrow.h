@@ -161,6 +161,30 @@ struct NarrowRow {
 
 typedef uint32_t NarrowEntries __attribute__((ext_vector_type(4)));  // four entries of a compiled list
 
+// What the first lane of this lane's group of GROUP (16 or 8) lanes holds: a lane move inside the row of 16.
+template <int GROUP>
+__device__ __forceinline__ uint32_t narrow_group_first(uint32_t v, int lane) {
+    const uint32_t of_row = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x150, 0xF, 0xF, true);  // row_share:0
+    if (GROUP == 16) return of_row;
+    const uint32_t of_upper = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x158, 0xF, 0xF, true);  // row_share:8
+    return (lane & 8) ? of_upper : of_row;
+}
+
+// The greatest of a value that is the same in all lanes of a group, over the groups of the wave (wave-uniform):
+// the rows of 16 lanes hand their value on to the next row and then to the upper half (row_bcast), lane 63 has it.
+template <int GROUP>
+__device__ __forceinline__ int narrow_max_over_groups(int v, int lane) {
+    if (GROUP == 8) {
+        const int other = __builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, true);  // row_ror:8: the row's other group
+        v = v > other ? v : other;
+    }
+    const int from_row_before = __builtin_amdgcn_update_dpp(v, v, 0x142, 0xA, 0xF, false);  // row_bcast:15, rows 1 and 3
+    v = v > from_row_before ? v : from_row_before;
+    const int from_lower_half = __builtin_amdgcn_update_dpp(v, v, 0x143, 0xC, 0xF, false);  // row_bcast:31, rows 2 and 3
+    v = v > from_lower_half ? v : from_lower_half;
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
 // Which clauses a stream takes when every clause is looked at (layer 0), in the format of the lists of clauses
 // still alive: the clauses by falling length of their compiled lists, dealt out to the streams in turn - stream q
 // takes ranks q, q + streams, ... - so that the groups of a wave, which stay together until the longest of their
@@ -278,6 +302,8 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
     uint32_t *my_list = lists + q * Shape::LIST_WORDS;
     const uint32_t *quad_entry = my_list + (lane & 3);
     const uint32_t ones_entry = (uint32_t)(rows_lds - 1 - (SRC == ROWS_MESSAGES ? 1 : 0)) * (uint32_t)rw * 4u;
+    uint32_t ones_in_lane = ones_entry;  // (in a vector register: as a scalar operand of a select it costs a move each time)
+    asm volatile("" : "+v"(ones_in_lane));
     // this group's lanes in a 64-bit vote: bits shift .. shift + GROUP - 1 of its low or high half
     const bool upper_half = lane >= 32;
     const uint32_t shift = (uint32_t)(group * GROUP) & 31u;
@@ -361,19 +387,12 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
             else
                 acc.fill(active && has ? 0xFFFFFFFFu : 0u);
             // header (entry 0, in lane 0 of each group): blocks of rows to AND | blocks of rows whose complements to AND << 16
-            uint32_t header = 0u;
-#pragma unroll
-            for (int g = 0; g < PER; ++g) {
-                const uint32_t h = __builtin_amdgcn_readlane(now.e[0].x, g * GROUP);
-                header = group == g ? h : header;
-            }
+            const uint32_t header = narrow_group_first<GROUP>(now.e[0].x, lane);
             int plain = (int)(header & 0xFFFFu), nb = plain + (int)(header >> 16);
             unsigned long long nzw = __ballot(acc.any());
             const bool arrived_alive = votes_of_group(nzw) != 0u;
             if (!has || !arrived_alive) nb = 0, plain = 0;
-            int nb_most = 0;
-#pragma unroll
-            for (int g = 0; g < PER; ++g) nb_most = max(nb_most, __builtin_amdgcn_readlane(nb, g * GROUP));
+            const int nb_most = narrow_max_over_groups<GROUP>(nb, lane);
             // does some group have a live clause with blocks left from block b on?
             auto work_left = [&](int b) { return __ballot(b < nb && votes_of_group(nzw) != 0u) != 0ull; };
 
@@ -392,8 +411,8 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
                 // whose list has no such window (it ended in an earlier one; no clause; a clause false everywhere on
                 // arrival: nb = 0) walks the all-ones row while the others go on.
                 const bool past = b0 * 8 >= ((nb * 8 + NARROW_LIST_AHEAD - 1) & ~(NARROW_LIST_AHEAD - 1));
-                if (past) e = NarrowEntries(ones_entry);
-                if (b0 == 0 && gl == 0) e.x = ones_entry;  // in the place of the header
+                if (past) e = NarrowEntries(ones_in_lane);
+                if (b0 == 0 && gl == 0) e.x = ones_in_lane;  // in the place of the header
                 *reinterpret_cast<NarrowEntries *>(my_list + 4 * gl) = e;
                 // (a wave's LDS accesses are carried out in order: the reads below see the entries just written)
                 const int lim_most = nb_most - b0 < WINDOW / 8 ? nb_most - b0 : WINDOW / 8;
