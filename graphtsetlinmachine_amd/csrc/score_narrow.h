@@ -140,6 +140,10 @@ __device__ __forceinline__ uint32_t narrow_and3(uint32_t a, uint32_t b, uint32_t
     return (uint32_t)__builtin_amdgcn_bitop3_b32((int)a, (int)b, (int)c, 0x80);
 }
 
+typedef uint32_t narrow_u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t narrow_u32x4 __attribute__((ext_vector_type(4)));
+constexpr int NARROW_BUFFER_FLAGS = 0x00020000;  // last word of a buffer descriptor for plain 32-bit data on this GPU family
+
 // The WPL words of a row that a lane holds (a native vector: the values stay in registers through copies and selects).
 template <int WPL>
 struct NarrowRow {
@@ -157,6 +161,29 @@ struct NarrowRow {
     }
     __device__ __forceinline__ void load(const uint32_t *p) { w = *reinterpret_cast<const Vec *>(p); }
     __device__ __forceinline__ void store(uint32_t *p) const { *reinterpret_cast<Vec *>(p) = w; }
+    // through a buffer descriptor, at a 32-bit byte offset (no 64-bit address arithmetic per lane)
+    __device__ __forceinline__ void load_at(__amdgpu_buffer_rsrc_t buffer, uint32_t at) {
+        if (WPL == 2) {
+            const narrow_u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(buffer, (int)at, 0, 0);
+            w[0] = v.x, w[1] = v.y;
+        } else {
+            const narrow_u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(buffer, (int)at, 0, 0);
+#pragma unroll
+            for (int u = 0; u < WPL; ++u) w[u] = v[u];
+        }
+    }
+    __device__ __forceinline__ void store_at(__amdgpu_buffer_rsrc_t buffer, uint32_t at) const {
+        if (WPL == 2) {
+            narrow_u32x2 v;
+            v.x = w[0], v.y = w[1];
+            __builtin_amdgcn_raw_buffer_store_b64(v, buffer, (int)at, 0, 0);
+        } else {
+            narrow_u32x4 v;
+#pragma unroll
+            for (int u = 0; u < WPL; ++u) v[u] = w[u];
+            __builtin_amdgcn_raw_buffer_store_b128(v, buffer, (int)at, 0, 0);
+        }
+    }
 };
 
 typedef uint32_t NarrowEntries __attribute__((ext_vector_type(4)));  // four entries of a compiled list
@@ -264,6 +291,11 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int q = PER * wave + group;  // this group's stream
     uint32_t *bitmap = a.bitmap + (int64_t)tile_local * C * tw;
+    // the compiled lists and this tile's truth rows, each through a buffer descriptor: an access is a multiply-add of
+    // 24-bit factors per lane (clause x bytes per clause + the lane's place), not a 64-bit multiply and add
+    const __amdgpu_buffer_rsrc_t lists_buffer =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(a.lists), 0, C * a.stride * 4, NARROW_BUFFER_FLAGS);
+    const __amdgpu_buffer_rsrc_t truth_buffer = __builtin_amdgcn_make_buffer_rsrc(bitmap, 0, C * tw * 4, NARROW_BUFFER_FLAGS);
 
     {  // rows -> LDS, 16 bytes per thread and trip, four loads in flight
         const uint4 *src;
@@ -357,11 +389,12 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
         }
         it.c = clause_of(i);
         const int c = it.c < 0 ? 0 : it.c;
-        const NarrowEntries *list = reinterpret_cast<const NarrowEntries *>(a.lists + (int64_t)c * a.stride + 4 * gl);
+        const uint32_t list_at = __umul24((uint32_t)c, (uint32_t)a.stride * 4u) + 16u * (uint32_t)gl;
 #pragma unroll
-        for (int v = 0; v < AHEAD_W; ++v) it.e[v] = list[v * (WINDOW / 4)];  // (a list is at least 128 entries long)
+        for (int v = 0; v < AHEAD_W; ++v)  // (a list is at least 128 entries long)
+            it.e[v] = __builtin_amdgcn_raw_buffer_load_b128(lists_buffer, (int)list_at + v * WINDOW * 4, 0, 0);
         it.truth.fill(0u);
-        if (SRC == ROWS_MESSAGES) it.truth.load(bitmap + (int64_t)c * tw + (active ? WPL * gl : 0));
+        if (SRC == ROWS_MESSAGES) it.truth.load_at(truth_buffer, __umul24((uint32_t)c, (uint32_t)tw * 4u) + (active ? 4u * WPL * gl : 0u));
     };
 
     // NARROW_AHEAD items are under way per stream: a clause's list and truth words come from L2 or further, a few
@@ -405,7 +438,8 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
 #pragma unroll
                     for (int v = 1; v < AHEAD_W; ++v) e = window == v ? now.e[v] : e;
                 } else {  // (a clause of more literals than that: its further windows are fetched when it gets there)
-                    e = *reinterpret_cast<const NarrowEntries *>(a.lists + (int64_t)c * a.stride + b0 * 8 + 4 * gl);
+                    e = __builtin_amdgcn_raw_buffer_load_b128(
+                        lists_buffer, (int)(__umul24((uint32_t)c, (uint32_t)a.stride * 4u) + 32u * (uint32_t)b0 + 16u * (uint32_t)gl), 0, 0);
                 }
                 // The compiled list is filled up with the all-ones row to a whole number of 128 entries.  A group
                 // whose list has no such window (it ended in an earlier one; no clause; a clause false everywhere on
@@ -471,7 +505,8 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
             if (has) {
                 if (!LAST) {
                     // (a clause that was false everywhere on arrival has its row of zeros in place already)
-                    if (active && (SRC == ROWS_HALF || arrived_alive)) acc.store(bitmap + (int64_t)c * tw + WPL * gl);
+                    if (active && (SRC == ROWS_HALF || arrived_alive))
+                        acc.store_at(truth_buffer, __umul24((uint32_t)c, (uint32_t)tw * 4u) + 4u * WPL * gl);
                     if (seg_out && nzg != 0u) {
                         if (gl == 0) seg_out[1 + n_out] = (uint32_t)c;
                         ++n_out;
