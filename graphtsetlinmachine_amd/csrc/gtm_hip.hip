@@ -1274,7 +1274,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     const int row_words_m = narrow_messages && !as_stored
                                 ? narrow_row_words(tg, shape, d.K, tile_message_rows(d.M), lds_limit) : tg.tw;
     // compiled clause: 8 words of packed 16-bit row entries (16 words of byte offsets on half tiles) + the include words
-    const int stride0 = half_rows0 ? w.list_stride : tg.half ? 16 + d.LA : two_phase ? 8 + d.LA : w.list_stride;
+    const int stride0 = half_rows0 ? w.list_stride : tg.half ? 16 + d.LA + HALF_RECORD_EXTRA_WORDS : two_phase ? 8 + d.LA : w.list_stride;
     SegmentPlan plan{};
     if (half_rows0)
         // rows as k_tile_layer_narrow<ROWS_HALF> stages them: positive literals, node types, all ones

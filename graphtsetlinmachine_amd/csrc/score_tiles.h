@@ -1782,20 +1782,28 @@ __device__ __forceinline__ void tile_segments_part(const SegmentPlan &sp, int bl
 // twice the graphs per tile: the scalar work, the address arithmetic and the phase-2 loads
 // of a (clause, tile) pair are spread over twice as many graphs.
 //
-// Compiled clause, 16 + LA words: 16 entries of 32 bits, then the include words.  Entry 0 =
-// variant (7 or 15 rows) | needs-phase-2 << 8 | positive pairs << 12; the others are rows as
+// Compiled clause, 16 + LA + 4 words: 16 entries of 32 bits, the include words, two more entries.  Entry 0 =
+// rows in use (7 or 17) | needs-phase-2 << 8 | positive pairs << 12; the others are rows as
 // LDS byte offsets, ready for use (a scalar load puts them in registers): entry 1 = the
-// node-type row; then literal rows in PAIRS, 3 or 7 of them: first the pairs of positive
+// node-type row; then literal rows in PAIRS, 3 or 8 of them (rows 15 and 16 are the two
+// entries after the include words): first the pairs of positive
 // literals (an odd one out is paired with the all-ones row), then the pairs of negated
 // ones (padded with the all-zero words that follow the rows in LDS).  With the signs fixed
 // per pair, a pair costs one 3-input bit operation per word of the lane - acc & a & b or
-// acc & ~(a | b) - and the clause's pattern (how many positive pairs) selects one of 8
+// acc & ~(a | b) - and the clause's pattern (how many positive pairs) selects one of 9
 // straight-line variants with a single scalar jump.
-// The filter takes the clause's rarest literals, at most 14, as many as fit the pairs.
+// The filter takes the clause's rarest literals, at most 16, as many as fit the pairs: measured on the
+// 361-node workload after one epoch, 6 pairs 0.409 ms per 10,000 graphs, 7 pairs 0.358, 8 pairs 0.353 - a
+// stronger filter leaves fewer lanes with candidates whose tests wait for memory in the open.
 
 struct alignas(16) Entries16 {
     uint32_t v[16];
 };
+
+// Row pairs that phase 1 of the half-tile kernel ANDs for a clause of many literals.  A record is 16 entries (header,
+// node-type row, 14 rows), the include words, and the rows past the 14th (4 words kept for them).
+constexpr int HALF_BIG_PAIRS = 8;
+constexpr int HALF_RECORD_EXTRA_WORDS = 4;
 
 // Index of the lowest set bit, ~0 for 0: what the instruction gives by itself (the compiler's count of trailing
 // zeros is either undefined for 0 or comes with a comparison and a select for it).
@@ -1815,7 +1823,7 @@ __global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C,
                                        int literals, int n_types, int tw, const uint32_t *__restrict__ order,
                                        uint32_t *__restrict__ records, int record_words, int K,
                                        const int32_t *__restrict__ weights, int32_t *__restrict__ wt, SegmentPlan sp) {
-    __shared__ uint32_t chosen_of_wave[4][16];
+    __shared__ uint32_t chosen_of_wave[4][2 + 2 * HALF_BIG_PAIRS + 2];
     if (sp.cus > 0) tile_segments_part(sp, blockIdx.x, gridDim.x, threadIdx.x, blockDim.x);  // which workgroup takes what (see above)
     const int lane = threadIdx.x & 63;
     const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -1826,7 +1834,7 @@ __global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C,
     const uint32_t ones_row = (uint32_t)(hv + n_types), zero_row = ones_row + 1u;  // the zeroed words after the rows
     uint32_t *rec = records + (int64_t)c * record_words;
     const uint32_t *inc = bank + (int64_t)c * chunks * B + (B - 1);
-    // the clause's 14 rarest included literals, in `order`
+    // the clause's 16 rarest included literals, in `order`
     int n = 0;
     for (int r0 = 0; r0 < literals; r0 += 64) {
         const int r = r0 + lane;
@@ -1837,25 +1845,25 @@ __global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C,
         const bool included = r < literals && ((word >> (lit & 31)) & 1u);
         const unsigned long long mask = __ballot(included);
         const int at = n + __popcll(mask & ((1ull << lane) - 1ull));
-        if (included && at < 14) chosen[at] = lit;
+        if (included && at < 2 * HALF_BIG_PAIRS) chosen[at] = lit;
         n += __popcll(mask);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-    int taken = n < 14 ? n : 14;
+    int taken = n < 2 * HALF_BIG_PAIRS ? n : 2 * HALF_BIG_PAIRS;
     const uint32_t lit = lane < taken ? chosen[lane] : 0u;
     bool positive = lane < taken && (int)lit < hv, negative = lane < taken && (int)lit >= hv;
     int p = __popcll(__ballot(positive)), q = __popcll(__ballot(negative));
-    // 7 pairs hold p positives and q negatives if ceil(p / 2) + ceil(q / 2) <= 7: 14 literals with an
-    // odd number of each sign do not fit, and then the least rare of the 14 is left to phase 2
-    if (p + q == 14 && (p & 1)) {
+    // 8 pairs hold p positives and q negatives if ceil(p / 2) + ceil(q / 2) <= 8: 16 literals with an
+    // odd number of each sign do not fit, and then the least rare of the 16 is left to phase 2
+    if (p + q == 2 * HALF_BIG_PAIRS && (p & 1)) {
         --taken;
         if (lane == taken) positive = negative = false;
         p = __popcll(__ballot(positive)), q = __popcll(__ballot(negative));
     }
     const int a = (p + 1) >> 1, b = (q + 1) >> 1;
-    const int pairs = a + b <= 3 ? 3 : 7;
+    const int pairs = a + b <= 3 ? 3 : HALF_BIG_PAIRS;
     const int pos_rank = __popcll(__ballot(positive) & ((1ull << lane) - 1ull));
     const int neg_rank = __popcll(__ballot(negative) & ((1ull << lane) - 1ull));
     // the 16 entries are put together in LDS (a wave's LDS accesses are carried out in order) and
@@ -1863,9 +1871,9 @@ __global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C,
     uint32_t *slots = chosen;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
     __builtin_amdgcn_wave_barrier();
-    if (lane < 16) {
+    if (lane < 2 + 2 * HALF_BIG_PAIRS) {
         uint32_t v = (lane >= 2 && lane < 2 + 2 * a ? ones_row : zero_row) * row16;
-        if (lane == 0) v = (uint32_t)((pairs == 3 ? 7 : 15) | (n > taken ? 0x100 : 0) | (a << 12));
+        if (lane == 0) v = (uint32_t)((2 * pairs + 1) | (n > taken ? 0x100 : 0) | (a << 12));
         if (lane == 1) v = (uint32_t)(hv + c % n_types) * row16;
         slots[lane] = v;
     }
@@ -1877,6 +1885,8 @@ __global__ void k_compile_clauses_half(const uint32_t *__restrict__ bank, int C,
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
     if (lane < 16) rec[lane] = lane == 0 ? slots[0] : slots[lane] << 4;  // rows as byte offsets: nothing to unpack
+    // (entries past the 16th follow the include words)
+    if (lane >= 16 && lane < 2 + 2 * HALF_BIG_PAIRS) rec[16 + chunks + (lane - 16)] = slots[lane] << 4;
     for (int w = lane; w < chunks; w += 64) {
         uint32_t word = inc[(int64_t)w * B];
         if (w == chunks - 1) word &= filter;
@@ -2057,6 +2067,10 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         return r;
     };
 
+    // Fetching the words of a lane's SECOND surviving slot along with the first's (so that the turns in the open start
+    // at the third candidate) paid with 7 row pairs in phase 1 (0.361 -> 0.359 ms per 10,000 graphs); with 8 pairs there
+    // are fewer candidates, and its 8 registers are the ones the 16th row needs (with both, the compiler spills).
+    constexpr bool SECOND_AHEAD = false;
     struct Pending {
         LaneWords<LW> acc;
         uint2 x[LA4], x2[LA4];   // the words of the lane's first and (for the class sums) second surviving slot
@@ -2070,8 +2084,8 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
 
     // Phase 1 and the loads of phase 2.  Every load is issued by all lanes whatever the clause
     // does, so that the number of loads in flight is known when the pending clause is finished.
-    auto begin = [&](Pending &p, const Entries16 &rec, uint32_t weights_at, char *truth_out, const uint32_t *record_next,
-                     Entries16 &next) {
+    auto begin = [&](Pending &p, const Entries16 &rec, const uint2 rec_more, uint32_t weights_at, char *truth_out,
+                     const uint32_t *record_next, Entries16 &next, uint2 &next_more) {
         p.live = true;
         p.weights_at = weights_at;
         p.truth_out = truth_out;
@@ -2082,23 +2096,25 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         }
         const uint32_t header = rec.v[0] & 0xFFFFu;
         const uint32_t positive_pairs = header >> 12;
-        LaneWords<LW> acc, r[14];
+        LaneWords<LW> acc, r[2 * HALF_BIG_PAIRS];
         acc.load(col + entry_of(rec, 1));  // the node-type row: zero past the graphs' nodes and in unused lanes
         if (!FULL && !active)
 #pragma unroll
             for (int u = 0; u < LW; ++u) acc.w[u] = 0u;
         if ((header & 0xFFu) > 7u) {
 #pragma unroll
-            for (int i = 0; i < 14; ++i) r[i].load(col + entry_of(rec, i + 2));
+            for (int i = 0; i < 2 * HALF_BIG_PAIRS; ++i)
+                r[i].load(col + (i + 2 < 16 ? entry_of(rec, i + 2 < 16 ? i + 2 : 0) : i + 2 == 16 ? rec_more.x : rec_more.y));
             switch (positive_pairs) {
-                case 0: half_combine<LW, 7, 0>(acc, r); break;
-                case 1: half_combine<LW, 7, 1>(acc, r); break;
-                case 2: half_combine<LW, 7, 2>(acc, r); break;
-                case 3: half_combine<LW, 7, 3>(acc, r); break;
-                case 4: half_combine<LW, 7, 4>(acc, r); break;
-                case 5: half_combine<LW, 7, 5>(acc, r); break;
-                case 6: half_combine<LW, 7, 6>(acc, r); break;
-                default: half_combine<LW, 7, 7>(acc, r); break;
+                case 0: half_combine<LW, HALF_BIG_PAIRS, 0>(acc, r); break;
+                case 1: half_combine<LW, HALF_BIG_PAIRS, 1>(acc, r); break;
+                case 2: half_combine<LW, HALF_BIG_PAIRS, 2>(acc, r); break;
+                case 3: half_combine<LW, HALF_BIG_PAIRS, 3>(acc, r); break;
+                case 4: half_combine<LW, HALF_BIG_PAIRS, 4>(acc, r); break;
+                case 5: half_combine<LW, HALF_BIG_PAIRS, 5>(acc, r); break;
+                case 6: half_combine<LW, HALF_BIG_PAIRS, 6>(acc, r); break;
+                case 7: half_combine<LW, HALF_BIG_PAIRS, 7>(acc, r); break;
+                default: half_combine<LW, HALF_BIG_PAIRS, HALF_BIG_PAIRS>(acc, r); break;
             }
         } else {
 #pragma unroll
@@ -2113,6 +2129,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         // (the next record is requested only now: scalar loads and LDS reads are waited for with one counter, so a
         // request before the rows would have been waited for along with them)
         next = *reinterpret_cast<const Entries16 *>(record_next);
+        next_more = *reinterpret_cast<const uint2 *>(record_next + 16 + LA);
         // lowest surviving slot of the lane: the smallest of its words' lowest set bits (~0 for a word without
         // one, which survives the OR with the word's base and loses every comparison: no slot)
         uint32_t bit = lowest_bit_or_ones(acc.w[0]);
@@ -2127,7 +2144,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         p.bit = bit;
         // lanes with nothing to test all read the tile's first slot (one cache line for the wave)
         load_x(bit != ~0u ? x_lane + bit * (LA * 2u) : 0u, p.x);
-        if (LAST) {
+        if (LAST && SECOND_AHEAD) {
             // The second surviving slot's words come along: a first candidate fails often enough, and a test that
             // starts only then has its memory round trip in the open.
             const LaneWords<LW> after = without_lowest_bit(acc);
@@ -2158,8 +2175,8 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
             int slots_left = 0;
 #pragma unroll
             for (int u = 0; u < LW; ++u) slots_left += __popc(acc.w[u]);
-            bool holds = tested && (!violates(include, p.x) || (slots_left > 1 && !violates(include, p.x2)));
-            const bool more = tested && !holds && slots_left > 2;
+            bool holds = tested && (!violates(include, p.x) || (SECOND_AHEAD && slots_left > 1 && !violates(include, p.x2)));
+            const bool more = tested && !holds && slots_left > (SECOND_AHEAD ? 2 : 1);
             if (__ballot(more) == 0ull) {
                 nz = __ballot(holds);
                 settled = true;
@@ -2170,14 +2187,14 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
                 // rows of all the clause's literals are ANDed instead, below.)
                 // (the candidate under test is always the lowest set bit of the lane's words taken as one number W:
                 // W & (W - 1) takes it out)
-                LaneWords<LW> rest = without_lowest_bit(without_lowest_bit(acc));
+                LaneWords<LW> rest = SECOND_AHEAD ? without_lowest_bit(without_lowest_bit(acc)) : without_lowest_bit(acc);
                 int others = 0;
 #pragma unroll
                 for (int u = 0; u < LW; ++u) {
                     rest.w[u] = more ? rest.w[u] : 0u;
                     others += __popc(rest.w[u]);
                 }
-                if (__ballot(others + 1 >= TWO_PHASE_WALK_FROM) == 0ull) {
+                if (__ballot(others + (SECOND_AHEAD ? 1 : 0) >= TWO_PHASE_WALK_FROM) == 0ull) {
                     while (__ballot(any_bit(rest)) != 0ull) {
                         uint32_t bit = lowest_bit_or_ones(rest.w[0]);
 #pragma unroll
@@ -2304,6 +2321,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
     uint32_t wt_a = LAST ? (uint32_t)(first * K) * 4u : 0u;
     char *truth_a = reinterpret_cast<char *>(bitmap + (int64_t)first * tw + (active ? lane * LW : 0));
     Entries16 ea = *reinterpret_cast<const Entries16 *>(rec_a);
+    uint2 ea_more = *reinterpret_cast<const uint2 *>(rec_a + 16 + LA), eb_more;
     Pending pa, pb;
     pa.live = pb.live = false;
     uint32_t at_pending = at_a;  // the record of the clause in pb (a valid record while there is none)
@@ -2317,7 +2335,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         // so only one clause's are in registers at a time.
         Words<LA> include = load_include(at_pending);
         Entries16 eb;
-        begin(pa, ea, wt_a, truth_a, rec_b, eb);
+        begin(pa, ea, ea_more, wt_a, truth_a, rec_b, eb, eb_more);
         finish(pb, include);
         include = load_include(at_a);
         const bool has_a = c + 2 * NWAVES < c_end;
@@ -2327,7 +2345,7 @@ __global__ __launch_bounds__(NWAVES * 64) void k_tile_two_phase_half(TileLayerAr
         char *truth_next = has_a ? truth_b + truth_step : truth_b;
         // without a second clause this repeats the first one and drops the result: keeping the
         // sequence of loads the same on every trip lets the waits stay partial
-        begin(pb, eb, wt_b, truth_b, rec_a, ea);
+        begin(pb, eb, eb_more, wt_b, truth_b, rec_a, ea, ea_more);
         pb.live = has_b;
         finish(pa, include);
         wt_a = wt_next;
