@@ -35,11 +35,11 @@ VALU_PEAK_LANE_OPS = 256 * 64 * 2.4e9  # 32-bit integer lane operations per seco
 # library was built from another text reports no counters rather than stale ones.
 MEASURED_COUNTERS = {
     "convolutional_images": {
-        "kernel": "k_tile_two_phase_half<score>", "commit": "0b8a39e",
+        "kernel": "k_tile_two_phase_half<score>", "commit": "8762096",
         "functions": ("tile_segments_part", "lowest_bit_or_ones", "k_compile_clauses_half", "half_combine",
                       "k_tile_two_phase_half"),
-        "source_sha256": "aa6f35fefebbfc73cbc5809aca6174aac775082da891033a30514a7a85e79b86",
-        "fetch_units": 118370.8, "write_units": 647.3, "valu_busy": 0.69, "graphs": 10000,
+        "source_sha256": "f53f163f2332f8e1e8a8475589e46d3e043090241be17a64c6dceac6a5b3cab0",
+        "fetch_units": 113499.4, "write_units": 647.3, "valu_busy": 0.63, "graphs": 10000,
     },
 }
 
