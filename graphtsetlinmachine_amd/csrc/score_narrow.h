@@ -41,6 +41,7 @@
 // truth rows of all clauses - after the first message layer most are false everywhere.  The truth
 // rows themselves stay complete: a clause that dies gets its row of zeros.
 #pragma once
+#include <type_traits>
 
 constexpr int ROWS_HALF = 3;  // layer 0 on the positive literals' rows (+ node types, all ones), staged in LDS
 
@@ -127,6 +128,28 @@ __device__ __forceinline__ void narrow_block_addresses(uint32_t lo, uint32_t hi,
         : "=&v"(adr[0]), "=&v"(adr[1]), "=&v"(adr[2]), "=&v"(adr[3]), "=&v"(adr[4]), "=&v"(adr[5]), "=&v"(adr[6]),
           "=&v"(adr[7])
         : "v"(lo), "v"(hi), "v"(base));
+}
+
+// The same with the block's entries still in the registers they were fetched into: lane l of a group of 16 holds
+// entries 4 l .. 4 l + 3 of the group's window of 64, so block BLOCK (entries 8 BLOCK ..) sits in lanes 2 BLOCK and
+// 2 BLOCK + 1 of the group's row of 16 lanes, and an entry reaches all 16 lanes inside the add (row broadcast): the
+// entries make no trip through LDS at all.
+template <int BLOCK>
+__device__ __forceinline__ void narrow_block_addresses_of_row(uint32_t e0, uint32_t e1, uint32_t e2, uint32_t e3,
+                                                              uint32_t base, uint32_t (&adr)[8]) {
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_add_u32_dpp %0, %8, %12 row_newbcast:%13 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_add_u32_dpp %1, %9, %12 row_newbcast:%13 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_add_u32_dpp %2, %10, %12 row_newbcast:%13 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_add_u32_dpp %3, %11, %12 row_newbcast:%13 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_add_u32_dpp %4, %8, %12 row_newbcast:%14 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_add_u32_dpp %5, %9, %12 row_newbcast:%14 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_add_u32_dpp %6, %10, %12 row_newbcast:%14 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_add_u32_dpp %7, %11, %12 row_newbcast:%14 row_mask:0xf bank_mask:0xf bound_ctrl:1"
+        : "=&v"(adr[0]), "=&v"(adr[1]), "=&v"(adr[2]), "=&v"(adr[3]), "=&v"(adr[4]), "=&v"(adr[5]), "=&v"(adr[6]),
+          "=&v"(adr[7])
+        : "v"(e0), "v"(e1), "v"(e2), "v"(e3), "v"(base), "n"(2 * BLOCK), "n"(2 * BLOCK + 1));
 }
 
 // AND of two rows that both come in as they are (flip = 0) or both inverted (flip = all ones): one
@@ -447,53 +470,89 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
                 const bool past = b0 * 8 >= ((nb * 8 + NARROW_LIST_AHEAD - 1) & ~(NARROW_LIST_AHEAD - 1));
                 if (past) e = NarrowEntries(ones_in_lane);
                 if (b0 == 0 && gl == 0) e.x = ones_in_lane;  // in the place of the header
-                *reinterpret_cast<NarrowEntries *>(my_list + 4 * gl) = e;
-                // (a wave's LDS accesses are carried out in order: the reads below see the entries just written)
                 const int lim_most = nb_most - b0 < WINDOW / 8 ? nb_most - b0 : WINDOW / 8;
                 // bit b: block b0 + b of this group's list is one of complements (blocks plain .. nb - 1): its rows come in inverted
                 const int from = plain - b0 < 0 ? 0 : plain - b0 > WINDOW / 8 ? WINDOW / 8 : plain - b0;
                 const int to = nb - b0 < 0 ? 0 : nb - b0 > WINDOW / 8 ? WINDOW / 8 : nb - b0;
                 const int flip_bits = to > from ? ((1 << to) - 1) & ~((1 << from) - 1) : 0;
-                uint32_t lo[TRIP], hi[TRIP];
+                // TRIP blocks of 8 rows: read, and ANDed into the running truth
+                auto and_rows = [&](const uint32_t (&adr)[TRIP][8], int at) {
+                    Row r[TRIP][8];
 #pragma unroll
-                for (int t = 0; t < TRIP; ++t) lo[t] = quad_entry[8 * t], hi[t] = quad_entry[8 * t + 4];
+                    for (int t = 0; t < TRIP; ++t)
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) r[t][u].load_lds(adr[t][u]);
+#pragma unroll
+                    for (int t = 0; t < TRIP; ++t) {
+                        // all ones for a block of complements, else zero (a signed one-bit field of flip_bits)
+                        const uint32_t flip = (uint32_t)__builtin_amdgcn_sbfe(flip_bits, at + t, 1);
+#pragma unroll
+                        for (int v = 0; v < WPL; ++v) {
+                            const uint32_t p0 = narrow_pair(r[t][0].w[v], r[t][1].w[v], flip);
+                            const uint32_t p1 = narrow_pair(r[t][2].w[v], r[t][3].w[v], flip);
+                            const uint32_t p2 = narrow_pair(r[t][4].w[v], r[t][5].w[v], flip);
+                            const uint32_t p3 = narrow_pair(r[t][6].w[v], r[t][7].w[v], flip);
+                            acc.w[v] = narrow_and3(narrow_and3(acc.w[v], p0, p1), p2, p3);
+                        }
+                    }
+                };
                 // Two trips between tests for "some group still has a live clause with blocks left": in the regime
                 // that costs the time every clause walks its whole list, and the test is a sixth of a trip's vector
                 // work.  (The blocks past a group's last one are the all-ones row: reading them changes nothing.)
-                for (int b = 0; b < lim_most && work_left(b0 + b); b += 2 * TRIP) {
-#pragma unroll
-                    for (int half = 0; half < 2; ++half) {
-                        const int at = b + half * TRIP;
-                        if (half == 1 && at >= lim_most) break;  // (no group has a block there; uniform over the wave)
-                        uint32_t n_lo[TRIP], n_hi[TRIP];
-#pragma unroll
-                        for (int t = 0; t < TRIP; ++t)
-                            n_lo[t] = quad_entry[8 * (at + TRIP + t)], n_hi[t] = quad_entry[8 * (at + TRIP + t) + 4];
-                        uint32_t adr[TRIP][8];
-#pragma unroll
-                        for (int t = 0; t < TRIP; ++t) narrow_block_addresses(lo[t], hi[t], col_lds, adr[t]);
-                        Row r[TRIP][8];
-#pragma unroll
-                        for (int t = 0; t < TRIP; ++t)
-#pragma unroll
-                            for (int u = 0; u < 8; ++u) r[t][u].load_lds(adr[t][u]);
-#pragma unroll
-                        for (int t = 0; t < TRIP; ++t) {
-                            // all ones for a block of complements, else zero (a signed one-bit field of flip_bits)
-                            const uint32_t flip = (uint32_t)__builtin_amdgcn_sbfe(flip_bits, at + t, 1);
-#pragma unroll
-                            for (int v = 0; v < WPL; ++v) {
-                                const uint32_t p0 = narrow_pair(r[t][0].w[v], r[t][1].w[v], flip);
-                                const uint32_t p1 = narrow_pair(r[t][2].w[v], r[t][3].w[v], flip);
-                                const uint32_t p2 = narrow_pair(r[t][4].w[v], r[t][5].w[v], flip);
-                                const uint32_t p3 = narrow_pair(r[t][6].w[v], r[t][7].w[v], flip);
-                                acc.w[v] = narrow_and3(narrow_and3(acc.w[v], p0, p1), p2, p3);
-                            }
+                if constexpr (GROUP == 16) {
+                    // the window's entries stay in the registers they came in (narrow_block_addresses_of_row): the walk
+                    // over its 8 blocks is unrolled, every block's source lanes being fixed
+                    bool go = true;
+                    auto two_trips = [&](auto first_block) {
+                        constexpr int b = decltype(first_block)::value;
+                        if (!go) return;
+                        if (!(b < lim_most && work_left(b0 + b))) {
+                            go = false;
+                            return;
                         }
-#pragma unroll
-                        for (int t = 0; t < TRIP; ++t) lo[t] = n_lo[t], hi[t] = n_hi[t];
+                        auto trip = [&](auto first) {
+                            constexpr int at = decltype(first)::value;
+                            uint32_t adr[TRIP][8];
+                            narrow_block_addresses_of_row<at>(e.x, e.y, e.z, e.w, col_lds, adr[0]);
+                            if constexpr (TRIP == 2) narrow_block_addresses_of_row<at + 1>(e.x, e.y, e.z, e.w, col_lds, adr[TRIP - 1]);
+                            and_rows(adr, at);
+                        };
+                        trip(std::integral_constant<int, b>{});
+                        if (b + TRIP < lim_most) trip(std::integral_constant<int, b + TRIP>{});  // (else no group has a block there)
+                        nzw = __ballot(acc.any());
+                    };
+                    two_trips(std::integral_constant<int, 0>{});
+                    two_trips(std::integral_constant<int, 2 * TRIP>{});
+                    if constexpr (TRIP == 1) {
+                        two_trips(std::integral_constant<int, 4>{});
+                        two_trips(std::integral_constant<int, 6>{});
                     }
-                    nzw = __ballot(acc.any());
+                } else {
+                    // groups of 8 lanes, two to a row of 16: the entries go through the group's words of LDS and come
+                    // back a block ahead of the rows, four lanes of every quad on entries 0..3 and 4..7 of a block
+                    *reinterpret_cast<NarrowEntries *>(my_list + 4 * gl) = e;
+                    // (a wave's LDS accesses are carried out in order: the reads below see the entries just written)
+                    uint32_t lo[TRIP], hi[TRIP];
+#pragma unroll
+                    for (int t = 0; t < TRIP; ++t) lo[t] = quad_entry[8 * t], hi[t] = quad_entry[8 * t + 4];
+                    for (int b = 0; b < lim_most && work_left(b0 + b); b += 2 * TRIP) {
+#pragma unroll
+                        for (int half = 0; half < 2; ++half) {
+                            const int at = b + half * TRIP;
+                            if (half == 1 && at >= lim_most) break;  // (no group has a block there; uniform over the wave)
+                            uint32_t n_lo[TRIP], n_hi[TRIP];
+#pragma unroll
+                            for (int t = 0; t < TRIP; ++t)
+                                n_lo[t] = quad_entry[8 * (at + TRIP + t)], n_hi[t] = quad_entry[8 * (at + TRIP + t) + 4];
+                            uint32_t adr[TRIP][8];
+#pragma unroll
+                            for (int t = 0; t < TRIP; ++t) narrow_block_addresses(lo[t], hi[t], col_lds, adr[t]);
+                            and_rows(adr, at);
+#pragma unroll
+                            for (int t = 0; t < TRIP; ++t) lo[t] = n_lo[t], hi[t] = n_hi[t];
+                        }
+                        nzw = __ballot(acc.any());
+                    }
                 }
             }
             if (SRC == ROWS_MESSAGES && any_empty) {
