@@ -155,27 +155,30 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
     const int hw = tid >> 5, hl = lane & 31;
     {
         const int n_blocks = MW * tw;
+        // block k * 32 + hw is (j, w) = (id / tw, id % tw): one division, then steps of 32 blocks
+        const int step_j = 32 / tw, step_w = 32 - step_j * tw;
+        const int j_first = hw / tw, w_first = hw - j_first * tw;
         uint32_t held[32];
+        int j = j_first, w = w_first;
 #pragma unroll
         for (int k = 0; k < 32; ++k) {
             held[k] = 0u;
             if (k * 32 >= n_blocks) continue;  // (the same for every thread)
             const int id = k * 32 + hw;
             uint32_t v = 0u;
-            if (id < n_blocks) {
-                const int j = id / tw, w = id - j * tw;
-                v = main_region[(32 * j + hl) * tw + w];
-            }
+            if (id < n_blocks) v = main_region[(32 * j + hl) * tw + w];
             held[k] = tile_transpose32(v, lane);
+            j += step_j, w += step_w;
+            if (w >= tw) w -= tw, ++j;
         }
         __syncthreads();
+        j = j_first, w = w_first;
 #pragma unroll
         for (int k = 0; k < 32; ++k) {
             const int id = k * 32 + hw;
-            if (id < n_blocks) {
-                const int j = id / tw, w = id - j * tw;
-                main_region[(32 * w + hl) * VS + j] = held[k];
-            }
+            if (id < n_blocks) main_region[(32 * w + hl) * VS + j] = held[k];
+            j += step_j, w += step_w;
+            if (w >= tw) w -= tw, ++j;
         }
     }
 
@@ -216,7 +219,10 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
             }
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) first[h][u] = (uint32_t)u < ne[h] ? out_edges[h][u] : make_uint2(0u, 0u);
+        for (int u = 0; u < 4; ++u) {
+            first[h][u] = (uint32_t)u < ne[h] ? out_edges[h][u] : make_uint2(0u, 0u);
+            first[h][u].y %= (uint32_t)M;  // (the edge's rotation, reduced once for all the passes)
+        }
         mine[h] = main_region + (slot < S ? slot : 0) * VS;
     }
 
@@ -225,35 +231,44 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
         for (int i = tid; i < nw * 32 * VS; i += NT) got[i] = 0u;
         __syncthreads();  // (also: every vector of step 2 is in place)
 
-        // 3. along the edges into the range
+        // 3. along the edges into the range: bit p of what arrives is bit (p - shift) mod M of what was sent, so word
+        // j of the node's vector, moved up by r = shift % 32 bits with the top of word j - 1 below it, lands in word
+        // (j + shift / 32) mod MW.  A word of the vector is read once for the (up to four) edges at hand, and the
+        // move is one 64-bit shift of (word j, word j - 1) by 32 - r.
 #pragma unroll
         for (int h = 0; h < SPT; ++h)
             for (uint32_t e0 = 0; e0 < ne[h]; e0 += 4) {
-                uint2 pair[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u)
-                    pair[u] = e0 == 0 ? first[h][u] : (e0 + u < ne[h] ? out_edges[h][e0 + u] : make_uint2(0u, 0u));
+                uint32_t *to[4];
+                uint32_t down[4];
+                int at[4];
+                bool on[4], any = false;
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    if (e0 + u >= ne[h]) break;
-                    const uint32_t dst = pair[u].x;
-                    if (dst >= nodes_of_graph[h]) continue;
-                    const int to_slot = slot0[h] + (int)dst, to_word = to_slot >> 5;
-                    if (to_word < w_lo || to_word >= w_hi) continue;
-                    const uint32_t shift = pair[u].y % (uint32_t)M;
-                    const int r = (int)(shift & 31u);
-                    uint32_t *to = got + (to_slot - 32 * w_lo) * VS;
-                    // bit p of what arrives is bit (p - shift) mod M of what was sent: word j, moved up by r bits with
-                    // the top of word j - 1 below it, lands in word (j + shift / 32) mod MW
-                    int at = (int)(shift >> 5);
-                    uint32_t below = mine[h][MW - 1];
-                    for (int j = 0; j < MW; ++j) {
-                        const uint32_t cur = mine[h][j];
-                        const uint32_t word = r ? (cur << r) | (below >> (32 - r)) : cur;
-                        if (word) atomicOr(&to[at], word);
-                        at = at + 1 == MW ? 0 : at + 1;
-                        below = cur;
+                    uint2 pair = first[h][u];
+                    if (e0 != 0) {
+                        pair = e0 + u < ne[h] ? out_edges[h][e0 + u] : make_uint2(0u, 0u);
+                        pair.y %= (uint32_t)M;
                     }
+                    const uint32_t dst = pair.x;
+                    const int to_slot = slot0[h] + (int)dst, to_word = to_slot >> 5;
+                    on[u] = e0 + u < ne[h] && dst < nodes_of_graph[h] && to_word >= w_lo && to_word < w_hi;
+                    to[u] = got + (on[u] ? to_slot - 32 * w_lo : 0) * VS;
+                    down[u] = 32u - (pair.y & 31u);
+                    at[u] = (int)(pair.y >> 5);
+                    any = any || on[u];
+                }
+                if (!any) continue;
+                uint32_t below = mine[h][MW - 1];
+                for (int j = 0; j < MW; ++j) {
+                    const uint32_t cur = mine[h][j];
+                    const unsigned long long both = ((unsigned long long)cur << 32) | below;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const uint32_t word = (uint32_t)(both >> down[u]);
+                        if (on[u] && word) atomicOr(&to[u][at[u]], word);
+                        at[u] = at[u] + 1 == MW ? 0 : at[u] + 1;
+                    }
+                    below = cur;
                 }
             }
         __syncthreads();
@@ -261,9 +276,11 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
         // 4. literal-major: block (j, w) of the range - word j of slots 32 w .. 32 w + 31 - becomes word w of rows
         // 32 j .. 32 j + 31; a half-wave turns four neighbouring blocks and each lane stores its row's four words at once
         const int nq = nw >> 2, n_units = MW * nq;
-        for (int k = 0; k * 32 < n_units; ++k) {
+        const int unit_step_j = 32 / nq, unit_step_w = 32 - unit_step_j * nq;  // (unit k * 32 + hw is (id / nq, id % nq))
+        int j = hw / nq, wq = hw - j * nq;
+        for (int k = 0; k * 32 < n_units; ++k, j += unit_step_j, wq += unit_step_w) {
+            if (wq >= nq) wq -= nq, ++j;
             const int id = k * 32 + hw;
-            const int j = id / nq, wq = id - j * nq;
             uint32_t column[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
