@@ -333,7 +333,11 @@ __global__ void k_compile_clauses(const uint32_t *__restrict__ bank, int C, int 
     for (int i = padded + lane; i < fill_to; i += 64) list[i] = ones;
     // entry 0: blocks of rows to AND | blocks of rows whose complements to AND << 16
     if (lane == 0) list[0] = (uint32_t)(plain_padded >> 3) | ((uint32_t)(neg_padded >> 3) << 16);
-    if (longest && lane == 0) atomicMax(longest, (uint32_t)padded);  // entries of the longest list (cleared by the caller)
+    // entries of the longest list (cleared by the caller).  Thousands of atomics on one word are carried out one after
+    // the other, about 10 ns each: a clause first looks whether the word already holds as much (it only ever grows,
+    // so an old value can only cause an atomic that was not needed, never miss one).
+    if (longest && lane == 0 && (uint32_t)padded > __hip_atomic_load(longest, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+        atomicMax(longest, (uint32_t)padded);
     if (weights)
         for (int k = lane; k < K; k += 64) wt[(int64_t)c * K + k] = weights[(int64_t)k * C + c];
 }
