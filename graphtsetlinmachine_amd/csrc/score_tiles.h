@@ -832,10 +832,9 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
         if (staged) {
             for (int i = tid; i <= M; i += NT) s_start[i] = bit_start[i];
             for (uint32_t i = tid; i < n_listed; i += NT) s_clauses[i] = bit_clauses[i];
-            for (int i = tid; i < C * used; i += NT) {
-                const int c = i / used, w = i - c * used;
-                s_truth[c * ts + w] = truth[(int64_t)c * tw + w];
-            }
+            // (half a wave per clause and trip: no division to find an element's clause and word)
+            for (int c = tid >> 5; c < C; c += NT / 32)
+                for (int w = tid & 31; w < used; w += 32) s_truth[c * ts + w] = truth[(int64_t)c * tw + w];
             __syncthreads();
         }
         const int hl = lane & 31, half = lane >> 5;
@@ -889,11 +888,12 @@ __global__ __launch_bounds__(TILE_FUSED_MESSAGES_BLOCK) void k_tile_messages_fus
                     uint32_t *to = got + dst * MWP + (dst >> 5);
                     if (MW <= IN_REGISTERS) {
                         int at = q;  // the word that word 0 of the vector goes to
+                        const uint32_t down = 32u - (uint32_t)r;  // (word j, word j - 1) moved down by 32 - r: one 64-bit shift
 #pragma unroll
                         for (int j = 0; j < IN_REGISTERS; ++j) {
                             if (j < MW) {
                                 const uint32_t below = j == 0 ? last : mine[j > 0 ? j - 1 : 0];
-                                const uint32_t word = r ? (mine[j] << r) | (below >> (32 - r)) : mine[j];
+                                const uint32_t word = (uint32_t)((((unsigned long long)mine[j] << 32) | below) >> down);
                                 if (word) atomicOr(&to[at], word);
                                 at = at + 1 == MW ? 0 : at + 1;
                             }
