@@ -387,6 +387,27 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
     int n_out = 0;
 
     const int pairs = tg.gpt * K, sw = tg.slot_words;
+    // Votes (last layer): lane p of a group adds weight k = p % K to graph j = p / K of the tile, for p = gl and
+    // gl + GROUP; which class that is and which lanes of the group hold the graph's words (per word v of a lane:
+    // ceil((w_lo - v) / WPL) <= l < ceil((w_hi - v) / WPL) for the graph's words [w_lo, w_hi)) does not depend on
+    // the clause and is worked out once.  More (graph, class) pairs than that take the loop further down.
+    constexpr int VOTES_AHEAD = 2;
+    const bool votes_ahead = LAST && pairs <= VOTES_AHEAD * GROUP;
+    int vote_class[VOTES_AHEAD];
+    uint32_t vote_lanes[VOTES_AHEAD][WPL];
+#pragma unroll
+    for (int i = 0; i < VOTES_AHEAD; ++i) {
+        const int p = gl + GROUP * i;
+        const bool on = LAST && p < pairs;
+        const int j = on ? p / K : 0;  // (a graph of the tile: the shifts below stay within the group's lanes)
+        vote_class[i] = on ? p - j * K : 0;
+        const int w_lo = j * sw, w_hi = w_lo + sw;
+#pragma unroll
+        for (int v = 0; v < WPL; ++v) {
+            const int l_lo = (w_lo + WPL - 1 - v) / WPL, l_hi = (w_hi + WPL - 1 - v) / WPL;
+            vote_lanes[i][v] = on ? ((1u << l_hi) - 1u) & ~((1u << l_lo) - 1u) : 0u;
+        }
+    }
 
     // The clause of item i of this stream (-1 past its end).  With a list of the clauses still alive, GROUP items
     // are held one per lane of the group and handed out with a lane read.
@@ -577,6 +598,15 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
 #pragma unroll
                     for (int v = 0; v < WPL; ++v) nonzero[v] = votes_of_group(__ballot(acc.w[v] != 0u));
                     const int32_t *weights_of_clause = a.wt + (int64_t)c * K;
+                    if (votes_ahead) {
+#pragma unroll
+                        for (int i = 0; i < VOTES_AHEAD; ++i) {
+                            uint32_t hit = 0u;
+#pragma unroll
+                            for (int v = 0; v < WPL; ++v) hit |= nonzero[v] & vote_lanes[i][v];
+                            if (hit) atomicAdd(&sums[gl + GROUP * i], weights_of_clause[vote_class[i]]);
+                        }
+                    } else
                     for (int p = gl; p < pairs; p += GROUP) {
                         const int j = p / K, k = p - j * K;
                         const int w_lo = j * sw, w_hi = w_lo + sw;  // the graph's words
