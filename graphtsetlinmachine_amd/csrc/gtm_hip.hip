@@ -1258,7 +1258,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     const char *narrow_reads = tune(T_NARROW_READS);
     const NarrowChoice shape = narrow_choice(tg, narrow_reads && atoi(narrow_reads) == 128);
     // (the kernel reaches lists and truth rows at 32-bit byte offsets formed from 24-bit factors)
-    const bool narrow_tiles = shape.group != 0 && !tune(T_NO_NARROW_LAYERS) && d.C < (1 << 24) &&
+    const bool narrow_tiles = shape.group != 0 && !tune(T_NO_NARROW_LAYERS) && d.C < (1 << 24) && (int64_t)d.C * d.K < (1 << 28) &&
                               (int64_t)d.C * std::max(w.list_stride, w.message_list_stride) * 4 < (1ll << 31);
     const bool narrow_messages =
         narrow_tiles && layers > 1 && narrow_lds_bytes(tg, shape, d.K, tile_message_rows(d.M), tg.tw) <= lds_limit;

@@ -319,6 +319,8 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
     const __amdgpu_buffer_rsrc_t lists_buffer =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t *>(a.lists), 0, C * a.stride * 4, NARROW_BUFFER_FLAGS);
     const __amdgpu_buffer_rsrc_t truth_buffer = __builtin_amdgcn_make_buffer_rsrc(bitmap, 0, C * tw * 4, NARROW_BUFFER_FLAGS);
+    const __amdgpu_buffer_rsrc_t weights_buffer =  // clause-major weights (last layer)
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t *>(LAST ? a.wt : nullptr), 0, LAST ? C * K * 4 : 0, NARROW_BUFFER_FLAGS);
 
     {  // rows -> LDS, 16 bytes per thread and trip, four loads in flight
         const uint4 *src;
@@ -597,14 +599,16 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
                     uint32_t nonzero[WPL];  // bit l: word WPL l + v
 #pragma unroll
                     for (int v = 0; v < WPL; ++v) nonzero[v] = votes_of_group(__ballot(acc.w[v] != 0u));
-                    const int32_t *weights_of_clause = a.wt + (int64_t)c * K;
+                    const uint32_t weights_at = __umul24((uint32_t)c, (uint32_t)K * 4u);  // byte offset of the clause's weights
                     if (votes_ahead) {
 #pragma unroll
                         for (int i = 0; i < VOTES_AHEAD; ++i) {
                             uint32_t hit = 0u;
 #pragma unroll
                             for (int v = 0; v < WPL; ++v) hit |= nonzero[v] & vote_lanes[i][v];
-                            if (hit) atomicAdd(&sums[gl + GROUP * i], weights_of_clause[vote_class[i]]);
+                            if (hit)
+                                atomicAdd(&sums[gl + GROUP * i],
+                                          (int)__builtin_amdgcn_raw_buffer_load_b32(weights_buffer, (int)(weights_at + 4u * (uint32_t)vote_class[i]), 0, 0));
                         }
                     } else
                     for (int p = gl; p < pairs; p += GROUP) {
@@ -617,7 +621,8 @@ __global__ __launch_bounds__(NARROW_WAVES * 64) void k_tile_layer_narrow(TileLay
                             const int l_lo = (w_lo + WPL - 1 - v) / WPL, l_hi = (w_hi + WPL - 1 - v) / WPL;
                             hit |= nonzero[v] & ((1u << l_hi) - 1u) & ~((1u << l_lo) - 1u);
                         }
-                        if (hit) atomicAdd(&sums[p], weights_of_clause[k]);
+                        if (hit)
+                            atomicAdd(&sums[p], (int)__builtin_amdgcn_raw_buffer_load_b32(weights_buffer, (int)(weights_at + 4u * (uint32_t)k), 0, 0));
                     }
                 }
             }
