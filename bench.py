@@ -35,7 +35,7 @@ VALU_PEAK_LANE_OPS = 256 * 64 * 2.4e9  # 32-bit integer lane operations per seco
 # library was built from another text reports no counters rather than stale ones.
 MEASURED_COUNTERS = {
     "convolutional_images": {
-        "kernel": "k_tile_two_phase_half<score>", "commit": "60acd24",
+        "kernel": "k_tile_two_phase_half<score>", "commit": "f694c07",
         "functions": ("tile_segments_part", "lowest_bit_or_ones", "k_compile_clauses_half", "half_combine",
                       "k_tile_two_phase_half"),
         "source_sha256": "f53f163f2332f8e1e8a8475589e46d3e043090241be17a64c6dceac6a5b3cab0",
