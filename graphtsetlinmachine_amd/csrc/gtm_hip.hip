@@ -1402,7 +1402,7 @@ int score_on_tiles(const Dims &d, const gtm_config *cfg, const gtm_graphs *g, co
     {
         const char *e = tune(T_MESSAGES_IN_LDS);
         const bool off = e && atoi(e) == 0, preferred = e && atoi(e) != 0;
-        if (layers > 1 && !off && (preferred || !fused_messages)) in_lds = tile_messages_lds_plan(tg, d.M, lds_limit);
+        if (layers > 1 && !off && d.C < (1 << 24) && (preferred || !fused_messages)) in_lds = tile_messages_lds_plan(tg, d.M, lds_limit);
     }
     if (in_lds.ok) {
         static thread_local size_t in_lds_set = 48 * 1024;

@@ -95,8 +95,12 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
         constexpr int WPL = WIDE ? 4 : 2;  // words of a truth row per lane
         typedef uint32_t Words __attribute__((ext_vector_type(WPL)));
         const int group = lane >> 4, gl = lane & 15;
-        const uint32_t *truth = bitmap + (int64_t)tile_local * C * tw;
+        // the tile's truth rows through a buffer descriptor: a row is reached by a multiply-add of 24-bit factors per
+        // lane (clause x bytes per row + the lane's place), not by a 64-bit multiply and add
+        const __amdgpu_buffer_rsrc_t truth = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint32_t *>(bitmap + (int64_t)tile_local * C * tw), 0, C * tw * 4, 0x00020000);
         const bool has_words = WPL * gl < tw;
+        const uint32_t place = has_words ? 4u * WPL * gl : 0u;
         // a quarter-wave takes the streams q, q + 64, ... of the evaluation that wrote the truth rows
         for (int q = wave * 4 + group; q < streams; q += TILE_MESSAGES_LDS_BLOCK / 16) {
         const uint32_t *list = alive ? alive + ((int64_t)tile_local * streams + q) * alive_stride : nullptr;
@@ -122,7 +126,12 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     c[u] = tile_row_share(id, u0 + u);  // (past the stream's end: its last clause once more)
-                    t[u] = *reinterpret_cast<const Words *>(truth + (int64_t)c[u] * tw + (has_words ? WPL * gl : 0));
+                    const int at = (int)(__umul24(c[u], (uint32_t)tw * 4u) + place);
+                    if constexpr (WIDE) {
+                        t[u] = __builtin_amdgcn_raw_buffer_load_b128(truth, at, 0, 0);
+                    } else {
+                        t[u] = __builtin_amdgcn_raw_buffer_load_b64(truth, at, 0, 0);
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
@@ -134,7 +143,7 @@ __global__ __launch_bounds__(TILE_MESSAGES_LDS_BLOCK) void k_tile_messages_in_ld
                         const uint32_t h = j == 0 ? h0 : j == 1 ? h1 : hv[(int64_t)c[u] * MB + j];
                         if (h >= (uint32_t)M) continue;
                         // (tw is a multiple of 4: each pair of words is one aligned 64-bit word of LDS)
-                        unsigned long long *row = reinterpret_cast<unsigned long long *>(main_region + h * tw + WPL * gl);
+                        unsigned long long *row = reinterpret_cast<unsigned long long *>(main_region + __umul24(h, (uint32_t)tw) + WPL * gl);
 #pragma unroll
                         for (int v = 0; v < WPL / 2; ++v) {
                             const unsigned long long both =
